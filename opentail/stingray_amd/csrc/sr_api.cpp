@@ -1,0 +1,458 @@
+// Host side of the C ABI declared in include/stingray_sampler.h: context and scratch ownership, the
+// packer that turns SamplingParams / PreviousTokens / LogitBias into device row descriptors, and the
+// per-entry-point launch sequences.  No vocabulary-sized work happens on the host.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "sr_host.h"
+
+namespace {
+
+inline bool has_history_penalty(const sr_row_params& p)
+{
+    return p.repetition_penalty != 1.0f || p.presence_penalty != 0.0f || p.frequency_penalty != 0.0f;
+}
+
+// Chunking of a row for the selection kernel: every chunk must fit the per-workgroup register window.
+void topk_geometry(int vocab, int dtype, int n_rows, int cu_count, int* chunks, int* chunk_len)
+{
+    const int epv = dtype == SR_DTYPE_BF16 ? 8 : 4;
+    const int window = SR_TK_VEC * SR_TK_THREADS * epv;
+    const int usable = window - epv;  // slack for a misaligned row start
+    int s_min = (vocab + usable - 1) / usable;
+    int s_par = (2 * cu_count + n_rows - 1) / std::max(n_rows, 1);  // aim for two workgroups per CU
+    int s_cap = std::max(1, vocab / 2048);
+    int s = std::max(s_min, std::min(s_par, s_cap));
+    int len = (vocab + s - 1) / s;
+    len = (len + 7) & ~7;
+    if (len > usable) len = usable & ~7;
+    s = (vocab + len - 1) / len;
+    *chunks = std::max(s, 1);
+    *chunk_len = std::max(len, 8);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* sr_version(void) { return "0.1.0"; }
+
+int sr_create(int device_ordinal, sr_ctx** out)
+{
+    if (!out) return SR_ERR_NULL_ARGUMENT;
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0 || device_ordinal < 0 || device_ordinal >= n)
+        return SR_ERR_NO_DEVICE;
+    sr_ctx* ctx = new (std::nothrow) sr_ctx();
+    if (!ctx) return SR_ERR_OUT_OF_MEMORY;
+    ctx->device = device_ordinal;
+    if (hipSetDevice(device_ordinal) != hipSuccess) { delete ctx; return SR_ERR_NO_DEVICE; }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device_ordinal) == hipSuccess) ctx->cu_count = prop.multiProcessorCount;
+    if (hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking) != hipSuccess) {
+        delete ctx;
+        return SR_ERR_HIP;
+    }
+    ctx->stream = ctx->own_stream;
+    *out = ctx;
+    return SR_OK;
+}
+
+void sr_destroy(sr_ctx* ctx)
+{
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
+    DeviceBuf* bufs[] = {&ctx->cand_val, &ctx->cand_idx, &ctx->cand_cnt, &ctx->row_done, &ctx->argmax_best,
+                         &ctx->work, &ctx->host_logits, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
+                         &ctx->uniforms_tmp};
+    for (DeviceBuf* b : bufs) b->release();
+    if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
+    delete ctx;
+}
+
+int sr_bind_thread(sr_ctx* ctx)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    return SR_OK;
+}
+
+int sr_set_stream(sr_ctx* ctx, void* hip_stream)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+    return SR_OK;
+}
+
+int sr_synchronize(sr_ctx* ctx)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return SR_OK;
+}
+
+const char* sr_last_error(sr_ctx* ctx) { return ctx ? ctx->err.c_str() : "null context"; }
+
+int sr_batch_create(sr_ctx* ctx, sr_batch** out)
+{
+    if (!ctx || !out) return SR_ERR_NULL_ARGUMENT;
+    sr_batch* b = new (std::nothrow) sr_batch();
+    if (!b) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "sr_batch_create: out of host memory");
+    b->ctx = ctx;
+    *out = b;
+    return SR_OK;
+}
+
+void sr_batch_destroy(sr_batch* b)
+{
+    if (!b) return;
+    if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
+    DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_mask, &b->d_uniforms};
+    for (DeviceBuf* d : bufs) d->release();
+    delete b;
+}
+
+int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_params* params,
+                    const int32_t* hist_ids, const int32_t* hist_offsets,
+                    const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                    const uint32_t* allow_mask, int64_t mask_stride_words, const uint8_t* mask_active,
+                    const double* uniforms, int32_t uniforms_per_row)
+{
+    if (!b || !b->ctx) return SR_ERR_NULL_ARGUMENT;
+    sr_ctx* ctx = b->ctx;
+    if (!params) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: params is null");
+    if (rows < 0 || vocab < 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_upload: negative shape");
+    if (hist_offsets && !hist_ids && hist_offsets[rows] > hist_offsets[0])
+        return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: hist_ids is null");
+    if (bias_offsets && (!bias_ids || !bias_vals) && bias_offsets[rows] > bias_offsets[0])
+        return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: bias arrays are null");
+    if (allow_mask && mask_stride_words < (vocab + 31) / 32)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_upload: mask stride shorter than ceil(vocab/32)");
+    if (uniforms_per_row < 0 || (uniforms_per_row > 0 && !uniforms))
+        return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: uniforms is null");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+
+    b->rows = rows;
+    b->vocab = vocab;
+    b->upr = uniforms_per_row;
+    b->h_rows.assign((size_t)rows, SrRow{});
+    b->h_edits.clear();
+    b->h_sel_list.clear();
+    b->h_full_list.clear();
+    b->has_mask = allow_mask != nullptr;
+    b->mask_stride = allow_mask ? mask_stride_words : 0;
+    b->max_sel = 0;
+
+    struct Occ { int32_t id; int32_t in_window; };
+    std::vector<Occ> occ;
+    for (int32_t r = 0; r < rows; r++) {
+        const sr_row_params& p = params[r];
+        SrRow& d = b->h_rows[(size_t)r];
+        const int32_t h0 = hist_offsets ? hist_offsets[r] : 0, h1 = hist_offsets ? hist_offsets[r + 1] : 0;
+        const int32_t n_prev = std::max(0, h1 - h0);
+        const int32_t* prev = hist_ids ? hist_ids + h0 : nullptr;
+        const int32_t b0 = bias_offsets ? bias_offsets[r] : 0, b1 = bias_offsets ? bias_offsets[r + 1] : 0;
+        const int32_t n_bias = std::max(0, b1 - b0);
+        const bool has_bias = n_bias > 0 || (p.flags & SR_ROW_HAS_LOGIT_BIAS);
+        const bool hist_pen = has_history_penalty(p);
+        const bool has_penalty = n_prev > 0 && hist_pen;
+
+        d.temperature = p.temperature;
+        d.top_p = p.top_p;
+        d.min_p = p.min_p;
+        d.rep = p.repetition_penalty;
+        d.presence = p.presence_penalty;
+        d.frequency = p.frequency_penalty;
+        d.p_min = p.spec_draft_p_min;
+        d.top_k = p.top_k;
+        d.n_prev = n_prev;
+        d.flags = (p.flags & 0xffu) | (has_bias ? (uint32_t)SR_ROW_HAS_LOGIT_BIAS : 0u) |
+                  (has_penalty ? SR_ROWFLAG_HAS_PENALTY : 0u);
+        d.mask_row = (allow_mask && (!mask_active || mask_active[r])) ? r : -1;
+        d.edit_off = (int32_t)b->h_edits.size();
+        d.edit_cnt = 0;
+        d.sel = 1;
+
+        // Sampler.Sample dispatch (Sampler.cs:19-39)
+        if (p.temperature <= 0.0f) {
+            d.path = has_penalty ? SR_PATH_GREEDY_PEN : SR_PATH_GREEDY;
+        } else if (p.top_k > 0 && p.top_k < vocab && !has_bias) {
+            d.path = SR_PATH_TOPK;
+            int64_t sel = (int64_t)p.top_k + (has_penalty ? n_prev : 0);
+            d.sel = (int32_t)std::min<int64_t>(sel, vocab);
+        } else {
+            d.path = SR_PATH_FULL;
+        }
+        const bool greedy = p.temperature <= 0.0f;
+        const bool want_hist = has_penalty;
+        const bool want_bias = n_bias > 0 && !greedy;  // LogitBias is ignored by the greedy paths
+        if (want_hist || want_bias) {
+            // occurrence counts of every in-range id: whole history and trailing repetition window
+            occ.clear();
+            if (want_hist) {
+                const int32_t ws = (p.repeat_last_n <= 0 || p.repeat_last_n >= n_prev) ? 0 : n_prev - p.repeat_last_n;
+                for (int32_t i = 0; i < n_prev; i++)
+                    if ((uint32_t)prev[i] < (uint32_t)vocab) occ.push_back({prev[i], i >= ws ? 1 : 0});
+                std::stable_sort(occ.begin(), occ.end(), [](const Occ& x, const Occ& y) { return x.id < y.id; });
+            }
+            std::vector<SrEdit>& ed = b->h_edits;
+            for (size_t i = 0; i < occ.size();) {
+                size_t j = i;
+                int32_t win = 0;
+                while (j < occ.size() && occ[j].id == occ[i].id) { win += occ[j].in_window; j++; }
+                SrEdit e{};
+                e.id = occ[i].id;
+                e.occ_all = (int32_t)(j - i);
+                e.occ_win = win;
+                e.pen = (p.repetition_penalty != 1.0f && win > 0) ? powf(p.repetition_penalty, (float)win) : 1.0f;
+                ed.push_back(e);
+                i = j;
+            }
+            if (want_bias) {
+                for (int32_t i = b0; i < b1; i++) {
+                    int32_t id = bias_ids[i];
+                    if ((uint32_t)id >= (uint32_t)vocab) continue;
+                    auto first = ed.begin() + d.edit_off;
+                    auto it = std::lower_bound(first, ed.end(), id, [](const SrEdit& e, int32_t v) { return e.id < v; });
+                    if (it == ed.end() || it->id != id) {
+                        SrEdit e{};
+                        e.id = id;
+                        e.pen = 1.0f;
+                        it = ed.insert(it, e);
+                    }
+                    it->bias = it->has_bias ? it->bias + bias_vals[i] : bias_vals[i];
+                    it->has_bias = 1u;
+                }
+            }
+            d.edit_cnt = (int32_t)ed.size() - d.edit_off;
+        }
+        if (d.path == SR_PATH_TOPK || d.path == SR_PATH_GREEDY) {
+            b->h_sel_list.push_back(r);
+            b->max_sel = std::max(b->max_sel, d.sel);
+        } else {
+            b->h_full_list.push_back(r);
+        }
+    }
+
+    auto up = [&](DeviceBuf& dst, const void* src, size_t bytes) -> hipError_t {
+        if (bytes == 0) return hipSuccess;
+        hipError_t e = dst.reserve(bytes, st);
+        if (e != hipSuccess) return e;
+        return hipMemcpyAsync(dst.p, src, bytes, hipMemcpyHostToDevice, st);
+    };
+    SR_HIP(ctx, up(b->d_rows, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow)));
+    SR_HIP(ctx, up(b->d_edits, b->h_edits.data(), b->h_edits.size() * sizeof(SrEdit)));
+    SR_HIP(ctx, up(b->d_sel_list, b->h_sel_list.data(), b->h_sel_list.size() * sizeof(int32_t)));
+    SR_HIP(ctx, up(b->d_full_list, b->h_full_list.data(), b->h_full_list.size() * sizeof(int32_t)));
+    if (allow_mask) SR_HIP(ctx, up(b->d_mask, allow_mask, (size_t)rows * (size_t)mask_stride_words * sizeof(uint32_t)));
+    if (uniforms_per_row > 0)
+        SR_HIP(ctx, up(b->d_uniforms, uniforms, (size_t)rows * (size_t)uniforms_per_row * sizeof(double)));
+    // the host vectors are read by the async copies above
+    SR_HIP(ctx, hipStreamSynchronize(st));
+    return SR_OK;
+}
+
+int sr_batch_set_uniforms(sr_batch* b, const double* uniforms)
+{
+    if (!b || !b->ctx) return SR_ERR_NULL_ARGUMENT;
+    sr_ctx* ctx = b->ctx;
+    if (!uniforms) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_set_uniforms: uniforms is null");
+    if (b->upr <= 0 || b->rows <= 0) return SR_OK;
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    SR_HIP(ctx, hipMemcpyAsync(b->d_uniforms.p, uniforms, (size_t)b->rows * b->upr * sizeof(double),
+                               hipMemcpyHostToDevice, ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return SR_OK;
+}
+
+int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride_elems,
+                     int32_t* out_tokens_dev, uint32_t* out_flags_dev)
+{
+    if (!ctx || !b) return SR_ERR_NULL_ARGUMENT;
+    if (b->rows == 0) return SR_OK;
+    if (!logits_dev || !out_tokens_dev) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_launch: null tensor");
+    if (dtype != SR_DTYPE_F32 && dtype != SR_DTYPE_BF16)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_launch: unknown dtype");
+    if (row_stride_elems < b->vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_launch: row stride < vocab");
+    if (b->vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_launch: empty vocabulary");
+    for (const SrRow& r : b->h_rows)
+        if (r.path != SR_PATH_GREEDY && r.path != SR_PATH_GREEDY_PEN && b->upr < 1)
+            return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_launch: a sampled row needs a uniform");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+
+    const int n_sel = (int)b->h_sel_list.size();
+    if (n_sel > 0) {
+        if (b->max_sel > SR_TK_SEL_MAX)
+            return sr_fail(ctx, SR_ERR_UNSUPPORTED,
+                        "sr_sample_launch: top_k + history length exceeds " + std::to_string(SR_TK_SEL_MAX));
+        SrTopkArgs a{};
+        a.logits = logits_dev;
+        a.row_stride = row_stride_elems;
+        a.vocab = b->vocab;
+        a.dtype = dtype;
+        topk_geometry(b->vocab, dtype, n_sel, ctx->cu_count, &a.chunks, &a.chunk_len);
+        const size_t slots = (size_t)n_sel * a.chunks;
+        SR_HIP(ctx, ctx->cand_val.reserve(slots * SR_TK_CAP * sizeof(float), st));
+        SR_HIP(ctx, ctx->cand_idx.reserve(slots * SR_TK_CAP * sizeof(int32_t), st));
+        SR_HIP(ctx, ctx->cand_cnt.reserve(slots * sizeof(int32_t), st));
+        SR_HIP(ctx, ctx->row_done.reserve((size_t)std::max(n_sel, 1024) * sizeof(uint32_t), st, true));
+        a.row_list = b->d_sel_list.as<int32_t>();
+        a.rows = b->d_rows.as<SrRow>();
+        a.edits = b->d_edits.as<SrEdit>();
+        a.mask = b->d_mask.as<uint32_t>();
+        a.mask_stride = b->mask_stride;
+        a.cand_val = ctx->cand_val.as<float>();
+        a.cand_idx = ctx->cand_idx.as<int32_t>();
+        a.cand_cnt = ctx->cand_cnt.as<int32_t>();
+        a.row_done = ctx->row_done.as<uint32_t>();
+        a.uniforms = b->d_uniforms.as<double>();
+        a.uniforms_per_row = b->upr;
+        a.out_tokens = out_tokens_dev;
+        a.out_flags = out_flags_dev;
+        SR_HIP(ctx, sr_launch_topk(a, n_sel, st));
+    }
+    if (!b->h_full_list.empty()) {
+        int rc = sr_full_rows_launch(ctx, b, logits_dev, dtype, row_stride_elems, out_tokens_dev, out_flags_dev);
+        if (rc != SR_OK) return rc;
+    }
+    return SR_OK;
+}
+
+static int stage_logits(sr_ctx* ctx, const void* logits, int dtype, int on_device, int32_t rows, int32_t vocab,
+                        int64_t stride, const void** dev)
+{
+    if (on_device) { *dev = logits; return SR_OK; }
+    const size_t es = dtype == SR_DTYPE_BF16 ? 2 : 4;
+    const size_t bytes = ((size_t)(rows - 1) * (size_t)stride + (size_t)vocab) * es;
+    SR_HIP(ctx, ctx->host_logits.reserve(bytes, ctx->stream));
+    SR_HIP(ctx, hipMemcpyAsync(ctx->host_logits.p, logits, bytes, hipMemcpyHostToDevice, ctx->stream));
+    *dev = ctx->host_logits.p;
+    return SR_OK;
+}
+
+int sr_sample_batch(sr_ctx* ctx, const void* logits, int dtype, int logits_on_device, int32_t rows, int32_t vocab,
+                    int64_t row_stride_elems, const sr_row_params* params,
+                    const int32_t* hist_ids, const int32_t* hist_offsets,
+                    const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                    const uint32_t* allow_mask, int64_t mask_stride_words, const uint8_t* mask_active,
+                    const double* uniforms, int32_t* out_tokens, uint32_t* out_flags)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0) return SR_OK;
+    if (!logits || !out_tokens || !params) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_batch: null argument");
+    if (rows < 0 || vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_batch: bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    if (!ctx->tmp_batch) {
+        int rc = sr_batch_create(ctx, &ctx->tmp_batch);
+        if (rc != SR_OK) return rc;
+    }
+    int rc = sr_batch_upload(ctx->tmp_batch, rows, vocab, params, hist_ids, hist_offsets, bias_ids, bias_vals,
+                             bias_offsets, allow_mask, mask_stride_words, mask_active, uniforms, uniforms ? 1 : 0);
+    if (rc != SR_OK) return rc;
+    const void* dev = nullptr;
+    rc = stage_logits(ctx, logits, dtype, logits_on_device, rows, vocab, row_stride_elems, &dev);
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, ctx->out_tokens.reserve((size_t)rows * sizeof(int32_t), ctx->stream));
+    SR_HIP(ctx, ctx->out_flags.reserve((size_t)rows * sizeof(uint32_t), ctx->stream));
+    rc = sr_sample_launch(ctx, ctx->tmp_batch, dev, dtype, row_stride_elems, ctx->out_tokens.as<int32_t>(),
+                          ctx->out_flags.as<uint32_t>());
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, hipMemcpyAsync(out_tokens, ctx->out_tokens.p, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost,
+                               ctx->stream));
+    if (out_flags)
+        SR_HIP(ctx, hipMemcpyAsync(out_flags, ctx->out_flags.p, (size_t)rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                   ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return SR_OK;
+}
+
+int sr_argmax_rows_launch(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows, int32_t vocab,
+                          int64_t row_stride_elems, int32_t* out_idx_dev, float* out_val_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0) return SR_OK;
+    if (!out_idx_dev || (!logits_dev && vocab > 0)) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_argmax_rows: null tensor");
+    if (rows < 0 || vocab < 0 || (vocab > 0 && row_stride_elems < vocab))
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_argmax_rows: bad shape");
+    if (dtype != SR_DTYPE_F32 && dtype != SR_DTYPE_BF16)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_argmax_rows: unknown dtype");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    SR_HIP(ctx, ctx->argmax_best.reserve((size_t)rows * sizeof(unsigned long long), ctx->stream));
+    SrArgmaxArgs a{};
+    a.logits = logits_dev;
+    a.row_stride = row_stride_elems;
+    a.vocab = vocab;
+    a.dtype = dtype;
+    a.rows = rows;
+    int s = std::max(1, std::min((4 * ctx->cu_count + rows - 1) / rows, std::max(1, vocab / 4096)));
+    a.chunk_len = (vocab + s - 1) / s;
+    if (a.chunk_len < 1) a.chunk_len = 1;
+    a.chunks = vocab > 0 ? (vocab + a.chunk_len - 1) / a.chunk_len : 1;
+    a.best = ctx->argmax_best.as<unsigned long long>();
+    a.out_idx = out_idx_dev;
+    a.out_val = out_val_dev;
+    SR_HIP(ctx, sr_launch_argmax_rows(a, ctx->stream));
+    return SR_OK;
+}
+
+int sr_argmax_rows(sr_ctx* ctx, const void* logits, int dtype, int logits_on_device, int32_t rows, int32_t vocab,
+                   int64_t row_stride_elems, int32_t* out_idx, float* out_val)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0) return SR_OK;
+    if (!out_idx) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_argmax_rows: out_idx is null");
+    if (rows < 0 || vocab < 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_argmax_rows: bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    const void* dev = logits;
+    if (vocab > 0) {
+        if (!logits) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_argmax_rows: logits is null");
+        int rc = stage_logits(ctx, logits, dtype, logits_on_device, rows, vocab, row_stride_elems, &dev);
+        if (rc != SR_OK) return rc;
+    }
+    SR_HIP(ctx, ctx->out_tokens.reserve((size_t)rows * sizeof(int32_t), ctx->stream));
+    SR_HIP(ctx, ctx->out_val.reserve((size_t)rows * sizeof(float), ctx->stream));
+    int rc = sr_argmax_rows_launch(ctx, dev, dtype, rows, vocab, row_stride_elems, ctx->out_tokens.as<int32_t>(),
+                                   ctx->out_val.as<float>());
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, hipMemcpyAsync(out_idx, ctx->out_tokens.p, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
+    if (out_val)
+        SR_HIP(ctx, hipMemcpyAsync(out_val, ctx->out_val.p, (size_t)rows * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return SR_OK;
+}
+
+int sr_pack_allow_mask(const float* masked_logits, int32_t vocab, uint32_t* out_words)
+{
+    if (!masked_logits || !out_words) return SR_ERR_NULL_ARGUMENT;
+    if (vocab < 0) return SR_ERR_INVALID_ARGUMENT;
+    const int32_t nw = (vocab + 31) / 32;
+    for (int32_t w = 0; w < nw; w++) {
+        uint32_t bits = 0;
+        const int32_t base = w * 32, n = std::min(32, vocab - base);
+        for (int32_t i = 0; i < n; i++) {
+            uint32_t u;
+            memcpy(&u, &masked_logits[base + i], 4);
+            if (u != 0xff800000u) bits |= 1u << i;
+        }
+        out_words[w] = bits;
+    }
+    return SR_OK;
+}
+
+// Test hook (not part of the public header): y[i] = the device expf for x[i], device pointers.
+SR_API int sr_selftest_expf(sr_ctx* ctx, const float* x_dev, float* y_dev, int64_t n)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    SR_HIP(ctx, sr_launch_selftest_expf(x_dev, y_dev, n, ctx->stream));
+    return SR_OK;
+}
+
+}  // extern "C"

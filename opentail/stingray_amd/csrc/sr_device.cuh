@@ -1,0 +1,121 @@
+// Device helpers shared by the kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define SR_WAVE 64
+#define SR_NEG_INF (__uint_as_float(0xff800000u))
+
+__device__ __forceinline__ uint32_t sr_f2u(float f) { return __float_as_uint(f); }
+__device__ __forceinline__ float sr_u2f(uint32_t u) { return __uint_as_float(u); }
+
+// Order-preserving map float -> uint32 (larger float = larger key).  -0 is folded onto +0 so that
+// key equality is float equality; NaN handling is the caller's business.
+__device__ __forceinline__ uint32_t sr_okey(float v)
+{
+    uint32_t b = sr_f2u(v);
+    if (b == 0x80000000u) b = 0u;
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float sr_okey_inv(uint32_t k)
+{
+    uint32_t b = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    return sr_u2f(b);
+}
+
+__device__ __forceinline__ float sr_bf16_to_f32(uint16_t h) { return sr_u2f(((uint32_t)h) << 16); }
+
+// glibc expf (2^(i/32) table, cubic in double, one rounding to float) with the FMA contractions of the
+// x86-64 -mfma build: the managed sampler's MathF.Exp on Linux.  Every operation is spelled with an
+// explicitly rounded intrinsic so the compiler can neither fuse nor reorder.
+__device__ static const uint64_t sr_exp2f_tab[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
+};
+
+__device__ __forceinline__ float sr_expf(float x)
+{
+    const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
+    const double shift = 0x1.8p+52;
+    const double c0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
+    const double c1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
+    const double c2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+    uint32_t xb = sr_f2u(x);
+    uint32_t abstop = (xb >> 20) & 0x7ffu;
+    if (abstop >= (0x42b00000u >> 20)) {
+        if (xb == 0xff800000u) return 0.0f;
+        if (abstop >= (0x7f800000u >> 20)) return __fadd_rn(x, x);
+        if (x > 0x1.62e42ep6f) return sr_u2f(0x7f800000u);
+        if (x < -0x1.9fe368p6f) return 0.0f;
+    }
+    double xd = (double)x;
+    double z = __dmul_rn(inv_ln2_n, xd);
+    double kd = __dadd_rn(z, shift);
+    uint64_t ki = (uint64_t)__double_as_longlong(kd);
+    kd = __dsub_rn(kd, shift);
+    double r = __fma_rn(inv_ln2_n, xd, -kd);
+    uint64_t t = sr_exp2f_tab[ki & 31u];
+    t += ki << (52 - 5);
+    double s = __longlong_as_double((long long)t);
+    double zz = __fma_rn(c0, r, c1);
+    double r2 = __dmul_rn(r, r);
+    double y = __fma_rn(c2, r, 1.0);
+    y = __fma_rn(zz, r2, y);
+    y = __dmul_rn(y, s);
+    return __double2float_rn(y);
+}
+
+// ---- wave / block primitives --------------------------------------------------------------------
+__device__ __forceinline__ int sr_lane() { return (int)(threadIdx.x & (SR_WAVE - 1)); }
+__device__ __forceinline__ int sr_wave_id() { return (int)(threadIdx.x >> 6); }
+
+__device__ __forceinline__ uint32_t sr_wave_max_u32(uint32_t v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { uint32_t w = __shfl_xor(v, o); v = w > v ? w : v; }
+    return v;
+}
+__device__ __forceinline__ uint32_t sr_wave_min_u32(uint32_t v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { uint32_t w = __shfl_xor(v, o); v = w < v ? w : v; }
+    return v;
+}
+__device__ __forceinline__ int sr_wave_sum_i32(int v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ int sr_wave_min_i32(int v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { int w = __shfl_xor(v, o); v = w < v ? w : v; }
+    return v;
+}
+__device__ __forceinline__ unsigned long long sr_wave_max_u64(unsigned long long v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        unsigned long long w = __shfl_xor(v, o);
+        v = w > v ? w : v;
+    }
+    return v;
+}
+// inclusive prefix sum across the wave
+__device__ __forceinline__ int sr_wave_incl_scan_i32(int v)
+{
+    const int lane = sr_lane();
+#pragma unroll
+    for (int o = 1; o < SR_WAVE; o <<= 1) {
+        int w = __shfl_up(v, o);
+        if (lane >= o) v += w;
+    }
+    return v;
+}

@@ -1,0 +1,90 @@
+// Host-side state shared by the translation units behind the C ABI.
+#pragma once
+#include "../../../include/stingray_sampler.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "sr_kernels.h"
+#include "sr_types.h"
+
+struct DeviceBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+    // Grows (never shrinks).  zero_new clears a newly allocated buffer on `stream`.
+    hipError_t reserve(size_t bytes, hipStream_t stream, bool zero_new = false)
+    {
+        if (bytes <= cap) return hipSuccess;
+        if (p) {
+            hipError_t e = hipStreamSynchronize(stream);
+            if (e != hipSuccess) return e;
+            (void)hipFree(p);
+            p = nullptr;
+            cap = 0;
+        }
+        size_t want = std::max(bytes, (size_t)256);
+        hipError_t e = hipMalloc(&p, want);
+        if (e != hipSuccess) { p = nullptr; return e; }
+        cap = want;
+        if (zero_new) return hipMemsetAsync(p, 0, want, stream);
+        return hipSuccess;
+    }
+    void release()
+    {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+    template <typename T> T* as() const { return (T*)p; }
+};
+
+struct sr_ctx {
+    int device = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    std::string err;
+    int cu_count = 256;
+    // scratch, lazily grown and reused across calls
+    DeviceBuf cand_val, cand_idx, cand_cnt, row_done, argmax_best;
+    DeviceBuf work;          // fp32 rows of the full-vocabulary path
+    DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
+    DeviceBuf host_logits;   // staging for host-resident logits
+    DeviceBuf out_tokens, out_flags, out_val, uniforms_tmp;
+    sr_batch* tmp_batch = nullptr;
+};
+
+struct sr_batch {
+    sr_ctx* ctx = nullptr;
+    int32_t rows = 0, vocab = 0, upr = 0;
+    std::vector<SrRow> h_rows;
+    std::vector<SrEdit> h_edits;
+    std::vector<int32_t> h_sel_list;   // rows on the selection kernel: TOPK and plain GREEDY
+    std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path (FULL and GREEDY_PEN)
+    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_mask, d_uniforms;
+    int64_t mask_stride = 0;
+    bool has_mask = false;
+    int32_t max_sel = 0;
+};
+
+inline int sr_fail(sr_ctx* ctx, int code, const std::string& msg)
+{
+    if (ctx) ctx->err = msg;
+    return code;
+}
+inline int sr_fail_hip(sr_ctx* ctx, hipError_t e, const char* what)
+{
+    return sr_fail(ctx, SR_ERR_HIP, std::string(what) + " failed: " + hipGetErrorString(e));
+}
+#define SR_HIP(ctx, call)                                             \
+    do {                                                              \
+        hipError_t _e = (call);                                       \
+        if (_e != hipSuccess) return sr_fail_hip((ctx), _e, #call);   \
+    } while (0)
+
+// Full-vocabulary rows of a batch (sr_full.cpp).  mode: 0 = sample, 1 = build distribution,
+// 2 = build distribution and sample from it.
+int sr_full_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
+                        int32_t* out_tokens_dev, uint32_t* out_flags_dev);

@@ -1,0 +1,49 @@
+// Structures shared by the host packer and the kernels.
+#pragma once
+#include <stdint.h>
+
+// How a row is dispatched; mirrors Sampler.Sample (Sampler.cs:17-39 of the reference engine).
+enum SrPath : int32_t {
+    SR_PATH_GREEDY = 0,      // Temperature <= 0, no history penalty      -> Greedy(masked logits)
+    SR_PATH_GREEDY_PEN = 1,  // Temperature <= 0 with history penalties   -> GreedyWithHistoryPenalties
+    SR_PATH_TOPK = 2,        // 0 < TopK < vocab and no logit bias        -> SampleTopK
+    SR_PATH_FULL = 3         // everything else                           -> full-vocabulary pipeline
+};
+
+struct SrRow {
+    float temperature;
+    float top_p;
+    float min_p;
+    float rep;
+    float presence;
+    float frequency;
+    float p_min;
+    int32_t top_k;
+    int32_t sel;        // TOPK: min(vocab, k + history length when penalties apply); GREEDY: 1
+    int32_t path;       // SrPath
+    int32_t edit_off;   // first SrEdit of this row
+    int32_t edit_cnt;
+    int32_t mask_row;   // row index into the allow-mask array, or -1
+    int32_t n_prev;
+    uint32_t flags;     // SR_ROW_* from the public header
+    int32_t pad;
+};
+
+// One distinct in-range token id that the row's history or logit bias touches; sorted by id per row.
+struct SrEdit {
+    int32_t id;
+    float bias;         // LogitBias value (applied first); valid when has_bias
+    int32_t occ_win;    // occurrences inside the trailing repetition window
+    int32_t occ_all;    // occurrences in the whole history
+    float pen;          // powf(repetition_penalty, occ_win), computed with the host libm (1 when unused)
+    uint32_t has_bias;
+};
+
+// Limits of the top-k selection kernel.
+#define SR_TK_THREADS 512
+#define SR_TK_VEC 19                       // 16-byte vectors held per thread
+#define SR_TK_GROUPS 4                     // group maxima per thread
+#define SR_TK_M (SR_TK_THREADS * SR_TK_GROUPS)
+#define SR_TK_CAP 3072                     // candidates one chunk may emit
+#define SR_TK_SEL_MAX 2048                 // largest k + history handled by the selection kernel
+#define SR_TK_SORT_CAP 4096                // candidates the row tail can sort

@@ -1,0 +1,48 @@
+"""Shared test plumbing: SamplingParams -> oracle parameters, oracle row loops."""
+from __future__ import annotations
+
+import numpy as np
+
+from oracle import binding as orc
+from opentail.stingray_amd import SamplingParams
+
+
+def to_oracle(p: SamplingParams) -> orc.Params:
+    return orc.Params(temperature=p.Temperature, top_k=p.TopK, top_p=p.TopP, min_p=p.MinP,
+                      repetition_penalty=p.RepetitionPenalty, repeat_last_n=p.RepeatLastN,
+                      presence_penalty=p.PresencePenalty, frequency_penalty=p.FrequencyPenalty,
+                      previous_tokens=p.PreviousTokens, logit_bias=p.LogitBias,
+                      spec_draft_p_min=p.SpecDraftPMin)
+
+
+def oracle_tokens(logits: np.ndarray, params, uniforms, allow_mask=None, mask_active=None) -> np.ndarray:
+    return orc.sample_batch(np.ascontiguousarray(logits, dtype=np.float32), [to_oracle(p) for p in params],
+                            np.asarray(uniforms, dtype=np.float64).reshape(len(params), -1)[:, 0].copy(),
+                            allow_mask, mask_active)
+
+
+class ReplayRandom:
+    """Stands in for System.Random: hands out the given NextDouble() values and counts the draws."""
+
+    def __init__(self, values):
+        self.values = list(values)
+        self.draws = 0
+
+    def NextDouble(self) -> float:
+        v = self.values[self.draws] if self.draws < len(self.values) else 0.0
+        self.draws += 1
+        return v
+
+
+class DotnetRandom:
+    """System.Random(seed) through the oracle's restatement of the runtime's generator."""
+
+    def __init__(self, seed: int):
+        self._r = orc.Rng(seed=seed)
+
+    def NextDouble(self) -> float:
+        return self._r.next_double()
+
+    @property
+    def draws(self) -> int:
+        return self._r.draws

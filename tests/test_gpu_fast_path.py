@@ -1,0 +1,226 @@
+"""GPU parity, through the C ABI: device expf, row argmax, greedy rows and the top-k-first path
+(Sampler.cs:216-357) against the CPU oracle.  Token ids must be bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import binding as orc
+from opentail.stingray_amd import Sampler, SamplerContext, SamplingParams, pack_allow_mask, synthetic
+from tests.helpers import DotnetRandom, ReplayRandom, oracle_tokens
+
+pytestmark = pytest.mark.gpu
+NEG_INF = np.float32("-inf")
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = SamplerContext(0)
+    yield c
+    c.close()
+
+
+def _cuda(a, dtype=None):
+    import torch
+
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.view(dtype)
+    return t.cuda()
+
+
+def test_device_expf_is_bit_identical_to_the_oracle(ctx):
+    import torch
+
+    rng = np.random.default_rng(1)
+    xs = np.concatenate([
+        -rng.exponential(6.0, 1_500_000), rng.uniform(-104.5, 0.0, 400_000), rng.uniform(0.0, 88.9, 100_000),
+        [0.0, -0.0, -87.9, -88.0, -103.0, -103.97, -103.98, -104.0, -1e-10, -1e-38, 88.7, 88.73, -np.inf, np.inf],
+    ]).astype(np.float32)
+    x = _cuda(xs)
+    y = torch.empty_like(x)
+    ctx._check(ctx.L.sr_selftest_expf(ctx.h, C.c_void_p(x.data_ptr()), C.c_void_p(y.data_ptr()), xs.size))
+    ctx.synchronize()
+    got = y.cpu().numpy()
+    lib = orc.lib()
+    want = np.array([lib.oracle_expf(C.c_float(v)) for v in xs[:300_000]], dtype=np.float32)
+    assert np.array_equal(got[:300_000].view(np.uint32), want.view(np.uint32))
+    tail = np.array([lib.oracle_expf(C.c_float(v)) for v in xs[-200_000:]], dtype=np.float32)
+    assert np.array_equal(got[-200_000:].view(np.uint32), tail.view(np.uint32))
+
+
+def test_argmax_matrix(ctx):
+    # CudaGpuArgmaxParityTests.cs:56-124: sizes across block boundaries and real vocabularies, maximum
+    # at {0, n/2, n-1}, tie -> lower index, all-equal -> 0, all-negative; value returned bit-identical.
+    for n in [1, 2, 3, 255, 256, 257, 1000, 65536, 152064, 262144]:
+        r = np.random.default_rng(1234 + n)
+        a = (r.random(n) * 20 - 10).astype(np.float32)
+        rows = [a]
+        for pos in (0, n // 2, n - 1):
+            b = a.copy()
+            b[pos] = 1000.0 + pos
+            rows.append(b)
+        m = np.stack(rows)
+        idx, val = ctx.argmax_rows(_cuda(m))
+        for i, row in enumerate(m):
+            assert idx[i] == orc.greedy(row)
+            assert val[i].tobytes() == row[idx[i]].tobytes()
+    a = np.full(5000, -1, dtype=np.float32)
+    a[700] = a[300] = 5
+    assert ctx.argmax_rows(_cuda(a[None]))[0][0] == 300
+    assert ctx.argmax_rows(_cuda(np.full((1, 8192), 3.5, np.float32)))[0][0] == 0
+    neg = (-np.random.default_rng(99).random(4096) * 50 - 1).astype(np.float32)
+    assert ctx.argmax_rows(_cuda(neg[None]))[0][0] == orc.greedy(neg)
+    assert ctx.argmax_rows(_cuda(np.full((1, 64), NEG_INF, np.float32)))[0][0] == 0
+
+
+def test_argmax_rows_batched_with_ties_and_bf16(ctx):
+    import torch
+
+    # CudaGpuArgmaxParityTests.cs:145-173
+    for vocab in (1024, 152064):
+        for rows in (1, 2, 4, 8):
+            r = np.random.default_rng(555 + rows * 31 + vocab)
+            flat = (r.random((rows, vocab)) * 10 - 5).astype(np.float32)
+            for i in range(rows):
+                pos = (i * 37) % vocab
+                flat[i, pos] = 50.0 + i
+                flat[i, (pos + 50) % vocab] = 50.0 + i
+            idx, val = ctx.argmax_rows(_cuda(flat))
+            for i in range(rows):
+                assert idx[i] == orc.greedy(flat[i]) and val[i] == flat[i, idx[i]]
+    bits = synthetic.to_bf16_bits(np.random.default_rng(3).normal(0, 2, (5, 3001)).astype(np.float32))
+    up = synthetic.bf16_bits_to_f32(bits)
+    idx, val = ctx.argmax_rows(_cuda(bits.view(np.int16), torch.bfloat16))
+    for i in range(5):
+        assert idx[i] == orc.greedy(up[i]) and val[i] == up[i, idx[i]]
+
+
+def test_reference_known_answers_through_the_sampler_mirror():
+    # SamplerTests.cs restated against the GPU path (any-uniform answers).
+    assert Sampler.Greedy([1, 5, 3, 2]) == 1 and Sampler.Greedy([10, 1, 2, 3]) == 0 and Sampler.Greedy([1, 2, 3, 100]) == 3
+    assert Sampler.Greedy([]) == 0
+    rng = ReplayRandom([0.3])
+    assert Sampler.Sample([1, 5, 3, 2], SamplingParams(Temperature=0.0), rng) == 1 and rng.draws == 0
+    logits = [10, 9.8, 0]
+    pres = SamplingParams(TopK=1, PresencePenalty=1.0, PreviousTokens=[0])
+    freq = SamplingParams(TopK=1, FrequencyPenalty=0.6, PreviousTokens=[0, 0])
+    for u in (0.0, 0.4, 0.999999):
+        assert Sampler.Sample(logits, pres, ReplayRandom([u])) == 1
+        assert Sampler.Sample(logits, freq, ReplayRandom([u])) == 1
+    # top-k 2 -> only {8, 9}; masks never sampled; all -inf -> index 0 with no draw
+    r = DotnetRandom(42)
+    seen = {Sampler.Sample(list(range(1, 11)), SamplingParams(TopK=2), r) for _ in range(200)}
+    assert seen <= {8, 9} and len(seen) == 2
+    masked = [2, NEG_INF, 5, NEG_INF, 1, 3]
+    r = DotnetRandom(3)
+    for _ in range(200):
+        assert masked[Sampler.Sample(masked, SamplingParams(TopK=5, TopP=0.95), r)] != NEG_INF
+    rr = ReplayRandom([0.5])
+    assert Sampler.Sample([NEG_INF] * 3, SamplingParams(TopK=2, TopP=0.9), rr) == 0
+    r = DotnetRandom(2)
+    assert {Sampler.Sample([6, 3, 2.5, 0, 0, 0, 0, 0], SamplingParams(TopK=3, TopP=0.5), r) for _ in range(100)} == {0}
+    # penalty over-selection (SamplerTests.cs:258-294)
+    p = SamplingParams(TopK=2, RepetitionPenalty=4.0, PreviousTokens=[1])
+    r = DotnetRandom(5)
+    reach = {Sampler.Sample([10, 8, 7, 1, 0], p, r) for _ in range(300)}
+    assert 1 not in reach and reach <= {0, 2} and 2 in reach
+
+
+def _check_rows(ctx, logits_f32, params, uniforms, device_tensor, allow_mask=None, mask_active=None):
+    got, flags = ctx.sample_batch(device_tensor, params, uniforms, allow_mask, mask_active, return_flags=True)
+    want = oracle_tokens(logits_f32, params, uniforms, allow_mask, mask_active)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, f"rows {bad[:8]} differ: gpu {got[bad[:8]]} oracle {want[bad[:8]]} flags {flags[bad[:8]]}"
+    return flags
+
+
+def test_small_rows_with_ties_masks_and_every_cut(ctx):
+    rng = np.random.default_rng(21)
+    for trial in range(40):
+        rows = int(rng.integers(1, 9))
+        n = int(rng.integers(2, 700))
+        logits = (rng.integers(-14, 14, (rows, n)) / 2.0).astype(np.float32)   # coarse grid: many ties
+        logits[rng.random((rows, n)) < 0.15] = NEG_INF
+        params = []
+        for _ in range(rows):
+            hist = rng.integers(-3, n + 3, int(rng.integers(0, 12))).tolist()
+            params.append(SamplingParams(
+                Temperature=float(rng.choice([0.0, 0.5, 1.0, 1.7])), TopK=int(rng.integers(1, n)),
+                TopP=float(rng.choice([1.0, 0.9, 0.5])), MinP=float(rng.choice([0.0, 0.05, 0.3])),
+                RepetitionPenalty=float(rng.choice([1.0, 1.3])), PresencePenalty=float(rng.choice([0.0, 0.4])),
+                FrequencyPenalty=float(rng.choice([0.0, 0.25])), RepeatLastN=int(rng.choice([0, 3, 64])),
+                PreviousTokens=hist))
+        # greedy rows with penalties go down the full-vocabulary path, covered by its own tests
+        for p in params:
+            if p.Temperature == 0.0:
+                p.PreviousTokens = None
+        _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits))
+
+
+def test_constant_and_quantised_rows(ctx):
+    # all-equal rows make every element tie with the threshold: lowest indices must win
+    V = 50_000
+    logits = np.zeros((3, V), dtype=np.float32)
+    logits[1] = 2.5
+    logits[2, ::7] = 1.0
+    params = [SamplingParams(TopK=50, TopP=0.9), SamplingParams(Temperature=0.0), SamplingParams(TopK=300, Temperature=0.7)]
+    for u in (0.0, 0.37, 0.93):
+        _check_rows(ctx, logits, params, [u, u, u], _cuda(logits))
+
+
+def test_config1_shape_many_steps(ctx):
+    w = synthetic.config1(steps=200)
+    flags = _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits))
+    assert np.all(flags & 2)   # every row took the top-k-first path
+
+
+def test_config3_shape_fp32_and_bf16(ctx):
+    import torch
+
+    w = synthetic.config3(rows=48, bf16=True)
+    _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits_bf16.view(np.int16), torch.bfloat16))
+    w = synthetic.config3(rows=48, bf16=False)
+    _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits))
+
+
+def test_config3_full_chain_with_penalties(ctx):
+    w = synthetic.config3(rows=48, bf16=False, full_chain=True)
+    _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits))
+
+
+def test_top_k_under_an_allow_mask_and_unaligned_rows(ctx):
+    import torch
+
+    rng = np.random.default_rng(8)
+    V = 30_011                                            # odd vocabulary: rows are not 16-byte aligned
+    logits = rng.normal(0, 1.5, (6, V)).astype(np.float32)
+    allowed = np.stack([synthetic.run_mask(rng, V, d) for d in (0.001, 0.01, 0.1, 0.5, 0.9, 0.0005)])
+    params = [SamplingParams(Temperature=0.9, TopK=int(k), TopP=0.95) for k in (1, 5, 40, 400, 1000, 64)]
+    params[2].Temperature = 0.0
+    mask = pack_allow_mask(allowed)
+    active = np.array([1, 1, 1, 1, 0, 1], dtype=np.uint8)
+    _check_rows(ctx, logits, params, rng.random(6), _cuda(logits), mask, active)
+    # a strided view: row stride larger than the vocabulary
+    big = torch.zeros((6, V + 37), dtype=torch.float32, device="cuda")
+    big[:, :V] = _cuda(logits)
+    _check_rows(ctx, logits, params, rng.random(6), big[:, :V], mask, active)
+
+
+def test_round_trip_properties_at_full_size(ctx):
+    # size-independent properties at the benchmark shape: every token is inside its row's top-k set and,
+    # for greedy rows, is the row argmax; re-running with the same uniforms is deterministic.
+    import torch
+
+    w = synthetic.config3(rows=256, bf16=False)
+    x = _cuda(w.logits)
+    t1 = ctx.sample_batch(x, w.params, w.uniforms)
+    t2 = ctx.sample_batch(x, w.params, w.uniforms)
+    assert np.array_equal(t1, t2)
+    kth = torch.topk(x, 1000, dim=1).values.cpu().numpy()
+    am, _ = ctx.argmax_rows(x)
+    for i, p in enumerate(w.params):
+        if p.Temperature <= 0:
+            assert t1[i] == am[i]
+        else:
+            assert w.logits[i, t1[i]] >= kth[i, p.TopK - 1]
