@@ -285,6 +285,13 @@ class SamplerContext:
             self.h = C.c_void_p()
 
     @staticmethod
+    def _row_stride(t) -> int:
+        """Row stride in elements; a single-row tensor may carry a meaningless stride."""
+        rows, vocab = t.shape[0], t.shape[-1]
+        assert t.stride(-1) == 1 or vocab <= 1, "rows must be contiguous"
+        return t.stride(0) if rows > 1 else max(int(t.stride(0)), vocab)
+
+    @staticmethod
     def _dtype_of(t) -> int:
         import torch
 
@@ -299,7 +306,7 @@ class SamplerContext:
         """Async: logits [rows, vocab] CUDA tensor (row stride in elements), outputs CUDA int32."""
         assert logits.is_cuda and out_tokens.is_cuda
         self._check(self.L.sr_sample_launch(
-            self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), logits.stride(0),
+            self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), self._row_stride(logits),
             C.c_void_p(out_tokens.data_ptr()), C.c_void_p(out_flags.data_ptr() if out_flags is not None else 0)))
 
     def sample_batch(self, logits, params: Sequence[SamplingParams], uniforms, allow_mask=None, mask_active=None,
@@ -328,7 +335,7 @@ class SamplerContext:
         val = torch.empty(rows, dtype=torch.float32, device=logits.device)
         self._check(self.L.sr_argmax_rows_launch(
             self.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), rows, vocab,
-            logits.stride(0) if rows > 0 and vocab > 0 else vocab, C.c_void_p(idx.data_ptr()), C.c_void_p(val.data_ptr())))
+            self._row_stride(logits) if rows > 0 and vocab > 0 else vocab, C.c_void_p(idx.data_ptr()), C.c_void_p(val.data_ptr())))
         self.synchronize()
         return idx.cpu().numpy(), val.cpu().numpy()
 
@@ -342,8 +349,8 @@ class SamplerContext:
         out = torch.zeros((rows, n), dtype=torch.float32, device=logits.device)
         try:
             self._check(self.L.sr_build_distribution_launch(
-                self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), logits.stride(0),
-                C.c_void_p(out.data_ptr()), out.stride(0), n))
+                self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), self._row_stride(logits),
+                C.c_void_p(out.data_ptr()), self._row_stride(out), n))
             self.synchronize()
         finally:
             batch.close()
@@ -358,8 +365,8 @@ class SamplerContext:
         toks = torch.empty(rows, dtype=torch.int32, device=logits.device)
         try:
             self._check(self.L.sr_sample_with_distribution_launch(
-                self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), logits.stride(0),
-                C.c_void_p(out.data_ptr()), out.stride(0), vocab, C.c_void_p(toks.data_ptr())))
+                self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), self._row_stride(logits),
+                C.c_void_p(out.data_ptr()), self._row_stride(out), vocab, C.c_void_p(toks.data_ptr())))
             self.synchronize()
         finally:
             batch.close()
@@ -372,7 +379,7 @@ class SamplerContext:
         u = None if uniforms is None else np.ascontiguousarray(np.asarray(uniforms, dtype=np.float64))
         toks = torch.empty(rows, dtype=torch.int32, device=probs.device)
         self._check(self.L.sr_sample_from_probs_launch(
-            self.h, C.c_void_p(probs.data_ptr()), rows, vocab, probs.stride(0), _ptr(u, C.c_double),
+            self.h, C.c_void_p(probs.data_ptr()), rows, vocab, self._row_stride(probs), _ptr(u, C.c_double),
             C.c_void_p(toks.data_ptr())))
         self.synchronize()
         return toks.cpu().numpy()
@@ -384,8 +391,8 @@ class SamplerContext:
         u = None if uniforms is None else np.ascontiguousarray(np.asarray(uniforms, dtype=np.float64))
         toks = torch.empty(rows, dtype=torch.int32, device=p.device)
         self._check(self.L.sr_resample_residual_launch(
-            self.h, C.c_void_p(p.data_ptr()), p.shape[1], p.stride(0), C.c_void_p(q.data_ptr()), q.shape[1],
-            q.stride(0), rows, _ptr(u, C.c_double), C.c_void_p(toks.data_ptr())))
+            self.h, C.c_void_p(p.data_ptr()), p.shape[1], self._row_stride(p), C.c_void_p(q.data_ptr()), q.shape[1],
+            self._row_stride(q), rows, _ptr(u, C.c_double), C.c_void_p(toks.data_ptr())))
         self.synchronize()
         return toks.cpu().numpy()
 
@@ -416,7 +423,7 @@ class SamplerContext:
         ok = torch.empty(rows, dtype=torch.int32, device=logits.device)
         pr = torch.empty(rows, dtype=torch.float32, device=logits.device)
         self._check(self.L.sr_mtp_verify_launch(
-            self.h, C.c_void_p(logits.data_ptr()), rows, vocab, logits.stride(0),
+            self.h, C.c_void_p(logits.data_ptr()), rows, vocab, self._row_stride(logits),
             C.c_void_p(draft_tokens.data_ptr()), p_min, C.c_void_p(am.data_ptr()), C.c_void_p(ok.data_ptr()),
             C.c_void_p(pr.data_ptr())))
         self.synchronize()

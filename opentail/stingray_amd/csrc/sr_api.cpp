@@ -232,7 +232,15 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
             }
             d.edit_cnt = (int32_t)ed.size() - d.edit_off;
         }
-        if (d.path == SR_PATH_TOPK || d.path == SR_PATH_GREEDY) {
+        if (d.path == SR_PATH_GREEDY_PEN) {
+            // over-select by the number of distinct history ids: one candidate outside the history
+            // is then guaranteed (see the row tail of the selection kernel)
+            d.sel = (int32_t)std::min<int64_t>((int64_t)d.edit_cnt + 1, vocab);
+        }
+        const bool on_selection_kernel =
+            d.path == SR_PATH_TOPK || d.path == SR_PATH_GREEDY ||
+            (d.path == SR_PATH_GREEDY_PEN && d.sel <= SR_TK_SEL_MAX);
+        if (on_selection_kernel) {
             b->h_sel_list.push_back(r);
             b->max_sel = std::max(b->max_sel, d.sel);
         } else {

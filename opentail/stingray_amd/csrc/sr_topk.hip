@@ -168,7 +168,7 @@ template <> struct VecOps<8> {  // eight bf16 per 16-byte vector; the upcast to 
     static __device__ __forceinline__ u32x4 neg_inf() { return (u32x4)(0xff80ff80u); }
 };
 
-__device__ __forceinline__ bool mask_bit(const uint32_t* m, int e) { return (m[e >> 5] >> (e & 31)) & 1u; }
+__device__ __forceinline__ bool mask_bit(const uint32_t* m, int e) { return ((m[e >> 5] >> (e & 31)) & 1u) != 0u; }
 
 // ---- the row tail ----------------------------------------------------------------------------------
 // Called by every thread of the last workgroup of a row.  slot = position of the row in this launch.
@@ -265,6 +265,60 @@ __device__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRo
     __syncthreads();
     block_bitonic_sort_desc(sm.sortbuf, P);
 
+    if (rd.path == SR_PATH_GREEDY_PEN) {
+        // GreedyWithHistoryPenalties (Sampler.cs:421-437): only the history ids change value, so the
+        // argmax is the better of (a) the best adjusted history id and (b) the best raw candidate that is
+        // not a history id -- one exists among the top (distinct ids + 1) candidates.
+        const SrEdit* ed = a.edits + rd.edit_off;
+        const int ne = rd.edit_cnt;
+        unsigned long long best = 0ull;
+        int first_free = 0x7fffffff;
+        for (int t = tid; t < m; t += kThreads) {
+            int id = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[t] & 0xffffffffull));
+            int lo = 0, hi = ne;
+            while (lo < hi) {
+                int mid = (lo + hi) >> 1;
+                if (ed[mid].id < id) lo = mid + 1; else hi = mid;
+            }
+            if (!(lo < ne && ed[lo].id == id)) { first_free = t; break; }
+        }
+        const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * (a.dtype == 1 ? 2 : 4);
+        const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+        for (int e = tid; e < ne; e += kThreads) {
+            const int id = ed[e].id;
+            float x = (a.dtype == 1) ? sr_bf16_to_f32(((const uint16_t*)rowp)[id]) : ((const float*)rowp)[id];
+            if (mrow && !mask_bit(mrow, id)) x = SR_NEG_INF;
+            if (rd.rep != 1.0f)
+                for (int o = 0; o < ed[e].occ_win; o++) x = x > 0.0f ? __fdiv_rn(x, rd.rep) : __fmul_rn(x, rd.rep);
+            if (rd.presence != 0.0f || rd.frequency != 0.0f)
+                x = __fsub_rn(x, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ed[e].occ_all)));
+            if (sr_f2u(x) != 0xff800000u && x == x) {
+                unsigned long long c = ((unsigned long long)sr_okey(x) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
+                best = c > best ? c : best;
+            }
+        }
+        first_free = sr_wave_min_i32(first_free);
+        best = sr_wave_max_u64(best);
+        __syncthreads();
+        if (sr_lane() == 0) {
+            sm.red[sr_wave_id()] = (uint32_t)first_free;
+            ((unsigned long long*)sm.vals)[sr_wave_id()] = best;  // vals is unused on this path
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int ff = 0x7fffffff;
+            for (int w = 0; w < kWaves; w++) {
+                ff = min(ff, (int)sm.red[w]);
+                unsigned long long c = ((unsigned long long*)sm.vals)[w];
+                best = c > best ? c : best;
+            }
+            if (ff != 0x7fffffff && sm.sortbuf[ff] > best) best = sm.sortbuf[ff];
+            // nothing finite at all: every adjusted logit is -inf and the first index wins
+            a.out_tokens[row] = best ? (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull)) : 0;
+            if (a.out_flags) a.out_flags[row] = out_flag | (best ? 0u : SR_KFLAG_DEGENERATE);
+        }
+        return;
+    }
     if (rd.path == SR_PATH_GREEDY) {
         if (tid == 0) {
             a.out_tokens[row] = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[0] & 0xffffffffull));
@@ -436,46 +490,64 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             int f = j * kThreads + tid;
             v[j] = (f < nvec) ? __builtin_nontemporal_load(&wp[f]) : VO::neg_inf();
         }
-        // edges of the window and the allow-mask
+        // edges of the window and the allow-mask: one keep-bit per element of the vector
+        const int mask_words = (int)a.mask_stride;
 #pragma unroll
         for (int j = 0; j < kVec; j++) {
-            int f = j * kThreads + tid;
-            if (f >= nvec) continue;
-            int e0 = wbase + f * EPV;
-            bool edge = (e0 < lo) || (e0 + EPV > hi);
-            if (edge) {
+            const int f = j * kThreads + tid;
+            if (f < nvec) {
+                const int e0 = wbase + f * EPV;
+                uint32_t keep = (1u << EPV) - 1u;
+                if (e0 < lo || e0 + EPV > hi) {
 #pragma unroll
-                for (int q = 0; q < EPV; q++) {
-                    int e = e0 + q;
-                    if (e < lo || e >= hi || (mrow && !mask_bit(mrow, e))) VO::kill(v[j], q);
+                    for (int q = 0; q < EPV; q++)
+                        if (e0 + q < lo || e0 + q >= hi) keep &= ~(1u << q);
                 }
-            } else if (mrow) {
-                int wi = e0 >> 5, sh = e0 & 31;
-                unsigned long long bits = mrow[wi];
-                if (sh + EPV > 32) bits |= (unsigned long long)mrow[wi + 1] << 32;
-                uint32_t nib = (uint32_t)(bits >> sh);
+                if (mrow) {
+                    const int es = e0 < 0 ? 0 : e0;       // first bit that exists
+                    const int wi = es >> 5, sh = es & 31;
+                    unsigned long long bits = mrow[wi];
+                    if (wi + 1 < mask_words) bits |= (unsigned long long)mrow[wi + 1] << 32;
+                    keep &= (uint32_t)(bits >> sh) << (es - e0);
+                }
+                if (keep != (1u << EPV) - 1u) {
 #pragma unroll
-                for (int q = 0; q < EPV; q++)
-                    if (!((nib >> q) & 1u)) VO::kill(v[j], q);
+                    for (int q = 0; q < EPV; q++)
+                        if (!((keep >> q) & 1u)) VO::kill(v[j], q);
+                }
             }
         }
 
-        // group maxima -> keys
-        uint32_t gk[SR_TK_GROUPS];
+        // A safe lower bound on the chunk's sel-th largest element.
+        uint32_t tkey;
+        if (nvec <= 4 * kThreads) {
+            // short chunk (at most four vectors per thread): select exactly over its elements
+            auto each_elem = [&](auto&& body) {
 #pragma unroll
-        for (int g = 0; g < SR_TK_GROUPS; g++) {
-            float mxv = SR_NEG_INF;
+                for (int j = 0; j < 4; j++)
 #pragma unroll
-            for (int j = g * 5; j < (g == SR_TK_GROUPS - 1 ? kVec : g * 5 + 5); j++)
+                    for (int q = 0; q < EPV; q++) body(sr_okey(VO::get(v[j], q)));
+            };
+            tkey = block_radix_select(each_elem, sel, sm);
+        } else {
+            // every thread owns four interleaved groups of vectors (j mod 4), all populated here; the
+            // sel-th largest of the 2048 disjoint-group maxima cannot exceed the sel-th largest element
+            uint32_t gk[SR_TK_GROUPS];
 #pragma unroll
-                for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, VO::get(v[j], q));
-            gk[g] = sr_okey(mxv);
+            for (int g = 0; g < SR_TK_GROUPS; g++) {
+                float mxv = SR_NEG_INF;
+#pragma unroll
+                for (int j = g; j < kVec; j += SR_TK_GROUPS)
+#pragma unroll
+                    for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, VO::get(v[j], q));
+                gk[g] = sr_okey(mxv);
+            }
+            auto each_gk = [&](auto&& body) {
+#pragma unroll
+                for (int g = 0; g < SR_TK_GROUPS; g++) body(gk[g]);
+            };
+            tkey = (sel > SR_TK_M) ? 0u : block_radix_select(each_gk, sel, sm);
         }
-        auto each_gk = [&](auto&& body) {
-#pragma unroll
-            for (int g = 0; g < SR_TK_GROUPS; g++) body(gk[g]);
-        };
-        uint32_t tkey = (sel > SR_TK_M) ? 0u : block_radix_select(each_gk, sel, sm);
         // -inf never enters the candidate set (Sampler.cs:240-249: strict v <= -inf rejects it)
         const float tval = (tkey <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(tkey);
 
