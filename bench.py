@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X token-sampling path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+One "step" = one batched sampling call (sr_sample_launch / sr_spec_verify_launch) over a batch of
+seeded synthetic logits that are already resident in HBM.  Four distinct logits buffers are rotated so
+every step streams cold data (4 x 155.6 MB exceeds the 256 MB Infinity Cache).  Prints ONE JSON line.
+
+Workloads (opentail/stingray_amd/synthetic.py):
+  c3_fp32_full  (default) batch 256 x vocab 151,936 fp32, heterogeneous top-k U{1..1000} / top-p / T,
+                10% greedy rows, plus min-p and repetition/presence/frequency penalties over a 64-token
+                history: the "full chain" the throughput target is quoted on.
+  c3_bf16       the same rows stored as bf16, no penalties (configuration 3 as written)
+  c3_fp32       fp32, no penalties
+  c1            batch 1 x vocab 49,152 (us/step is the figure of interest)
+  c2, c4        full-vocabulary path (batch 64 / batch 32 with allow-masks)
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+def make_workload(name: str):
+    from opentail.stingray_amd import synthetic
+
+    if name == "c3_fp32_full":
+        return synthetic.config3(rows=256, bf16=False, full_chain=True)
+    if name == "c3_fp32":
+        return synthetic.config3(rows=256, bf16=False)
+    if name == "c3_bf16":
+        return synthetic.config3(rows=256, bf16=True)
+    if name == "c1":
+        return synthetic.config1(steps=1)
+    if name == "c2":
+        return synthetic.config2()
+    if name == "c4":
+        return synthetic.config4()
+    raise SystemExit(f"unknown workload {name}")
+
+
+def cpu_baseline(w, budget_s: float):
+    """The CPU oracle (a port of the reference sampler) on one core, rows in order, same inputs."""
+    from oracle import binding as orc
+    from tests.helpers import to_oracle
+
+    params = [to_oracle(p) for p in w.params]
+    u = np.asarray(w.uniforms, dtype=np.float64).reshape(w.rows, -1)[:, 0].copy()
+    orc.sample_batch(w.logits[:2], params[:2], u[:2],
+                     None if w.allow_mask is None else w.allow_mask[:2],
+                     None if w.mask_active is None else w.mask_active[:2])  # warm-up
+    done = 0
+    t0 = time.perf_counter()
+    passes = 0
+    while True:
+        orc.sample_batch(w.logits, params, u, w.allow_mask, w.mask_active)
+        done += w.rows
+        passes += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or passes >= 50:
+            break
+    return done / el, done, el
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c3_fp32_full")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget (0 = skip)")
+    ap.add_argument("--no-parity", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on one GPU (rows shard across GPUs without any exchange); "
+                         "run with --gpus 1")
+
+    import torch
+
+    from opentail.stingray_amd import SamplerContext
+    from oracle import binding as orc  # checker + CPU baseline only
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU: the sampler has no CPU path")
+    torch.cuda.set_device(0)
+    w = make_workload(args.workload)
+    rows, vocab = w.rows, w.vocab
+    stream = torch.cuda.Stream()            # a real (non-null) stream shared by torch and the library,
+    torch.cuda.set_stream(stream)           # so HIP events recorded here bracket the sampler's kernels
+    ctx = SamplerContext(0)
+
+    # four distinct resident logits buffers (row-rotated copies of the seeded tensor) + their batches
+    n_buf = 4
+    bufs, batches, host_logits = [], [], []
+    for i in range(n_buf):
+        sh = (i * 7) % rows
+        lg = np.roll(w.logits, sh, axis=0)
+        host_logits.append(lg)
+        if w.logits_bf16 is not None:
+            t = torch.from_numpy(np.roll(w.logits_bf16, sh, axis=0).view(np.int16)).view(torch.bfloat16).cuda()
+        else:
+            t = torch.from_numpy(lg).cuda()
+        bufs.append(t)
+        batches.append(ctx.new_batch().upload(w.params, vocab, w.uniforms, w.allow_mask, w.mask_active))
+    toks = [torch.full((rows,), -7, dtype=torch.int32, device="cuda") for _ in range(n_buf)]
+    flags = [torch.zeros(rows, dtype=torch.int32, device="cuda") for _ in range(n_buf)]
+
+    def step(i):
+        b = i % n_buf
+        ctx.sample_launch(batches[b], bufs[b], toks[b], flags[b])
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for i in range(args.steps):
+        step(i)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = ev0.elapsed_time(ev1)
+    ms_per_step = wall * 1e3 / args.steps
+    kern_us = dev_ms * 1e3 / args.steps  # device time per launch from HIP events on the launch stream
+
+    # parity of the measured outputs against the oracle (outside the timed region)
+    parity = None
+    if not args.no_parity:
+        from tests.helpers import oracle_tokens
+
+        n_chk = min(rows, 24)
+        got = toks[0].cpu().numpy()[:n_chk]
+        want = oracle_tokens(host_logits[0][:n_chk], w.params[:n_chk], np.asarray(w.uniforms)[:n_chk],
+                             None if w.allow_mask is None else w.allow_mask[:n_chk],
+                             None if w.mask_active is None else w.mask_active[:n_chk])
+        parity = {"rows_checked": int(n_chk), "mismatches": int((got != want).sum())}
+    unsupported = int(sum(int((f.cpu().numpy().view(np.uint32) >> 31).sum()) for f in flags))
+
+    elem = 2 if w.logits_bf16 is not None else 4
+    alg_bytes = rows * vocab * elem + (0 if w.allow_mask is None else w.allow_mask.nbytes) + rows * 8
+    achieved = alg_bytes / (kern_us * 1e-6) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", f"traffic_{args.workload}.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+
+    cpu = None
+    if args.cpu_seconds > 0:
+        tps, n_done, el = cpu_baseline(w, args.cpu_seconds)
+        cpu = {"value": tps, "unit": "tokens/s", "cores": 1, "kind": "port",
+               "sample": f"{n_done} rows of the same workload ({args.workload}), rows in order on one thread, "
+                         f"{el:.1f} s; oracle = C port of the reference sampler (no .NET runtime on this box)"}
+
+    out = {
+        "metric": "sampled tokens/sec at B=256x152k vocab" if rows == 256 else f"sampled tokens/sec at B={rows}x{vocab} vocab",
+        "value": rows * args.steps / wall,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "us_per_step_device": kern_us,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if elem == 4 else "bf16->f32",
+        "data": "synthetic (seeded Gaussian + Zipf-head logits, 4 rotated resident buffers)",
+        "config": {"workload": args.workload, "rows": rows, "vocab": vocab,
+                   "chain": "penalties+top-k+top-p+min-p" if args.workload == "c3_fp32_full" else args.workload},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "algorithmic_bytes_per_launch": alg_bytes, "kernel": "k_topk_rows",
+                     "kernel_us": kern_us},
+        "cpu_baseline": cpu,
+        "parity": parity,
+        "rows_unsupported": unsupported,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

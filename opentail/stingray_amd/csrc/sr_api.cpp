@@ -16,19 +16,23 @@ inline bool has_history_penalty(const sr_row_params& p)
 }
 
 // Chunking of a row for the selection kernel: every chunk must fit the per-workgroup register window.
-void topk_geometry(int vocab, int dtype, int n_rows, int cu_count, int* chunks, int* chunk_len)
+void topk_geometry(int vocab, int dtype, int n_rows, int max_sel, int cu_count, int* chunks, int* chunk_len)
 {
     const int epv = dtype == SR_DTYPE_BF16 ? 8 : 4;
     const int window = SR_TK_VEC * SR_TK_THREADS * epv;
     const int usable = window - epv;  // slack for a misaligned row start
     int s_min = (vocab + usable - 1) / usable;
     int s_par = (2 * cu_count + n_rows - 1) / std::max(n_rows, 1);  // aim for two workgroups per CU
-    int s_cap = std::max(1, vocab / 2048);
+    int s_cap = std::min(SR_TK_MAX_CHUNKS, std::max(1, vocab / 2048));
+    // every chunk hands at most min(chunk, 2 * sel + 128) candidates to the row tail, which holds
+    // SR_TK_TAIL_CAP of them
+    s_cap = std::min(s_cap, std::max(1, SR_TK_TAIL_CAP / (2 * max_sel + 128)));
     int s = std::max(s_min, std::min(s_par, s_cap));
     int len = (vocab + s - 1) / s;
     len = (len + 7) & ~7;
     if (len > usable) len = usable & ~7;
     s = (vocab + len - 1) / len;
+    // a row too long for SR_TK_MAX_CHUNKS register windows cannot be handled by the selection kernel
     *chunks = std::max(s, 1);
     *chunk_len = std::max(len, 8);
 }
@@ -248,6 +252,12 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         }
     }
 
+    // Rows with the longest tails (largest top_k + history) go first, so that their sequential tails
+    // overlap the streaming of the rows behind them and only short tails are left at the end.
+    std::stable_sort(b->h_sel_list.begin(), b->h_sel_list.end(), [&](int32_t x, int32_t y) {
+        return b->h_rows[(size_t)x].sel > b->h_rows[(size_t)y].sel;
+    });
+
     auto up = [&](DeviceBuf& dst, const void* src, size_t bytes) -> hipError_t {
         if (bytes == 0) return hipSuccess;
         hipError_t e = dst.reserve(bytes, st);
@@ -305,7 +315,9 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.row_stride = row_stride_elems;
         a.vocab = b->vocab;
         a.dtype = dtype;
-        topk_geometry(b->vocab, dtype, n_sel, ctx->cu_count, &a.chunks, &a.chunk_len);
+        topk_geometry(b->vocab, dtype, n_sel, b->max_sel, ctx->cu_count, &a.chunks, &a.chunk_len);
+        if ((int64_t)a.chunks * std::min(a.chunk_len, 2 * b->max_sel + 128) > SR_TK_TAIL_CAP || a.chunks > SR_TK_MAX_CHUNKS)
+            return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary x (top_k + history) too large for the selection kernel");
         const size_t slots = (size_t)n_sel * a.chunks;
         SR_HIP(ctx, ctx->cand_val.reserve(slots * SR_TK_CAP * sizeof(float), st));
         SR_HIP(ctx, ctx->cand_idx.reserve(slots * SR_TK_CAP * sizeof(int32_t), st));
@@ -324,6 +336,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.uniforms_per_row = b->upr;
         a.out_tokens = out_tokens_dev;
         a.out_flags = out_flags_dev;
+        a.prof = ctx->prof;
         SR_HIP(ctx, sr_launch_topk(a, n_sel, st));
     }
     if (!b->h_full_list.empty()) {
@@ -451,6 +464,14 @@ int sr_pack_allow_mask(const float* masked_logits, int32_t vocab, uint32_t* out_
         }
         out_words[w] = bits;
     }
+    return SR_OK;
+}
+
+// Test hook: phase timestamps (wall_clock64, 100 MHz) of the selection kernel go to prof_dev[grid][16].
+SR_API int sr_debug_set_profile(sr_ctx* ctx, unsigned long long* prof_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    ctx->prof = prof_dev;
     return SR_OK;
 }
 

@@ -71,6 +71,21 @@ __device__ __forceinline__ float sr_expf(float x)
     return __double2float_rn(y);
 }
 
+// ---- cross-workgroup hand-off without a full L2 write-back ----------------------------------------
+// Data one workgroup leaves for another (possibly on another XCD) is written with agent-scope stores
+// (write-through past the XCD-private L2) and read back with agent-scope loads; the writer drains its
+// own stores (s_waitcnt) before the workgroup barrier that precedes the hand-off counter.  A release
+// fence would instead write back every dirty line of the L2.
+template <typename T> __device__ __forceinline__ void sr_store_agent(T* p, T v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T> __device__ __forceinline__ T sr_load_agent(const T* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void sr_drain_stores() { __builtin_amdgcn_s_waitcnt(0); }
+
 // ---- wave / block primitives --------------------------------------------------------------------
 __device__ __forceinline__ int sr_lane() { return (int)(threadIdx.x & (SR_WAVE - 1)); }
 __device__ __forceinline__ int sr_wave_id() { return (int)(threadIdx.x >> 6); }

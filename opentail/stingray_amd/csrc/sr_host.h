@@ -54,6 +54,7 @@ struct sr_ctx {
     DeviceBuf host_logits;   // staging for host-resident logits
     DeviceBuf out_tokens, out_flags, out_val, uniforms_tmp;
     sr_batch* tmp_batch = nullptr;
+    unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
 };
 
 struct sr_batch {

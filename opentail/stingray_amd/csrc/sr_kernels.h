@@ -33,6 +33,7 @@ struct SrTopkArgs {
     int32_t uniforms_per_row;
     int32_t* out_tokens;
     uint32_t* out_flags;     // may be null
+    unsigned long long* prof; // optional phase timestamps [grid][16] (test hook), normally null
 };
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream);
 

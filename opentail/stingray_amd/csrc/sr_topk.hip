@@ -13,30 +13,39 @@
 
 namespace {
 
+#define SR_PROF(a, slot_) do { if ((a).prof && threadIdx.x == 0) (a).prof[(size_t)blockIdx.x * 16 + (slot_)] = (unsigned long long)wall_clock64(); } while (0)
+
 constexpr int kThreads = SR_TK_THREADS;
 constexpr int kWaves = kThreads / SR_WAVE;
 constexpr int kVec = SR_TK_VEC;
 constexpr int kCap = SR_TK_CAP;
-constexpr int kSortCap = SR_TK_SORT_CAP;
 constexpr int kSelMax = SR_TK_SEL_MAX;
 constexpr uint32_t kKeyNegInf = 0x007fffffu;  // sr_okey(-inf)
 constexpr uint32_t kRowHasPenalty = SR_ROWFLAG_HAS_PENALTY;
 
+constexpr int kCandRegs = 32;                   // candidate keys a thread holds in the row tail
+constexpr int kCandMax = kCandRegs * kThreads;  // 16384 merged candidates per row
+constexpr int kMaxChunks = SR_TK_MAX_CHUNKS;
+constexpr int kSortRegs = kSelMax / kThreads;   // 4 sort elements per thread
+
 struct TopkSmem {
-    unsigned long long sortbuf[kSortCap];
+    uint32_t xa[kSelMax];  // gathered list, then sort exchange (three 32-bit words per element)
+    uint32_t xb[kSelMax];
+    uint32_t xc[kSelMax];
     float vals[kSelMax];
     int idxs[kSelMax];
-    float probs[kSelMax];
+    __attribute__((aligned(16))) float probs[kSelMax + 8];
     uint32_t hist[256];
     uint32_t red[2 * kWaves];
-    uint32_t bcast[8];
+    uint32_t bcast[16];
+    int offs[kMaxChunks + 1];
 };
 
 // ---- block-wide radix select over keys produced by a per-thread enumerator -----------------------
 // Returns the need-th largest key (1-based) among all keys every thread enumerates.  Keys equal to 0
 // act as "absent".  Must be called by all threads of the block.
 template <typename ForEach>
-__device__ uint32_t block_radix_select(ForEach for_each_key, int need, TopkSmem& sm)
+__device__ __forceinline__ uint32_t block_radix_select(ForEach for_each_key, int need, TopkSmem& sm)
 {
     const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
     uint32_t lmax = 0u, lmin = 0xffffffffu;
@@ -101,32 +110,6 @@ __device__ uint32_t block_radix_select(ForEach for_each_key, int need, TopkSmem&
     return prefix;
 }
 
-// ---- bitonic sort, descending, of sm.sortbuf[0 .. n_pow2) ----------------------------------------
-__device__ void block_bitonic_sort_desc(unsigned long long* s, int n_pow2)
-{
-    const int tid = threadIdx.x;
-    for (int k2 = 2; k2 <= n_pow2; k2 <<= 1) {
-        for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
-            for (int i = tid; i < n_pow2; i += kThreads) {
-                int ixj = i ^ j2;
-                if (ixj > i) {
-                    unsigned long long a = s[i], b = s[ixj];
-                    bool desc_block = ((i & k2) == 0);
-                    if ((a < b) == desc_block) { s[i] = b; s[ixj] = a; }
-                }
-            }
-            __syncthreads();
-        }
-    }
-}
-
-__device__ __forceinline__ int next_pow2(int n)
-{
-    int p = 1;
-    while (p < n) p <<= 1;
-    return p;
-}
-
 // ---- block-wide exclusive scan of one int per thread; returns the exclusive prefix, total in *tot ---
 __device__ __forceinline__ int block_excl_scan(int v, int* tot, TopkSmem& sm)
 {
@@ -170,117 +153,241 @@ template <> struct VecOps<8> {  // eight bf16 per 16-byte vector; the upcast to 
 
 __device__ __forceinline__ bool mask_bit(const uint32_t* m, int e) { return ((m[e >> 5] >> (e & 31)) & 1u) != 0u; }
 
+// ---- bitonic sort, descending, of 3-word keys held in registers -----------------------------------
+// Element i lives in thread (i mod 512), register (i div 512).  Strides of 512 and more pair registers
+// of one thread, strides below 64 pair lanes of one wave (shuffles), only the strides in between go
+// through LDS.  n_pow2 <= 2048.  Keys are compared as (hi, mid, lo).
+__device__ __forceinline__ bool key3_less(uint32_t ah, uint32_t am, uint32_t al, uint32_t bh, uint32_t bm, uint32_t bl)
+{
+    return ah < bh || (ah == bh && (am < bm || (am == bm && al < bl)));
+}
+
+template <bool kThree>
+__device__ __forceinline__ void block_bitonic_sort_desc(uint32_t (&hi)[kSortRegs], uint32_t (&mid)[kSortRegs],
+                                                        uint32_t (&lo)[kSortRegs], int n_pow2, TopkSmem& sm)
+{
+    const int tid = threadIdx.x;
+    auto less = [&](uint32_t ah, uint32_t am, uint32_t al, uint32_t bh, uint32_t bm, uint32_t bl) -> bool {
+        if (kThree) return key3_less(ah, am, al, bh, bm, bl);
+        return ah < bh || (ah == bh && al < bl);
+    };
+    auto cx = [&](int r0, int r1, int k2) {  // compare-exchange two registers of this thread (r0 < r1)
+        const bool desc = (((r0 * kThreads + tid) & k2) == 0);
+        const bool l = less(hi[r0], mid[r0], lo[r0], hi[r1], mid[r1], lo[r1]);
+        if (l == desc) {
+            uint32_t t;
+            t = hi[r0]; hi[r0] = hi[r1]; hi[r1] = t;
+            if (kThree) { t = mid[r0]; mid[r0] = mid[r1]; mid[r1] = t; }
+            t = lo[r0]; lo[r0] = lo[r1]; lo[r1] = t;
+        }
+    };
+    const int regs = (n_pow2 + kThreads - 1) / kThreads;  // registers that hold real elements
+    for (int k2 = 2; k2 <= n_pow2; k2 <<= 1) {
+        for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
+            if (j2 == 2 * kThreads) {
+                cx(0, 2, k2); cx(1, 3, k2);
+            } else if (j2 == kThreads) {
+                cx(0, 1, k2);
+                if (regs > 2) cx(2, 3, k2);
+            } else if (j2 >= SR_WAVE) {
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < kSortRegs; r++) {
+                    if (r < regs) {
+                        const int i = r * kThreads + tid;
+                        sm.xa[i] = hi[r];
+                        if (kThree) sm.xb[i] = mid[r];
+                        sm.xc[i] = lo[r];
+                    }
+                }
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < kSortRegs; r++) {
+                    const int i = r * kThreads + tid;
+                    if (r < regs && i < n_pow2) {
+                        const int pi = i ^ j2;
+                        const uint32_t ph = sm.xa[pi], pm = kThree ? sm.xb[pi] : 0u, pl = sm.xc[pi];
+                        const bool want_max = (((i & k2) == 0) == ((i & j2) == 0));
+                        const bool l = less(hi[r], mid[r], lo[r], ph, pm, pl);
+                        if (want_max == l) { hi[r] = ph; if (kThree) mid[r] = pm; lo[r] = pl; }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < kSortRegs; r++) {
+                    if (r < regs) {
+                        const int i = r * kThreads + tid;
+                        const uint32_t ph = __shfl_xor(hi[r], j2), pm = kThree ? __shfl_xor(mid[r], j2) : 0u,
+                                       pl = __shfl_xor(lo[r], j2);
+                        const bool want_max = (((i & k2) == 0) == ((i & j2) == 0));
+                        const bool l = less(hi[r], mid[r], lo[r], ph, pm, pl);
+                        if (want_max == l) { hi[r] = ph; if (kThree) mid[r] = pm; lo[r] = pl; }
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ int next_pow2(int n)
+{
+    int p = 1;
+    while (p < n) p <<= 1;
+    return p;
+}
+
+// block-wide reductions through sm.red (all threads must call)
+__device__ __forceinline__ int block_sum_i32(int v, TopkSmem& sm)
+{
+    v = sr_wave_sum_i32(v);
+    __syncthreads();
+    if (sr_lane() == 0) sm.red[sr_wave_id()] = (uint32_t)v;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) t += (int)sm.red[w];
+    return t;
+}
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t v, TopkSmem& sm)
+{
+    v = sr_wave_max_u32(v);
+    __syncthreads();
+    if (sr_lane() == 0) sm.red[sr_wave_id()] = v;
+    __syncthreads();
+    uint32_t t = 0u;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) t = sm.red[w] > t ? sm.red[w] : t;
+    return t;
+}
+__device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
+{
+    v = sr_wave_min_i32(v);
+    __syncthreads();
+    if (sr_lane() == 0) sm.red[sr_wave_id()] = (uint32_t)v;
+    __syncthreads();
+    int t = 0x7fffffff;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) t = min(t, (int)sm.red[w]);
+    return t;
+}
+
 // ---- the row tail ----------------------------------------------------------------------------------
 // Called by every thread of the last workgroup of a row.  slot = position of the row in this launch.
-__device__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, TopkSmem& sm)
+// The merged candidates are read once, straight into registers; every later pass runs from registers
+// or LDS.
+__device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, TopkSmem& sm)
 {
     const int tid = threadIdx.x;
     const int S = a.chunks;
     const float* cval = a.cand_val + (size_t)slot * S * kCap;
     const int* cidx = a.cand_idx + (size_t)slot * S * kCap;
     const int* ccnt = a.cand_cnt + (size_t)slot * S;
-
-    uint32_t out_flag = (rd.path == SR_PATH_TOPK) ? SR_KFLAG_TOPK : SR_KFLAG_GREEDY;
-    bool overflow = false;
-    int n_total = 0;
-    for (int c = 0; c < S; c++) {
-        int n = ccnt[c];
-        if (n > kCap) overflow = true;
-        n_total += n;
-    }
+    const uint32_t out_flag = (rd.path == SR_PATH_TOPK) ? SR_KFLAG_TOPK : SR_KFLAG_GREEDY;
     const int sel = rd.sel;
-    if (overflow || sel > kSelMax) {
+    auto give_up = [&](uint32_t extra, int token) {
         if (tid == 0) {
-            a.out_tokens[row] = -1;
-            if (a.out_flags) a.out_flags[row] = out_flag | SR_KFLAG_UNSUPPORTED;
-        }
-        return;
-    }
-    if (n_total == 0) {
-        // no finite logit anywhere: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
-        if (tid == 0) {
-            a.out_tokens[row] = 0;
-            if (a.out_flags) a.out_flags[row] = out_flag | SR_KFLAG_DEGENERATE;
-        }
-        return;
-    }
-
-    // exact key of the sel-th largest candidate
-    auto each_key = [&](auto&& body) {
-        for (int c = 0; c < S; c++) {
-            int n = ccnt[c];
-            const float* v = cval + (size_t)c * kCap;
-            for (int i = tid; i < n; i += kThreads) body(sr_okey(v[i]));
+            a.out_tokens[row] = token;
+            if (a.out_flags) a.out_flags[row] = out_flag | extra;
         }
     };
-    uint32_t tkey = (n_total <= sel) ? 0u : block_radix_select(each_key, sel, sm);
 
-    // How many candidates sit at or above that key?  With few ties they are all sorted; with many
-    // (quantised or constant rows) only the lowest-index ties that still fit into sel are kept.
-    int c_ge = 0, c_gt = 0;
-    each_key([&](uint32_t k) { c_ge += (k >= tkey) ? 1 : 0; c_gt += (k > tkey) ? 1 : 0; });
-    int m_ge, m_gt;
-    block_excl_scan(c_ge, &m_ge, sm);
-    block_excl_scan(c_gt, &m_gt, sm);
-    uint32_t tidx_key = 0u;  // ties need (0xffffffff - idx) >= tidx_key
-    if (m_ge > kSortCap) {
-        auto each_tie = [&](auto&& body) {
-            for (int c = 0; c < S; c++) {
-                int n = ccnt[c];
-                const float* v = cval + (size_t)c * kCap;
-                const int* ix = cidx + (size_t)c * kCap;
-                for (int i = tid; i < n; i += kThreads)
-                    if (sr_okey(v[i]) == tkey) body(0xffffffffu - (uint32_t)ix[i]);
-            }
-        };
-        tidx_key = block_radix_select(each_tie, sel - m_gt, sm);
+    // chunk counts -> exclusive offsets
+    if (tid < S) sm.offs[tid + 1] = sr_load_agent(&ccnt[tid]);
+    __syncthreads();
+    if (tid == 0) {
+        int acc = 0, mx = 0;
+        uint32_t ovf = 0u;
+        sm.offs[0] = 0;
+        for (int c = 0; c < S; c++) {
+            int n = sm.offs[c + 1];
+            if (n > kCap) ovf = 1u;
+            mx = max(mx, n);
+            acc += n;
+            sm.offs[c + 1] = acc;
+        }
+        sm.bcast[8] = ovf;
+        sm.bcast[9] = (uint32_t)mx;
     }
     __syncthreads();
-    if (tid == 0) sm.bcast[4] = 0u;
-    __syncthreads();
-    for (int c = 0; c < S; c++) {
-        int n = ccnt[c];
-        const float* v = cval + (size_t)c * kCap;
-        const int* ix = cidx + (size_t)c * kCap;
-        for (int i = tid; i < n; i += kThreads) {
-            uint32_t k = sr_okey(v[i]);
-            uint32_t ik = 0xffffffffu - (uint32_t)ix[i];
-            if (k > tkey || (k == tkey && ik >= tidx_key)) {
-                uint32_t pos = atomicAdd(&sm.bcast[4], 1u);
-                if (pos < (uint32_t)kSortCap) sm.sortbuf[pos] = ((unsigned long long)k << 32) | (unsigned long long)ik;
-            }
-        }
+    const int n_total = sm.offs[S];
+    if (sm.bcast[8] || sel > kSelMax || n_total > kCandMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
+    // no finite logit anywhere: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
+    if (n_total == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
+
+    SR_PROF(a, 11);
+    // flattened position g -> (chunk g / pitch, element g mod pitch), pitch a power of two >= the
+    // longest chunk list; the host sizes the chunking so that chunks x pitch fits the registers
+    const int pitch = next_pow2(max((int)sm.bcast[9], 1));
+    const int pshift = 31 - __clz(pitch);
+    if ((long long)pitch * S > kCandMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
+    auto cand_addr = [&](int r) -> int {  // index into cval / cidx of this thread's r-th candidate
+        const int g = r * kThreads + tid;
+        return (g >> pshift) * kCap + (g & (pitch - 1));
+    };
+    const int nr = (S * pitch + kThreads - 1) / kThreads;  // register slots that can hold a candidate
+    uint32_t kreg[kCandRegs];  // 0 = no candidate in this slot
+#pragma unroll
+    for (int r = 0; r < kCandRegs; r++) {
+        kreg[r] = 0u;
+        if (r >= nr) continue;
+        const int g = r * kThreads + tid;
+        const int c = g >> pshift, i = g & (pitch - 1);
+        const int cc = min(c, S - 1);
+        const bool ok = c < S && i < sm.offs[cc + 1] - sm.offs[cc];
+        kreg[r] = ok ? sr_okey(sr_load_agent(&cval[c * kCap + i])) : 0u;
     }
-    __syncthreads();
-    const int m = (int)sm.bcast[4];
-    if (m > kSortCap) {  // cannot happen: m <= max(sel, kSortCap); kept as a guard
-        if (tid == 0) {
-            a.out_tokens[row] = -1;
-            if (a.out_flags) a.out_flags[row] = out_flag | SR_KFLAG_UNSUPPORTED;
+    SR_PROF(a, 12);
+    auto each_key = [&](auto&& body) {
+#pragma unroll
+        for (int r = 0; r < kCandRegs; r++)
+            if (r < nr) body(kreg[r]);
+    };
+
+    // history / bias ids of the row, staged for binary search
+    const SrEdit* ed = a.edits + rd.edit_off;
+    const bool use_edits = (rd.flags & kRowHasPenalty) != 0u;
+    const int ne = use_edits ? rd.edit_cnt : 0;   // <= kSelMax - 1 on this kernel
+    int* edit_ids = sm.idxs;
+    if (use_edits)
+        for (int e = tid; e < ne; e += kThreads) edit_ids[e] = ed[e].id;
+    auto find_edit = [&](int id) -> int {
+        int lo = 0, hi = ne;
+        while (lo < hi) {
+            int mid = (lo + hi) >> 1;
+            if (edit_ids[mid] < id) lo = mid + 1; else hi = mid;
         }
+        return (lo < ne && edit_ids[lo] == id) ? lo : -1;
+    };
+
+    if (rd.path == SR_PATH_GREEDY) {
+        // argmax: highest key, lowest index among its ties
+        uint32_t kmax = 0u;
+        each_key([&](uint32_t k) { kmax = k > kmax ? k : kmax; });
+        kmax = block_max_u32(kmax, sm);
+        int best = 0x7fffffff;
+#pragma unroll
+        for (int r = 0; r < kCandRegs; r++)
+            if (kreg[r] == kmax && kreg[r] != 0u) best = min(best, sr_load_agent(&cidx[cand_addr(r)]));
+        best = block_min_i32(best, sm);
+        give_up(0u, best);
         return;
     }
-    int P = next_pow2(m < 2 ? 2 : m);
-    for (int i = m + tid; i < P; i += kThreads) sm.sortbuf[i] = 0ull;
-    __syncthreads();
-    block_bitonic_sort_desc(sm.sortbuf, P);
 
     if (rd.path == SR_PATH_GREEDY_PEN) {
         // GreedyWithHistoryPenalties (Sampler.cs:421-437): only the history ids change value, so the
-        // argmax is the better of (a) the best adjusted history id and (b) the best raw candidate that is
-        // not a history id -- one exists among the top (distinct ids + 1) candidates.
-        const SrEdit* ed = a.edits + rd.edit_off;
-        const int ne = rd.edit_cnt;
+        // argmax is the better of (a) the best adjusted history id and (b) the best raw candidate that
+        // is not a history id -- one exists among the top (distinct ids + 1) candidates.
+        __syncthreads();  // edit_ids staged
         unsigned long long best = 0ull;
-        int first_free = 0x7fffffff;
-        for (int t = tid; t < m; t += kThreads) {
-            int id = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[t] & 0xffffffffull));
-            int lo = 0, hi = ne;
-            while (lo < hi) {
-                int mid = (lo + hi) >> 1;
-                if (ed[mid].id < id) lo = mid + 1; else hi = mid;
+#pragma unroll
+        for (int r = 0; r < kCandRegs; r++) {
+            if (kreg[r] == 0u) continue;
+            const int id = sr_load_agent(&cidx[cand_addr(r)]);
+            if (find_edit(id) < 0) {
+                unsigned long long cmp = ((unsigned long long)kreg[r] << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
+                best = cmp > best ? cmp : best;
             }
-            if (!(lo < ne && ed[lo].id == id)) { first_free = t; break; }
         }
         const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * (a.dtype == 1 ? 2 : 4);
         const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
@@ -293,140 +400,194 @@ __device__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRo
             if (rd.presence != 0.0f || rd.frequency != 0.0f)
                 x = __fsub_rn(x, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ed[e].occ_all)));
             if (sr_f2u(x) != 0xff800000u && x == x) {
-                unsigned long long c = ((unsigned long long)sr_okey(x) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
-                best = c > best ? c : best;
+                unsigned long long cmp = ((unsigned long long)sr_okey(x) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
+                best = cmp > best ? cmp : best;
             }
         }
-        first_free = sr_wave_min_i32(first_free);
         best = sr_wave_max_u64(best);
         __syncthreads();
-        if (sr_lane() == 0) {
-            sm.red[sr_wave_id()] = (uint32_t)first_free;
-            ((unsigned long long*)sm.vals)[sr_wave_id()] = best;  // vals is unused on this path
-        }
+        if (sr_lane() == 0) ((unsigned long long*)sm.vals)[sr_wave_id()] = best;
         __syncthreads();
         if (tid == 0) {
-            int ff = 0x7fffffff;
             for (int w = 0; w < kWaves; w++) {
-                ff = min(ff, (int)sm.red[w]);
-                unsigned long long c = ((unsigned long long*)sm.vals)[w];
-                best = c > best ? c : best;
+                unsigned long long cmp = ((unsigned long long*)sm.vals)[w];
+                best = cmp > best ? cmp : best;
             }
-            if (ff != 0x7fffffff && sm.sortbuf[ff] > best) best = sm.sortbuf[ff];
             // nothing finite at all: every adjusted logit is -inf and the first index wins
             a.out_tokens[row] = best ? (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull)) : 0;
             if (a.out_flags) a.out_flags[row] = out_flag | (best ? 0u : SR_KFLAG_DEGENERATE);
         }
         return;
     }
-    if (rd.path == SR_PATH_GREEDY) {
-        if (tid == 0) {
-            a.out_tokens[row] = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[0] & 0xffffffffull));
-            if (a.out_flags) a.out_flags[row] = out_flag;
-        }
-        return;
-    }
 
-    // vals/idx: the sel best in (value desc, index asc) order; unfilled slots are (-inf, -1)
-    for (int t = tid; t < sel; t += kThreads) {
-        if (t < m) {
-            unsigned long long e = sm.sortbuf[t];
-            sm.vals[t] = sr_okey_inv((uint32_t)(e >> 32));
-            sm.idxs[t] = (int)(0xffffffffu - (uint32_t)(e & 0xffffffffull));
-        } else {
-            sm.vals[t] = SR_NEG_INF;
-            sm.idxs[t] = -1;
-        }
+    // ---- SampleTopK (Sampler.cs:216-357) ---------------------------------------------------------
+    // exact key of the sel-th largest candidate, then the set at or above it
+    const uint32_t tkey = (n_total <= sel) ? 0u : block_radix_select(each_key, sel, sm);
+    SR_PROF(a, 5);
+    int c_ge = 0, c_gt = 0;
+    each_key([&](uint32_t k) { c_ge += (k != 0u && k >= tkey) ? 1 : 0; c_gt += (k != 0u && k > tkey) ? 1 : 0; });
+    const int m_ge = block_sum_i32(c_ge, sm);
+    uint32_t tidx_key = 0u;  // ties additionally need (0xffffffff - idx) >= tidx_key
+    if (m_ge > kSelMax) {
+        // many candidates tie with the sel-th value (quantised or constant rows): equal values rank by
+        // ascending index, so only the (sel - #above) lowest-index ties belong to the set
+        const int m_gt = block_sum_i32(c_gt, sm);
+        uint32_t tie_key[kCandRegs];
+#pragma unroll
+        for (int r = 0; r < kCandRegs; r++)
+            tie_key[r] = (kreg[r] != 0u && kreg[r] == tkey) ? 0xffffffffu - (uint32_t)sr_load_agent(&cidx[cand_addr(r)]) : 0u;
+        auto each_tie = [&](auto&& body) {
+#pragma unroll
+            for (int r = 0; r < kCandRegs; r++) body(tie_key[r]);
+        };
+        tidx_key = block_radix_select(each_tie, sel - m_gt, sm);
     }
-    __syncthreads();
-
-    if (rd.flags & kRowHasPenalty) {
-        // Sampler.cs:261-294: pen = pow(rep, occWindow) once, presence/frequency over the whole
-        // history, then a stable re-sort by value.
-        const SrEdit* ed = a.edits + rd.edit_off;
-        const int ne = rd.edit_cnt;
-        for (int t = tid; t < sel; t += kThreads) {
-            int id = sm.idxs[t];
-            if (id < 0) continue;
-            int lo = 0, hi = ne;
-            while (lo < hi) {
-                int mid = (lo + hi) >> 1;
-                if (ed[mid].id < id) lo = mid + 1; else hi = mid;
+    // gather (key, idx) of the set into LDS: count, scan, then fetch the indices and write
+    auto in_set = [&](int r) -> bool {
+        if (kreg[r] == 0u || kreg[r] < tkey) return false;
+        if (kreg[r] > tkey || tidx_key == 0u) return true;
+        return (0xffffffffu - (uint32_t)sr_load_agent(&cidx[cand_addr(r)])) >= tidx_key;
+    };
+    int mine = 0;
+#pragma unroll
+    for (int r = 0; r < kCandRegs; r++)
+        if (r < nr) mine += in_set(r) ? 1 : 0;
+    int m;
+    int pos = block_excl_scan(mine, &m, sm);
+    if (mine > 0) {
+#pragma unroll
+        for (int r = 0; r < kCandRegs; r++)
+            if (r < nr && in_set(r) && pos < kSelMax) {
+                sm.xa[pos] = kreg[r];
+                sm.xb[pos] = (uint32_t)sr_load_agent(&cidx[cand_addr(r)]);
+                pos++;
             }
-            if (lo < ne && ed[lo].id == id && ed[lo].occ_all > 0) {
-                float v = sm.vals[t];
-                if (rd.rep != 1.0f && ed[lo].occ_win > 0) {
-                    float pen = ed[lo].pen;
-                    v = v > 0.0f ? __fdiv_rn(v, pen) : __fmul_rn(v, pen);
+    }
+    __syncthreads();  // also orders the staging of edit_ids
+    if (m > kSelMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }  // guard; m <= max(sel, kSelMax)
+    SR_PROF(a, 6);
+
+    // sort keys: (value after penalties, value before, ~index) descending -- the reference's selection
+    // order (value desc, index asc) followed by its stable re-sort after penalties, in one sort
+    uint32_t hi[kSortRegs], mid[kSortRegs], lo[kSortRegs];
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) {
+        const int i = r * kThreads + tid;
+        hi[r] = mid[r] = lo[r] = 0u;
+        if (i < m) {
+            const uint32_t key = sm.xa[i];
+            const int id = (int)sm.xb[i];
+            uint32_t nkey = key;
+            if (use_edits) {
+                // Sampler.cs:261-287: pen = pow(rep, occWindow) once; presence/frequency over the whole history
+                const int e = find_edit(id);
+                if (e >= 0) {
+                    const SrEdit ee = ed[e];
+                    if (ee.occ_all > 0) {
+                        float v = sr_okey_inv(key);
+                        if (rd.rep != 1.0f && ee.occ_win > 0) v = v > 0.0f ? __fdiv_rn(v, ee.pen) : __fmul_rn(v, ee.pen);
+                        v = __fsub_rn(v, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ee.occ_all)));
+                        nkey = sr_okey(v);
+                    }
                 }
-                float sub = __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ed[lo].occ_all));
-                sm.vals[t] = __fsub_rn(v, sub);
             }
+            hi[r] = nkey; mid[r] = key; lo[r] = 0xffffffffu - (uint32_t)id;
         }
-        __syncthreads();
-        int P2 = next_pow2(sel < 2 ? 2 : sel);
-        for (int t = tid; t < P2; t += kThreads)
-            sm.sortbuf[t] = (t < sel) ? (((unsigned long long)sr_okey(sm.vals[t]) << 32) |
-                                         (unsigned long long)(0xffffffffu - (uint32_t)t))
-                                      : 0ull;
-        __syncthreads();
-        block_bitonic_sort_desc(sm.sortbuf, P2);
-        // permute (value, idx) by the sorted ranks; read everything before anything is overwritten
-        float nv[kSelMax / kThreads];
-        int ni[kSelMax / kThreads];
-#pragma unroll
-        for (int q = 0; q < kSelMax / kThreads; q++) {
-            int t = tid + q * kThreads;
-            if (t < sel) {
-                unsigned long long e = sm.sortbuf[t];
-                int old = (int)(0xffffffffu - (uint32_t)(e & 0xffffffffull));
-                nv[q] = sm.vals[old];
-                ni[q] = sm.idxs[old];
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int q = 0; q < kSelMax / kThreads; q++) {
-            int t = tid + q * kThreads;
-            if (t < sel) { sm.vals[t] = nv[q]; sm.idxs[t] = ni[q]; }
-        }
-        __syncthreads();
     }
-
-    // Sampler.cs:297-349
-    const int k = rd.top_k;  // k <= sel
+    SR_PROF(a, 7);
+    // Candidates whose e = expf(v / T - max) is below 2^-26 are dropped before the sort: with e_0 = 1
+    // they change neither running sum (they are under half an ulp of a sum >= 1, and of a cumulative
+    // probability >= probs[0]) and the draw can never stop on them, so the result is bit-identical.
+    // x < -18.1 implies e < 1.4e-8 < 2^-26.
+    uint32_t lmaxk = 0u;
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) lmaxk = hi[r] > lmaxk ? hi[r] : lmaxk;
+    const uint32_t kmaxn = block_max_u32(lmaxk, sm);
     const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
-    const float mx = __fmul_rn(sm.vals[0], inv_temp);
-    for (int t = tid; t < k; t += kThreads) {
-        float v = sm.vals[t];
-        sm.probs[t] = (sr_f2u(v) == 0xff800000u) ? 0.0f : sr_expf(__fsub_rn(__fmul_rn(v, inv_temp), mx));
+    const float mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
+    int nlive = 0;
+    bool alive[kSortRegs];
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) {
+        const int i = r * kThreads + tid;
+        const float x = __fsub_rn(__fmul_rn(sr_okey_inv(hi[r]), inv_temp), mx);
+        alive[r] = (i < m) && !(x < -18.1f);
+        nlive += alive[r] ? 1 : 0;
+    }
+    int m2;
+    int lpos = block_excl_scan(nlive, &m2, sm);
+    if (m2 < m) {
+        // compact the live candidates (all threads have their elements in registers by now)
+#pragma unroll
+        for (int r = 0; r < kSortRegs; r++)
+            if (alive[r]) { sm.xa[lpos] = hi[r]; sm.xb[lpos] = mid[r]; sm.xc[lpos] = lo[r]; lpos++; }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kSortRegs; r++) {
+            const int i = r * kThreads + tid;
+            hi[r] = (i < m2) ? sm.xa[i] : 0u;
+            mid[r] = (i < m2) ? sm.xb[i] : 0u;
+            lo[r] = (i < m2) ? sm.xc[i] : 0u;
+        }
+    }
+    if (use_edits) block_bitonic_sort_desc<true>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
+    else block_bitonic_sort_desc<false>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
+
+    // the k best that are still alive
+    const int k = min(rd.top_k, m2);  // top_k <= sel; everything past m2 is a no-op or does not exist
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) {
+        const int i = r * kThreads + tid;
+        if (i < k) {
+            sm.vals[i] = sr_okey_inv(hi[r]);
+            sm.idxs[i] = (int)(0xffffffffu - lo[r]);
+        }
     }
     __syncthreads();
+    SR_PROF(a, 8);
+
+    // Sampler.cs:297-313: e_t = expf(v_t / T - max), sequential fp32 sum, probs = e * (1 / sum)
+    int live = 0;  // one past the last e_t that can still change a sum that is already >= 1
+    for (int t = tid; t < k; t += kThreads) {
+        const float v = sm.vals[t];
+        const float e = sr_expf(__fsub_rn(__fmul_rn(v, inv_temp), mx));
+        sm.probs[t] = e;
+        if (!(e < 5.9604644775390625e-08f)) live = t + 1;  // 2^-24: below half an ulp of any sum >= 1
+    }
+    if (tid < 8) sm.probs[k + tid] = 0.0f;
+    live = (int)block_max_u32((uint32_t)live, sm);
     if (tid == 0) {
+        // e_0 = expf(0) = 1, so from t = 1 on the running sum is >= 1 and terms below 2^-24 leave it
+        // unchanged: stopping at `live` gives the same bits as running to k
+        const int n = max(live, 1);
         float sum = 0.0f;
-        for (int t = 0; t < k; t++) sum = __fadd_rn(sum, sm.probs[t]);
+        const float4* p4 = (const float4*)sm.probs;
+        float4 cur = p4[0];
+        for (int t = 0; t < n; t += 4) {
+            const float4 nxt = p4[(t >> 2) + 1];
+            sum = __fadd_rn(sum, cur.x); sum = __fadd_rn(sum, cur.y);
+            sum = __fadd_rn(sum, cur.z); sum = __fadd_rn(sum, cur.w);
+            cur = nxt;
+        }
         sm.bcast[5] = sr_f2u(sum);
     }
     __syncthreads();
+    SR_PROF(a, 9);
     const float sum = sr_u2f(sm.bcast[5]);
     const float inv_sum = sum > 0.0f ? __fdiv_rn(1.0f, sum) : 0.0f;
     for (int t = tid; t < k; t += kThreads) sm.probs[t] = __fmul_rn(sm.probs[t], inv_sum);
     __syncthreads();
 
-    // min-p: first t with probs[t] < thr bounds the survivors
+    // Sampler.cs:315-324 min-p: the first probs[t] < thr bounds the survivors
     int count = k;
     if (rd.min_p > 0.0f) {
         const float thr = __fmul_rn(rd.min_p, sm.probs[0]);
         int first = k;
         for (int t = tid; t < k; t += kThreads)
             if (sm.probs[t] < thr) { first = t; break; }
-        first = sr_wave_min_i32(first);
-        __syncthreads();
-        if (sr_lane() == 0) sm.red[sr_wave_id()] = (uint32_t)first;
-        __syncthreads();
-        for (int w = 0; w < kWaves; w++) count = min(count, (int)sm.red[w]);
+        count = min(count, block_min_i32(first, sm));
     }
-    // running sum; probs[t] becomes cum[t].  top-p cuts after the first cum >= TopP.
+    // Sampler.cs:326-349: running sum (probs[t] becomes cum[t]); top-p cuts after the first cum >= TopP
     if (tid == 0) {
         const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
         float cum = 0.0f;
@@ -440,19 +601,15 @@ __device__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRo
     }
     __syncthreads();
     count = (int)sm.bcast[6];
+    SR_PROF(a, 10);
     const float kept_sum = count > 0 ? sm.probs[count - 1] : 0.0f;
     const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept_sum);
     int first = 0x7fffffff;
     for (int t = tid; t < count; t += kThreads)
         if (r <= sm.probs[t] && sm.idxs[t] >= 0) { first = t; break; }
-    first = sr_wave_min_i32(first);
-    __syncthreads();
-    if (sr_lane() == 0) sm.red[sr_wave_id()] = (uint32_t)first;
-    __syncthreads();
+    first = block_min_i32(first, sm);
     if (tid == 0) {
-        int best = 0x7fffffff;
-        for (int w = 0; w < kWaves; w++) best = min(best, (int)sm.red[w]);
-        a.out_tokens[row] = (best != 0x7fffffff) ? sm.idxs[best] : sm.idxs[0];
+        a.out_tokens[row] = (first != 0x7fffffff) ? sm.idxs[first] : sm.idxs[0];
         if (a.out_flags) a.out_flags[row] = out_flag;
     }
 }
@@ -473,6 +630,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     const int hi = min(V, lo + a.chunk_len);
     const int sel = rd.sel;
     int total = 0;
+    SR_PROF(a, 0);
 
     if (lo < hi && sel <= kSelMax) {
         constexpr int ES = (EPV == 4) ? 4 : 2;  // element size in bytes
@@ -490,6 +648,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             int f = j * kThreads + tid;
             v[j] = (f < nvec) ? __builtin_nontemporal_load(&wp[f]) : VO::neg_inf();
         }
+        SR_PROF(a, 1);
         // edges of the window and the allow-mask: one keep-bit per element of the vector
         const int mask_words = (int)a.mask_stride;
 #pragma unroll
@@ -548,6 +707,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             };
             tkey = (sel > SR_TK_M) ? 0u : block_radix_select(each_gk, sel, sm);
         }
+        SR_PROF(a, 2);
         // -inf never enters the candidate set (Sampler.cs:240-249: strict v <= -inf rejects it)
         const float tval = (tkey <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(tkey);
 
@@ -558,8 +718,10 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         for (int j = 0; j < kVec; j++)
 #pragma unroll
             for (int q = 0; q < EPV; q++) cnt += (VO::get(v[j], q) >= tval) ? 1 : 0;
+        // a chunk hands over at most `lim` candidates, so that the row tail can hold all chunks of a row
+        const int lim = min(kCap, 2 * sel + 128);
         int pos = block_excl_scan(cnt, &total, sm);
-        if (total <= kCap) {
+        if (total <= lim) {
             if (cnt > 0) {
 #pragma unroll
                 for (int j = 0; j < kVec; j++) {
@@ -567,7 +729,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                     for (int q = 0; q < EPV; q++) {
                         float x = VO::get(v[j], q);
-                        if (x >= tval) { cv[pos] = x; ci[pos] = e0 + q; pos++; }
+                        if (x >= tval) { sr_store_agent(&cv[pos], x); sr_store_agent(&ci[pos], e0 + q); pos++; }
                     }
                 }
             }
@@ -581,8 +743,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 for (int q = 0; q < EPV; q++) cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
             int total_gt;
             int pgt = block_excl_scan(cgt, &total_gt, sm);
-            if (total_gt > kCap) {
-                total = total_gt;  // genuine overflow: the row is reported as unsupported
+            if (total_gt > lim) {
+                total = kCap + 1;  // genuine overflow: the row is reported as unsupported
             } else {
                 if (cgt > 0) {
 #pragma unroll
@@ -591,11 +753,11 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                         for (int q = 0; q < EPV; q++) {
                             float x = VO::get(v[j], q);
-                            if (x > tval) { cv[pgt] = x; ci[pgt] = e0 + q; pgt++; }
+                            if (x > tval) { sr_store_agent(&cv[pgt], x); sr_store_agent(&ci[pgt], e0 + q); pgt++; }
                         }
                     }
                 }
-                const int need_eq = min(sel - total_gt, kCap - total_gt);
+                const int need_eq = min(sel - total_gt, lim - total_gt);
                 int emitted = 0;
                 if (need_eq > 0) {
 #pragma unroll
@@ -611,7 +773,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                             for (int q = 0; q < EPV; q++) {
                                 if (VO::get(v[j], q) == tval) {
-                                    if (rank < need_eq) { cv[total_gt + rank] = tval; ci[total_gt + rank] = e0 + q; }
+                                    if (rank < need_eq) { sr_store_agent(&cv[total_gt + rank], tval); sr_store_agent(&ci[total_gt + rank], e0 + q); }
                                     rank++;
                                 }
                             }
@@ -623,20 +785,22 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             }
         }
     }
-    if (tid == 0) a.cand_cnt[(size_t)slot * S + c] = total;
+    SR_PROF(a, 3);
+    if (tid == 0) sr_store_agent(&a.cand_cnt[(size_t)slot * S + c], total);
 
-    // publish, then let the last workgroup of the row run the tail
-    __threadfence();
+    // hand the chunk over: drain this wave's write-through stores, meet, then count the chunk in
+    sr_drain_stores();
     __syncthreads();
     if (tid == 0) {
-        uint32_t prev = atomicAdd(&a.row_done[slot], 1u);
+        uint32_t prev = __hip_atomic_fetch_add(&a.row_done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         sm.bcast[7] = (prev == (uint32_t)(S - 1)) ? 1u : 0u;
     }
     __syncthreads();
     if (!sm.bcast[7]) return;
-    __threadfence();
-    if (tid == 0) a.row_done[slot] = 0u;  // ready for the next launch
+    if (tid == 0) sr_store_agent(&a.row_done[slot], 0u);  // ready for the next launch
+    SR_PROF(a, 4);
     topk_row_tail(a, slot, row, rd, sm);
+    SR_PROF(a, 15);
 }
 
 }  // namespace

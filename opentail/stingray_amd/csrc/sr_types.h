@@ -46,4 +46,5 @@ struct SrEdit {
 #define SR_TK_M (SR_TK_THREADS * SR_TK_GROUPS)
 #define SR_TK_CAP 3072                     // candidates one chunk may emit
 #define SR_TK_SEL_MAX 2048                 // largest k + history handled by the selection kernel
-#define SR_TK_SORT_CAP 4096                // candidates the row tail can sort
+#define SR_TK_TAIL_CAP 16384                // merged candidates the row tail holds (32 per thread)
+#define SR_TK_MAX_CHUNKS 128               // most workgroups one row is split over
