@@ -1,0 +1,672 @@
+// Full-vocabulary sampling: the reference's slow path (Sampler.cs:41-95), BuildFilteredDistribution
+// (:118-163), GreedyWithHistoryPenalties (:421-437), SampleFromDistribution (:564-576) and
+// ResampleResidual (:587-618).
+//
+// The row is materialised in an fp32 work row exactly as the reference copies it, and every stage is
+// one pass of a 1024-thread workgroup over that row.  All running sums that the reference evaluates
+// left to right go through the exact evaluator in sr_seqsum.cuh, so probabilities, cut-offs and draws
+// carry the reference's bits.
+#include "sr_device.cuh"
+#include "sr_kernels.h"
+#include "sr_seqsum.cuh"
+#include "sr_types.h"
+
+namespace {
+
+constexpr int kT = SR_SEQ_THREADS;
+constexpr int kW = SR_SEQ_WAVES;
+constexpr int kSmall = SR_FULL_SMALL_CAP;  // survivors sorted inside the kernel
+
+struct FullSmem {
+    SrSeqSmem seq;
+    float redf[kW];
+    uint32_t redu[kW];
+    int redi[kW];
+    uint32_t hist[256];
+    uint32_t bc[16];
+    unsigned long long sortbuf[kSmall];
+    float sprob[kSmall];
+};
+
+// ---- block reductions ------------------------------------------------------------------------------
+__device__ __forceinline__ float blk_max_f(float v, bool* any_nan, FullSmem& sm)
+{
+    // NaN propagates (TensorPrimitives.Max)
+    uint32_t nanf = (v != v) ? 1u : 0u;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float w = __shfl_xor(v, o);
+        uint32_t wn = __shfl_xor(nanf, o);
+        v = fmaxf(v, w);
+        nanf |= wn;
+    }
+    __syncthreads();
+    if (sr_lane() == 0) { sm.redf[sr_wave_id()] = v; sm.redu[sr_wave_id()] = nanf; }
+    __syncthreads();
+    float m = sm.redf[0];
+    uint32_t n = sm.redu[0];
+#pragma unroll
+    for (int w = 1; w < kW; w++) { m = fmaxf(m, sm.redf[w]); n |= sm.redu[w]; }
+    *any_nan = n != 0u;
+    return m;
+}
+__device__ __forceinline__ int blk_sum_i(int v, FullSmem& sm)
+{
+    v = sr_wave_sum_i32(v);
+    __syncthreads();
+    if (sr_lane() == 0) sm.redi[sr_wave_id()] = v;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < kW; w++) t += sm.redi[w];
+    return t;
+}
+__device__ __forceinline__ unsigned long long blk_max_u64(unsigned long long v, FullSmem& sm)
+{
+    v = sr_wave_max_u64(v);
+    __syncthreads();
+    if (sr_lane() == 0) sm.sortbuf[sr_wave_id()] = v;
+    __syncthreads();
+    unsigned long long t = 0ull;
+#pragma unroll
+    for (int w = 0; w < kW; w++) t = sm.sortbuf[w] > t ? sm.sortbuf[w] : t;
+    __syncthreads();
+    return t;
+}
+// exclusive scan of one int per thread
+__device__ __forceinline__ int blk_excl_scan(int v, int* total, FullSmem& sm)
+{
+    int incl = sr_wave_incl_scan_i32(v);
+    __syncthreads();
+    if (sr_lane() == SR_WAVE - 1) sm.redi[sr_wave_id()] = incl;
+    __syncthreads();
+    int base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kW; w++) {
+        int t = sm.redi[w];
+        if (w < sr_wave_id()) base += t;
+        tot += t;
+    }
+    *total = tot;
+    return base + incl - v;
+}
+
+// ---- exact left-to-right sum over term(i), i in [0, n) ------------------------------------------------
+// term(i) must be >= 0 (or +0 for "skipped").  With kSearch, stops at the first i whose running sum is
+// >= target and returns it in *found (else -1).
+template <bool kSearch, typename Term>
+__device__ __forceinline__ float seq_sum(Term term, int n, float s0, float target, int* found, FullSmem& sm)
+{
+    float s = s0;
+    *found = -1;
+    for (int base = 0; base < n; base += SR_SEQ_TILE) {
+        float x[SR_SEQ_RUN];
+        const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? term(i0 + j) : 0.0f;
+        int f;
+        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+        if (kSearch && f >= 0) {
+            *found = base + f;
+            return s;
+        }
+    }
+    return s;
+}
+
+// TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
+// ragged tail folded in through an overlapped last vector, pairwise horizontal add.
+template <typename Term>
+__device__ float tp_sum(Term term, int n, FullSmem& sm)
+{
+    int dummy;
+    if (n < 4) {
+        return seq_sum<false>(term, n, 0.0f, 0.0f, &dummy, sm);
+    }
+    const int w = n >= 8 ? 8 : 4;
+    const int nv = n / w, rem = n - nv * w;
+    float lane_sum[8];
+#pragma unroll
+    for (int l = 0; l < 8; l++) {
+        lane_sum[l] = 0.0f;
+        if (l < w) {
+            const bool extra = rem > 0 && l >= w - rem;
+            const int cnt = nv + (extra ? 1 : 0);
+            auto lt = [&](int i) -> float { return i < nv ? term(i * w + l) : term(n - w + l); };
+            lane_sum[l] = seq_sum<false>(lt, cnt, 0.0f, 0.0f, &dummy, sm);
+        }
+    }
+    if (w == 8)
+        return __fadd_rn(__fadd_rn(__fadd_rn(lane_sum[0], lane_sum[1]), __fadd_rn(lane_sum[2], lane_sum[3])),
+                         __fadd_rn(__fadd_rn(lane_sum[4], lane_sum[5]), __fadd_rn(lane_sum[6], lane_sum[7])));
+    return __fadd_rn(__fadd_rn(lane_sum[0], lane_sum[1]), __fadd_rn(lane_sum[2], lane_sum[3]));
+}
+
+// Normalize (Sampler.cs:553-562)
+__device__ void normalize_row(float* p, int n, FullSmem& sm)
+{
+    const float sum = tp_sum([&](int i) -> float { return p[i]; }, n, sm);
+    if (sum > 0.0f && sum != 1.0f) {
+        const float inv = __fdiv_rn(1.0f, sum);
+        for (int i = threadIdx.x; i < n; i += kT) p[i] = __fmul_rn(p[i], inv);
+    }
+    __syncthreads();
+}
+
+// k-th largest value of p[0..n) (1-based), p >= 0: FindKthLargest (Sampler.cs:624-645).
+__device__ float kth_largest(const float* p, int n, int k, FullSmem& sm)
+{
+    uint32_t prefix = 0u, pmask = 0u;
+    int need = k;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (threadIdx.x < 256) sm.hist[threadIdx.x] = 0u;
+        __syncthreads();
+        for (int i = threadIdx.x; i < n; i += kT) {
+            const uint32_t key = sr_f2u(p[i]);
+            if ((key & pmask) == prefix) atomicAdd(&sm.hist[(key >> shift) & 0xffu], 1u);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int c = 0, d = 255;
+            for (; d > 0; d--) {
+                if (c + (int)sm.hist[d] >= need) break;
+                c += (int)sm.hist[d];
+            }
+            sm.bc[0] = (uint32_t)d;
+            sm.bc[1] = (uint32_t)(need - c);
+        }
+        __syncthreads();
+        prefix |= sm.bc[0] << shift;
+        pmask |= 0xffu << shift;
+        need = (int)sm.bc[1];
+        __syncthreads();
+    }
+    return sr_u2f(prefix);
+}
+
+// bitonic sort (descending) of sm.sortbuf[0 .. n_pow2)
+__device__ void sort_small_desc(FullSmem& sm, int n_pow2)
+{
+    for (int k2 = 2; k2 <= n_pow2; k2 <<= 1) {
+        for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
+            for (int i = threadIdx.x; i < n_pow2; i += kT) {
+                const int ixj = i ^ j2;
+                if (ixj > i) {
+                    const unsigned long long a = sm.sortbuf[i], b = sm.sortbuf[ixj];
+                    if ((a < b) == ((i & k2) == 0)) { sm.sortbuf[i] = b; sm.sortbuf[ixj] = a; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+template <int ES>
+__device__ __forceinline__ float load_logit(const char* rowp, int i)
+{
+    if (ES == 4) return ((const float*)rowp)[i];
+    return sr_bf16_to_f32(((const uint16_t*)rowp)[i]);
+}
+
+// ---- stage 1: the masked (and temperature-scaled) copy of the row ------------------------------------
+template <int ES>
+__global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
+{
+    const int slot = blockIdx.y;
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+    float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+    const bool scale = rd.temperature > 0.0f && rd.temperature != 1.0f;
+    const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256) {
+        float x = load_logit<ES>(rowp, i);
+        if (mrow && !((mrow[i >> 5] >> (i & 31)) & 1u)) x = SR_NEG_INF;
+        if (scale) x = __fmul_rn(x, inv_temp);
+        w[i] = x;
+    }
+}
+
+// ---- stage 2: logit bias and history penalties on the few ids they touch (Sampler.cs:51-58, :367-419)
+template <int ES>
+__global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
+{
+    const int slot = blockIdx.x;
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    if (rd.edit_cnt <= 0) return;
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+    float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+    const bool sampled = rd.temperature > 0.0f;
+    const bool scale = sampled && rd.temperature != 1.0f;
+    const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+    const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u;
+    const SrEdit* ed = a.edits + rd.edit_off;
+    for (int e = threadIdx.x; e < rd.edit_cnt; e += 256) {
+        const int id = ed[e].id;
+        float x = load_logit<ES>(rowp, id);
+        if (mrow && !((mrow[id >> 5] >> (id & 31)) & 1u)) x = SR_NEG_INF;
+        if (sampled && ed[e].has_bias) x = __fadd_rn(x, ed[e].bias);
+        if (pen && ed[e].occ_all > 0) {
+            if (rd.rep != 1.0f)
+                for (int o = 0; o < ed[e].occ_win; o++) x = x > 0.0f ? __fdiv_rn(x, rd.rep) : __fmul_rn(x, rd.rep);
+            if (rd.presence != 0.0f || rd.frequency != 0.0f)
+                x = __fsub_rn(x, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ed[e].occ_all)));
+        }
+        if (scale) x = __fmul_rn(x, inv_temp);
+        w[id] = x;
+    }
+}
+
+// ---- argmax of an fp32 row: first index of the maximum, first NaN wins -------------------------------
+__device__ int row_argmax(const float* w, int n, FullSmem& sm)
+{
+    unsigned long long best = 0ull;
+    for (int i = threadIdx.x; i < n; i += kT) {
+        const float v = w[i];
+        const uint32_t k = (v != v) ? 0xffffffffu : sr_okey(v);
+        const unsigned long long e = ((unsigned long long)k << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+        best = e > best ? e : best;
+    }
+    best = blk_max_u64(best, sm);
+    return best ? (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull)) : 0;
+}
+
+// first index whose running fp32 sum reaches r = (float)u; last index as the rounding fallback
+// (SampleFromDistribution, Sampler.cs:564-576)
+__device__ int draw_from_row(const float* p, int n, double u, FullSmem& sm)
+{
+    const float r = __double2float_rn(u);
+    int found;
+    seq_sum<true>([&](int i) -> float { return p[i]; }, n, 0.0f, r, &found, sm);
+    return found >= 0 ? found : n - 1;
+}
+
+// ---- stage 3: softmax, top-k, min-p, top-p on the work row --------------------------------------------
+// phase 1 ends after top-p for rows whose nucleus candidates fit the kernel (<= kSmall survivors), or
+// after compacting the survivors for the device-wide sort otherwise; phase 2 finishes those rows and
+// then normalises, draws and writes results for every row.
+__global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
+{
+    __shared__ FullSmem sm;
+    const int tid = threadIdx.x;
+    const int slot = blockIdx.x;
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    const int n = a.vocab;
+    float* p = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    SrFullState* st = a.state + slot;
+    const bool greedy = rd.temperature <= 0.0f;
+    const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
+
+    if (greedy) {
+        if (phase == 2) return;
+        // Greedy / GreedyWithHistoryPenalties on the adjusted row; distributions become one-hot
+        const int am = row_argmax(p, n, sm);
+        if (a.mode != 0) {
+            __syncthreads();
+            for (int i = tid; i < n; i += kT) p[i] = (i == am) ? 1.0f : 0.0f;
+        }
+        if (tid == 0) {
+            if (a.out_tokens) a.out_tokens[row] = am;
+            if (a.out_flags) a.out_flags[row] = SR_KFLAG_GREEDY | SR_KFLAG_FULL;
+        }
+        return;
+    }
+
+    if (phase == 1) {
+        // Softmax (Sampler.cs:448-472)
+        float m = SR_NEG_INF;
+        bool nanv = false;
+        for (int i = tid; i < n; i += kT) {
+            const float v = p[i];
+            if (v != v) nanv = true;
+            m = fmaxf(m, v);
+        }
+        bool any_nan;
+        m = blk_max_f(nanv ? __uint_as_float(0x7fc00000u) : m, &any_nan, sm);
+        uint32_t flags = SR_KFLAG_FULL;
+        if (any_nan || sr_f2u(m) == 0xff800000u) {
+            const float uni = n > 0 ? __fdiv_rn(1.0f, (float)n) : 0.0f;
+            for (int i = tid; i < n; i += kT) p[i] = uni;
+            flags |= SR_KFLAG_DEGENERATE;
+            __syncthreads();
+        } else {
+            int dummy;
+            const float sum = seq_sum<false>(
+                [&](int i) -> float {
+                    const float e = sr_expf(__fsub_rn(p[i], m));
+                    p[i] = e;
+                    return e;
+                },
+                n, 0.0f, 0.0f, &dummy, sm);
+            __syncthreads();
+            if (sum > 0.0f && sum != 1.0f) {
+                const float inv = __fdiv_rn(1.0f, sum);
+                for (int i = tid; i < n; i += kT) p[i] = __fmul_rn(p[i], inv);
+            }
+            __syncthreads();
+        }
+        // ApplyTopK + Normalize (Sampler.cs:71-81, :477-488): everything equal to the k-th value survives
+        if (rd.top_k > 0 && rd.top_k < n) {
+            const float kth = kth_largest(p, n, rd.top_k, sm);
+            for (int i = tid; i < n; i += kT)
+                if (p[i] < kth) p[i] = 0.0f;
+            __syncthreads();
+            normalize_row(p, n, sm);
+        }
+        // ApplyMinP (Sampler.cs:493-503)
+        if (rd.min_p > 0.0f) {
+            float mp = 0.0f;
+            for (int i = tid; i < n; i += kT) mp = fmaxf(mp, p[i]);
+            bool nn;
+            mp = blk_max_f(mp, &nn, sm);
+            const float thr = __fmul_rn(rd.min_p, mp);
+            for (int i = tid; i < n; i += kT)
+                if (p[i] < thr) p[i] = 0.0f;
+            __syncthreads();
+        }
+        // ApplyTopP (Sampler.cs:516-551)
+        int big = 0;
+        if (use_top_p) {
+            int cnt = 0;
+            for (int i = tid; i < n; i += kT) cnt += p[i] > 0.0f ? 1 : 0;
+            int ns;
+            // positions in index order (stable input for the device-wide sort)
+            // each thread owns the strided indices tid, tid + kT, ...; a second pass assigns slots per tile
+            ns = blk_sum_i(cnt, sm);
+            if (ns > kSmall) {
+                big = 1;
+                // compact (prob bits, idx) in ascending index order into this row's segment
+                uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
+                int* vals = a.sort_vals_in + (size_t)slot * a.sort_stride;
+                int base = 0;
+                for (int i0 = 0; i0 < n; i0 += kT) {
+                    const int i = i0 + tid;
+                    const float v = i < n ? p[i] : 0.0f;
+                    int tot;
+                    const int pos = blk_excl_scan(v > 0.0f ? 1 : 0, &tot, sm);
+                    if (v > 0.0f) { keys[base + pos] = sr_f2u(v); vals[base + pos] = i; }
+                    base += tot;
+                }
+            } else if (ns > 0) {
+                if (tid == 0) sm.bc[4] = 0u;
+                __syncthreads();
+                for (int i = tid; i < n; i += kT) {
+                    const float v = p[i];
+                    if (v > 0.0f) {
+                        const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
+                        sm.sortbuf[pos] = ((unsigned long long)sr_f2u(v) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+                    }
+                }
+                __syncthreads();
+                int P = 2;
+                while (P < ns) P <<= 1;
+                for (int i = ns + tid; i < P; i += kT) sm.sortbuf[i] = 0ull;
+                __syncthreads();
+                sort_small_desc(sm, P);
+                for (int i = tid; i < ns; i += kT) sm.sprob[i] = sr_u2f((uint32_t)(sm.sortbuf[i] >> 32));
+                __syncthreads();
+                int found;
+                seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, ns, 0.0f, rd.top_p, &found, sm);
+                const int cutoff = found >= 0 ? found + 1 : ns;
+                for (int i = cutoff + tid; i < ns; i += kT)
+                    p[0xffffffffu - (uint32_t)(sm.sortbuf[i] & 0xffffffffull)] = 0.0f;
+                __syncthreads();
+            }
+            if (tid == 0) st->n_survivors = ns;
+        }
+        if (tid == 0) {
+            st->big = big;
+            st->flags = flags;
+            a.seg_begin[slot] = (int)((size_t)slot * a.sort_stride);
+            a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + (big ? st->n_survivors : 0);
+        }
+        if (a.two_phase) return;
+        __syncthreads();
+    }
+
+    // ---- phase 2 --------------------------------------------------------------------------------------
+    if (a.two_phase && st->big) {
+        // nucleus over the device-sorted survivors (descending probability, ascending index on ties)
+        const uint32_t* keys = a.sort_keys_out + (size_t)slot * a.sort_stride;
+        const int* vals = a.sort_vals_out + (size_t)slot * a.sort_stride;
+        const int ns = st->n_survivors;
+        int found;
+        seq_sum<true>([&](int i) -> float { return sr_u2f(keys[i]); }, ns, 0.0f, rd.top_p, &found, sm);
+        const int cutoff = found >= 0 ? found + 1 : ns;
+        for (int i = cutoff + tid; i < ns; i += kT) p[vals[i]] = 0.0f;
+        __syncthreads();
+    }
+    // final Normalize (Sampler.cs:91-92)
+    normalize_row(p, n, sm);
+    int token = -1;
+    if (a.mode != 1) {
+        token = draw_from_row(p, n, a.uniforms[(size_t)row * a.uniforms_per_row], sm);
+        if (tid == 0 && a.out_tokens) a.out_tokens[row] = token;
+    }
+    if (tid == 0 && a.out_flags) a.out_flags[row] = st->flags;
+}
+
+// ---- SampleFromProbs / ResampleResidual on caller-provided distributions ------------------------------
+__global__ __launch_bounds__(kT) void k_draw_rows(const float* probs, int64_t stride, int n, const double* uniforms,
+                                                   int* out_tokens)
+{
+    __shared__ FullSmem sm;
+    const int row = blockIdx.x;
+    const int t = draw_from_row(probs + (size_t)row * stride, n, uniforms[row], sm);
+    if (threadIdx.x == 0) out_tokens[row] = t;
+}
+
+// residual = max(0, p - q): first the left-to-right sum of the positive residuals, then the first index
+// whose running residual reaches (float)u * sum; degenerate residual -> draw from p (Sampler.cs:587-618)
+__device__ int resample_residual_row(const float* p, const float* q, int n, double u, FullSmem& sm)
+{
+    int dummy;
+    auto res = [&](int i) -> float {
+        const float r = __fsub_rn(p[i], q[i]);
+        return r > 0.0f ? r : 0.0f;
+    };
+    const float sum = seq_sum<false>(res, n, 0.0f, 0.0f, &dummy, sm);
+    if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm);  // sum <= 0 or NaN
+    const float target = __fmul_rn(__double2float_rn(u), sum);
+    // `target <= cum` is only tested on positive residuals: a zero target must not stop on a zero term
+    int found;
+    if (target <= 0.0f) {
+        int first = 0x7fffffff;
+        for (int i = threadIdx.x; i < n; i += kT)
+            if (res(i) > 0.0f) { first = i; break; }
+        first = sr_wave_min_i32(first);
+        __syncthreads();
+        if (sr_lane() == 0) sm.redi[sr_wave_id()] = first;
+        __syncthreads();
+        int f = 0x7fffffff;
+        for (int w = 0; w < kW; w++) f = min(f, sm.redi[w]);
+        __syncthreads();
+        return f;  // sum > 0 guarantees a positive residual exists
+    }
+    seq_sum<true>(res, n, 0.0f, target, &found, sm);
+    if (found >= 0) return found;
+    // rounding fallback: the last index with a positive residual
+    int last = -1;
+    for (int i = threadIdx.x; i < n; i += kT)
+        if (res(i) > 0.0f) last = i;
+    last = -sr_wave_min_i32(-last);
+    __syncthreads();
+    if (sr_lane() == 0) sm.redi[sr_wave_id()] = last;
+    __syncthreads();
+    int l = -1;
+    for (int w = 0; w < kW; w++) l = max(l, sm.redi[w]);
+    __syncthreads();
+    return l;
+}
+
+__global__ __launch_bounds__(kT) void k_residual_rows(const float* p, int64_t ps, const float* q, int64_t qs, int n,
+                                                       const double* uniforms, int* out_tokens)
+{
+    __shared__ FullSmem sm;
+    const int row = blockIdx.x;
+    const int t = resample_residual_row(p + (size_t)row * ps, q + (size_t)row * qs, n, uniforms[row], sm);
+    if (threadIdx.x == 0) out_tokens[row] = t;
+}
+
+// ---- speculative verification: the accept loop of StepSampled (SpeculativeDecoder.cs:530-559) ---------
+// p_all holds the filtered target distributions of every position, [rows][n_draft + 1][n].
+__global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
+{
+    __shared__ FullSmem sm;
+    const int row = blockIdx.x;
+    const SrRow rd = a.rows[row];
+    const int n = a.vocab, L = a.n_draft;
+    const float* pr = a.p_all + (size_t)row * (L + 1) * n;
+    const float* lg = a.target_logits + (size_t)row * (L + 1) * n;
+    const double* u = a.uniforms + (size_t)row * a.uniforms_per_row;
+    int* out = a.out_tokens + (size_t)row * (L + 1);
+    const bool true_spec = !(rd.p_min > 0.0f && rd.p_min < 1.0f);  // SpeculativeDecoder.cs:192
+    for (int i = threadIdx.x; i <= L; i += kT) out[i] = -1;
+    __syncthreads();
+    int accepted = 0, udraws = 0, correction = -1;
+    for (int i = 0; i < L; i++) {
+        const float* pd = pr + (size_t)i * n;
+        const float* qd = a.draft_probs + ((size_t)row * L + i) * n;
+        const int tok = a.draft_tokens[(size_t)row * L + i];
+        const float px = pd[tok];
+        bool accept;
+        if (true_spec) {
+            const float qx = qd[tok];
+            const float acc = qx > 0.0f ? fminf(1.0f, __fdiv_rn(px, qx)) : (px > 0.0f ? 1.0f : 0.0f);
+            accept = u[udraws++] < (double)acc;
+        } else {
+            accept = px >= rd.p_min;
+            if (!accept) accept = tok == row_argmax(lg + (size_t)i * n, n, sm);  // block-uniform branch
+        }
+        if (accept) {
+            if (threadIdx.x == 0) out[accepted] = tok;
+            accepted++;
+            continue;
+        }
+        correction = true_spec ? resample_residual_row(pd, qd, n, u[udraws++], sm)
+                               : draw_from_row(pd, n, u[udraws++], sm);
+        break;
+    }
+    if (correction < 0) {
+        // every draft accepted: bonus token from the last position (greedy rows: its argmax, no draw)
+        const float* pd = pr + (size_t)L * n;
+        correction = rd.temperature <= 0.0f ? row_argmax(pd, n, sm) : draw_from_row(pd, n, u[udraws++], sm);
+    }
+    if (threadIdx.x == 0) {
+        out[accepted] = correction;
+        a.out_accepted[row] = accepted;
+    }
+}
+
+// ---- MtpDecoder.AcceptDraft / SoftmaxProbAt (MtpDecoder.cs:562-596) ------------------------------------
+__global__ __launch_bounds__(kT) void k_mtp_verify(const float* logits, int64_t stride, int n, const int* draft,
+                                                    float p_min, int* out_argmax, int* out_accept, float* out_prob)
+{
+    __shared__ FullSmem sm;
+    __shared__ double dred[kW];
+    const int row = blockIdx.x;
+    const float* l = logits + (size_t)row * stride;
+    const int am = row_argmax(l, n, sm);
+    const int d = draft[row];
+    float prob = 0.0f;
+    int ok = d == am ? 1 : 0;
+    if (!ok && p_min < 1.0f) {
+        // max, sum of exp(l - max) in double, ratio cast to float.  The double sum is a tree reduction:
+        // it can differ from the reference's left-to-right double sum in the last bits, far below the
+        // float result's 1e-5 tolerance.
+        float m = l[0];
+        for (int i = threadIdx.x; i < n; i += kT) m = fmaxf(m, l[i]);
+        bool nn;
+        m = blk_max_f(m, &nn, sm);
+        double s = 0.0;
+        for (int i = threadIdx.x; i < n; i += kT) s += exp((double)__fsub_rn(l[i], m));
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+        __syncthreads();
+        if (sr_lane() == 0) dred[sr_wave_id()] = s;
+        __syncthreads();
+        double tot = 0.0;
+        for (int w = 0; w < kW; w++) tot += dred[w];
+        if (tot > 0.0 && d >= 0 && d < n) prob = (float)(exp((double)__fsub_rn(l[d], m)) / tot);
+        ok = prob >= p_min ? 1 : 0;
+    }
+    if (threadIdx.x == 0) {
+        out_argmax[row] = am;
+        out_accept[row] = ok;
+        if (out_prob) out_prob[row] = prob;
+    }
+}
+
+__global__ __launch_bounds__(kT) void k_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum,
+                                                         int* out_idx)
+{
+    __shared__ FullSmem sm;
+    int found;
+    float s;
+    if (target == target)
+        s = seq_sum<true>([&](int i) -> float { return x[i]; }, n, s0, target, &found, sm);
+    else
+        s = seq_sum<false>([&](int i) -> float { return x[i]; }, n, s0, 0.0f, &found, sm);
+    if (threadIdx.x == 0) { *out_sum = s; *out_idx = found; }
+}
+
+}  // namespace
+
+hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
+{
+    if (n_rows <= 0) return hipSuccess;
+    const int bx = max(1, min(64, (a.vocab + 256 * 16 - 1) / (256 * 16)));
+    dim3 grid(bx, n_rows);
+    if (a.dtype == 1) {
+        hipLaunchKernelGGL(k_full_prep<2>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(k_full_edits<2>, dim3(n_rows), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(k_full_prep<4>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(k_full_edits<4>, dim3(n_rows), dim3(256), 0, st, a);
+    }
+    return hipGetLastError();
+}
+hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st)
+{
+    if (n_rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_full_row, dim3(n_rows), dim3(kT), 0, st, a, phase);
+    return hipGetLastError();
+}
+hipError_t sr_launch_draw_rows(const float* probs, int64_t stride, int n, int rows, const double* u, int* out,
+                               hipStream_t st)
+{
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_draw_rows, dim3(rows), dim3(kT), 0, st, probs, stride, n, u, out);
+    return hipGetLastError();
+}
+hipError_t sr_launch_residual_rows(const float* p, int64_t ps, const float* q, int64_t qs, int n, int rows,
+                                   const double* u, int* out, hipStream_t st)
+{
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_residual_rows, dim3(rows), dim3(kT), 0, st, p, ps, q, qs, n, u, out);
+    return hipGetLastError();
+}
+hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st)
+{
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_spec_verify, dim3(rows), dim3(kT), 0, st, a);
+    return hipGetLastError();
+}
+hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int rows, const int* draft, float p_min,
+                                int* out_argmax, int* out_accept, float* out_prob, hipStream_t st)
+{
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_mtp_verify, dim3(rows), dim3(kT), 0, st, logits, stride, n, draft, p_min, out_argmax,
+                       out_accept, out_prob);
+    return hipGetLastError();
+}
+hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum, int* out_idx,
+                                     hipStream_t st)
+{
+    hipLaunchKernelGGL(k_selftest_seqsum, dim3(1), dim3(kT), 0, st, x, n, s0, target, out_sum, out_idx);
+    return hipGetLastError();
+}

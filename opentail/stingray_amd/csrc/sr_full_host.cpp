@@ -1,0 +1,305 @@
+// Host side of the full-vocabulary entry points: the slow path of Sampler.Sample, BuildFilteredDistribution,
+// SampleWithDistribution, SampleFromProbs, ResampleResidual, the speculative accept loop and the MTP
+// accept test.  Launch sequences only; all arithmetic is in sr_full.hip.
+#include <cstring>
+
+#include "sr_host.h"
+
+namespace {
+
+// Runs the full-vocabulary pipeline for the rows in `list` (device array of n_rows row indices).
+//   mode 0: work rows live in ctx scratch, tokens out.   mode 1/2: work rows ARE the caller's probs rows.
+int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows, bool any_top_p, const void* logits_dev,
+             int dtype, int64_t row_stride, int mode, float* probs_dev, int64_t probs_stride, int32_t* out_tokens_dev,
+             uint32_t* out_flags_dev)
+{
+    if (n_rows <= 0) return SR_OK;
+    hipStream_t st = ctx->stream;
+    const int vocab = b->vocab;
+    SrFullArgs a{};
+    a.logits = logits_dev;
+    a.row_stride = row_stride;
+    a.vocab = vocab;
+    a.dtype = dtype;
+    a.row_list = list_dev;
+    a.rows = b->d_rows.as<SrRow>();
+    a.edits = b->d_edits.as<SrEdit>();
+    a.mask = b->d_mask.as<uint32_t>();
+    a.mask_stride = b->mask_stride;
+    a.mode = mode;
+    if (mode == 0) {
+        const int64_t ws = (vocab + 3) & ~3;
+        SR_HIP(ctx, ctx->work.reserve((size_t)n_rows * ws * sizeof(float), st));
+        a.work = ctx->work.as<float>();
+        a.work_stride = ws;
+        a.work_by_row = 0;
+    } else {
+        a.work = probs_dev;
+        a.work_stride = probs_stride;
+        a.work_by_row = 1;
+    }
+    a.two_phase = any_top_p ? 1 : 0;
+    SR_HIP(ctx, ctx->full_state.reserve((size_t)n_rows * sizeof(SrFullState), st));
+    a.state = ctx->full_state.as<SrFullState>();
+    SR_HIP(ctx, ctx->seg.reserve((size_t)n_rows * 2 * sizeof(int32_t), st));
+    a.seg_begin = ctx->seg.as<int32_t>();
+    a.seg_end = a.seg_begin + n_rows;
+    // sort segments are laid out with the work stride of mode 0; in modes 1/2 use a private stride
+    const int64_t seg_stride = (vocab + 3) & ~3;
+    if ((int64_t)n_rows * seg_stride >= (int64_t)1 << 31)
+        return sr_fail(ctx, SR_ERR_UNSUPPORTED, "full-vocabulary path: rows x vocab exceeds 2^31 entries");
+    size_t tmp_bytes = 0;
+    if (a.two_phase) {
+        const size_t items = (size_t)n_rows * seg_stride;
+        SR_HIP(ctx, ctx->sort_k0.reserve(items * 4, st));
+        SR_HIP(ctx, ctx->sort_k1.reserve(items * 4, st));
+        SR_HIP(ctx, ctx->sort_v0.reserve(items * 4, st));
+        SR_HIP(ctx, ctx->sort_v1.reserve(items * 4, st));
+        a.sort_keys_in = ctx->sort_k0.as<uint32_t>();
+        a.sort_vals_in = ctx->sort_v0.as<int32_t>();
+        a.sort_keys_out = ctx->sort_k1.as<uint32_t>();
+        a.sort_vals_out = ctx->sort_v1.as<int32_t>();
+        SR_HIP(ctx, sr_segmented_sort_desc(nullptr, &tmp_bytes, a.sort_keys_in, ctx->sort_k1.as<uint32_t>(), a.sort_vals_in,
+                                           ctx->sort_v1.as<int32_t>(), (int64_t)items, n_rows, a.seg_begin, a.seg_end, st));
+        SR_HIP(ctx, ctx->sort_tmp.reserve(tmp_bytes + 256, st));
+    }
+    // the kernels index sort segments with work_stride; keep both strides equal in mode 0 and pass the
+    // segment stride separately otherwise
+    a.sort_stride = seg_stride;
+    a.uniforms = b->d_uniforms.as<double>();
+    a.uniforms_per_row = b->upr;
+    a.out_tokens = out_tokens_dev;
+    a.out_flags = out_flags_dev;
+
+    SR_HIP(ctx, sr_launch_full_prep(a, n_rows, st));
+    SR_HIP(ctx, sr_launch_full_row(a, n_rows, 1, st));
+    if (a.two_phase) {
+        const size_t items = (size_t)n_rows * seg_stride;
+        SR_HIP(ctx, sr_segmented_sort_desc(ctx->sort_tmp.p, &tmp_bytes, a.sort_keys_in, ctx->sort_k1.as<uint32_t>(),
+                                           a.sort_vals_in, ctx->sort_v1.as<int32_t>(), (int64_t)items, n_rows, a.seg_begin,
+                                           a.seg_end, st));
+        SR_HIP(ctx, sr_launch_full_row(a, n_rows, 2, st));
+    }
+    return SR_OK;
+}
+
+bool row_uses_top_p(const SrRow& r) { return r.temperature > 0.0f && r.top_p < 1.0f && r.top_p > 0.0f; }
+
+int check_batch_call(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride, const char* who)
+{
+    if (!logits_dev) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, std::string(who) + ": logits is null");
+    if (dtype != SR_DTYPE_F32 && dtype != SR_DTYPE_BF16) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": unknown dtype");
+    if (b->vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": empty vocabulary");
+    if (row_stride < b->vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": row stride < vocab");
+    return SR_OK;
+}
+
+// identity row list [0, rows) on the device
+int identity_list(sr_ctx* ctx, int rows, const int32_t** out)
+{
+    if (ctx->ident_rows < rows) {
+        std::vector<int32_t> h((size_t)rows);
+        for (int i = 0; i < rows; i++) h[(size_t)i] = i;
+        SR_HIP(ctx, ctx->ident.reserve((size_t)rows * sizeof(int32_t), ctx->stream));
+        SR_HIP(ctx, hipMemcpyAsync(ctx->ident.p, h.data(), (size_t)rows * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+        SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        ctx->ident_rows = rows;
+    }
+    *out = ctx->ident.as<int32_t>();
+    return SR_OK;
+}
+
+int upload_uniforms(sr_ctx* ctx, const double* uniforms, int rows, const double** dev)
+{
+    SR_HIP(ctx, ctx->uniforms_tmp.reserve((size_t)rows * sizeof(double), ctx->stream));
+    SR_HIP(ctx, hipMemcpyAsync(ctx->uniforms_tmp.p, uniforms, (size_t)rows * sizeof(double), hipMemcpyHostToDevice, ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the host array may go away
+    *dev = ctx->uniforms_tmp.as<double>();
+    return SR_OK;
+}
+
+}  // namespace
+
+int sr_full_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
+                        int32_t* out_tokens_dev, uint32_t* out_flags_dev)
+{
+    bool any_top_p = false;
+    for (int32_t r : b->h_full_list) any_top_p = any_top_p || row_uses_top_p(b->h_rows[(size_t)r]);
+    return run_full(ctx, b, b->d_full_list.as<int32_t>(), (int)b->h_full_list.size(), any_top_p, logits_dev, dtype,
+                    row_stride, 0, nullptr, 0, out_tokens_dev, out_flags_dev);
+}
+
+extern "C" {
+
+int sr_build_distribution_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
+                                 float* out_probs_dev, int64_t probs_stride, int32_t probs_len)
+{
+    if (!ctx || !b) return SR_ERR_NULL_ARGUMENT;
+    if (b->rows == 0) return SR_OK;
+    if (probs_len != b->vocab)  // Sampler.cs:121-123
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "probs length (" + std::to_string(probs_len) + ") must equal logits length (" +
+                                                         std::to_string(b->vocab) + ").");
+    int rc = check_batch_call(ctx, b, logits_dev, dtype, row_stride, "sr_build_distribution_launch");
+    if (rc != SR_OK) return rc;
+    if (!out_probs_dev) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_build_distribution_launch: probs is null");
+    if (probs_stride < b->vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_build_distribution_launch: probs stride < vocab");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    const int32_t* list = nullptr;
+    rc = identity_list(ctx, b->rows, &list);
+    if (rc != SR_OK) return rc;
+    bool any_top_p = false;
+    for (const SrRow& r : b->h_rows) any_top_p = any_top_p || row_uses_top_p(r);
+    return run_full(ctx, b, list, b->rows, any_top_p, logits_dev, dtype, row_stride, 1, out_probs_dev, probs_stride, nullptr, nullptr);
+}
+
+int sr_sample_with_distribution_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
+                                       float* out_probs_dev, int64_t probs_stride, int32_t probs_len, int32_t* out_tokens_dev)
+{
+    if (!ctx || !b) return SR_ERR_NULL_ARGUMENT;
+    if (b->rows == 0) return SR_OK;
+    if (probs_len != b->vocab)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "probs length (" + std::to_string(probs_len) + ") must equal logits length (" +
+                                                         std::to_string(b->vocab) + ").");
+    int rc = check_batch_call(ctx, b, logits_dev, dtype, row_stride, "sr_sample_with_distribution_launch");
+    if (rc != SR_OK) return rc;
+    if (!out_probs_dev || !out_tokens_dev) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_with_distribution_launch: null output");
+    if (probs_stride < b->vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_with_distribution_launch: probs stride < vocab");
+    for (const SrRow& r : b->h_rows)
+        if (r.temperature > 0.0f && b->upr < 1)
+            return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_with_distribution_launch: a sampled row needs a uniform");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    const int32_t* list = nullptr;
+    rc = identity_list(ctx, b->rows, &list);
+    if (rc != SR_OK) return rc;
+    bool any_top_p = false;
+    for (const SrRow& r : b->h_rows) any_top_p = any_top_p || row_uses_top_p(r);
+    return run_full(ctx, b, list, b->rows, any_top_p, logits_dev, dtype, row_stride, 2, out_probs_dev, probs_stride, out_tokens_dev, nullptr);
+}
+
+int sr_sample_from_probs_launch(sr_ctx* ctx, const float* probs_dev, int32_t rows, int32_t vocab, int64_t probs_stride,
+                                const double* uniforms, int32_t* out_tokens_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (!uniforms) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "rng");  // ArgumentNullException(rng), Sampler.cs:197
+    if (rows == 0) return SR_OK;
+    if (!probs_dev || !out_tokens_dev) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_from_probs_launch: null tensor");
+    if (rows < 0 || vocab <= 0 || probs_stride < vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_from_probs_launch: bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    const double* u = nullptr;
+    int rc = upload_uniforms(ctx, uniforms, rows, &u);
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, sr_launch_draw_rows(probs_dev, probs_stride, vocab, rows, u, out_tokens_dev, ctx->stream));
+    return SR_OK;
+}
+
+int sr_resample_residual_launch(sr_ctx* ctx, const float* p_dev, int32_t p_len, int64_t p_stride, const float* q_dev,
+                                int32_t q_len, int64_t q_stride, int32_t rows, const double* uniforms, int32_t* out_tokens_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (!uniforms) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "rng");  // Sampler.cs:589
+    if (p_len != q_len)                                                // Sampler.cs:590-592
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT,
+                       "p and q must have equal length (" + std::to_string(p_len) + " vs " + std::to_string(q_len) + ").");
+    if (rows == 0) return SR_OK;
+    if (!p_dev || !q_dev || !out_tokens_dev) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_resample_residual_launch: null tensor");
+    if (rows < 0 || p_len <= 0 || p_stride < p_len || q_stride < q_len)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_resample_residual_launch: bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    const double* u = nullptr;
+    int rc = upload_uniforms(ctx, uniforms, rows, &u);
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, sr_launch_residual_rows(p_dev, p_stride, q_dev, q_stride, p_len, rows, u, out_tokens_dev, ctx->stream));
+    return SR_OK;
+}
+
+int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_logits_dev, const float* draft_probs_dev,
+                          const int32_t* draft_tokens_dev, int32_t n_draft, int32_t* out_accepted_dev, int32_t* out_tokens_dev)
+{
+    if (!ctx || !b) return SR_ERR_NULL_ARGUMENT;
+    if (b->rows == 0) return SR_OK;
+    if (n_draft < 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_spec_verify_launch: negative draft length");
+    if (!target_logits_dev || !out_accepted_dev || !out_tokens_dev || (n_draft > 0 && (!draft_probs_dev || !draft_tokens_dev)))
+        return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_spec_verify_launch: null tensor");
+    if (b->vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_spec_verify_launch: empty vocabulary");
+    if (b->upr < n_draft + 1) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_spec_verify_launch: needs n_draft + 1 uniforms per row");
+    if (b->has_mask) return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_spec_verify_launch: allow-masks are not part of speculative verification");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    const int rows = b->rows, V = b->vocab, P = n_draft + 1;
+    // Every position of a row is filtered with the row's parameters (SpeculativeDecoder.cs:535): expand the
+    // batch's row descriptors to rows x positions and build all distributions in one pass.
+    if ((int64_t)rows * P * V >= (int64_t)1 << 31)
+        return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_spec_verify_launch: rows x positions x vocab exceeds 2^31 entries");
+    std::vector<SrRow> exp_rows((size_t)rows * P);
+    bool any_top_p = false;
+    for (int r = 0; r < rows; r++)
+        for (int i = 0; i < P; i++) {
+            SrRow d = b->h_rows[(size_t)r];
+            d.mask_row = -1;
+            exp_rows[(size_t)r * P + i] = d;
+            any_top_p = any_top_p || row_uses_top_p(d);
+        }
+    SR_HIP(ctx, ctx->spec_rows.reserve(exp_rows.size() * sizeof(SrRow), st));
+    SR_HIP(ctx, hipMemcpyAsync(ctx->spec_rows.p, exp_rows.data(), exp_rows.size() * sizeof(SrRow), hipMemcpyHostToDevice, st));
+    SR_HIP(ctx, hipStreamSynchronize(st));
+    SR_HIP(ctx, ctx->spec_probs.reserve((size_t)rows * P * V * sizeof(float), st));
+    sr_batch tmp;  // a view: expanded rows, the original edits
+    tmp.ctx = ctx;
+    tmp.rows = rows * P;
+    tmp.vocab = V;
+    tmp.upr = 0;
+    tmp.d_rows.p = ctx->spec_rows.p;
+    tmp.d_edits.p = b->d_edits.p;
+    tmp.mask_stride = 0;
+    const int32_t* list = nullptr;
+    int rc = identity_list(ctx, rows * P, &list);
+    if (rc == SR_OK)
+        rc = run_full(ctx, &tmp, list, rows * P, any_top_p, target_logits_dev, SR_DTYPE_F32, V, 1, ctx->spec_probs.as<float>(), V,
+                      nullptr, nullptr);
+    tmp.d_rows.p = nullptr;  // borrowed
+    tmp.d_edits.p = nullptr;
+    if (rc != SR_OK) return rc;
+    SrSpecArgs a{};
+    a.rows = b->d_rows.as<SrRow>();
+    a.vocab = V;
+    a.n_draft = n_draft;
+    a.p_all = ctx->spec_probs.as<float>();
+    a.target_logits = target_logits_dev;
+    a.draft_probs = draft_probs_dev;
+    a.draft_tokens = draft_tokens_dev;
+    a.uniforms = b->d_uniforms.as<double>();
+    a.uniforms_per_row = b->upr;
+    a.out_accepted = out_accepted_dev;
+    a.out_tokens = out_tokens_dev;
+    SR_HIP(ctx, sr_launch_spec_verify(a, rows, st));
+    return SR_OK;
+}
+
+int sr_mtp_verify_launch(sr_ctx* ctx, const float* logits_dev, int32_t rows, int32_t vocab, int64_t row_stride,
+                         const int32_t* draft_tokens_dev, float p_min, int32_t* out_argmax_dev, int32_t* out_accept_dev,
+                         float* out_prob_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0) return SR_OK;
+    if (!logits_dev || !draft_tokens_dev || !out_argmax_dev || !out_accept_dev)
+        return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_mtp_verify_launch: null tensor");
+    if (rows < 0 || vocab <= 0 || row_stride < vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mtp_verify_launch: bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    // p_min <= 0 means "argmax match only" (SamplingParams.SpecDraftPMin, Sampler.cs:791)
+    const float pm = p_min > 0.0f ? p_min : 1.0f;
+    SR_HIP(ctx, sr_launch_mtp_verify(logits_dev, row_stride, vocab, rows, draft_tokens_dev, pm, out_argmax_dev, out_accept_dev,
+                                     out_prob_dev, ctx->stream));
+    return SR_OK;
+}
+
+// Test hook: exact left-to-right sum of x_dev[0..n) from s0; target = NaN disables the search.
+SR_API int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float s0, float target, float* out_sum_dev,
+                              int32_t* out_idx_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    SR_HIP(ctx, sr_launch_selftest_seqsum(x_dev, n, s0, target, out_sum_dev, out_idx_dev, ctx->stream));
+    return SR_OK;
+}
+
+}  // extern "C"

@@ -53,6 +53,10 @@ struct sr_ctx {
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits
     DeviceBuf out_tokens, out_flags, out_val, uniforms_tmp;
+    DeviceBuf seg, sort_k0, sort_k1, sort_v0, sort_v1, sort_tmp;  // device-wide sort of large nuclei
+    DeviceBuf ident;         // identity row list
+    int ident_rows = 0;
+    DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
 };
@@ -85,7 +89,7 @@ inline int sr_fail_hip(sr_ctx* ctx, hipError_t e, const char* what)
         if (_e != hipSuccess) return sr_fail_hip((ctx), _e, #call);   \
     } while (0)
 
-// Full-vocabulary rows of a batch (sr_full.cpp).  mode: 0 = sample, 1 = build distribution,
+// Full-vocabulary rows of a batch (sr_full_host.cpp).  mode: 0 = sample, 1 = build distribution,
 // 2 = build distribution and sample from it.
 int sr_full_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
                         int32_t* out_tokens_dev, uint32_t* out_flags_dev);

@@ -52,3 +52,71 @@ struct SrArgmaxArgs {
 hipError_t sr_launch_argmax_rows(const SrArgmaxArgs& a, hipStream_t stream);
 
 hipError_t sr_launch_selftest_expf(const float* x, float* y, int64_t n, hipStream_t stream);
+
+// ---- full-vocabulary path (sr_full.hip) ---------------------------------------------------------------
+struct SrFullState {
+    int32_t n_survivors;  // entries with probability > 0 when top-p starts
+    int32_t big;          // survivors exceed what the row kernel sorts itself: device-wide sort needed
+    uint32_t flags;
+    int32_t pad;
+};
+
+struct SrFullArgs {
+    const void* logits;
+    int64_t row_stride;
+    int32_t vocab;
+    int32_t dtype;
+    const int32_t* row_list;   // rows handled (device)
+    const SrRow* rows;
+    const SrEdit* edits;
+    const uint32_t* mask;
+    int64_t mask_stride;
+    float* work;               // fp32 rows: [slot] or, with work_by_row, [row]
+    int64_t work_stride;
+    int32_t work_by_row;
+    int32_t mode;              // 0 = sample, 1 = distribution only, 2 = distribution and sample
+    int32_t two_phase;         // a device-wide sort of large nuclei runs between phase 1 and phase 2
+    SrFullState* state;        // [slot]
+    uint32_t* sort_keys_in;    // [slot][sort_stride]
+    int32_t* sort_vals_in;
+    const uint32_t* sort_keys_out;
+    const int32_t* sort_vals_out;
+    int64_t sort_stride;       // entries per row segment in the sort buffers
+    int32_t* seg_begin;        // [slot]
+    int32_t* seg_end;
+    const double* uniforms;
+    int32_t uniforms_per_row;
+    int32_t* out_tokens;       // [row], may be null in mode 1
+    uint32_t* out_flags;       // [row], may be null
+};
+hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
+hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st);
+hipError_t sr_launch_draw_rows(const float* probs, int64_t stride, int n, int rows, const double* u, int* out,
+                               hipStream_t st);
+hipError_t sr_launch_residual_rows(const float* p, int64_t ps, const float* q, int64_t qs, int n, int rows,
+                                   const double* u, int* out, hipStream_t st);
+
+struct SrSpecArgs {
+    const SrRow* rows;
+    int32_t vocab;
+    int32_t n_draft;
+    const float* p_all;          // [rows][n_draft + 1][vocab] filtered target distributions
+    const float* target_logits;  // [rows][n_draft + 1][vocab]
+    const float* draft_probs;    // [rows][n_draft][vocab]
+    const int32_t* draft_tokens; // [rows][n_draft]
+    const double* uniforms;
+    int32_t uniforms_per_row;
+    int32_t* out_accepted;       // [rows]
+    int32_t* out_tokens;         // [rows][n_draft + 1]
+};
+hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st);
+hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int rows, const int* draft, float p_min,
+                                int* out_argmax, int* out_accept, float* out_prob, hipStream_t st);
+hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum, int* out_idx,
+                                     hipStream_t st);
+
+// Stable descending segmented sort of (probability bits, index) pairs (sr_sort.hip, rocPRIM/hipCUB).
+// With tmp == nullptr only *tmp_bytes is set.
+hipError_t sr_segmented_sort_desc(void* tmp, size_t* tmp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
+                                  const int32_t* vals_in, int32_t* vals_out, int64_t n_items, int n_segments,
+                                  const int32_t* seg_begin, const int32_t* seg_end, hipStream_t st);

@@ -48,3 +48,6 @@ struct SrEdit {
 #define SR_TK_SEL_MAX 2048                 // largest k + history handled by the selection kernel
 #define SR_TK_TAIL_CAP 16384                // merged candidates the row tail holds (32 per thread)
 #define SR_TK_MAX_CHUNKS 128               // most workgroups one row is split over
+
+// Full-vocabulary path: nucleus candidates up to this count are sorted inside the row kernel.
+#define SR_FULL_SMALL_CAP 4096

@@ -171,6 +171,8 @@ def lib():
     L.oracle_mtp_accept_draft.restype = C.c_int32
     L.oracle_sample_batch.argtypes = [fp, C.c_int64, C.c_int32, C.c_int32, pp, C.POINTER(C.c_uint32),
                                       C.c_int64, C.POINTER(C.c_uint8), C.POINTER(C.c_double), fp, ip]
+    L.oracle_seq_sum.argtypes = [fp, C.c_int64, C.c_float, C.c_float, C.POINTER(C.c_int64)]
+    L.oracle_seq_sum.restype = C.c_float
     _lib = L
     return L
 
@@ -181,6 +183,14 @@ def _f32(a) -> np.ndarray:
 
 def _fp(a: np.ndarray):
     return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def seq_sum(x, s0: float = 0.0, target: float = float("inf")):
+    """(left-to-right fp32 sum, first index whose running sum >= target or -1)"""
+    a = _f32(x)
+    at = C.c_int64(-1)
+    s = lib().oracle_seq_sum(_fp(a), len(a), s0, target, C.byref(at))
+    return np.float32(s), int(at.value)
 
 
 def expf(x: float) -> float:

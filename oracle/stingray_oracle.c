@@ -669,6 +669,18 @@ int32_t oracle_mtp_accept_draft(int32_t draft, int32_t target, const float* logi
     return *draft_prob >= p_min;
 }
 
+float oracle_seq_sum(const float* x, int64_t n, float s0, float target, int64_t* first_reach)
+{
+    float s = s0;
+    int64_t at = -1;
+    for (int64_t i = 0; i < n; i++) {
+        s += x[i];
+        if (at < 0 && s >= target) at = i;
+    }
+    if (first_reach) *first_reach = at;
+    return s;
+}
+
 /* ContinuousBatchingEngine.cs:609-650: rows in order, Filter(row) then Greedy|Sample. */
 void oracle_sample_batch(const float* logits, int64_t row_stride, int32_t rows, int32_t n,
                          const oracle_params* params, const uint32_t* allow_mask,

@@ -111,6 +111,11 @@ float oracle_softmax_prob_at(const float* logits, int32_t n, int32_t idx);
 int32_t oracle_mtp_accept_draft(int32_t draft, int32_t target, const float* logits, int32_t n,
                                 float p_min, float* draft_prob);
 
+/* Plain left-to-right fp32 running sum of x[0..n) starting from s0, as the reference's scalar loops do
+ * (e.g. Sampler.cs:460-465).  When first_reach is non-NULL it receives the first index at which the running
+ * sum is >= target (-1 if never).  Used to pin the GPU's parallel evaluation of such sums. */
+float oracle_seq_sum(const float* x, int64_t n, float s0, float target, int64_t* first_reach);
+
 /* Row loops used by tests and by the bench's CPU-baseline leg (one thread, rows in order, as the
  * reference's batcher does at ContinuousBatchingEngine.cs:609-650). */
 void oracle_sample_batch(const float* logits, int64_t row_stride, int32_t rows, int32_t n,

@@ -1,0 +1,273 @@
+"""GPU parity of the full-vocabulary path through the C ABI: the exact left-to-right running sum, the slow
+path of Sampler.Sample, BuildFilteredDistribution, SampleWithDistribution, SampleFromProbs,
+ResampleResidual, speculative verification and the MTP accept test, against the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import binding as orc
+from opentail.stingray_amd import Sampler, SamplerContext, SamplingParams, pack_allow_mask, synthetic
+from tests.helpers import DotnetRandom, ReplayRandom, oracle_tokens, to_oracle
+
+pytestmark = pytest.mark.gpu
+NEG_INF = np.float32("-inf")
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = SamplerContext(0)
+    c.L.sr_selftest_seqsum.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_void_p]
+    yield c
+    c.close()
+
+
+def _cuda(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _gpu_seq_sum(ctx, x, s0=0.0, target=float("nan")):
+    import torch
+
+    xd = _cuda(np.asarray(x, dtype=np.float32))
+    s = torch.zeros(1, dtype=torch.float32, device="cuda")
+    idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ctx._check(ctx.L.sr_selftest_seqsum(ctx.h, C.c_void_p(xd.data_ptr()), len(x), s0, target,
+                                        C.c_void_p(s.data_ptr()), C.c_void_p(idx.data_ptr())))
+    ctx.synchronize()
+    return np.float32(s.cpu().numpy()[0]), int(idx.cpu().numpy()[0])
+
+
+def test_exact_running_sum_matches_the_left_to_right_loop(ctx):
+    rng = np.random.default_rng(4)
+    cases = []
+    # softmax-like terms spanning many binades, in index order
+    for n in (1, 5, 16, 17, 1000, 16384, 16385, 50000, 151936):
+        z = rng.normal(0, 2.5, n)
+        cases.append(np.exp(z - z.max()).astype(np.float32))
+    # exact ties: terms that are exactly half an ulp of the running sum, with odd and even states
+    t = np.full(4000, 2.0 ** -24, dtype=np.float32)
+    cases.append(np.concatenate([[1.0], t]).astype(np.float32))
+    cases.append(np.concatenate([[1.0 + 2.0 ** -23], t]).astype(np.float32))
+    cases.append(np.concatenate([[1.0], np.tile([2.0 ** -24, 2.0 ** -23, 3 * 2.0 ** -25], 3000)]).astype(np.float32))
+    # subnormals, zeros, a late large term, all-zero
+    cases.append((rng.random(30000) * 1e-44).astype(np.float32))
+    cases.append(np.concatenate([np.zeros(500), rng.random(20000) * 1e-39, [3.5], rng.random(9000)]).astype(np.float32))
+    cases.append(np.zeros(20000, dtype=np.float32))
+    # many binade crossings inside one tile
+    cases.append((2.0 ** np.arange(-60, 40, 0.01)).astype(np.float32))
+    cases.append(rng.random(100000).astype(np.float32))
+    for x in cases:
+        want, _ = orc.seq_sum(x)
+        got, _ = _gpu_seq_sum(ctx, x)
+        assert got.tobytes() == want.tobytes(), (len(x), got, want)
+        # search: first index whose running sum reaches the target
+        for frac in (0.0, 1e-9, 0.3, 0.77, 0.999999, 1.5):
+            tgt = np.float32(frac * float(want))
+            ws, wi = orc.seq_sum(x, 0.0, float(tgt))
+            gs, gi = _gpu_seq_sum(ctx, x, 0.0, float(tgt))
+            assert gi == wi, (len(x), frac, gi, wi)
+    # a non-zero start
+    x = cases[3]
+    assert _gpu_seq_sum(ctx, x, 0.75)[0].tobytes() == orc.seq_sum(x, 0.75)[0].tobytes()
+
+
+def _check_rows(ctx, logits, params, uniforms, allow_mask=None, mask_active=None):
+    got, flags = ctx.sample_batch(_cuda(logits), params, uniforms, allow_mask, mask_active, return_flags=True)
+    want = oracle_tokens(logits, params, uniforms, allow_mask, mask_active)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, f"rows {bad[:8]} differ: gpu {got[bad[:8]]} oracle {want[bad[:8]]} flags {flags[bad[:8]]}"
+    return flags
+
+
+def _check_distribution(ctx, logits, params, allow_mask=None, mask_active=None):
+    got = ctx.build_distribution(_cuda(logits), params, None, allow_mask, mask_active).cpu().numpy()
+    for r, p in enumerate(params):
+        row = logits[r]
+        if allow_mask is not None and (mask_active is None or mask_active[r]):
+            row = orc.apply_allow_mask(row, allow_mask[r])
+        want = orc.build_filtered_distribution(row, to_oracle(p))
+        assert np.array_equal(got[r] > 0, want > 0), f"row {r}: support differs"
+        nz = want > 0
+        assert np.allclose(got[r][nz], want[nz], rtol=1e-5, atol=0), f"row {r}"
+        # the arithmetic is the reference's, so the bits agree as well
+        assert np.array_equal(got[r].view(np.uint32), want.view(np.uint32)), f"row {r}: bits differ"
+
+
+def test_slow_path_small_rows_every_stage(ctx):
+    rng = np.random.default_rng(31)
+    for trial in range(25):
+        rows = int(rng.integers(1, 7))
+        n = int(rng.integers(1, 900))
+        logits = (rng.integers(-14, 14, (rows, n)) / 2.0).astype(np.float32)
+        logits[rng.random((rows, n)) < 0.15] = NEG_INF
+        params = []
+        for _ in range(rows):
+            hist = rng.integers(-3, n + 3, int(rng.integers(0, 12))).tolist()
+            bias = {int(rng.integers(-2, n + 2)): float(rng.normal(0, 3)) for _ in range(int(rng.integers(0, 4)))}
+            params.append(SamplingParams(
+                Temperature=float(rng.choice([0.0, 0.5, 1.0, 1.7])), TopK=int(rng.choice([0, 0, 3, n + 5])),
+                TopP=float(rng.choice([1.0, 0.9, 0.5])), MinP=float(rng.choice([0.0, 0.05, 0.3])),
+                RepetitionPenalty=float(rng.choice([1.0, 1.3, 0.8])), PresencePenalty=float(rng.choice([0.0, 0.4, -0.3])),
+                FrequencyPenalty=float(rng.choice([0.0, 0.25])), RepeatLastN=int(rng.choice([0, 3, 64])),
+                PreviousTokens=hist, LogitBias=bias or None))
+        u = rng.random(rows)
+        _check_rows(ctx, logits, params, u)
+        _check_distribution(ctx, logits, params)
+
+
+def test_reference_known_answers_slow_path():
+    # SamplerTests.cs: logit bias, BuildFilteredDistribution, SampleWithDistribution, ResampleResidual
+    r = DotnetRandom(42)
+    assert 0 not in {Sampler.Sample([10, 1, 1, 1], SamplingParams(LogitBias={0: -100.0}), r) for _ in range(100)}
+    r = DotnetRandom(42)
+    assert {Sampler.Sample([0, 0, 0, 0], SamplingParams(LogitBias={2: 100.0}), r) for _ in range(100)} == {2}
+    assert 0 <= Sampler.Sample([1, 2, 3], SamplingParams(LogitBias={999: 100.0, -1: 100.0}), DotnetRandom(42)) <= 2
+    assert Sampler.Sample([10, 9.8], SamplingParams(Temperature=0.0, PresencePenalty=1.0, PreviousTokens=[0])) == 1
+    probs = Sampler.BuildFilteredDistribution([1.0, 2.0, 3.0, 0.0], SamplingParams()).cpu().numpy()
+    e = np.exp(np.array([1.0, 2.0, 3.0, 0.0]) - 3.0)
+    assert np.allclose(probs, e / e.sum(), atol=5e-6) and abs(probs.sum() - 1) < 5e-6
+    probs = Sampler.BuildFilteredDistribution([1, 9, 3, 2], SamplingParams(Temperature=0.0)).cpu().numpy()
+    assert probs[1] == 1.0 and probs[0] + probs[2] + probs[3] == 0.0
+    probs = Sampler.BuildFilteredDistribution([5, 4, 3, 2, 1], SamplingParams(TopK=2)).cpu().numpy()
+    assert probs[0] > 0 and probs[1] > 0 and probs[2:].sum() == 0 and abs(probs.sum() - 1) < 5e-6
+    with pytest.raises(ValueError):
+        Sampler.BuildFilteredDistribution([1, 2, 3], SamplingParams(), probs_len=4)
+    tok, probs = Sampler.SampleWithDistribution([0, 12, 0, 0], SamplingParams(Temperature=0.1), DotnetRandom(7))
+    assert tok == 1 and probs[1] > 0.99
+    r = DotnetRandom(3)
+    for _ in range(50):
+        assert Sampler.ResampleResidual([0, .5, .5, 0], [0, 1.0, 0, 0], r) == 2
+    assert 0 <= Sampler.ResampleResidual([.25] * 4, [.25] * 4, DotnetRandom(5)) < 4
+    with pytest.raises(ValueError):
+        Sampler.ResampleResidual([0.0] * 4, [0.0] * 3, DotnetRandom(1))
+    with pytest.raises(TypeError):
+        Sampler.SampleFromProbs([0.5, 0.5], None)
+    # draw quirks: u == 0 -> index 0 even when probs[0] == 0; rounding fallback -> last index
+    assert Sampler.SampleFromProbs([0.0, 1.0], ReplayRandom([0.0])) == 0
+    assert Sampler.SampleFromProbs([0.25, 0.25, 0.25], ReplayRandom([0.99])) == 2
+    # fully masked row -> uniform over all tokens
+    assert Sampler.Sample([NEG_INF] * 4, SamplingParams(), ReplayRandom([0.6])) == 2
+
+
+def test_config2_shape(ctx):
+    w = synthetic.config2(rows=8)
+    flags = _check_rows(ctx, w.logits, w.params, w.uniforms)
+    assert np.all(flags & 4)
+    _check_distribution(ctx, w.logits[:2], w.params[:2])
+
+
+def test_config4_shape_masks_and_large_nuclei(ctx):
+    w = synthetic.config4(rows=12)
+    _check_rows(ctx, w.logits, w.params, w.uniforms, w.allow_mask, w.mask_active)
+    sampled = [i for i in range(12) if w.params[i].Temperature > 0][:3]
+    _check_distribution(ctx, w.logits[sampled], [w.params[i] for i in sampled], w.allow_mask[sampled],
+                        w.mask_active[sampled])
+
+
+def test_top_k_above_the_kernel_limit_goes_down_the_slow_path_of_the_oracle_too(ctx):
+    # TopK >= vocab disables top-k in the reference (Sampler.cs:38,71); huge LogitBias rows keep ties at the k-th value
+    rng = np.random.default_rng(2)
+    logits = rng.normal(0, 1.5, (3, 5000)).astype(np.float32)
+    logits[1, 100:140] = 3.25   # ties at the k-th value survive ApplyTopK
+    params = [SamplingParams(TopK=5000), SamplingParams(TopK=20, LogitBias={-1: 0.0}, TopP=0.9),
+              SamplingParams(TopK=7, LogitBias={5: 2.0}, MinP=0.01, Temperature=0.7)]
+    _check_rows(ctx, logits, params, rng.random(3))
+    _check_distribution(ctx, logits, params)
+
+
+def test_sample_from_probs_and_resample_residual_rows(ctx):
+    rng = np.random.default_rng(9)
+    V = 40_000
+    z = rng.normal(0, 2, (6, V))
+    p = (np.exp(z) / np.exp(z).sum(1, keepdims=True)).astype(np.float32)
+    z2 = z + rng.normal(0, 0.5, (6, V))
+    q = (np.exp(z2) / np.exp(z2).sum(1, keepdims=True)).astype(np.float32)
+    q[4] = p[4]                      # empty residual -> falls back to sampling p
+    u = rng.random(6)
+    u[5] = 0.0
+    got = ctx.sample_from_probs(_cuda(p), u)
+    for r in range(6):
+        assert got[r] == orc.sample_from_probs(p[r], orc.Rng(replay=[u[r]]))
+    got = ctx.resample_residual(_cuda(p), _cuda(q), u)
+    for r in range(6):
+        assert got[r] == orc.resample_residual(p[r], q[r], orc.Rng(replay=[u[r]])), r
+
+
+def _spec_case(rows, L, V, params, seed, filtered_q):
+    rng = np.random.default_rng(seed)
+    draft = synthetic.zipf_head_logits(rng, rows * L, V).reshape(rows, L, V)
+    target = np.empty((rows, L + 1, V), dtype=np.float32)
+    target[:, :L] = draft + rng.normal(0, 0.5, (rows, L, V)).astype(np.float32)
+    target[:, L] = synthetic.zipf_head_logits(rng, rows, V)
+    q = np.empty((rows, L, V), dtype=np.float32)
+    toks = np.empty((rows, L), dtype=np.int32)
+    for r in range(rows):
+        for i in range(L):
+            t, d = orc.sample_with_distribution(draft[r, i], to_oracle(params[r] if filtered_q else SamplingParams()),
+                                                orc.Rng(replay=[rng.random()]))
+            q[r, i], toks[r, i] = d, t
+    return target, q, toks, rng.random((rows, L + 1))
+
+
+def _check_spec(ctx, target, q, toks, params, u):
+    acc, out = ctx.spec_verify(_cuda(target), _cuda(q), _cuda(toks), params, u)
+    for r in range(target.shape[0]):
+        wa, wt = orc.spec_verify_row(target[r], q[r], toks[r], to_oracle(params[r]), orc.Rng(replay=u[r]))
+        assert acc[r] == wa, (r, acc[r], wa)
+        assert list(out[r][: wa + 1]) == list(wt), (r, out[r], wt)
+        assert np.all(out[r][wa + 1:] == -1)
+
+
+def test_speculative_verification_rows(ctx):
+    V, L = 20_000, 4
+    # unfiltered p and q (the benchmark's choice), the CLI defaults, and the looser p-min accept
+    p1 = [SamplingParams() for _ in range(6)]
+    _check_spec(ctx, *_spec_case(6, L, V, p1, 1, False)[:3], p1, _spec_case(6, L, V, p1, 1, False)[3])
+    p2 = [SamplingParams(Temperature=0.7, TopK=40, TopP=0.95, MinP=0.05) for _ in range(6)]
+    t, q, k, u = _spec_case(6, L, V, p2, 2, True)
+    _check_spec(ctx, t, q, k, p2, u)
+    p3 = [SamplingParams(Temperature=0.8, SpecDraftPMin=0.05) for _ in range(4)] + [SamplingParams(Temperature=0.0)]
+    t, q, k, u = _spec_case(5, L, V, p3, 3, True)
+    _check_spec(ctx, t, q, k, p3, u)
+
+
+def test_reference_distribution_preservation_invariant(ctx):
+    # SpeculativeSamplingTests.cs:21-50 at a GPU-sized batch: with fixed target/draft rows the emitted
+    # histogram of (accepted drafts + correction) follows softmax(target) regardless of the draft.
+    P_T = np.array([0.2, 2.5, 0.1, 1.0, 0.3, 1.8, 0.0, 0.5], dtype=np.float32)
+    Q_D = np.array([2.0, 0.1, 1.5, 0.2, 1.0, 0.0, 2.2, 0.3], dtype=np.float32)
+    rows, L = 4096, 3
+    rng = DotnetRandom(12345)
+    p = SamplingParams()
+    q1 = orc.build_filtered_distribution(Q_D, to_oracle(p))
+    qc = np.cumsum(q1)
+    toks = np.searchsorted(qc, [rng.NextDouble() for _ in range(rows * L)]).clip(0, 7).astype(np.int32).reshape(rows, L)
+    target = np.tile(P_T, (rows, L + 1, 1))
+    q = np.tile(q1, (rows, L, 1))
+    u = np.array([rng.NextDouble() for _ in range(rows * (L + 1))]).reshape(rows, L + 1)
+    acc, out = ctx.spec_verify(_cuda(target), _cuda(q), _cuda(toks), [p] * rows, u)
+    # first emitted token of every step is distributed as softmax(target)
+    first = np.array([out[r][0] for r in range(rows)])
+    e = np.exp(P_T - P_T.max())
+    assert np.abs(np.bincount(first, minlength=8) / rows - e / e.sum()).max() < 0.03
+    assert 0.01 < acc.mean() / L < 0.99
+
+
+def test_mtp_accept_draft(ctx):
+    import torch
+
+    rng = np.random.default_rng(6)
+    V = 50_000
+    logits = rng.normal(0, 2, (8, V)).astype(np.float32)
+    am = logits.argmax(1)
+    draft = np.array([am[0], 5, am[2], 7, 11, am[5], 13, 17], dtype=np.int32)
+    logits[3, 7] = logits[3].max() - 0.2     # high-probability non-argmax draft
+    for p_min in (1.0, 0.2, 0.001):
+        g_am, g_ok, g_pr = ctx.mtp_verify(_cuda(logits), torch.from_numpy(draft).cuda(), p_min)
+        for r in range(8):
+            ok, pr = orc.mtp_accept_draft(int(draft[r]), int(am[r]), logits[r], p_min)
+            assert g_am[r] == am[r] and bool(g_ok[r]) == ok
+            assert abs(g_pr[r] - pr) <= 1e-5 * max(pr, 1e-30)
