@@ -15,6 +15,7 @@ Workloads (opentail/stingray_amd/synthetic.py):
   c3_fp32       fp32, no penalties
   c1            batch 1 x vocab 49,152 (us/step is the figure of interest)
   c2, c4        full-vocabulary path (batch 64 / batch 32 with allow-masks)
+  c5            speculative verification, batch 16 x 8 drafts x vocab 262,144 (sr_spec_verify_launch)
 """
 from __future__ import annotations
 
@@ -47,6 +48,8 @@ def make_workload(name: str):
         return synthetic.config2()
     if name == "c4":
         return synthetic.config4()
+    if name == "c5":
+        return synthetic.config5()
     raise SystemExit(f"unknown workload {name}")
 
 
@@ -73,6 +76,91 @@ def cpu_baseline(w, budget_s: float):
     return done / el, done, el
 
 
+def bench_spec(args, w, ctx, stream):
+    """Speculative verification: target logits [rows, L+1, V], draft distributions [rows, L, V] and draft
+    tokens resident; two distinct input sets are rotated (2 x 285 MB exceeds the Infinity Cache)."""
+    import torch
+
+    from opentail.stingray_amd import SamplingParams
+    from oracle import binding as orc
+    from tests.helpers import to_oracle
+
+    L = w.extra["n_draft"]
+    rows = len(w.params)
+    V = w.vocab
+    sets = []
+    for k in range(2):
+        draft = torch.from_numpy(np.roll(w.extra["draft_logits"], k * 3, axis=0)).cuda()
+        q = ctx.build_distribution(draft, [SamplingParams()] * (rows * L))          # q = softmax(draft)
+        toks = torch.from_numpy(ctx.sample_from_probs(q, w.extra["draft_uniforms"])).cuda().reshape(rows, L)
+        target = torch.from_numpy(np.roll(w.logits.reshape(rows, L + 1, V), k, axis=0)).cuda()
+        batch = ctx.new_batch().upload(w.params, V, w.uniforms, uniforms_per_row=L + 1)
+        acc = torch.empty(rows, dtype=torch.int32, device="cuda")
+        out = torch.empty((rows, L + 1), dtype=torch.int32, device="cuda")
+        sets.append((target, q.reshape(rows, L, V), toks.contiguous(), batch, acc, out))
+    import ctypes as C
+
+    def step(i):
+        t, q, k, b, acc, out = sets[i % 2]
+        ctx._check(ctx.L.sr_spec_verify_launch(ctx.h, b.h, C.c_void_p(t.data_ptr()), C.c_void_p(q.data_ptr()),
+                                               C.c_void_p(k.data_ptr()), L, C.c_void_p(acc.data_ptr()),
+                                               C.c_void_p(out.data_ptr())))
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for i in range(args.steps):
+        step(i)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_us = ev0.elapsed_time(ev1) * 1e3 / args.steps
+
+    t, q, k, b, acc, out = sets[0]
+    acc_h, out_h = acc.cpu().numpy(), out.cpu().numpy()
+    parity = None
+    if not args.no_parity:
+        n_chk = 3
+        tn, qn, kn = t[:n_chk].cpu().numpy(), q[:n_chk].cpu().numpy(), k[:n_chk].cpu().numpy()
+        bad = 0
+        for r in range(n_chk):
+            wa, wt = orc.spec_verify_row(tn[r], qn[r], kn[r], to_oracle(w.params[r]), orc.Rng(replay=w.uniforms[r]))
+            bad += int(wa != acc_h[r] or list(wt) != list(out_h[r][: wa + 1]))
+        parity = {"rows_checked": n_chk, "mismatches": bad}
+    cpu = None
+    if args.cpu_seconds > 0:
+        tn, qn, kn = t[:4].cpu().numpy(), q[:4].cpu().numpy(), k[:4].cpu().numpy()
+        c0 = time.perf_counter()
+        done = 0
+        while time.perf_counter() - c0 < args.cpu_seconds and done < 64:
+            r = done % 4
+            orc.spec_verify_row(tn[r], qn[r], kn[r], to_oracle(w.params[r]), orc.Rng(replay=w.uniforms[r]))
+            done += 1
+        el = time.perf_counter() - c0
+        cpu = {"value": done / el, "unit": "rows/s", "cores": 1, "kind": "port",
+               "sample": f"{done} row verifications (8 drafts each) of the same workload on one thread, {el:.1f} s"}
+    # every target position is read for its distribution; the draft distribution of the rejected position
+    # and the bonus / residual pass add one more row each
+    alg_bytes = rows * (L + 1) * V * 4 + rows * V * 4 + rows * L * 8
+    achieved = alg_bytes / (dev_us * 1e-6) / 1e9
+    emitted = float((acc_h + 1).mean())
+    out_j = {
+        "metric": f"verified rows/sec at B={rows}x{L} drafts x {V} vocab", "value": rows * args.steps / wall,
+        "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps,
+        "us_per_step_device": dev_us, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (target = draft + N(0, .5^2), q = softmax(draft), 2 rotated resident sets)",
+        "config": {"workload": "c5", "rows": rows, "n_draft": L, "vocab": V, "mean_tokens_emitted_per_row": emitted},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                     "kernel": "k_full_row", "kernel_us": dev_us},
+        "cpu_baseline": cpu, "parity": parity,
+    }
+    print(json.dumps(out_j))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -81,6 +169,9 @@ def main():
     ap.add_argument("--workload", default="c3_fp32_full")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget (0 = skip)")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain device copy of one logits buffer (known size) so that a counter run\n"
+                         "under rocprofv3 --pmc has a reference dispatch to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU (rows shard across GPUs without any exchange); "
@@ -99,6 +190,9 @@ def main():
     stream = torch.cuda.Stream()            # a real (non-null) stream shared by torch and the library,
     torch.cuda.set_stream(stream)           # so HIP events recorded here bracket the sampler's kernels
     ctx = SamplerContext(0)
+
+    if args.workload == "c5":
+        return bench_spec(args, w, ctx, stream)
 
     # four distinct resident logits buffers (row-rotated copies of the seeded tensor) + their batches
     n_buf = 4
@@ -123,6 +217,11 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
+    if args.copy_probe:
+        probe = torch.empty_like(bufs[0])
+        for _ in range(3):
+            probe.copy_(bufs[0])   # reads and writes bufs[0].numel() * element_size bytes
+        torch.cuda.synchronize()
 
     ev0 = torch.cuda.Event(enable_timing=True)
     ev1 = torch.cuda.Event(enable_timing=True)
@@ -154,7 +253,7 @@ def main():
     alg_bytes = rows * vocab * elem + (0 if w.allow_mask is None else w.allow_mask.nbytes) + rows * 8
     achieved = alg_bytes / (kern_us * 1e-6) / 1e9
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", f"traffic_{args.workload}.json")
+    tpath = os.path.join(ROOT, "profiles", f"traffic_{args.workload}.json.txt")
     if os.path.exists(tpath):
         try:
             traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
@@ -186,7 +285,8 @@ def main():
                    "chain": "penalties+top-k+top-p+min-p" if args.workload == "c3_fp32_full" else args.workload},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "algorithmic_bytes_per_launch": alg_bytes, "kernel": "k_topk_rows",
+                     "algorithmic_bytes_per_launch": alg_bytes,
+                     "kernel": "k_topk_rows" if args.workload.startswith(("c1", "c3")) else "k_full_row",
                      "kernel_us": kern_us},
         "cpu_baseline": cpu,
         "parity": parity,
