@@ -316,9 +316,12 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.row_stride = row_stride_elems;
         a.vocab = b->vocab;
         a.dtype = dtype;
+        a.n_rows = n_sel;
         topk_geometry(b->vocab, dtype, n_sel, b->max_sel, ctx->cu_count, &a.chunks, &a.chunk_len);
         if ((int64_t)a.chunks * std::min(a.chunk_len, 2 * b->max_sel + 128) > SR_TK_TAIL_CAP || a.chunks > SR_TK_MAX_CHUNKS)
             return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary x (top_k + history) too large for the selection kernel");
+        // one full round of resident workgroups (two per CU) between a row's chunks and its tail
+        a.tail_lag = std::min(n_sel, std::max(1, (2 * ctx->cu_count + a.chunks - 1) / a.chunks));
         const size_t slots = (size_t)n_sel * a.chunks;
         SR_HIP(ctx, ctx->cand_val.reserve(slots * SR_TK_CAP * sizeof(float), st));
         SR_HIP(ctx, ctx->cand_idx.reserve(slots * SR_TK_CAP * sizeof(int32_t), st));

@@ -18,7 +18,9 @@ struct SrTopkArgs {
     int64_t row_stride;      // elements
     int32_t vocab;
     int32_t dtype;           // 0 = f32, 1 = bf16
-    int32_t chunks;          // workgroups per row
+    int32_t chunks;          // chunk workgroups per row
+    int32_t tail_lag;        // the tail of row i is dispatched after the chunks of row i + tail_lag (<= n_rows)
+    int32_t n_rows;          // rows in this launch: grid = n_rows * chunks chunk workgroups + n_rows tail workgroups
     int32_t chunk_len;       // elements per chunk
     const int32_t* row_list; // rows handled by this launch (device)
     const SrRow* rows;

@@ -230,6 +230,104 @@ __device__ __forceinline__ void block_bitonic_sort_desc(uint32_t (&hi)[kSortRegs
     __syncthreads();
 }
 
+// ---- sample sort, descending, of m (> 128) 3-word keys held in registers ---------------------------
+// 63 splitters (a 64-element sample sorted by one wave) cut the keys into 64..65 buckets; every key finds
+// its bucket by binary search, is scattered bucket-contiguously, and ranks itself against the few members
+// of its own bucket.  Far fewer instructions than a full bitonic network.  The sorted (hi, lo) words end
+// up in sm.xa / sm.xc at positions [0, m); sm.vals / idxs / probs are used as the scatter area.
+template <bool kThree>
+__device__ __forceinline__ void block_sample_sort_desc(const uint32_t (&hi)[kSortRegs], const uint32_t (&mid)[kSortRegs],
+                                                       const uint32_t (&lo)[kSortRegs], int m, TopkSmem& sm)
+{
+    const int tid = threadIdx.x, lane = sr_lane();
+    uint32_t* bh = (uint32_t*)sm.vals;
+    uint32_t* bm = (uint32_t*)sm.idxs;
+    uint32_t* bl = (uint32_t*)sm.probs;
+    uint32_t* bcnt = sm.hist;        // [0, 65)
+    uint32_t* boff = sm.hist + 128;  // [0, 66)
+    uint32_t* sph = sm.hist + 64;    // splitters do not fit hist: kept in xb tail-free slots below
+    auto less = [&](uint32_t ah, uint32_t am, uint32_t al, uint32_t b_h, uint32_t b_m, uint32_t b_l) -> bool {
+        if (kThree) return key3_less(ah, am, al, b_h, b_m, b_l);
+        return ah < b_h || (ah == b_h && al < b_l);
+    };
+    (void)sph;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) {
+        const int i = r * kThreads + tid;
+        if (i < m) { sm.xa[i] = hi[r]; sm.xb[i] = mid[r]; sm.xc[i] = lo[r]; }
+    }
+    if (tid < 65) bcnt[tid] = 0u;
+    __syncthreads();
+    // every wave sorts the same 64-element sample (no barrier needed to share the splitters)
+    uint32_t sh, smid, sl;
+    {
+        const int src = (int)(((long long)lane * m) >> 6);
+        sh = sm.xa[src]; smid = sm.xb[src]; sl = sm.xc[src];
+#pragma unroll
+        for (int k2 = 2; k2 <= SR_WAVE; k2 <<= 1) {
+#pragma unroll
+            for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
+                const uint32_t ph = __shfl_xor(sh, j2), pm = kThree ? __shfl_xor(smid, j2) : 0u, pl = __shfl_xor(sl, j2);
+                const bool want_max = (((lane & k2) == 0) == ((lane & j2) == 0));
+                const bool l = less(sh, smid, sl, ph, pm, pl);
+                if (want_max == l) { sh = ph; smid = pm; sl = pl; }
+            }
+        }
+    }
+    // lane j now holds the j-th largest sample element; lanes 0..62 are the splitters
+    int bucket[kSortRegs], slot[kSortRegs];
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) {
+        const int i = r * kThreads + tid;
+        bucket[r] = 0; slot[r] = 0;
+        // number of splitters strictly greater than the key (binary search over lanes 0..62)
+        int lo_b = 0, hi_b = 63;
+#pragma unroll
+        for (int it = 0; it < 6; it++) {
+            const int midb = (lo_b + hi_b) >> 1;
+            const uint32_t ph = __shfl(sh, midb), pm = kThree ? __shfl(smid, midb) : 0u, pl = __shfl(sl, midb);
+            const bool splitter_greater = less(hi[r], mid[r], lo[r], ph, pm, pl);
+            if (lo_b < hi_b) { if (splitter_greater) lo_b = midb + 1; else hi_b = midb; }
+        }
+        if (i < m) {
+            bucket[r] = lo_b;
+            slot[r] = (int)atomicAdd(&bcnt[lo_b], 1u);
+        }
+    }
+    __syncthreads();
+    if (tid < SR_WAVE) {
+        // exclusive scan of the 65 bucket counts (lane l owns bucket l; bucket 64 follows the total)
+        const int c = (int)bcnt[lane];
+        const int incl = sr_wave_incl_scan_i32(c);
+        boff[lane] = (uint32_t)(incl - c);
+        if (lane == SR_WAVE - 1) { boff[64] = (uint32_t)incl; boff[65] = (uint32_t)incl + bcnt[64]; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) {
+        const int i = r * kThreads + tid;
+        if (i < m) {
+            const int p = (int)boff[bucket[r]] + slot[r];
+            bh[p] = hi[r]; if (kThree) bm[p] = mid[r]; bl[p] = lo[r];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSortRegs; r++) {
+        const int i = r * kThreads + tid;
+        if (i < m) {
+            const int b0 = (int)boff[bucket[r]], b1 = (int)boff[bucket[r] + 1];
+            int rank = b0;
+            for (int p = b0; p < b1; p++)
+                rank += less(hi[r], mid[r], lo[r], bh[p], kThree ? bm[p] : 0u, bl[p]) ? 1 : 0;
+            sm.xa[rank] = hi[r];
+            sm.xc[rank] = lo[r];
+        }
+    }
+    __syncthreads();
+}
+
 __device__ __forceinline__ int next_pow2(int n)
 {
     int p = 1;
@@ -530,17 +628,26 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             lo[r] = (i < m2) ? sm.xc[i] : 0u;
         }
     }
-    if (use_edits) block_bitonic_sort_desc<true>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
-    else block_bitonic_sort_desc<false>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
-
     // the k best that are still alive
     const int k = min(rd.top_k, m2);  // top_k <= sel; everything past m2 is a no-op or does not exist
+    if (m2 > 128) {
+        if (use_edits) block_sample_sort_desc<true>(hi, mid, lo, m2, sm);
+        else block_sample_sort_desc<false>(hi, mid, lo, m2, sm);
+        // sorted (value key, ~index) are in xa / xc; the scatter area (vals / idxs / probs) is free again
+        for (int i = tid; i < k; i += kThreads) {
+            sm.vals[i] = sr_okey_inv(sm.xa[i]);
+            sm.idxs[i] = (int)(0xffffffffu - sm.xc[i]);
+        }
+    } else {
+        if (use_edits) block_bitonic_sort_desc<true>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
+        else block_bitonic_sort_desc<false>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
 #pragma unroll
-    for (int r = 0; r < kSortRegs; r++) {
-        const int i = r * kThreads + tid;
-        if (i < k) {
-            sm.vals[i] = sr_okey_inv(hi[r]);
-            sm.idxs[i] = (int)(0xffffffffu - lo[r]);
+        for (int r = 0; r < kSortRegs; r++) {
+            const int i = r * kThreads + tid;
+            if (i < k) {
+                sm.vals[i] = sr_okey_inv(hi[r]);
+                sm.idxs[i] = (int)(0xffffffffu - lo[r]);
+            }
         }
     }
     __syncthreads();
@@ -622,7 +729,55 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     using VO = VecOps<EPV>;
     const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
     const int S = a.chunks;
-    const int slot = blockIdx.x / S, c = blockIdx.x - slot * S;
+    // Grid order: [chunks of row 0] ... and, from row `lag` on, the tail of row i - lag right after the chunks
+    // of row i; the tails of the last `lag` rows close the grid.  A tail workgroup is therefore dispatched
+    // after all chunk workgroups of its row (it waits, bounded, only on work that is already running),
+    // about one full round of workgroups later, so it rarely waits at all and overlaps later rows' streaming.
+    const int lag = a.tail_lag;
+    const int bid = (int)blockIdx.x;
+    const int head = lag * S;                       // rows [0, lag): chunks only
+    const int per = S + 1;                          // rows [lag, n_rows): S chunks + one tail
+    const int mid_end = head + (a.n_rows - lag) * per;
+    int slot_, c_;
+    bool is_tail;
+    if (bid < head) {
+        slot_ = bid / S; c_ = bid - slot_ * S; is_tail = false;
+    } else if (bid < mid_end) {
+        const int g = (bid - head) / per, w = (bid - head) - g * per;
+        is_tail = (w == S);
+        slot_ = is_tail ? g : lag + g;
+        c_ = w;
+    } else {
+        is_tail = true;
+        slot_ = (a.n_rows - lag) + (bid - mid_end);
+        c_ = 0;
+    }
+    if (is_tail) {
+        const int tslot = slot_;
+        const int trow = a.row_list[tslot];
+        if (tid == 0) {
+            uint32_t ok = 0u;
+            for (int it = 0; it < (1 << 22); it++) {
+                if (sr_load_agent(&a.row_done[tslot]) == (uint32_t)S) { ok = 1u; break; }
+                __builtin_amdgcn_s_sleep(4);
+            }
+            sr_store_agent(&a.row_done[tslot], 0u);  // ready for the next launch
+            sm.bcast[7] = ok;
+        }
+        __syncthreads();
+        if (!sm.bcast[7]) {
+            if (tid == 0) {
+                a.out_tokens[trow] = -1;
+                if (a.out_flags) a.out_flags[trow] = SR_KFLAG_UNSUPPORTED;
+            }
+            return;
+        }
+        SR_PROF(a, 4);
+        topk_row_tail(a, tslot, trow, a.rows[trow], sm);
+        SR_PROF(a, 15);
+        return;
+    }
+    const int slot = slot_, c = c_;
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
     const int V = a.vocab;
@@ -791,16 +946,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     // hand the chunk over: drain this wave's write-through stores, meet, then count the chunk in
     sr_drain_stores();
     __syncthreads();
-    if (tid == 0) {
-        uint32_t prev = __hip_atomic_fetch_add(&a.row_done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        sm.bcast[7] = (prev == (uint32_t)(S - 1)) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (!sm.bcast[7]) return;
-    if (tid == 0) sr_store_agent(&a.row_done[slot], 0u);  // ready for the next launch
-    SR_PROF(a, 4);
-    topk_row_tail(a, slot, row, rd, sm);
-    SR_PROF(a, 15);
+    if (tid == 0) __hip_atomic_fetch_add(&a.row_done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace
@@ -808,7 +954,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
 {
     if (n_rows <= 0) return hipSuccess;
-    dim3 grid((unsigned)(n_rows * a.chunks)), block(kThreads);
+    dim3 grid((unsigned)(n_rows * a.chunks + n_rows)), block(kThreads);  // chunk workgroups + one tail per row
     if (a.dtype == 1)
         hipLaunchKernelGGL(k_topk_rows<8>, grid, block, 0, stream, a);
     else
