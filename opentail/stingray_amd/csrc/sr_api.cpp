@@ -23,7 +23,7 @@ void topk_geometry(int vocab, int dtype, int n_rows, int max_sel, int cu_count, 
     const int usable = window - epv;  // slack for a misaligned row start
     int s_min = (vocab + usable - 1) / usable;
     int s_par = (2 * cu_count + n_rows - 1) / std::max(n_rows, 1);  // aim for two workgroups per CU
-    int s_cap = std::min(SR_TK_MAX_CHUNKS, std::max(1, vocab / 2048));
+    int s_cap = std::min(SR_TK_MAX_CHUNKS, std::max(1, vocab / 8192));  // short chunks only multiply the candidates
     // every chunk hands at most min(chunk, 2 * sel + 128) candidates to the row tail, which holds
     // SR_TK_TAIL_CAP of them
     s_cap = std::min(s_cap, std::max(1, SR_TK_TAIL_CAP / (2 * max_sel + 128)));
