@@ -3,6 +3,7 @@
 // per-entry-point launch sequences.  No vocabulary-sized work happens on the host.
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -15,26 +16,75 @@ inline bool has_history_penalty(const sr_row_params& p)
     return p.repetition_penalty != 1.0f || p.presence_penalty != 0.0f || p.frequency_penalty != 0.0f;
 }
 
-// Chunking of a row for the selection kernel: every chunk must fit the per-workgroup register window.
-void topk_geometry(int vocab, int dtype, int n_rows, int max_sel, int cu_count, int* chunks, int* chunk_len)
+// Chunking of a row for the selection kernel: a chunk is a whole number of 64-vector blocks of the row's
+// window of 16-byte vectors and must fit the per-workgroup register window.
+void topk_geometry(int vocab, int dtype, int n_rows, int max_sel, int cu_count, int* chunks, int* chunk_vecs)
 {
     const int epv = dtype == SR_DTYPE_BF16 ? 8 : 4;
-    const int window = SR_TK_VEC * SR_TK_THREADS * epv;
-    const int usable = window - epv;  // slack for a misaligned row start
-    int s_min = (vocab + usable - 1) / usable;
+    const int window = SR_TK_VEC * SR_TK_THREADS;                  // vectors a workgroup holds
+    const int nvt = (vocab + 2 * epv - 2) / epv;                   // vectors of a row that starts mid-vector
+    int s_min = (nvt + window - 1) / window;
     int s_par = (2 * cu_count + n_rows - 1) / std::max(n_rows, 1);  // aim for two workgroups per CU
     int s_cap = std::min(SR_TK_MAX_CHUNKS, std::max(1, vocab / 8192));  // short chunks only multiply the candidates
-    // every chunk hands at most min(chunk, 2 * sel + 128) candidates to the row tail, which holds
-    // SR_TK_TAIL_CAP of them
-    s_cap = std::min(s_cap, std::max(1, SR_TK_TAIL_CAP / (2 * max_sel + 128)));
+    // all chunks of a row share the SR_TK_ROW_CAP entries of its candidate list: a wave of the per-wave scan
+    // (sel <= 64) wants SR_TK_WAVE_LIM of them, a chunk of the workgroup-wide scan 2 * sel + 128
+    if (max_sel <= 64)
+        s_cap = std::min(s_cap, SR_TK_ROW_CAP / (SR_TK_WAVE_LIM * (SR_TK_THREADS / 64)));
+    else
+        s_cap = std::min(s_cap, std::max(1, SR_TK_ROW_CAP / (2 * std::min(max_sel, SR_TK_SEL_MAX) + 128)));
     int s = std::max(s_min, std::min(s_par, s_cap));
-    int len = (vocab + s - 1) / s;
-    len = (len + 7) & ~7;
-    if (len > usable) len = usable & ~7;
-    s = (vocab + len - 1) / len;
-    // a row too long for SR_TK_MAX_CHUNKS register windows cannot be handled by the selection kernel
+    int cv = (nvt + s - 1) / s;
+    cv = (cv + 63) & ~63;
+    if (cv > window) cv = window;  // window is a multiple of 64
+    s = (nvt + cv - 1) / cv;
     *chunks = std::max(s, 1);
-    *chunk_len = std::max(len, 8);
+    *chunk_vecs = cv;
+}
+
+// (Re)builds the scan masks of a batch for logits of the given vector width and alignment.  Rows without an
+// allow-mask and without excluded history ids share one mask row when every row starts at the same offset
+// inside its first vector.
+int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long stride_bytes)
+{
+    sr_ctx* ctx = b->ctx;
+    hipStream_t st = ctx->stream;
+    const int base_mod = (int)(base_addr & 15ull), stride_mod = (int)(stride_bytes & 15ll);
+    if (b->scan_epv == epv && b->scan_base_mod == base_mod && b->scan_stride_mod == stride_mod) return SR_OK;
+    const bool can_share = stride_mod == 0 || b->rows <= 1;
+    b->h_scan.clear();
+    int shared = -1;
+    bool rows_changed = false;
+    for (int32_t r : b->h_sel_list) {
+        SrRow& d = b->h_rows[(size_t)r];
+        const uint32_t need = b->h_scan_need[(size_t)r];
+        int32_t idx;
+        if (need == 0u && can_share) {
+            if (shared < 0) { shared = (int)b->h_scan.size(); b->h_scan.push_back(SrScanDesc{r, 0u}); }
+            idx = shared;
+        } else {
+            idx = (int32_t)b->h_scan.size();
+            b->h_scan.push_back(SrScanDesc{r, need});
+        }
+        if (d.scan_row != idx) { d.scan_row = idx; rows_changed = true; }
+    }
+    b->scan_epv = epv;
+    b->scan_base_mod = base_mod;
+    b->scan_stride_mod = stride_mod;
+    if (b->h_scan.empty()) return SR_OK;
+    const int64_t blocks = ((int64_t)b->vocab + 2 * epv - 2) / epv / 64 + 1;
+    b->scan_stride = blocks * epv;
+    if (rows_changed)
+        SR_HIP(ctx, hipMemcpyAsync(b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), hipMemcpyHostToDevice, st));
+    SR_HIP(ctx, b->d_scan_desc.reserve(b->h_scan.size() * sizeof(SrScanDesc), st));
+    SR_HIP(ctx, hipMemcpyAsync(b->d_scan_desc.p, b->h_scan.data(), b->h_scan.size() * sizeof(SrScanDesc), hipMemcpyHostToDevice, st));
+    SR_HIP(ctx, b->d_scan_mask.reserve(b->h_scan.size() * (size_t)b->scan_stride * sizeof(unsigned long long), st));
+    SR_HIP(ctx, sr_launch_build_scan_mask(b->d_scan_desc.as<SrScanDesc>(), (int)b->h_scan.size(), b->d_rows.as<SrRow>(),
+                                          b->d_edits.as<SrEdit>(), b->d_mask.as<uint32_t>(), b->mask_stride,
+                                          b->d_scan_mask.as<unsigned long long>(), b->scan_stride, b->vocab, epv,
+                                          base_addr, stride_bytes, st));
+    // the host vectors are read by the async copies above
+    SR_HIP(ctx, hipStreamSynchronize(st));
+    return SR_OK;
 }
 
 }  // namespace
@@ -71,7 +121,7 @@ void sr_destroy(sr_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
-    DeviceBuf* bufs[] = {&ctx->cand_val, &ctx->cand_idx, &ctx->cand_cnt, &ctx->row_done, &ctx->argmax_best,
+    DeviceBuf* bufs[] = {&ctx->cand, &ctx->cand_cnt, &ctx->row_done, &ctx->argmax_best,
                          &ctx->work, &ctx->host_logits, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->spec_rows, &ctx->spec_probs};
@@ -117,7 +167,8 @@ void sr_batch_destroy(sr_batch* b)
 {
     if (!b) return;
     if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
-    DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_mask, &b->d_uniforms};
+    DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_scan_desc,
+                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms};
     for (DeviceBuf* d : bufs) d->release();
     delete b;
 }
@@ -150,6 +201,9 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
     b->h_edits.clear();
     b->h_sel_list.clear();
     b->h_full_list.clear();
+    b->h_scan.clear();
+    b->h_scan_need.assign((size_t)rows, 0u);
+    b->scan_epv = 0;
     b->has_mask = allow_mask != nullptr;
     b->mask_stride = allow_mask ? mask_stride_words : 0;
     b->max_sel = 0;
@@ -182,6 +236,7 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         d.mask_row = (allow_mask && (!mask_active || mask_active[r])) ? r : -1;
         d.edit_off = (int32_t)b->h_edits.size();
         d.edit_cnt = 0;
+        d.scan_row = -1;
         d.sel = 1;
 
         // Sampler.Sample dispatch (Sampler.cs:19-39)
@@ -237,15 +292,22 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
             }
             d.edit_cnt = (int32_t)ed.size() - d.edit_off;
         }
-        if (d.path == SR_PATH_GREEDY_PEN) {
-            // over-select by the number of distinct history ids: one candidate outside the history
-            // is then guaranteed (see the row tail of the selection kernel)
-            d.sel = (int32_t)std::min<int64_t>((int64_t)d.edit_cnt + 1, vocab);
+        // Penalties that can only lower a logit (Sampler.cs:281-286 with repetition >= 1, presence >= 0 and
+        // frequency >= 0) cannot lift a history token past a token outside the history: the scan then skips
+        // the history ids and asks for the k best of the rest, and the row tail fetches the history logits by
+        // id.  GreedyWithHistoryPenalties changes history ids only, whatever the sign.  Penalties that may
+        // raise a logit keep the reference's over-selection by the history length (Sampler.cs:224-225).
+        const bool lowering = p.repetition_penalty >= 1.0f && p.presence_penalty >= 0.0f && p.frequency_penalty >= 0.0f;
+        if (has_penalty && d.edit_cnt > 0 &&
+            (d.path == SR_PATH_GREEDY_PEN || (d.path == SR_PATH_TOPK && lowering))) {
+            d.flags |= SR_ROWFLAG_HIST_EXCL;
+            b->h_scan_need[(size_t)r] |= SR_SCAN_HIST;
+            d.sel = d.path == SR_PATH_TOPK ? p.top_k : 1;
+        } else if (d.path == SR_PATH_TOPK && d.edit_cnt == 0) {
+            d.sel = p.top_k;  // no history id inside the vocabulary: nothing is ever penalised
         }
-        const bool on_selection_kernel =
-            d.path == SR_PATH_TOPK || d.path == SR_PATH_GREEDY ||
-            (d.path == SR_PATH_GREEDY_PEN && d.sel <= SR_TK_SEL_MAX);
-        if (on_selection_kernel) {
+        if (d.path != SR_PATH_FULL) {
+            if (d.mask_row >= 0) b->h_scan_need[(size_t)r] |= SR_SCAN_ALLOW;
             b->h_sel_list.push_back(r);
             b->max_sel = std::max(b->max_sel, d.sel);
         } else {
@@ -274,6 +336,12 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         SR_HIP(ctx, up(b->d_uniforms, uniforms, (size_t)rows * (size_t)uniforms_per_row * sizeof(double)));
     // the host vectors are read by the async copies above
     SR_HIP(ctx, hipStreamSynchronize(st));
+    // scan masks for the layout of the last launch (16-byte aligned rows); a launch with another layout rebuilds
+    if (!b->h_sel_list.empty()) {
+        const int epv = ctx->last_epv;
+        int rc = prepare_scan(b, epv, 0ull, 0ll);
+        if (rc != SR_OK) return rc;
+    }
     return SR_OK;
 }
 
@@ -308,32 +376,33 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
 
     const int n_sel = (int)b->h_sel_list.size();
     if (n_sel > 0) {
-        if (b->max_sel > SR_TK_SEL_MAX)
-            return sr_fail(ctx, SR_ERR_UNSUPPORTED,
-                        "sr_sample_launch: top_k + history length exceeds " + std::to_string(SR_TK_SEL_MAX));
         SrTopkArgs a{};
         a.logits = logits_dev;
         a.row_stride = row_stride_elems;
         a.vocab = b->vocab;
         a.dtype = dtype;
         a.n_rows = n_sel;
-        topk_geometry(b->vocab, dtype, n_sel, b->max_sel, ctx->cu_count, &a.chunks, &a.chunk_len);
-        if ((int64_t)a.chunks * std::min(a.chunk_len, 2 * b->max_sel + 128) > SR_TK_TAIL_CAP || a.chunks > SR_TK_MAX_CHUNKS)
-            return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary x (top_k + history) too large for the selection kernel");
+        const int epv = dtype == SR_DTYPE_BF16 ? 8 : 4;
+        ctx->last_epv = epv;
+        int rc = prepare_scan(const_cast<sr_batch*>(b), epv, (unsigned long long)(uintptr_t)logits_dev,
+                              (long long)row_stride_elems * (dtype == SR_DTYPE_BF16 ? 2 : 4));
+        if (rc != SR_OK) return rc;
+        topk_geometry(b->vocab, dtype, n_sel, b->max_sel, ctx->cu_count, &a.chunks, &a.chunk_vecs);
+        if (a.chunks > SR_TK_MAX_CHUNKS)
+            return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary too large for the selection kernel");
         // one full round of resident workgroups (two per CU) between a row's chunks and its tail
         a.tail_lag = std::min(n_sel, std::max(1, (2 * ctx->cu_count + a.chunks - 1) / a.chunks));
-        const size_t slots = (size_t)n_sel * a.chunks;
-        SR_HIP(ctx, ctx->cand_val.reserve(slots * SR_TK_CAP * sizeof(float), st));
-        SR_HIP(ctx, ctx->cand_idx.reserve(slots * SR_TK_CAP * sizeof(int32_t), st));
-        SR_HIP(ctx, ctx->cand_cnt.reserve(slots * sizeof(int32_t), st));
+        SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));
+        SR_HIP(ctx, ctx->cand_cnt.reserve((size_t)std::max(n_sel, 1024) * sizeof(int32_t), st, true));
         SR_HIP(ctx, ctx->row_done.reserve((size_t)std::max(n_sel, 1024) * sizeof(uint32_t), st, true));
         a.row_list = b->d_sel_list.as<int32_t>();
         a.rows = b->d_rows.as<SrRow>();
         a.edits = b->d_edits.as<SrEdit>();
         a.mask = b->d_mask.as<uint32_t>();
         a.mask_stride = b->mask_stride;
-        a.cand_val = ctx->cand_val.as<float>();
-        a.cand_idx = ctx->cand_idx.as<int32_t>();
+        a.scan_mask = b->d_scan_mask.as<unsigned long long>();
+        a.scan_stride = b->scan_stride;
+        a.cand = ctx->cand.as<unsigned long long>();
         a.cand_cnt = ctx->cand_cnt.as<int32_t>();
         a.row_done = ctx->row_done.as<uint32_t>();
         a.uniforms = b->d_uniforms.as<double>();

@@ -48,7 +48,7 @@ struct sr_ctx {
     std::string err;
     int cu_count = 256;
     // scratch, lazily grown and reused across calls
-    DeviceBuf cand_val, cand_idx, cand_cnt, row_done, argmax_best;
+    DeviceBuf cand, cand_cnt, row_done, argmax_best;
     DeviceBuf work;          // fp32 rows of the full-vocabulary path
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits
@@ -59,6 +59,7 @@ struct sr_ctx {
     DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
+    int last_epv = 4;                    // vector width of the last launch: what an upload builds scan masks for
 };
 
 struct sr_batch {
@@ -67,9 +68,14 @@ struct sr_batch {
     std::vector<SrRow> h_rows;
     std::vector<SrEdit> h_edits;
     std::vector<int32_t> h_sel_list;   // rows on the selection kernel: TOPK and plain GREEDY
-    std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path (FULL and GREEDY_PEN)
-    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_mask, d_uniforms;
-    int64_t mask_stride = 0;
+    std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path
+    std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel
+    std::vector<uint32_t> h_scan_need; // per batch row: SR_SCAN_* bits the row's scan mask must carry
+    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms;
+    int64_t mask_stride = 0, scan_stride = 0;
+    // what the scan masks were built for: elements per 16-byte vector, the logits base address modulo 16 and
+    // the row stride in bytes modulo 16 (rows share a mask row only when all start at the same offset)
+    int32_t scan_epv = 0, scan_base_mod = -1, scan_stride_mod = -1;
     bool has_mask = false;
     int32_t max_sel = 0;
 };

@@ -12,6 +12,9 @@
 #define SR_KFLAG_UNSUPPORTED (1u << 31)
 // internal bit of SrRow.flags: the row has a history and at least one active penalty
 #define SR_ROWFLAG_HAS_PENALTY (1u << 8)
+// internal bit: the penalties can only lower a logit, so the scan skips the history ids (scan mask) and
+// the row tail fetches their logits by id instead of over-selecting by the history length
+#define SR_ROWFLAG_HIST_EXCL (1u << 9)
 
 struct SrTopkArgs {
     const void* logits;
@@ -21,15 +24,16 @@ struct SrTopkArgs {
     int32_t chunks;          // chunk workgroups per row
     int32_t tail_lag;        // the tail of row i is dispatched after the chunks of row i + tail_lag (<= n_rows)
     int32_t n_rows;          // rows in this launch: grid = n_rows * chunks chunk workgroups + n_rows tail workgroups
-    int32_t chunk_len;       // elements per chunk
+    int32_t chunk_vecs;      // 16-byte vectors per chunk, a multiple of 64
     const int32_t* row_list; // rows handled by this launch (device)
     const SrRow* rows;
     const SrEdit* edits;
     const uint32_t* mask;
     int64_t mask_stride;     // words
-    float* cand_val;         // [n_rows][chunks][SR_TK_CAP]
-    int32_t* cand_idx;
-    int32_t* cand_cnt;       // [n_rows][chunks]
+    const unsigned long long* scan_mask; // keep-bits of every row in the kernel's access order (SrRow.scan_row)
+    int64_t scan_stride;     // 64-bit words per scan row
+    unsigned long long* cand; // [n_rows][SR_TK_ROW_CAP] (value bits << 32 | index), appended by the chunks
+    int32_t* cand_cnt;       // [n_rows] append cursor, zero on entry, left zero on exit
     uint32_t* row_done;      // [n_rows], zero on entry, left zero on exit
     const double* uniforms;
     int32_t uniforms_per_row;
@@ -38,6 +42,12 @@ struct SrTopkArgs {
     unsigned long long* prof; // optional phase timestamps [grid][16] (test hook), normally null
 };
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream);
+// Builds scan row i for descs[i]; base_addr / stride_bytes are those of the logits the mask is used with
+// (they decide where a row starts inside its first 16-byte vector), epv = 4 (fp32) or 8 (bf16).
+hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, int n_scan, const SrRow* rows, const SrEdit* edits,
+                                     const uint32_t* mask, int64_t mask_stride, unsigned long long* scan_mask,
+                                     int64_t scan_stride, int vocab, int epv, unsigned long long base_addr,
+                                     long long stride_bytes, hipStream_t stream);
 
 struct SrArgmaxArgs {
     const void* logits;

@@ -1,12 +1,24 @@
-// Top-k-first sampling (the reference's SampleTopK, Sampler.cs:216-357) and plain greedy rows.
+// Top-k-first sampling (the reference's SampleTopK, Sampler.cs:216-357) and the greedy rows.
 //
-// One launch, grid = rows x chunks.  A workgroup loads one contiguous chunk of a row ONCE into
-// registers (19 x 16 B per thread), derives a safe chunk-local threshold from per-thread group maxima
-// (the sel-th largest of 2048 disjoint-group maxima can never exceed the chunk's sel-th largest
-// element), emits the few elements at or above it, and signals the row.  The workgroup that arrives
-// last for a row runs the row tail: exact top-(k + history) selection of the merged candidates by
-// (value desc, index asc) with LDS radix histograms, a bitonic sort, penalties + stable re-sort, then
-// the softmax / min-p / top-p / draw arithmetic in the reference's sequential fp32 order.
+// One launch, grid = rows x chunks chunk workgroups + one tail workgroup per row.  A chunk workgroup
+// loads one contiguous chunk of a row ONCE into registers (19 x 16 B per thread), derives a safe
+// threshold (a lower bound on the sel-th largest scanned logit), appends the few elements at or above
+// it to the row's candidate list and signals the row.  For sel <= 64 every wave works on its own:
+// the sel-th largest of its 64 lane maxima bounds the sel-th largest element from below and no
+// workgroup barrier is needed; larger sel take the sel-th largest of 2048 disjoint-group maxima of the
+// whole workgroup (LDS radix histograms).
+//
+// When the history penalties can only lower a logit (repetition >= 1, presence and frequency >= 0) the
+// scan skips the history ids (a per-row scan mask built when the batch is uploaded) and asks for the
+// top k only; the row tail fetches the history logits by id.  That set holds every token the
+// reference's top (k + history length) selection can rank among its final k: a token outside the
+// history is in the final k only if it is among the k best outside the history, and a history token
+// that the reference's over-selection misses has more than k unpenalised tokens above it.  Penalties
+// that can raise a logit keep the reference's literal over-selection.
+//
+// The row tail merges the candidates: penalties, pruning of candidates too small to change any fp32
+// sum, a sort by (value after penalties, value before, index), then the softmax / min-p / top-p / draw
+// arithmetic in the reference's sequential fp32 order.
 #include "sr_device.cuh"
 #include "sr_types.h"
 #include "sr_kernels.h"
@@ -18,15 +30,16 @@ namespace {
 constexpr int kThreads = SR_TK_THREADS;
 constexpr int kWaves = kThreads / SR_WAVE;
 constexpr int kVec = SR_TK_VEC;
-constexpr int kCap = SR_TK_CAP;
 constexpr int kSelMax = SR_TK_SEL_MAX;
+constexpr int kRowCap = SR_TK_ROW_CAP;
 constexpr uint32_t kKeyNegInf = 0x007fffffu;  // sr_okey(-inf)
 constexpr uint32_t kRowHasPenalty = SR_ROWFLAG_HAS_PENALTY;
+constexpr uint32_t kRowHistExcl = SR_ROWFLAG_HIST_EXCL;
+constexpr int kOverflowMark = 1 << 24;        // added to a row's cursor by a chunk that cannot hand over its candidates
 
-constexpr int kCandRegs = 32;                   // candidate keys a thread holds in the row tail
-constexpr int kCandMax = kCandRegs * kThreads;  // 16384 merged candidates per row
-constexpr int kMaxChunks = SR_TK_MAX_CHUNKS;
-constexpr int kSortRegs = kSelMax / kThreads;   // 4 sort elements per thread
+constexpr int kCandRegs = kRowCap / kThreads;   // candidates a thread holds in the row tail (16)
+constexpr int kSortRegs = kSelMax / kThreads;   // sort elements per thread (4)
+constexpr int kHistRegs = kSelMax / kThreads;   // history ids per thread (4)
 
 struct TopkSmem {
     uint32_t xa[kSelMax];  // gathered list, then sort exchange (three 32-bit words per element)
@@ -38,7 +51,8 @@ struct TopkSmem {
     uint32_t hist[256];
     uint32_t red[2 * kWaves];
     uint32_t bcast[16];
-    int offs[kMaxChunks + 1];
+    uint32_t boff[257];    // first list position of every histogram bin
+    uint32_t bfill[256];   // entries scattered into the bin so far
 };
 
 // ---- block-wide radix select over keys produced by a per-thread enumerator -----------------------
@@ -134,7 +148,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <int EPV> struct VecOps;
 template <> struct VecOps<4> {  // four fp32 per 16-byte vector
     static __device__ __forceinline__ float get(const u32x4& v, int c) { return sr_u2f(v[c]); }
-    static __device__ __forceinline__ void kill(u32x4& v, int c) { v[c] = 0xff800000u; }
+    static __device__ __forceinline__ void keep_if(u32x4& v, int c, bool keep) { v[c] = keep ? v[c] : 0xff800000u; }
     static __device__ __forceinline__ u32x4 neg_inf() { return (u32x4)(0xff800000u); }
 };
 template <> struct VecOps<8> {  // eight bf16 per 16-byte vector; the upcast to fp32 is exact
@@ -143,10 +157,11 @@ template <> struct VecOps<8> {  // eight bf16 per 16-byte vector; the upcast to 
         uint32_t w = v[c >> 1];
         return sr_u2f((c & 1) ? (w & 0xffff0000u) : (w << 16));
     }
-    static __device__ __forceinline__ void kill(u32x4& v, int c)
+    static __device__ __forceinline__ void keep_if(u32x4& v, int c, bool keep)
     {
-        uint32_t w = v[c >> 1];
-        v[c >> 1] = (c & 1) ? ((w & 0x0000ffffu) | 0xff800000u) : ((w & 0xffff0000u) | 0x0000ff80u);
+        const uint32_t w = v[c >> 1];
+        const uint32_t dead = (c & 1) ? ((w & 0x0000ffffu) | 0xff800000u) : ((w & 0xffff0000u) | 0x0000ff80u);
+        v[c >> 1] = keep ? w : dead;
     }
     static __device__ __forceinline__ u32x4 neg_inf() { return (u32x4)(0xff80ff80u); }
 };
@@ -370,136 +385,89 @@ __device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
     return t;
 }
 
+#define SR_INL __attribute__((always_inline))
+
 // ---- the row tail ----------------------------------------------------------------------------------
-// Called by every thread of the last workgroup of a row.  slot = position of the row in this launch.
-// The merged candidates are read once, straight into registers; every later pass runs from registers
-// or LDS.
-__device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, TopkSmem& sm)
+// Called by every thread of the tail workgroup of a row once all chunks have appended their candidates.
+// slot = position of the row in this launch, n_c = candidates in the row's list.  The list is read once,
+// straight into registers; every later pass runs from registers or LDS.
+__device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, int n_c,
+                                              TopkSmem& sm)
 {
     const int tid = threadIdx.x;
-    const int S = a.chunks;
-    const float* cval = a.cand_val + (size_t)slot * S * kCap;
-    const int* cidx = a.cand_idx + (size_t)slot * S * kCap;
-    const int* ccnt = a.cand_cnt + (size_t)slot * S;
+    const unsigned long long* cand = a.cand + (size_t)slot * kRowCap;
     const uint32_t out_flag = (rd.path == SR_PATH_TOPK) ? SR_KFLAG_TOPK : SR_KFLAG_GREEDY;
     const int sel = rd.sel;
-    auto give_up = [&](uint32_t extra, int token) {
+    auto give_up = [&](uint32_t extra, int token) SR_INL {
         if (tid == 0) {
             a.out_tokens[row] = token;
             if (a.out_flags) a.out_flags[row] = out_flag | extra;
         }
     };
+    if (sel > kSelMax || n_c < 0 || n_c > kRowCap) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
 
-    // chunk counts -> exclusive offsets
-    if (tid < S) sm.offs[tid + 1] = sr_load_agent(&ccnt[tid]);
-    __syncthreads();
-    if (tid == 0) {
-        int acc = 0, mx = 0;
-        uint32_t ovf = 0u;
-        sm.offs[0] = 0;
-        for (int c = 0; c < S; c++) {
-            int n = sm.offs[c + 1];
-            if (n > kCap) ovf = 1u;
-            mx = max(mx, n);
-            acc += n;
-            sm.offs[c + 1] = acc;
-        }
-        sm.bcast[8] = ovf;
-        sm.bcast[9] = (uint32_t)mx;
-    }
-    __syncthreads();
-    const int n_total = sm.offs[S];
-    if (sm.bcast[8] || sel > kSelMax || n_total > kCandMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
-    // no finite logit anywhere: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
-    if (n_total == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
+    const SrEdit* ed = a.edits + rd.edit_off;
+    const bool use_edits = (rd.flags & kRowHasPenalty) != 0u && rd.edit_cnt > 0;
+    const bool excl = use_edits && (rd.flags & kRowHistExcl) != 0u;  // the scan skipped the history ids
+    const int ne = use_edits ? rd.edit_cnt : 0;
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * (a.dtype == 1 ? 2 : 4);
+    const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+    auto hist_logit = [&](int id) SR_INL -> float {  // the masked logit of one token id
+        float x = (a.dtype == 1) ? sr_bf16_to_f32(((const uint16_t*)rowp)[id]) : ((const float*)rowp)[id];
+        if (mrow && !mask_bit(mrow, id)) x = SR_NEG_INF;
+        return x;
+    };
 
     SR_PROF(a, 11);
-    // flattened position g -> (chunk g / pitch, element g mod pitch), pitch a power of two >= the
-    // longest chunk list; the host sizes the chunking so that chunks x pitch fits the registers
-    const int pitch = next_pow2(max((int)sm.bcast[9], 1));
-    const int pshift = 31 - __clz(pitch);
-    if ((long long)pitch * S > kCandMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
-    auto cand_addr = [&](int r) -> int {  // index into cval / cidx of this thread's r-th candidate
-        const int g = r * kThreads + tid;
-        return (g >> pshift) * kCap + (g & (pitch - 1));
-    };
-    const int nr = (S * pitch + kThreads - 1) / kThreads;  // register slots that can hold a candidate
-    uint32_t kreg[kCandRegs];  // 0 = no candidate in this slot
+    const int nr = (n_c + kThreads - 1) / kThreads;  // register slots that can hold a candidate
+    uint32_t kreg[kCandRegs];                         // 0 = no candidate in this slot
+    int kid[kCandRegs];
 #pragma unroll
     for (int r = 0; r < kCandRegs; r++) {
         kreg[r] = 0u;
+        kid[r] = 0;
         if (r >= nr) continue;
         const int g = r * kThreads + tid;
-        const int c = g >> pshift, i = g & (pitch - 1);
-        const int cc = min(c, S - 1);
-        const bool ok = c < S && i < sm.offs[cc + 1] - sm.offs[cc];
-        kreg[r] = ok ? sr_okey(sr_load_agent(&cval[c * kCap + i])) : 0u;
+        if (g < n_c) {
+            const unsigned long long cv = sr_load_agent(&cand[g]);
+            kreg[r] = sr_okey(sr_u2f((uint32_t)(cv >> 32)));
+            kid[r] = (int)(uint32_t)cv;
+        }
     }
+    auto cand_id = [&](int r) SR_INL -> int { return kid[r]; };
     SR_PROF(a, 12);
-    auto each_key = [&](auto&& body) {
+    auto each_key = [&](auto&& body) SR_INL {
 #pragma unroll
         for (int r = 0; r < kCandRegs; r++)
             if (r < nr) body(kreg[r]);
     };
 
-    // history / bias ids of the row, staged for binary search
-    const SrEdit* ed = a.edits + rd.edit_off;
-    const bool use_edits = (rd.flags & kRowHasPenalty) != 0u;
-    const int ne = use_edits ? rd.edit_cnt : 0;   // <= kSelMax - 1 on this kernel
-    int* edit_ids = sm.idxs;
-    if (use_edits)
-        for (int e = tid; e < ne; e += kThreads) edit_ids[e] = ed[e].id;
-    auto find_edit = [&](int id) -> int {
-        int lo = 0, hi = ne;
-        while (lo < hi) {
-            int mid = (lo + hi) >> 1;
-            if (edit_ids[mid] < id) lo = mid + 1; else hi = mid;
-        }
-        return (lo < ne && edit_ids[lo] == id) ? lo : -1;
-    };
-
-    if (rd.path == SR_PATH_GREEDY) {
-        // argmax: highest key, lowest index among its ties
+    if (rd.path == SR_PATH_GREEDY || rd.path == SR_PATH_GREEDY_PEN) {
+        // best candidate: highest key, lowest index among its ties.  With penalties the candidates are
+        // the tokens outside the history (GreedyWithHistoryPenalties, Sampler.cs:421-437: only history ids
+        // change value), and the adjusted history ids compete with the best of them.
         uint32_t kmax = 0u;
         each_key([&](uint32_t k) { kmax = k > kmax ? k : kmax; });
         kmax = block_max_u32(kmax, sm);
-        int best = 0x7fffffff;
-#pragma unroll
-        for (int r = 0; r < kCandRegs; r++)
-            if (kreg[r] == kmax && kreg[r] != 0u) best = min(best, sr_load_agent(&cidx[cand_addr(r)]));
-        best = block_min_i32(best, sm);
-        give_up(0u, best);
-        return;
-    }
-
-    if (rd.path == SR_PATH_GREEDY_PEN) {
-        // GreedyWithHistoryPenalties (Sampler.cs:421-437): only the history ids change value, so the
-        // argmax is the better of (a) the best adjusted history id and (b) the best raw candidate that
-        // is not a history id -- one exists among the top (distinct ids + 1) candidates.
-        __syncthreads();  // edit_ids staged
         unsigned long long best = 0ull;
 #pragma unroll
-        for (int r = 0; r < kCandRegs; r++) {
-            if (kreg[r] == 0u) continue;
-            const int id = sr_load_agent(&cidx[cand_addr(r)]);
-            if (find_edit(id) < 0) {
-                unsigned long long cmp = ((unsigned long long)kreg[r] << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
+        for (int r = 0; r < kCandRegs; r++)
+            if (r < nr && kreg[r] == kmax && kreg[r] != 0u) {
+                unsigned long long cmp = ((unsigned long long)kreg[r] << 32) | (unsigned long long)(0xffffffffu - (uint32_t)cand_id(r));
                 best = cmp > best ? cmp : best;
             }
-        }
-        const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * (a.dtype == 1 ? 2 : 4);
-        const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
-        for (int e = tid; e < ne; e += kThreads) {
-            const int id = ed[e].id;
-            float x = (a.dtype == 1) ? sr_bf16_to_f32(((const uint16_t*)rowp)[id]) : ((const float*)rowp)[id];
-            if (mrow && !mask_bit(mrow, id)) x = SR_NEG_INF;
-            if (rd.rep != 1.0f)
-                for (int o = 0; o < ed[e].occ_win; o++) x = x > 0.0f ? __fdiv_rn(x, rd.rep) : __fmul_rn(x, rd.rep);
-            if (rd.presence != 0.0f || rd.frequency != 0.0f)
-                x = __fsub_rn(x, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ed[e].occ_all)));
-            if (sr_f2u(x) != 0xff800000u && x == x) {
-                unsigned long long cmp = ((unsigned long long)sr_okey(x) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
-                best = cmp > best ? cmp : best;
+        if (rd.path == SR_PATH_GREEDY_PEN) {
+            for (int e = tid; e < ne; e += kThreads) {
+                const int id = ed[e].id;
+                float x = hist_logit(id);
+                if (rd.rep != 1.0f)
+                    for (int o = 0; o < ed[e].occ_win; o++) x = x > 0.0f ? __fdiv_rn(x, rd.rep) : __fmul_rn(x, rd.rep);
+                if (rd.presence != 0.0f || rd.frequency != 0.0f)
+                    x = __fsub_rn(x, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ed[e].occ_all)));
+                if (sr_f2u(x) != 0xff800000u && x == x) {
+                    unsigned long long cmp = ((unsigned long long)sr_okey(x) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
+                    best = cmp > best ? cmp : best;
+                }
             }
         }
         best = sr_wave_max_u64(best);
@@ -511,7 +479,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 unsigned long long cmp = ((unsigned long long*)sm.vals)[w];
                 best = cmp > best ? cmp : best;
             }
-            // nothing finite at all: every adjusted logit is -inf and the first index wins
+            // nothing finite at all: every (adjusted) logit is -inf and the first index wins
             a.out_tokens[row] = best ? (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull)) : 0;
             if (a.out_flags) a.out_flags[row] = out_flag | (best ? 0u : SR_KFLAG_DEGENERATE);
         }
@@ -519,64 +487,93 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     }
 
     // ---- SampleTopK (Sampler.cs:216-357) ---------------------------------------------------------
-    // exact key of the sel-th largest candidate, then the set at or above it
-    const uint32_t tkey = (n_total <= sel) ? 0u : block_radix_select(each_key, sel, sm);
-    SR_PROF(a, 5);
-    int c_ge = 0, c_gt = 0;
-    each_key([&](uint32_t k) { c_ge += (k != 0u && k >= tkey) ? 1 : 0; c_gt += (k != 0u && k > tkey) ? 1 : 0; });
-    const int m_ge = block_sum_i32(c_ge, sm);
-    uint32_t tidx_key = 0u;  // ties additionally need (0xffffffff - idx) >= tidx_key
-    if (m_ge > kSelMax) {
-        // many candidates tie with the sel-th value (quantised or constant rows): equal values rank by
-        // ascending index, so only the (sel - #above) lowest-index ties belong to the set
-        const int m_gt = block_sum_i32(c_gt, sm);
-        uint32_t tie_key[kCandRegs];
+    // exact top-`need` of the candidates by (value desc, index asc): key of the need-th largest, and for
+    // its ties the (0xffffffff - index) bound that admits only the lowest indices
+    uint32_t tkey = 0u, tidx_key = 0u;
+    auto select_top = [&](int need) SR_INL {
+        tkey = block_radix_select(each_key, need, sm);
+        int c_ge = 0, c_gt = 0;
+        each_key([&](uint32_t k) { c_ge += (k != 0u && k >= tkey) ? 1 : 0; c_gt += (k != 0u && k > tkey) ? 1 : 0; });
+        const int m_ge = block_sum_i32(c_ge, sm);
+        if (m_ge > need) {
+            const int m_gt = block_sum_i32(c_gt, sm);
+            uint32_t tie_key[kCandRegs];
 #pragma unroll
-        for (int r = 0; r < kCandRegs; r++)
-            tie_key[r] = (kreg[r] != 0u && kreg[r] == tkey) ? 0xffffffffu - (uint32_t)sr_load_agent(&cidx[cand_addr(r)]) : 0u;
-        auto each_tie = [&](auto&& body) {
+            for (int r = 0; r < kCandRegs; r++)
+                tie_key[r] = (r < nr && kreg[r] != 0u && kreg[r] == tkey) ? 0xffffffffu - (uint32_t)cand_id(r) : 0u;
+            auto each_tie = [&](auto&& body) SR_INL {
 #pragma unroll
-            for (int r = 0; r < kCandRegs; r++) body(tie_key[r]);
-        };
-        tidx_key = block_radix_select(each_tie, sel - m_gt, sm);
-    }
-    // gather (key, idx) of the set into LDS: count, scan, then fetch the indices and write
-    auto in_set = [&](int r) -> bool {
+                for (int r = 0; r < kCandRegs; r++)
+                    if (r < nr) body(tie_key[r]);
+            };
+            tidx_key = block_radix_select(each_tie, need - m_gt, sm);
+        }
+    };
+    auto in_set = [&](int r) SR_INL -> bool {
         if (kreg[r] == 0u || kreg[r] < tkey) return false;
         if (kreg[r] > tkey || tidx_key == 0u) return true;
-        return (0xffffffffu - (uint32_t)sr_load_agent(&cidx[cand_addr(r)])) >= tidx_key;
+        return (0xffffffffu - (uint32_t)cand_id(r)) >= tidx_key;
     };
-    int mine = 0;
-#pragma unroll
-    for (int r = 0; r < kCandRegs; r++)
-        if (r < nr) mine += in_set(r) ? 1 : 0;
-    int m;
-    int pos = block_excl_scan(mine, &m, sm);
-    if (mine > 0) {
-#pragma unroll
-        for (int r = 0; r < kCandRegs; r++)
-            if (r < nr && in_set(r) && pos < kSelMax) {
-                sm.xa[pos] = kreg[r];
-                sm.xb[pos] = (uint32_t)sr_load_agent(&cidx[cand_addr(r)]);
-                pos++;
-            }
-    }
-    __syncthreads();  // also orders the staging of edit_ids
-    if (m > kSelMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }  // guard; m <= max(sel, kSelMax)
-    SR_PROF(a, 6);
 
+    const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
+    float mx;
+    // Candidates whose e = expf(v / T - max) is below 2^-26 are dropped before the sort: with e_0 = 1
+    // they change neither running sum (they are under half an ulp of a sum >= 1, and of a cumulative
+    // probability >= probs[0]) and the draw can never stop on them, so the result is bit-identical.
+    // x < -18.1 implies e < 1.4e-8 < 2^-26.
+    auto alive_key = [&](uint32_t key) SR_INL -> bool {
+        const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx);
+        return key != 0u && !(x < -18.1f);
+    };
     // sort keys: (value after penalties, value before, ~index) descending -- the reference's selection
     // order (value desc, index asc) followed by its stable re-sort after penalties, in one sort
     uint32_t hi[kSortRegs], mid[kSortRegs], lo[kSortRegs];
+    int m2;          // live entries (at most top_k of them are used)
+    int sort_n = 0;  // entries handed to the sort
+    bool ranked = false;  // sm.vals / sm.idxs already hold the k first entries
+
+    if (use_edits && !excl) {
+        // ---- penalties that may raise a logit: the reference's literal top-(k + history length) set ------
+        if (n_c == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }  // Sampler.cs:254-255: Greedy(raw) = index 0
+        if (ne > kSelMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
+        int* edit_ids = sm.idxs;  // history ids of the row, staged for binary search
+        for (int e = tid; e < ne; e += kThreads) edit_ids[e] = ed[e].id;
+        auto find_edit = [&](int id) SR_INL -> int {
+            int lo_e = 0, hi_e = ne;
+            while (lo_e < hi_e) {
+                int mid_e = (lo_e + hi_e) >> 1;
+                if (edit_ids[mid_e] < id) lo_e = mid_e + 1; else hi_e = mid_e;
+            }
+            return (lo_e < ne && edit_ids[lo_e] == id) ? lo_e : -1;
+        };
+        if (n_c > sel) select_top(sel);
+        SR_PROF(a, 5);
+        int mine = 0;
 #pragma unroll
-    for (int r = 0; r < kSortRegs; r++) {
-        const int i = r * kThreads + tid;
-        hi[r] = mid[r] = lo[r] = 0u;
-        if (i < m) {
-            const uint32_t key = sm.xa[i];
-            const int id = (int)sm.xb[i];
-            uint32_t nkey = key;
-            if (use_edits) {
+        for (int r = 0; r < kCandRegs; r++)
+            if (r < nr) mine += in_set(r) ? 1 : 0;
+        int m;
+        int pos = block_excl_scan(mine, &m, sm);
+        if (mine > 0) {
+#pragma unroll
+            for (int r = 0; r < kCandRegs; r++)
+                if (r < nr && in_set(r) && pos < kSelMax) {
+                    sm.xa[pos] = kreg[r];
+                    sm.xb[pos] = (uint32_t)cand_id(r);
+                    pos++;
+                }
+        }
+        __syncthreads();  // also orders the staging of edit_ids
+        if (m > kSelMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }  // guard; m <= sel
+        SR_PROF(a, 6);
+#pragma unroll
+        for (int r = 0; r < kSortRegs; r++) {
+            const int i = r * kThreads + tid;
+            hi[r] = mid[r] = lo[r] = 0u;
+            if (i < m) {
+                const uint32_t key = sm.xa[i];
+                const int id = (int)sm.xb[i];
+                uint32_t nkey = key;
                 // Sampler.cs:261-287: pen = pow(rep, occWindow) once; presence/frequency over the whole history
                 const int e = find_edit(id);
                 if (e >= 0) {
@@ -588,59 +585,235 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                         nkey = sr_okey(v);
                     }
                 }
+                hi[r] = nkey; mid[r] = key; lo[r] = 0xffffffffu - (uint32_t)id;
             }
-            hi[r] = nkey; mid[r] = key; lo[r] = 0xffffffffu - (uint32_t)id;
         }
-    }
-    SR_PROF(a, 7);
-    // Candidates whose e = expf(v / T - max) is below 2^-26 are dropped before the sort: with e_0 = 1
-    // they change neither running sum (they are under half an ulp of a sum >= 1, and of a cumulative
-    // probability >= probs[0]) and the draw can never stop on them, so the result is bit-identical.
-    // x < -18.1 implies e < 1.4e-8 < 2^-26.
-    uint32_t lmaxk = 0u;
+        SR_PROF(a, 7);
+        uint32_t lmaxk = 0u;
 #pragma unroll
-    for (int r = 0; r < kSortRegs; r++) lmaxk = hi[r] > lmaxk ? hi[r] : lmaxk;
-    const uint32_t kmaxn = block_max_u32(lmaxk, sm);
-    const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
-    const float mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
-    int nlive = 0;
-    bool alive[kSortRegs];
-#pragma unroll
-    for (int r = 0; r < kSortRegs; r++) {
-        const int i = r * kThreads + tid;
-        const float x = __fsub_rn(__fmul_rn(sr_okey_inv(hi[r]), inv_temp), mx);
-        alive[r] = (i < m) && !(x < -18.1f);
-        nlive += alive[r] ? 1 : 0;
-    }
-    int m2;
-    int lpos = block_excl_scan(nlive, &m2, sm);
-    if (m2 < m) {
-        // compact the live candidates (all threads have their elements in registers by now)
-#pragma unroll
-        for (int r = 0; r < kSortRegs; r++)
-            if (alive[r]) { sm.xa[lpos] = hi[r]; sm.xb[lpos] = mid[r]; sm.xc[lpos] = lo[r]; lpos++; }
-        __syncthreads();
+        for (int r = 0; r < kSortRegs; r++) lmaxk = hi[r] > lmaxk ? hi[r] : lmaxk;
+        const uint32_t kmaxn = block_max_u32(lmaxk, sm);
+        mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
+        int nlive = 0;
+        bool alive[kSortRegs];
 #pragma unroll
         for (int r = 0; r < kSortRegs; r++) {
             const int i = r * kThreads + tid;
-            hi[r] = (i < m2) ? sm.xa[i] : 0u;
-            mid[r] = (i < m2) ? sm.xb[i] : 0u;
-            lo[r] = (i < m2) ? sm.xc[i] : 0u;
+            alive[r] = (i < m) && alive_key(hi[r]);
+            nlive += alive[r] ? 1 : 0;
         }
+        int lpos = block_excl_scan(nlive, &m2, sm);
+        if (m2 < m) {
+            // compact the live candidates (all threads have their elements in registers by now)
+#pragma unroll
+            for (int r = 0; r < kSortRegs; r++)
+                if (alive[r]) { sm.xa[lpos] = hi[r]; sm.xb[lpos] = mid[r]; sm.xc[lpos] = lo[r]; lpos++; }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < kSortRegs; r++) {
+                const int i = r * kThreads + tid;
+                hi[r] = (i < m2) ? sm.xa[i] : 0u;
+                mid[r] = (i < m2) ? sm.xb[i] : 0u;
+                lo[r] = (i < m2) ? sm.xc[i] : 0u;
+            }
+        }
+        sort_n = m2;
+    } else {
+        // ---- no penalties, or penalties that only lower: candidates outside the history + the history ids --
+        if (ne > kHistRegs * kThreads) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
+        uint32_t hadj[kHistRegs], hraw[kHistRegs];
+#pragma unroll
+        for (int r = 0; r < kHistRegs; r++) {
+            hadj[r] = hraw[r] = 0u;
+            const int e = r * kThreads + tid;
+            if (e < ne) {
+                const SrEdit ee = ed[e];
+                const float x = hist_logit(ee.id);
+                // -inf never enters the reference's selection (Sampler.cs:240-249)
+                if (x == x && sr_f2u(x) != 0xff800000u) {
+                    float v = x;
+                    // Sampler.cs:261-287: pen = pow(rep, occWindow) once; presence/frequency over the whole history
+                    if (ee.occ_all > 0) {
+                        if (rd.rep != 1.0f && ee.occ_win > 0) v = v > 0.0f ? __fdiv_rn(v, ee.pen) : __fmul_rn(v, ee.pen);
+                        v = __fsub_rn(v, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ee.occ_all)));
+                    }
+                    hraw[r] = sr_okey(x);
+                    hadj[r] = sr_okey(v);
+                }
+            }
+        }
+        SR_PROF(a, 5);
+        uint32_t lmaxk = 0u;
+        each_key([&](uint32_t k) { lmaxk = k > lmaxk ? k : lmaxk; });
+#pragma unroll
+        for (int r = 0; r < kHistRegs; r++) lmaxk = (hraw[r] != 0u && hadj[r] > lmaxk) ? hadj[r] : lmaxk;
+        if (tid < 256) sm.hist[tid] = 0u;
+        if (tid == 0) sm.bcast[4] = 0u;
+        const uint32_t kmaxn = block_max_u32(lmaxk, sm);  // its barriers also publish the cleared histogram
+        // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
+        if (kmaxn == 0u) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
+        mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
+        // How far an entry lies below the maximum, in 1/14 of a log-unit: -1 = absent or dead, else 0..255.
+        // Monotone in the key, so "bin <= b" is a prefix of the descending order.
+        auto bin_of = [&](uint32_t key) SR_INL -> int {
+            if (key == 0u) return -1;
+            const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx);
+            if (x < -18.1f) return -1;
+            return min(max((int)__fmul_rn(x, -14.0f), 0), 255);
+        };
+#pragma unroll
+        for (int r = 0; r < kCandRegs; r++)
+            if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.hist[b], 1u); }
+#pragma unroll
+        for (int r = 0; r < kHistRegs; r++) {
+            const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
+            if (b >= 0) atomicAdd(&sm.hist[b], 1u);
+        }
+        __syncthreads();
+        // every wave reads the histogram: live entries, and the first bin at which the k best are complete
+        int bstar = 255, n_live, n_keep, max_bin;
+        {
+            const int lane = sr_lane();
+            const uint32_t h0 = sm.hist[4 * lane], h1 = sm.hist[4 * lane + 1], h2 = sm.hist[4 * lane + 2],
+                           h3 = sm.hist[4 * lane + 3];
+            const int tot = (int)(h0 + h1 + h2 + h3);
+            const int incl = sr_wave_incl_scan_i32(tot);
+            n_live = __shfl(incl, SR_WAVE - 1);
+            n_keep = n_live;
+            const int need = min(rd.top_k, n_live);
+            const unsigned long long bal = __ballot(incl >= need);
+            const int L = bal ? (int)__ffsll((long long)bal) - 1 : SR_WAVE - 1;
+            const int c = incl - tot;
+            int bq = 4 * lane + 3, cq = incl;
+            if (c + (int)h0 >= need) { bq = 4 * lane; cq = c + (int)h0; }
+            else if (c + (int)(h0 + h1) >= need) { bq = 4 * lane + 1; cq = c + (int)(h0 + h1); }
+            else if (c + (int)(h0 + h1 + h2) >= need) { bq = 4 * lane + 2; cq = c + (int)(h0 + h1 + h2); }
+            bstar = __shfl(bq, L);
+            n_keep = __shfl(cq, L);
+            // the fullest kept bin bounds the ranking loop below
+            uint32_t hm = 0u;
+            if (4 * lane <= bstar) hm = h0;
+            if (4 * lane + 1 <= bstar) hm = max(hm, h1);
+            if (4 * lane + 2 <= bstar) hm = max(hm, h2);
+            if (4 * lane + 3 <= bstar) hm = max(hm, h3);
+            max_bin = (int)sr_wave_max_u32(hm);
+            if (sr_wave_id() == 0) {
+                sm.boff[4 * lane] = (uint32_t)c;
+                sm.boff[4 * lane + 1] = (uint32_t)c + h0;
+                sm.boff[4 * lane + 2] = (uint32_t)c + h0 + h1;
+                sm.boff[4 * lane + 3] = (uint32_t)c + h0 + h1 + h2;
+                if (lane == SR_WAVE - 1) sm.boff[256] = (uint32_t)incl;
+                sm.bfill[4 * lane] = 0u; sm.bfill[4 * lane + 1] = 0u; sm.bfill[4 * lane + 2] = 0u; sm.bfill[4 * lane + 3] = 0u;
+            }
+        }
+        m2 = n_live;
+        bool by_bins = true;  // kept entries are laid out bin by bin and ranked inside their bin
+        if (n_keep > kSelMax) {
+            // a flat row: only the k best candidates outside the history can matter
+            by_bins = false;
+            if (n_c > rd.top_k) select_top(rd.top_k);
+            bstar = 255;
+            int mine = 0;
+#pragma unroll
+            for (int r = 0; r < kCandRegs; r++)
+                if (r < nr) mine += (bin_of(kreg[r]) >= 0 && in_set(r)) ? 1 : 0;
+#pragma unroll
+            for (int r = 0; r < kHistRegs; r++) mine += (hraw[r] != 0u && bin_of(hadj[r]) >= 0) ? 1 : 0;
+            n_keep = block_sum_i32(mine, sm);
+            if (n_keep > kSelMax) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
+        } else if (max_bin > 96) {
+            by_bins = false;
+        }
+        __syncthreads();  // boff / bfill written
+        SR_PROF(a, 6);
+        // gather the kept entries: bin by bin, or in any order when a sort follows
+        {
+            int mine = 0;
+            if (!by_bins) {
+#pragma unroll
+                for (int r = 0; r < kCandRegs; r++)
+                    if (r < nr) { const int b = bin_of(kreg[r]); mine += (b >= 0 && b <= bstar && in_set(r)) ? 1 : 0; }
+#pragma unroll
+                for (int r = 0; r < kHistRegs; r++) {
+                    const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
+                    mine += (b >= 0 && b <= bstar) ? 1 : 0;
+                }
+            }
+            int pos_any = (mine > 0) ? (int)atomicAdd(&sm.bcast[4], (uint32_t)mine) : 0;
+#pragma unroll
+            for (int r = 0; r < kCandRegs; r++)
+                if (r < nr) {
+                    const int b = bin_of(kreg[r]);
+                    if (b >= 0 && b <= bstar && in_set(r)) {
+                        const int pos = by_bins ? (int)(sm.boff[b] + atomicAdd(&sm.bfill[b], 1u)) : pos_any++;
+                        if (pos < kSelMax) {
+                            sm.xa[pos] = kreg[r];
+                            sm.xb[pos] = kreg[r];
+                            sm.xc[pos] = 0xffffffffu - (uint32_t)cand_id(r);
+                        }
+                    }
+                }
+#pragma unroll
+            for (int r = 0; r < kHistRegs; r++) {
+                const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
+                if (b >= 0 && b <= bstar) {
+                    const int pos = by_bins ? (int)(sm.boff[b] + atomicAdd(&sm.bfill[b], 1u)) : pos_any++;
+                    if (pos < kSelMax) {
+                        sm.xa[pos] = hadj[r];
+                        sm.xb[pos] = hraw[r];
+                        sm.xc[pos] = 0xffffffffu - (uint32_t)ed[r * kThreads + tid].id;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const int ms = by_bins ? min(n_keep, kSelMax) : min((int)sm.bcast[4], kSelMax);
+        // the first min(top_k, live) of the kept entries are the first of all live entries
+        m2 = min(min(m2, max(rd.top_k, 0)), ms);
+        sort_n = ms;
+        if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 13] = (unsigned long long)n_c; a.prof[(size_t)blockIdx.x * 16 + 14] = ((unsigned long long)n_live << 32) | (unsigned long long)ms; }
+        if (by_bins) {
+            // bins descend with the key, so an entry's rank is its bin's first position plus the entries of
+            // the bin that precede it
+            ranked = true;
+            const int kk = min(rd.top_k, m2);
+            for (int i = tid; i < ms; i += kThreads) {
+                const uint32_t mh = sm.xa[i], mm = sm.xb[i], ml = sm.xc[i];
+                const int b = bin_of(mh);
+                const int p0 = (int)sm.boff[b], p1 = p0 + (int)sm.hist[b];
+                int rank = p0;
+                for (int j = p0; j < p1; j++) rank += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
+                if (rank < kk) {
+                    sm.vals[rank] = sr_okey_inv(mh);
+                    sm.idxs[rank] = (int)(0xffffffffu - ml);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < kSortRegs; r++) {
+                const int i = r * kThreads + tid;
+                hi[r] = (i < ms) ? sm.xa[i] : 0u;
+                mid[r] = (i < ms) ? sm.xb[i] : 0u;
+                lo[r] = (i < ms) ? sm.xc[i] : 0u;
+            }
+        }
+        SR_PROF(a, 7);
     }
+
     // the k best that are still alive
-    const int k = min(rd.top_k, m2);  // top_k <= sel; everything past m2 is a no-op or does not exist
-    if (m2 > 128) {
-        if (use_edits) block_sample_sort_desc<true>(hi, mid, lo, m2, sm);
-        else block_sample_sort_desc<false>(hi, mid, lo, m2, sm);
+    const int k = min(rd.top_k, m2);  // everything past m2 is a no-op or does not exist
+    if (ranked) {
+    } else if (sort_n > 128) {
+        if (use_edits) block_sample_sort_desc<true>(hi, mid, lo, sort_n, sm);
+        else block_sample_sort_desc<false>(hi, mid, lo, sort_n, sm);
         // sorted (value key, ~index) are in xa / xc; the scatter area (vals / idxs / probs) is free again
         for (int i = tid; i < k; i += kThreads) {
             sm.vals[i] = sr_okey_inv(sm.xa[i]);
             sm.idxs[i] = (int)(0xffffffffu - sm.xc[i]);
         }
     } else {
-        if (use_edits) block_bitonic_sort_desc<true>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
-        else block_bitonic_sort_desc<false>(hi, mid, lo, next_pow2(m2 < 2 ? 2 : m2), sm);
+        if (use_edits) block_bitonic_sort_desc<true>(hi, mid, lo, next_pow2(sort_n < 2 ? 2 : sort_n), sm);
+        else block_bitonic_sort_desc<false>(hi, mid, lo, next_pow2(sort_n < 2 ? 2 : sort_n), sm);
 #pragma unroll
         for (int r = 0; r < kSortRegs; r++) {
             const int i = r * kThreads + tid;
@@ -727,7 +900,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 {
     __shared__ TopkSmem sm;
     using VO = VecOps<EPV>;
-    const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
+    const int tid = threadIdx.x, lane = sr_lane();
     const int S = a.chunks;
     // Grid order: [chunks of row 0] ... and, from row `lag` on, the tail of row i - lag right after the chunks
     // of row i; the tails of the last `lag` rows close the grid.  A tail workgroup is therefore dispatched
@@ -761,7 +934,10 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 if (sr_load_agent(&a.row_done[tslot]) == (uint32_t)S) { ok = 1u; break; }
                 __builtin_amdgcn_s_sleep(4);
             }
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);
+            sm.bcast[8] = (uint32_t)sr_load_agent(&a.cand_cnt[tslot]);
             sr_store_agent(&a.row_done[tslot], 0u);  // ready for the next launch
+            sr_store_agent(&a.cand_cnt[tslot], 0);
             sm.bcast[7] = ok;
         }
         __syncthreads();
@@ -773,7 +949,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             return;
         }
         SR_PROF(a, 4);
-        topk_row_tail(a, tslot, trow, a.rows[trow], sm);
+        topk_row_tail(a, tslot, trow, a.rows[trow], (int)sm.bcast[8], sm);
         SR_PROF(a, 15);
         return;
     }
@@ -781,71 +957,57 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
     const int V = a.vocab;
-    const int lo = c * a.chunk_len;
-    const int hi = min(V, lo + a.chunk_len);
     const int sel = rd.sel;
-    int total = 0;
+    unsigned long long* crow = a.cand + (size_t)slot * kRowCap;
+    int* cursor = a.cand_cnt + slot;
+    auto pack = [](float x, int idx) SR_INL -> unsigned long long {
+        return ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx;
+    };
     SR_PROF(a, 0);
 
-    if (lo < hi && sel <= kSelMax) {
-        constexpr int ES = (EPV == 4) ? 4 : 2;  // element size in bytes
-        const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
-        const uintptr_t addr = (uintptr_t)(rowp + (size_t)lo * ES);
-        const int mis = (int)((addr & 15u) / ES);
-        const u32x4* wp = (const u32x4*)(addr - (uintptr_t)mis * ES);
-        const int wbase = lo - mis;  // row element index of window element 0
-        const int nvec = (hi - wbase + EPV - 1) / EPV;
-        const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+    // The row is read as 16-byte vectors from the aligned address at or below its start: window element
+    // p is row element p - mis.  Chunks are whole multiples of 64 vectors of that window.
+    constexpr int ES = (EPV == 4) ? 4 : 2;  // element size in bytes
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+    const int mis = (int)(((uintptr_t)rowp & 15u) / ES);
+    const int nvt = (V + mis + EPV - 1) / EPV;        // vectors of the row window
+    const int f0 = c * a.chunk_vecs;                   // first vector of this chunk
+    const int nv = min(a.chunk_vecs, nvt - f0);        // vectors of this chunk
+    const int wbase = f0 * EPV - mis;                  // row element index of the chunk's first window element
 
+    if (nv > 0 && sel <= kSelMax) {
+        const u32x4* cp = (const u32x4*)(rowp - (size_t)mis * ES) + f0;
         u32x4 v[kVec];
 #pragma unroll
         for (int j = 0; j < kVec; j++) {
-            int f = j * kThreads + tid;
-            v[j] = (f < nvec) ? __builtin_nontemporal_load(&wp[f]) : VO::neg_inf();
-        }
-        SR_PROF(a, 1);
-        // edges of the window and the allow-mask: one keep-bit per element of the vector
-        const int mask_words = (int)a.mask_stride;
-#pragma unroll
-        for (int j = 0; j < kVec; j++) {
             const int f = j * kThreads + tid;
-            if (f < nvec) {
-                const int e0 = wbase + f * EPV;
-                uint32_t keep = (1u << EPV) - 1u;
-                if (e0 < lo || e0 + EPV > hi) {
+            v[j] = (f < nv) ? __builtin_nontemporal_load(&cp[f]) : VO::neg_inf();
+        }
+        // The scan mask holds one keep-bit per window element in this kernel's access order: for every
+        // block of 64 vectors, EPV 64-bit words, word q bit l = element q of the vector of lane l.  It
+        // carries the row's edges, its allow-mask and, when the row tail fetches them, its history ids,
+        // and is wave-uniform: scalar loads, one select per element.
+        {
+            const unsigned long long* srow = a.scan_mask + (size_t)rd.scan_row * (size_t)a.scan_stride;
+            const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+            const int nblk = (nvt + 63) >> 6;
 #pragma unroll
-                    for (int q = 0; q < EPV; q++)
-                        if (e0 + q < lo || e0 + q >= hi) keep &= ~(1u << q);
-                }
-                if (mrow) {
-                    const int es = e0 < 0 ? 0 : e0;       // first bit that exists
-                    const int wi = es >> 5, sh = es & 31;
-                    unsigned long long bits = mrow[wi];
-                    if (wi + 1 < mask_words) bits |= (unsigned long long)mrow[wi + 1] << 32;
-                    keep &= (uint32_t)(bits >> sh) << (es - e0);
-                }
-                if (keep != (1u << EPV) - 1u) {
+            for (int j = 0; j < kVec; j++) {
+                const int blk = (f0 >> 6) + j * (kThreads / SR_WAVE) + wave_u;
+                if (blk < nblk) {
+                    const unsigned long long* mp = srow + (size_t)blk * EPV;
 #pragma unroll
-                    for (int q = 0; q < EPV; q++)
-                        if (!((keep >> q) & 1u)) VO::kill(v[j], q);
+                    for (int q = 0; q < EPV; q++) VO::keep_if(v[j], q, __builtin_amdgcn_inverse_ballot_w64(mp[q]));
                 }
             }
         }
+        SR_PROF(a, 1);
 
-        // A safe lower bound on the chunk's sel-th largest element.
-        uint32_t tkey;
-        if (nvec <= 4 * kThreads) {
-            // short chunk (at most four vectors per thread): select exactly over its elements
-            auto each_elem = [&](auto&& body) {
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-#pragma unroll
-                    for (int q = 0; q < EPV; q++) body(sr_okey(VO::get(v[j], q)));
-            };
-            tkey = block_radix_select(each_elem, sel, sm);
-        } else {
-            // every thread owns four interleaved groups of vectors (j mod 4), all populated here; the
-            // sel-th largest of the 2048 disjoint-group maxima cannot exceed the sel-th largest element
+        const int wlim = kRowCap / (S * kWaves);  // candidates one wave may hand over
+        if (sel <= SR_WAVE && wlim >= SR_TK_WAVE_LIM) {
+            // ---- every wave on its own: no workgroup barrier --------------------------------------------
+            // every lane owns four interleaved groups of vectors (j mod 4); the sel-th largest of the wave's
+            // 256 group maxima, found bit by bit, is a lower bound on the wave's sel-th largest element
             uint32_t gk[SR_TK_GROUPS];
 #pragma unroll
             for (int g = 0; g < SR_TK_GROUPS; g++) {
@@ -856,97 +1018,306 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                     for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, VO::get(v[j], q));
                 gk[g] = sr_okey(mxv);
             }
-            auto each_gk = [&](auto&& body) {
+            uint32_t K = 0u;
+#pragma unroll 1
+            for (int bit = 31; bit >= 0; bit--) {
+                const uint32_t cnd = K | (1u << bit);
+                int cge = 0;
 #pragma unroll
-                for (int g = 0; g < SR_TK_GROUPS; g++) body(gk[g]);
-            };
-            tkey = (sel > SR_TK_M) ? 0u : block_radix_select(each_gk, sel, sm);
-        }
-        SR_PROF(a, 2);
-        // -inf never enters the candidate set (Sampler.cs:240-249: strict v <= -inf rejects it)
-        const float tval = (tkey <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(tkey);
-
-        float* cv = a.cand_val + ((size_t)slot * S + c) * kCap;
-        int* ci = a.cand_idx + ((size_t)slot * S + c) * kCap;
-        int cnt = 0;
-#pragma unroll
-        for (int j = 0; j < kVec; j++)
-#pragma unroll
-            for (int q = 0; q < EPV; q++) cnt += (VO::get(v[j], q) >= tval) ? 1 : 0;
-        // a chunk hands over at most `lim` candidates, so that the row tail can hold all chunks of a row
-        const int lim = min(kCap, 2 * sel + 128);
-        int pos = block_excl_scan(cnt, &total, sm);
-        if (total <= lim) {
-            if (cnt > 0) {
-#pragma unroll
-                for (int j = 0; j < kVec; j++) {
-                    int e0 = wbase + (j * kThreads + tid) * EPV;
-#pragma unroll
-                    for (int q = 0; q < EPV; q++) {
-                        float x = VO::get(v[j], q);
-                        if (x >= tval) { sr_store_agent(&cv[pos], x); sr_store_agent(&ci[pos], e0 + q); pos++; }
-                    }
-                }
+                for (int g = 0; g < SR_TK_GROUPS; g++) cge += __popcll(__ballot(gk[g] >= cnd));
+                if (cge >= sel) K = cnd;
             }
-        } else {
-            // Many elements tie with the threshold value.  Equal values rank by ascending index, so
-            // besides everything above the threshold only the first (sel - #above) ties can matter.
-            int cgt = 0;
+            // -inf never enters the candidate set (Sampler.cs:240-249: strict v <= -inf rejects it)
+            float tval = (K <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(K);
+            SR_PROF(a, 2);
+            int total = 0;  // wave-uniform: the comparisons land in scalar registers
 #pragma unroll
             for (int j = 0; j < kVec; j++)
 #pragma unroll
-                for (int q = 0; q < EPV; q++) cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
-            int total_gt;
-            int pgt = block_excl_scan(cgt, &total_gt, sm);
-            if (total_gt > lim) {
-                total = kCap + 1;  // genuine overflow: the row is reported as unsupported
-            } else {
-                if (cgt > 0) {
+                for (int q = 0; q < EPV; q++) total += __popcll(__ballot(VO::get(v[j], q) >= tval));
+            if (total <= wlim) {
+                int base = 0;
+                if (lane == 0 && total > 0)
+                    base = __hip_atomic_fetch_add(cursor, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                base = __builtin_amdgcn_readfirstlane(base);
+                if (total > 0 && base >= 0 && base + total <= kRowCap) {
+                    int off = base;
 #pragma unroll
                     for (int j = 0; j < kVec; j++) {
-                        int e0 = wbase + (j * kThreads + tid) * EPV;
+                        const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                         for (int q = 0; q < EPV; q++) {
-                            float x = VO::get(v[j], q);
-                            if (x > tval) { sr_store_agent(&cv[pgt], x); sr_store_agent(&ci[pgt], e0 + q); pgt++; }
+                            const float x = VO::get(v[j], q);
+                            const unsigned long long bal = __ballot(x >= tval);
+                            if (bal) {
+                                if (x >= tval) {
+                                    const int pos = off + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32),
+                                                              __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u));
+                                    sr_store_agent(&crow[pos], pack(x, e0 + q));
+                                }
+                                off += __popcll(bal);
+                            }
                         }
                     }
                 }
-                const int need_eq = min(sel - total_gt, lim - total_gt);
-                int emitted = 0;
-                if (need_eq > 0) {
+            } else {
+                // Many elements at or above the bound.  Equal values rank by ascending index, so besides
+                // everything above the threshold only the first (sel - #above) ties can matter.
+                int cgt = 0;
 #pragma unroll
-                    for (int j = 0; j < kVec; j++) {  // ascending j, then tid, then q = ascending index
-                        if (emitted >= need_eq) continue;  // block-uniform
+                for (int j = 0; j < kVec; j++)
+#pragma unroll
+                    for (int q = 0; q < EPV; q++) cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
+                int total_gt = sr_wave_sum_i32(cgt);
+                if (total_gt > wlim) {
+                    // the lane maxima bound is too loose (the large values sit in few lanes): the exact sel-th
+                    // largest element of the wave, bit by bit
+                    // (compared as floats: a key in the NaN range compares false, and the answer is finite)
+                    uint32_t K2 = 0u;
+#pragma unroll 1
+                    for (int bit = 31; bit >= 0; bit--) {
+                        const uint32_t cnd = K2 | (1u << bit);
+                        const float fc = sr_okey_inv(cnd);
+                        int cge = 0;
+#pragma unroll
+                        for (int j = 0; j < kVec; j++)
+#pragma unroll
+                            for (int q = 0; q < EPV; q++) cge += __popcll(__ballot(VO::get(v[j], q) >= fc));
+                        if (cge >= sel) K2 = cnd;
+                    }
+                    tval = sr_okey_inv(K2);
+                    cgt = 0;
+#pragma unroll
+                    for (int j = 0; j < kVec; j++)
+#pragma unroll
+                        for (int q = 0; q < EPV; q++) cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
+                    total_gt = sr_wave_sum_i32(cgt);
+                }
+                int total_eq = 0;
+#pragma unroll
+                for (int j = 0; j < kVec; j++)
+#pragma unroll
+                    for (int q = 0; q < EPV; q++) total_eq += __popcll(__ballot(VO::get(v[j], q) == tval));
+                const int n_eq = max(0, min(min(sel - total_gt, wlim - total_gt), total_eq));
+                const int incl = sr_wave_incl_scan_i32(cgt);
+                total = total_gt + n_eq;
+                int base = 0;
+                if (lane == 0 && total > 0)
+                    base = __hip_atomic_fetch_add(cursor, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                base = __builtin_amdgcn_readfirstlane(base);
+                if (total > 0 && base >= 0 && base + total <= kRowCap) {
+                    int pos = base + incl - cgt;
+                    if (cgt > 0) {
+#pragma unroll
+                        for (int j = 0; j < kVec; j++) {
+                            const int e0 = wbase + (j * kThreads + tid) * EPV;
+#pragma unroll
+                            for (int q = 0; q < EPV; q++) {
+                                const float x = VO::get(v[j], q);
+                                if (x > tval) { sr_store_agent(&crow[pos], pack(x, e0 + q)); pos++; }
+                            }
+                        }
+                    }
+                    int emitted = 0;
+#pragma unroll
+                    for (int j = 0; j < kVec; j++) {  // ascending j, then lane, then q = ascending index
+                        if (emitted >= n_eq) continue;  // wave-uniform
                         int ceq = 0;
 #pragma unroll
                         for (int q = 0; q < EPV; q++) ceq += (VO::get(v[j], q) == tval) ? 1 : 0;
-                        int tj;
-                        int rank = emitted + block_excl_scan(ceq, &tj, sm);
+                        const int ie = sr_wave_incl_scan_i32(ceq);
+                        int rank = emitted + ie - ceq;
                         if (ceq > 0) {
-                            int e0 = wbase + (j * kThreads + tid) * EPV;
+                            const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                             for (int q = 0; q < EPV; q++) {
                                 if (VO::get(v[j], q) == tval) {
-                                    if (rank < need_eq) { sr_store_agent(&cv[total_gt + rank], tval); sr_store_agent(&ci[total_gt + rank], e0 + q); }
+                                    if (rank < n_eq) sr_store_agent(&crow[base + total_gt + rank], pack(tval, e0 + q));
                                     rank++;
                                 }
                             }
                         }
-                        emitted += tj;
+                        emitted += __shfl(ie, SR_WAVE - 1);
                     }
                 }
-                total = total_gt + max(0, min(need_eq, emitted));
+            }
+        } else {
+            // ---- the whole workgroup: threshold from 2048 group maxima (or exactly, on a short chunk) ------
+            auto reserve = [&](int n) SR_INL -> int {  // all threads; returns the first list position
+                __syncthreads();
+                if (tid == 0)
+                    sm.bcast[3] = (uint32_t)__hip_atomic_fetch_add(cursor, n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                return (int)sm.bcast[3];
+            };
+            uint32_t tkey;
+            if (nv <= 4 * kThreads) {
+                // short chunk (at most four vectors per thread): select exactly over its elements
+                auto each_elem = [&](auto&& body) SR_INL {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int q = 0; q < EPV; q++) body(sr_okey(VO::get(v[j], q)));
+                };
+                tkey = block_radix_select(each_elem, sel, sm);
+            } else {
+                // every thread owns four interleaved groups of vectors (j mod 4), all populated here; the
+                // sel-th largest of the 2048 disjoint-group maxima cannot exceed the sel-th largest element
+                uint32_t gk[SR_TK_GROUPS];
+#pragma unroll
+                for (int g = 0; g < SR_TK_GROUPS; g++) {
+                    float mxv = SR_NEG_INF;
+#pragma unroll
+                    for (int j = g; j < kVec; j += SR_TK_GROUPS)
+#pragma unroll
+                        for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, VO::get(v[j], q));
+                    gk[g] = sr_okey(mxv);
+                }
+                auto each_gk = [&](auto&& body) SR_INL {
+#pragma unroll
+                    for (int g = 0; g < SR_TK_GROUPS; g++) body(gk[g]);
+                };
+                tkey = (sel > SR_TK_M) ? 0u : block_radix_select(each_gk, sel, sm);
+            }
+            SR_PROF(a, 2);
+            const float tval = (tkey <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(tkey);
+            int cnt = 0;
+#pragma unroll
+            for (int j = 0; j < kVec; j++)
+#pragma unroll
+                for (int q = 0; q < EPV; q++) cnt += (VO::get(v[j], q) >= tval) ? 1 : 0;
+            // a chunk hands over at most `lim` candidates, so that the row list can hold all chunks of a row
+            const int lim = min(kRowCap / S, 2 * sel + 128);
+            int total;
+            int pos = block_excl_scan(cnt, &total, sm);
+            if (lim < sel) {
+                (void)reserve(kOverflowMark);  // the row is reported as unsupported
+            } else if (total <= lim) {
+                const int base = reserve(total);
+                if (cnt > 0 && base >= 0 && base + total <= kRowCap) {
+                    pos += base;
+#pragma unroll
+                    for (int j = 0; j < kVec; j++) {
+                        const int e0 = wbase + (j * kThreads + tid) * EPV;
+#pragma unroll
+                        for (int q = 0; q < EPV; q++) {
+                            const float x = VO::get(v[j], q);
+                            if (x >= tval) { sr_store_agent(&crow[pos], pack(x, e0 + q)); pos++; }
+                        }
+                    }
+                }
+            } else {
+                // Many elements tie with the threshold value.  Equal values rank by ascending index, so
+                // besides everything above the threshold only the first (sel - #above) ties can matter.
+                int cgt = 0, ceq_all = 0;
+#pragma unroll
+                for (int j = 0; j < kVec; j++)
+#pragma unroll
+                    for (int q = 0; q < EPV; q++) {
+                        cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
+                        ceq_all += (VO::get(v[j], q) == tval) ? 1 : 0;
+                    }
+                int total_gt;
+                int pgt = block_excl_scan(cgt, &total_gt, sm);
+                const int total_eq = block_sum_i32(ceq_all, sm);
+                if (total_gt > lim) {
+                    (void)reserve(kOverflowMark);  // genuine overflow: the row is reported as unsupported
+                } else {
+                    const int n_eq = max(0, min(min(sel - total_gt, lim - total_gt), total_eq));
+                    const int base = reserve(total_gt + n_eq);
+                    const bool fits = base >= 0 && base + total_gt + n_eq <= kRowCap;
+                    if (cgt > 0 && fits) {
+                        pgt += base;
+#pragma unroll
+                        for (int j = 0; j < kVec; j++) {
+                            const int e0 = wbase + (j * kThreads + tid) * EPV;
+#pragma unroll
+                            for (int q = 0; q < EPV; q++) {
+                                const float x = VO::get(v[j], q);
+                                if (x > tval) { sr_store_agent(&crow[pgt], pack(x, e0 + q)); pgt++; }
+                            }
+                        }
+                    }
+                    int emitted = 0;
+                    if (n_eq > 0) {
+#pragma unroll
+                        for (int j = 0; j < kVec; j++) {  // ascending j, then tid, then q = ascending index
+                            if (emitted >= n_eq) continue;  // block-uniform
+                            int ceq = 0;
+#pragma unroll
+                            for (int q = 0; q < EPV; q++) ceq += (VO::get(v[j], q) == tval) ? 1 : 0;
+                            int tj;
+                            int rank = emitted + block_excl_scan(ceq, &tj, sm);
+                            if (ceq > 0 && fits) {
+                                const int e0 = wbase + (j * kThreads + tid) * EPV;
+#pragma unroll
+                                for (int q = 0; q < EPV; q++) {
+                                    if (VO::get(v[j], q) == tval) {
+                                        if (rank < n_eq) sr_store_agent(&crow[base + total_gt + rank], pack(tval, e0 + q));
+                                        rank++;
+                                    }
+                                }
+                            }
+                            emitted += tj;
+                        }
+                    }
+                }
             }
         }
+    } else if (nv > 0 && tid == 0) {
+        (void)__hip_atomic_fetch_add(cursor, kOverflowMark, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     SR_PROF(a, 3);
-    if (tid == 0) sr_store_agent(&a.cand_cnt[(size_t)slot * S + c], total);
+    if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 13] = (unsigned long long)sel; a.prof[(size_t)blockIdx.x * 16 + 14] = (unsigned long long)slot; }
 
     // hand the chunk over: drain this wave's write-through stores, meet, then count the chunk in
     sr_drain_stores();
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_add(&a.row_done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- scan mask ---------------------------------------------------------------------------------------
+// One keep-bit per window element of a row, in the selection kernel's access order: for every block of 64
+// 16-byte vectors, epv 64-bit words; bit l of word q = element q of the vector that lane l loads.  A bit is
+// set when the element lies inside the row, its allow-mask (if any) admits it and, for rows whose tail
+// fetches the history logits by id, it is not a history id.
+__global__ __launch_bounds__(256) void k_build_scan_mask(const SrScanDesc* descs, const SrRow* rows, const SrEdit* edits,
+                                                         const uint32_t* mask, int64_t mask_stride,
+                                                         unsigned long long* scan_mask, int64_t scan_stride, int vocab,
+                                                         int epv, int es, unsigned long long base_addr,
+                                                         long long stride_bytes)
+{
+    const SrScanDesc d = descs[blockIdx.x];
+    const SrRow rd = rows[d.row];
+    const int mis = (int)(((base_addr + (unsigned long long)d.row * (unsigned long long)stride_bytes) & 15ull) / (unsigned)es);
+    unsigned long long* dst = scan_mask + (size_t)blockIdx.x * scan_stride;
+    const uint32_t* src = ((d.flags & SR_SCAN_ALLOW) && rd.mask_row >= 0) ? mask + (size_t)rd.mask_row * mask_stride : nullptr;
+    for (int w = threadIdx.x; w < (int)scan_stride; w += blockDim.x) {
+        const int b = w / epv, q = w - b * epv;
+        const long long e_first = (long long)b * 64 * epv + q - mis;  // the element under lane 0
+        unsigned long long bits = 0ull;
+        if (!src && e_first >= 0 && e_first + 63ll * epv < vocab) {
+            bits = ~0ull;
+        } else {
+            for (int l = 0; l < 64; l++) {
+                const long long e = e_first + (long long)l * epv;
+                if (e >= 0 && e < vocab && (!src || mask_bit(src, (int)e))) bits |= 1ull << l;
+            }
+        }
+        dst[w] = bits;
+    }
+    __threadfence_block();
+    __syncthreads();
+    if (d.flags & SR_SCAN_HIST) {
+        const SrEdit* ed = edits + rd.edit_off;
+        uint32_t* dst32 = (uint32_t*)dst;
+        for (int e = threadIdx.x; e < rd.edit_cnt; e += blockDim.x) {
+            const int p = ed[e].id + mis;
+            const int b = p / (64 * epv), r = p - b * 64 * epv;
+            const int l = r / epv, q = r - l * epv;
+            atomicAnd(&dst32[((size_t)b * epv + q) * 2 + (l >> 5)], ~(1u << (l & 31)));
+        }
+    }
 }
 
 }  // namespace
@@ -959,5 +1330,16 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
         hipLaunchKernelGGL(k_topk_rows<8>, grid, block, 0, stream, a);
     else
         hipLaunchKernelGGL(k_topk_rows<4>, grid, block, 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, int n_scan, const SrRow* rows, const SrEdit* edits,
+                                     const uint32_t* mask, int64_t mask_stride, unsigned long long* scan_mask,
+                                     int64_t scan_stride, int vocab, int epv, unsigned long long base_addr,
+                                     long long stride_bytes, hipStream_t stream)
+{
+    if (n_scan <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_build_scan_mask, dim3((unsigned)n_scan), dim3(256), 0, stream, descs, rows, edits, mask,
+                       mask_stride, scan_mask, scan_stride, vocab, epv, epv == 8 ? 2 : 4, base_addr, stride_bytes);
     return hipGetLastError();
 }

@@ -19,14 +19,14 @@ struct SrRow {
     float frequency;
     float p_min;
     int32_t top_k;
-    int32_t sel;        // TOPK: min(vocab, k + history length when penalties apply); GREEDY: 1
+    int32_t sel;        // how many of the largest scanned logits the row needs (see the packer)
     int32_t path;       // SrPath
     int32_t edit_off;   // first SrEdit of this row
     int32_t edit_cnt;
     int32_t mask_row;   // row index into the allow-mask array, or -1
     int32_t n_prev;
     uint32_t flags;     // SR_ROW_* from the public header
-    int32_t pad;
+    int32_t scan_row;   // row index into the scan-mask array (row edges, allow-mask, history ids)
 };
 
 // One distinct in-range token id that the row's history or logit bias touches; sorted by id per row.
@@ -39,14 +39,22 @@ struct SrEdit {
     uint32_t has_bias;
 };
 
+// One row of the scan-mask array of the selection kernel: which batch row it is built for, and from what.
+struct SrScanDesc {
+    int32_t row;
+    uint32_t flags;
+};
+#define SR_SCAN_ALLOW 1u  // start from the row's allow-mask
+#define SR_SCAN_HIST 2u   // clear the row's history ids
+
 // Limits of the top-k selection kernel.
 #define SR_TK_THREADS 512
 #define SR_TK_VEC 19                       // 16-byte vectors held per thread
 #define SR_TK_GROUPS 4                     // group maxima per thread
 #define SR_TK_M (SR_TK_THREADS * SR_TK_GROUPS)
-#define SR_TK_CAP 3072                     // candidates one chunk may emit
-#define SR_TK_SEL_MAX 2048                 // largest k + history handled by the selection kernel
-#define SR_TK_TAIL_CAP 16384                // merged candidates the row tail holds (32 per thread)
+#define SR_TK_SEL_MAX 2048                 // most entries (candidates + history ids) the row tail sorts
+#define SR_TK_ROW_CAP 8192                 // candidates all chunks of a row may hand to its tail (16 per thread)
+#define SR_TK_WAVE_LIM 128                 // least per-wave share of SR_TK_ROW_CAP for the per-wave scan
 #define SR_TK_MAX_CHUNKS 128               // most workgroups one row is split over
 
 // Full-vocabulary path: nucleus candidates up to this count are sorted inside the row kernel.
