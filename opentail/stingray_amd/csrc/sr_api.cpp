@@ -21,7 +21,7 @@ inline bool has_history_penalty(const sr_row_params& p)
 void topk_geometry(int vocab, int dtype, int n_rows, int max_sel, int cu_count, int* chunks, int* chunk_vecs)
 {
     const int epv = dtype == SR_DTYPE_BF16 ? 8 : 4;
-    const int window = SR_TK_VEC * SR_TK_THREADS;                  // vectors a workgroup holds
+    const int window = (dtype == SR_DTYPE_BF16 ? SR_TK_VEC_BF16 : SR_TK_VEC) * SR_TK_THREADS;  // vectors a workgroup holds
     const int nvt = (vocab + 2 * epv - 2) / epv;                   // vectors of a row that starts mid-vector
     int s_min = (nvt + window - 1) / window;
     int s_par = (2 * cu_count + n_rows - 1) / std::max(n_rows, 1);  // aim for two workgroups per CU
@@ -121,7 +121,7 @@ void sr_destroy(sr_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
-    DeviceBuf* bufs[] = {&ctx->cand, &ctx->cand_cnt, &ctx->row_done, &ctx->argmax_best,
+    DeviceBuf* bufs[] = {&ctx->cand, &ctx->cand_cnt, &ctx->sched, &ctx->row_done, &ctx->argmax_best,
                          &ctx->work, &ctx->host_logits, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->spec_rows, &ctx->spec_probs};
@@ -390,8 +390,40 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         topk_geometry(b->vocab, dtype, n_sel, b->max_sel, ctx->cu_count, &a.chunks, &a.chunk_vecs);
         if (a.chunks > SR_TK_MAX_CHUNKS)
             return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary too large for the selection kernel");
-        // one full round of resident workgroups (two per CU) between a row's chunks and its tail
-        a.tail_lag = std::min(n_sel, std::max(1, (2 * ctx->cu_count + a.chunks - 1) / a.chunks));
+        // Dispatch order.  Workgroups are dispatched in grid order, two resident per CU; a round is that many
+        // consecutive workgroups.  A row's tail goes to the head of the round after the one that holds the row's
+        // last chunk: its chunks have at least all been dispatched by then and have usually finished, and tails
+        // that are ready do not queue behind later rows' chunks.
+        if (ctx->sched_rows != n_sel || ctx->sched_chunks != a.chunks) {
+            const int round = 2 * ctx->cu_count;
+            std::vector<uint32_t> sched;
+            sched.reserve((size_t)n_sel * (a.chunks + 1));
+            std::vector<int> ready_at((size_t)n_sel, 0);  // first position at which the row's tail may be placed
+            int next_tail = 0, row = 0, c = 0;
+            while (next_tail < n_sel) {
+                const int pos = (int)sched.size();
+                if (next_tail < row && pos >= ready_at[(size_t)next_tail]) {
+                    sched.push_back(0x80000000u | (uint32_t)next_tail);
+                    next_tail++;
+                } else if (row < n_sel) {
+                    sched.push_back(((uint32_t)c << 24) | (uint32_t)row);
+                    if (++c == a.chunks) {
+                        ready_at[(size_t)row] = (pos / round + 1) * round;
+                        c = 0;
+                        row++;
+                    }
+                } else {
+                    sched.push_back(0x80000000u | (uint32_t)next_tail);  // nothing left to overlap with
+                    next_tail++;
+                }
+            }
+            SR_HIP(ctx, ctx->sched.reserve(sched.size() * sizeof(uint32_t), st));
+            SR_HIP(ctx, hipMemcpyAsync(ctx->sched.p, sched.data(), sched.size() * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+            SR_HIP(ctx, hipStreamSynchronize(st));
+            ctx->sched_rows = n_sel;
+            ctx->sched_chunks = a.chunks;
+        }
+        a.sched = ctx->sched.as<uint32_t>();
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));
         SR_HIP(ctx, ctx->cand_cnt.reserve((size_t)std::max(n_sel, 1024) * sizeof(int32_t), st, true));
         SR_HIP(ctx, ctx->row_done.reserve((size_t)std::max(n_sel, 1024) * sizeof(uint32_t), st, true));

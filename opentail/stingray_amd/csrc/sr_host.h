@@ -59,6 +59,8 @@ struct sr_ctx {
     DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
+    DeviceBuf sched;                     // dispatch order of the selection kernel's workgroups
+    int sched_rows = 0, sched_chunks = 0;
     int last_epv = 4;                    // vector width of the last launch: what an upload builds scan masks for
 };
 

@@ -22,9 +22,9 @@ struct SrTopkArgs {
     int32_t vocab;
     int32_t dtype;           // 0 = f32, 1 = bf16
     int32_t chunks;          // chunk workgroups per row
-    int32_t tail_lag;        // the tail of row i is dispatched after the chunks of row i + tail_lag (<= n_rows)
     int32_t n_rows;          // rows in this launch: grid = n_rows * chunks chunk workgroups + n_rows tail workgroups
     int32_t chunk_vecs;      // 16-byte vectors per chunk, a multiple of 64
+    const uint32_t* sched;   // per workgroup in dispatch order: bit 31 = row tail, bits 24..30 = chunk, bits 0..23 = slot
     const int32_t* row_list; // rows handled by this launch (device)
     const SrRow* rows;
     const SrEdit* edits;

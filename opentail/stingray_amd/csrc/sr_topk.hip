@@ -29,7 +29,6 @@ namespace {
 
 constexpr int kThreads = SR_TK_THREADS;
 constexpr int kWaves = kThreads / SR_WAVE;
-constexpr int kVec = SR_TK_VEC;
 constexpr int kSelMax = SR_TK_SEL_MAX;
 constexpr int kRowCap = SR_TK_ROW_CAP;
 constexpr uint32_t kKeyNegInf = 0x007fffffu;  // sr_okey(-inf)
@@ -40,6 +39,8 @@ constexpr int kOverflowMark = 1 << 24;        // added to a row's cursor by a ch
 constexpr int kCandRegs = kRowCap / kThreads;   // candidates a thread holds in the row tail (16)
 constexpr int kSortRegs = kSelMax / kThreads;   // sort elements per thread (4)
 constexpr int kHistRegs = kSelMax / kThreads;   // history ids per thread (4)
+constexpr int kBins = 1024;                     // histogram bins of the row tail
+constexpr int kBinsPerLane = kBins / SR_WAVE;
 
 struct TopkSmem {
     uint32_t xa[kSelMax];  // gathered list, then sort exchange (three 32-bit words per element)
@@ -51,8 +52,11 @@ struct TopkSmem {
     uint32_t hist[256];
     uint32_t red[2 * kWaves];
     uint32_t bcast[16];
-    uint32_t boff[257];    // first list position of every histogram bin
-    uint32_t bfill[256];   // entries scattered into the bin so far
+    unsigned long long ksum;   // chunk scan: sum of the waves' threshold estimates
+    uint32_t btotal;           // chunk scan: elements of the chunk at or above the shared threshold
+    uint32_t bhist[kBins];     // live entries per bin of distance below the maximum
+    uint32_t boff[kBins + 1];  // first list position of every bin
+    uint32_t bfill[kBins];     // entries scattered into the bin so far
 };
 
 // ---- block-wide radix select over keys produced by a per-thread enumerator -----------------------
@@ -148,7 +152,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <int EPV> struct VecOps;
 template <> struct VecOps<4> {  // four fp32 per 16-byte vector
     static __device__ __forceinline__ float get(const u32x4& v, int c) { return sr_u2f(v[c]); }
-    static __device__ __forceinline__ void keep_if(u32x4& v, int c, bool keep) { v[c] = keep ? v[c] : 0xff800000u; }
     static __device__ __forceinline__ u32x4 neg_inf() { return (u32x4)(0xff800000u); }
 };
 template <> struct VecOps<8> {  // eight bf16 per 16-byte vector; the upcast to fp32 is exact
@@ -156,12 +159,6 @@ template <> struct VecOps<8> {  // eight bf16 per 16-byte vector; the upcast to 
     {
         uint32_t w = v[c >> 1];
         return sr_u2f((c & 1) ? (w & 0xffff0000u) : (w << 16));
-    }
-    static __device__ __forceinline__ void keep_if(u32x4& v, int c, bool keep)
-    {
-        const uint32_t w = v[c >> 1];
-        const uint32_t dead = (c & 1) ? ((w & 0x0000ffffu) | 0xff800000u) : ((w & 0xffff0000u) | 0x0000ff80u);
-        v[c >> 1] = keep ? w : dead;
     }
     static __device__ __forceinline__ u32x4 neg_inf() { return (u32x4)(0xff80ff80u); }
 };
@@ -647,64 +644,61 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         each_key([&](uint32_t k) { lmaxk = k > lmaxk ? k : lmaxk; });
 #pragma unroll
         for (int r = 0; r < kHistRegs; r++) lmaxk = (hraw[r] != 0u && hadj[r] > lmaxk) ? hadj[r] : lmaxk;
-        if (tid < 256) sm.hist[tid] = 0u;
+        for (int i = tid; i < kBins; i += kThreads) { sm.bhist[i] = 0u; sm.bfill[i] = 0u; }
         if (tid == 0) sm.bcast[4] = 0u;
         const uint32_t kmaxn = block_max_u32(lmaxk, sm);  // its barriers also publish the cleared histogram
         // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
         if (kmaxn == 0u) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
         mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
-        // How far an entry lies below the maximum, in 1/14 of a log-unit: -1 = absent or dead, else 0..255.
+        // How far an entry lies below the maximum, in 1/56 of a log-unit: -1 = absent or dead, else 0..1023.
         // Monotone in the key, so "bin <= b" is a prefix of the descending order.
         auto bin_of = [&](uint32_t key) SR_INL -> int {
             if (key == 0u) return -1;
             const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx);
             if (x < -18.1f) return -1;
-            return min(max((int)__fmul_rn(x, -14.0f), 0), 255);
+            return min(max((int)__fmul_rn(x, -56.0f), 0), kBins - 1);
         };
 #pragma unroll
         for (int r = 0; r < kCandRegs; r++)
-            if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.hist[b], 1u); }
+            if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.bhist[b], 1u); }
 #pragma unroll
         for (int r = 0; r < kHistRegs; r++) {
             const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
-            if (b >= 0) atomicAdd(&sm.hist[b], 1u);
+            if (b >= 0) atomicAdd(&sm.bhist[b], 1u);
         }
         __syncthreads();
         // every wave reads the histogram: live entries, and the first bin at which the k best are complete
-        int bstar = 255, n_live, n_keep, max_bin;
+        int bstar = kBins - 1, n_live, n_keep, max_bin;
         {
+            // lane l owns bins [l * kBinsPerLane, (l + 1) * kBinsPerLane)
             const int lane = sr_lane();
-            const uint32_t h0 = sm.hist[4 * lane], h1 = sm.hist[4 * lane + 1], h2 = sm.hist[4 * lane + 2],
-                           h3 = sm.hist[4 * lane + 3];
-            const int tot = (int)(h0 + h1 + h2 + h3);
+            const uint32_t* hb = sm.bhist + lane * kBinsPerLane;
+            int tot = 0;
+#pragma unroll
+            for (int q = 0; q < kBinsPerLane; q++) tot += (int)hb[q];
             const int incl = sr_wave_incl_scan_i32(tot);
             n_live = __shfl(incl, SR_WAVE - 1);
-            n_keep = n_live;
             const int need = min(rd.top_k, n_live);
             const unsigned long long bal = __ballot(incl >= need);
             const int L = bal ? (int)__ffsll((long long)bal) - 1 : SR_WAVE - 1;
-            const int c = incl - tot;
-            int bq = 4 * lane + 3, cq = incl;
-            if (c + (int)h0 >= need) { bq = 4 * lane; cq = c + (int)h0; }
-            else if (c + (int)(h0 + h1) >= need) { bq = 4 * lane + 1; cq = c + (int)(h0 + h1); }
-            else if (c + (int)(h0 + h1 + h2) >= need) { bq = 4 * lane + 2; cq = c + (int)(h0 + h1 + h2); }
+            int c = incl - tot, bq = lane * kBinsPerLane + kBinsPerLane - 1, cq = incl;
+            bool found = false;
+            uint32_t hm = 0u;
+            const bool w0 = sr_wave_id() == 0;
+#pragma unroll
+            for (int q = 0; q < kBinsPerLane; q++) {
+                const uint32_t h = hb[q];
+                if (w0) sm.boff[lane * kBinsPerLane + q] = (uint32_t)c;
+                c += (int)h;
+                if (!found) hm = max(hm, h);  // bins up to and including the one that completes the k best
+                if (!found && c >= need) { bq = lane * kBinsPerLane + q; cq = c; found = true; }
+            }
+            if (w0 && lane == SR_WAVE - 1) sm.boff[kBins] = (uint32_t)incl;
             bstar = __shfl(bq, L);
             n_keep = __shfl(cq, L);
             // the fullest kept bin bounds the ranking loop below
-            uint32_t hm = 0u;
-            if (4 * lane <= bstar) hm = h0;
-            if (4 * lane + 1 <= bstar) hm = max(hm, h1);
-            if (4 * lane + 2 <= bstar) hm = max(hm, h2);
-            if (4 * lane + 3 <= bstar) hm = max(hm, h3);
+            if (lane > L) hm = 0u;
             max_bin = (int)sr_wave_max_u32(hm);
-            if (sr_wave_id() == 0) {
-                sm.boff[4 * lane] = (uint32_t)c;
-                sm.boff[4 * lane + 1] = (uint32_t)c + h0;
-                sm.boff[4 * lane + 2] = (uint32_t)c + h0 + h1;
-                sm.boff[4 * lane + 3] = (uint32_t)c + h0 + h1 + h2;
-                if (lane == SR_WAVE - 1) sm.boff[256] = (uint32_t)incl;
-                sm.bfill[4 * lane] = 0u; sm.bfill[4 * lane + 1] = 0u; sm.bfill[4 * lane + 2] = 0u; sm.bfill[4 * lane + 3] = 0u;
-            }
         }
         m2 = n_live;
         bool by_bins = true;  // kept entries are laid out bin by bin and ranked inside their bin
@@ -712,7 +706,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             // a flat row: only the k best candidates outside the history can matter
             by_bins = false;
             if (n_c > rd.top_k) select_top(rd.top_k);
-            bstar = 255;
+            bstar = kBins - 1;
             int mine = 0;
 #pragma unroll
             for (int r = 0; r < kCandRegs; r++)
@@ -780,7 +774,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             for (int i = tid; i < ms; i += kThreads) {
                 const uint32_t mh = sm.xa[i], mm = sm.xb[i], ml = sm.xc[i];
                 const int b = bin_of(mh);
-                const int p0 = (int)sm.boff[b], p1 = p0 + (int)sm.hist[b];
+                const int p0 = (int)sm.boff[b], p1 = p0 + (int)sm.bhist[b];
                 int rank = p0;
                 for (int j = p0; j < p1; j++) rank += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
                 if (rank < kk) {
@@ -870,12 +864,28 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     // Sampler.cs:326-349: running sum (probs[t] becomes cum[t]); top-p cuts after the first cum >= TopP
     if (tid == 0) {
         const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
+        const float top_p = use_top_p ? rd.top_p : __uint_as_float(0x7f800000u);  // +inf: never reached
         float cum = 0.0f;
         int cnt = count;
-        for (int t = 0; t < count; t++) {
-            cum = __fadd_rn(cum, sm.probs[t]);
-            sm.probs[t] = cum;
-            if (use_top_p && cum >= rd.top_p) { cnt = t + 1; break; }
+        // four entries per step, the next four already in flight (the stores of a step must not hold up the loads
+        // of the following one); entries past `count` are computed but never looked at
+        float4* p4 = (float4*)sm.probs;
+        float4 cur = p4[0];
+        for (int t = 0; t < count; t += 4) {
+            const float4 nxt = p4[(t >> 2) + 1];
+            float4 c;
+            c.x = __fadd_rn(cum, cur.x);
+            c.y = __fadd_rn(c.x, cur.y);
+            c.z = __fadd_rn(c.y, cur.z);
+            c.w = __fadd_rn(c.z, cur.w);
+            p4[t >> 2] = c;
+            if (c.w >= top_p) {  // the sums never decrease: the first one to reach TopP is among these four
+                const int q = (c.x >= top_p) ? 0 : (c.y >= top_p) ? 1 : (c.z >= top_p) ? 2 : 3;
+                if (t + q < count) cnt = t + q + 1;
+                break;
+            }
+            cum = c.w;
+            cur = nxt;
         }
         sm.bcast[6] = (uint32_t)cnt;
     }
@@ -895,36 +905,19 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 }
 
 // ---- the kernel --------------------------------------------------------------------------------------
-template <int EPV>
+template <int EPV, int kVec>
 __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 {
     __shared__ TopkSmem sm;
     using VO = VecOps<EPV>;
     const int tid = threadIdx.x, lane = sr_lane();
     const int S = a.chunks;
-    // Grid order: [chunks of row 0] ... and, from row `lag` on, the tail of row i - lag right after the chunks
-    // of row i; the tails of the last `lag` rows close the grid.  A tail workgroup is therefore dispatched
-    // after all chunk workgroups of its row (it waits, bounded, only on work that is already running),
-    // about one full round of workgroups later, so it rarely waits at all and overlaps later rows' streaming.
-    const int lag = a.tail_lag;
-    const int bid = (int)blockIdx.x;
-    const int head = lag * S;                       // rows [0, lag): chunks only
-    const int per = S + 1;                          // rows [lag, n_rows): S chunks + one tail
-    const int mid_end = head + (a.n_rows - lag) * per;
-    int slot_, c_;
-    bool is_tail;
-    if (bid < head) {
-        slot_ = bid / S; c_ = bid - slot_ * S; is_tail = false;
-    } else if (bid < mid_end) {
-        const int g = (bid - head) / per, w = (bid - head) - g * per;
-        is_tail = (w == S);
-        slot_ = is_tail ? g : lag + g;
-        c_ = w;
-    } else {
-        is_tail = true;
-        slot_ = (a.n_rows - lag) + (bid - mid_end);
-        c_ = 0;
-    }
+    // The host lays the workgroups out in dispatch order: chunk workgroups row by row, and the tail of a row
+    // one full round of resident workgroups after the row's last chunk, so that a tail is dispatched after all
+    // chunk workgroups of its row (it waits, bounded, only on work that is already running) and rarely waits.
+    const uint32_t item = a.sched[blockIdx.x];
+    const bool is_tail = (item >> 31) != 0u;
+    const int slot_ = (int)(item & 0xffffffu), c_ = (int)((item >> 24) & 0x7fu);
     if (is_tail) {
         const int tslot = slot_;
         const int trow = a.row_list[tslot];
@@ -960,10 +953,21 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     const int sel = rd.sel;
     unsigned long long* crow = a.cand + (size_t)slot * kRowCap;
     int* cursor = a.cand_cnt + slot;
-    auto pack = [](float x, int idx) SR_INL -> unsigned long long {
-        return ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx;
+    // a 32-bit byte offset from the wave-uniform list base: the base stays in scalar registers
+    auto cand_store = [](unsigned long long* base, uint32_t pos, unsigned long long v) SR_INL {
+        sr_store_agent((unsigned long long*)((char*)base + (size_t)(pos * 8u)), v);
     };
-    SR_PROF(a, 0);
+    auto pack = [](float x, int idx) SR_INL -> unsigned long long {
+        // A real copy that the compiler cannot fold: otherwise every register of the chunk is coalesced with the
+        // high half of a 64-bit store operand, which must sit in an odd register -- and only half of them are.
+        float xc;
+        asm volatile("v_mov_b32 %0, %1" : "=v"(xc) : "v"(x));
+        return ((unsigned long long)sr_f2u(xc) << 32) | (unsigned long long)(uint32_t)idx;
+    };
+    // phase timestamps stay in registers until the end: a store ahead of the scan-mask loads would keep the
+    // compiler from using scalar loads for them
+    unsigned long long pt0 = 0, pt1 = 0, pt2 = 0;
+    if (a.prof) pt0 = wall_clock64();
 
     // The row is read as 16-byte vectors from the aligned address at or below its start: window element
     // p is row element p - mis.  Chunks are whole multiples of 64 vectors of that window.
@@ -977,37 +981,64 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 
     if (nv > 0 && sel <= kSelMax) {
         const u32x4* cp = (const u32x4*)(rowp - (size_t)mis * ES) + f0;
-        u32x4 v[kVec];
+        // the chunk as fp32 in registers (the upcast of bf16 is exact)
+        float xv[kVec * EPV];
+        {
+            u32x4 t[kVec];
 #pragma unroll
-        for (int j = 0; j < kVec; j++) {
-            const int f = j * kThreads + tid;
-            v[j] = (f < nv) ? __builtin_nontemporal_load(&cp[f]) : VO::neg_inf();
+            for (int j = 0; j < kVec; j++) {
+                const int f = j * kThreads + tid;
+                t[j] = (f < nv) ? __builtin_nontemporal_load(&cp[f]) : VO::neg_inf();
+            }
+            // unpack in load order, one vector at a time, so that a packed vector's registers are free again
+            // before the next one is widened
+#pragma unroll
+            for (int j = 0; j < kVec; j++) {
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int q = 0; q < EPV; q++) xv[j * EPV + q] = VO::get(t[j], q);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         // The scan mask holds one keep-bit per window element in this kernel's access order: for every
         // block of 64 vectors, EPV 64-bit words, word q bit l = element q of the vector of lane l.  It
         // carries the row's edges, its allow-mask and, when the row tail fetches them, its history ids,
         // and is wave-uniform: scalar loads, one select per element.
         {
-            const unsigned long long* srow = a.scan_mask + (size_t)rd.scan_row * (size_t)a.scan_stride;
+            // read through the constant address space: the mask was written by an earlier launch, and scalar
+            // loads need the compiler to know that nothing in this kernel writes it
+            typedef const unsigned long long __attribute__((address_space(4))) const_u64;
+            const_u64* srow = (const_u64*)(uintptr_t)(a.scan_mask + (size_t)rd.scan_row * (size_t)a.scan_stride);
             const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
             const int nblk = (nvt + 63) >> 6;
 #pragma unroll
             for (int j = 0; j < kVec; j++) {
                 const int blk = (f0 >> 6) + j * (kThreads / SR_WAVE) + wave_u;
                 if (blk < nblk) {
-                    const unsigned long long* mp = srow + (size_t)blk * EPV;
+                    const_u64* mp = srow + (size_t)blk * EPV;
 #pragma unroll
-                    for (int q = 0; q < EPV; q++) VO::keep_if(v[j], q, __builtin_amdgcn_inverse_ballot_w64(mp[q]));
+                    for (int q = 0; q < EPV; q++) xv[j * EPV + q] = __builtin_amdgcn_inverse_ballot_w64(mp[q]) ? xv[j * EPV + q] : SR_NEG_INF;
                 }
             }
         }
-        SR_PROF(a, 1);
+        if (a.prof) pt1 = wall_clock64();
 
-        const int wlim = kRowCap / (S * kWaves);  // candidates one wave may hand over
-        if (sel <= SR_WAVE && wlim >= SR_TK_WAVE_LIM) {
-            // ---- every wave on its own: no workgroup barrier --------------------------------------------
-            // every lane owns four interleaved groups of vectors (j mod 4); the sel-th largest of the wave's
-            // 256 group maxima, found bit by bit, is a lower bound on the wave's sel-th largest element
+        const int wlim = kRowCap / (S * kWaves);  // candidates one wave may hand over when waves work alone
+        const int blim = min(kRowCap / S, 2 * sel + 128);  // candidates the chunk may hand over otherwise
+        // sel <= 64: every wave on its own, no workgroup barrier.  Larger sel: the waves agree on one threshold
+        // estimated from their group maxima, and keep it if the chunk holds between sel and blim elements at
+        // or above it; else (and on short chunks) the exact selection further down decides.
+        const bool wave_mode = sel <= SR_WAVE && wlim >= SR_TK_WAVE_LIM;
+        const bool shared_mode = !wave_mode && nv > 4 * kThreads && sel <= SR_TK_M && blim >= sel;
+        bool handed_over = false;
+        if (shared_mode) {
+            if (tid == 0) { sm.ksum = 0ull; sm.btotal = 0u; }
+            __syncthreads();
+        }
+        if (wave_mode || shared_mode) {
+            // every lane owns four interleaved groups of vectors (j mod 4); the need-th largest of the wave's
+            // 256 group maxima is found bit by bit.  need = sel makes it a lower bound on the wave's sel-th
+            // largest element.
             uint32_t gk[SR_TK_GROUPS];
 #pragma unroll
             for (int g = 0; g < SR_TK_GROUPS; g++) {
@@ -1015,8 +1046,19 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                 for (int j = g; j < kVec; j += SR_TK_GROUPS)
 #pragma unroll
-                    for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, VO::get(v[j], q));
+                    for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, xv[j * EPV + q]);
                 gk[g] = sr_okey(mxv);
+            }
+            int need = sel;
+            if (shared_mode) {
+                // aim a little above sel elements (the estimate scatters by a few percent): with a fraction p of the
+                // chunk above the threshold,
+                // a group of n_g elements has its maximum above it with probability 1 - (1 - p)^n_g
+                const float n_elem = (float)nv * (float)EPV;
+                const float p = fminf(fminf(1.12f * (float)sel + 40.0f, 0.5f * (float)(sel + blim)) / n_elem, 0.5f);
+                const float n_g = n_elem / (float)SR_TK_M;
+                const float frac = 1.0f - __expf(n_g * __logf(1.0f - p));
+                need = min(max((int)(frac * (float)(SR_WAVE * SR_TK_GROUPS) + 0.5f), 1), SR_WAVE * SR_TK_GROUPS);
             }
             uint32_t K = 0u;
 #pragma unroll 1
@@ -1025,49 +1067,67 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 int cge = 0;
 #pragma unroll
                 for (int g = 0; g < SR_TK_GROUPS; g++) cge += __popcll(__ballot(gk[g] >= cnd));
-                if (cge >= sel) K = cnd;
+                if (cge >= need) K = cnd;
+            }
+            if (shared_mode) {
+                // the mean of the waves' estimates (as keys: they lie close together)
+                if (lane == 0) atomicAdd(&sm.ksum, (unsigned long long)K);
+                __syncthreads();
+                K = (uint32_t)(sm.ksum / (unsigned long long)kWaves);
             }
             // -inf never enters the candidate set (Sampler.cs:240-249: strict v <= -inf rejects it)
             float tval = (K <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(K);
-            SR_PROF(a, 2);
+            if (a.prof) pt2 = wall_clock64();
             int total = 0;  // wave-uniform: the comparisons land in scalar registers
 #pragma unroll
             for (int j = 0; j < kVec; j++)
 #pragma unroll
-                for (int q = 0; q < EPV; q++) total += __popcll(__ballot(VO::get(v[j], q) >= tval));
-            if (total <= wlim) {
+                for (int q = 0; q < EPV; q++) total += __popcll(__ballot(xv[j * EPV + q] >= tval));
+            bool emit_all = wave_mode && total <= wlim;
+            if (shared_mode) {
+                if (lane == 0) atomicAdd(&sm.btotal, (uint32_t)total);
+                __syncthreads();
+                const int bt = (int)sm.btotal;
+                emit_all = bt >= sel && bt <= blim;
+            }
+            handed_over = wave_mode || emit_all;
+            if (emit_all) {
                 int base = 0;
                 if (lane == 0 && total > 0)
                     base = __hip_atomic_fetch_add(cursor, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 base = __builtin_amdgcn_readfirstlane(base);
                 if (total > 0 && base >= 0 && base + total <= kRowCap) {
                     int off = base;
+                    // an opaque copy: the comparisons of the counting pass must not be kept alive (two scalar
+                    // registers each) for this pass
+                    float tv = tval;
+                    asm volatile("" : "+v"(tv));
 #pragma unroll
                     for (int j = 0; j < kVec; j++) {
                         const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                         for (int q = 0; q < EPV; q++) {
-                            const float x = VO::get(v[j], q);
-                            const unsigned long long bal = __ballot(x >= tval);
+                            const float x = xv[j * EPV + q];
+                            const unsigned long long bal = __ballot(x >= tv);
                             if (bal) {
-                                if (x >= tval) {
+                                if (x >= tv) {
                                     const int pos = off + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32),
                                                               __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u));
-                                    sr_store_agent(&crow[pos], pack(x, e0 + q));
+                                    cand_store(crow, (uint32_t)(pos), pack(x, e0 + q));
                                 }
                                 off += __popcll(bal);
                             }
                         }
                     }
                 }
-            } else {
+            } else if (wave_mode) {
                 // Many elements at or above the bound.  Equal values rank by ascending index, so besides
                 // everything above the threshold only the first (sel - #above) ties can matter.
                 int cgt = 0;
 #pragma unroll
                 for (int j = 0; j < kVec; j++)
 #pragma unroll
-                    for (int q = 0; q < EPV; q++) cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
+                    for (int q = 0; q < EPV; q++) cgt += (xv[j * EPV + q] > tval) ? 1 : 0;
                 int total_gt = sr_wave_sum_i32(cgt);
                 if (total_gt > wlim) {
                     // the lane maxima bound is too loose (the large values sit in few lanes): the exact sel-th
@@ -1082,7 +1142,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                         for (int j = 0; j < kVec; j++)
 #pragma unroll
-                            for (int q = 0; q < EPV; q++) cge += __popcll(__ballot(VO::get(v[j], q) >= fc));
+                            for (int q = 0; q < EPV; q++) cge += __popcll(__ballot(xv[j * EPV + q] >= fc));
                         if (cge >= sel) K2 = cnd;
                     }
                     tval = sr_okey_inv(K2);
@@ -1090,14 +1150,14 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                     for (int j = 0; j < kVec; j++)
 #pragma unroll
-                        for (int q = 0; q < EPV; q++) cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
+                        for (int q = 0; q < EPV; q++) cgt += (xv[j * EPV + q] > tval) ? 1 : 0;
                     total_gt = sr_wave_sum_i32(cgt);
                 }
                 int total_eq = 0;
 #pragma unroll
                 for (int j = 0; j < kVec; j++)
 #pragma unroll
-                    for (int q = 0; q < EPV; q++) total_eq += __popcll(__ballot(VO::get(v[j], q) == tval));
+                    for (int q = 0; q < EPV; q++) total_eq += __popcll(__ballot(xv[j * EPV + q] == tval));
                 const int n_eq = max(0, min(min(sel - total_gt, wlim - total_gt), total_eq));
                 const int incl = sr_wave_incl_scan_i32(cgt);
                 total = total_gt + n_eq;
@@ -1113,8 +1173,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                             const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                             for (int q = 0; q < EPV; q++) {
-                                const float x = VO::get(v[j], q);
-                                if (x > tval) { sr_store_agent(&crow[pos], pack(x, e0 + q)); pos++; }
+                                const float x = xv[j * EPV + q];
+                                if (x > tval) { cand_store(crow, (uint32_t)(pos), pack(x, e0 + q)); pos++; }
                             }
                         }
                     }
@@ -1124,15 +1184,15 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                         if (emitted >= n_eq) continue;  // wave-uniform
                         int ceq = 0;
 #pragma unroll
-                        for (int q = 0; q < EPV; q++) ceq += (VO::get(v[j], q) == tval) ? 1 : 0;
+                        for (int q = 0; q < EPV; q++) ceq += (xv[j * EPV + q] == tval) ? 1 : 0;
                         const int ie = sr_wave_incl_scan_i32(ceq);
                         int rank = emitted + ie - ceq;
                         if (ceq > 0) {
                             const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                             for (int q = 0; q < EPV; q++) {
-                                if (VO::get(v[j], q) == tval) {
-                                    if (rank < n_eq) sr_store_agent(&crow[base + total_gt + rank], pack(tval, e0 + q));
+                                if (xv[j * EPV + q] == tval) {
+                                    if (rank < n_eq) cand_store(crow, (uint32_t)(base + total_gt + rank), pack(tval, e0 + q));
                                     rank++;
                                 }
                             }
@@ -1141,7 +1201,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                     }
                 }
             }
-        } else {
+        }
+        if (!handed_over) {
             // ---- the whole workgroup: threshold from 2048 group maxima (or exactly, on a short chunk) ------
             auto reserve = [&](int n) SR_INL -> int {  // all threads; returns the first list position
                 __syncthreads();
@@ -1157,7 +1218,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
-                        for (int q = 0; q < EPV; q++) body(sr_okey(VO::get(v[j], q)));
+                        for (int q = 0; q < EPV; q++) body(sr_okey(xv[j * EPV + q]));
                 };
                 tkey = block_radix_select(each_elem, sel, sm);
             } else {
@@ -1170,7 +1231,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #pragma unroll
                     for (int j = g; j < kVec; j += SR_TK_GROUPS)
 #pragma unroll
-                        for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, VO::get(v[j], q));
+                        for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, xv[j * EPV + q]);
                     gk[g] = sr_okey(mxv);
                 }
                 auto each_gk = [&](auto&& body) SR_INL {
@@ -1179,13 +1240,13 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 };
                 tkey = (sel > SR_TK_M) ? 0u : block_radix_select(each_gk, sel, sm);
             }
-            SR_PROF(a, 2);
+            if (a.prof) pt2 = wall_clock64();
             const float tval = (tkey <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(tkey);
             int cnt = 0;
 #pragma unroll
             for (int j = 0; j < kVec; j++)
 #pragma unroll
-                for (int q = 0; q < EPV; q++) cnt += (VO::get(v[j], q) >= tval) ? 1 : 0;
+                for (int q = 0; q < EPV; q++) cnt += (xv[j * EPV + q] >= tval) ? 1 : 0;
             // a chunk hands over at most `lim` candidates, so that the row list can hold all chunks of a row
             const int lim = min(kRowCap / S, 2 * sel + 128);
             int total;
@@ -1201,8 +1262,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                         const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                         for (int q = 0; q < EPV; q++) {
-                            const float x = VO::get(v[j], q);
-                            if (x >= tval) { sr_store_agent(&crow[pos], pack(x, e0 + q)); pos++; }
+                            const float x = xv[j * EPV + q];
+                            if (x >= tval) { cand_store(crow, (uint32_t)(pos), pack(x, e0 + q)); pos++; }
                         }
                     }
                 }
@@ -1214,8 +1275,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 for (int j = 0; j < kVec; j++)
 #pragma unroll
                     for (int q = 0; q < EPV; q++) {
-                        cgt += (VO::get(v[j], q) > tval) ? 1 : 0;
-                        ceq_all += (VO::get(v[j], q) == tval) ? 1 : 0;
+                        cgt += (xv[j * EPV + q] > tval) ? 1 : 0;
+                        ceq_all += (xv[j * EPV + q] == tval) ? 1 : 0;
                     }
                 int total_gt;
                 int pgt = block_excl_scan(cgt, &total_gt, sm);
@@ -1233,8 +1294,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                             const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                             for (int q = 0; q < EPV; q++) {
-                                const float x = VO::get(v[j], q);
-                                if (x > tval) { sr_store_agent(&crow[pgt], pack(x, e0 + q)); pgt++; }
+                                const float x = xv[j * EPV + q];
+                                if (x > tval) { cand_store(crow, (uint32_t)(pgt), pack(x, e0 + q)); pgt++; }
                             }
                         }
                     }
@@ -1245,15 +1306,15 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                             if (emitted >= n_eq) continue;  // block-uniform
                             int ceq = 0;
 #pragma unroll
-                            for (int q = 0; q < EPV; q++) ceq += (VO::get(v[j], q) == tval) ? 1 : 0;
+                            for (int q = 0; q < EPV; q++) ceq += (xv[j * EPV + q] == tval) ? 1 : 0;
                             int tj;
                             int rank = emitted + block_excl_scan(ceq, &tj, sm);
                             if (ceq > 0 && fits) {
                                 const int e0 = wbase + (j * kThreads + tid) * EPV;
 #pragma unroll
                                 for (int q = 0; q < EPV; q++) {
-                                    if (VO::get(v[j], q) == tval) {
-                                        if (rank < n_eq) sr_store_agent(&crow[base + total_gt + rank], pack(tval, e0 + q));
+                                    if (xv[j * EPV + q] == tval) {
+                                        if (rank < n_eq) cand_store(crow, (uint32_t)(base + total_gt + rank), pack(tval, e0 + q));
                                         rank++;
                                     }
                                 }
@@ -1268,6 +1329,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         (void)__hip_atomic_fetch_add(cursor, kOverflowMark, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     SR_PROF(a, 3);
+    if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 0] = pt0; a.prof[(size_t)blockIdx.x * 16 + 1] = pt1; a.prof[(size_t)blockIdx.x * 16 + 2] = pt2; }
     if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 13] = (unsigned long long)sel; a.prof[(size_t)blockIdx.x * 16 + 14] = (unsigned long long)slot; }
 
     // hand the chunk over: drain this wave's write-through stores, meet, then count the chunk in
@@ -1327,9 +1389,9 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
     if (n_rows <= 0) return hipSuccess;
     dim3 grid((unsigned)(n_rows * a.chunks + n_rows)), block(kThreads);  // chunk workgroups + one tail per row
     if (a.dtype == 1)
-        hipLaunchKernelGGL(k_topk_rows<8>, grid, block, 0, stream, a);
+        hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL(k_topk_rows<4>, grid, block, 0, stream, a);
+        hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC>), grid, block, 0, stream, a);
     return hipGetLastError();
 }
 

@@ -49,7 +49,8 @@ struct SrScanDesc {
 
 // Limits of the top-k selection kernel.
 #define SR_TK_THREADS 512
-#define SR_TK_VEC 19                       // 16-byte vectors held per thread
+#define SR_TK_VEC 19                       // 16-byte vectors of fp32 logits held per thread
+#define SR_TK_VEC_BF16 10                  // ... of bf16 logits: the same 40 thousand elements per workgroup
 #define SR_TK_GROUPS 4                     // group maxima per thread
 #define SR_TK_M (SR_TK_THREADS * SR_TK_GROUPS)
 #define SR_TK_SEL_MAX 2048                 // most entries (candidates + history ids) the row tail sorts
