@@ -151,10 +151,6 @@ def test_small_rows_with_ties_masks_and_every_cut(ctx):
                 RepetitionPenalty=float(rng.choice([1.0, 1.3])), PresencePenalty=float(rng.choice([0.0, 0.4])),
                 FrequencyPenalty=float(rng.choice([0.0, 0.25])), RepeatLastN=int(rng.choice([0, 3, 64])),
                 PreviousTokens=hist))
-        # greedy rows with penalties go down the full-vocabulary path, covered by its own tests
-        for p in params:
-            if p.Temperature == 0.0:
-                p.PreviousTokens = None
         _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits))
 
 
@@ -224,3 +220,82 @@ def test_round_trip_properties_at_full_size(ctx):
             assert t1[i] == am[i]
         else:
             assert w.logits[i, t1[i]] >= kth[i, p.TopK - 1]
+
+
+def test_penalties_that_raise_a_logit_keep_the_reference_over_selection(ctx):
+    # Sampler.cs:224-225 only ever looks at the raw top-(k + history length): a history token outside that
+    # set is not considered even when a negative penalty would lift it to the top.
+    logits = np.array([[10, 9, 8, 1, 0, -1, -2, -3]], dtype=np.float32)
+    p = SamplingParams(TopK=1, PresencePenalty=-20.0, PreviousTokens=[3])
+    for u in (0.0, 0.5, 0.99):
+        assert _check_rows(ctx, logits, [p], [u], _cuda(logits))[0] & 2
+    rng = np.random.default_rng(31)
+    V, rows = 40_000, 16
+    logits = rng.normal(0, 2.0, (rows, V)).astype(np.float32)
+    head = np.argsort(-logits, axis=1)
+    params = []
+    for i, k in enumerate([1, 5, 40, 64, 65, 200, 700, 1500, 3, 64, 65, 300, 33, 1, 900, 128]):
+        n_hist = int(rng.integers(20, 300))
+        hist = np.concatenate([head[i, rng.integers(0, 2 * k + 50, n_hist // 2)], rng.integers(0, V, n_hist - n_hist // 2)])
+        rng.shuffle(hist)
+        params.append(SamplingParams(
+            Temperature=float(rng.choice([0.0, 0.7, 1.2])) if i % 5 == 4 else float(rng.uniform(0.6, 1.3)), TopK=k,
+            TopP=float(rng.choice([1.0, 0.9])), MinP=float(rng.choice([0.0, 0.02])),
+            RepetitionPenalty=float(rng.choice([0.7, 1.0, 1.3])), PresencePenalty=float(rng.choice([-0.8, 0.0, 0.5])),
+            FrequencyPenalty=float(rng.choice([-0.3, 0.0, 0.2])), RepeatLastN=int(rng.choice([0, 16, 64])),
+            PreviousTokens=hist.tolist()))
+    for _ in range(3):
+        _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits))
+
+
+def test_large_values_concentrated_in_few_lanes(ctx):
+    # the per-wave bound comes from lane-group maxima: put every large value into 16 lanes of a wave so the bound
+    # is loose and the exact per-wave selection has to take over
+    rng = np.random.default_rng(32)
+    V, rows = 40_000, 8
+    logits = rng.normal(0, 1.0, (rows, V)).astype(np.float32)
+    e = np.arange(V)
+    hot = ((e // 4) % 512) < 16
+    logits[:, hot] += 40.0 + rng.random((rows, int(hot.sum()))).astype(np.float32)
+    params = [SamplingParams(Temperature=float(t), TopK=int(k), TopP=0.97)
+              for t, k in zip([1.0, 0.8, 1.3, 0.0, 1.0, 0.9, 1.1, 1.0], [64, 64, 40, 1, 7, 64, 33, 200])]
+    params[1].PreviousTokens = np.nonzero(hot)[0][:120].tolist()
+    params[1].RepetitionPenalty = 1.2
+    _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits))
+
+
+def test_flat_rows_with_a_history(ctx):
+    # every logit equal: the candidates all tie, the lowest indices win, and the penalised history ids drop out
+    V = 50_000
+    rng = np.random.default_rng(33)
+    logits = np.zeros((3, V), dtype=np.float32)
+    logits[2] = 1.25
+    hist = rng.integers(0, 3000, 300).tolist()
+    params = [SamplingParams(Temperature=1.0, TopK=1200, TopP=0.999, RepetitionPenalty=1.2, PreviousTokens=hist),
+              SamplingParams(Temperature=1.5, TopK=60, PresencePenalty=0.5, PreviousTokens=hist),
+              SamplingParams(Temperature=0.0, FrequencyPenalty=0.25, PreviousTokens=list(range(0, 40)))]
+    for u in (0.0, 0.31, 0.77, 0.9999):
+        _check_rows(ctx, logits, params, [u, u, u], _cuda(logits))
+
+
+def test_history_on_unaligned_rows_and_bf16(ctx):
+    import torch
+
+    rng = np.random.default_rng(34)
+    V, rows = 30_011, 6                                   # odd vocabulary: every row starts at another offset
+    logits = rng.normal(0, 1.5, (rows, V)).astype(np.float32)
+    head = np.argsort(-logits, axis=1)
+    params = []
+    for i, k in enumerate([1, 20, 64, 65, 400, 1000]):
+        hist = np.concatenate([head[i, :30], rng.integers(0, V, 100)]).tolist()
+        params.append(SamplingParams(Temperature=0.9 if i != 2 else 0.0, TopK=k, TopP=0.95, RepetitionPenalty=1.15,
+                                     FrequencyPenalty=0.1, PreviousTokens=hist))
+    allowed = np.stack([synthetic.run_mask(rng, V, d) for d in (0.5, 0.9, 0.3, 0.01, 0.8, 0.6)])
+    mask = pack_allow_mask(allowed)
+    _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits))
+    _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits), mask, np.array([1, 0, 1, 1, 1, 0], dtype=np.uint8))
+    bits = synthetic.to_bf16_bits(logits)
+    up = synthetic.bf16_bits_to_f32(bits)
+    _check_rows(ctx, up, params, rng.random(rows), _cuda(bits.view(np.int16), torch.bfloat16))
+    w = synthetic.config3(rows=32, bf16=True, full_chain=True)
+    _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits_bf16.view(np.int16), torch.bfloat16))
