@@ -39,7 +39,9 @@ __device__ static const uint64_t sr_exp2f_tab[32] = {
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
 };
 
-__device__ __forceinline__ float sr_expf(float x)
+// tab: the 32-entry table above, or a copy of it in LDS (a lookup per element from global memory is a long
+// dependent load)
+__device__ __forceinline__ float sr_expf_tab(float x, const uint64_t* tab)
 {
     const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
     const double shift = 0x1.8p+52;
@@ -60,7 +62,7 @@ __device__ __forceinline__ float sr_expf(float x)
     uint64_t ki = (uint64_t)__double_as_longlong(kd);
     kd = __dsub_rn(kd, shift);
     double r = __fma_rn(inv_ln2_n, xd, -kd);
-    uint64_t t = sr_exp2f_tab[ki & 31u];
+    uint64_t t = tab[ki & 31u];
     t += ki << (52 - 5);
     double s = __longlong_as_double((long long)t);
     double zz = __fma_rn(c0, r, c1);
@@ -70,6 +72,7 @@ __device__ __forceinline__ float sr_expf(float x)
     y = __dmul_rn(y, s);
     return __double2float_rn(y);
 }
+__device__ __forceinline__ float sr_expf(float x) { return sr_expf_tab(x, sr_exp2f_tab); }
 
 // ---- cross-workgroup hand-off without a full L2 write-back ----------------------------------------
 // Data one workgroup leaves for another (possibly on another XCD) is written with agent-scope stores

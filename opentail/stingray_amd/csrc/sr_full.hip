@@ -13,12 +13,17 @@
 
 namespace {
 
+#define FPROF(a, slot_, i_) do { if ((a).prof && (slot_) == 0 && threadIdx.x == 0) (a).prof[(i_)] = (unsigned long long)wall_clock64(); } while (0)
+
 constexpr int kT = SR_SEQ_THREADS;
 constexpr int kW = SR_SEQ_WAVES;
 constexpr int kSmall = SR_FULL_SMALL_CAP;  // survivors sorted inside the kernel
 
 struct FullSmem {
+    uint64_t exp_tab[32];  // copy of the expf table
     SrSeqSmem seq;
+    SrSeq8Smem seq8;
+    float lane_sum[SR_SEQ_CHAINS];
     float redf[kW];
     uint32_t redu[kW];
     int redi[kW];
@@ -91,6 +96,43 @@ __device__ __forceinline__ int blk_excl_scan(int v, int* total, FullSmem& sm)
     return base + incl - v;
 }
 
+
+// ---- one pass of the workgroup over a row ---------------------------------------------------------------
+// Calls f(value, index) for every element, any order, with 16-byte loads (four in flight per thread) where the
+// row allows it; with kWrite the value returned by f is stored back.  The caller synchronises.
+template <bool kWrite, typename F>
+__device__ __forceinline__ void row_pass(float* p, int n, F f)
+{
+    const int tid = threadIdx.x;
+    const int head = min(n, (int)((4u - (unsigned)(((uintptr_t)p >> 2) & 3u)) & 3u));  // elements before 16-byte alignment
+    if (tid < head) {
+        const float y = f(p[tid], tid);
+        if (kWrite) p[tid] = y;
+    }
+    float4* p4 = (float4*)(p + head);
+    const int nv = (n - head) >> 2;
+    auto one = [&](float4& a, int v) __attribute__((always_inline)) {
+        const int i = head + 4 * v;
+        a.x = f(a.x, i); a.y = f(a.y, i + 1); a.z = f(a.z, i + 2); a.w = f(a.w, i + 3);
+    };
+    int v = tid;
+    for (; v + 3 * kT < nv; v += 4 * kT) {
+        float4 a = p4[v], b = p4[v + kT], c = p4[v + 2 * kT], d = p4[v + 3 * kT];
+        one(a, v); one(b, v + kT); one(c, v + 2 * kT); one(d, v + 3 * kT);
+        if (kWrite) { p4[v] = a; p4[v + kT] = b; p4[v + 2 * kT] = c; p4[v + 3 * kT] = d; }
+    }
+    for (; v < nv; v += kT) {
+        float4 a = p4[v];
+        one(a, v);
+        if (kWrite) p4[v] = a;
+    }
+    const int done = head + 4 * nv;
+    if (tid < n - done) {
+        const float y = f(p[done + tid], done + tid);
+        if (kWrite) p[done + tid] = y;
+    }
+}
+
 // ---- exact left-to-right sum over term(i), i in [0, n) ------------------------------------------------
 // term(i) must be >= 0 (or +0 for "skipped").  With kSearch, stops at the first i whose running sum is
 // >= target and returns it in *found (else -1).
@@ -123,22 +165,41 @@ __device__ float tp_sum(Term term, int n, FullSmem& sm)
     if (n < 4) {
         return seq_sum<false>(term, n, 0.0f, 0.0f, &dummy, sm);
     }
-    const int w = n >= 8 ? 8 : 4;
-    const int nv = n / w, rem = n - nv * w;
-    float lane_sum[8];
+    if (n >= 8) {
+        // the eight lane accumulators as eight chains advanced together: one pass over the row
+        const int nv = n / 8, rem = n - nv * 8;
+        const int g = (int)threadIdx.x & (SR_SEQ_CHAINS - 1), lt = (int)threadIdx.x >> 3;
+        const bool extra = rem > 0 && g >= 8 - rem;
+        const int cnt = nv + (extra ? 1 : 0);
+        float s = 0.0f;
+        for (int base = 0; base < nv + 1; base += SR_SEQ_CHAIN_TILE) {
+            float x[SR_SEQ_RUN];
+            const int i0 = base + lt * SR_SEQ_RUN;
 #pragma unroll
-    for (int l = 0; l < 8; l++) {
-        lane_sum[l] = 0.0f;
-        if (l < w) {
-            const bool extra = rem > 0 && l >= w - rem;
-            const int cnt = nv + (extra ? 1 : 0);
-            auto lt = [&](int i) -> float { return i < nv ? term(i * w + l) : term(n - w + l); };
-            lane_sum[l] = seq_sum<false>(lt, cnt, 0.0f, 0.0f, &dummy, sm);
+            for (int j = 0; j < SR_SEQ_RUN; j++) {
+                const int i = i0 + j;
+                x[j] = (i < cnt) ? (i < nv ? term(i * 8 + g) : term(n - 8 + g)) : 0.0f;
+            }
+            sr_seq_tile8(x, &s, sm.seq8);
         }
+        __syncthreads();
+        if (lt == 0) sm.lane_sum[g] = s;
+        __syncthreads();
+        const float l0 = sm.lane_sum[0], l1 = sm.lane_sum[1], l2 = sm.lane_sum[2], l3 = sm.lane_sum[3],
+                    l4 = sm.lane_sum[4], l5 = sm.lane_sum[5], l6 = sm.lane_sum[6], l7 = sm.lane_sum[7];
+        __syncthreads();
+        return __fadd_rn(__fadd_rn(__fadd_rn(l0, l1), __fadd_rn(l2, l3)), __fadd_rn(__fadd_rn(l4, l5), __fadd_rn(l6, l7)));
     }
-    if (w == 8)
-        return __fadd_rn(__fadd_rn(__fadd_rn(lane_sum[0], lane_sum[1]), __fadd_rn(lane_sum[2], lane_sum[3])),
-                         __fadd_rn(__fadd_rn(lane_sum[4], lane_sum[5]), __fadd_rn(lane_sum[6], lane_sum[7])));
+    const int w = 4;
+    const int nv = n / w, rem = n - nv * w;
+    float lane_sum[4];
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+        const bool extra = rem > 0 && l >= w - rem;
+        const int cnt = nv + (extra ? 1 : 0);
+        auto lt = [&](int i) -> float { return i < nv ? term(i * w + l) : term(n - w + l); };
+        lane_sum[l] = seq_sum<false>(lt, cnt, 0.0f, 0.0f, &dummy, sm);
+    }
     return __fadd_rn(__fadd_rn(lane_sum[0], lane_sum[1]), __fadd_rn(lane_sum[2], lane_sum[3]));
 }
 
@@ -148,23 +209,26 @@ __device__ void normalize_row(float* p, int n, FullSmem& sm)
     const float sum = tp_sum([&](int i) -> float { return p[i]; }, n, sm);
     if (sum > 0.0f && sum != 1.0f) {
         const float inv = __fdiv_rn(1.0f, sum);
-        for (int i = threadIdx.x; i < n; i += kT) p[i] = __fmul_rn(p[i], inv);
+        row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
     }
     __syncthreads();
 }
 
 // k-th largest value of p[0..n) (1-based), p >= 0: FindKthLargest (Sampler.cs:624-645).
-__device__ float kth_largest(const float* p, int n, int k, FullSmem& sm)
+// With last_shift = 16 only the upper 16 bits are resolved: the result is then the smallest value of the
+// 65536-value bucket that holds the k-th largest.
+__device__ float kth_largest(const float* p, int n, int k, FullSmem& sm, int last_shift = 0)
 {
     uint32_t prefix = 0u, pmask = 0u;
     int need = k;
-    for (int shift = 24; shift >= 0; shift -= 8) {
+    for (int shift = 24; shift >= last_shift; shift -= 8) {
         if (threadIdx.x < 256) sm.hist[threadIdx.x] = 0u;
         __syncthreads();
-        for (int i = threadIdx.x; i < n; i += kT) {
-            const uint32_t key = sr_f2u(p[i]);
+        row_pass<false>(const_cast<float*>(p), n, [&](float x, int) -> float {
+            const uint32_t key = sr_f2u(x);
             if ((key & pmask) == prefix) atomicAdd(&sm.hist[(key >> shift) & 0xffu], 1u);
-        }
+            return x;
+        });
         __syncthreads();
         if (threadIdx.x == 0) {
             int c = 0, d = 255;
@@ -264,12 +328,12 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
 __device__ int row_argmax(const float* w, int n, FullSmem& sm)
 {
     unsigned long long best = 0ull;
-    for (int i = threadIdx.x; i < n; i += kT) {
-        const float v = w[i];
+    row_pass<false>(const_cast<float*>(w), n, [&](float v, int i) -> float {
         const uint32_t k = (v != v) ? 0xffffffffu : sr_okey(v);
         const unsigned long long e = ((unsigned long long)k << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
         best = e > best ? e : best;
-    }
+        return v;
+    });
     best = blk_max_u64(best, sm);
     return best ? (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull)) : 0;
 }
@@ -307,7 +371,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         const int am = row_argmax(p, n, sm);
         if (a.mode != 0) {
             __syncthreads();
-            for (int i = tid; i < n; i += kT) p[i] = (i == am) ? 1.0f : 0.0f;
+            row_pass<true>(p, n, [&](float, int i) -> float { return (i == am) ? 1.0f : 0.0f; });
         }
         if (tid == 0) {
             if (a.out_tokens) a.out_tokens[row] = am;
@@ -317,107 +381,122 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
     }
 
     if (phase == 1) {
+        if (tid < 32) sm.exp_tab[tid] = sr_exp2f_tab[tid];  // published by the barriers of the maximum below
+        FPROF(a, slot, 0);
         // Softmax (Sampler.cs:448-472)
         float m = SR_NEG_INF;
         bool nanv = false;
-        for (int i = tid; i < n; i += kT) {
-            const float v = p[i];
+        row_pass<false>(p, n, [&](float v, int) -> float {
             if (v != v) nanv = true;
             m = fmaxf(m, v);
-        }
+            return v;
+        });
         bool any_nan;
         m = blk_max_f(nanv ? __uint_as_float(0x7fc00000u) : m, &any_nan, sm);
+        FPROF(a, slot, 1);
         uint32_t flags = SR_KFLAG_FULL;
         if (any_nan || sr_f2u(m) == 0xff800000u) {
             const float uni = n > 0 ? __fdiv_rn(1.0f, (float)n) : 0.0f;
-            for (int i = tid; i < n; i += kT) p[i] = uni;
+            row_pass<true>(p, n, [&](float, int) -> float { return uni; });
             flags |= SR_KFLAG_DEGENERATE;
             __syncthreads();
         } else {
             int dummy;
             const float sum = seq_sum<false>(
                 [&](int i) -> float {
-                    const float e = sr_expf(__fsub_rn(p[i], m));
+                    const float e = sr_expf_tab(__fsub_rn(p[i], m), sm.exp_tab);
                     p[i] = e;
                     return e;
                 },
                 n, 0.0f, 0.0f, &dummy, sm);
             __syncthreads();
+            FPROF(a, slot, 2);
             if (sum > 0.0f && sum != 1.0f) {
                 const float inv = __fdiv_rn(1.0f, sum);
-                for (int i = tid; i < n; i += kT) p[i] = __fmul_rn(p[i], inv);
+                row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
             }
             __syncthreads();
         }
+        FPROF(a, slot, 3);
         // ApplyTopK + Normalize (Sampler.cs:71-81, :477-488): everything equal to the k-th value survives
         if (rd.top_k > 0 && rd.top_k < n) {
             const float kth = kth_largest(p, n, rd.top_k, sm);
-            for (int i = tid; i < n; i += kT)
-                if (p[i] < kth) p[i] = 0.0f;
+            row_pass<true>(p, n, [&](float x, int) -> float { return x < kth ? 0.0f : x; });
             __syncthreads();
             normalize_row(p, n, sm);
         }
+        FPROF(a, slot, 4);
         // ApplyMinP (Sampler.cs:493-503)
         if (rd.min_p > 0.0f) {
             float mp = 0.0f;
-            for (int i = tid; i < n; i += kT) mp = fmaxf(mp, p[i]);
+            row_pass<false>(p, n, [&](float x, int) -> float { mp = fmaxf(mp, x); return x; });
             bool nn;
             mp = blk_max_f(mp, &nn, sm);
             const float thr = __fmul_rn(rd.min_p, mp);
-            for (int i = tid; i < n; i += kT)
-                if (p[i] < thr) p[i] = 0.0f;
+            row_pass<true>(p, n, [&](float x, int) -> float { return x < thr ? 0.0f : x; });
             __syncthreads();
         }
+        FPROF(a, slot, 5);
         // ApplyTopP (Sampler.cs:516-551)
         int big = 0;
         if (use_top_p) {
             int cnt = 0;
-            for (int i = tid; i < n; i += kT) cnt += p[i] > 0.0f ? 1 : 0;
+            row_pass<false>(p, n, [&](float x, int) -> float { cnt += x > 0.0f ? 1 : 0; return x; });
             int ns;
             // positions in index order (stable input for the device-wide sort)
             // each thread owns the strided indices tid, tid + kT, ...; a second pass assigns slots per tile
             ns = blk_sum_i(cnt, sm);
+            int nc = ns;           // candidates sorted inside the kernel
+            float c_above = -1.0f;  // ... are the probabilities strictly above this value
             if (ns > kSmall) {
-                big = 1;
-                // compact (prob bits, idx) in ascending index order into this row's segment
-                uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
-                int* vals = a.sort_vals_in + (size_t)slot * a.sort_stride;
-                int base = 0;
-                for (int i0 = 0; i0 < n; i0 += kT) {
-                    const int i = i0 + tid;
-                    const float v = i < n ? p[i] : 0.0f;
-                    int tot;
-                    const int pos = blk_excl_scan(v > 0.0f ? 1 : 0, &tot, sm);
-                    if (v > 0.0f) { keys[base + pos] = sr_f2u(v); vals[base + pos] = i; }
-                    base += tot;
-                }
-            } else if (ns > 0) {
+                // Many survivors (a masked row without min-p): the nucleus is still short.  Take the largest
+                // probabilities -- everything above the 65536-value bucket that holds the kSmall-th largest --
+                // and look for the cut-off among them; only if the nucleus does not close there is the whole row
+                // sorted.
+                c_above = sr_u2f(sr_f2u(kth_largest(p, n, kSmall, sm, 16)) | 0xffffu);
+                int cg = 0;
+                row_pass<false>(p, n, [&](float x, int) -> float { cg += x > c_above ? 1 : 0; return x; });
+                nc = blk_sum_i(cg, sm);  // < kSmall
+            }
+            bool closed = false;
+            if (nc > 0 && nc <= kSmall) {
                 if (tid == 0) sm.bc[4] = 0u;
                 __syncthreads();
-                for (int i = tid; i < n; i += kT) {
-                    const float v = p[i];
-                    if (v > 0.0f) {
+                row_pass<false>(p, n, [&](float v, int i) -> float {
+                    if (v > 0.0f && v > c_above) {
                         const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
                         sm.sortbuf[pos] = ((unsigned long long)sr_f2u(v) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
                     }
-                }
+                    return v;
+                });
                 __syncthreads();
                 int P = 2;
-                while (P < ns) P <<= 1;
-                for (int i = ns + tid; i < P; i += kT) sm.sortbuf[i] = 0ull;
+                while (P < nc) P <<= 1;
+                for (int i = nc + tid; i < P; i += kT) sm.sortbuf[i] = 0ull;
                 __syncthreads();
                 sort_small_desc(sm, P);
-                for (int i = tid; i < ns; i += kT) sm.sprob[i] = sr_u2f((uint32_t)(sm.sortbuf[i] >> 32));
+                for (int i = tid; i < nc; i += kT) sm.sprob[i] = sr_u2f((uint32_t)(sm.sortbuf[i] >> 32));
                 __syncthreads();
                 int found;
-                seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, ns, 0.0f, rd.top_p, &found, sm);
-                const int cutoff = found >= 0 ? found + 1 : ns;
-                for (int i = cutoff + tid; i < ns; i += kT)
-                    p[0xffffffffu - (uint32_t)(sm.sortbuf[i] & 0xffffffffull)] = 0.0f;
-                __syncthreads();
+                seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, 0.0f, rd.top_p, &found, sm);
+                closed = found >= 0 || nc == ns;
+                if (closed) {
+                    const int cutoff = found >= 0 ? found + 1 : nc;
+                    for (int i = cutoff + tid; i < nc; i += kT)
+                        p[0xffffffffu - (uint32_t)(sm.sortbuf[i] & 0xffffffffull)] = 0.0f;
+                    __syncthreads();
+                    if (nc < ns) {  // everything that was not a candidate comes later in the order
+                        row_pass<true>(p, n, [&](float x, int) -> float { return x > c_above ? x : 0.0f; });
+                        __syncthreads();
+                    }
+                }
+            }
+            if (ns > 0 && !closed) {
+                big = 1;
             }
             if (tid == 0) st->n_survivors = ns;
         }
+        FPROF(a, slot, 6);
         if (tid == 0) {
             st->big = big;
             st->flags = flags;
@@ -440,13 +519,16 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         for (int i = cutoff + tid; i < ns; i += kT) p[vals[i]] = 0.0f;
         __syncthreads();
     }
+    FPROF(a, slot, 7);
     // final Normalize (Sampler.cs:91-92)
     normalize_row(p, n, sm);
+    FPROF(a, slot, 8);
     int token = -1;
     if (a.mode != 1) {
         token = draw_from_row(p, n, a.uniforms[(size_t)row * a.uniforms_per_row], sm);
         if (tid == 0 && a.out_tokens) a.out_tokens[row] = token;
     }
+    FPROF(a, slot, 9);
     if (tid == 0 && a.out_flags) a.out_flags[row] = st->flags;
 }
 

@@ -27,6 +27,7 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     a.mask = b->d_mask.as<uint32_t>();
     a.mask_stride = b->mask_stride;
     a.mode = mode;
+    a.prof = ctx->prof;
     if (mode == 0) {
         const int64_t ws = (vocab + 3) & ~3;
         SR_HIP(ctx, ctx->work.reserve((size_t)n_rows * ws * sizeof(float), st));

@@ -100,6 +100,7 @@ struct SrFullArgs {
     int32_t uniforms_per_row;
     int32_t* out_tokens;       // [row], may be null in mode 1
     uint32_t* out_flags;       // [row], may be null
+    unsigned long long* prof;  // optional phase timestamps of slot 0 [32] (test hook), normally null
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st);

@@ -29,6 +29,8 @@
 struct SrSeqSmem {
     uint32_t wa0[SR_SEQ_WAVES];
     uint32_t wa1[SR_SEQ_WAVES];
+    uint32_t pa0[SR_SEQ_WAVES + 1];  // exclusive prefix of every wave, then the block total
+    uint32_t pa1[SR_SEQ_WAVES + 1];
     uint32_t misc[8];
     int first[SR_SEQ_WAVES];
 };
@@ -61,81 +63,41 @@ __device__ __forceinline__ void sr_split(float s, uint32_t* n, int* eb)
 }
 __device__ __forceinline__ float sr_join(uint32_t n, int eb) { return sr_u2f(n + ((uint32_t)(eb - 1) << 23)); }
 
-// The increment function of `cnt` terms x[0..cnt) in the binade with exponent field eb.
+// The increment function of the terms x[0..SR_SEQ_RUN) in the binade with exponent field eb: the hardware's
+// own round-to-nearest-even adds, run once from the binade's first even value and once from its first odd
+// value.  While such a chain stays inside the binade its bit pattern minus the start's is the number of ulps
+// gained, and that number is the same for every start of the same parity.  A chain that leaves the binade
+// (the run gains 2^23 ulps or more, or a term is too large for it) saturates: the caller replays that run.
 __device__ __forceinline__ SrInc sr_run_inc(const float (&x)[SR_SEQ_RUN], int eb)
 {
-    uint32_t A = 0u, B = 1u;  // running n for an even / odd start
-    bool hard = false;
+    const uint32_t base = eb > 1 ? ((uint32_t)eb << 23) : 0u;    // n = 2^23 (or 0 below the normal range): even
+    const uint32_t limit = eb > 1 ? base + (1u << 23) : (1u << 24);  // first bit pattern outside the binade
+    float sa = sr_u2f(base), sb = sr_u2f(base + 1u);
 #pragma unroll
     for (int j = 0; j < SR_SEQ_RUN; j++) {
-        const uint32_t b = sr_f2u(x[j]);
-        const uint32_t e = b >> 23;
-        const uint32_t M = (b & 0x7fffffu) | (e ? 0x800000u : 0u);
-        const int d = eb - (e ? (int)e : 1);
-        uint32_t fl = 0u, up = 0u, tie = 0u;
-        if (M != 0u) {
-            if (d < 0) {
-                hard = true;
-            } else if (d == 0) {
-                fl = M;  // same ulp: exact integer add (a normal s then leaves the binade, caught below)
-            } else if (d <= 24) {
-                fl = M >> d;
-                const uint32_t rem = M & ((1u << d) - 1u), half = 1u << (d - 1);
-                up = rem > half ? 1u : 0u;
-                tie = rem == half ? 1u : 0u;
-            }
-        }
-        A = A + fl + up + (tie & (A + fl) & 1u);
-        B = B + fl + up + (tie & (B + fl) & 1u);
+        sa = __fadd_rn(sa, x[j]);
+        sb = __fadd_rn(sb, x[j]);
     }
+    const uint32_t ba = sr_f2u(sa), bb = sr_f2u(sb);
     SrInc r;
-    r.a0 = hard ? SR_SEQ_SAT : (A > SR_SEQ_SAT ? SR_SEQ_SAT : A);
-    r.a1 = hard ? SR_SEQ_SAT : (B - 1u > SR_SEQ_SAT ? SR_SEQ_SAT : B - 1u);
+    r.a0 = (ba < limit) ? ba - base : SR_SEQ_SAT;
+    r.a1 = (bb < limit) ? bb - (base + 1u) : SR_SEQ_SAT;
     return r;
-}
-
-// Inclusive scan of the per-thread increment functions over the block.  Returns the EXCLUSIVE prefix
-// (the function of all lower threads); *total receives the function of the whole block.
-__device__ __forceinline__ SrInc sr_block_scan_inc(SrInc v, SrInc* total, SrSeqSmem& sm)
-{
-    const int lane = sr_lane(), wave = sr_wave_id();
-    SrInc incl = v;
-#pragma unroll
-    for (int o = 1; o < SR_WAVE; o <<= 1) {
-        SrInc lo;
-        lo.a0 = __shfl_up(incl.a0, o);
-        lo.a1 = __shfl_up(incl.a1, o);
-        if (lane >= o) incl = sr_compose(lo, incl);
-    }
-    __syncthreads();
-    if (lane == SR_WAVE - 1) { sm.wa0[wave] = incl.a0; sm.wa1[wave] = incl.a1; }
-    __syncthreads();
-    SrInc pre; pre.a0 = 0u; pre.a1 = 0u;
-    SrInc all; all.a0 = 0u; all.a1 = 0u;
-#pragma unroll
-    for (int w = 0; w < SR_SEQ_WAVES; w++) {
-        SrInc t; t.a0 = sm.wa0[w]; t.a1 = sm.wa1[w];
-        if (w < wave) pre = sr_compose(pre, t);
-        all = sr_compose(all, t);
-    }
-    *total = all;
-    // exclusive within the wave
-    SrInc ex;
-    ex.a0 = __shfl_up(incl.a0, 1);
-    ex.a1 = __shfl_up(incl.a1, 1);
-    if (lane == 0) { ex.a0 = 0u; ex.a1 = 0u; }
-    return sr_compose(pre, ex);
 }
 
 // One tile: adds this thread's SR_SEQ_RUN terms (thread order = term order) to the running sum *s
 // (uniform across the block on entry and exit).  When kSearch, also looks for the first term index at
 // which the running sum reaches `target` (fl(s) >= target); on success returns its tile-local index
 // (thread * SR_SEQ_RUN + j) in *found (uniform), else leaves -1.  Terms past the end must be 0.
+//
+// Per round: every wave scans its threads' increment functions; the first wave scans the wave totals, which
+// also shows the first wave in which the sum leaves the binade (or reaches the target); that wave alone finds
+// the thread and replays its run with real float adds; everything after it is rescanned in the new binade.
 template <bool kSearch>
 __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float* s, float target, int* found,
                                             SrSeqSmem& sm)
 {
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
     int start = 0;  // threads below `start` are settled
     float s_in = *s;
     *found = -1;
@@ -146,48 +108,180 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
         SrInc mine;
         mine.a0 = 0u; mine.a1 = 0u;
         if (tid >= start) mine = sr_run_inc(x, eb);
-        SrInc total;
-        const SrInc ex = sr_block_scan_inc(mine, &total, sm);
-        // exact integer state before / after this thread's run, valid while below 2^24
-        const uint32_t before = sr_sat_add(n_in, (n_in & 1u) ? ex.a1 : ex.a0);
-        const SrInc thr = sr_compose(ex, mine);
-        const uint32_t after = sr_sat_add(n_in, (n_in & 1u) ? thr.a1 : thr.a0);
-        const bool leaves = tid >= start && after >= (1u << 24);
-        bool hit = false;
-        if (kSearch) hit = tid >= start && !leaves && sr_join(after, eb) >= target;
-        // first thread that leaves the binade, first thread that reaches the target
-        int cand = (leaves || hit) ? tid : 0x7fffffff;
-        cand = sr_wave_min_i32(cand);
-        __syncthreads();
-        if (sr_lane() == 0) sm.first[sr_wave_id()] = cand;
-        __syncthreads();
-        int fst = 0x7fffffff;
+        SrInc incl = mine;
 #pragma unroll
-        for (int w = 0; w < SR_SEQ_WAVES; w++) fst = min(fst, sm.first[w]);
-        if (fst == 0x7fffffff) {
+        for (int o = 1; o < SR_WAVE; o <<= 1) {
+            SrInc lo;
+            lo.a0 = __shfl_up(incl.a0, o);
+            lo.a1 = __shfl_up(incl.a1, o);
+            if (lane >= o) incl = sr_compose(lo, incl);
+        }
+        __syncthreads();  // the previous round's readers are done with the arrays below
+        if (lane == SR_WAVE - 1) { sm.wa0[wave] = incl.a0; sm.wa1[wave] = incl.a1; }
+        __syncthreads();
+        if (wave == 0) {
+            SrInc ti; ti.a0 = 0u; ti.a1 = 0u;
+            if (lane < SR_SEQ_WAVES) { ti.a0 = sm.wa0[lane]; ti.a1 = sm.wa1[lane]; }
+#pragma unroll
+            for (int o = 1; o < SR_SEQ_WAVES; o <<= 1) {
+                SrInc lo;
+                lo.a0 = __shfl_up(ti.a0, o);
+                lo.a1 = __shfl_up(ti.a1, o);
+                if (lane >= o) ti = sr_compose(lo, ti);
+            }
+            // state at the end of every wave; the running value never decreases, so the first wave whose end
+            // state has left the binade (or reached the target) holds the first such thread
+            const uint32_t end_n = sr_sat_add(n_in, (n_in & 1u) ? ti.a1 : ti.a0);
+            bool event = end_n >= (1u << 24);
+            if (kSearch) event = event || sr_join(end_n, eb) >= target;
+            const unsigned long long ev = __ballot(event && lane < SR_SEQ_WAVES);
+            SrInc te;
+            te.a0 = __shfl_up(ti.a0, 1);
+            te.a1 = __shfl_up(ti.a1, 1);
+            if (lane == 0) { te.a0 = 0u; te.a1 = 0u; }
+            if (lane < SR_SEQ_WAVES) { sm.pa0[lane] = te.a0; sm.pa1[lane] = te.a1; }
+            if (lane == SR_SEQ_WAVES - 1) { sm.pa0[SR_SEQ_WAVES] = ti.a0; sm.pa1[SR_SEQ_WAVES] = ti.a1; }
+            if (lane == 0) sm.first[0] = ev ? (int)__ffsll((long long)ev) - 1 : -1;
+        }
+        __syncthreads();
+        const int ev_wave = sm.first[0];
+        if (ev_wave < 0) {
             // the whole remainder stays in the binade: settle with the block total
-            const uint32_t n_out = n_in + ((n_in & 1u) ? total.a1 : total.a0);
-            *s = sr_join(n_out, eb);
+            const uint32_t tot = (n_in & 1u) ? sm.pa1[SR_SEQ_WAVES] : sm.pa0[SR_SEQ_WAVES];
+            *s = sr_join(n_in + tot, eb);
             return;
         }
-        // thread fst replays its run with real float adds from its exact input
-        if (tid == fst) {
-            float acc = sr_join(before, eb);
-            int where = -1;
+        if (wave == ev_wave) {
+            SrInc pre; pre.a0 = sm.pa0[wave]; pre.a1 = sm.pa1[wave];
+            SrInc ex;
+            ex.a0 = __shfl_up(incl.a0, 1);
+            ex.a1 = __shfl_up(incl.a1, 1);
+            if (lane == 0) { ex.a0 = 0u; ex.a1 = 0u; }
+            ex = sr_compose(pre, ex);
+            // exact integer state before / after this thread's run, valid while below 2^24
+            const uint32_t before = sr_sat_add(n_in, (n_in & 1u) ? ex.a1 : ex.a0);
+            const SrInc thr = sr_compose(ex, mine);
+            const uint32_t after = sr_sat_add(n_in, (n_in & 1u) ? thr.a1 : thr.a0);
+            bool event = after >= (1u << 24);
+            if (kSearch) event = event || sr_join(after, eb) >= target;
+            const unsigned long long ev = __ballot(event && tid >= start);
+            const int fl = ev ? (int)__ffsll((long long)ev) - 1 : SR_WAVE - 1;  // ev != 0 by construction
+            if (lane == fl) {
+                // replay this run with real float adds from its exact input
+                float acc = sr_join(before, eb);
+                int where = -1;
 #pragma unroll
-            for (int j = 0; j < SR_SEQ_RUN; j++) {
-                acc = __fadd_rn(acc, x[j]);
-                if (kSearch && where < 0 && acc >= target) where = fst * SR_SEQ_RUN + j;
+                for (int j = 0; j < SR_SEQ_RUN; j++) {
+                    acc = __fadd_rn(acc, x[j]);
+                    if (kSearch && where < 0 && acc >= target) where = tid * SR_SEQ_RUN + j;
+                }
+                sm.misc[0] = sr_f2u(acc);
+                sm.misc[1] = (uint32_t)where;
+                sm.misc[2] = (uint32_t)tid;
             }
-            sm.misc[0] = sr_f2u(acc);
-            sm.misc[1] = (uint32_t)where;
         }
         __syncthreads();
         s_in = sr_u2f(sm.misc[0]);
         const int where = (int)sm.misc[1];
-        __syncthreads();
+        const int fst = (int)sm.misc[2];
         if (kSearch && where >= 0) { *found = where; *s = s_in; return; }
         start = fst + 1;
         if (start >= SR_SEQ_THREADS) { *s = s_in; return; }
     }
+}
+
+// ---- eight independent chains at once -----------------------------------------------------------------
+// Thread t serves chain (t & 7) with the SR_SEQ_RUN terms number (t >> 3) * SR_SEQ_RUN ... of that chain's
+// tile, so one tile covers SR_SEQ_THREADS / 8 * SR_SEQ_RUN terms of every chain.  *s is the running sum
+// of the caller's chain (uniform across the threads of a chain).  Terms past the end must be 0.  All
+// threads of the block must call.
+#define SR_SEQ_CHAINS 8
+#define SR_SEQ_CHAIN_THREADS (SR_SEQ_THREADS / SR_SEQ_CHAINS)
+#define SR_SEQ_CHAIN_TILE (SR_SEQ_CHAIN_THREADS * SR_SEQ_RUN)
+
+struct SrSeq8Smem {
+    uint32_t wa0[SR_SEQ_WAVES][SR_SEQ_CHAINS];
+    uint32_t wa1[SR_SEQ_WAVES][SR_SEQ_CHAINS];
+    int first[SR_SEQ_WAVES][SR_SEQ_CHAINS];
+    uint32_t acc[SR_SEQ_CHAINS];
+    uint32_t busy;
+};
+
+__device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN], float* s, SrSeq8Smem& sm)
+{
+    const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
+    const int g = tid & (SR_SEQ_CHAINS - 1), lt = tid >> 3;  // chain, position inside the chain
+    int start = 0;     // chain threads below `start` are settled
+    bool done = false; // this chain has finished the tile
+    float s_in = *s;
+    for (;;) {
+        uint32_t n_in;
+        int eb;
+        sr_split(s_in, &n_in, &eb);
+        SrInc mine;
+        mine.a0 = 0u; mine.a1 = 0u;
+        if (!done && lt >= start) mine = sr_run_inc(x, eb);
+        // inclusive scan over the lanes of the same chain (lanes 8 apart), then over the waves
+        SrInc incl = mine;
+#pragma unroll
+        for (int o = SR_SEQ_CHAINS; o < SR_WAVE; o <<= 1) {
+            SrInc lo;
+            lo.a0 = __shfl_up(incl.a0, o);
+            lo.a1 = __shfl_up(incl.a1, o);
+            if (lane >= o) incl = sr_compose(lo, incl);
+        }
+        __syncthreads();
+        if (lane >= SR_WAVE - SR_SEQ_CHAINS) { sm.wa0[wave][g] = incl.a0; sm.wa1[wave][g] = incl.a1; }
+        if (tid == 0) sm.busy = 0u;
+        __syncthreads();
+        SrInc pre; pre.a0 = 0u; pre.a1 = 0u;
+        SrInc total; total.a0 = 0u; total.a1 = 0u;
+#pragma unroll
+        for (int w = 0; w < SR_SEQ_WAVES; w++) {
+            SrInc t; t.a0 = sm.wa0[w][g]; t.a1 = sm.wa1[w][g];
+            if (w < wave) pre = sr_compose(pre, t);
+            total = sr_compose(total, t);
+        }
+        SrInc ex;
+        ex.a0 = __shfl_up(incl.a0, SR_SEQ_CHAINS);
+        ex.a1 = __shfl_up(incl.a1, SR_SEQ_CHAINS);
+        if (lane < SR_SEQ_CHAINS) { ex.a0 = 0u; ex.a1 = 0u; }
+        ex = sr_compose(pre, ex);
+        const uint32_t before = sr_sat_add(n_in, (n_in & 1u) ? ex.a1 : ex.a0);
+        const SrInc thr = sr_compose(ex, mine);
+        const uint32_t after = sr_sat_add(n_in, (n_in & 1u) ? thr.a1 : thr.a0);
+        const bool leaves = !done && lt >= start && after >= (1u << 24);
+        // first thread of the chain that leaves the binade
+        int cand = leaves ? lt : 0x7fffffff;
+#pragma unroll
+        for (int o = SR_SEQ_CHAINS; o < SR_WAVE; o <<= 1) cand = min(cand, __shfl_xor(cand, o));
+        if (lane < SR_SEQ_CHAINS) sm.first[wave][g] = cand;
+        __syncthreads();
+        int fst = 0x7fffffff;
+#pragma unroll
+        for (int w = 0; w < SR_SEQ_WAVES; w++) fst = min(fst, sm.first[w][g]);
+        if (!done) {
+            if (fst == 0x7fffffff) {
+                // the chain's remainder stays in the binade: settle with the chain total
+                s_in = sr_join(n_in + ((n_in & 1u) ? total.a1 : total.a0), eb);
+                done = true;
+            } else if (lt == fst) {
+                // replay this run with real float adds from its exact input
+                float acc = sr_join(before, eb);
+#pragma unroll
+                for (int j = 0; j < SR_SEQ_RUN; j++) acc = __fadd_rn(acc, x[j]);
+                sm.acc[g] = sr_f2u(acc);
+                sm.busy = 1u;
+            }
+        }
+        __syncthreads();
+        const bool again = sm.busy != 0u;
+        if (!done) {
+            s_in = sr_u2f(sm.acc[g]);
+            start = fst + 1;
+            if (start >= SR_SEQ_CHAIN_THREADS) done = true;
+        }
+        if (!again) break;
+    }
+    *s = s_in;
 }
