@@ -1360,6 +1360,29 @@ __global__ __launch_bounds__(256) void k_build_scan_mask(const SrScanDesc* descs
         unsigned long long bits = 0ull;
         if (!src && e_first >= 0 && e_first + 63ll * epv < vocab) {
             bits = ~0ull;
+        } else if (src && mis == 0) {
+            // every epv-th bit of the 64 * epv allow-bits of the block, starting at bit q, squeezed together
+            const int words_in = 2 * epv, first = b * words_in, per = 32 / epv;  // 8 or 4 bits from each input word
+            for (int k = 0; k < words_in; k++) {
+                const long long e0w = (long long)(first + k) * 32;
+                uint32_t x = 0u;
+                if (e0w < vocab) {
+                    x = src[first + k];
+                    if (e0w + 32 > vocab) x &= (1u << (vocab - e0w)) - 1u;
+                }
+                x >>= q;
+                if (epv == 4) {
+                    x &= 0x11111111u;
+                    x = (x | (x >> 3)) & 0x03030303u;
+                    x = (x | (x >> 6)) & 0x000f000fu;
+                    x = (x | (x >> 12)) & 0xffu;
+                } else {
+                    x &= 0x01010101u;
+                    x = (x | (x >> 7)) & 0x00030003u;
+                    x = (x | (x >> 14)) & 0xfu;
+                }
+                bits |= (unsigned long long)x << (k * per);
+            }
         } else {
             for (int l = 0; l < 64; l++) {
                 const long long e = e_first + (long long)l * epv;
