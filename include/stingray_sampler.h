@@ -203,6 +203,22 @@ SR_API int sr_sample_with_distribution_launch(sr_ctx* ctx, const sr_batch* batch
                                               float* out_probs_dev, int64_t probs_stride_elems,
                                               int32_t probs_len, int32_t* out_tokens_dev);
 
+/* Span-shaped forms of the two calls above: HOST fp32 logits in, HOST probabilities (and tokens) out, side inputs
+ * as for sr_sample_batch (no allow-mask: the managed methods take none).  uniforms: HOST double[rows], one per row
+ * (may be NULL for sr_build_distribution and when every row is greedy). */
+SR_API int sr_build_distribution(sr_ctx* ctx, const float* logits, int32_t rows, int32_t vocab, int64_t row_stride_elems,
+                                 const sr_row_params* params,
+                                 const int32_t* hist_ids, const int32_t* hist_offsets,
+                                 const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                                 float* out_probs, int64_t probs_stride_elems, int32_t probs_len);
+SR_API int sr_sample_with_distribution(sr_ctx* ctx, const float* logits, int32_t rows, int32_t vocab,
+                                       int64_t row_stride_elems, const sr_row_params* params,
+                                       const int32_t* hist_ids, const int32_t* hist_offsets,
+                                       const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                                       const double* uniforms,
+                                       float* out_probs, int64_t probs_stride_elems, int32_t probs_len,
+                                       int32_t* out_tokens);
+
 /*
  * int Sampler.SampleFromProbs(ReadOnlySpan<float> probs, Random rng) per row (Sampler.cs:195-199):
  * first index whose running fp32 sum reaches (float)u, last index as the rounding fallback.
@@ -212,6 +228,10 @@ SR_API int sr_sample_from_probs_launch(sr_ctx* ctx, const float* probs_dev, int3
                                        int64_t probs_stride_elems, const double* uniforms,
                                        int32_t* out_tokens_dev);
 
+/* Span-shaped form: HOST probabilities in, HOST tokens out. */
+SR_API int sr_sample_from_probs(sr_ctx* ctx, const float* probs, int32_t rows, int32_t vocab,
+                                int64_t probs_stride_elems, const double* uniforms, int32_t* out_tokens);
+
 /*
  * int Sampler.ResampleResidual(p, q, rng) per row (Sampler.cs:587-618).  p_len != q_len ->
  * SR_ERR_INVALID_ARGUMENT; uniforms NULL -> SR_ERR_NULL_ARGUMENT.
@@ -219,6 +239,11 @@ SR_API int sr_sample_from_probs_launch(sr_ctx* ctx, const float* probs_dev, int3
 SR_API int sr_resample_residual_launch(sr_ctx* ctx, const float* p_dev, int32_t p_len, int64_t p_stride_elems,
                                        const float* q_dev, int32_t q_len, int64_t q_stride_elems,
                                        int32_t rows, const double* uniforms, int32_t* out_tokens_dev);
+
+/* Span-shaped form: HOST distributions in, HOST tokens out. */
+SR_API int sr_resample_residual(sr_ctx* ctx, const float* p, int32_t p_len, int64_t p_stride_elems,
+                                const float* q, int32_t q_len, int64_t q_stride_elems,
+                                int32_t rows, const double* uniforms, int32_t* out_tokens);
 
 /*
  * The accept / reject loop of SpeculativeDecoder.StepSampled

@@ -47,6 +47,7 @@ EXPORTED_SYMBOLS = [
     "sr_sample_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows",
     "sr_build_distribution_launch", "sr_sample_with_distribution_launch", "sr_sample_from_probs_launch",
     "sr_resample_residual_launch", "sr_spec_verify_launch", "sr_mtp_verify_launch", "sr_pack_allow_mask",
+    "sr_build_distribution", "sr_sample_with_distribution", "sr_sample_from_probs", "sr_resample_residual",
 ]
 
 

@@ -57,5 +57,23 @@ def build(force: bool = False) -> str:
     return LIB
 
 
+CPP_TEST_SRC = os.path.join(HERE, "..", "..", "tests", "cpp", "host_mirror_test.cpp")
+CPP_TEST_BIN = os.path.join(HERE, "..", "..", "tests", "cpp", "host_mirror_test")
+
+
+def build_cpp_test(oracle_lib: str) -> str:
+    """Compiles the C++ host-mirror test (g++; links the C ABI library and, as its checker, the oracle)."""
+    root = os.path.normpath(os.path.join(HERE, "..", ".."))
+    cmd = ["g++", "-std=c++17", "-O1", "-o", os.path.normpath(CPP_TEST_BIN), os.path.normpath(CPP_TEST_SRC),
+           "-I" + os.path.join(root, "include"), "-I" + os.path.join(root, "oracle"),
+           "-L" + LIB_DIR, "-lstingray_sampler", "-L" + os.path.dirname(os.path.abspath(oracle_lib)), "-lstingray_oracle",
+           "-Wl,-rpath,$ORIGIN/../../opentail/stingray_amd/lib", "-Wl,-rpath,$ORIGIN/../../oracle/_build",
+           "-Wl,-rpath,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"g++ failed for the host-mirror test:\n{r.stdout}\n{r.stderr}")
+    return os.path.normpath(CPP_TEST_BIN)
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv))

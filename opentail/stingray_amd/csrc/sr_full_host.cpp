@@ -213,6 +213,125 @@ int sr_resample_residual_launch(sr_ctx* ctx, const float* p_dev, int32_t p_len, 
     return SR_OK;
 }
 
+
+// ---- span-shaped forms: host buffers in, host results out ------------------------------------------------
+
+static int stage_up(sr_ctx* ctx, DeviceBuf& buf, const void* src, size_t bytes)
+{
+    SR_HIP(ctx, buf.reserve(bytes, ctx->stream));
+    SR_HIP(ctx, hipMemcpyAsync(buf.p, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    return SR_OK;
+}
+
+static int distribution_host(sr_ctx* ctx, const char* what, bool sample, const float* logits, int32_t rows, int32_t vocab,
+                             int64_t row_stride, const sr_row_params* params, const int32_t* hist_ids,
+                             const int32_t* hist_offsets, const int32_t* bias_ids, const float* bias_vals,
+                             const int32_t* bias_offsets, const double* uniforms, float* out_probs, int64_t probs_stride,
+                             int32_t probs_len, int32_t* out_tokens)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0) return SR_OK;
+    if (probs_len != vocab)  // Sampler.cs:121-123
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "probs length (" + std::to_string(probs_len) + ") must equal logits length (" +
+                                                         std::to_string(vocab) + ").");
+    if (!logits || !params || !out_probs || (sample && !out_tokens))
+        return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, std::string(what) + ": null argument");
+    if (rows < 0 || vocab <= 0 || row_stride < vocab || probs_stride < vocab)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(what) + ": bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    if (!ctx->tmp_batch) {
+        int rc = sr_batch_create(ctx, &ctx->tmp_batch);
+        if (rc != SR_OK) return rc;
+    }
+    int rc = sr_batch_upload(ctx->tmp_batch, rows, vocab, params, hist_ids, hist_offsets, bias_ids, bias_vals, bias_offsets,
+                             nullptr, 0, nullptr, uniforms, uniforms ? 1 : 0);
+    if (rc != SR_OK) return rc;
+    const size_t in_bytes = ((size_t)(rows - 1) * (size_t)row_stride + (size_t)vocab) * sizeof(float);
+    rc = stage_up(ctx, ctx->host_logits, logits, in_bytes);
+    if (rc != SR_OK) return rc;
+    const int64_t ps = (vocab + 3) & ~3;
+    SR_HIP(ctx, ctx->stage_probs.reserve((size_t)rows * (size_t)ps * sizeof(float), ctx->stream));
+    SR_HIP(ctx, ctx->out_tokens.reserve((size_t)rows * sizeof(int32_t), ctx->stream));
+    if (sample)
+        rc = sr_sample_with_distribution_launch(ctx, ctx->tmp_batch, ctx->host_logits.p, SR_DTYPE_F32, row_stride,
+                                                ctx->stage_probs.as<float>(), ps, probs_len, ctx->out_tokens.as<int32_t>());
+    else
+        rc = sr_build_distribution_launch(ctx, ctx->tmp_batch, ctx->host_logits.p, SR_DTYPE_F32, row_stride,
+                                          ctx->stage_probs.as<float>(), ps, probs_len);
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, hipMemcpy2DAsync(out_probs, (size_t)probs_stride * sizeof(float), ctx->stage_probs.p, (size_t)ps * sizeof(float),
+                                 (size_t)vocab * sizeof(float), (size_t)rows, hipMemcpyDeviceToHost, ctx->stream));
+    if (sample)
+        SR_HIP(ctx, hipMemcpyAsync(out_tokens, ctx->out_tokens.p, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return SR_OK;
+}
+
+int sr_build_distribution(sr_ctx* ctx, const float* logits, int32_t rows, int32_t vocab, int64_t row_stride,
+                          const sr_row_params* params, const int32_t* hist_ids, const int32_t* hist_offsets,
+                          const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets, float* out_probs,
+                          int64_t probs_stride, int32_t probs_len)
+{
+    return distribution_host(ctx, "sr_build_distribution", false, logits, rows, vocab, row_stride, params, hist_ids, hist_offsets,
+                             bias_ids, bias_vals, bias_offsets, nullptr, out_probs, probs_stride, probs_len, nullptr);
+}
+
+int sr_sample_with_distribution(sr_ctx* ctx, const float* logits, int32_t rows, int32_t vocab, int64_t row_stride,
+                                const sr_row_params* params, const int32_t* hist_ids, const int32_t* hist_offsets,
+                                const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                                const double* uniforms, float* out_probs, int64_t probs_stride, int32_t probs_len,
+                                int32_t* out_tokens)
+{
+    return distribution_host(ctx, "sr_sample_with_distribution", true, logits, rows, vocab, row_stride, params, hist_ids,
+                             hist_offsets, bias_ids, bias_vals, bias_offsets, uniforms, out_probs, probs_stride, probs_len,
+                             out_tokens);
+}
+
+int sr_sample_from_probs(sr_ctx* ctx, const float* probs, int32_t rows, int32_t vocab, int64_t probs_stride,
+                         const double* uniforms, int32_t* out_tokens)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (!uniforms) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "rng");  // ArgumentNullException(rng), Sampler.cs:197
+    if (rows == 0) return SR_OK;
+    if (!probs || !out_tokens) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_from_probs: null argument");
+    if (rows < 0 || vocab <= 0 || probs_stride < vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_from_probs: bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    int rc = stage_up(ctx, ctx->host_logits, probs, ((size_t)(rows - 1) * (size_t)probs_stride + (size_t)vocab) * sizeof(float));
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, ctx->out_tokens.reserve((size_t)rows * sizeof(int32_t), ctx->stream));
+    rc = sr_sample_from_probs_launch(ctx, ctx->host_logits.as<float>(), rows, vocab, probs_stride, uniforms, ctx->out_tokens.as<int32_t>());
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, hipMemcpyAsync(out_tokens, ctx->out_tokens.p, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return SR_OK;
+}
+
+int sr_resample_residual(sr_ctx* ctx, const float* p, int32_t p_len, int64_t p_stride, const float* q, int32_t q_len,
+                         int64_t q_stride, int32_t rows, const double* uniforms, int32_t* out_tokens)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (!uniforms) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "rng");  // Sampler.cs:589
+    if (p_len != q_len)                                                // Sampler.cs:590-592
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT,
+                       "p and q must have equal length (" + std::to_string(p_len) + " vs " + std::to_string(q_len) + ").");
+    if (rows == 0) return SR_OK;
+    if (!p || !q || !out_tokens) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_resample_residual: null argument");
+    if (rows < 0 || p_len <= 0 || p_stride < p_len || q_stride < q_len)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_resample_residual: bad shape");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    int rc = stage_up(ctx, ctx->host_logits, p, ((size_t)(rows - 1) * (size_t)p_stride + (size_t)p_len) * sizeof(float));
+    if (rc != SR_OK) return rc;
+    rc = stage_up(ctx, ctx->stage_probs, q, ((size_t)(rows - 1) * (size_t)q_stride + (size_t)q_len) * sizeof(float));
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, ctx->out_tokens.reserve((size_t)rows * sizeof(int32_t), ctx->stream));
+    rc = sr_resample_residual_launch(ctx, ctx->host_logits.as<float>(), p_len, p_stride, ctx->stage_probs.as<float>(), q_len, q_stride,
+                                     rows, uniforms, ctx->out_tokens.as<int32_t>());
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, hipMemcpyAsync(out_tokens, ctx->out_tokens.p, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return SR_OK;
+}
+
 int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_logits_dev, const float* draft_probs_dev,
                           const int32_t* draft_tokens_dev, int32_t n_draft, int32_t* out_accepted_dev, int32_t* out_tokens_dev)
 {

@@ -52,6 +52,7 @@ struct sr_ctx {
     DeviceBuf work;          // fp32 rows of the full-vocabulary path
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits
+    DeviceBuf stage_probs;   // staging for host-resident distributions
     DeviceBuf out_tokens, out_flags, out_val, uniforms_tmp;
     DeviceBuf seg, sort_k0, sort_k1, sort_v0, sort_v1, sort_tmp;  // device-wide sort of large nuclei
     DeviceBuf ident;         // identity row list
