@@ -18,20 +18,15 @@ inline bool has_history_penalty(const sr_row_params& p)
 
 // Chunking of a row for the selection kernel: a chunk is a whole number of 64-vector blocks of the row's
 // window of 16-byte vectors and must fit the per-workgroup register window.
-void topk_geometry(int vocab, int dtype, int n_rows, int max_sel, int cu_count, int* chunks, int* chunk_vecs)
+void topk_geometry(int vocab, int dtype, int n_rows, int cu_count, int* chunks, int* chunk_vecs)
 {
     const int epv = dtype == SR_DTYPE_BF16 ? 8 : 4;
     const int window = (dtype == SR_DTYPE_BF16 ? SR_TK_VEC_BF16 : SR_TK_VEC) * SR_TK_THREADS;  // vectors a workgroup holds
     const int nvt = (vocab + 2 * epv - 2) / epv;                   // vectors of a row that starts mid-vector
     int s_min = (nvt + window - 1) / window;
     int s_par = (2 * cu_count + n_rows - 1) / std::max(n_rows, 1);  // aim for two workgroups per CU
-    int s_cap = std::min(SR_TK_MAX_CHUNKS, std::max(1, vocab / 8192));  // short chunks only multiply the candidates
-    // all chunks of a row share the SR_TK_ROW_CAP entries of its candidate list: a wave of the per-wave scan
-    // (sel <= 64) wants SR_TK_WAVE_LIM of them, a chunk of the workgroup-wide scan 2 * sel + 128
-    if (max_sel <= 64)
-        s_cap = std::min(s_cap, SR_TK_ROW_CAP / (SR_TK_WAVE_LIM * (SR_TK_THREADS / 64)));
-    else
-        s_cap = std::min(s_cap, std::max(1, SR_TK_ROW_CAP / (2 * std::min(max_sel, SR_TK_SEL_MAX) + 128)));
+    // the row tail keeps the per-group results of up to 4 chunks in registers; more chunks only when the row needs them
+    int s_cap = std::min(4, std::max(1, vocab / 8192));
     int s = std::max(s_min, std::min(s_par, s_cap));
     int cv = (nvt + s - 1) / s;
     cv = (cv + 63) & ~63;
@@ -71,6 +66,19 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     b->scan_base_mod = base_mod;
     b->scan_stride_mod = stride_mod;
     if (b->h_scan.empty()) return SR_OK;
+    {
+        std::vector<int32_t> info;
+        info.reserve(b->h_sel_list.size() * 4);
+        for (int32_t r : b->h_sel_list) {
+            info.push_back(r);
+            info.push_back(b->h_rows[(size_t)r].scan_row);
+            info.push_back(b->h_rows[(size_t)r].sel);
+            info.push_back(0);
+        }
+        SR_HIP(ctx, b->d_slot_info.reserve(info.size() * sizeof(int32_t), st));
+        SR_HIP(ctx, hipMemcpyAsync(b->d_slot_info.p, info.data(), info.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+        SR_HIP(ctx, hipStreamSynchronize(st));
+    }
     const int64_t blocks = ((int64_t)b->vocab + 2 * epv - 2) / epv / 64 + 1;
     b->scan_stride = blocks * epv;
     if (rows_changed)
@@ -121,7 +129,7 @@ void sr_destroy(sr_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
-    DeviceBuf* bufs[] = {&ctx->cand, &ctx->cand_cnt, &ctx->sched, &ctx->row_done, &ctx->argmax_best,
+    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->sched, &ctx->row_done, &ctx->argmax_best,
                          &ctx->work, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->spec_rows, &ctx->spec_probs};
@@ -168,7 +176,7 @@ void sr_batch_destroy(sr_batch* b)
     if (!b) return;
     if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
     DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_scan_desc,
-                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms};
+                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_slot_info};
     for (DeviceBuf* d : bufs) d->release();
     delete b;
 }
@@ -387,7 +395,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         int rc = prepare_scan(const_cast<sr_batch*>(b), epv, (unsigned long long)(uintptr_t)logits_dev,
                               (long long)row_stride_elems * (dtype == SR_DTYPE_BF16 ? 2 : 4));
         if (rc != SR_OK) return rc;
-        topk_geometry(b->vocab, dtype, n_sel, b->max_sel, ctx->cu_count, &a.chunks, &a.chunk_vecs);
+        topk_geometry(b->vocab, dtype, n_sel, ctx->cu_count, &a.chunks, &a.chunk_vecs);
         if (a.chunks > SR_TK_MAX_CHUNKS)
             return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary too large for the selection kernel");
         // Dispatch order.  Workgroups are dispatched in grid order, two resident per CU; a round is that many
@@ -425,9 +433,12 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         }
         a.sched = ctx->sched.as<uint32_t>();
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));
-        SR_HIP(ctx, ctx->cand_cnt.reserve((size_t)std::max(n_sel, 1024) * sizeof(int32_t), st, true));
+        SR_HIP(ctx, ctx->gmax.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
+        SR_HIP(ctx, ctx->gmax2.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
+        SR_HIP(ctx, ctx->gpos.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * sizeof(uint32_t), st));
+        SR_HIP(ctx, ctx->gbound.reserve((size_t)n_sel * a.chunks * (SR_TK_THREADS / 64) * sizeof(uint32_t), st));
         SR_HIP(ctx, ctx->row_done.reserve((size_t)std::max(n_sel, 1024) * sizeof(uint32_t), st, true));
-        a.row_list = b->d_sel_list.as<int32_t>();
+        a.slot_info = b->d_slot_info.as<int4>();
         a.rows = b->d_rows.as<SrRow>();
         a.edits = b->d_edits.as<SrEdit>();
         a.mask = b->d_mask.as<uint32_t>();
@@ -435,7 +446,10 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.scan_mask = b->d_scan_mask.as<unsigned long long>();
         a.scan_stride = b->scan_stride;
         a.cand = ctx->cand.as<unsigned long long>();
-        a.cand_cnt = ctx->cand_cnt.as<int32_t>();
+        a.gmax = ctx->gmax.as<float4>();
+        a.gmax2 = ctx->gmax2.as<float4>();
+        a.gpos = ctx->gpos.as<uint32_t>();
+        a.gbound = ctx->gbound.as<uint32_t>();
         a.row_done = ctx->row_done.as<uint32_t>();
         a.uniforms = b->d_uniforms.as<double>();
         a.uniforms_per_row = b->upr;

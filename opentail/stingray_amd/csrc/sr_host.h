@@ -48,7 +48,7 @@ struct sr_ctx {
     std::string err;
     int cu_count = 256;
     // scratch, lazily grown and reused across calls
-    DeviceBuf cand, cand_cnt, row_done, argmax_best;
+    DeviceBuf cand, gmax, gmax2, gpos, gbound, row_done, argmax_best;
     DeviceBuf work;          // fp32 rows of the full-vocabulary path
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits
@@ -74,7 +74,7 @@ struct sr_batch {
     std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path
     std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel
     std::vector<uint32_t> h_scan_need; // per batch row: SR_SCAN_* bits the row's scan mask must carry
-    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms;
+    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms, d_slot_info;
     int64_t mask_stride = 0, scan_stride = 0;
     // what the scan masks were built for: elements per 16-byte vector, the logits base address modulo 16 and
     // the row stride in bytes modulo 16 (rows share a mask row only when all start at the same offset)

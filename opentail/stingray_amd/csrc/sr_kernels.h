@@ -25,15 +25,18 @@ struct SrTopkArgs {
     int32_t n_rows;          // rows in this launch: grid = n_rows * chunks chunk workgroups + n_rows tail workgroups
     int32_t chunk_vecs;      // 16-byte vectors per chunk, a multiple of 64
     const uint32_t* sched;   // per workgroup in dispatch order: bit 31 = row tail, bits 24..30 = chunk, bits 0..23 = slot
-    const int32_t* row_list; // rows handled by this launch (device)
+    const int4* slot_info;   // per row of this launch, in launch order: (batch row, scan-mask row, sel, 0)
     const SrRow* rows;
     const SrEdit* edits;
     const uint32_t* mask;
     int64_t mask_stride;     // words
     const unsigned long long* scan_mask; // keep-bits of every row in the kernel's access order (SrRow.scan_row)
     int64_t scan_stride;     // 64-bit words per scan row
-    unsigned long long* cand; // [n_rows][SR_TK_ROW_CAP] (value bits << 32 | index), appended by the chunks
-    int32_t* cand_cnt;       // [n_rows] append cursor, zero on entry, left zero on exit
+    float4* gmax;            // [n_rows][chunks][SR_TK_THREADS]: the four group maxima of every thread of every chunk
+    float4* gmax2;           // ... the second largest element of each of those groups
+    uint32_t* gpos;          // ... the position of the largest inside its group, 8 bits per group
+    uint32_t* gbound;        // [n_rows][chunks][waves]: every chunk wave's share of the row's bound (an ordered key)
+    unsigned long long* cand; // [n_rows][SR_TK_ROW_CAP] (value bits << 32 | index), built by the row's tail
     uint32_t* row_done;      // [n_rows], zero on entry, left zero on exit
     const double* uniforms;
     int32_t uniforms_per_row;

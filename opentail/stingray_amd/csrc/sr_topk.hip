@@ -34,7 +34,7 @@ constexpr int kRowCap = SR_TK_ROW_CAP;
 constexpr uint32_t kKeyNegInf = 0x007fffffu;  // sr_okey(-inf)
 constexpr uint32_t kRowHasPenalty = SR_ROWFLAG_HAS_PENALTY;
 constexpr uint32_t kRowHistExcl = SR_ROWFLAG_HIST_EXCL;
-constexpr int kOverflowMark = 1 << 24;        // added to a row's cursor by a chunk that cannot hand over its candidates
+constexpr int kQCap = 2 * kSelMax;            // groups of a row whose elements the row tail fetches
 
 constexpr int kCandRegs = kRowCap / kThreads;   // candidates a thread holds in the row tail (16)
 constexpr int kSortRegs = kSelMax / kThreads;   // sort elements per thread (4)
@@ -388,8 +388,12 @@ __device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
 // Called by every thread of the tail workgroup of a row once all chunks have appended their candidates.
 // slot = position of the row in this launch, n_c = candidates in the row's list.  The list is read once,
 // straight into registers; every later pass runs from registers or LDS.
-__device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, int n_c,
-                                              TopkSmem& sm)
+template <int EPV, int kVec, typename Early, typename Late>
+__device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, Early&& early,
+                                                Late&& late, TopkSmem& sm);
+
+template <int EPV, int kVec>
+__device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, TopkSmem& sm)
 {
     const int tid = threadIdx.x;
     const unsigned long long* cand = a.cand + (size_t)slot * kRowCap;
@@ -401,8 +405,6 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             if (a.out_flags) a.out_flags[row] = out_flag | extra;
         }
     };
-    if (sel > kSelMax || n_c < 0 || n_c > kRowCap) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
-
     const SrEdit* ed = a.edits + rd.edit_off;
     const bool use_edits = (rd.flags & kRowHasPenalty) != 0u && rd.edit_cnt > 0;
     const bool excl = use_edits && (rd.flags & kRowHistExcl) != 0u;  // the scan skipped the history ids
@@ -415,6 +417,32 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         return x;
     };
 
+    // The history ids and their logits are fetched behind the candidate builder's own loads, so that neither
+    // waits for the other.
+    const bool hist_regs = excl && rd.path == SR_PATH_TOPK && ne <= kHistRegs * kThreads;
+    SrEdit hee[kHistRegs];
+    float hx[kHistRegs];
+#pragma unroll
+    for (int r = 0; r < kHistRegs; r++) { hee[r] = SrEdit{}; hx[r] = SR_NEG_INF; }
+    const int n_c = build_candidates<EPV, kVec>(
+        a, slot, row, rd,
+        [&]() SR_INL {
+#pragma unroll
+            for (int r = 0; r < kHistRegs; r++) {
+                const int e = r * kThreads + tid;
+                if (hist_regs && e < ne) hee[r] = ed[e];
+            }
+        },
+        [&]() SR_INL {
+#pragma unroll
+            for (int r = 0; r < kHistRegs; r++) {
+                const int e = r * kThreads + tid;
+                if (hist_regs && e < ne) hx[r] = hist_logit(hee[r].id);
+            }
+        },
+        sm);
+    if (sel > kSelMax || n_c < 0 || n_c > kRowCap) { give_up(SR_KFLAG_UNSUPPORTED, -1); return; }
+
     SR_PROF(a, 11);
     const int nr = (n_c + kThreads - 1) / kThreads;  // register slots that can hold a candidate
     uint32_t kreg[kCandRegs];                         // 0 = no candidate in this slot
@@ -426,11 +454,17 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         if (r >= nr) continue;
         const int g = r * kThreads + tid;
         if (g < n_c) {
-            const unsigned long long cv = sr_load_agent(&cand[g]);
-            kreg[r] = sr_okey(sr_u2f((uint32_t)(cv >> 32)));
-            kid[r] = (int)(uint32_t)cv;
+            if (g < kSelMax) {  // the first candidates lie in LDS, only an unusually long list continues in memory
+                kreg[r] = sr_okey(sm.vals[g]);
+                kid[r] = sm.idxs[g];
+            } else {
+                const unsigned long long cv = sr_load_agent(&cand[g]);
+                kreg[r] = sr_okey(sr_u2f((uint32_t)(cv >> 32)));
+                kid[r] = (int)(uint32_t)cv;
+            }
         }
     }
+    __syncthreads();  // sm.vals / sm.idxs may be reused from here on
     auto cand_id = [&](int r) SR_INL -> int { return kid[r]; };
     SR_PROF(a, 12);
     auto each_key = [&](auto&& body) SR_INL {
@@ -624,8 +658,8 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             hadj[r] = hraw[r] = 0u;
             const int e = r * kThreads + tid;
             if (e < ne) {
-                const SrEdit ee = ed[e];
-                const float x = hist_logit(ee.id);
+                const SrEdit ee = hee[r];
+                const float x = hx[r];
                 // -inf never enters the reference's selection (Sampler.cs:240-249)
                 if (x == x && sr_f2u(x) != 0xff800000u) {
                     float v = x;
@@ -755,7 +789,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                     if (pos < kSelMax) {
                         sm.xa[pos] = hadj[r];
                         sm.xb[pos] = hraw[r];
-                        sm.xc[pos] = 0xffffffffu - (uint32_t)ed[r * kThreads + tid].id;
+                        sm.xc[pos] = 0xffffffffu - (uint32_t)hee[r].id;
                     }
                 }
             }
@@ -904,6 +938,268 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     }
 }
 
+
+// ---- candidates of a row from its group maxima ---------------------------------------------------------
+// The chunk workgroups left, per thread and chunk, the maxima of four disjoint groups of the row's elements.
+// Any value with at least sel group maxima at or above it is a lower bound on the row's sel-th largest element,
+// so only the groups at or above it can hold one of the sel largest: their elements are fetched again (a few
+// KB, from L2 / memory-side cache) and those at or above the bound become the row's candidates -- the first
+// SR_TK_SEL_MAX in sm.vals / sm.idxs, the rest of an unusually long list in a.cand.  Returns the number of
+// candidates, or -1 when the row cannot be handled.  Called by every thread of the tail workgroup; the two
+// hooks let the caller issue loads of its own behind the group maxima's (early) and after the first wait (late).
+template <int EPV, int kVec, typename Early, typename Late>
+__device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, Early&& early,
+                                                Late&& late, TopkSmem& sm)
+{
+    using VO = VecOps<EPV>;
+    constexpr int ES = (EPV == 4) ? 4 : 2;
+    constexpr int kGV = (kVec + SR_TK_GROUPS - 1) / SR_TK_GROUPS;  // vectors per group
+    constexpr int kGmRegs = 8;                                     // chunks whose maxima a thread keeps in registers
+    constexpr int kBatch = (EPV == 4) ? 8 : 4;                     // (group, vector) items fetched at once
+    const int tid = threadIdx.x, lane = sr_lane(), S = a.chunks, sel = rd.sel;
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+    const int mis = (int)(((uintptr_t)rowp & 15u) / ES);
+    const int nvt = (a.vocab + mis + EPV - 1) / EPV;
+    const u32x4* wp = (const u32x4*)(rowp - (size_t)mis * ES);
+    const uint32_t* keep32 = (const uint32_t*)(a.scan_mask + (size_t)rd.scan_row * (size_t)a.scan_stride);
+    const float4* gm = a.gmax + (size_t)slot * S * kThreads + tid;
+    unsigned long long* crow = a.cand + (size_t)slot * kRowCap;
+    uint32_t* qlist = sm.xa;  // kQCap entries: xa and xb lie back to back
+    auto gm_load = [&](int c) SR_INL -> float4 { return gm[(size_t)c * kThreads]; };
+    float4 gmr[kGmRegs];
+#pragma unroll
+    for (int c = 0; c < kGmRegs; c++) gmr[c] = c < S ? gm_load(c) : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+    // with few chunks the second maxima and the positions of the maxima come along in the same batch of loads
+    constexpr int kG2Regs = 4;
+    const bool direct = S <= kG2Regs;  // a group whose second largest is below the bound hands over its largest directly
+    float4 g2r[kG2Regs];
+    uint32_t gpr[kG2Regs];
+#pragma unroll
+    for (int c = 0; c < kG2Regs; c++) {
+        const bool in = direct && c < S;
+        g2r[c] = in ? a.gmax2[((size_t)slot * S + c) * kThreads + tid] : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+        gpr[c] = in ? a.gpos[((size_t)slot * S + c) * kThreads + tid] : 0u;
+    }
+    early();
+    auto each_gm = [&](auto&& f) SR_INL {
+#pragma unroll
+        for (int c = 0; c < kGmRegs; c++)
+            if (c < S) f(c, gmr[c]);
+        for (int c = kGmRegs; c < S; c++) f(c, gm_load(c));
+    };
+    // wave-aggregated append to a list in LDS: one atomic per wave and call
+    auto wave_slot = [&](bool want, uint32_t* counter) SR_INL -> int {
+        const unsigned long long bal = __ballot(want);
+        if (bal == 0ull) return -1;
+        uint32_t base = 0u;
+        if (lane == (int)__ffsll((long long)bal) - 1) base = atomicAdd(counter, (uint32_t)__popcll(bal));
+        base = __shfl(base, (int)__ffsll((long long)bal) - 1);
+        return want ? (int)(base + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))) : -1;
+    };
+    auto append = [&](bool want, float x, int idx) SR_INL {
+        const int pos = wave_slot(want, &sm.bcast[12]);
+        if (pos >= 0) {
+            if (pos < kSelMax) {
+                sm.vals[pos] = x;
+                sm.idxs[pos] = idx;
+            } else if (pos < kRowCap) {
+                sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx);
+            }
+        }
+    };
+    auto list_group = [&](bool want, int c, int g) SR_INL {
+        const int pos = wave_slot(want, &sm.bcast[13]);
+        if (pos >= 0 && pos < kQCap) qlist[pos] = ((uint32_t)(c * kThreads + tid) << 2) | (uint32_t)g;
+    };
+    // fetches the listed groups, kBatch (group, vector) items per thread at a time -- values and the keep-bit halves
+    // of all of them in one batch of loads -- and hands every kept element to f(value, index)
+    auto gather = [&](int nq, auto&& f) SR_INL {
+        const int n_items = nq * kGV;
+        for (int i0 = 0; i0 < n_items; i0 += kBatch * kThreads) {
+            u32x4 v[kBatch];
+            uint32_t kw[kBatch][EPV];
+            int fvs[kBatch];
+#pragma unroll
+            for (int r = 0; r < kBatch; r++) {
+                const int i = i0 + r * kThreads + tid;
+                fvs[r] = -1;
+                v[r] = VO::neg_inf();
+#pragma unroll
+                for (int q = 0; q < EPV; q++) kw[r][q] = 0u;
+                if (i < n_items) {
+                    const uint32_t gid = qlist[i / kGV];
+                    const int m = i - (i / kGV) * kGV;
+                    const int g = (int)(gid & 3u), t = (int)((gid >> 2) & (kThreads - 1)), c = (int)(gid >> 11);
+                    const int f0 = c * a.chunk_vecs;
+                    const int nv = min(a.chunk_vecs, nvt - f0);
+                    const int j = g + m * SR_TK_GROUPS;
+                    const int fl = j * kThreads + t;
+                    if (j < kVec && fl < nv) {
+                        const int fv = f0 + fl;
+                        fvs[r] = fv;
+                        v[r] = wp[fv];
+                        const uint32_t* kp = keep32 + ((size_t)(fv >> 6) * EPV) * 2 + ((fv & 63) >> 5);
+#pragma unroll
+                        for (int q = 0; q < EPV; q++) kw[r][q] = kp[2 * q];
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < kBatch; r++) {
+#pragma unroll
+                for (int q = 0; q < EPV; q++) {
+                    const bool kept = fvs[r] >= 0 && ((kw[r][q] >> (fvs[r] & 31)) & 1u) != 0u;
+                    f(kept, VO::get(v[r], q), fvs[r] * EPV + q - mis);
+                }
+            }
+        }
+    };
+
+    if (tid == 0) { sm.bcast[12] = 0u; sm.bcast[13] = 0u; }
+    __syncthreads();
+    if (sel > kSelMax || sel < 1) return -1;
+    // The chunk workgroups' waves each left a value with their share of sel group maxima at or above it: the
+    // smallest of them has at least sel group maxima of the row at or above it.
+    float tval = -3.402823466e38f;
+    {
+        const int nb = S * kWaves;
+        uint32_t k = 0xffffffffu;
+        for (int i = lane; i < nb; i += SR_WAVE) k = min(k, a.gbound[(size_t)slot * nb + i]);
+        k = sr_wave_min_u32(k);
+        if (k > kKeyNegInf) tval = sr_okey_inv(k);
+    }
+    late();
+    SR_PROF(a, 1);
+    if (direct) {
+        // the element index of the largest element of group g of chunk c: p = (vector inside the group) * EPV + q
+        auto idx_of = [&](int c, int g, uint32_t p) SR_INL -> int {
+            const int fv = c * a.chunk_vecs + (g + (int)(p / EPV) * SR_TK_GROUPS) * kThreads + tid;
+            return fv * EPV + (int)(p % EPV) - mis;
+        };
+        // two passes over the 16 groups of the thread: count per wave (ballots, scalar), reserve both lists' slices
+        // with one atomic each, then place
+        int n_list = 0, n_app = 0;
+#pragma unroll
+        for (int c = 0; c < kG2Regs; c++) {
+            if (c < S) {
+                const float m1[4] = {gmr[c].x, gmr[c].y, gmr[c].z, gmr[c].w};
+                const float m2[4] = {g2r[c].x, g2r[c].y, g2r[c].z, g2r[c].w};
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    n_list += __popcll(__ballot(m2[g] >= tval));
+                    n_app += __popcll(__ballot(m1[g] >= tval && !(m2[g] >= tval)));
+                }
+            }
+        }
+        uint32_t base_l = 0u, base_a = 0u;
+        if (lane == 0) {
+            if (n_list > 0) base_l = atomicAdd(&sm.bcast[13], (uint32_t)n_list);
+            if (n_app > 0) base_a = atomicAdd(&sm.bcast[12], (uint32_t)n_app);
+        }
+        base_l = __builtin_amdgcn_readfirstlane(base_l);
+        base_a = __builtin_amdgcn_readfirstlane(base_a);
+#pragma unroll
+        for (int c = 0; c < kG2Regs; c++) {
+            if (c < S) {
+                const float m1[4] = {gmr[c].x, gmr[c].y, gmr[c].z, gmr[c].w};
+                const float m2[4] = {g2r[c].x, g2r[c].y, g2r[c].z, g2r[c].w};
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const bool q2 = m2[g] >= tval, q1 = m1[g] >= tval && !q2;
+                    const unsigned long long b2 = __ballot(q2), b1 = __ballot(q1);
+                    if (q2) {  // may hold more than one: fetched below
+                        const uint32_t pos = base_l + __builtin_amdgcn_mbcnt_hi((uint32_t)(b2 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b2, 0u));
+                        if (pos < (uint32_t)kQCap) qlist[pos] = ((uint32_t)(c * kThreads + tid) << 2) | (uint32_t)g;
+                    }
+                    if (q1) {  // holds exactly one
+                        const uint32_t pos = base_a + __builtin_amdgcn_mbcnt_hi((uint32_t)(b1 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b1, 0u));
+                        const int idx = idx_of(c, g, (gpr[c] >> (8 * g)) & 0xffu);
+                        if (pos < (uint32_t)kSelMax) {
+                            sm.vals[pos] = m1[g];
+                            sm.idxs[pos] = idx;
+                        } else if (pos < (uint32_t)kRowCap) {
+                            sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(m1[g]) << 32) | (unsigned long long)(uint32_t)idx);
+                        }
+                    }
+                    base_l += (uint32_t)__popcll(b2);
+                    base_a += (uint32_t)__popcll(b1);
+                }
+            }
+        }
+    } else {
+        each_gm([&](int c, const float4& v) {
+            list_group(v.x >= tval, c, 0);
+            list_group(v.y >= tval, c, 1);
+            list_group(v.z >= tval, c, 2);
+            list_group(v.w >= tval, c, 3);
+        });
+    }
+    __syncthreads();
+    const int n_q = (int)sm.bcast[13];
+    SR_PROF(a, 2);
+    if (n_q <= kQCap) {
+        SR_PROF(a, 3);
+        gather(n_q, [&](bool kept, float x, int idx) { append(kept && x >= tval, x, idx); });
+    } else {
+        // Too many groups at or above the bound: the row is flat or heavily tied (or has too many chunks for the
+        // per-wave bound).  Exact bound instead: the sel-th largest group maximum; every element above it lies in a
+        // group whose maximum is above it (fewer than sel groups); of the elements equal to it only the first few by
+        // index can matter, and those come from a scan of the row in index order that stops as soon as it has them.
+        auto each_gk = [&](auto&& body) SR_INL {
+            each_gm([&](int, const float4& v) {
+                body(sr_okey(v.x)); body(sr_okey(v.y)); body(sr_okey(v.z)); body(sr_okey(v.w));
+            });
+        };
+        const uint32_t tkey = block_radix_select(each_gk, sel, sm);
+        const float tx = (tkey <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(tkey);
+        __syncthreads();
+        if (tid == 0) { sm.bcast[13] = 0u; sm.bcast[12] = 0u; }  // candidates handed over so far are found again below
+        __syncthreads();
+        each_gm([&](int c, const float4& v) {
+            list_group(v.x > tx, c, 0);
+            list_group(v.y > tx, c, 1);
+            list_group(v.z > tx, c, 2);
+            list_group(v.w > tx, c, 3);
+        });
+        __syncthreads();
+        const int nq = min((int)sm.bcast[13], kQCap);  // < sel
+        gather(nq, [&](bool kept, float x, int idx) { append(kept && x > tx, x, idx); });
+        __syncthreads();
+        const int n_gt = (int)sm.bcast[12];
+        const int need_eq = sel - n_gt;
+        int emitted = 0;
+        for (int f_base = 0; f_base < nvt && emitted < need_eq; f_base += kThreads) {
+            const int fv = f_base + tid;
+            int ceq = 0;
+            bool is_eq[EPV];
+#pragma unroll
+            for (int q = 0; q < EPV; q++) is_eq[q] = false;
+            if (fv < nvt) {
+                const u32x4 v = wp[fv];
+                const uint32_t* kp = keep32 + ((size_t)(fv >> 6) * EPV) * 2 + ((fv & 63) >> 5);
+#pragma unroll
+                for (int q = 0; q < EPV; q++) {
+                    is_eq[q] = VO::get(v, q) == tx && ((kp[2 * q] >> (fv & 31)) & 1u) != 0u;
+                    ceq += is_eq[q] ? 1 : 0;
+                }
+            }
+            int tile_total;
+            int rank = emitted + block_excl_scan(ceq, &tile_total, sm);
+#pragma unroll
+            for (int q = 0; q < EPV; q++) {
+                append(is_eq[q] && rank < need_eq, tx, fv * EPV + q - mis);
+                rank += is_eq[q] ? 1 : 0;
+            }
+            emitted += tile_total;
+        }
+    }
+    sr_drain_stores();
+    __syncthreads();
+    const uint32_t n_c = sm.bcast[12];
+    __syncthreads();
+    return n_c > (uint32_t)kRowCap ? -1 : (int)n_c;
+}
+
 // ---- the kernel --------------------------------------------------------------------------------------
 template <int EPV, int kVec>
 __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
@@ -920,17 +1216,18 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     const int slot_ = (int)(item & 0xffffffu), c_ = (int)((item >> 24) & 0x7fu);
     if (is_tail) {
         const int tslot = slot_;
-        const int trow = a.row_list[tslot];
+        // the row's descriptor does not depend on the chunks: fetched before the wait
+        const int trow = a.slot_info[tslot].x;
+        const SrRow trd = a.rows[trow];
         if (tid == 0) {
             uint32_t ok = 0u;
             for (int it = 0; it < (1 << 22); it++) {
                 if (sr_load_agent(&a.row_done[tslot]) == (uint32_t)S) { ok = 1u; break; }
                 __builtin_amdgcn_s_sleep(4);
             }
-            __atomic_signal_fence(__ATOMIC_SEQ_CST);
-            sm.bcast[8] = (uint32_t)sr_load_agent(&a.cand_cnt[tslot]);
+            // the chunks' results were written through to L2: drop what this CU's L1 may hold of an earlier launch
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
             sr_store_agent(&a.row_done[tslot], 0u);  // ready for the next launch
-            sr_store_agent(&a.cand_cnt[tslot], 0);
             sm.bcast[7] = ok;
         }
         __syncthreads();
@@ -942,28 +1239,14 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             return;
         }
         SR_PROF(a, 4);
-        topk_row_tail(a, tslot, trow, a.rows[trow], (int)sm.bcast[8], sm);
+        topk_row_tail<EPV, kVec>(a, tslot, trow, trd, sm);
         SR_PROF(a, 15);
         return;
     }
     const int slot = slot_, c = c_;
-    const int row = a.row_list[slot];
-    const SrRow rd = a.rows[row];
+    const int4 info = a.slot_info[slot];  // (row, scan-mask row, sel): one load between the workgroup and its data
+    const int row = info.x;
     const int V = a.vocab;
-    const int sel = rd.sel;
-    unsigned long long* crow = a.cand + (size_t)slot * kRowCap;
-    int* cursor = a.cand_cnt + slot;
-    // a 32-bit byte offset from the wave-uniform list base: the base stays in scalar registers
-    auto cand_store = [](unsigned long long* base, uint32_t pos, unsigned long long v) SR_INL {
-        sr_store_agent((unsigned long long*)((char*)base + (size_t)(pos * 8u)), v);
-    };
-    auto pack = [](float x, int idx) SR_INL -> unsigned long long {
-        // A real copy that the compiler cannot fold: otherwise every register of the chunk is coalesced with the
-        // high half of a 64-bit store operand, which must sit in an odd register -- and only half of them are.
-        float xc;
-        asm volatile("v_mov_b32 %0, %1" : "=v"(xc) : "v"(x));
-        return ((unsigned long long)sr_f2u(xc) << 32) | (unsigned long long)(uint32_t)idx;
-    };
     // phase timestamps stay in registers until the end: a store ahead of the scan-mask loads would keep the
     // compiler from using scalar loads for them
     unsigned long long pt0 = 0, pt1 = 0, pt2 = 0;
@@ -979,7 +1262,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     const int nv = min(a.chunk_vecs, nvt - f0);        // vectors of this chunk
     const int wbase = f0 * EPV - mis;                  // row element index of the chunk's first window element
 
-    if (nv > 0 && sel <= kSelMax) {
+    if (nv > 0) {
         const u32x4* cp = (const u32x4*)(rowp - (size_t)mis * ES) + f0;
         // the chunk as fp32 in registers (the upcast of bf16 is exact)
         float xv[kVec * EPV];
@@ -1008,7 +1291,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             // read through the constant address space: the mask was written by an earlier launch, and scalar
             // loads need the compiler to know that nothing in this kernel writes it
             typedef const unsigned long long __attribute__((address_space(4))) const_u64;
-            const_u64* srow = (const_u64*)(uintptr_t)(a.scan_mask + (size_t)rd.scan_row * (size_t)a.scan_stride);
+            const_u64* srow = (const_u64*)(uintptr_t)(a.scan_mask + (size_t)info.y * (size_t)a.scan_stride);
             const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
             const int nblk = (nvt + 63) >> 6;
 #pragma unroll
@@ -1023,314 +1306,75 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         }
         if (a.prof) pt1 = wall_clock64();
 
-        const int wlim = kRowCap / (S * kWaves);  // candidates one wave may hand over when waves work alone
-        const int blim = min(kRowCap / S, 2 * sel + 128);  // candidates the chunk may hand over otherwise
-        // sel <= 64: every wave on its own, no workgroup barrier.  Larger sel: the waves agree on one threshold
-        // estimated from their group maxima, and keep it if the chunk holds between sel and blim elements at
-        // or above it; else (and on short chunks) the exact selection further down decides.
-        const bool wave_mode = sel <= SR_WAVE && wlim >= SR_TK_WAVE_LIM;
-        const bool shared_mode = !wave_mode && nv > 4 * kThreads && sel <= SR_TK_M && blim >= sel;
-        bool handed_over = false;
-        if (shared_mode) {
-            if (tid == 0) { sm.ksum = 0ull; sm.btotal = 0u; }
-            __syncthreads();
+        // Every lane owns four interleaved groups of vectors (j mod 4).  Of each group the row tail gets the largest
+        // element with its position inside the group, and the second largest: a group whose second largest is below
+        // the row's bound contributes its largest element directly and is never read again.
+        float gm1[SR_TK_GROUPS], gm2[SR_TK_GROUPS];
+        uint32_t gpk = 0u;
+#pragma unroll
+        for (int g = 0; g < SR_TK_GROUPS; g++) {
+            float m1 = SR_NEG_INF, m2 = SR_NEG_INF;
+            int p1 = 0;
+#pragma unroll
+            for (int j = g; j < kVec; j += SR_TK_GROUPS)
+#pragma unroll
+                for (int q = 0; q < EPV; q++) {
+                    const float x = xv[j * EPV + q];
+                    p1 = x > m1 ? (j / SR_TK_GROUPS) * EPV + q : p1;  // strict: the first of equal values stays
+                    m2 = fmaxf(m2, fminf(m1, x));
+                    m1 = fmaxf(m1, x);
+                }
+            gm1[g] = m1;
+            gm2[g] = m2;
+            gpk |= (uint32_t)p1 << (8 * g);
         }
-        if (wave_mode || shared_mode) {
-            // every lane owns four interleaved groups of vectors (j mod 4); the need-th largest of the wave's
-            // 256 group maxima is found bit by bit.  need = sel makes it a lower bound on the wave's sel-th
-            // largest element.
-            uint32_t gk[SR_TK_GROUPS];
-#pragma unroll
-            for (int g = 0; g < SR_TK_GROUPS; g++) {
-                float mxv = SR_NEG_INF;
-#pragma unroll
-                for (int j = g; j < kVec; j += SR_TK_GROUPS)
-#pragma unroll
-                    for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, xv[j * EPV + q]);
-                gk[g] = sr_okey(mxv);
-            }
-            int need = sel;
-            if (shared_mode) {
-                // aim a little above sel elements (the estimate scatters by a few percent): with a fraction p of the
-                // chunk above the threshold,
-                // a group of n_g elements has its maximum above it with probability 1 - (1 - p)^n_g
-                const float n_elem = (float)nv * (float)EPV;
-                const float p = fminf(fminf(1.12f * (float)sel + 40.0f, 0.5f * (float)(sel + blim)) / n_elem, 0.5f);
-                const float n_g = n_elem / (float)SR_TK_M;
-                const float frac = 1.0f - __expf(n_g * __logf(1.0f - p));
-                need = min(max((int)(frac * (float)(SR_WAVE * SR_TK_GROUPS) + 0.5f), 1), SR_WAVE * SR_TK_GROUPS);
-            }
+        if (a.prof) pt2 = wall_clock64();
+        const size_t go = ((size_t)slot * S + c) * kThreads + tid;
+        float4* gout = a.gmax + go;
+        __hip_atomic_store(&gout->x, gm1[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout->y, gm1[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout->z, gm1[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout->w, gm1[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float4* gout2 = a.gmax2 + go;
+        __hip_atomic_store(&gout2->x, gm2[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout2->y, gm2[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout2->z, gm2[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout2->w, gm2[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(a.gpos + go, gpk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // The wave's share of the row's bound: a value, to 16 bits and rounded down, with at least
+        // ceil(sel / (chunks x 8)) of the wave's 256 group maxima at or above it (found bit by bit with ballots).
+        // The smallest of all the row's waves' values then has at least sel group maxima at or above it.
+        __builtin_amdgcn_sched_barrier(0);  // after the stores: the chunk's registers are free by now
+        {
+            const int need = (__builtin_amdgcn_readfirstlane(info.z) + S * kWaves - 1) / (S * kWaves);
             uint32_t K = 0u;
 #pragma unroll 1
-            for (int bit = 31; bit >= 0; bit--) {
+            for (int bit = 31; bit >= 16; bit--) {
                 const uint32_t cnd = K | (1u << bit);
-                int cge = 0;
-#pragma unroll
-                for (int g = 0; g < SR_TK_GROUPS; g++) cge += __popcll(__ballot(gk[g] >= cnd));
+                const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
+                const int cge = __popcll(__ballot(gm1[0] >= fc)) + __popcll(__ballot(gm1[1] >= fc)) +
+                                __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc));
                 if (cge >= need) K = cnd;
             }
-            if (shared_mode) {
-                // the mean of the waves' estimates (as keys: they lie close together)
-                if (lane == 0) atomicAdd(&sm.ksum, (unsigned long long)K);
-                __syncthreads();
-                K = (uint32_t)(sm.ksum / (unsigned long long)kWaves);
-            }
-            // -inf never enters the candidate set (Sampler.cs:240-249: strict v <= -inf rejects it)
-            float tval = (K <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(K);
-            if (a.prof) pt2 = wall_clock64();
-            int total = 0;  // wave-uniform: the comparisons land in scalar registers
-#pragma unroll
-            for (int j = 0; j < kVec; j++)
-#pragma unroll
-                for (int q = 0; q < EPV; q++) total += __popcll(__ballot(xv[j * EPV + q] >= tval));
-            bool emit_all = wave_mode && total <= wlim;
-            if (shared_mode) {
-                if (lane == 0) atomicAdd(&sm.btotal, (uint32_t)total);
-                __syncthreads();
-                const int bt = (int)sm.btotal;
-                emit_all = bt >= sel && bt <= blim;
-            }
-            handed_over = wave_mode || emit_all;
-            if (emit_all) {
-                int base = 0;
-                if (lane == 0 && total > 0)
-                    base = __hip_atomic_fetch_add(cursor, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                base = __builtin_amdgcn_readfirstlane(base);
-                if (total > 0 && base >= 0 && base + total <= kRowCap) {
-                    int off = base;
-                    // an opaque copy: the comparisons of the counting pass must not be kept alive (two scalar
-                    // registers each) for this pass
-                    float tv = tval;
-                    asm volatile("" : "+v"(tv));
-#pragma unroll
-                    for (int j = 0; j < kVec; j++) {
-                        const int e0 = wbase + (j * kThreads + tid) * EPV;
-#pragma unroll
-                        for (int q = 0; q < EPV; q++) {
-                            const float x = xv[j * EPV + q];
-                            const unsigned long long bal = __ballot(x >= tv);
-                            if (bal) {
-                                if (x >= tv) {
-                                    const int pos = off + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32),
-                                                              __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u));
-                                    cand_store(crow, (uint32_t)(pos), pack(x, e0 + q));
-                                }
-                                off += __popcll(bal);
-                            }
-                        }
-                    }
-                }
-            } else if (wave_mode) {
-                // Many elements at or above the bound.  Equal values rank by ascending index, so besides
-                // everything above the threshold only the first (sel - #above) ties can matter.
-                int cgt = 0;
-#pragma unroll
-                for (int j = 0; j < kVec; j++)
-#pragma unroll
-                    for (int q = 0; q < EPV; q++) cgt += (xv[j * EPV + q] > tval) ? 1 : 0;
-                int total_gt = sr_wave_sum_i32(cgt);
-                if (total_gt > wlim) {
-                    // the lane maxima bound is too loose (the large values sit in few lanes): the exact sel-th
-                    // largest element of the wave, bit by bit
-                    // (compared as floats: a key in the NaN range compares false, and the answer is finite)
-                    uint32_t K2 = 0u;
-#pragma unroll 1
-                    for (int bit = 31; bit >= 0; bit--) {
-                        const uint32_t cnd = K2 | (1u << bit);
-                        const float fc = sr_okey_inv(cnd);
-                        int cge = 0;
-#pragma unroll
-                        for (int j = 0; j < kVec; j++)
-#pragma unroll
-                            for (int q = 0; q < EPV; q++) cge += __popcll(__ballot(xv[j * EPV + q] >= fc));
-                        if (cge >= sel) K2 = cnd;
-                    }
-                    tval = sr_okey_inv(K2);
-                    cgt = 0;
-#pragma unroll
-                    for (int j = 0; j < kVec; j++)
-#pragma unroll
-                        for (int q = 0; q < EPV; q++) cgt += (xv[j * EPV + q] > tval) ? 1 : 0;
-                    total_gt = sr_wave_sum_i32(cgt);
-                }
-                int total_eq = 0;
-#pragma unroll
-                for (int j = 0; j < kVec; j++)
-#pragma unroll
-                    for (int q = 0; q < EPV; q++) total_eq += __popcll(__ballot(xv[j * EPV + q] == tval));
-                const int n_eq = max(0, min(min(sel - total_gt, wlim - total_gt), total_eq));
-                const int incl = sr_wave_incl_scan_i32(cgt);
-                total = total_gt + n_eq;
-                int base = 0;
-                if (lane == 0 && total > 0)
-                    base = __hip_atomic_fetch_add(cursor, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                base = __builtin_amdgcn_readfirstlane(base);
-                if (total > 0 && base >= 0 && base + total <= kRowCap) {
-                    int pos = base + incl - cgt;
-                    if (cgt > 0) {
-#pragma unroll
-                        for (int j = 0; j < kVec; j++) {
-                            const int e0 = wbase + (j * kThreads + tid) * EPV;
-#pragma unroll
-                            for (int q = 0; q < EPV; q++) {
-                                const float x = xv[j * EPV + q];
-                                if (x > tval) { cand_store(crow, (uint32_t)(pos), pack(x, e0 + q)); pos++; }
-                            }
-                        }
-                    }
-                    int emitted = 0;
-#pragma unroll
-                    for (int j = 0; j < kVec; j++) {  // ascending j, then lane, then q = ascending index
-                        if (emitted >= n_eq) continue;  // wave-uniform
-                        int ceq = 0;
-#pragma unroll
-                        for (int q = 0; q < EPV; q++) ceq += (xv[j * EPV + q] == tval) ? 1 : 0;
-                        const int ie = sr_wave_incl_scan_i32(ceq);
-                        int rank = emitted + ie - ceq;
-                        if (ceq > 0) {
-                            const int e0 = wbase + (j * kThreads + tid) * EPV;
-#pragma unroll
-                            for (int q = 0; q < EPV; q++) {
-                                if (xv[j * EPV + q] == tval) {
-                                    if (rank < n_eq) cand_store(crow, (uint32_t)(base + total_gt + rank), pack(tval, e0 + q));
-                                    rank++;
-                                }
-                            }
-                        }
-                        emitted += __shfl(ie, SR_WAVE - 1);
-                    }
-                }
-            }
+            if (lane == 0) __hip_atomic_store(a.gbound + ((size_t)slot * S + c) * kWaves + (tid >> 6), K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (!handed_over) {
-            // ---- the whole workgroup: threshold from 2048 group maxima (or exactly, on a short chunk) ------
-            auto reserve = [&](int n) SR_INL -> int {  // all threads; returns the first list position
-                __syncthreads();
-                if (tid == 0)
-                    sm.bcast[3] = (uint32_t)__hip_atomic_fetch_add(cursor, n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __syncthreads();
-                return (int)sm.bcast[3];
-            };
-            uint32_t tkey;
-            if (nv <= 4 * kThreads) {
-                // short chunk (at most four vectors per thread): select exactly over its elements
-                auto each_elem = [&](auto&& body) SR_INL {
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-#pragma unroll
-                        for (int q = 0; q < EPV; q++) body(sr_okey(xv[j * EPV + q]));
-                };
-                tkey = block_radix_select(each_elem, sel, sm);
-            } else {
-                // every thread owns four interleaved groups of vectors (j mod 4), all populated here; the
-                // sel-th largest of the 2048 disjoint-group maxima cannot exceed the sel-th largest element
-                uint32_t gk[SR_TK_GROUPS];
-#pragma unroll
-                for (int g = 0; g < SR_TK_GROUPS; g++) {
-                    float mxv = SR_NEG_INF;
-#pragma unroll
-                    for (int j = g; j < kVec; j += SR_TK_GROUPS)
-#pragma unroll
-                        for (int q = 0; q < EPV; q++) mxv = fmaxf(mxv, xv[j * EPV + q]);
-                    gk[g] = sr_okey(mxv);
-                }
-                auto each_gk = [&](auto&& body) SR_INL {
-#pragma unroll
-                    for (int g = 0; g < SR_TK_GROUPS; g++) body(gk[g]);
-                };
-                tkey = (sel > SR_TK_M) ? 0u : block_radix_select(each_gk, sel, sm);
-            }
-            if (a.prof) pt2 = wall_clock64();
-            const float tval = (tkey <= kKeyNegInf) ? -3.402823466e38f : sr_okey_inv(tkey);
-            int cnt = 0;
-#pragma unroll
-            for (int j = 0; j < kVec; j++)
-#pragma unroll
-                for (int q = 0; q < EPV; q++) cnt += (xv[j * EPV + q] >= tval) ? 1 : 0;
-            // a chunk hands over at most `lim` candidates, so that the row list can hold all chunks of a row
-            const int lim = min(kRowCap / S, 2 * sel + 128);
-            int total;
-            int pos = block_excl_scan(cnt, &total, sm);
-            if (lim < sel) {
-                (void)reserve(kOverflowMark);  // the row is reported as unsupported
-            } else if (total <= lim) {
-                const int base = reserve(total);
-                if (cnt > 0 && base >= 0 && base + total <= kRowCap) {
-                    pos += base;
-#pragma unroll
-                    for (int j = 0; j < kVec; j++) {
-                        const int e0 = wbase + (j * kThreads + tid) * EPV;
-#pragma unroll
-                        for (int q = 0; q < EPV; q++) {
-                            const float x = xv[j * EPV + q];
-                            if (x >= tval) { cand_store(crow, (uint32_t)(pos), pack(x, e0 + q)); pos++; }
-                        }
-                    }
-                }
-            } else {
-                // Many elements tie with the threshold value.  Equal values rank by ascending index, so
-                // besides everything above the threshold only the first (sel - #above) ties can matter.
-                int cgt = 0, ceq_all = 0;
-#pragma unroll
-                for (int j = 0; j < kVec; j++)
-#pragma unroll
-                    for (int q = 0; q < EPV; q++) {
-                        cgt += (xv[j * EPV + q] > tval) ? 1 : 0;
-                        ceq_all += (xv[j * EPV + q] == tval) ? 1 : 0;
-                    }
-                int total_gt;
-                int pgt = block_excl_scan(cgt, &total_gt, sm);
-                const int total_eq = block_sum_i32(ceq_all, sm);
-                if (total_gt > lim) {
-                    (void)reserve(kOverflowMark);  // genuine overflow: the row is reported as unsupported
-                } else {
-                    const int n_eq = max(0, min(min(sel - total_gt, lim - total_gt), total_eq));
-                    const int base = reserve(total_gt + n_eq);
-                    const bool fits = base >= 0 && base + total_gt + n_eq <= kRowCap;
-                    if (cgt > 0 && fits) {
-                        pgt += base;
-#pragma unroll
-                        for (int j = 0; j < kVec; j++) {
-                            const int e0 = wbase + (j * kThreads + tid) * EPV;
-#pragma unroll
-                            for (int q = 0; q < EPV; q++) {
-                                const float x = xv[j * EPV + q];
-                                if (x > tval) { cand_store(crow, (uint32_t)(pgt), pack(x, e0 + q)); pgt++; }
-                            }
-                        }
-                    }
-                    int emitted = 0;
-                    if (n_eq > 0) {
-#pragma unroll
-                        for (int j = 0; j < kVec; j++) {  // ascending j, then tid, then q = ascending index
-                            if (emitted >= n_eq) continue;  // block-uniform
-                            int ceq = 0;
-#pragma unroll
-                            for (int q = 0; q < EPV; q++) ceq += (xv[j * EPV + q] == tval) ? 1 : 0;
-                            int tj;
-                            int rank = emitted + block_excl_scan(ceq, &tj, sm);
-                            if (ceq > 0 && fits) {
-                                const int e0 = wbase + (j * kThreads + tid) * EPV;
-#pragma unroll
-                                for (int q = 0; q < EPV; q++) {
-                                    if (xv[j * EPV + q] == tval) {
-                                        if (rank < n_eq) cand_store(crow, (uint32_t)(base + total_gt + rank), pack(tval, e0 + q));
-                                        rank++;
-                                    }
-                                }
-                            }
-                            emitted += tj;
-                        }
-                    }
-                }
-            }
-        }
-    } else if (nv > 0 && tid == 0) {
-        (void)__hip_atomic_fetch_add(cursor, kOverflowMark, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        float4* gout = a.gmax + ((size_t)slot * S + c) * kThreads + tid;
+        __hip_atomic_store(&gout->x, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout->y, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout->z, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout->w, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float4* gout2 = a.gmax2 + ((size_t)slot * S + c) * kThreads + tid;
+        __hip_atomic_store(&gout2->x, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout2->y, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout2->z, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&gout2->w, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(a.gpos + ((size_t)slot * S + c) * kThreads + tid, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) __hip_atomic_store(a.gbound + ((size_t)slot * S + c) * kWaves + (tid >> 6), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     SR_PROF(a, 3);
     if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 0] = pt0; a.prof[(size_t)blockIdx.x * 16 + 1] = pt1; a.prof[(size_t)blockIdx.x * 16 + 2] = pt2; }
-    if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 13] = (unsigned long long)sel; a.prof[(size_t)blockIdx.x * 16 + 14] = (unsigned long long)slot; }
+    if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 13] = (unsigned long long)a.rows[row].sel; a.prof[(size_t)blockIdx.x * 16 + 14] = (unsigned long long)slot; }
 
     // hand the chunk over: drain this wave's write-through stores, meet, then count the chunk in
     sr_drain_stores();
