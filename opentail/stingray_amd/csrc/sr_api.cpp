@@ -67,16 +67,45 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     b->scan_stride_mod = stride_mod;
     if (b->h_scan.empty()) return SR_OK;
     {
-        std::vector<int32_t> info;
-        info.reserve(b->h_sel_list.size() * 4);
-        for (int32_t r : b->h_sel_list) {
-            info.push_back(r);
-            info.push_back(b->h_rows[(size_t)r].scan_row);
-            info.push_back(b->h_rows[(size_t)r].sel);
-            info.push_back(0);
+        // Dispatch order.  Workgroups are dispatched in grid order, two resident per CU; a round is that many
+        // consecutive workgroups.  A row's tail goes to the head of the round after the one that holds the row's
+        // last chunk: its chunks have at least all been dispatched by then and have usually finished, and tails
+        // that are ready do not queue behind later rows' chunks.  Every entry carries what its workgroup needs
+        // to find its data.
+        const int n_sel = (int)b->h_sel_list.size();
+        int chunks = 1, chunk_vecs = 0;
+        topk_geometry(b->vocab, epv == 8 ? SR_DTYPE_BF16 : SR_DTYPE_F32, n_sel, ctx->cu_count, &chunks, &chunk_vecs);
+        const int round = 2 * ctx->cu_count;
+        std::vector<int32_t> sched;
+        sched.reserve((size_t)n_sel * (size_t)(chunks + 1) * 4);
+        auto push = [&](uint32_t item, int slot) {
+            const int32_t r = b->h_sel_list[(size_t)slot];
+            sched.push_back((int32_t)item);
+            sched.push_back(r);
+            sched.push_back(b->h_rows[(size_t)r].scan_row);
+            sched.push_back(b->h_rows[(size_t)r].sel);
+        };
+        std::vector<int> ready_at((size_t)n_sel, 0);  // first position at which the row's tail may be placed
+        int next_tail = 0, row = 0, c = 0;
+        while (next_tail < n_sel) {
+            const int pos = (int)(sched.size() / 4);
+            if (next_tail < row && pos >= ready_at[(size_t)next_tail]) {
+                push(0x80000000u | (uint32_t)next_tail, next_tail);
+                next_tail++;
+            } else if (row < n_sel) {
+                push(((uint32_t)c << 24) | (uint32_t)row, row);
+                if (++c == chunks) {
+                    ready_at[(size_t)row] = (pos / round + 1) * round;
+                    c = 0;
+                    row++;
+                }
+            } else {
+                push(0x80000000u | (uint32_t)next_tail, next_tail);  // nothing left to overlap with
+                next_tail++;
+            }
         }
-        SR_HIP(ctx, b->d_slot_info.reserve(info.size() * sizeof(int32_t), st));
-        SR_HIP(ctx, hipMemcpyAsync(b->d_slot_info.p, info.data(), info.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+        SR_HIP(ctx, b->d_sched.reserve(sched.size() * sizeof(int32_t), st));
+        SR_HIP(ctx, hipMemcpyAsync(b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
         SR_HIP(ctx, hipStreamSynchronize(st));
     }
     const int64_t blocks = ((int64_t)b->vocab + 2 * epv - 2) / epv / 64 + 1;
@@ -129,7 +158,7 @@ void sr_destroy(sr_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
-    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->sched, &ctx->row_done, &ctx->argmax_best,
+    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best,
                          &ctx->work, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->spec_rows, &ctx->spec_probs};
@@ -176,7 +205,7 @@ void sr_batch_destroy(sr_batch* b)
     if (!b) return;
     if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
     DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_scan_desc,
-                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_slot_info};
+                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched};
     for (DeviceBuf* d : bufs) d->release();
     delete b;
 }
@@ -398,47 +427,13 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         topk_geometry(b->vocab, dtype, n_sel, ctx->cu_count, &a.chunks, &a.chunk_vecs);
         if (a.chunks > SR_TK_MAX_CHUNKS)
             return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary too large for the selection kernel");
-        // Dispatch order.  Workgroups are dispatched in grid order, two resident per CU; a round is that many
-        // consecutive workgroups.  A row's tail goes to the head of the round after the one that holds the row's
-        // last chunk: its chunks have at least all been dispatched by then and have usually finished, and tails
-        // that are ready do not queue behind later rows' chunks.
-        if (ctx->sched_rows != n_sel || ctx->sched_chunks != a.chunks) {
-            const int round = 2 * ctx->cu_count;
-            std::vector<uint32_t> sched;
-            sched.reserve((size_t)n_sel * (a.chunks + 1));
-            std::vector<int> ready_at((size_t)n_sel, 0);  // first position at which the row's tail may be placed
-            int next_tail = 0, row = 0, c = 0;
-            while (next_tail < n_sel) {
-                const int pos = (int)sched.size();
-                if (next_tail < row && pos >= ready_at[(size_t)next_tail]) {
-                    sched.push_back(0x80000000u | (uint32_t)next_tail);
-                    next_tail++;
-                } else if (row < n_sel) {
-                    sched.push_back(((uint32_t)c << 24) | (uint32_t)row);
-                    if (++c == a.chunks) {
-                        ready_at[(size_t)row] = (pos / round + 1) * round;
-                        c = 0;
-                        row++;
-                    }
-                } else {
-                    sched.push_back(0x80000000u | (uint32_t)next_tail);  // nothing left to overlap with
-                    next_tail++;
-                }
-            }
-            SR_HIP(ctx, ctx->sched.reserve(sched.size() * sizeof(uint32_t), st));
-            SR_HIP(ctx, hipMemcpyAsync(ctx->sched.p, sched.data(), sched.size() * sizeof(uint32_t), hipMemcpyHostToDevice, st));
-            SR_HIP(ctx, hipStreamSynchronize(st));
-            ctx->sched_rows = n_sel;
-            ctx->sched_chunks = a.chunks;
-        }
-        a.sched = ctx->sched.as<uint32_t>();
+        a.sched = b->d_sched.as<int4>();
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));
         SR_HIP(ctx, ctx->gmax.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
         SR_HIP(ctx, ctx->gmax2.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
         SR_HIP(ctx, ctx->gpos.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * sizeof(uint32_t), st));
         SR_HIP(ctx, ctx->gbound.reserve((size_t)n_sel * a.chunks * (SR_TK_THREADS / 64) * sizeof(uint32_t), st));
         SR_HIP(ctx, ctx->row_done.reserve((size_t)std::max(n_sel, 1024) * sizeof(uint32_t), st, true));
-        a.slot_info = b->d_slot_info.as<int4>();
         a.rows = b->d_rows.as<SrRow>();
         a.edits = b->d_edits.as<SrEdit>();
         a.mask = b->d_mask.as<uint32_t>();

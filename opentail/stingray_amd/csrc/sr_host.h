@@ -60,8 +60,6 @@ struct sr_ctx {
     DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
-    DeviceBuf sched;                     // dispatch order of the selection kernel's workgroups
-    int sched_rows = 0, sched_chunks = 0;
     int last_epv = 4;                    // vector width of the last launch: what an upload builds scan masks for
 };
 
@@ -74,7 +72,7 @@ struct sr_batch {
     std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path
     std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel
     std::vector<uint32_t> h_scan_need; // per batch row: SR_SCAN_* bits the row's scan mask must carry
-    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms, d_slot_info;
+    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms, d_sched;
     int64_t mask_stride = 0, scan_stride = 0;
     // what the scan masks were built for: elements per 16-byte vector, the logits base address modulo 16 and
     // the row stride in bytes modulo 16 (rows share a mask row only when all start at the same offset)

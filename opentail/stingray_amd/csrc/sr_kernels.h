@@ -24,8 +24,9 @@ struct SrTopkArgs {
     int32_t chunks;          // chunk workgroups per row
     int32_t n_rows;          // rows in this launch: grid = n_rows * chunks chunk workgroups + n_rows tail workgroups
     int32_t chunk_vecs;      // 16-byte vectors per chunk, a multiple of 64
-    const uint32_t* sched;   // per workgroup in dispatch order: bit 31 = row tail, bits 24..30 = chunk, bits 0..23 = slot
-    const int4* slot_info;   // per row of this launch, in launch order: (batch row, scan-mask row, sel, 0)
+    // per workgroup in dispatch order: x = bit 31 row tail | bits 24..30 chunk | bits 0..23 launch slot of the row,
+    // y = batch row, z = scan-mask row, w = sel -- all a workgroup needs to find its data, in one 16-byte load
+    const int4* sched;
     const SrRow* rows;
     const SrEdit* edits;
     const uint32_t* mask;

@@ -954,7 +954,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     using VO = VecOps<EPV>;
     constexpr int ES = (EPV == 4) ? 4 : 2;
     constexpr int kGV = (kVec + SR_TK_GROUPS - 1) / SR_TK_GROUPS;  // vectors per group
-    constexpr int kGmRegs = 8;                                     // chunks whose maxima a thread keeps in registers
+    constexpr int kGmRegs = 4;                                     // chunks whose maxima a thread keeps in registers
     constexpr int kBatch = (EPV == 4) ? 8 : 4;                     // (group, vector) items fetched at once
     const int tid = threadIdx.x, lane = sr_lane(), S = a.chunks, sel = rd.sel;
     const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
@@ -966,6 +966,41 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     unsigned long long* crow = a.cand + (size_t)slot * kRowCap;
     uint32_t* qlist = sm.xa;  // kQCap entries: xa and xb lie back to back
     auto gm_load = [&](int c) SR_INL -> float4 { return gm[(size_t)c * kThreads]; };
+    // the element index of the largest element of group g of chunk c: p = (vector inside the group) * EPV + q
+    auto idx_of = [&](int c, int g, uint32_t p) SR_INL -> int {
+        const int fv = c * a.chunk_vecs + (g + (int)(p / EPV) * SR_TK_GROUPS) * kThreads + tid;
+        return fv * EPV + (int)(p % EPV) - mis;
+    };
+    if (sel == 1) {
+        // one candidate: the row's largest kept element, the first by index among equals -- the largest group
+        // maximum, and of the groups that reach it the lowest position of their (first) largest element
+        early();
+        uint32_t km = 0u;
+        for (int c = 0; c < S; c++) {
+            const float4 m = gm_load(c);
+            km = max(max(max(km, sr_okey(m.x)), max(sr_okey(m.y), sr_okey(m.z))), sr_okey(m.w));
+        }
+        late();
+        km = block_max_u32(km, sm);
+        const bool any = km > kKeyNegInf;
+        int best = 0x7fffffff;
+        for (int c = 0; c < S && any; c++) {
+            const float4 m = gm_load(c);
+            if (max(max(sr_okey(m.x), sr_okey(m.y)), max(sr_okey(m.z), sr_okey(m.w))) != km) continue;
+            const uint32_t gp = a.gpos[((size_t)slot * S + c) * kThreads + tid];
+            const float m1[4] = {m.x, m.y, m.z, m.w};
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                if (sr_okey(m1[g]) == km) best = min(best, idx_of(c, g, (gp >> (8 * g)) & 0xffu));
+        }
+        best = block_min_i32(best, sm);
+        if (tid == 0 && any) {
+            sm.vals[0] = sr_okey_inv(km);
+            sm.idxs[0] = best;
+        }
+        __syncthreads();
+        return any ? 1 : 0;
+    }
     float4 gmr[kGmRegs];
 #pragma unroll
     for (int c = 0; c < kGmRegs; c++) gmr[c] = c < S ? gm_load(c) : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
@@ -1071,11 +1106,6 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     late();
     SR_PROF(a, 1);
     if (direct) {
-        // the element index of the largest element of group g of chunk c: p = (vector inside the group) * EPV + q
-        auto idx_of = [&](int c, int g, uint32_t p) SR_INL -> int {
-            const int fv = c * a.chunk_vecs + (g + (int)(p / EPV) * SR_TK_GROUPS) * kThreads + tid;
-            return fv * EPV + (int)(p % EPV) - mis;
-        };
         // two passes over the 16 groups of the thread: count per wave (ballots, scalar), reserve both lists' slices
         // with one atomic each, then place
         int n_list = 0, n_app = 0;
@@ -1211,13 +1241,18 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     // The host lays the workgroups out in dispatch order: chunk workgroups row by row, and the tail of a row
     // one full round of resident workgroups after the row's last chunk, so that a tail is dispatched after all
     // chunk workgroups of its row (it waits, bounded, only on work that is already running) and rarely waits.
-    const uint32_t item = a.sched[blockIdx.x];
+    // read through the constant address space (the host wrote it before the launch): one scalar 16-byte load
+    typedef int __attribute__((ext_vector_type(4))) i32x4;
+    typedef const i32x4 __attribute__((address_space(4))) const_i32x4;
+    const i32x4 info = ((const_i32x4*)(uintptr_t)a.sched)[blockIdx.x];  // (item, row, scan-mask row, sel)
+    const uint32_t item = (uint32_t)info.x;
     const bool is_tail = (item >> 31) != 0u;
     const int slot_ = (int)(item & 0xffffffu), c_ = (int)((item >> 24) & 0x7fu);
     if (is_tail) {
         const int tslot = slot_;
         // the row's descriptor does not depend on the chunks: fetched before the wait
-        const int trow = a.slot_info[tslot].x;
+        const int trow = info.y;
+        SR_PROF(a, 0);
         const SrRow trd = a.rows[trow];
         if (tid == 0) {
             uint32_t ok = 0u;
@@ -1244,8 +1279,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         return;
     }
     const int slot = slot_, c = c_;
-    const int4 info = a.slot_info[slot];  // (row, scan-mask row, sel): one load between the workgroup and its data
-    const int row = info.x;
+    const int row = info.y;
     const int V = a.vocab;
     // phase timestamps stay in registers until the end: a store ahead of the scan-mask loads would keep the
     // compiler from using scalar loads for them
@@ -1291,7 +1325,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             // read through the constant address space: the mask was written by an earlier launch, and scalar
             // loads need the compiler to know that nothing in this kernel writes it
             typedef const unsigned long long __attribute__((address_space(4))) const_u64;
-            const_u64* srow = (const_u64*)(uintptr_t)(a.scan_mask + (size_t)info.y * (size_t)a.scan_stride);
+            const_u64* srow = (const_u64*)(uintptr_t)(a.scan_mask + (size_t)info.z * (size_t)a.scan_stride);
             const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
             const int nblk = (nvt + 63) >> 6;
 #pragma unroll
@@ -1346,7 +1380,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         // The smallest of all the row's waves' values then has at least sel group maxima at or above it.
         __builtin_amdgcn_sched_barrier(0);  // after the stores: the chunk's registers are free by now
         {
-            const int need = (__builtin_amdgcn_readfirstlane(info.z) + S * kWaves - 1) / (S * kWaves);
+            const int need = (info.w + S * kWaves - 1) / (S * kWaves);
             uint32_t K = 0u;
 #pragma unroll 1
             for (int bit = 31; bit >= 16; bit--) {
@@ -1380,6 +1414,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     sr_drain_stores();
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_add(&a.row_done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    SR_PROF(a, 5);
 }
 
 // ---- scan mask ---------------------------------------------------------------------------------------
