@@ -68,10 +68,10 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     if (b->h_scan.empty()) return SR_OK;
     {
         // Dispatch order.  Workgroups are dispatched in grid order, two resident per CU; a round is that many
-        // consecutive workgroups.  A row's tail goes to the head of the round after the one that holds the row's
-        // last chunk: its chunks have at least all been dispatched by then and have usually finished, and tails
-        // that are ready do not queue behind later rows' chunks.  Every entry carries what its workgroup needs
-        // to find its data.
+        // consecutive workgroups.  A row's tail goes to the middle of the round after the one that holds the row's
+        // last chunk: half of that round's workgroups have retired by the time it is dispatched, so its chunks have
+        // usually finished and it does not hold a slot while it waits, yet it does not queue behind all of the
+        // later rows' chunks either.  Every entry carries what its workgroup needs to find its data.
         const int n_sel = (int)b->h_sel_list.size();
         int chunks = 1, chunk_vecs = 0;
         topk_geometry(b->vocab, epv == 8 ? SR_DTYPE_BF16 : SR_DTYPE_F32, n_sel, ctx->cu_count, &chunks, &chunk_vecs);
@@ -95,7 +95,7 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
             } else if (row < n_sel) {
                 push(((uint32_t)c << 24) | (uint32_t)row, row);
                 if (++c == chunks) {
-                    ready_at[(size_t)row] = (pos / round + 1) * round;
+                    ready_at[(size_t)row] = (pos / round + 1) * round + round / 2;
                     c = 0;
                     row++;
                 }

@@ -41,6 +41,10 @@ constexpr int kSortRegs = kSelMax / kThreads;   // sort elements per thread (4)
 constexpr int kHistRegs = kSelMax / kThreads;   // history ids per thread (4)
 constexpr int kBins = 1024;                     // histogram bins of the row tail
 constexpr int kBinsPerLane = kBins / SR_WAVE;
+// Bin b lives at word b + b / kBinsPerLane: the strip of kBinsPerLane bins that a lane scans starts one word
+// further than a multiple of the strip length, so that the 64 lanes of a wave fall on different LDS banks.
+constexpr int kBinsPad = kBins + SR_WAVE + 1;
+__device__ __forceinline__ int bin_word(int b) { return b + b / kBinsPerLane; }
 
 struct TopkSmem {
     uint32_t xa[kSelMax];  // gathered list, then sort exchange (three 32-bit words per element)
@@ -54,9 +58,9 @@ struct TopkSmem {
     uint32_t bcast[16];
     unsigned long long ksum;   // chunk scan: sum of the waves' threshold estimates
     uint32_t btotal;           // chunk scan: elements of the chunk at or above the shared threshold
-    uint32_t bhist[kBins];     // live entries per bin of distance below the maximum
-    uint32_t boff[kBins + 1];  // first list position of every bin
-    uint32_t bfill[kBins];     // entries scattered into the bin so far
+    uint32_t bhist[kBinsPad];  // live entries per bin of distance below the maximum
+    uint32_t boff[kBinsPad];   // first list position of every bin
+    uint32_t bfill[kBinsPad];  // entries scattered into the bin so far
 };
 
 // ---- block-wide radix select over keys produced by a per-thread enumerator -----------------------
@@ -678,7 +682,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         each_key([&](uint32_t k) { lmaxk = k > lmaxk ? k : lmaxk; });
 #pragma unroll
         for (int r = 0; r < kHistRegs; r++) lmaxk = (hraw[r] != 0u && hadj[r] > lmaxk) ? hadj[r] : lmaxk;
-        for (int i = tid; i < kBins; i += kThreads) { sm.bhist[i] = 0u; sm.bfill[i] = 0u; }
+        for (int i = tid; i < kBinsPad; i += kThreads) { sm.bhist[i] = 0u; sm.bfill[i] = 0u; }
         if (tid == 0) sm.bcast[4] = 0u;
         const uint32_t kmaxn = block_max_u32(lmaxk, sm);  // its barriers also publish the cleared histogram
         // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
@@ -694,11 +698,11 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         };
 #pragma unroll
         for (int r = 0; r < kCandRegs; r++)
-            if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.bhist[b], 1u); }
+            if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.bhist[bin_word(b)], 1u); }
 #pragma unroll
         for (int r = 0; r < kHistRegs; r++) {
             const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
-            if (b >= 0) atomicAdd(&sm.bhist[b], 1u);
+            if (b >= 0) atomicAdd(&sm.bhist[bin_word(b)], 1u);
         }
         __syncthreads();
         // every wave reads the histogram: live entries, and the first bin at which the k best are complete
@@ -706,7 +710,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         {
             // lane l owns bins [l * kBinsPerLane, (l + 1) * kBinsPerLane)
             const int lane = sr_lane();
-            const uint32_t* hb = sm.bhist + lane * kBinsPerLane;
+            const uint32_t* hb = sm.bhist + lane * (kBinsPerLane + 1);
             int tot = 0;
 #pragma unroll
             for (int q = 0; q < kBinsPerLane; q++) tot += (int)hb[q];
@@ -722,12 +726,11 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 #pragma unroll
             for (int q = 0; q < kBinsPerLane; q++) {
                 const uint32_t h = hb[q];
-                if (w0) sm.boff[lane * kBinsPerLane + q] = (uint32_t)c;
+                if (w0) sm.boff[lane * (kBinsPerLane + 1) + q] = (uint32_t)c;
                 c += (int)h;
                 if (!found) hm = max(hm, h);  // bins up to and including the one that completes the k best
                 if (!found && c >= need) { bq = lane * kBinsPerLane + q; cq = c; found = true; }
             }
-            if (w0 && lane == SR_WAVE - 1) sm.boff[kBins] = (uint32_t)incl;
             bstar = __shfl(bq, L);
             n_keep = __shfl(cq, L);
             // the fullest kept bin bounds the ranking loop below
@@ -773,7 +776,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 if (r < nr) {
                     const int b = bin_of(kreg[r]);
                     if (b >= 0 && b <= bstar && in_set(r)) {
-                        const int pos = by_bins ? (int)(sm.boff[b] + atomicAdd(&sm.bfill[b], 1u)) : pos_any++;
+                        const int pos = by_bins ? (int)(sm.boff[bin_word(b)] + atomicAdd(&sm.bfill[bin_word(b)], 1u)) : pos_any++;
                         if (pos < kSelMax) {
                             sm.xa[pos] = kreg[r];
                             sm.xb[pos] = kreg[r];
@@ -785,7 +788,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             for (int r = 0; r < kHistRegs; r++) {
                 const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
                 if (b >= 0 && b <= bstar) {
-                    const int pos = by_bins ? (int)(sm.boff[b] + atomicAdd(&sm.bfill[b], 1u)) : pos_any++;
+                    const int pos = by_bins ? (int)(sm.boff[bin_word(b)] + atomicAdd(&sm.bfill[bin_word(b)], 1u)) : pos_any++;
                     if (pos < kSelMax) {
                         sm.xa[pos] = hadj[r];
                         sm.xb[pos] = hraw[r];
@@ -808,7 +811,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             for (int i = tid; i < ms; i += kThreads) {
                 const uint32_t mh = sm.xa[i], mm = sm.xb[i], ml = sm.xc[i];
                 const int b = bin_of(mh);
-                const int p0 = (int)sm.boff[b], p1 = p0 + (int)sm.bhist[b];
+                const int p0 = (int)sm.boff[bin_word(b)], p1 = p0 + (int)sm.bhist[bin_word(b)];
                 int rank = p0;
                 for (int j = p0; j < p1; j++) rank += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
                 if (rank < kk) {
