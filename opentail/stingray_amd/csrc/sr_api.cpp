@@ -432,7 +432,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         SR_HIP(ctx, ctx->gmax.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
         SR_HIP(ctx, ctx->gmax2.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
         SR_HIP(ctx, ctx->gpos.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * sizeof(uint32_t), st));
-        SR_HIP(ctx, ctx->gbound.reserve((size_t)n_sel * a.chunks * (SR_TK_THREADS / 64) * sizeof(uint32_t), st));
+        SR_HIP(ctx, ctx->gbound.reserve((size_t)n_sel * a.chunks * (SR_TK_THREADS / 64) * 2 * sizeof(uint32_t), st));
         SR_HIP(ctx, ctx->row_done.reserve((size_t)std::max(n_sel, 1024) * sizeof(uint32_t), st, true));
         a.rows = b->d_rows.as<SrRow>();
         a.edits = b->d_edits.as<SrEdit>();

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #define SR_WAVE 64
 #define SR_NEG_INF (__uint_as_float(0xff800000u))
@@ -93,47 +94,69 @@ __device__ __forceinline__ void sr_drain_stores() { __builtin_amdgcn_s_waitcnt(0
 __device__ __forceinline__ int sr_lane() { return (int)(threadIdx.x & (SR_WAVE - 1)); }
 __device__ __forceinline__ int sr_wave_id() { return (int)(threadIdx.x >> 6); }
 
+// Wave-wide reductions and the scan move data with DPP inside rows of 16 lanes and with v_readlane across
+// rows: no LDS traffic and no address registers.  Every lane of the wave must be active.
+template <int kCtrl> __device__ __forceinline__ uint32_t sr_dpp_u32(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, 0xf, 0xf, true);
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+template <typename Op> __device__ __forceinline__ uint32_t sr_wave_reduce_u32(uint32_t v, Op op)
+{
+    v = op(v, sr_dpp_u32<kDppXor1>(v));
+    v = op(v, sr_dpp_u32<kDppXor2>(v));
+    v = op(v, sr_dpp_u32<kDppHalfMirror>(v));
+    v = op(v, sr_dpp_u32<kDppMirror>(v));
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return op(op(a, b), op(c, d));
+}
 __device__ __forceinline__ uint32_t sr_wave_max_u32(uint32_t v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) { uint32_t w = __shfl_xor(v, o); v = w > v ? w : v; }
-    return v;
+    return sr_wave_reduce_u32(v, [](uint32_t x, uint32_t y) { return x > y ? x : y; });
 }
 __device__ __forceinline__ uint32_t sr_wave_min_u32(uint32_t v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) { uint32_t w = __shfl_xor(v, o); v = w < v ? w : v; }
-    return v;
+    return sr_wave_reduce_u32(v, [](uint32_t x, uint32_t y) { return x < y ? x : y; });
 }
 __device__ __forceinline__ int sr_wave_sum_i32(int v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
+    return (int)sr_wave_reduce_u32((uint32_t)v, [](uint32_t x, uint32_t y) { return x + y; });
 }
 __device__ __forceinline__ int sr_wave_min_i32(int v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) { int w = __shfl_xor(v, o); v = w < v ? w : v; }
-    return v;
+    return (int)sr_wave_reduce_u32((uint32_t)v, [](uint32_t x, uint32_t y) { return (int)x < (int)y ? x : y; });
 }
 __device__ __forceinline__ unsigned long long sr_wave_max_u64(unsigned long long v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        unsigned long long w = __shfl_xor(v, o);
+    auto step = [&](auto ctrl) {
+        constexpr int kC = decltype(ctrl)::value;
+        const unsigned long long w = ((unsigned long long)sr_dpp_u32<kC>((uint32_t)(v >> 32)) << 32) | sr_dpp_u32<kC>((uint32_t)v);
         v = w > v ? w : v;
+    };
+    step(std::integral_constant<int, kDppXor1>{});
+    step(std::integral_constant<int, kDppXor2>{});
+    step(std::integral_constant<int, kDppHalfMirror>{});
+    step(std::integral_constant<int, kDppMirror>{});
+    unsigned long long r = 0ull;
+#pragma unroll
+    for (int l = 0; l < SR_WAVE; l += 16) {
+        const unsigned long long w = ((unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), l) << 32) |
+                                     (unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, l);
+        r = w > r ? w : r;
     }
-    return v;
+    return r;
 }
 // inclusive prefix sum across the wave
 __device__ __forceinline__ int sr_wave_incl_scan_i32(int v)
 {
-    const int lane = sr_lane();
-#pragma unroll
-    for (int o = 1; o < SR_WAVE; o <<= 1) {
-        int w = __shfl_up(v, o);
-        if (lane >= o) v += w;
-    }
-    return v;
+    // inside every row of 16 lanes: shifts by 1, 2, 4, 8 with zero fill
+    v += (int)sr_dpp_u32<0x111>((uint32_t)v);
+    v += (int)sr_dpp_u32<0x112>((uint32_t)v);
+    v += (int)sr_dpp_u32<0x114>((uint32_t)v);
+    v += (int)sr_dpp_u32<0x118>((uint32_t)v);
+    // the rows before this lane's
+    const int r0 = __builtin_amdgcn_readlane(v, 15), r1 = __builtin_amdgcn_readlane(v, 31), r2 = __builtin_amdgcn_readlane(v, 47);
+    const int row = sr_lane() >> 4;
+    return v + (row >= 1 ? r0 : 0) + (row >= 2 ? r1 : 0) + (row >= 3 ? r2 : 0);
 }

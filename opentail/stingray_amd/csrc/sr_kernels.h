@@ -36,7 +36,8 @@ struct SrTopkArgs {
     float4* gmax;            // [n_rows][chunks][SR_TK_THREADS]: the four group maxima of every thread of every chunk
     float4* gmax2;           // ... the second largest element of each of those groups
     uint32_t* gpos;          // ... the position of the largest inside its group, 8 bits per group
-    uint32_t* gbound;        // [n_rows][chunks][waves]: every chunk wave's share of the row's bound (an ordered key)
+    uint32_t* gbound;        // [n_rows][chunks][waves][2]: every chunk wave's share of the row's bound and its largest kept
+                             // element (ordered keys)
     unsigned long long* cand; // [n_rows][SR_TK_ROW_CAP] (value bits << 32 | index), built by the row's tail
     uint32_t* row_done;      // [n_rows], zero on entry, left zero on exit
     const double* uniforms;

@@ -428,8 +428,13 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     float hx[kHistRegs];
 #pragma unroll
     for (int r = 0; r < kHistRegs; r++) { hee[r] = SrEdit{}; hx[r] = SR_NEG_INF; }
+    const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
+    // rows without penalties that may raise a logit have their candidates binned while they are collected
+    const bool want_bins = rd.path == SR_PATH_TOPK && (!use_edits || hist_regs);
+    bool binned = false;
+    float mx0 = 0.0f;
     const int n_c = build_candidates<EPV, kVec>(
-        a, slot, row, rd,
+        a, slot, row, rd, want_bins, inv_temp, &mx0, &binned,
         [&]() SR_INL {
 #pragma unroll
             for (int r = 0; r < kHistRegs; r++) {
@@ -451,24 +456,27 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     const int nr = (n_c + kThreads - 1) / kThreads;  // register slots that can hold a candidate
     uint32_t kreg[kCandRegs];                         // 0 = no candidate in this slot
     int kid[kCandRegs];
+    auto load_cands = [&]() SR_INL {
 #pragma unroll
-    for (int r = 0; r < kCandRegs; r++) {
-        kreg[r] = 0u;
-        kid[r] = 0;
-        if (r >= nr) continue;
-        const int g = r * kThreads + tid;
-        if (g < n_c) {
-            if (g < kSelMax) {  // the first candidates lie in LDS, only an unusually long list continues in memory
-                kreg[r] = sr_okey(sm.vals[g]);
-                kid[r] = sm.idxs[g];
-            } else {
-                const unsigned long long cv = sr_load_agent(&cand[g]);
-                kreg[r] = sr_okey(sr_u2f((uint32_t)(cv >> 32)));
-                kid[r] = (int)(uint32_t)cv;
+        for (int r = 0; r < kCandRegs; r++) {
+            kreg[r] = 0u;
+            kid[r] = 0;
+            if (r >= nr) continue;
+            const int g = r * kThreads + tid;
+            if (g < n_c) {
+                if (g < kSelMax) {  // the first candidates lie in LDS, only an unusually long list continues in memory
+                    kreg[r] = sr_okey(sm.vals[g]);
+                    kid[r] = sm.idxs[g];
+                } else {
+                    const unsigned long long cv = sr_load_agent(&cand[g]);
+                    kreg[r] = sr_okey(sr_u2f((uint32_t)(cv >> 32)));
+                    kid[r] = (int)(uint32_t)cv;
+                }
             }
         }
-    }
-    __syncthreads();  // sm.vals / sm.idxs may be reused from here on
+        __syncthreads();  // sm.vals / sm.idxs may be reused from here on
+    };
+    if (!binned) load_cands();  // binned candidates stay in their list until they are laid out by bins
     auto cand_id = [&](int r) SR_INL -> int { return kid[r]; };
     SR_PROF(a, 12);
     auto each_key = [&](auto&& body) SR_INL {
@@ -550,8 +558,8 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         return (0xffffffffu - (uint32_t)cand_id(r)) >= tidx_key;
     };
 
-    const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
     float mx;
+    float mx_bins = 0.0f;  // what the bins are measured from: mx, or the largest kept element outside the history
     // Candidates whose e = expf(v / T - max) is below 2^-26 are dropped before the sort: with e_0 = 1
     // they change neither running sum (they are under half an ulp of a sum >= 1, and of a cumulative
     // probability >= probs[0]) and the draw can never stop on them, so the result is bit-identical.
@@ -566,6 +574,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     int m2;          // live entries (at most top_k of them are used)
     int sort_n = 0;  // entries handed to the sort
     bool ranked = false;  // sm.vals / sm.idxs already hold the k first entries
+    bool placed = false;  // ... laid out from the binned candidate list: the maximum is the first ranked entry
 
     if (use_edits && !excl) {
         // ---- penalties that may raise a logit: the reference's literal top-(k + history length) set ------
@@ -678,36 +687,18 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             }
         }
         SR_PROF(a, 5);
-        uint32_t lmaxk = 0u;
-        each_key([&](uint32_t k) { lmaxk = k > lmaxk ? k : lmaxk; });
-#pragma unroll
-        for (int r = 0; r < kHistRegs; r++) lmaxk = (hraw[r] != 0u && hadj[r] > lmaxk) ? hadj[r] : lmaxk;
-        for (int i = tid; i < kBinsPad; i += kThreads) { sm.bhist[i] = 0u; sm.bfill[i] = 0u; }
-        if (tid == 0) sm.bcast[4] = 0u;
-        const uint32_t kmaxn = block_max_u32(lmaxk, sm);  // its barriers also publish the cleared histogram
-        // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
-        if (kmaxn == 0u) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
-        mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
-        // How far an entry lies below the maximum, in 1/56 of a log-unit: -1 = absent or dead, else 0..1023.
-        // Monotone in the key, so "bin <= b" is a prefix of the descending order.
+        // How far an entry lies below the bins' origin, in 1/56 of a log-unit: -1 = absent or dropped, else
+        // 0..1023.  Never increasing with the key, so "bin <= b" is a prefix of the descending order.
         auto bin_of = [&](uint32_t key) SR_INL -> int {
             if (key == 0u) return -1;
-            const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx);
+            const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx_bins);
             if (x < -18.1f) return -1;
             return min(max((int)__fmul_rn(x, -56.0f), 0), kBins - 1);
         };
-#pragma unroll
-        for (int r = 0; r < kCandRegs; r++)
-            if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.bhist[bin_word(b)], 1u); }
-#pragma unroll
-        for (int r = 0; r < kHistRegs; r++) {
-            const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
-            if (b >= 0) atomicAdd(&sm.bhist[bin_word(b)], 1u);
-        }
-        __syncthreads();
-        // every wave reads the histogram: live entries, and the first bin at which the k best are complete
-        int bstar = kBins - 1, n_live, n_keep, max_bin;
-        {
+        int bstar = kBins - 1, n_live = 0, n_keep = 0, max_bin = 0;
+        // every wave reads the histogram: live entries, and the first bin at which the k best are complete;
+        // wave 0 leaves every bin's first list position in sm.boff
+        auto scan_bins = [&]() SR_INL {
             // lane l owns bins [l * kBinsPerLane, (l + 1) * kBinsPerLane)
             const int lane = sr_lane();
             const uint32_t* hb = sm.bhist + lane * (kBinsPerLane + 1);
@@ -736,9 +727,74 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             // the fullest kept bin bounds the ranking loop below
             if (lane > L) hm = 0u;
             max_bin = (int)sr_wave_max_u32(hm);
-        }
-        m2 = n_live;
+        };
         bool by_bins = true;  // kept entries are laid out bin by bin and ranked inside their bin
+        if (binned) {
+            // The candidates were counted into the histogram as they were collected; the history ids join them.
+            mx_bins = mx0;
+            uint32_t hmeta[kHistRegs];
+#pragma unroll
+            for (int r = 0; r < kHistRegs; r++) {
+                const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
+                hmeta[r] = b >= 0 ? (((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u)) : 0xffffffffu;
+            }
+            __syncthreads();
+            scan_bins();
+            // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
+            if (n_live == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
+            __syncthreads();  // sm.boff written, every wave done with the histogram
+            SR_PROF(a, 6);
+            if (n_keep <= kSelMax && max_bin <= 96) {
+                const uint32_t* meta = (const uint32_t*)sm.probs;
+                for (int i = tid; i < n_c; i += kThreads) {
+                    const uint32_t mt = meta[i];
+                    const int b = (int)(mt >> 16);
+                    if (b <= bstar) {
+                        const int pos = (int)(sm.boff[bin_word(b)] + (mt & 0xffffu));
+                        const uint32_t key = sr_okey(sm.vals[i]);
+                        sm.xa[pos] = key;
+                        sm.xb[pos] = key;
+                        sm.xc[pos] = 0xffffffffu - (uint32_t)sm.idxs[i];
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < kHistRegs; r++) {
+                    const int b = (int)(hmeta[r] >> 16);
+                    if (hmeta[r] != 0xffffffffu && b <= bstar) {
+                        const int pos = (int)(sm.boff[bin_word(b)] + (hmeta[r] & 0xffffu));
+                        sm.xa[pos] = hadj[r];
+                        sm.xb[pos] = hraw[r];
+                        sm.xc[pos] = 0xffffffffu - (uint32_t)hee[r].id;
+                    }
+                }
+                __syncthreads();
+                placed = true;
+            } else {
+                load_cands();  // a flat or heavily tied row: the general way below
+            }
+        }
+        if (!placed) {
+        uint32_t lmaxk = 0u;
+        each_key([&](uint32_t k) { lmaxk = k > lmaxk ? k : lmaxk; });
+#pragma unroll
+        for (int r = 0; r < kHistRegs; r++) lmaxk = (hraw[r] != 0u && hadj[r] > lmaxk) ? hadj[r] : lmaxk;
+        for (int i = tid; i < kBinsPad; i += kThreads) { sm.bhist[i] = 0u; sm.bfill[i] = 0u; }
+        if (tid == 0) sm.bcast[4] = 0u;
+        const uint32_t kmaxn = block_max_u32(lmaxk, sm);  // its barriers also publish the cleared histogram
+        // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
+        if (kmaxn == 0u) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
+        mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
+        mx_bins = mx;
+#pragma unroll
+        for (int r = 0; r < kCandRegs; r++)
+            if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.bhist[bin_word(b)], 1u); }
+#pragma unroll
+        for (int r = 0; r < kHistRegs; r++) {
+            const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
+            if (b >= 0) atomicAdd(&sm.bhist[bin_word(b)], 1u);
+        }
+        __syncthreads();
+        scan_bins();
         if (n_keep > kSelMax) {
             // a flat row: only the k best candidates outside the history can matter
             by_bins = false;
@@ -798,6 +854,8 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             }
         }
         __syncthreads();
+        }  // !placed
+        m2 = n_live;
         const int ms = by_bins ? min(n_keep, kSelMax) : min((int)sm.bcast[4], kSelMax);
         // the first min(top_k, live) of the kept entries are the first of all live entries
         m2 = min(min(m2, max(rd.top_k, 0)), ms);
@@ -855,6 +913,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         }
     }
     __syncthreads();
+    if (placed) mx = __fmul_rn(sm.vals[0], inv_temp);
     SR_PROF(a, 8);
 
     // Sampler.cs:297-313: e_t = expf(v_t / T - max), sequential fp32 sum, probs = e * (1 / sum)
@@ -950,10 +1009,18 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 // SR_TK_SEL_MAX in sm.vals / sm.idxs, the rest of an unusually long list in a.cand.  Returns the number of
 // candidates, or -1 when the row cannot be handled.  Called by every thread of the tail workgroup; the two
 // hooks let the caller issue loads of its own behind the group maxima's (early) and after the first wait (late).
+// With want_bins the candidates are also counted into the tail's histogram of distances below the row's largest
+// kept element (sm.bhist, bins of 1/56 in units of the temperature; entries more than 18.1 below it are dropped on
+// the spot), and every candidate remembers its bin and its arrival number inside the bin (sm.probs, as integers):
+// the tail can then lay the candidates out bin by bin without another pass of atomics.  *binned tells whether
+// that happened (few chunks, a short enough list, a finite maximum); *mx0 is the maximum times inv_temp.
 template <int EPV, int kVec, typename Early, typename Late>
-__device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, Early&& early,
-                                                Late&& late, TopkSmem& sm)
+__device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
+                                                float inv_temp, float* mx0_out, bool* binned, Early&& early, Late&& late,
+                                                TopkSmem& sm)
 {
+    *binned = false;
+    *mx0_out = 0.0f;
     using VO = VecOps<EPV>;
     constexpr int ES = (EPV == 4) ? 4 : 2;
     constexpr int kGV = (kVec + SR_TK_GROUPS - 1) / SR_TK_GROUPS;  // vectors per group
@@ -1034,12 +1101,27 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         base = __shfl(base, (int)__ffsll((long long)bal) - 1);
         return want ? (int)(base + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))) : -1;
     };
+    bool bins = false;
+    float mx0 = 0.0f;
+    uint32_t* meta = (uint32_t*)sm.probs;
+    // the bin of a value: -1 = dropped, else 0 .. kBins - 1, never increasing with the value
+    auto bin0 = [&](float x) SR_INL -> int {
+        const float d = __fsub_rn(__fmul_rn(x, inv_temp), mx0);
+        if (d < -18.1f) return -1;
+        return min(max((int)__fmul_rn(d, -56.0f), 0), kBins - 1);
+    };
     auto append = [&](bool want, float x, int idx) SR_INL {
+        int b = 0;
+        if (bins) {
+            b = bin0(x);
+            want = want && b >= 0;
+        }
         const int pos = wave_slot(want, &sm.bcast[12]);
         if (pos >= 0) {
             if (pos < kSelMax) {
                 sm.vals[pos] = x;
                 sm.idxs[pos] = idx;
+                if (bins) meta[pos] = ((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u);
             } else if (pos < kRowCap) {
                 sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx);
             }
@@ -1094,6 +1176,8 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     };
 
     if (tid == 0) { sm.bcast[12] = 0u; sm.bcast[13] = 0u; }
+    if (want_bins)
+        for (int i = tid; i < kBinsPad; i += kThreads) sm.bhist[i] = 0u;
     __syncthreads();
     if (sel > kSelMax || sel < 1) return -1;
     // The chunk workgroups' waves each left a value with their share of sel group maxima at or above it: the
@@ -1101,10 +1185,27 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     float tval = -3.402823466e38f;
     {
         const int nb = S * kWaves;
-        uint32_t k = 0xffffffffu;
-        for (int i = lane; i < nb; i += SR_WAVE) k = min(k, a.gbound[(size_t)slot * nb + i]);
+        uint32_t k = 0xffffffffu, km = 0u;
+        const uint2* gb = (const uint2*)a.gbound + (size_t)slot * nb;
+        for (int i = lane; i < nb; i += SR_WAVE) {
+            const uint2 b = gb[i];
+            k = min(k, b.x);
+            km = max(km, b.y);
+        }
         k = sr_wave_min_u32(k);
+        km = sr_wave_max_u32(km);
         if (k > kKeyNegInf) tval = sr_okey_inv(k);
+        // An element 19 T below the row's largest kept element has expf((v - max) / T) < 2^-26 whatever else
+        // joins the row (penalties that only lower cannot raise the maximum's rivals above it, and the maximum of
+        // the final set is at least this one): the row tail drops such entries anyway, so they need not become
+        // candidates.  Rows whose penalties may raise a logit keep the plain bound.
+        const bool lowering_only = (rd.flags & kRowHasPenalty) == 0u || rd.edit_cnt <= 0 || (rd.flags & kRowHistExcl) != 0u;
+        if (rd.path == SR_PATH_TOPK && lowering_only && km > kKeyNegInf && rd.temperature > 0.0f) {
+            const float tdead = __fsub_rn(sr_okey_inv(km), __fmul_rn(19.0f, rd.temperature));
+            tval = fmaxf(tval, tdead);
+        }
+        bins = want_bins && direct && km > kKeyNegInf;
+        mx0 = __fmul_rn(sr_okey_inv(km), inv_temp);
     }
     late();
     SR_PROF(a, 1);
@@ -1120,7 +1221,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     n_list += __popcll(__ballot(m2[g] >= tval));
-                    n_app += __popcll(__ballot(m1[g] >= tval && !(m2[g] >= tval)));
+                    n_app += __popcll(__ballot(m1[g] >= tval && !(m2[g] >= tval) && (!bins || bin0(m1[g]) >= 0)));
                 }
             }
         }
@@ -1138,7 +1239,8 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                 const float m2[4] = {g2r[c].x, g2r[c].y, g2r[c].z, g2r[c].w};
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const bool q2 = m2[g] >= tval, q1 = m1[g] >= tval && !q2;
+                    const int bn = bins ? bin0(m1[g]) : 0;
+                    const bool q2 = m2[g] >= tval, q1 = m1[g] >= tval && !q2 && bn >= 0;
                     const unsigned long long b2 = __ballot(q2), b1 = __ballot(q1);
                     if (q2) {  // may hold more than one: fetched below
                         const uint32_t pos = base_l + __builtin_amdgcn_mbcnt_hi((uint32_t)(b2 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b2, 0u));
@@ -1150,6 +1252,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                         if (pos < (uint32_t)kSelMax) {
                             sm.vals[pos] = m1[g];
                             sm.idxs[pos] = idx;
+                            if (bins) meta[pos] = ((uint32_t)bn << 16) | atomicAdd(&sm.bhist[bin_word(bn)], 1u);
                         } else if (pos < (uint32_t)kRowCap) {
                             sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(m1[g]) << 32) | (unsigned long long)(uint32_t)idx);
                         }
@@ -1170,10 +1273,13 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     __syncthreads();
     const int n_q = (int)sm.bcast[13];
     SR_PROF(a, 2);
+    bool listed = false;
     if (n_q <= kQCap) {
         SR_PROF(a, 3);
         gather(n_q, [&](bool kept, float x, int idx) { append(kept && x >= tval, x, idx); });
+        listed = true;
     } else {
+        bins = false;  // the exact bound below starts the list again
         // Too many groups at or above the bound: the row is flat or heavily tied (or has too many chunks for the
         // per-wave bound).  Exact bound instead: the sel-th largest group maximum; every element above it lies in a
         // group whose maximum is above it (fewer than sel groups); of the elements equal to it only the first few by
@@ -1230,6 +1336,8 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     __syncthreads();
     const uint32_t n_c = sm.bcast[12];
     __syncthreads();
+    *binned = bins && listed && n_c <= (uint32_t)kSelMax;
+    *mx0_out = mx0;
     return n_c > (uint32_t)kRowCap ? -1 : (int)n_c;
 }
 
@@ -1242,9 +1350,10 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     const int tid = threadIdx.x, lane = sr_lane();
     const int S = a.chunks;
     // The host lays the workgroups out in dispatch order: chunk workgroups row by row, and the tail of a row
-    // one full round of resident workgroups after the row's last chunk, so that a tail is dispatched after all
-    // chunk workgroups of its row (it waits, bounded, only on work that is already running) and rarely waits.
-    // read through the constant address space (the host wrote it before the launch): one scalar 16-byte load
+    // about a round and a half of resident workgroups after the row's last chunk, so that a tail is dispatched
+    // after all chunk workgroups of its row (it waits, bounded, only on work that is already running) and
+    // rarely waits.  The entry is read through the constant address space (the host wrote it before the
+    // launch): one scalar 16-byte load.
     typedef int __attribute__((ext_vector_type(4))) i32x4;
     typedef const i32x4 __attribute__((address_space(4))) const_i32x4;
     const i32x4 info = ((const_i32x4*)(uintptr_t)a.sched)[blockIdx.x];  // (item, row, scan-mask row, sel)
@@ -1277,6 +1386,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             return;
         }
         SR_PROF(a, 4);
+        __builtin_amdgcn_s_setprio(3);  // the tail is the longer dependent chain: its waves go first
         topk_row_tail<EPV, kVec>(a, tslot, trow, trd, sm);
         SR_PROF(a, 15);
         return;
@@ -1393,7 +1503,13 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                                 __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc));
                 if (cge >= need) K = cnd;
             }
-            if (lane == 0) __hip_atomic_store(a.gbound + ((size_t)slot * S + c) * kWaves + (tid >> 6), K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // ... and the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
+            const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(gm1[0], gm1[1]), fmaxf(gm1[2], gm1[3]))));
+            if (lane == 0) {
+                uint32_t* gb = a.gbound + (((size_t)slot * S + c) * kWaves + (tid >> 6)) * 2;
+                __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(gb + 1, wmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     } else {
         float4* gout = a.gmax + ((size_t)slot * S + c) * kThreads + tid;
@@ -1407,7 +1523,11 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         __hip_atomic_store(&gout2->z, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&gout2->w, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(a.gpos + ((size_t)slot * S + c) * kThreads + tid, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (lane == 0) __hip_atomic_store(a.gbound + ((size_t)slot * S + c) * kWaves + (tid >> 6), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) {
+            uint32_t* gb = a.gbound + (((size_t)slot * S + c) * kWaves + (tid >> 6)) * 2;
+            __hip_atomic_store(gb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(gb + 1, kKeyNegInf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     SR_PROF(a, 3);
     if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 0] = pt0; a.prof[(size_t)blockIdx.x * 16 + 1] = pt1; a.prof[(size_t)blockIdx.x * 16 + 2] = pt2; }
