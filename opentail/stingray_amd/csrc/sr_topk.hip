@@ -1478,15 +1478,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         if (a.prof) pt2 = wall_clock64();
         const size_t go = ((size_t)slot * S + c) * kThreads + tid;
         float4* gout = a.gmax + go;
-        __hip_atomic_store(&gout->x, gm1[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout->y, gm1[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout->z, gm1[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout->w, gm1[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        float4* gout2 = a.gmax2 + go;
-        __hip_atomic_store(&gout2->x, gm2[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout2->y, gm2[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout2->z, gm2[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout2->w, gm2[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sr_store_agent_f4(gout, gm1[0], gm1[1], gm1[2], gm1[3]);
+        sr_store_agent_f4(a.gmax2 + go, gm2[0], gm2[1], gm2[2], gm2[3]);
         __hip_atomic_store(a.gpos + go, gpk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // The wave's share of the row's bound: a value, to 16 bits and rounded down, with at least
         // ceil(sel / (chunks x 8)) of the wave's 256 group maxima at or above it (found bit by bit with ballots).
@@ -1513,15 +1506,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         }
     } else {
         float4* gout = a.gmax + ((size_t)slot * S + c) * kThreads + tid;
-        __hip_atomic_store(&gout->x, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout->y, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout->z, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout->w, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        float4* gout2 = a.gmax2 + ((size_t)slot * S + c) * kThreads + tid;
-        __hip_atomic_store(&gout2->x, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout2->y, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout2->z, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&gout2->w, SR_NEG_INF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sr_store_agent_f4(gout, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+        sr_store_agent_f4(a.gmax2 + ((size_t)slot * S + c) * kThreads + tid, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
         __hip_atomic_store(a.gpos + ((size_t)slot * S + c) * kThreads + tid, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (lane == 0) {
             uint32_t* gb = a.gbound + (((size_t)slot * S + c) * kWaves + (tid >> 6)) * 2;
