@@ -299,3 +299,38 @@ def test_history_on_unaligned_rows_and_bf16(ctx):
     _check_rows(ctx, up, params, rng.random(rows), _cuda(bits.view(np.int16), torch.bfloat16))
     w = synthetic.config3(rows=32, bf16=True, full_chain=True)
     _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits_bf16.view(np.int16), torch.bfloat16))
+
+
+def test_vocabularies_of_more_than_four_chunks_per_row(ctx):
+    # beyond 155,648 fp32 (327,680 bf16) elements a row takes more than four chunk workgroups and the row tail
+    # works from the group maxima alone: histories, masks, boosts, greedy rows, ties
+    import torch
+
+    rng = np.random.default_rng(35)
+    V, rows = 262_144, 8
+    logits = rng.normal(0, 1.5, (rows, V)).astype(np.float32)
+    logits[6] = np.round(logits[6] * 2) / 2               # heavily tied
+    logits[7] = 0.5                                       # flat
+    head = np.argsort(-logits, axis=1)
+    ks = [1, 40, 64, 500, 1000, 1, 300, 50]
+    params = []
+    for i, k in enumerate(ks):
+        hist = np.concatenate([head[i, :20], rng.integers(0, V, 44)]).tolist()
+        params.append(SamplingParams(Temperature=0.0 if i == 5 else float(rng.uniform(0.6, 1.4)), TopK=k,
+                                     TopP=float(rng.choice([1.0, 0.9])), MinP=float(rng.choice([0.0, 0.02])),
+                                     RepetitionPenalty=1.1, PresencePenalty=0.1 if i != 3 else -0.4,
+                                     PreviousTokens=hist if i != 0 else []))
+    allowed = np.stack([synthetic.run_mask(rng, V, d) for d in (0.5, 0.9, 0.3, 0.6, 0.8, 0.6, 0.7, 0.2)])
+    mask = pack_allow_mask(allowed)
+    for _ in range(2):
+        _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits))
+    _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits), mask, np.array([1, 0, 1, 1, 1, 1, 0, 1], dtype=np.uint8))
+    Vb = 400_003                                          # bf16, unaligned rows, 10 chunks
+    lb = rng.normal(0, 1.5, (4, Vb)).astype(np.float32)
+    bits = synthetic.to_bf16_bits(lb)
+    up = synthetic.bf16_bits_to_f32(bits)
+    hb = np.argsort(-up, axis=1)
+    pb = [SamplingParams(Temperature=0.9 if i != 1 else 0.0, TopK=k, TopP=0.95, RepetitionPenalty=1.2,
+                         PreviousTokens=hb[i, :25].tolist() + rng.integers(0, Vb, 30).tolist())
+          for i, k in enumerate([5, 1, 200, 900])]
+    _check_rows(ctx, up, pb, rng.random(4), _cuda(bits.view(np.int16), torch.bfloat16))
