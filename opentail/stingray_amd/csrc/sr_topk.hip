@@ -695,6 +695,11 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             if (x < -18.1f) return -1;
             return min(max((int)__fmul_rn(x, -56.0f), 0), kBins - 1);
         };
+        // the bin of an entry that was kept (binned candidates are never dropped once they are on the list)
+        auto bin_kept = [&](uint32_t key) SR_INL -> int {
+            const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx_bins);
+            return min(max((int)__fmul_rn(x, -56.0f), 0), kBins - 1);
+        };
         int bstar = kBins - 1, n_live = 0, n_keep = 0, max_bin = 0;
         // every wave reads the histogram: live entries, and the first bin at which the k best are complete;
         // wave 0 leaves every bin's first list position in sm.boff
@@ -868,7 +873,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             const int kk = min(rd.top_k, m2);
             for (int i = tid; i < ms; i += kThreads) {
                 const uint32_t mh = sm.xa[i], mm = sm.xb[i], ml = sm.xc[i];
-                const int b = bin_of(mh);
+                const int b = bin_kept(mh);
                 const int p0 = (int)sm.boff[bin_word(b)], p1 = p0 + (int)sm.bhist[bin_word(b)];
                 int rank = p0;
                 for (int j = p0; j < p1; j++) rank += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
@@ -1104,24 +1109,40 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     bool bins = false;
     float mx0 = 0.0f;
     uint32_t* meta = (uint32_t*)sm.probs;
-    // the bin of a value: -1 = dropped, else 0 .. kBins - 1, never increasing with the value
+    // the bin of a candidate: 0 .. kBins - 1, never increasing with the value (what lies too far below the maximum
+    // to matter never gets here: the bound is at least the maximum minus 18 T, see below)
     auto bin0 = [&](float x) SR_INL -> int {
         const float d = __fsub_rn(__fmul_rn(x, inv_temp), mx0);
-        if (d < -18.1f) return -1;
         return min(max((int)__fmul_rn(d, -56.0f), 0), kBins - 1);
     };
-    auto append = [&](bool want, float x, int idx) SR_INL {
-        int b = 0;
-        if (bins) {
-            b = bin0(x);
-            want = want && b >= 0;
+    // one candidate at list position pos
+    auto place = [&](uint32_t pos, float x, int idx) SR_INL {
+        if (pos < (uint32_t)kSelMax) {
+            sm.vals[pos] = x;
+            sm.idxs[pos] = idx;
+            if (bins) {
+                const int b = bin0(x);
+                meta[pos] = ((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u);
+            }
+        } else if (pos < (uint32_t)kRowCap) {
+            sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx);
         }
+    };
+    // Every lane brings n_own entries for a list: one atomic per wave reserves the wave's slice, the lane's own
+    // slice starts at the returned position.  All lanes of the wave call this.
+    auto wave_reserve = [&](int n_own, uint32_t* counter) SR_INL -> uint32_t {
+        const int incl = sr_wave_incl_scan_i32(n_own);
+        const int total = __builtin_amdgcn_readlane(incl, SR_WAVE - 1);
+        uint32_t base = 0u;
+        if (total > 0 && lane == 0) base = atomicAdd(counter, (uint32_t)total);
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)base) + (uint32_t)(incl - n_own);
+    };
+    auto append = [&](bool want, float x, int idx) SR_INL {
         const int pos = wave_slot(want, &sm.bcast[12]);
         if (pos >= 0) {
             if (pos < kSelMax) {
                 sm.vals[pos] = x;
                 sm.idxs[pos] = idx;
-                if (bins) meta[pos] = ((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u);
             } else if (pos < kRowCap) {
                 sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx);
             }
@@ -1132,8 +1153,8 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         if (pos >= 0 && pos < kQCap) qlist[pos] = ((uint32_t)(c * kThreads + tid) << 2) | (uint32_t)g;
     };
     // fetches the listed groups, kBatch (group, vector) items per thread at a time -- values and the keep-bit halves
-    // of all of them in one batch of loads -- and hands every kept element to f(value, index)
-    auto gather = [&](int nq, auto&& f) SR_INL {
+    // of all of them in one batch of loads -- and appends every kept element that pred admits to the candidates
+    auto gather = [&](int nq, auto&& pred) SR_INL {
         const int n_items = nq * kGV;
         for (int i0 = 0; i0 < n_items; i0 += kBatch * kThreads) {
             u32x4 v[kBatch];
@@ -1146,7 +1167,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                 v[r] = VO::neg_inf();
 #pragma unroll
                 for (int q = 0; q < EPV; q++) kw[r][q] = 0u;
-                if (i < n_items) {
+                if (i0 + r * kThreads < n_items && i < n_items) {  // the first test is uniform: unused slots cost nothing
                     const uint32_t gid = qlist[i / kGV];
                     const int m = i - (i / kGV) * kGV;
                     const int g = (int)(gid & 3u), t = (int)((gid >> 2) & (kThreads - 1)), c = (int)(gid >> 11);
@@ -1166,11 +1187,17 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
             }
 #pragma unroll
             for (int r = 0; r < kBatch; r++) {
+                if (i0 + r * kThreads >= n_items) continue;  // uniform
+                uint32_t own = 0u;
 #pragma unroll
                 for (int q = 0; q < EPV; q++) {
                     const bool kept = fvs[r] >= 0 && ((kw[r][q] >> (fvs[r] & 31)) & 1u) != 0u;
-                    f(kept, VO::get(v[r], q), fvs[r] * EPV + q - mis);
+                    own |= (kept && pred(VO::get(v[r], q))) ? (1u << q) : 0u;
                 }
+                uint32_t pos = wave_reserve(__popc(own), &sm.bcast[12]);
+#pragma unroll
+                for (int q = 0; q < EPV; q++)
+                    if ((own >> q) & 1u) place(pos++, VO::get(v[r], q), fvs[r] * EPV + q - mis);
             }
         }
     };
@@ -1197,8 +1224,8 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         if (k > kKeyNegInf) tval = sr_okey_inv(k);
         // An element 19 T below the row's largest kept element has expf((v - max) / T) < 2^-26 whatever else
         // joins the row (penalties that only lower cannot raise the maximum's rivals above it, and the maximum of
-        // the final set is at least this one): the row tail drops such entries anyway, so they need not become
-        // candidates.  Rows whose penalties may raise a logit keep the plain bound.
+        // the final set is at least this one): such entries change neither running sum nor can the draw stop on
+        // them, so they need not become candidates.  Rows whose penalties may raise a logit keep the plain bound.
         const bool lowering_only = (rd.flags & kRowHasPenalty) == 0u || rd.edit_cnt <= 0 || (rd.flags & kRowHistExcl) != 0u;
         if (rd.path == SR_PATH_TOPK && lowering_only && km > kKeyNegInf && rd.temperature > 0.0f) {
             const float tdead = __fsub_rn(sr_okey_inv(km), __fmul_rn(19.0f, rd.temperature));
@@ -1210,9 +1237,10 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     late();
     SR_PROF(a, 1);
     if (direct) {
-        // two passes over the 16 groups of the thread: count per wave (ballots, scalar), reserve both lists' slices
-        // with one atomic each, then place
-        int n_list = 0, n_app = 0;
+        // The thread's 16 groups as two bit masks -- largest element at or above the bound with the second largest
+        // below it (handed over directly), second largest at or above it (listed, fetched below) --, one
+        // reservation per wave and list, then every lane places its own.
+        uint32_t mq1 = 0u, mq2 = 0u;
 #pragma unroll
         for (int c = 0; c < kG2Regs; c++) {
             if (c < S) {
@@ -1220,45 +1248,36 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                 const float m2[4] = {g2r[c].x, g2r[c].y, g2r[c].z, g2r[c].w};
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    n_list += __popcll(__ballot(m2[g] >= tval));
-                    n_app += __popcll(__ballot(m1[g] >= tval && !(m2[g] >= tval) && (!bins || bin0(m1[g]) >= 0)));
+                    const bool q2 = m2[g] >= tval, q1 = m1[g] >= tval && !q2;
+                    mq2 |= q2 ? (1u << (c * 4 + g)) : 0u;
+                    mq1 |= q1 ? (1u << (c * 4 + g)) : 0u;
                 }
             }
         }
-        uint32_t base_l = 0u, base_a = 0u;
+        // both counts in one scan: at most 16 per lane, 1,024 per wave
+        const int n_own = __popc(mq1) | (__popc(mq2) << 16);
+        const int incl = sr_wave_incl_scan_i32(n_own);
+        const int total = __builtin_amdgcn_readlane(incl, SR_WAVE - 1);
+        uint32_t base_a = 0u, base_l = 0u;
         if (lane == 0) {
-            if (n_list > 0) base_l = atomicAdd(&sm.bcast[13], (uint32_t)n_list);
-            if (n_app > 0) base_a = atomicAdd(&sm.bcast[12], (uint32_t)n_app);
+            if ((total & 0xffff) > 0) base_a = atomicAdd(&sm.bcast[12], (uint32_t)(total & 0xffff));
+            if ((total >> 16) > 0) base_l = atomicAdd(&sm.bcast[13], (uint32_t)(total >> 16));
         }
-        base_l = __builtin_amdgcn_readfirstlane(base_l);
-        base_a = __builtin_amdgcn_readfirstlane(base_a);
+        base_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)base_a) + (uint32_t)((incl - n_own) & 0xffff);
+        base_l = (uint32_t)__builtin_amdgcn_readfirstlane((int)base_l) + (uint32_t)((incl - n_own) >> 16);
 #pragma unroll
         for (int c = 0; c < kG2Regs; c++) {
             if (c < S) {
                 const float m1[4] = {gmr[c].x, gmr[c].y, gmr[c].z, gmr[c].w};
-                const float m2[4] = {g2r[c].x, g2r[c].y, g2r[c].z, g2r[c].w};
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const int bn = bins ? bin0(m1[g]) : 0;
-                    const bool q2 = m2[g] >= tval, q1 = m1[g] >= tval && !q2 && bn >= 0;
-                    const unsigned long long b2 = __ballot(q2), b1 = __ballot(q1);
-                    if (q2) {  // may hold more than one: fetched below
-                        const uint32_t pos = base_l + __builtin_amdgcn_mbcnt_hi((uint32_t)(b2 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b2, 0u));
+                    const uint32_t bit = 1u << (c * 4 + g);
+                    if (mq2 & bit) {  // may hold more than one: fetched below
+                        const uint32_t pos = base_l + (uint32_t)__popc(mq2 & (bit - 1u));
                         if (pos < (uint32_t)kQCap) qlist[pos] = ((uint32_t)(c * kThreads + tid) << 2) | (uint32_t)g;
                     }
-                    if (q1) {  // holds exactly one
-                        const uint32_t pos = base_a + __builtin_amdgcn_mbcnt_hi((uint32_t)(b1 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b1, 0u));
-                        const int idx = idx_of(c, g, (gpr[c] >> (8 * g)) & 0xffu);
-                        if (pos < (uint32_t)kSelMax) {
-                            sm.vals[pos] = m1[g];
-                            sm.idxs[pos] = idx;
-                            if (bins) meta[pos] = ((uint32_t)bn << 16) | atomicAdd(&sm.bhist[bin_word(bn)], 1u);
-                        } else if (pos < (uint32_t)kRowCap) {
-                            sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(m1[g]) << 32) | (unsigned long long)(uint32_t)idx);
-                        }
-                    }
-                    base_l += (uint32_t)__popcll(b2);
-                    base_a += (uint32_t)__popcll(b1);
+                    if (mq1 & bit)  // holds exactly one
+                        place(base_a + (uint32_t)__popc(mq1 & (bit - 1u)), m1[g], idx_of(c, g, (gpr[c] >> (8 * g)) & 0xffu));
                 }
             }
         }
@@ -1276,7 +1295,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     bool listed = false;
     if (n_q <= kQCap) {
         SR_PROF(a, 3);
-        gather(n_q, [&](bool kept, float x, int idx) { append(kept && x >= tval, x, idx); });
+        gather(n_q, [&](float x) { return x >= tval; });
         listed = true;
     } else {
         bins = false;  // the exact bound below starts the list again
@@ -1302,7 +1321,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         });
         __syncthreads();
         const int nq = min((int)sm.bcast[13], kQCap);  // < sel
-        gather(nq, [&](bool kept, float x, int idx) { append(kept && x > tx, x, idx); });
+        gather(nq, [&](float x) { return x > tx; });
         __syncthreads();
         const int n_gt = (int)sm.bcast[12];
         const int need_eq = sel - n_gt;
