@@ -432,9 +432,9 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     // rows without penalties that may raise a logit have their candidates binned while they are collected
     const bool want_bins = rd.path == SR_PATH_TOPK && (!use_edits || hist_regs);
     bool binned = false;
-    float mx0 = 0.0f;
+    float mx0 = 0.0f, bscale0 = -56.0f, bound0 = 0.0f;
     const int n_c = build_candidates<EPV, kVec>(
-        a, slot, row, rd, want_bins, inv_temp, &mx0, &binned,
+        a, slot, row, rd, want_bins, inv_temp, &mx0, &bscale0, &bound0, &binned,
         [&]() SR_INL {
 #pragma unroll
             for (int r = 0; r < kHistRegs; r++) {
@@ -560,6 +560,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 
     float mx;
     float mx_bins = 0.0f;  // what the bins are measured from: mx, or the largest kept element outside the history
+    float bscale = -56.0f;  // bins per unit of (v / T), negated
     // Candidates whose e = expf(v / T - max) is below 2^-26 are dropped before the sort: with e_0 = 1
     // they change neither running sum (they are under half an ulp of a sum >= 1, and of a cumulative
     // probability >= probs[0]) and the draw can never stop on them, so the result is bit-identical.
@@ -693,12 +694,12 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             if (key == 0u) return -1;
             const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx_bins);
             if (x < -18.1f) return -1;
-            return min(max((int)__fmul_rn(x, -56.0f), 0), kBins - 1);
+            return min(max((int)__fmul_rn(x, bscale), 0), kBins - 1);
         };
         // the bin of an entry that was kept (binned candidates are never dropped once they are on the list)
         auto bin_kept = [&](uint32_t key) SR_INL -> int {
             const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx_bins);
-            return min(max((int)__fmul_rn(x, -56.0f), 0), kBins - 1);
+            return min(max((int)__fmul_rn(x, bscale), 0), kBins - 1);
         };
         int bstar = kBins - 1, n_live = 0, n_keep = 0, max_bin = 0;
         // every wave reads the histogram: live entries, and the first bin at which the k best are complete;
@@ -737,10 +738,14 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         if (binned) {
             // The candidates were counted into the histogram as they were collected; the history ids join them.
             mx_bins = mx0;
+            bscale = bscale0;
+            // a history id whose adjusted logit is below the candidates' bound has at least top_k candidates above
+            // it, or lies too far below the maximum to matter
+            const uint32_t bound_key = sr_okey(bound0);
             uint32_t hmeta[kHistRegs];
 #pragma unroll
             for (int r = 0; r < kHistRegs; r++) {
-                const int b = hraw[r] != 0u ? bin_of(hadj[r]) : -1;
+                const int b = (hraw[r] != 0u && hadj[r] >= bound_key) ? bin_of(hadj[r]) : -1;
                 hmeta[r] = b >= 0 ? (((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u)) : 0xffffffffu;
             }
             __syncthreads();
@@ -776,6 +781,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 placed = true;
             } else {
                 load_cands();  // a flat or heavily tied row: the general way below
+                bscale = -56.0f;
             }
         }
         if (!placed) {
@@ -1021,11 +1027,13 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 // that happened (few chunks, a short enough list, a finite maximum); *mx0 is the maximum times inv_temp.
 template <int EPV, int kVec, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
-                                                float inv_temp, float* mx0_out, bool* binned, Early&& early, Late&& late,
-                                                TopkSmem& sm)
+                                                float inv_temp, float* mx0_out, float* bscale_out, float* bound_out,
+                                                bool* binned, Early&& early, Late&& late, TopkSmem& sm)
 {
     *binned = false;
     *mx0_out = 0.0f;
+    *bscale_out = -56.0f;
+    *bound_out = -3.402823466e38f;
     using VO = VecOps<EPV>;
     constexpr int ES = (EPV == 4) ? 4 : 2;
     constexpr int kGV = (kVec + SR_TK_GROUPS - 1) / SR_TK_GROUPS;  // vectors per group
@@ -1107,13 +1115,13 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         return want ? (int)(base + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))) : -1;
     };
     bool bins = false;
-    float mx0 = 0.0f;
+    float mx0 = 0.0f, bscale = -56.0f;
     uint32_t* meta = (uint32_t*)sm.probs;
     // the bin of a candidate: 0 .. kBins - 1, never increasing with the value (what lies too far below the maximum
     // to matter never gets here: the bound is at least the maximum minus 18 T, see below)
     auto bin0 = [&](float x) SR_INL -> int {
         const float d = __fsub_rn(__fmul_rn(x, inv_temp), mx0);
-        return min(max((int)__fmul_rn(d, -56.0f), 0), kBins - 1);
+        return min(max((int)__fmul_rn(d, bscale), 0), kBins - 1);
     };
     // one candidate at list position pos
     auto place = [&](uint32_t pos, float x, int idx) SR_INL {
@@ -1233,6 +1241,9 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         }
         bins = want_bins && direct && km > kKeyNegInf;
         mx0 = __fmul_rn(sr_okey_inv(km), inv_temp);
+        // the bins span what can become a candidate: from the maximum down to the bound
+        const float span = __fsub_rn(mx0, __fmul_rn(tval, inv_temp));
+        if (bins && span > 1e-3f && span < 1e30f) bscale = -fminf(__fdiv_rn((float)(kBins - 1), span), 65536.0f);
     }
     late();
     SR_PROF(a, 1);
@@ -1357,6 +1368,8 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     __syncthreads();
     *binned = bins && listed && n_c <= (uint32_t)kSelMax;
     *mx0_out = mx0;
+    *bscale_out = bscale;
+    *bound_out = tval;
     return n_c > (uint32_t)kRowCap ? -1 : (int)n_c;
 }
 
