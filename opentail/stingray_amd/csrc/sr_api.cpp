@@ -66,15 +66,15 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     b->scan_base_mod = base_mod;
     b->scan_stride_mod = stride_mod;
     if (b->h_scan.empty()) return SR_OK;
+    const int n_sel = (int)b->h_sel_list.size();
+    int chunks = 1, chunk_vecs = 0;
+    topk_geometry(b->vocab, epv == 8 ? SR_DTYPE_BF16 : SR_DTYPE_F32, n_sel, ctx->cu_count, &chunks, &chunk_vecs);
     {
         // Dispatch order.  Workgroups are dispatched in grid order, two resident per CU; a round is that many
         // consecutive workgroups.  A row's tail goes to the middle of the round after the one that holds the row's
         // last chunk: half of that round's workgroups have retired by the time it is dispatched, so its chunks have
         // usually finished and it does not hold a slot while it waits, yet it does not queue behind all of the
         // later rows' chunks either.  Every entry carries what its workgroup needs to find its data.
-        const int n_sel = (int)b->h_sel_list.size();
-        int chunks = 1, chunk_vecs = 0;
-        topk_geometry(b->vocab, epv == 8 ? SR_DTYPE_BF16 : SR_DTYPE_F32, n_sel, ctx->cu_count, &chunks, &chunk_vecs);
         const int round = 2 * ctx->cu_count;
         std::vector<int32_t> sched;
         sched.reserve((size_t)n_sel * (size_t)(chunks + 1) * 4);
@@ -108,16 +108,15 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
         SR_HIP(ctx, hipMemcpyAsync(b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
         SR_HIP(ctx, hipStreamSynchronize(st));
     }
-    const int64_t blocks = ((int64_t)b->vocab + 2 * epv - 2) / epv / 64 + 1;
-    b->scan_stride = blocks * epv;
+    b->scan_stride = (int64_t)chunks * SR_TK_THREADS * SR_TK_MASK_WORDS;
     if (rows_changed)
         SR_HIP(ctx, hipMemcpyAsync(b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), hipMemcpyHostToDevice, st));
     SR_HIP(ctx, b->d_scan_desc.reserve(b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, hipMemcpyAsync(b->d_scan_desc.p, b->h_scan.data(), b->h_scan.size() * sizeof(SrScanDesc), hipMemcpyHostToDevice, st));
-    SR_HIP(ctx, b->d_scan_mask.reserve(b->h_scan.size() * (size_t)b->scan_stride * sizeof(unsigned long long), st));
+    SR_HIP(ctx, b->d_scan_mask.reserve(b->h_scan.size() * (size_t)b->scan_stride * sizeof(uint32_t), st));
     SR_HIP(ctx, sr_launch_build_scan_mask(b->d_scan_desc.as<SrScanDesc>(), (int)b->h_scan.size(), b->d_rows.as<SrRow>(),
                                           b->d_edits.as<SrEdit>(), b->d_mask.as<uint32_t>(), b->mask_stride,
-                                          b->d_scan_mask.as<unsigned long long>(), b->scan_stride, b->vocab, epv,
+                                          b->d_scan_mask.as<uint32_t>(), b->scan_stride, b->vocab, epv, chunks, chunk_vecs,
                                           base_addr, stride_bytes, st));
     // the host vectors are read by the async copies above
     SR_HIP(ctx, hipStreamSynchronize(st));
@@ -438,7 +437,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.edits = b->d_edits.as<SrEdit>();
         a.mask = b->d_mask.as<uint32_t>();
         a.mask_stride = b->mask_stride;
-        a.scan_mask = b->d_scan_mask.as<unsigned long long>();
+        a.scan_mask = b->d_scan_mask.as<uint32_t>();
         a.scan_stride = b->scan_stride;
         a.cand = ctx->cand.as<unsigned long long>();
         a.gmax = ctx->gmax.as<float4>();

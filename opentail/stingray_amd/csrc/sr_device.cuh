@@ -89,12 +89,14 @@ template <typename T> __device__ __forceinline__ T sr_load_agent(const T* p)
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // 16 bytes in one write-through store (four separate 4-byte stores of a thread reach memory as four partial
-// writes of the same line).  The compiler does not count this store: sr_drain_stores() waits for it.
+// writes of the same line).  The compiler neither counts this store (sr_drain_stores() waits for it) nor
+// knows its hazards: a store of more than 8 bytes reads its data registers a few cycles after issue, so the
+// wait states that must separate it from the next write of those registers are part of the statement.
 __device__ __forceinline__ void sr_store_agent_f4(float4* p, float x, float y, float z, float w)
 {
     typedef float __attribute__((ext_vector_type(4))) f32x4;
     const f32x4 v = {x, y, z, w};
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 3" ::"v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ void sr_drain_stores() { __builtin_amdgcn_s_waitcnt(0); }
 

@@ -31,8 +31,8 @@ struct SrTopkArgs {
     const SrEdit* edits;
     const uint32_t* mask;
     int64_t mask_stride;     // words
-    const unsigned long long* scan_mask; // keep-bits of every row in the kernel's access order (SrRow.scan_row)
-    int64_t scan_stride;     // 64-bit words per scan row
+    const uint32_t* scan_mask; // keep-bits of every row in the kernel's access order (SrRow.scan_row)
+    int64_t scan_stride;     // 32-bit words per scan row: chunks x threads x SR_TK_MASK_WORDS
     float4* gmax;            // [n_rows][chunks][SR_TK_THREADS]: the four group maxima of every thread of every chunk
     float4* gmax2;           // ... the second largest element of each of those groups
     uint32_t* gpos;          // ... the position of the largest inside its group, 8 bits per group
@@ -50,8 +50,8 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream);
 // Builds scan row i for descs[i]; base_addr / stride_bytes are those of the logits the mask is used with
 // (they decide where a row starts inside its first 16-byte vector), epv = 4 (fp32) or 8 (bf16).
 hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, int n_scan, const SrRow* rows, const SrEdit* edits,
-                                     const uint32_t* mask, int64_t mask_stride, unsigned long long* scan_mask,
-                                     int64_t scan_stride, int vocab, int epv, unsigned long long base_addr,
+                                     const uint32_t* mask, int64_t mask_stride, uint32_t* scan_mask, int64_t scan_stride,
+                                     int vocab, int epv, int chunks, int chunk_vecs, unsigned long long base_addr,
                                      long long stride_bytes, hipStream_t stream);
 
 struct SrArgmaxArgs {

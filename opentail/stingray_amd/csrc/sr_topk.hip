@@ -1044,7 +1044,11 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     const int mis = (int)(((uintptr_t)rowp & 15u) / ES);
     const int nvt = (a.vocab + mis + EPV - 1) / EPV;
     const u32x4* wp = (const u32x4*)(rowp - (size_t)mis * ES);
-    const uint32_t* keep32 = (const uint32_t*)(a.scan_mask + (size_t)rd.scan_row * (size_t)a.scan_stride);
+    const uint32_t* keep32 = a.scan_mask + (size_t)rd.scan_row * (size_t)a.scan_stride;
+    // the EPV keep-bits of vector j of thread t of chunk c (they never straddle a word: EPV divides 32)
+    auto keep_bits = [&](int c, int j, int t) SR_INL -> uint32_t {
+        return (keep32[((size_t)c * kThreads + t) * SR_TK_MASK_WORDS + ((j * EPV) >> 5)] >> ((j * EPV) & 31)) & ((1u << EPV) - 1u);
+    };
     const float4* gm = a.gmax + (size_t)slot * S * kThreads + tid;
     unsigned long long* crow = a.cand + (size_t)slot * kRowCap;
     uint32_t* qlist = sm.xa;  // kQCap entries: xa and xb lie back to back
@@ -1160,21 +1164,20 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         const int pos = wave_slot(want, &sm.bcast[13]);
         if (pos >= 0 && pos < kQCap) qlist[pos] = ((uint32_t)(c * kThreads + tid) << 2) | (uint32_t)g;
     };
-    // fetches the listed groups, kBatch (group, vector) items per thread at a time -- values and the keep-bit halves
+    // fetches the listed groups, kBatch (group, vector) items per thread at a time -- values and keep-bits
     // of all of them in one batch of loads -- and appends every kept element that pred admits to the candidates
     auto gather = [&](int nq, auto&& pred) SR_INL {
         const int n_items = nq * kGV;
         for (int i0 = 0; i0 < n_items; i0 += kBatch * kThreads) {
             u32x4 v[kBatch];
-            uint32_t kw[kBatch][EPV];
+            uint32_t kw[kBatch];
             int fvs[kBatch];
 #pragma unroll
             for (int r = 0; r < kBatch; r++) {
                 const int i = i0 + r * kThreads + tid;
                 fvs[r] = -1;
                 v[r] = VO::neg_inf();
-#pragma unroll
-                for (int q = 0; q < EPV; q++) kw[r][q] = 0u;
+                kw[r] = 0u;
                 if (i0 + r * kThreads < n_items && i < n_items) {  // the first test is uniform: unused slots cost nothing
                     const uint32_t gid = qlist[i / kGV];
                     const int m = i - (i / kGV) * kGV;
@@ -1187,9 +1190,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                         const int fv = f0 + fl;
                         fvs[r] = fv;
                         v[r] = wp[fv];
-                        const uint32_t* kp = keep32 + ((size_t)(fv >> 6) * EPV) * 2 + ((fv & 63) >> 5);
-#pragma unroll
-                        for (int q = 0; q < EPV; q++) kw[r][q] = kp[2 * q];
+                        kw[r] = keep_bits(c, j, t);
                     }
                 }
             }
@@ -1199,7 +1200,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                 uint32_t own = 0u;
 #pragma unroll
                 for (int q = 0; q < EPV; q++) {
-                    const bool kept = fvs[r] >= 0 && ((kw[r][q] >> (fvs[r] & 31)) & 1u) != 0u;
+                    const bool kept = ((kw[r] >> q) & 1u) != 0u;
                     own |= (kept && pred(VO::get(v[r], q))) ? (1u << q) : 0u;
                 }
                 uint32_t pos = wave_reserve(__popc(own), &sm.bcast[12]);
@@ -1345,10 +1346,11 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
             for (int q = 0; q < EPV; q++) is_eq[q] = false;
             if (fv < nvt) {
                 const u32x4 v = wp[fv];
-                const uint32_t* kp = keep32 + ((size_t)(fv >> 6) * EPV) * 2 + ((fv & 63) >> 5);
+                const int c = fv / a.chunk_vecs, fl = fv - c * a.chunk_vecs;
+                const uint32_t kb = keep_bits(c, fl / kThreads, fl % kThreads);
 #pragma unroll
                 for (int q = 0; q < EPV; q++) {
-                    is_eq[q] = VO::get(v, q) == tx && ((kp[2 * q] >> (fv & 31)) & 1u) != 0u;
+                    is_eq[q] = VO::get(v, q) == tx && ((kb >> q) & 1u) != 0u;
                     ceq += is_eq[q] ? 1 : 0;
                 }
             }
@@ -1443,6 +1445,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 
     if (nv > 0) {
         const u32x4* cp = (const u32x4*)(rowp - (size_t)mis * ES) + f0;
+        const uint32_t* mw = a.scan_mask + (size_t)info.z * (size_t)a.scan_stride + ((size_t)c * kThreads + tid) * SR_TK_MASK_WORDS;
+        const uint32_t kw0 = mw[0], kw1 = mw[1], kw2 = mw[2];
         // the chunk as fp32 in registers (the upcast of bf16 is exact)
         float xv[kVec * EPV];
         {
@@ -1462,27 +1466,19 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        // The scan mask holds one keep-bit per window element in this kernel's access order: for every
-        // block of 64 vectors, EPV 64-bit words, word q bit l = element q of the vector of lane l.  It
-        // carries the row's edges, its allow-mask and, when the row tail fetches them, its history ids,
-        // and is wave-uniform: scalar loads, one select per element.
-        {
-            // read through the constant address space: the mask was written by an earlier launch, and scalar
-            // loads need the compiler to know that nothing in this kernel writes it
-            typedef const unsigned long long __attribute__((address_space(4))) const_u64;
-            const_u64* srow = (const_u64*)(uintptr_t)(a.scan_mask + (size_t)info.z * (size_t)a.scan_stride);
-            const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
-            const int nblk = (nvt + 63) >> 6;
+        // The scan mask holds one keep-bit per window element in this kernel's access order: the thread's own
+        // three words (loaded ahead of the data), bit j * EPV + q = element q of its j-th vector.  They carry the
+        // row's edges, its allow-mask and, when the row tail fetches them, its history ids: two operations per
+        // element replace all per-element edge, allow-mask and history logic.
 #pragma unroll
-            for (int j = 0; j < kVec; j++) {
-                const int blk = (f0 >> 6) + j * (kThreads / SR_WAVE) + wave_u;
-                if (blk < nblk) {
-                    const_u64* mp = srow + (size_t)blk * EPV;
+        for (int j = 0; j < kVec; j++)
 #pragma unroll
-                    for (int q = 0; q < EPV; q++) xv[j * EPV + q] = __builtin_amdgcn_inverse_ballot_w64(mp[q]) ? xv[j * EPV + q] : SR_NEG_INF;
-                }
+            for (int q = 0; q < EPV; q++) {
+                const int bit = j * EPV + q;
+                const uint32_t w = bit < 32 ? kw0 : bit < 64 ? kw1 : kw2;
+                const uint32_t t = (uint32_t)((int)(w << (31 - (bit & 31))) >> 31);  // all ones = keep
+                xv[j * EPV + q] = sr_u2f((sr_f2u(xv[j * EPV + q]) & t) | (0xff800000u & ~t));
             }
-        }
         if (a.prof) pt1 = wall_clock64();
 
         // Every lane owns four interleaved groups of vectors (j mod 4).  Of each group the row tail gets the largest
@@ -1559,70 +1555,64 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 }
 
 // ---- scan mask ---------------------------------------------------------------------------------------
-// One keep-bit per window element of a row, in the selection kernel's access order: for every block of 64
-// 16-byte vectors, epv 64-bit words; bit l of word q = element q of the vector that lane l loads.  A bit is
-// set when the element lies inside the row, its allow-mask (if any) admits it and, for rows whose tail
-// fetches the history logits by id, it is not a history id.
-__global__ __launch_bounds__(256) void k_build_scan_mask(const SrScanDesc* descs, const SrRow* rows, const SrEdit* edits,
-                                                         const uint32_t* mask, int64_t mask_stride,
-                                                         unsigned long long* scan_mask, int64_t scan_stride, int vocab,
-                                                         int epv, int es, unsigned long long base_addr,
-                                                         long long stride_bytes)
+// One keep-bit per window element of a row, in the selection kernel's access order: SR_TK_MASK_WORDS 32-bit words
+// per chunk and thread, bit j * epv + q = element q of the thread's j-th vector.  A bit is set when the element
+// lies inside the row, its allow-mask (if any) admits it and, for rows whose tail fetches the history logits by
+// id, it is not a history id.  One workgroup per (scan row, chunk): the words are built in LDS, the history ids
+// that fall into the chunk are cleared there, then the words are written out.
+__global__ __launch_bounds__(kThreads) void k_build_scan_mask(const SrScanDesc* descs, const SrRow* rows, const SrEdit* edits,
+                                                              const uint32_t* mask, int64_t mask_stride, uint32_t* scan_mask,
+                                                              int64_t scan_stride, int vocab, int epv, int es, int chunks,
+                                                              int chunk_vecs, int vecs_per_thread,
+                                                              unsigned long long base_addr, long long stride_bytes)
 {
-    const SrScanDesc d = descs[blockIdx.x];
+    __shared__ uint32_t words[kThreads * SR_TK_MASK_WORDS];
+    const int srow = blockIdx.x / chunks, c = blockIdx.x - srow * chunks;
+    const int t = threadIdx.x;
+    const SrScanDesc d = descs[srow];
     const SrRow rd = rows[d.row];
     const int mis = (int)(((base_addr + (unsigned long long)d.row * (unsigned long long)stride_bytes) & 15ull) / (unsigned)es);
-    unsigned long long* dst = scan_mask + (size_t)blockIdx.x * scan_stride;
+    const int nvt = (vocab + mis + epv - 1) / epv;
+    const int f0 = c * chunk_vecs;
+    const int nv = min(chunk_vecs, nvt - f0);
     const uint32_t* src = ((d.flags & SR_SCAN_ALLOW) && rd.mask_row >= 0) ? mask + (size_t)rd.mask_row * mask_stride : nullptr;
-    for (int w = threadIdx.x; w < (int)scan_stride; w += blockDim.x) {
-        const int b = w / epv, q = w - b * epv;
-        const long long e_first = (long long)b * 64 * epv + q - mis;  // the element under lane 0
-        unsigned long long bits = 0ull;
-        if (!src && e_first >= 0 && e_first + 63ll * epv < vocab) {
-            bits = ~0ull;
-        } else if (src && mis == 0) {
-            // every epv-th bit of the 64 * epv allow-bits of the block, starting at bit q, squeezed together
-            const int words_in = 2 * epv, first = b * words_in, per = 32 / epv;  // 8 or 4 bits from each input word
-            for (int k = 0; k < words_in; k++) {
-                const long long e0w = (long long)(first + k) * 32;
-                uint32_t x = 0u;
-                if (e0w < vocab) {
-                    x = src[first + k];
-                    if (e0w + 32 > vocab) x &= (1u << (vocab - e0w)) - 1u;
-                }
-                x >>= q;
-                if (epv == 4) {
-                    x &= 0x11111111u;
-                    x = (x | (x >> 3)) & 0x03030303u;
-                    x = (x | (x >> 6)) & 0x000f000fu;
-                    x = (x | (x >> 12)) & 0xffu;
-                } else {
-                    x &= 0x01010101u;
-                    x = (x | (x >> 7)) & 0x00030003u;
-                    x = (x | (x >> 14)) & 0xfu;
-                }
-                bits |= (unsigned long long)x << (k * per);
-            }
+    uint32_t w[SR_TK_MASK_WORDS];
+#pragma unroll
+    for (int k = 0; k < SR_TK_MASK_WORDS; k++) w[k] = 0u;
+    for (int j = 0; j < vecs_per_thread; j++) {
+        const int fl = j * kThreads + t;
+        if (fl >= nv) break;
+        const long long e0 = (long long)(f0 + fl) * epv - mis;  // row element under q = 0
+        uint32_t bits = 0u;
+        if (!src && e0 >= 0 && e0 + epv <= vocab) {
+            bits = (1u << epv) - 1u;
         } else {
-            for (int l = 0; l < 64; l++) {
-                const long long e = e_first + (long long)l * epv;
-                if (e >= 0 && e < vocab && (!src || mask_bit(src, (int)e))) bits |= 1ull << l;
+            for (int q = 0; q < epv; q++) {
+                const long long e = e0 + q;
+                if (e >= 0 && e < vocab && (!src || mask_bit(src, (int)e))) bits |= 1u << q;
             }
         }
-        dst[w] = bits;
+        const int b = j * epv;
+        w[b >> 5] |= bits << (b & 31);
     }
-    __threadfence_block();
+#pragma unroll
+    for (int k = 0; k < SR_TK_MASK_WORDS; k++) words[t * SR_TK_MASK_WORDS + k] = w[k];
     __syncthreads();
     if (d.flags & SR_SCAN_HIST) {
         const SrEdit* ed = edits + rd.edit_off;
-        uint32_t* dst32 = (uint32_t*)dst;
-        for (int e = threadIdx.x; e < rd.edit_cnt; e += blockDim.x) {
+        for (int e = t; e < rd.edit_cnt; e += kThreads) {
             const int p = ed[e].id + mis;
-            const int b = p / (64 * epv), r = p - b * 64 * epv;
-            const int l = r / epv, q = r - l * epv;
-            atomicAnd(&dst32[((size_t)b * epv + q) * 2 + (l >> 5)], ~(1u << (l & 31)));
+            const int fv = p / epv, q = p - fv * epv;
+            const int fl = fv - f0;
+            if (fl < 0 || fl >= nv) continue;
+            const int j = fl / kThreads, tt = fl - j * kThreads;
+            const int b = j * epv + q;
+            atomicAnd(&words[tt * SR_TK_MASK_WORDS + (b >> 5)], ~(1u << (b & 31)));
         }
+        __syncthreads();
     }
+    uint32_t* dst = scan_mask + (size_t)srow * scan_stride + (size_t)c * kThreads * SR_TK_MASK_WORDS;
+    for (int i = t; i < kThreads * SR_TK_MASK_WORDS; i += kThreads) dst[i] = words[i];
 }
 
 }  // namespace
@@ -1639,12 +1629,13 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
 }
 
 hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, int n_scan, const SrRow* rows, const SrEdit* edits,
-                                     const uint32_t* mask, int64_t mask_stride, unsigned long long* scan_mask,
-                                     int64_t scan_stride, int vocab, int epv, unsigned long long base_addr,
+                                     const uint32_t* mask, int64_t mask_stride, uint32_t* scan_mask, int64_t scan_stride,
+                                     int vocab, int epv, int chunks, int chunk_vecs, unsigned long long base_addr,
                                      long long stride_bytes, hipStream_t stream)
 {
     if (n_scan <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_build_scan_mask, dim3((unsigned)n_scan), dim3(256), 0, stream, descs, rows, edits, mask,
-                       mask_stride, scan_mask, scan_stride, vocab, epv, epv == 8 ? 2 : 4, base_addr, stride_bytes);
+    hipLaunchKernelGGL(k_build_scan_mask, dim3((unsigned)(n_scan * chunks)), dim3(kThreads), 0, stream, descs, rows, edits,
+                       mask, mask_stride, scan_mask, scan_stride, vocab, epv, epv == 8 ? 2 : 4, chunks, chunk_vecs,
+                       epv == 8 ? SR_TK_VEC_BF16 : SR_TK_VEC, base_addr, stride_bytes);
     return hipGetLastError();
 }
