@@ -1496,7 +1496,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 for (int q = 0; q < EPV; q++) {
                     const float x = xv[j * EPV + q];
                     p1 = x > m1 ? (j / SR_TK_GROUPS) * EPV + q : p1;  // strict: the first of equal values stays
-                    m2 = fmaxf(m2, fminf(m1, x));
+                    m2 = __builtin_amdgcn_fmed3f(m1, m2, x);  // m2 <= m1: the median of the three is the new second largest
                     m1 = fmaxf(m1, x);
                 }
             gm1[g] = m1;
