@@ -1,12 +1,15 @@
 // Top-k-first sampling (the reference's SampleTopK, Sampler.cs:216-357) and the greedy rows.
 //
 // One launch, grid = rows x chunks chunk workgroups + one tail workgroup per row.  A chunk workgroup
-// loads one contiguous chunk of a row ONCE into registers (19 x 16 B per thread), derives a safe
-// threshold (a lower bound on the sel-th largest scanned logit), appends the few elements at or above
-// it to the row's candidate list and signals the row.  For sel <= 64 every wave works on its own:
-// the sel-th largest of its 64 lane maxima bounds the sel-th largest element from below and no
-// workgroup barrier is needed; larger sel take the sel-th largest of 2048 disjoint-group maxima of the
-// whole workgroup (LDS radix histograms).
+// loads one contiguous chunk of a row ONCE into registers (19 x 16 B per thread), applies the row's scan
+// mask, and leaves per lane and group of ~19 elements the largest element, its position and the second
+// largest, plus per wave a share of the row's bound.  Nothing is selected there: the workgroup streams.
+//
+// The row tail derives a lower bound on the row's sel-th largest element from the waves' shares, takes the
+// largest element of every group whose second largest is below the bound directly, fetches the few groups
+// with more than one element above it again, and merges: penalties, pruning of candidates too small to
+// change any fp32 sum, an order by (value after penalties, value before, index), then the softmax / min-p /
+// top-p / draw arithmetic in the reference's sequential fp32 order.
 //
 // When the history penalties can only lower a logit (repetition >= 1, presence and frequency >= 0) the
 // scan skips the history ids (a per-row scan mask built when the batch is uploaded) and asks for the
@@ -15,10 +18,6 @@
 // history is in the final k only if it is among the k best outside the history, and a history token
 // that the reference's over-selection misses has more than k unpenalised tokens above it.  Penalties
 // that can raise a logit keep the reference's literal over-selection.
-//
-// The row tail merges the candidates: penalties, pruning of candidates too small to change any fp32
-// sum, a sort by (value after penalties, value before, index), then the softmax / min-p / top-p / draw
-// arithmetic in the reference's sequential fp32 order.
 #include "sr_device.cuh"
 #include "sr_types.h"
 #include "sr_kernels.h"
@@ -47,17 +46,16 @@ constexpr int kBinsPad = kBins + SR_WAVE + 1;
 __device__ __forceinline__ int bin_word(int b) { return b + b / kBinsPerLane; }
 
 struct TopkSmem {
-    uint32_t xa[kSelMax];  // gathered list, then sort exchange (three 32-bit words per element)
+    uint32_t xa[kSelMax];  // list of groups to fetch (xa and xb), then the kept entries by bin / the sort exchange
+                           // (three 32-bit words per entry)
     uint32_t xb[kSelMax];
     uint32_t xc[kSelMax];
-    float vals[kSelMax];
-    int idxs[kSelMax];
-    __attribute__((aligned(16))) float probs[kSelMax + 8];
+    float vals[kSelMax];   // candidate values, later the k best in order
+    int idxs[kSelMax];     // ... and their indices
+    __attribute__((aligned(16))) float probs[kSelMax + 8];  // per candidate (bin, arrival), later e, then the running sums
     uint32_t hist[256];
     uint32_t red[2 * kWaves];
     uint32_t bcast[16];
-    unsigned long long ksum;   // chunk scan: sum of the waves' threshold estimates
-    uint32_t btotal;           // chunk scan: elements of the chunk at or above the shared threshold
     uint32_t bhist[kBinsPad];  // live entries per bin of distance below the maximum
     uint32_t boff[kBinsPad];   // first list position of every bin
     uint32_t bfill[kBinsPad];  // entries scattered into the bin so far
@@ -389,12 +387,12 @@ __device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
 #define SR_INL __attribute__((always_inline))
 
 // ---- the row tail ----------------------------------------------------------------------------------
-// Called by every thread of the tail workgroup of a row once all chunks have appended their candidates.
-// slot = position of the row in this launch, n_c = candidates in the row's list.  The list is read once,
-// straight into registers; every later pass runs from registers or LDS.
+// Called by every thread of the tail workgroup of a row once all chunks of the row have been counted in.
+// slot = position of the row in this launch.
 template <int EPV, int kVec, typename Early, typename Late>
-__device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, Early&& early,
-                                                Late&& late, TopkSmem& sm);
+__device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
+                                                float inv_temp, float* mx0_out, float* bscale_out, float* bound_out,
+                                                bool* binned, Early&& early, Late&& late, TopkSmem& sm);
 
 template <int EPV, int kVec>
 __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, TopkSmem& sm)

@@ -53,10 +53,8 @@ struct SrScanDesc {
 #define SR_TK_VEC_BF16 10                  // ... of bf16 logits: the same 40 thousand elements per workgroup
 #define SR_TK_MASK_WORDS 3                 // 32-bit keep-words per chunk thread: 19 x 4 and 10 x 8 bits both fit 96
 #define SR_TK_GROUPS 4                     // group maxima per thread
-#define SR_TK_M (SR_TK_THREADS * SR_TK_GROUPS)
 #define SR_TK_SEL_MAX 2048                 // most entries (candidates + history ids) the row tail sorts
 #define SR_TK_ROW_CAP 8192                 // candidates all chunks of a row may hand to its tail (16 per thread)
-#define SR_TK_WAVE_LIM 128                 // least per-wave share of SR_TK_ROW_CAP for the per-wave scan
 #define SR_TK_MAX_CHUNKS 128               // most workgroups one row is split over
 
 // Full-vocabulary path: nucleus candidates up to this count are sorted inside the row kernel.
