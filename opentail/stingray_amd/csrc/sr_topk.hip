@@ -966,45 +966,58 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             if (sm.probs[t] < thr) { first = t; break; }
         count = min(count, block_min_i32(first, sm));
     }
-    // Sampler.cs:326-349: running sum (probs[t] becomes cum[t]); top-p cuts after the first cum >= TopP
+    // Sampler.cs:326-349: running sum; top-p cuts after the first cum >= TopP.  Then the draw (:351-357): the first
+    // entry whose running sum reaches r = u * (sum of the kept entries).  One lane runs both chains and nothing is
+    // stored in between: the second chain repeats the additions of the first (same operands, same order, same
+    // bits) up to where the draw stops.  The sums never decrease, so whole blocks of 32 entries are added without
+    // a look (eight loads in flight, one chain of 32 additions) until a block's last sum has reached the target;
+    // only that block, or the remainder of the list, is walked entry by entry.
     if (tid == 0) {
         const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
         const float top_p = use_top_p ? rd.top_p : __uint_as_float(0x7f800000u);  // +inf: never reached
-        float cum = 0.0f;
-        int cnt = count;
-        // four entries per step, the next four already in flight (the stores of a step must not hold up the loads
-        // of the following one); entries past `count` are computed but never looked at
-        float4* p4 = (float4*)sm.probs;
-        float4 cur = p4[0];
-        for (int t = 0; t < count; t += 4) {
-            const float4 nxt = p4[(t >> 2) + 1];
-            float4 c;
-            c.x = __fadd_rn(cum, cur.x);
-            c.y = __fadd_rn(c.x, cur.y);
-            c.z = __fadd_rn(c.y, cur.z);
-            c.w = __fadd_rn(c.z, cur.w);
-            p4[t >> 2] = c;
-            if (c.w >= top_p) {  // the sums never decrease: the first one to reach TopP is among these four
-                const int q = (c.x >= top_p) ? 0 : (c.y >= top_p) ? 1 : (c.z >= top_p) ? 2 : 3;
-                if (t + q < count) cnt = t + q + 1;
-                break;
+        const float4* p4 = (const float4*)sm.probs;
+        // first t < limit whose running sum is >= target (else -1); *val = that sum, or the sum of all `limit` entries
+        auto first_reach = [&](float target, int limit, float* val) SR_INL -> int {
+            float cum = 0.0f;
+            int t = 0;
+            while (t + 32 <= limit) {
+                float4 v[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = p4[(t >> 2) + i];
+                float c = cum;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    c = __fadd_rn(c, v[i].x); c = __fadd_rn(c, v[i].y);
+                    c = __fadd_rn(c, v[i].z); c = __fadd_rn(c, v[i].w);
+                }
+                if (c >= target) break;
+                cum = c;
+                t += 32;
             }
-            cum = c.w;
-            cur = nxt;
-        }
-        sm.bcast[6] = (uint32_t)cnt;
-    }
-    __syncthreads();
-    count = (int)sm.bcast[6];
-    SR_PROF(a, 10);
-    const float kept_sum = count > 0 ? sm.probs[count - 1] : 0.0f;
-    const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept_sum);
-    int first = 0x7fffffff;
-    for (int t = tid; t < count; t += kThreads)
-        if (r <= sm.probs[t] && sm.idxs[t] >= 0) { first = t; break; }
-    first = block_min_i32(first, sm);
-    if (tid == 0) {
-        a.out_tokens[row] = (first != 0x7fffffff) ? sm.idxs[first] : sm.idxs[0];
+            for (; t < limit; t += 4) {
+                const float4 v = p4[t >> 2];
+                const float cx = __fadd_rn(cum, v.x), cy = __fadd_rn(cx, v.y), cz = __fadd_rn(cy, v.z), cw = __fadd_rn(cz, v.w);
+                const int left = limit - t;  // entries of this step that exist
+                if (cx >= target) { *val = cx; return t; }
+                if (left == 1) { *val = cx; return -1; }
+                if (cy >= target) { *val = cy; return t + 1; }
+                if (left == 2) { *val = cy; return -1; }
+                if (cz >= target) { *val = cz; return t + 2; }
+                if (left == 3) { *val = cz; return -1; }
+                if (cw >= target) { *val = cw; return t + 3; }
+                cum = cw;
+            }
+            *val = cum;
+            return -1;
+        };
+        float kept_sum = 0.0f;
+        const int hit = first_reach(top_p, count, &kept_sum);
+        const int cnt = hit >= 0 ? hit + 1 : count;
+        SR_PROF(a, 10);
+        const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept_sum);
+        float unused;
+        const int first = first_reach(r, cnt, &unused);
+        a.out_tokens[row] = sm.idxs[first >= 0 ? first : 0];
         if (a.out_flags) a.out_flags[row] = out_flag;
     }
 }
