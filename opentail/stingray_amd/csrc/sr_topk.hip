@@ -1288,20 +1288,31 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         }
         base_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)base_a) + (uint32_t)((incl - n_own) & 0xffff);
         base_l = (uint32_t)__builtin_amdgcn_readfirstlane((int)base_l) + (uint32_t)((incl - n_own) >> 16);
-#pragma unroll
-        for (int c = 0; c < kG2Regs; c++) {
-            if (c < S) {
-                const float m1[4] = {gmr[c].x, gmr[c].y, gmr[c].z, gmr[c].w};
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const uint32_t bit = 1u << (c * 4 + g);
-                    if (mq2 & bit) {  // may hold more than one: fetched below
-                        const uint32_t pos = base_l + (uint32_t)__popc(mq2 & (bit - 1u));
-                        if (pos < (uint32_t)kQCap) qlist[pos] = ((uint32_t)(c * kThreads + tid) << 2) | (uint32_t)g;
-                    }
-                    if (mq1 & bit)  // holds exactly one
-                        place(base_a + (uint32_t)__popc(mq1 & (bit - 1u)), m1[g], idx_of(c, g, (gpr[c] >> (8 * g)) & 0xffu));
-                }
+        // Every lane walks its own set bits, lowest first: the wave makes as many rounds as its busiest lane has
+        // groups to hand over (a handful) instead of one per group of the thread (16).  The group's largest
+        // element and its position are picked out of the thread's registers by the bit number.
+        auto pick4 = [](const float4& v, int g) SR_INL -> float { return g == 0 ? v.x : g == 1 ? v.y : g == 2 ? v.z : v.w; };
+        {
+            uint32_t m = mq1, pos = base_a;
+            while (__ballot(m != 0u) != 0ull) {
+                const bool on = m != 0u;
+                const int bit = on ? __ffs((int)m) - 1 : 0;
+                m &= m - 1u;
+                const int c = bit >> 2, g = bit & 3;
+                const float r0 = pick4(gmr[0], g), r1 = pick4(gmr[1], g), r2 = pick4(gmr[2], g), r3 = pick4(gmr[3], g);
+                const float x = c == 0 ? r0 : c == 1 ? r1 : c == 2 ? r2 : r3;
+                const uint32_t gp = c == 0 ? gpr[0] : c == 1 ? gpr[1] : c == 2 ? gpr[2] : gpr[3];
+                if (on) place(pos++, x, idx_of(c, g, (gp >> (8 * g)) & 0xffu));
+            }
+        }
+        {
+            uint32_t m = mq2, pos = base_l;
+            while (__ballot(m != 0u) != 0ull) {  // groups that may hold more than one: fetched below
+                const bool on = m != 0u;
+                const int bit = on ? __ffs((int)m) - 1 : 0;
+                m &= m - 1u;
+                if (on && pos < (uint32_t)kQCap) qlist[pos] = ((uint32_t)((bit >> 2) * kThreads + tid) << 2) | (uint32_t)(bit & 3);
+                pos++;
             }
         }
     } else {
