@@ -1291,7 +1291,14 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         // Every lane walks its own set bits, lowest first: the wave makes as many rounds as its busiest lane has
         // groups to hand over (a handful) instead of one per group of the thread (16).  The group's largest
         // element and its position are picked out of the thread's registers by the bit number.
-        auto pick4 = [](const float4& v, int g) SR_INL -> float { return g == 0 ? v.x : g == 1 ? v.y : g == 2 ? v.z : v.w; };
+        // selects written as mask arithmetic: as conditionals the compiler may turn them into branches
+        auto sel = [](uint32_t x0, uint32_t x1, int bit) SR_INL -> uint32_t {
+            const uint32_t m = 0u - (uint32_t)(bit & 1);
+            return (x0 & ~m) | (x1 & m);
+        };
+        auto pick4 = [&](const float4& v, int g) SR_INL -> uint32_t {
+            return sel(sel(sr_f2u(v.x), sr_f2u(v.y), g), sel(sr_f2u(v.z), sr_f2u(v.w), g), g >> 1);
+        };
         {
             uint32_t m = mq1, pos = base_a;
             while (__ballot(m != 0u) != 0ull) {
@@ -1299,9 +1306,8 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                 const int bit = on ? __ffs((int)m) - 1 : 0;
                 m &= m - 1u;
                 const int c = bit >> 2, g = bit & 3;
-                const float r0 = pick4(gmr[0], g), r1 = pick4(gmr[1], g), r2 = pick4(gmr[2], g), r3 = pick4(gmr[3], g);
-                const float x = c == 0 ? r0 : c == 1 ? r1 : c == 2 ? r2 : r3;
-                const uint32_t gp = c == 0 ? gpr[0] : c == 1 ? gpr[1] : c == 2 ? gpr[2] : gpr[3];
+                const float x = sr_u2f(sel(sel(pick4(gmr[0], g), pick4(gmr[1], g), c), sel(pick4(gmr[2], g), pick4(gmr[3], g), c), c >> 1));
+                const uint32_t gp = sel(sel(gpr[0], gpr[1], c), sel(gpr[2], gpr[3], c), c >> 1);
                 if (on) place(pos++, x, idx_of(c, g, (gp >> (8 * g)) & 0xffu));
             }
         }
