@@ -348,6 +348,59 @@ __device__ int draw_from_row(const float* p, int n, double u, FullSmem& sm)
     return found >= 0 ? found : n - 1;
 }
 
+// Final Normalize (Sampler.cs:91-92, :553-562) and draw (:564-576) of a row whose m survivors are listed in
+// sm.sortbuf (probability bits << 32 | ~index) and whose other entries are all zero.  Adding zero changes no
+// running sum, so the eight strided chains of TensorPrimitives.Sum (plus its overlapped tail) and the running sum
+// of the draw are taken over the survivors alone, in index order: a chain's terms are the survivors whose index
+// falls on it, and the tail's indices lie behind every body index, so one order serves all eight chains.
+__device__ void finish_from_list(const SrFullArgs& a, float* p, int n, int m, int row, FullSmem& sm)
+{
+    const int tid = threadIdx.x;
+    int P = 2;
+    while (P < m) P <<= 1;
+    __syncthreads();
+    for (int i = tid; i < P; i += kT) {
+        const unsigned long long v = sm.sortbuf[i];
+        sm.sortbuf[i] = (i < m) ? ((v & 0xffffffffull) << 32) | (v >> 32) : 0ull;  // ~index on top: descending = index ascending
+    }
+    __syncthreads();
+    sort_small_desc(sm, P);
+    const int nv8 = (n / 8) * 8;
+    if (tid < SR_SEQ_CHAINS) {
+        float s = 0.0f;
+        for (int i = 0; i < m; i++) {
+            const unsigned long long v = sm.sortbuf[i];
+            const int e = (int)(0xffffffffu - (uint32_t)(v >> 32));
+            const int chain = e < nv8 ? (e & 7) : e - (n - 8);
+            if (chain == tid) s = __fadd_rn(s, sr_u2f((uint32_t)v));
+        }
+        sm.lane_sum[tid] = s;
+    }
+    __syncthreads();
+    const float l0 = sm.lane_sum[0], l1 = sm.lane_sum[1], l2 = sm.lane_sum[2], l3 = sm.lane_sum[3],
+                l4 = sm.lane_sum[4], l5 = sm.lane_sum[5], l6 = sm.lane_sum[6], l7 = sm.lane_sum[7];
+    const float sum = __fadd_rn(__fadd_rn(__fadd_rn(l0, l1), __fadd_rn(l2, l3)), __fadd_rn(__fadd_rn(l4, l5), __fadd_rn(l6, l7)));
+    const bool scale = sum > 0.0f && sum != 1.0f;
+    const float inv = scale ? __fdiv_rn(1.0f, sum) : 1.0f;
+    if (a.mode != 0 && scale) row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
+    if (a.mode != 1 && tid == 0) {
+        const float r = __double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]);
+        int token = n - 1;
+        if (!(r > 0.0f)) {
+            token = 0;  // the running sum starts at p[0] >= 0: index 0 reaches a target of zero whatever it holds
+        } else {
+            float acc = 0.0f;
+            for (int i = 0; i < m; i++) {
+                const unsigned long long v = sm.sortbuf[i];
+                const float x = sr_u2f((uint32_t)v);
+                acc = __fadd_rn(acc, scale ? __fmul_rn(x, inv) : x);
+                if (acc >= r) { token = (int)(0xffffffffu - (uint32_t)(v >> 32)); break; }
+            }
+        }
+        if (a.out_tokens) a.out_tokens[row] = token;
+    }
+}
+
 // ---- stage 3: softmax, top-k, min-p, top-p on the work row --------------------------------------------
 // phase 1 ends after top-p for rows whose nucleus candidates fit the kernel (<= kSmall survivors), or
 // after compacting the survivors for the device-wide sort otherwise; phase 2 finishes those rows and
@@ -439,6 +492,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         FPROF(a, slot, 5);
         // ApplyTopP (Sampler.cs:516-551)
         int big = 0;
+        int listed = -1;  // the row's survivors are sm.sortbuf[0, listed)
         if (use_top_p) {
             int cnt = 0;
             row_pass<false>(p, n, [&](float x, int) -> float { cnt += x > 0.0f ? 1 : 0; return x; });
@@ -489,6 +543,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                         row_pass<true>(p, n, [&](float x, int) -> float { return x > c_above ? x : 0.0f; });
                         __syncthreads();
                     }
+                    listed = cutoff;
                 }
             }
             if (ns > 0 && !closed) {
@@ -497,15 +552,25 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             if (tid == 0) st->n_survivors = ns;
         }
         FPROF(a, slot, 6);
+        // (up to a thousand members: beyond that the passes over the row are the faster way)
+        const bool finish_here = listed > 0 && listed <= 1024 && n >= 8;
         if (tid == 0) {
             st->big = big;
             st->flags = flags;
+            st->pad = finish_here ? 1 : 0;  // 1 = the row is finished in this phase
             a.seg_begin[slot] = (int)((size_t)slot * a.sort_stride);
             a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + (big ? st->n_survivors : 0);
+        }
+        if (finish_here) {
+            // the nucleus closed inside the kernel and its members are at hand: no pass over the row is needed
+            finish_from_list(a, p, n, listed, row, sm);
+            if (tid == 0 && a.out_flags) a.out_flags[row] = flags;
+            return;
         }
         if (a.two_phase) return;
         __syncthreads();
     }
+    if (a.two_phase && st->pad == 1) return;  // finished in phase 1
 
     // ---- phase 2 --------------------------------------------------------------------------------------
     if (a.two_phase && st->big) {

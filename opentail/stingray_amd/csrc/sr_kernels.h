@@ -75,7 +75,7 @@ struct SrFullState {
     int32_t n_survivors;  // entries with probability > 0 when top-p starts
     int32_t big;          // survivors exceed what the row kernel sorts itself: device-wide sort needed
     uint32_t flags;
-    int32_t pad;
+    int32_t pad;          // 1 = the row was finished by the first phase
 };
 
 struct SrFullArgs {

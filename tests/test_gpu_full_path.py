@@ -271,3 +271,22 @@ def test_mtp_accept_draft(ctx):
             ok, pr = orc.mtp_accept_draft(int(draft[r]), int(am[r]), logits[r], p_min)
             assert g_am[r] == am[r] and bool(g_ok[r]) == ok
             assert abs(g_pr[r] - pr) <= 1e-5 * max(pr, 1e-30)
+
+
+def test_nucleus_finished_from_the_list_of_its_members(ctx):
+    # Rows whose nucleus closes inside the kernel are normalised and drawn from the list of their members, not
+    # by passes over the row: vocabulary lengths around multiples of 8 (the overlapped tail of the eight-lane
+    # sum), members inside that tail, a uniform of exactly 0 (index 0 wins whatever it holds) and one just below 1.
+    rng = np.random.default_rng(37)
+    for n in (8, 9, 15, 16, 17, 23, 1000, 1001, 1007, 4099):
+        rows = 6
+        logits = rng.normal(0, 2.0, (rows, n)).astype(np.float32)
+        logits[:, n - 1] += 6.0                               # a member in the last, ragged vector
+        logits[1, 0] = NEG_INF                                # index 0 outside the nucleus
+        logits[2, : n // 2] = NEG_INF
+        params = [SamplingParams(Temperature=float(t), TopK=0, TopP=float(p), MinP=float(mp))
+                  for t, p, mp in zip([1.0, 0.7, 1.3, 1.0, 0.9, 2.0], [0.9, 0.5, 0.95, 0.999, 0.3, 0.97],
+                                      [0.0, 0.0, 0.05, 0.0, 0.02, 0.0])]
+        for u in ([0.0] * rows, [0.99999994] * rows, rng.random(rows).tolist()):
+            _check_rows(ctx, logits, params, u)
+        _check_distribution(ctx, logits, params)
