@@ -20,7 +20,6 @@ constexpr int kW = SR_SEQ_WAVES;
 constexpr int kSmall = SR_FULL_SMALL_CAP;  // survivors sorted inside the kernel
 
 struct FullSmem {
-    uint64_t exp_tab[32];  // copy of the expf table
     SrSeqSmem seq;
     SrSeq8Smem seq8;
     float lane_sum[SR_SEQ_CHAINS];
@@ -284,6 +283,7 @@ __global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
     const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
     const bool scale = rd.temperature > 0.0f && rd.temperature != 1.0f;
     const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+    if (blockIdx.x == 0 && threadIdx.x == 0) a.state[slot].maxkey = 0u;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256) {
         float x = load_logit<ES>(rowp, i);
         if (mrow && !((mrow[i >> 5] >> (i & 31)) & 1u)) x = SR_NEG_INF;
@@ -322,6 +322,43 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
         if (scale) x = __fmul_rn(x, inv_temp);
         w[id] = x;
     }
+}
+
+// ---- stage 2b: the row maximum and expf(x - max) of the sampled rows, spread over the whole device ------
+// (Softmax, Sampler.cs:448-459.)  One workgroup per row would spend most of its time in the double-precision
+// expf of 150 thousand entries; here every row is cut into up to 64 pieces.
+__global__ __launch_bounds__(256) void k_full_max(SrFullArgs a)
+{
+    __shared__ uint32_t wmax[4];
+    const int slot = blockIdx.y;
+    const int row = a.row_list[slot];
+    if (a.rows[row].temperature <= 0.0f) return;  // greedy rows keep their logits
+    const float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    uint32_t k = 0u;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256) {
+        const float v = w[i];
+        const uint32_t kv = (v != v) ? 0xffffffffu : sr_okey(v);  // NaN propagates (TensorPrimitives.Max)
+        k = kv > k ? kv : k;
+    }
+    k = sr_wave_max_u32(k);
+    if (sr_lane() == 0) wmax[sr_wave_id()] = k;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        k = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+        if (k != 0u) atomicMax(&a.state[slot].maxkey, k);
+    }
+}
+__global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
+{
+    const int slot = blockIdx.y;
+    const int row = a.row_list[slot];
+    if (a.rows[row].temperature <= 0.0f) return;
+    const uint32_t mk = a.state[slot].maxkey;
+    if (mk == 0xffffffffu || mk <= 0x007fffffu) return;  // NaN, or nothing above -inf: the row kernel makes it uniform
+    const float m = sr_okey_inv(mk);
+    float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256)
+        w[i] = sr_expf(__fsub_rn(w[i], m));
 }
 
 // ---- argmax of an fp32 row: first index of the maximum, first NaN wins -------------------------------
@@ -434,18 +471,11 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
     }
 
     if (phase == 1) {
-        if (tid < 32) sm.exp_tab[tid] = sr_exp2f_tab[tid];  // published by the barriers of the maximum below
         FPROF(a, slot, 0);
-        // Softmax (Sampler.cs:448-472)
-        float m = SR_NEG_INF;
-        bool nanv = false;
-        row_pass<false>(p, n, [&](float v, int) -> float {
-            if (v != v) nanv = true;
-            m = fmaxf(m, v);
-            return v;
-        });
-        bool any_nan;
-        m = blk_max_f(nanv ? __uint_as_float(0x7fc00000u) : m, &any_nan, sm);
+        // Softmax (Sampler.cs:448-472): the maximum and e = expf(x - max) were computed by the kernels before
+        const uint32_t mk = st->maxkey;
+        const bool any_nan = mk == 0xffffffffu;
+        const float m = mk == 0u ? SR_NEG_INF : sr_okey_inv(mk);
         FPROF(a, slot, 1);
         uint32_t flags = SR_KFLAG_FULL;
         if (any_nan || sr_f2u(m) == 0xff800000u) {
@@ -455,13 +485,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             __syncthreads();
         } else {
             int dummy;
-            const float sum = seq_sum<false>(
-                [&](int i) -> float {
-                    const float e = sr_expf_tab(__fsub_rn(p[i], m), sm.exp_tab);
-                    p[i] = e;
-                    return e;
-                },
-                n, 0.0f, 0.0f, &dummy, sm);
+            const float sum = seq_sum<false>([&](int i) -> float { return p[i]; }, n, 0.0f, 0.0f, &dummy, sm);
             __syncthreads();
             FPROF(a, slot, 2);
             if (sum > 0.0f && sum != 1.0f) {
@@ -775,6 +799,8 @@ hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
         hipLaunchKernelGGL(k_full_prep<4>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(k_full_edits<4>, dim3(n_rows), dim3(256), 0, st, a);
     }
+    hipLaunchKernelGGL(k_full_max, grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL(k_full_exp, grid, dim3(256), 0, st, a);
     return hipGetLastError();
 }
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st)

@@ -76,6 +76,8 @@ struct SrFullState {
     int32_t big;          // survivors exceed what the row kernel sorts itself: device-wide sort needed
     uint32_t flags;
     int32_t pad;          // 1 = the row was finished by the first phase
+    uint32_t maxkey;      // ordered key of the row's largest adjusted logit (0xffffffff = the row holds a NaN)
+    int32_t pad2[3];
 };
 
 struct SrFullArgs {
