@@ -155,6 +155,39 @@ __device__ __forceinline__ float seq_sum(Term term, int n, float s0, float targe
     return s;
 }
 
+// The same over a row in memory: a thread's SR_SEQ_RUN consecutive terms come in with four 16-byte loads when the
+// row is 16-byte aligned (one 4-byte load per term makes every load instruction of a wave touch 64 cache lines).
+template <bool kSearch>
+__device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm)
+{
+    static_assert(SR_SEQ_RUN == 16, "four float4 per thread");
+    float s = s0;
+    *found = -1;
+    const bool aligned = ((uintptr_t)p & 15u) == 0u;
+    for (int base = 0; base < n; base += SR_SEQ_TILE) {
+        float x[SR_SEQ_RUN];
+        const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
+        if (aligned && i0 + SR_SEQ_RUN <= n) {
+            const float4* v = (const float4*)(p + i0);
+            const float4 a0 = v[0], a1 = v[1], a2 = v[2], a3 = v[3];
+            x[0] = a0.x; x[1] = a0.y; x[2] = a0.z; x[3] = a0.w;
+            x[4] = a1.x; x[5] = a1.y; x[6] = a1.z; x[7] = a1.w;
+            x[8] = a2.x; x[9] = a2.y; x[10] = a2.z; x[11] = a2.w;
+            x[12] = a3.x; x[13] = a3.y; x[14] = a3.z; x[15] = a3.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? p[i0 + j] : 0.0f;
+        }
+        int f;
+        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+        if (kSearch && f >= 0) {
+            *found = base + f;
+            return s;
+        }
+    }
+    return s;
+}
+
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
 // ragged tail folded in through an overlapped last vector, pairwise horizontal add.
 template <typename Term>
@@ -381,7 +414,7 @@ __device__ int draw_from_row(const float* p, int n, double u, FullSmem& sm)
 {
     const float r = __double2float_rn(u);
     int found;
-    seq_sum<true>([&](int i) -> float { return p[i]; }, n, 0.0f, r, &found, sm);
+    seq_sum_row<true>(p, n, 0.0f, r, &found, sm);
     return found >= 0 ? found : n - 1;
 }
 
@@ -485,7 +518,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             __syncthreads();
         } else {
             int dummy;
-            const float sum = seq_sum<false>([&](int i) -> float { return p[i]; }, n, 0.0f, 0.0f, &dummy, sm);
+            const float sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm);
             __syncthreads();
             FPROF(a, slot, 2);
             if (sum > 0.0f && sum != 1.0f) {
