@@ -511,6 +511,8 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         const float m = mk == 0u ? SR_NEG_INF : sr_okey_inv(mk);
         FPROF(a, slot, 1);
         uint32_t flags = SR_KFLAG_FULL;
+        bool fused = false;  // scaling, min-p and the count of survivors were done in one pass
+        int survivors = 0;   // ... this thread's share of the count
         if (any_nan || sr_f2u(m) == 0xff800000u) {
             const float uni = n > 0 ? __fdiv_rn(1.0f, (float)n) : 0.0f;
             row_pass<true>(p, n, [&](float, int) -> float { return uni; });
@@ -521,8 +523,25 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             const float sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm);
             __syncthreads();
             FPROF(a, slot, 2);
-            if (sum > 0.0f && sum != 1.0f) {
-                const float inv = __fdiv_rn(1.0f, sum);
+            const bool do_scale = sum > 0.0f && sum != 1.0f;
+            const float inv = do_scale ? __fdiv_rn(1.0f, sum) : 1.0f;
+            if (!(rd.top_k > 0 && rd.top_k < n) && (rd.min_p > 0.0f || use_top_p)) {
+                // No top-k stage in between: the scaling, the min-p cut (Sampler.cs:493-503) and the count of
+                // survivors that top-p starts from share one pass.  The largest probability needs no search: the
+                // largest e is expf(0) = 1, so it is 1 * (1 / sum).
+                const float mp = do_scale ? __fmul_rn(1.0f, inv) : 1.0f;
+                const bool use_min_p = rd.min_p > 0.0f;
+                const float thr = use_min_p ? __fmul_rn(rd.min_p, mp) : 0.0f;
+                int c = 0;
+                row_pass<true>(p, n, [&](float x, int) -> float {
+                    float y = do_scale ? __fmul_rn(x, inv) : x;
+                    if (use_min_p && y < thr) y = 0.0f;
+                    c += y > 0.0f ? 1 : 0;
+                    return y;
+                });
+                survivors = c;
+                fused = true;
+            } else if (do_scale) {
                 row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
             }
             __syncthreads();
@@ -537,7 +556,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         }
         FPROF(a, slot, 4);
         // ApplyMinP (Sampler.cs:493-503)
-        if (rd.min_p > 0.0f) {
+        if (rd.min_p > 0.0f && !fused) {
             float mp = 0.0f;
             row_pass<false>(p, n, [&](float x, int) -> float { mp = fmaxf(mp, x); return x; });
             bool nn;
@@ -551,8 +570,8 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         int big = 0;
         int listed = -1;  // the row's survivors are sm.sortbuf[0, listed)
         if (use_top_p) {
-            int cnt = 0;
-            row_pass<false>(p, n, [&](float x, int) -> float { cnt += x > 0.0f ? 1 : 0; return x; });
+            int cnt = survivors;
+            if (!fused) row_pass<false>(p, n, [&](float x, int) -> float { cnt += x > 0.0f ? 1 : 0; return x; });
             int ns;
             // positions in index order (stable input for the device-wide sort)
             // each thread owns the strided indices tid, tid + kT, ...; a second pass assigns slots per tile
