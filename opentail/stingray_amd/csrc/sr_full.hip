@@ -188,6 +188,45 @@ __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, fl
     return s;
 }
 
+// ... and over the positive part of the difference of two rows (residual resampling)
+template <bool kSearch>
+__device__ __forceinline__ float seq_sum_residual(const float* p, const float* q, int n, float s0, float target, int* found,
+                                                  FullSmem& sm)
+{
+    static_assert(SR_SEQ_RUN == 16, "four float4 per thread");
+    float s = s0;
+    *found = -1;
+    const bool aligned = (((uintptr_t)p | (uintptr_t)q) & 15u) == 0u;
+    auto res = [](float a, float b) -> float {
+        const float r = __fsub_rn(a, b);
+        return r > 0.0f ? r : 0.0f;
+    };
+    for (int base = 0; base < n; base += SR_SEQ_TILE) {
+        float x[SR_SEQ_RUN];
+        const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
+        if (aligned && i0 + SR_SEQ_RUN <= n) {
+            const float4* vp = (const float4*)(p + i0);
+            const float4* vq = (const float4*)(q + i0);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float4 a = vp[k], b = vq[k];
+                x[4 * k] = res(a.x, b.x); x[4 * k + 1] = res(a.y, b.y);
+                x[4 * k + 2] = res(a.z, b.z); x[4 * k + 3] = res(a.w, b.w);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? res(p[i0 + j], q[i0 + j]) : 0.0f;
+        }
+        int f;
+        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+        if (kSearch && f >= 0) {
+            *found = base + f;
+            return s;
+        }
+    }
+    return s;
+}
+
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
 // ragged tail folded in through an overlapped last vector, pairwise horizontal add.
 template <typename Term>
@@ -692,7 +731,7 @@ __device__ int resample_residual_row(const float* p, const float* q, int n, doub
         const float r = __fsub_rn(p[i], q[i]);
         return r > 0.0f ? r : 0.0f;
     };
-    const float sum = seq_sum<false>(res, n, 0.0f, 0.0f, &dummy, sm);
+    const float sum = seq_sum_residual<false>(p, q, n, 0.0f, 0.0f, &dummy, sm);
     if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm);  // sum <= 0 or NaN
     const float target = __fmul_rn(__double2float_rn(u), sum);
     // `target <= cum` is only tested on positive residuals: a zero target must not stop on a zero term
@@ -710,7 +749,7 @@ __device__ int resample_residual_row(const float* p, const float* q, int n, doub
         __syncthreads();
         return f;  // sum > 0 guarantees a positive residual exists
     }
-    seq_sum<true>(res, n, 0.0f, target, &found, sm);
+    seq_sum_residual<true>(p, q, n, 0.0f, target, &found, sm);
     if (found >= 0) return found;
     // rounding fallback: the last index with a positive residual
     int last = -1;
