@@ -156,16 +156,38 @@ __device__ __forceinline__ float seq_sum(Term term, int n, float s0, float targe
 }
 
 // The same over a row in memory: a thread's SR_SEQ_RUN consecutive terms come in with four 16-byte loads when the
-// row is 16-byte aligned (one 4-byte load per term makes every load instruction of a wave touch 64 cache lines).
+// row is 16-byte aligned (one 4-byte load per term makes every load instruction of a wave touch 64 cache lines),
+// and the loads of the next tile are in flight while the current one is scanned.
+template <bool kSearch, typename Load>
+__device__ __forceinline__ float seq_sum_tiles(Load load, int n, float s0, float target, int* found, FullSmem& sm)
+{
+    float s = s0;
+    *found = -1;
+    float x[SR_SEQ_RUN];
+    if (n > 0) load(0, x);
+    for (int base = 0; base < n; base += SR_SEQ_TILE) {
+        float nx[SR_SEQ_RUN];
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) nx[j] = 0.0f;
+        if (base + SR_SEQ_TILE < n) load(base + SR_SEQ_TILE, nx);
+        int f;
+        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+        if (kSearch && f >= 0) {
+            *found = base + f;
+            return s;
+        }
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = nx[j];
+    }
+    return s;
+}
+
 template <bool kSearch>
 __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm)
 {
     static_assert(SR_SEQ_RUN == 16, "four float4 per thread");
-    float s = s0;
-    *found = -1;
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
-    for (int base = 0; base < n; base += SR_SEQ_TILE) {
-        float x[SR_SEQ_RUN];
+    auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
         const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
         if (aligned && i0 + SR_SEQ_RUN <= n) {
             const float4* v = (const float4*)(p + i0);
@@ -178,14 +200,8 @@ __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, fl
 #pragma unroll
             for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? p[i0 + j] : 0.0f;
         }
-        int f;
-        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
-        if (kSearch && f >= 0) {
-            *found = base + f;
-            return s;
-        }
-    }
-    return s;
+    };
+    return seq_sum_tiles<kSearch>(load, n, s0, target, found, sm);
 }
 
 // ... and over the positive part of the difference of two rows (residual resampling)
@@ -194,37 +210,28 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
                                                   FullSmem& sm)
 {
     static_assert(SR_SEQ_RUN == 16, "four float4 per thread");
-    float s = s0;
-    *found = -1;
     const bool aligned = (((uintptr_t)p | (uintptr_t)q) & 15u) == 0u;
     auto res = [](float a, float b) -> float {
         const float r = __fsub_rn(a, b);
         return r > 0.0f ? r : 0.0f;
     };
-    for (int base = 0; base < n; base += SR_SEQ_TILE) {
-        float x[SR_SEQ_RUN];
+    auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
         const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
         if (aligned && i0 + SR_SEQ_RUN <= n) {
             const float4* vp = (const float4*)(p + i0);
             const float4* vq = (const float4*)(q + i0);
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float4 a = vp[k], b = vq[k];
-                x[4 * k] = res(a.x, b.x); x[4 * k + 1] = res(a.y, b.y);
-                x[4 * k + 2] = res(a.z, b.z); x[4 * k + 3] = res(a.w, b.w);
-            }
+            const float4 a0 = vp[0], a1 = vp[1], a2 = vp[2], a3 = vp[3];
+            const float4 b0 = vq[0], b1 = vq[1], b2 = vq[2], b3 = vq[3];
+            x[0] = res(a0.x, b0.x); x[1] = res(a0.y, b0.y); x[2] = res(a0.z, b0.z); x[3] = res(a0.w, b0.w);
+            x[4] = res(a1.x, b1.x); x[5] = res(a1.y, b1.y); x[6] = res(a1.z, b1.z); x[7] = res(a1.w, b1.w);
+            x[8] = res(a2.x, b2.x); x[9] = res(a2.y, b2.y); x[10] = res(a2.z, b2.z); x[11] = res(a2.w, b2.w);
+            x[12] = res(a3.x, b3.x); x[13] = res(a3.y, b3.y); x[14] = res(a3.z, b3.z); x[15] = res(a3.w, b3.w);
         } else {
 #pragma unroll
             for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? res(p[i0 + j], q[i0 + j]) : 0.0f;
         }
-        int f;
-        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
-        if (kSearch && f >= 0) {
-            *found = base + f;
-            return s;
-        }
-    }
-    return s;
+    };
+    return seq_sum_tiles<kSearch>(load, n, s0, target, found, sm);
 }
 
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
@@ -243,15 +250,29 @@ __device__ float tp_sum(Term term, int n, FullSmem& sm)
         const bool extra = rem > 0 && g >= 8 - rem;
         const int cnt = nv + (extra ? 1 : 0);
         float s = 0.0f;
-        for (int base = 0; base < nv + 1; base += SR_SEQ_CHAIN_TILE) {
-            float x[SR_SEQ_RUN];
+        auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
             const int i0 = base + lt * SR_SEQ_RUN;
+            if (i0 + SR_SEQ_RUN <= nv) {
 #pragma unroll
-            for (int j = 0; j < SR_SEQ_RUN; j++) {
-                const int i = i0 + j;
-                x[j] = (i < cnt) ? (i < nv ? term(i * 8 + g) : term(n - 8 + g)) : 0.0f;
+                for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = term((i0 + j) * 8 + g);
+            } else {
+#pragma unroll
+                for (int j = 0; j < SR_SEQ_RUN; j++) {
+                    const int i = i0 + j;
+                    x[j] = (i < cnt) ? (i < nv ? term(i * 8 + g) : term(n - 8 + g)) : 0.0f;
+                }
             }
+        };
+        float x[SR_SEQ_RUN];
+        load(0, x);
+        for (int base = 0; base < nv + 1; base += SR_SEQ_CHAIN_TILE) {
+            float nx[SR_SEQ_RUN];
+#pragma unroll
+            for (int j = 0; j < SR_SEQ_RUN; j++) nx[j] = 0.0f;
+            if (base + SR_SEQ_CHAIN_TILE < nv + 1) load(base + SR_SEQ_CHAIN_TILE, nx);
             sr_seq_tile8(x, &s, sm.seq8);
+#pragma unroll
+            for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = nx[j];
         }
         __syncthreads();
         if (lt == 0) sm.lane_sum[g] = s;

@@ -27,13 +27,11 @@
 #define SR_SEQ_SAT (1u << 26)  // saturated increment: "this run leaves the binade"
 
 struct SrSeqSmem {
-    uint32_t wa0[SR_SEQ_WAVES];
+    uint32_t wa0[SR_SEQ_WAVES];  // every wave's increment function ...
     uint32_t wa1[SR_SEQ_WAVES];
-    uint32_t pa0[SR_SEQ_WAVES + 1];  // exclusive prefix of every wave, then the block total
-    uint32_t pa1[SR_SEQ_WAVES + 1];
     uint32_t misc[8];
-    int first[SR_SEQ_WAVES];
 };
+static_assert(SR_SEQ_WAVES == 16, "the wave totals are scanned inside one DPP row of 16 lanes");
 
 // n -> n + a[n & 1]
 struct SrInc {
@@ -85,22 +83,56 @@ __device__ __forceinline__ SrInc sr_run_inc(const float (&x)[SR_SEQ_RUN], int eb
     return r;
 }
 
+// Inclusive scan of increment functions: DPP shifts with zero fill inside rows of 16 lanes ((0, 0) is the identity
+// of sr_compose), v_readlane for the rows before.  With kRowOnly the rows stay separate.
+template <bool kRowOnly>
+__device__ __forceinline__ SrInc sr_scan_inc(SrInc v)
+{
+    auto step = [&](auto ctrl) {
+        constexpr int kC = decltype(ctrl)::value;
+        SrInc lo;
+        lo.a0 = sr_dpp_u32<kC>(v.a0);
+        lo.a1 = sr_dpp_u32<kC>(v.a1);
+        v = sr_compose(lo, v);
+    };
+    step(std::integral_constant<int, 0x111>{});
+    step(std::integral_constant<int, 0x112>{});
+    step(std::integral_constant<int, 0x114>{});
+    step(std::integral_constant<int, 0x118>{});
+    if (kRowOnly) return v;
+    auto total = [&](int l) {
+        SrInc t;
+        t.a0 = (uint32_t)__builtin_amdgcn_readlane((int)v.a0, l);
+        t.a1 = (uint32_t)__builtin_amdgcn_readlane((int)v.a1, l);
+        return t;
+    };
+    const SrInc p1 = total(15), p2 = sr_compose(p1, total(31)), p3 = sr_compose(p2, total(47));
+    const int row = sr_lane() >> 4;
+    SrInc pre;
+    pre.a0 = row == 1 ? p1.a0 : row == 2 ? p2.a0 : row == 3 ? p3.a0 : 0u;
+    pre.a1 = row == 1 ? p1.a1 : row == 2 ? p2.a1 : row == 3 ? p3.a1 : 0u;
+    return sr_compose(pre, v);
+}
+
 // One tile: adds this thread's SR_SEQ_RUN terms (thread order = term order) to the running sum *s
 // (uniform across the block on entry and exit).  When kSearch, also looks for the first term index at
 // which the running sum reaches `target` (fl(s) >= target); on success returns its tile-local index
 // (thread * SR_SEQ_RUN + j) in *found (uniform), else leaves -1.  Terms past the end must be 0.
 //
-// Per round: every wave scans its threads' increment functions; the first wave scans the wave totals, which
-// also shows the first wave in which the sum leaves the binade (or reaches the target); that wave alone finds
-// the thread and replays its run with real float adds; everything after it is rescanned in the new binade.
+// Per round: every wave scans its threads' increment functions and publishes its total; every wave then scans the
+// sixteen totals itself, which also shows the first wave in which the sum leaves the binade (or reaches the
+// target); that wave alone finds the thread and replays its run with real float adds; everything after it is
+// rescanned in the new binade.  A tile that stays in its binade costs two barriers.
 template <bool kSearch>
 __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float* s, float target, int* found,
                                             SrSeqSmem& sm)
 {
-    const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
+    const int tid = threadIdx.x, lane = sr_lane();
+    const int wave = __builtin_amdgcn_readfirstlane(sr_wave_id());
     int start = 0;  // threads below `start` are settled
     float s_in = *s;
     *found = -1;
+    __syncthreads();  // the previous call's readers are done with the arrays below
     for (;;) {
         uint32_t n_in;
         int eb;
@@ -108,51 +140,32 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
         SrInc mine;
         mine.a0 = 0u; mine.a1 = 0u;
         if (tid >= start) mine = sr_run_inc(x, eb);
-        SrInc incl = mine;
-#pragma unroll
-        for (int o = 1; o < SR_WAVE; o <<= 1) {
-            SrInc lo;
-            lo.a0 = __shfl_up(incl.a0, o);
-            lo.a1 = __shfl_up(incl.a1, o);
-            if (lane >= o) incl = sr_compose(lo, incl);
-        }
-        __syncthreads();  // the previous round's readers are done with the arrays below
+        const SrInc incl = sr_scan_inc<false>(mine);
+        // (a later round writes after the barrier that ends this one, when every read below is done)
         if (lane == SR_WAVE - 1) { sm.wa0[wave] = incl.a0; sm.wa1[wave] = incl.a1; }
         __syncthreads();
-        if (wave == 0) {
-            SrInc ti; ti.a0 = 0u; ti.a1 = 0u;
-            if (lane < SR_SEQ_WAVES) { ti.a0 = sm.wa0[lane]; ti.a1 = sm.wa1[lane]; }
-#pragma unroll
-            for (int o = 1; o < SR_SEQ_WAVES; o <<= 1) {
-                SrInc lo;
-                lo.a0 = __shfl_up(ti.a0, o);
-                lo.a1 = __shfl_up(ti.a1, o);
-                if (lane >= o) ti = sr_compose(lo, ti);
-            }
-            // state at the end of every wave; the running value never decreases, so the first wave whose end
-            // state has left the binade (or reached the target) holds the first such thread
-            const uint32_t end_n = sr_sat_add(n_in, (n_in & 1u) ? ti.a1 : ti.a0);
-            bool event = end_n >= (1u << 24);
-            if (kSearch) event = event || sr_join(end_n, eb) >= target;
-            const unsigned long long ev = __ballot(event && lane < SR_SEQ_WAVES);
-            SrInc te;
-            te.a0 = __shfl_up(ti.a0, 1);
-            te.a1 = __shfl_up(ti.a1, 1);
-            if (lane == 0) { te.a0 = 0u; te.a1 = 0u; }
-            if (lane < SR_SEQ_WAVES) { sm.pa0[lane] = te.a0; sm.pa1[lane] = te.a1; }
-            if (lane == SR_SEQ_WAVES - 1) { sm.pa0[SR_SEQ_WAVES] = ti.a0; sm.pa1[SR_SEQ_WAVES] = ti.a1; }
-            if (lane == 0) sm.first[0] = ev ? (int)__ffsll((long long)ev) - 1 : -1;
-        }
-        __syncthreads();
-        const int ev_wave = sm.first[0];
-        if (ev_wave < 0) {
+        SrInc ti; ti.a0 = 0u; ti.a1 = 0u;
+        if (lane < SR_SEQ_WAVES) { ti.a0 = sm.wa0[lane]; ti.a1 = sm.wa1[lane]; }
+        ti = sr_scan_inc<true>(ti);  // lanes 0..15: the state function at the end of every wave
+        // the running value never decreases, so the first wave whose end state has left the binade (or reached
+        // the target) holds the first such thread
+        const uint32_t end_n = sr_sat_add(n_in, (n_in & 1u) ? ti.a1 : ti.a0);
+        bool event = end_n >= (1u << 24);
+        if (kSearch) event = event || sr_join(end_n, eb) >= target;
+        const unsigned long long ev = __ballot(event && lane < SR_SEQ_WAVES);
+        if (!ev) {
             // the whole remainder stays in the binade: settle with the block total
-            const uint32_t tot = (n_in & 1u) ? sm.pa1[SR_SEQ_WAVES] : sm.pa0[SR_SEQ_WAVES];
+            const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)((n_in & 1u) ? ti.a1 : ti.a0), SR_SEQ_WAVES - 1);
             *s = sr_join(n_in + tot, eb);
             return;
         }
+        const int ev_wave = (int)__ffsll((long long)ev) - 1;
         if (wave == ev_wave) {
-            SrInc pre; pre.a0 = sm.pa0[wave]; pre.a1 = sm.pa1[wave];
+            SrInc pre; pre.a0 = 0u; pre.a1 = 0u;
+            if (wave > 0) {
+                pre.a0 = (uint32_t)__builtin_amdgcn_readlane((int)ti.a0, wave - 1);
+                pre.a1 = (uint32_t)__builtin_amdgcn_readlane((int)ti.a1, wave - 1);
+            }
             SrInc ex;
             ex.a0 = __shfl_up(incl.a0, 1);
             ex.a1 = __shfl_up(incl.a1, 1);
@@ -162,10 +175,10 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
             const uint32_t before = sr_sat_add(n_in, (n_in & 1u) ? ex.a1 : ex.a0);
             const SrInc thr = sr_compose(ex, mine);
             const uint32_t after = sr_sat_add(n_in, (n_in & 1u) ? thr.a1 : thr.a0);
-            bool event = after >= (1u << 24);
-            if (kSearch) event = event || sr_join(after, eb) >= target;
-            const unsigned long long ev = __ballot(event && tid >= start);
-            const int fl = ev ? (int)__ffsll((long long)ev) - 1 : SR_WAVE - 1;  // ev != 0 by construction
+            bool mine_ev = after >= (1u << 24);
+            if (kSearch) mine_ev = mine_ev || sr_join(after, eb) >= target;
+            const unsigned long long evl = __ballot(mine_ev && tid >= start);
+            const int fl = evl ? (int)__ffsll((long long)evl) - 1 : SR_WAVE - 1;  // evl != 0 by construction
             if (lane == fl) {
                 // replay this run with real float adds from its exact input
                 float acc = sr_join(before, eb);
