@@ -65,7 +65,7 @@ enum {
     SR_OUT_PATH_TOPK_FAST = 1u << 1,   /* SampleTopK (Sampler.cs:216-357)                       */
     SR_OUT_PATH_FULL_VOCAB = 1u << 2,  /* slow path (Sampler.cs:41-95)                          */
     SR_OUT_DEGENERATE = 1u << 3,       /* all -inf row: greedy / uniform fallback was taken     */
-    SR_OUT_ROW_UNSUPPORTED = 1u << 31  /* row exceeded a kernel limit; its token is -1          */
+    SR_OUT_ROW_UNSUPPORTED = 1u << 31  /* thousands of equal logits at the top-k cut: token is -1 */
 };
 
 /*

@@ -203,7 +203,7 @@ void sr_batch_destroy(sr_batch* b)
 {
     if (!b) return;
     if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
-    DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_scan_desc,
+    DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_wide_list, &b->d_scan_desc,
                          &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched};
     for (DeviceBuf* d : bufs) d->release();
     delete b;
@@ -237,6 +237,7 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
     b->h_edits.clear();
     b->h_sel_list.clear();
     b->h_full_list.clear();
+    b->h_wide_list.clear();
     b->h_scan.clear();
     b->h_scan_need.assign((size_t)rows, 0u);
     b->scan_epv = 0;
@@ -334,6 +335,13 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         // id.  GreedyWithHistoryPenalties changes history ids only, whatever the sign.  Penalties that may
         // raise a logit keep the reference's over-selection by the history length (Sampler.cs:224-225).
         const bool lowering = p.repetition_penalty >= 1.0f && p.presence_penalty >= 0.0f && p.frequency_penalty >= 0.0f;
+        if (d.path == SR_PATH_TOPK) {
+            // The selection kernel's row tail sorts up to SR_TK_SEL_MAX entries: the k best outside the history plus
+            // the history ids (lowering penalties), or the k + history-length best (penalties that may raise).
+            const bool excl = has_penalty && d.edit_cnt > 0 && lowering;
+            const int64_t need = excl ? (int64_t)p.top_k + d.edit_cnt : (d.edit_cnt == 0 ? (int64_t)p.top_k : (int64_t)d.sel);
+            if (need > SR_TK_SEL_MAX || d.edit_cnt > SR_TK_SEL_MAX) d.path = SR_PATH_TOPK_WIDE;  // d.sel stays k + history length
+        }
         if (has_penalty && d.edit_cnt > 0 &&
             (d.path == SR_PATH_GREEDY_PEN || (d.path == SR_PATH_TOPK && lowering))) {
             d.flags |= SR_ROWFLAG_HIST_EXCL;
@@ -342,7 +350,9 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         } else if (d.path == SR_PATH_TOPK && d.edit_cnt == 0) {
             d.sel = p.top_k;  // no history id inside the vocabulary: nothing is ever penalised
         }
-        if (d.path != SR_PATH_FULL) {
+        if (d.path == SR_PATH_TOPK_WIDE) {
+            b->h_wide_list.push_back(r);
+        } else if (d.path != SR_PATH_FULL) {
             if (d.mask_row >= 0) b->h_scan_need[(size_t)r] |= SR_SCAN_ALLOW;
             b->h_sel_list.push_back(r);
             b->max_sel = std::max(b->max_sel, d.sel);
@@ -367,6 +377,7 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
     SR_HIP(ctx, up(b->d_edits, b->h_edits.data(), b->h_edits.size() * sizeof(SrEdit)));
     SR_HIP(ctx, up(b->d_sel_list, b->h_sel_list.data(), b->h_sel_list.size() * sizeof(int32_t)));
     SR_HIP(ctx, up(b->d_full_list, b->h_full_list.data(), b->h_full_list.size() * sizeof(int32_t)));
+    SR_HIP(ctx, up(b->d_wide_list, b->h_wide_list.data(), b->h_wide_list.size() * sizeof(int32_t)));
     if (allow_mask) SR_HIP(ctx, up(b->d_mask, allow_mask, (size_t)rows * (size_t)mask_stride_words * sizeof(uint32_t)));
     if (uniforms_per_row > 0)
         SR_HIP(ctx, up(b->d_uniforms, uniforms, (size_t)rows * (size_t)uniforms_per_row * sizeof(double)));
@@ -454,6 +465,10 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
     }
     if (!b->h_full_list.empty()) {
         int rc = sr_full_rows_launch(ctx, b, logits_dev, dtype, row_stride_elems, out_tokens_dev, out_flags_dev);
+        if (rc != SR_OK) return rc;
+    }
+    if (!b->h_wide_list.empty()) {
+        int rc = sr_wide_rows_launch(ctx, b, logits_dev, dtype, row_stride_elems, out_tokens_dev, out_flags_dev);
         if (rc != SR_OK) return rc;
     }
     return SR_OK;

@@ -733,6 +733,134 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
     if (tid == 0 && a.out_flags) a.out_flags[row] = st->flags;
 }
 
+// ---- SampleTopK (Sampler.cs:216-357) for rows wider than the selection kernel takes -----------------------
+// The reference keeps the k + history-length largest raw logits (earlier index first among equals), applies the
+// history penalties to those, orders them again (stable), and samples among the first k.  Here the whole row is
+// sorted device-wide by (raw logit descending, index ascending), the first `sel` entries are adjusted and sorted
+// again, and one workgroup per row walks the result.
+template <int ES>
+__global__ __launch_bounds__(256) void k_wide_keys(SrFullArgs a)
+{
+    const int slot = blockIdx.y;
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+    const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+    uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
+    int32_t* ids = a.sort_vals_in + (size_t)slot * a.sort_stride;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        a.seg_begin[slot] = (int)((size_t)slot * a.sort_stride);
+        a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + a.vocab;
+    }
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256) {
+        float x = load_logit<ES>(rowp, i);
+        if (mrow && !((mrow[i >> 5] >> (i & 31)) & 1u)) x = SR_NEG_INF;
+        keys[i] = sr_okey(x);
+        ids[i] = i;
+    }
+}
+
+// the first `sel` sorted entries with the history penalties of SampleTopK applied (Sampler.cs:262-297); entries
+// that hold -inf are the reference's unfilled slots (index -1)
+__global__ __launch_bounds__(256) void k_wide_adjust(SrFullArgs a)
+{
+    const int slot = blockIdx.y;
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    const uint32_t* skeys = a.sort_keys_out + (size_t)slot * a.sort_stride;
+    const int32_t* sids = a.sort_vals_out + (size_t)slot * a.sort_stride;
+    uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
+    int32_t* ids = a.sort_vals_in + (size_t)slot * a.sort_stride;
+    const int sel = min(rd.sel, a.vocab);
+    if (blockIdx.x == 0 && threadIdx.x == 0) a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + sel;
+    const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u && rd.edit_cnt > 0;
+    const SrEdit* ed = a.edits + rd.edit_off;
+    for (int t = blockIdx.x * 256 + threadIdx.x; t < sel; t += gridDim.x * 256) {
+        float v = sr_okey_inv(skeys[t]);
+        int id = sids[t];
+        if (sr_f2u(v) == 0xff800000u) {
+            id = -1;
+        } else if (pen) {
+            int lo = 0, hi = rd.edit_cnt;
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (ed[mid].id < id) lo = mid + 1; else hi = mid;
+            }
+            if (lo < rd.edit_cnt && ed[lo].id == id && ed[lo].occ_all > 0) {
+                const SrEdit ee = ed[lo];
+                if (rd.rep != 1.0f && ee.occ_win > 0) v = v > 0.0f ? __fdiv_rn(v, ee.pen) : __fmul_rn(v, ee.pen);
+                v = __fsub_rn(v, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ee.occ_all)));
+            }
+        }
+        keys[t] = sr_okey(v);
+        ids[t] = id;
+    }
+}
+
+// temperature softmax over the first k entries, min-p, top-p and the draw, all left to right (Sampler.cs:299-356)
+__global__ __launch_bounds__(kT) void k_wide_tail(SrFullArgs a)
+{
+    __shared__ FullSmem sm;
+    const int tid = threadIdx.x;
+    const int slot = blockIdx.x;
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    const uint32_t* keys = a.sort_keys_out + (size_t)slot * a.sort_stride;
+    const int32_t* ids = a.sort_vals_out + (size_t)slot * a.sort_stride;
+    float* probs = a.work + (size_t)slot * a.work_stride;
+    const int k = min(rd.top_k, min(rd.sel, a.vocab));
+    const float v0 = sr_okey_inv(keys[0]);
+    const int id0 = ids[0];
+    if (id0 < 0 || sr_f2u(v0) == 0xff800000u) {
+        // nothing above -inf (Sampler.cs:254-255): Greedy over a row of -inf returns index 0
+        if (tid == 0) {
+            a.out_tokens[row] = 0;
+            if (a.out_flags) a.out_flags[row] = SR_KFLAG_TOPK | SR_KFLAG_DEGENERATE;
+        }
+        return;
+    }
+    const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
+    const float mx = __fmul_rn(v0, inv_temp);
+    for (int t = tid; t < k; t += kT) {
+        const float v = sr_okey_inv(keys[t]);
+        probs[t] = sr_f2u(v) == 0xff800000u ? 0.0f : sr_expf(__fsub_rn(__fmul_rn(v, inv_temp), mx));
+    }
+    __syncthreads();
+    int found;
+    const float sum = seq_sum_row<false>(probs, k, 0.0f, 0.0f, &found, sm);
+    const float inv_sum = sum > 0.0f ? __fdiv_rn(1.0f, sum) : 0.0f;
+    __syncthreads();
+    row_pass<true>(probs, k, [&](float x, int) -> float { return __fmul_rn(x, inv_sum); });
+    __syncthreads();
+    int count = k;
+    if (rd.min_p > 0.0f) {
+        const float thr = __fmul_rn(rd.min_p, probs[0]);
+        unsigned long long first = 0ull;  // ~index of the first entry below the threshold
+        row_pass<false>(probs, k, [&](float x, int i) -> float {
+            if (x < thr) {
+                const unsigned long long e = 0xffffffffull - (unsigned long long)(uint32_t)i;
+                first = e > first ? e : first;
+            }
+            return x;
+        });
+        first = blk_max_u64(first, sm);
+        if (first) count = (int)(0xffffffffull - first);
+    }
+    if (rd.top_p < 1.0f && rd.top_p > 0.0f) {
+        seq_sum_row<true>(probs, count, 0.0f, rd.top_p, &found, sm);
+        if (found >= 0) count = found + 1;
+    }
+    const float kept = seq_sum_row<false>(probs, count, 0.0f, 0.0f, &found, sm);
+    const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept);
+    seq_sum_row<true>(probs, count, 0.0f, r, &found, sm);
+    if (tid == 0) {
+        int token = id0;
+        if (found >= 0 && ids[found] >= 0) token = ids[found];
+        a.out_tokens[row] = token;
+        if (a.out_flags) a.out_flags[row] = SR_KFLAG_TOPK;
+    }
+}
+
 // ---- SampleFromProbs / ResampleResidual on caller-provided distributions ------------------------------
 __global__ __launch_bounds__(kT) void k_draw_rows(const float* probs, int64_t stride, int n, const double* uniforms,
                                                    int* out_tokens)
@@ -913,6 +1041,26 @@ hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
     }
     hipLaunchKernelGGL(k_full_max, grid, dim3(256), 0, st, a);
     hipLaunchKernelGGL(k_full_exp, grid, dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+hipError_t sr_launch_wide_keys(const SrFullArgs& a, int n_rows, hipStream_t st)
+{
+    if (n_rows <= 0) return hipSuccess;
+    dim3 grid(max(1, min(64, (a.vocab + 256 * 16 - 1) / (256 * 16))), n_rows);
+    if (a.dtype == 1) hipLaunchKernelGGL(k_wide_keys<2>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(k_wide_keys<4>, grid, dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+hipError_t sr_launch_wide_adjust(const SrFullArgs& a, int n_rows, hipStream_t st)
+{
+    if (n_rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_wide_adjust, dim3(32, n_rows), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+hipError_t sr_launch_wide_tail(const SrFullArgs& a, int n_rows, hipStream_t st)
+{
+    if (n_rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_wide_tail, dim3(n_rows), dim3(kT), 0, st, a);
     return hipGetLastError();
 }
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st)

@@ -70,9 +70,10 @@ struct sr_batch {
     std::vector<SrEdit> h_edits;
     std::vector<int32_t> h_sel_list;   // rows on the selection kernel: TOPK and plain GREEDY
     std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path
+    std::vector<int32_t> h_wide_list;  // SampleTopK rows too wide for the selection kernel
     std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel
     std::vector<uint32_t> h_scan_need; // per batch row: SR_SCAN_* bits the row's scan mask must carry
-    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms, d_sched;
+    DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_wide_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms, d_sched;
     int64_t mask_stride = 0, scan_stride = 0;
     // what the scan masks were built for: elements per 16-byte vector, the logits base address modulo 16 and
     // the row stride in bytes modulo 16 (rows share a mask row only when all start at the same offset)
@@ -99,4 +100,7 @@ inline int sr_fail_hip(sr_ctx* ctx, hipError_t e, const char* what)
 // Full-vocabulary rows of a batch (sr_full_host.cpp).  mode: 0 = sample, 1 = build distribution,
 // 2 = build distribution and sample from it.
 int sr_full_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
+                        int32_t* out_tokens_dev, uint32_t* out_flags_dev);
+// SampleTopK for the rows of b->h_wide_list (sr_full_host.cpp)
+int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
                         int32_t* out_tokens_dev, uint32_t* out_flags_dev);

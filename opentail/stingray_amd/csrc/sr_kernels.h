@@ -111,6 +111,11 @@ struct SrFullArgs {
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st);
+// SampleTopK by device-wide sorts (rows beyond the selection kernel's limits): keys of the whole row, the adjusted
+// first `sel` entries, the walk over the sorted result
+hipError_t sr_launch_wide_keys(const SrFullArgs& a, int n_rows, hipStream_t st);
+hipError_t sr_launch_wide_adjust(const SrFullArgs& a, int n_rows, hipStream_t st);
+hipError_t sr_launch_wide_tail(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_draw_rows(const float* probs, int64_t stride, int n, int rows, const double* u, int* out,
                                hipStream_t st);
 hipError_t sr_launch_residual_rows(const float* p, int64_t ps, const float* q, int64_t qs, int n, int rows,

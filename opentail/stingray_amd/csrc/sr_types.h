@@ -7,7 +7,8 @@ enum SrPath : int32_t {
     SR_PATH_GREEDY = 0,      // Temperature <= 0, no history penalty      -> Greedy(masked logits)
     SR_PATH_GREEDY_PEN = 1,  // Temperature <= 0 with history penalties   -> GreedyWithHistoryPenalties
     SR_PATH_TOPK = 2,        // 0 < TopK < vocab and no logit bias        -> SampleTopK
-    SR_PATH_FULL = 3         // everything else                           -> full-vocabulary pipeline
+    SR_PATH_FULL = 3,        // everything else                           -> full-vocabulary pipeline
+    SR_PATH_TOPK_WIDE = 4    // SampleTopK beyond the selection kernel's limits -> device-wide sort of the row
 };
 
 struct SrRow {
