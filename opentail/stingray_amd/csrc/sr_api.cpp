@@ -75,35 +75,53 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
         // last chunk: half of that round's workgroups have retired by the time it is dispatched, so its chunks have
         // usually finished and it does not hold a slot while it waits, yet it does not queue behind all of the
         // later rows' chunks either.  Every entry carries what its workgroup needs to find its data.
-        const int round = 2 * ctx->cu_count;
-        std::vector<int32_t> sched;
-        sched.reserve((size_t)n_sel * (size_t)(chunks + 1) * 4);
-        auto push = [&](uint32_t item, int slot) {
-            const int32_t r = b->h_sel_list[(size_t)slot];
-            sched.push_back((int32_t)item);
-            sched.push_back(r);
-            sched.push_back(b->h_rows[(size_t)r].scan_row);
-            sched.push_back(b->h_rows[(size_t)r].sel);
-        };
-        std::vector<int> ready_at((size_t)n_sel, 0);  // first position at which the row's tail may be placed
-        int next_tail = 0, row = 0, c = 0;
-        while (next_tail < n_sel) {
-            const int pos = (int)(sched.size() / 4);
-            if (next_tail < row && pos >= ready_at[(size_t)next_tail]) {
-                push(0x80000000u | (uint32_t)next_tail, next_tail);
-                next_tail++;
-            } else if (row < n_sel) {
-                push(((uint32_t)c << 24) | (uint32_t)row, row);
-                if (++c == chunks) {
-                    ready_at[(size_t)row] = (pos / round + 1) * round + round / 2;
-                    c = 0;
-                    row++;
+        //
+        // The device's compute dies (XCDs, 32 CUs and one L2 each) take the workgroups of a grid in turn: workgroup i
+        // runs on die i mod n_xcd.  Row slot s is given to die s mod n_xcd and the order above is built per die, so
+        // that what a row's chunk workgroups write is in the L2 that its tail reads from.  Nothing depends on that
+        // placement for correctness.
+        const int n_xcd = std::max(1, ctx->cu_count / 32);
+        const int round = std::max(2, 2 * ctx->cu_count / n_xcd);
+        std::vector<std::vector<int32_t>> queue((size_t)n_xcd);
+        size_t longest = 0;
+        for (int x = 0; x < n_xcd; x++) {
+            std::vector<int32_t>& q = queue[(size_t)x];
+            auto push = [&](uint32_t item, int slot) {
+                const int32_t r = b->h_sel_list[(size_t)slot];
+                q.push_back((int32_t)item);
+                q.push_back(r);
+                q.push_back(b->h_rows[(size_t)r].scan_row);
+                q.push_back(b->h_rows[(size_t)r].sel);
+            };
+            const int n_mine = n_sel > x ? (n_sel - x + n_xcd - 1) / n_xcd : 0;  // slots x, x + n_xcd, ...
+            std::vector<int> ready_at((size_t)n_mine, 0);  // first position at which the row's tail may be placed
+            int next_tail = 0, row = 0, c = 0;
+            while (next_tail < n_mine) {
+                const int pos = (int)(q.size() / 4);
+                const int tail_slot = x + next_tail * n_xcd, row_slot = x + row * n_xcd;
+                if (next_tail < row && pos >= ready_at[(size_t)next_tail]) {
+                    push(0x80000000u | (uint32_t)tail_slot, tail_slot);
+                    next_tail++;
+                } else if (row < n_mine) {
+                    push(((uint32_t)c << 24) | (uint32_t)row_slot, row_slot);
+                    if (++c == chunks) {
+                        ready_at[(size_t)row] = (pos / round + 1) * round + round / 2;
+                        c = 0;
+                        row++;
+                    }
+                } else {
+                    push(0x80000000u | (uint32_t)tail_slot, tail_slot);  // nothing left to overlap with
+                    next_tail++;
                 }
-            } else {
-                push(0x80000000u | (uint32_t)next_tail, next_tail);  // nothing left to overlap with
-                next_tail++;
             }
+            longest = std::max(longest, q.size() / 4);
         }
+        // interleave the dies' queues; a die with fewer rows gets entries that end at once
+        std::vector<int32_t> sched(longest * (size_t)n_xcd * 4, -1);
+        for (int x = 0; x < n_xcd; x++)
+            for (size_t i = 0; i < queue[(size_t)x].size() / 4; i++)
+                for (int w = 0; w < 4; w++) sched[(i * (size_t)n_xcd + (size_t)x) * 4 + (size_t)w] = queue[(size_t)x][i * 4 + (size_t)w];
+        b->sched_len = (int32_t)(longest * (size_t)n_xcd);
         SR_HIP(ctx, b->d_sched.reserve(sched.size() * sizeof(int32_t), st));
         SR_HIP(ctx, hipMemcpyAsync(b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
         SR_HIP(ctx, hipStreamSynchronize(st));
@@ -438,6 +456,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         if (a.chunks > SR_TK_MAX_CHUNKS)
             return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary too large for the selection kernel");
         a.sched = b->d_sched.as<int4>();
+        a.n_wgs = b->sched_len;
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));
         SR_HIP(ctx, ctx->gmax.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
         SR_HIP(ctx, ctx->gmax2.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));

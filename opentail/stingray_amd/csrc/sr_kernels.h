@@ -27,6 +27,7 @@ struct SrTopkArgs {
     // per workgroup in dispatch order: x = bit 31 row tail | bits 24..30 chunk | bits 0..23 launch slot of the row,
     // y = batch row, z = scan-mask row, w = sel -- all a workgroup needs to find its data, in one 16-byte load
     const int4* sched;
+    int32_t n_wgs;           // entries of sched = workgroups of the grid
     const SrRow* rows;
     const SrEdit* edits;
     const uint32_t* mask;

@@ -1420,6 +1420,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     typedef const i32x4 __attribute__((address_space(4))) const_i32x4;
     const i32x4 info = ((const_i32x4*)(uintptr_t)a.sched)[blockIdx.x];  // (item, row, scan-mask row, sel)
     const uint32_t item = (uint32_t)info.x;
+    if (item == 0xffffffffu) return;  // padding entry
     const bool is_tail = (item >> 31) != 0u;
     const int slot_ = (int)(item & 0xffffffu), c_ = (int)((item >> 24) & 0x7fu);
     if (is_tail) {
@@ -1648,7 +1649,7 @@ __global__ __launch_bounds__(kThreads) void k_build_scan_mask(const SrScanDesc* 
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
 {
     if (n_rows <= 0) return hipSuccess;
-    dim3 grid((unsigned)(n_rows * a.chunks + n_rows)), block(kThreads);  // chunk workgroups + one tail per row
+    dim3 grid((unsigned)a.n_wgs), block(kThreads);  // chunk workgroups + one tail per row (+ padding entries)
     if (a.dtype == 1)
         hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16>), grid, block, 0, stream, a);
     else
