@@ -163,21 +163,26 @@ __device__ __forceinline__ float seq_sum_tiles(Load load, int n, float s0, float
 {
     float s = s0;
     *found = -1;
-    float x[SR_SEQ_RUN];
-    if (n > 0) load(0, x);
-    for (int base = 0; base < n; base += SR_SEQ_TILE) {
-        float nx[SR_SEQ_RUN];
+    // two register sets take turns, so that no copy (which would wait for the loads) sits between the tiles
+    float xa[SR_SEQ_RUN], xb[SR_SEQ_RUN];
 #pragma unroll
-        for (int j = 0; j < SR_SEQ_RUN; j++) nx[j] = 0.0f;
-        if (base + SR_SEQ_TILE < n) load(base + SR_SEQ_TILE, nx);
+    for (int j = 0; j < SR_SEQ_RUN; j++) xa[j] = xb[j] = 0.0f;
+    if (n > 0) load(0, xa);
+    for (int base = 0; base < n; base += 2 * SR_SEQ_TILE) {
         int f;
-        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+        if (base + SR_SEQ_TILE < n) load(base + SR_SEQ_TILE, xb);
+        sr_seq_tile<kSearch>(xa, &s, target, &f, sm.seq);
         if (kSearch && f >= 0) {
             *found = base + f;
             return s;
         }
-#pragma unroll
-        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = nx[j];
+        if (base + SR_SEQ_TILE >= n) break;
+        if (base + 2 * SR_SEQ_TILE < n) load(base + 2 * SR_SEQ_TILE, xa);
+        sr_seq_tile<kSearch>(xb, &s, target, &f, sm.seq);
+        if (kSearch && f >= 0) {
+            *found = base + SR_SEQ_TILE + f;
+            return s;
+        }
     }
     return s;
 }
@@ -185,17 +190,17 @@ __device__ __forceinline__ float seq_sum_tiles(Load load, int n, float s0, float
 template <bool kSearch>
 __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm)
 {
-    static_assert(SR_SEQ_RUN == 16, "four float4 per thread");
+    static_assert(SR_SEQ_RUN % 4 == 0, "whole float4 per thread");
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
     auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
         const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
         if (aligned && i0 + SR_SEQ_RUN <= n) {
             const float4* v = (const float4*)(p + i0);
-            const float4 a0 = v[0], a1 = v[1], a2 = v[2], a3 = v[3];
-            x[0] = a0.x; x[1] = a0.y; x[2] = a0.z; x[3] = a0.w;
-            x[4] = a1.x; x[5] = a1.y; x[6] = a1.z; x[7] = a1.w;
-            x[8] = a2.x; x[9] = a2.y; x[10] = a2.z; x[11] = a2.w;
-            x[12] = a3.x; x[13] = a3.y; x[14] = a3.z; x[15] = a3.w;
+#pragma unroll
+            for (int k = 0; k < SR_SEQ_RUN / 4; k++) {
+                const float4 a = v[k];
+                x[4 * k] = a.x; x[4 * k + 1] = a.y; x[4 * k + 2] = a.z; x[4 * k + 3] = a.w;
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? p[i0 + j] : 0.0f;
@@ -209,7 +214,6 @@ template <bool kSearch>
 __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q, int n, float s0, float target, int* found,
                                                   FullSmem& sm)
 {
-    static_assert(SR_SEQ_RUN == 16, "four float4 per thread");
     const bool aligned = (((uintptr_t)p | (uintptr_t)q) & 15u) == 0u;
     auto res = [](float a, float b) -> float {
         const float r = __fsub_rn(a, b);
@@ -220,12 +224,12 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
         if (aligned && i0 + SR_SEQ_RUN <= n) {
             const float4* vp = (const float4*)(p + i0);
             const float4* vq = (const float4*)(q + i0);
-            const float4 a0 = vp[0], a1 = vp[1], a2 = vp[2], a3 = vp[3];
-            const float4 b0 = vq[0], b1 = vq[1], b2 = vq[2], b3 = vq[3];
-            x[0] = res(a0.x, b0.x); x[1] = res(a0.y, b0.y); x[2] = res(a0.z, b0.z); x[3] = res(a0.w, b0.w);
-            x[4] = res(a1.x, b1.x); x[5] = res(a1.y, b1.y); x[6] = res(a1.z, b1.z); x[7] = res(a1.w, b1.w);
-            x[8] = res(a2.x, b2.x); x[9] = res(a2.y, b2.y); x[10] = res(a2.z, b2.z); x[11] = res(a2.w, b2.w);
-            x[12] = res(a3.x, b3.x); x[13] = res(a3.y, b3.y); x[14] = res(a3.z, b3.z); x[15] = res(a3.w, b3.w);
+#pragma unroll
+            for (int k = 0; k < SR_SEQ_RUN / 4; k++) {
+                const float4 a = vp[k], b = vq[k];
+                x[4 * k] = res(a.x, b.x); x[4 * k + 1] = res(a.y, b.y);
+                x[4 * k + 2] = res(a.z, b.z); x[4 * k + 3] = res(a.w, b.w);
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? res(p[i0 + j], q[i0 + j]) : 0.0f;
@@ -237,7 +241,7 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
 // ragged tail folded in through an overlapped last vector, pairwise horizontal add.
 template <typename Term>
-__device__ float tp_sum(Term term, int n, FullSmem& sm)
+__device__ __forceinline__ float tp_sum(Term term, int n, FullSmem& sm)
 {
     int dummy;
     if (n < 4) {
@@ -250,29 +254,30 @@ __device__ float tp_sum(Term term, int n, FullSmem& sm)
         const bool extra = rem > 0 && g >= 8 - rem;
         const int cnt = nv + (extra ? 1 : 0);
         float s = 0.0f;
-        auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
-            const int i0 = base + lt * SR_SEQ_RUN;
-            if (i0 + SR_SEQ_RUN <= nv) {
+        auto load = [&](int base, float (&x)[SR_SEQ_RUN8]) __attribute__((always_inline)) {
+            const int i0 = base + lt * SR_SEQ_RUN8;
+            if (i0 + SR_SEQ_RUN8 <= nv) {
 #pragma unroll
-                for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = term((i0 + j) * 8 + g);
+                for (int j = 0; j < SR_SEQ_RUN8; j++) x[j] = term((i0 + j) * 8 + g);
             } else {
 #pragma unroll
-                for (int j = 0; j < SR_SEQ_RUN; j++) {
+                for (int j = 0; j < SR_SEQ_RUN8; j++) {
                     const int i = i0 + j;
                     x[j] = (i < cnt) ? (i < nv ? term(i * 8 + g) : term(n - 8 + g)) : 0.0f;
                 }
             }
         };
-        float x[SR_SEQ_RUN];
-        load(0, x);
-        for (int base = 0; base < nv + 1; base += SR_SEQ_CHAIN_TILE) {
-            float nx[SR_SEQ_RUN];
+        // two register sets take turns: no copy, which would wait for the loads, sits between the tiles
+        float xa[SR_SEQ_RUN8], xb[SR_SEQ_RUN8];
 #pragma unroll
-            for (int j = 0; j < SR_SEQ_RUN; j++) nx[j] = 0.0f;
-            if (base + SR_SEQ_CHAIN_TILE < nv + 1) load(base + SR_SEQ_CHAIN_TILE, nx);
-            sr_seq_tile8(x, &s, sm.seq8);
-#pragma unroll
-            for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = nx[j];
+        for (int j = 0; j < SR_SEQ_RUN8; j++) xa[j] = xb[j] = 0.0f;
+        load(0, xa);
+        for (int base = 0; base < nv + 1; base += 2 * SR_SEQ_CHAIN_TILE) {
+            if (base + SR_SEQ_CHAIN_TILE < nv + 1) load(base + SR_SEQ_CHAIN_TILE, xb);
+            sr_seq_tile8(xa, &s, sm.seq8);
+            if (base + SR_SEQ_CHAIN_TILE >= nv + 1) break;
+            if (base + 2 * SR_SEQ_CHAIN_TILE < nv + 1) load(base + 2 * SR_SEQ_CHAIN_TILE, xa);
+            sr_seq_tile8(xb, &s, sm.seq8);
         }
         __syncthreads();
         if (lt == 0) sm.lane_sum[g] = s;
@@ -296,7 +301,7 @@ __device__ float tp_sum(Term term, int n, FullSmem& sm)
 }
 
 // Normalize (Sampler.cs:553-562)
-__device__ void normalize_row(float* p, int n, FullSmem& sm)
+__device__ __forceinline__ void normalize_row(float* p, int n, FullSmem& sm)
 {
     const float sum = tp_sum([&](int i) -> float { return p[i]; }, n, sm);
     if (sum > 0.0f && sum != 1.0f) {
@@ -309,7 +314,7 @@ __device__ void normalize_row(float* p, int n, FullSmem& sm)
 // k-th largest value of p[0..n) (1-based), p >= 0: FindKthLargest (Sampler.cs:624-645).
 // With last_shift = 16 only the upper 16 bits are resolved: the result is then the smallest value of the
 // 65536-value bucket that holds the k-th largest.
-__device__ float kth_largest(const float* p, int n, int k, FullSmem& sm, int last_shift = 0)
+__device__ __forceinline__ float kth_largest(const float* p, int n, int k, FullSmem& sm, int last_shift = 0)
 {
     uint32_t prefix = 0u, pmask = 0u;
     int need = k;
@@ -341,7 +346,7 @@ __device__ float kth_largest(const float* p, int n, int k, FullSmem& sm, int las
 }
 
 // bitonic sort (descending) of sm.sortbuf[0 .. n_pow2)
-__device__ void sort_small_desc(FullSmem& sm, int n_pow2)
+__device__ __forceinline__ void sort_small_desc(FullSmem& sm, int n_pow2)
 {
     for (int k2 = 2; k2 <= n_pow2; k2 <<= 1) {
         for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
@@ -455,7 +460,7 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
 }
 
 // ---- argmax of an fp32 row: first index of the maximum, first NaN wins -------------------------------
-__device__ int row_argmax(const float* w, int n, FullSmem& sm)
+__device__ __forceinline__ int row_argmax(const float* w, int n, FullSmem& sm)
 {
     unsigned long long best = 0ull;
     row_pass<false>(const_cast<float*>(w), n, [&](float v, int i) -> float {
@@ -470,7 +475,7 @@ __device__ int row_argmax(const float* w, int n, FullSmem& sm)
 
 // first index whose running fp32 sum reaches r = (float)u; last index as the rounding fallback
 // (SampleFromDistribution, Sampler.cs:564-576)
-__device__ int draw_from_row(const float* p, int n, double u, FullSmem& sm)
+__device__ __forceinline__ int draw_from_row(const float* p, int n, double u, FullSmem& sm)
 {
     const float r = __double2float_rn(u);
     int found;
@@ -483,7 +488,7 @@ __device__ int draw_from_row(const float* p, int n, double u, FullSmem& sm)
 // running sum, so the eight strided chains of TensorPrimitives.Sum (plus its overlapped tail) and the running sum
 // of the draw are taken over the survivors alone, in index order: a chain's terms are the survivors whose index
 // falls on it, and the tail's indices lie behind every body index, so one order serves all eight chains.
-__device__ void finish_from_list(const SrFullArgs& a, float* p, int n, int m, int row, FullSmem& sm)
+__device__ __forceinline__ void finish_from_list(const SrFullArgs& a, float* p, int n, int m, int row, FullSmem& sm)
 {
     const int tid = threadIdx.x;
     int P = 2;
@@ -873,7 +878,7 @@ __global__ __launch_bounds__(kT) void k_draw_rows(const float* probs, int64_t st
 
 // residual = max(0, p - q): first the left-to-right sum of the positive residuals, then the first index
 // whose running residual reaches (float)u * sum; degenerate residual -> draw from p (Sampler.cs:587-618)
-__device__ int resample_residual_row(const float* p, const float* q, int n, double u, FullSmem& sm)
+__device__ __forceinline__ int resample_residual_row(const float* p, const float* q, int n, double u, FullSmem& sm)
 {
     int dummy;
     auto res = [&](int i) -> float {
@@ -1019,9 +1024,9 @@ __global__ __launch_bounds__(kT) void k_selftest_seqsum(const float* x, int n, f
     int found;
     float s;
     if (target == target)
-        s = seq_sum<true>([&](int i) -> float { return x[i]; }, n, s0, target, &found, sm);
+        s = seq_sum_row<true>(x, n, s0, target, &found, sm);
     else
-        s = seq_sum<false>([&](int i) -> float { return x[i]; }, n, s0, 0.0f, &found, sm);
+        s = seq_sum_row<false>(x, n, s0, 0.0f, &found, sm);
     if (threadIdx.x == 0) { *out_sum = s; *out_idx = found; }
 }
 

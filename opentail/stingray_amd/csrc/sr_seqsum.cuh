@@ -22,13 +22,14 @@
 
 #define SR_SEQ_THREADS 1024
 #define SR_SEQ_RUN 16
+#define SR_SEQ_RUN8 16  // terms per thread of the eight-chain tile
 #define SR_SEQ_TILE (SR_SEQ_THREADS * SR_SEQ_RUN)
 #define SR_SEQ_WAVES (SR_SEQ_THREADS / SR_WAVE)
 #define SR_SEQ_SAT (1u << 26)  // saturated increment: "this run leaves the binade"
 
 struct SrSeqSmem {
-    uint32_t wa0[SR_SEQ_WAVES];  // every wave's increment function ...
-    uint32_t wa1[SR_SEQ_WAVES];
+    uint32_t wa0[2][SR_SEQ_WAVES];  // every wave's increment function, rounds alternate between the two copies
+    uint32_t wa1[2][SR_SEQ_WAVES];
     uint32_t misc[8];
 };
 static_assert(SR_SEQ_WAVES == 16, "the wave totals are scanned inside one DPP row of 16 lanes");
@@ -61,18 +62,18 @@ __device__ __forceinline__ void sr_split(float s, uint32_t* n, int* eb)
 }
 __device__ __forceinline__ float sr_join(uint32_t n, int eb) { return sr_u2f(n + ((uint32_t)(eb - 1) << 23)); }
 
-// The increment function of the terms x[0..SR_SEQ_RUN) in the binade with exponent field eb: the hardware's
+// The increment function of the terms x[0..N) in the binade with exponent field eb: the hardware's
 // own round-to-nearest-even adds, run once from the binade's first even value and once from its first odd
 // value.  While such a chain stays inside the binade its bit pattern minus the start's is the number of ulps
 // gained, and that number is the same for every start of the same parity.  A chain that leaves the binade
 // (the run gains 2^23 ulps or more, or a term is too large for it) saturates: the caller replays that run.
-__device__ __forceinline__ SrInc sr_run_inc(const float (&x)[SR_SEQ_RUN], int eb)
+template <int N> __device__ __forceinline__ SrInc sr_run_inc(const float (&x)[N], int eb)
 {
     const uint32_t base = eb > 1 ? ((uint32_t)eb << 23) : 0u;    // n = 2^23 (or 0 below the normal range): even
     const uint32_t limit = eb > 1 ? base + (1u << 23) : (1u << 24);  // first bit pattern outside the binade
     float sa = sr_u2f(base), sb = sr_u2f(base + 1u);
 #pragma unroll
-    for (int j = 0; j < SR_SEQ_RUN; j++) {
+    for (int j = 0; j < N; j++) {
         sa = __fadd_rn(sa, x[j]);
         sb = __fadd_rn(sb, x[j]);
     }
@@ -123,29 +124,39 @@ __device__ __forceinline__ SrInc sr_scan_inc(SrInc v)
 // sixteen totals itself, which also shows the first wave in which the sum leaves the binade (or reaches the
 // target); that wave alone finds the thread and replays its run with real float adds; everything after it is
 // rescanned in the new binade.  A tile that stays in its binade costs two barriers.
+//
+// A sum that starts small doubles within a few terms, again within twice as many, and so on: after a crossing at
+// thread f the next one is expected near thread 2f.  The round after a crossing therefore looks at the threads up to
+// 2f + 64 only (waves outside that window skip the arithmetic and the scan); a window that passes without a
+// crossing is settled like a whole tile and the rest of the tile follows in one more round.
 template <bool kSearch>
 __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float* s, float target, int* found,
                                             SrSeqSmem& sm)
 {
     const int tid = threadIdx.x, lane = sr_lane();
     const int wave = __builtin_amdgcn_readfirstlane(sr_wave_id());
-    int start = 0;  // threads below `start` are settled
+    int start = 0;             // threads below `start` are settled
+    int wend = SR_SEQ_THREADS;  // this round looks at the threads [start, wend); a multiple of the wave size
     float s_in = *s;
     *found = -1;
     __syncthreads();  // the previous call's readers are done with the arrays below
-    for (;;) {
+    for (int round = 0;; round++) {
+        const int buf = round & 1;
         uint32_t n_in;
         int eb;
         sr_split(s_in, &n_in, &eb);
         SrInc mine;
         mine.a0 = 0u; mine.a1 = 0u;
-        if (tid >= start) mine = sr_run_inc(x, eb);
-        const SrInc incl = sr_scan_inc<false>(mine);
-        // (a later round writes after the barrier that ends this one, when every read below is done)
-        if (lane == SR_WAVE - 1) { sm.wa0[wave] = incl.a0; sm.wa1[wave] = incl.a1; }
+        SrInc incl = mine;
+        if ((wave + 1) * SR_WAVE > start && wave * SR_WAVE < wend) {  // (uniform per wave)
+            if (tid >= start) mine = sr_run_inc(x, eb);
+            incl = sr_scan_inc<false>(mine);
+        }
+        // (this copy is written again two rounds on, behind a barrier that every reader of it has passed)
+        if (lane == SR_WAVE - 1) { sm.wa0[buf][wave] = incl.a0; sm.wa1[buf][wave] = incl.a1; }
         __syncthreads();
         SrInc ti; ti.a0 = 0u; ti.a1 = 0u;
-        if (lane < SR_SEQ_WAVES) { ti.a0 = sm.wa0[lane]; ti.a1 = sm.wa1[lane]; }
+        if (lane < SR_SEQ_WAVES) { ti.a0 = sm.wa0[buf][lane]; ti.a1 = sm.wa1[buf][lane]; }
         ti = sr_scan_inc<true>(ti);  // lanes 0..15: the state function at the end of every wave
         // the running value never decreases, so the first wave whose end state has left the binade (or reached
         // the target) holds the first such thread
@@ -154,10 +165,13 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
         if (kSearch) event = event || sr_join(end_n, eb) >= target;
         const unsigned long long ev = __ballot(event && lane < SR_SEQ_WAVES);
         if (!ev) {
-            // the whole remainder stays in the binade: settle with the block total
+            // everything up to the window's end stays in the binade: settle with the total
             const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)((n_in & 1u) ? ti.a1 : ti.a0), SR_SEQ_WAVES - 1);
-            *s = sr_join(n_in + tot, eb);
-            return;
+            s_in = sr_join(n_in + tot, eb);
+            if (wend >= SR_SEQ_THREADS) { *s = s_in; return; }
+            start = wend;
+            wend = SR_SEQ_THREADS;
+            continue;
         }
         const int ev_wave = (int)__ffsll((long long)ev) - 1;
         if (wave == ev_wave) {
@@ -200,17 +214,18 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
         if (kSearch && where >= 0) { *found = where; *s = s_in; return; }
         start = fst + 1;
         if (start >= SR_SEQ_THREADS) { *s = s_in; return; }
+        wend = min(SR_SEQ_THREADS, (2 * start + 2 * SR_WAVE - 1) & ~(SR_WAVE - 1));
     }
 }
 
 // ---- eight independent chains at once -----------------------------------------------------------------
-// Thread t serves chain (t & 7) with the SR_SEQ_RUN terms number (t >> 3) * SR_SEQ_RUN ... of that chain's
-// tile, so one tile covers SR_SEQ_THREADS / 8 * SR_SEQ_RUN terms of every chain.  *s is the running sum
+// Thread t serves chain (t & 7) with the SR_SEQ_RUN8 terms number (t >> 3) * SR_SEQ_RUN8 ... of that chain's
+// tile, so one tile covers SR_SEQ_THREADS / 8 * SR_SEQ_RUN8 terms of every chain.  *s is the running sum
 // of the caller's chain (uniform across the threads of a chain).  Terms past the end must be 0.  All
 // threads of the block must call.
 #define SR_SEQ_CHAINS 8
 #define SR_SEQ_CHAIN_THREADS (SR_SEQ_THREADS / SR_SEQ_CHAINS)
-#define SR_SEQ_CHAIN_TILE (SR_SEQ_CHAIN_THREADS * SR_SEQ_RUN)
+#define SR_SEQ_CHAIN_TILE (SR_SEQ_CHAIN_THREADS * SR_SEQ_RUN8)
 
 struct SrSeq8Smem {
     uint32_t wa0[SR_SEQ_WAVES][SR_SEQ_CHAINS];
@@ -220,7 +235,7 @@ struct SrSeq8Smem {
     uint32_t busy;
 };
 
-__device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN], float* s, SrSeq8Smem& sm)
+__device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN8], float* s, SrSeq8Smem& sm)
 {
     const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
     const int g = tid & (SR_SEQ_CHAINS - 1), lt = tid >> 3;  // chain, position inside the chain
@@ -282,7 +297,7 @@ __device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN], float
                 // replay this run with real float adds from its exact input
                 float acc = sr_join(before, eb);
 #pragma unroll
-                for (int j = 0; j < SR_SEQ_RUN; j++) acc = __fadd_rn(acc, x[j]);
+                for (int j = 0; j < SR_SEQ_RUN8; j++) acc = __fadd_rn(acc, x[j]);
                 sm.acc[g] = sr_f2u(acc);
                 sm.busy = 1u;
             }
