@@ -369,6 +369,85 @@ __device__ __forceinline__ float load_logit(const char* rowp, int i)
     return sr_bf16_to_f32(((const uint16_t*)rowp)[i]);
 }
 
+// A sampled row that no logit bias and no history penalty touches needs no adjusted copy: the masked, scaled logit
+// is recomputed from the input where it is read (the row maximum and the expf pass), which saves one pass.
+__device__ __forceinline__ bool row_is_direct(const SrRow& rd) { return rd.temperature > 0.0f && rd.edit_cnt <= 0; }
+
+// ---- one pass of the grid's x dimension over a row of logits ---------------------------------------------
+// The masked (and temperature-scaled) logits of a row, sixteen input bytes per thread and load, four loads in flight;
+// body(i, x, c) gets c consecutive values starting at element i (c = 4 or 8 on the vector path, 1 on the scalar
+// path that rows with an unaligned start and the last elements of a row take).
+template <int ES>
+struct RowSource {
+    const char* rowp;
+    const uint32_t* mrow;
+    bool scale;
+    float inv_temp;
+    __device__ __forceinline__ float fix(float x, uint32_t keep) const
+    {
+        if (!keep) x = SR_NEG_INF;
+        return scale ? __fmul_rn(x, inv_temp) : x;
+    }
+};
+template <int ES, typename Body>
+__device__ __forceinline__ void stream_row(const RowSource<ES>& src, int n, Body body)
+{
+    constexpr int E = 16 / ES, kU = 4;
+    const int nv = (((uintptr_t)src.rowp & 15u) == 0u) ? n / E : 0;
+    const int step = (int)gridDim.x * 256;
+    for (int v0 = (int)blockIdx.x * 256 + (int)threadIdx.x; v0 < nv; v0 += step * kU) {
+        uint4 raw[kU];
+        uint32_t keep[kU];
+#pragma unroll
+        for (int u = 0; u < kU; u++) {
+            const int v = v0 + u * step;
+            raw[u] = make_uint4(0u, 0u, 0u, 0u);
+            keep[u] = 0xffu;
+            if (v < nv) {
+                raw[u] = ((const uint4*)src.rowp)[v];
+                if (src.mrow) keep[u] = src.mrow[(v * E) >> 5] >> ((v * E) & 31);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kU; u++) {
+            const int v = v0 + u * step;
+            if (v >= nv) break;
+            float x[E];
+            if (ES == 4) {
+                x[0] = sr_u2f(raw[u].x); x[1] = sr_u2f(raw[u].y); x[2] = sr_u2f(raw[u].z); x[3] = sr_u2f(raw[u].w);
+            } else {
+                const uint32_t r[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    x[(2 * q) % E] = sr_u2f(r[q] << 16);
+                    x[(2 * q + 1) % E] = sr_u2f(r[q] & 0xffff0000u);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < E; q++) x[q] = src.fix(x[q], (keep[u] >> q) & 1u);
+            body(v * E, x, E);
+        }
+    }
+    for (int i = nv * E + (int)blockIdx.x * 256 + (int)threadIdx.x; i < n; i += step) {
+        float x[E];
+        x[0] = src.fix(load_logit<ES>(src.rowp, i), src.mrow ? (src.mrow[i >> 5] >> (i & 31)) & 1u : 1u);
+        body(i, x, 1);
+    }
+}
+// stores c values (c = 1, 4 or 8) at w + i, with 16-byte stores where the address allows
+template <int E>
+__device__ __forceinline__ void store_run(float* w, int i, const float (&x)[E], int c)
+{
+    if (c == E && (((uintptr_t)(w + i)) & 15u) == 0u) {
+#pragma unroll
+        for (int q = 0; q < E; q += 4) *(float4*)(w + i + q) = make_float4(x[q], x[q + 1], x[q + 2], x[q + 3]);
+    } else {
+#pragma unroll
+        for (int q = 0; q < E; q++)
+            if (q < c) w[i + q] = x[q];
+    }
+}
+
 // ---- stage 1: the masked (and temperature-scaled) copy of the row ------------------------------------
 template <int ES>
 __global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
@@ -376,18 +455,15 @@ __global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
     const int slot = blockIdx.y;
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
-    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
     float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
-    const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
-    const bool scale = rd.temperature > 0.0f && rd.temperature != 1.0f;
-    const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+    RowSource<ES> src;
+    src.rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+    src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+    src.scale = rd.temperature > 0.0f && rd.temperature != 1.0f;
+    src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
     if (blockIdx.x == 0 && threadIdx.x == 0) a.state[slot].maxkey = 0u;
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256) {
-        float x = load_logit<ES>(rowp, i);
-        if (mrow && !((mrow[i >> 5] >> (i & 31)) & 1u)) x = SR_NEG_INF;
-        if (scale) x = __fmul_rn(x, inv_temp);
-        w[i] = x;
-    }
+    if (row_is_direct(rd)) return;  // nothing edits this row: the kernels behind read the logits themselves
+    stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c) { store_run(w, i, x, c); });
 }
 
 // ---- stage 2: logit bias and history penalties on the few ids they touch (Sampler.cs:51-58, :367-419)
@@ -425,18 +501,41 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
 // ---- stage 2b: the row maximum and expf(x - max) of the sampled rows, spread over the whole device ------
 // (Softmax, Sampler.cs:448-459.)  One workgroup per row would spend most of its time in the double-precision
 // expf of 150 thousand entries; here every row is cut into up to 64 pieces.
+template <int ES>
 __global__ __launch_bounds__(256) void k_full_max(SrFullArgs a)
 {
     __shared__ uint32_t wmax[4];
     const int slot = blockIdx.y;
     const int row = a.row_list[slot];
-    if (a.rows[row].temperature <= 0.0f) return;  // greedy rows keep their logits
-    const float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    const SrRow rd = a.rows[row];
+    if (rd.temperature <= 0.0f) return;  // greedy rows keep their logits
     uint32_t k = 0u;
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256) {
-        const float v = w[i];
+    auto fold = [&](float v) {
         const uint32_t kv = (v != v) ? 0xffffffffu : sr_okey(v);  // NaN propagates (TensorPrimitives.Max)
         k = kv > k ? kv : k;
+    };
+    if (row_is_direct(rd)) {
+        RowSource<ES> src;
+        src.rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+        src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+        src.scale = rd.temperature != 1.0f;
+        src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+        stream_row<ES>(src, a.vocab, [&](int, const float (&x)[16 / ES], int c) {
+#pragma unroll
+            for (int q = 0; q < 16 / ES; q++)
+                if (q < c) fold(x[q]);
+        });
+    } else {
+        RowSource<4> src;  // the adjusted copy
+        src.rowp = (const char*)(a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride);
+        src.mrow = nullptr;
+        src.scale = false;
+        src.inv_temp = 1.0f;
+        stream_row<4>(src, a.vocab, [&](int, const float (&x)[4], int c) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                if (q < c) fold(x[q]);
+        });
     }
     k = sr_wave_max_u32(k);
     if (sr_lane() == 0) wmax[sr_wave_id()] = k;
@@ -446,17 +545,42 @@ __global__ __launch_bounds__(256) void k_full_max(SrFullArgs a)
         if (k != 0u) atomicMax(&a.state[slot].maxkey, k);
     }
 }
+template <int ES>
 __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
 {
     const int slot = blockIdx.y;
     const int row = a.row_list[slot];
-    if (a.rows[row].temperature <= 0.0f) return;
+    const SrRow rd = a.rows[row];
+    if (rd.temperature <= 0.0f) return;
     const uint32_t mk = a.state[slot].maxkey;
     if (mk == 0xffffffffu || mk <= 0x007fffffu) return;  // NaN, or nothing above -inf: the row kernel makes it uniform
     const float m = sr_okey_inv(mk);
     float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256)
-        w[i] = sr_expf(__fsub_rn(w[i], m));
+    if (row_is_direct(rd)) {
+        RowSource<ES> src;
+        src.rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+        src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+        src.scale = rd.temperature != 1.0f;
+        src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+        stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c) {
+            float e[16 / ES];
+#pragma unroll
+            for (int q = 0; q < 16 / ES; q++) e[q] = q < c ? sr_expf(__fsub_rn(x[q], m)) : 0.0f;
+            store_run(w, i, e, c);
+        });
+    } else {
+        RowSource<4> src;  // the adjusted copy, replaced in place
+        src.rowp = (const char*)w;
+        src.mrow = nullptr;
+        src.scale = false;
+        src.inv_temp = 1.0f;
+        stream_row<4>(src, a.vocab, [&](int i, const float (&x)[4], int c) {
+            float e[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) e[q] = q < c ? sr_expf(__fsub_rn(x[q], m)) : 0.0f;
+            store_run(w, i, e, c);
+        });
+    }
 }
 
 // ---- argmax of an fp32 row: first index of the maximum, first NaN wins -------------------------------
@@ -1044,8 +1168,13 @@ hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
         hipLaunchKernelGGL(k_full_prep<4>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(k_full_edits<4>, dim3(n_rows), dim3(256), 0, st, a);
     }
-    hipLaunchKernelGGL(k_full_max, grid, dim3(256), 0, st, a);
-    hipLaunchKernelGGL(k_full_exp, grid, dim3(256), 0, st, a);
+    if (a.dtype == 1) {
+        hipLaunchKernelGGL(k_full_max<2>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(k_full_exp<2>, grid, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(k_full_max<4>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(k_full_exp<4>, grid, dim3(256), 0, st, a);
+    }
     return hipGetLastError();
 }
 hipError_t sr_launch_wide_keys(const SrFullArgs& a, int n_rows, hipStream_t st)
