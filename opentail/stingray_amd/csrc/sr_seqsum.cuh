@@ -228,88 +228,116 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
 #define SR_SEQ_CHAIN_TILE (SR_SEQ_CHAIN_THREADS * SR_SEQ_RUN8)
 
 struct SrSeq8Smem {
-    uint32_t wa0[SR_SEQ_WAVES][SR_SEQ_CHAINS];
-    uint32_t wa1[SR_SEQ_WAVES][SR_SEQ_CHAINS];
-    int first[SR_SEQ_WAVES][SR_SEQ_CHAINS];
-    uint32_t acc[SR_SEQ_CHAINS];
-    uint32_t busy;
+    uint32_t wa0[2][SR_SEQ_WAVES][SR_SEQ_CHAINS];  // every wave's increment function per chain; rounds alternate
+    uint32_t wa1[2][SR_SEQ_WAVES][SR_SEQ_CHAINS];
+    uint32_t acc[SR_SEQ_CHAINS];                   // a chain's exact sum behind the run that left the binade ...
+    int first[SR_SEQ_CHAINS];                      // ... and the chain thread that run belongs to
 };
 
+// inclusive scan of increment functions over the lanes of a wave that are 8, 16, ... apart (one chain's lanes)
+__device__ __forceinline__ SrInc sr_scan_inc_chain(SrInc v)
+{
+    const int lane = sr_lane();
+    SrInc lo;
+#pragma unroll
+    for (int o = SR_SEQ_CHAINS; o < SR_WAVE; o <<= 1) {
+        lo.a0 = __shfl_up(v.a0, o);
+        lo.a1 = __shfl_up(v.a1, o);
+        if (lane >= o) v = sr_compose(lo, v);
+    }
+    return v;
+}
+
+// One tile of all eight chains.  Per round: every wave scans its threads' increment functions chain by chain and
+// publishes the eight wave totals; every wave then scans the 16 x 8 totals itself (two per lane), which gives each
+// thread its chain's state at its wave's start and at the tile's end, and shows, per chain, the first wave in which
+// the chain's sum leaves the binade.  That wave finds the thread and replays its run with real float adds; the
+// chain's later threads are rescanned in the new binade.  A tile in which no chain leaves its binade costs two
+// barriers.
 __device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN8], float* s, SrSeq8Smem& sm)
 {
-    const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
+    static_assert(SR_SEQ_WAVES == 16 && SR_SEQ_CHAINS == 8 && SR_WAVE == 64, "two wave totals per lane and chain");
+    const int tid = threadIdx.x, lane = sr_lane();
+    const int wave = __builtin_amdgcn_readfirstlane(sr_wave_id());
     const int g = tid & (SR_SEQ_CHAINS - 1), lt = tid >> 3;  // chain, position inside the chain
+    const unsigned long long chain_lanes = 0x0101010101010101ull << g;
     int start = 0;     // chain threads below `start` are settled
     bool done = false; // this chain has finished the tile
     float s_in = *s;
-    for (;;) {
+    __syncthreads();  // the previous call's readers are done with the arrays below
+    for (int round = 0;; round++) {
+        const int buf = round & 1;
         uint32_t n_in;
         int eb;
         sr_split(s_in, &n_in, &eb);
+        const bool odd = (n_in & 1u) != 0u;
         SrInc mine;
         mine.a0 = 0u; mine.a1 = 0u;
         if (!done && lt >= start) mine = sr_run_inc(x, eb);
-        // inclusive scan over the lanes of the same chain (lanes 8 apart), then over the waves
-        SrInc incl = mine;
-#pragma unroll
-        for (int o = SR_SEQ_CHAINS; o < SR_WAVE; o <<= 1) {
-            SrInc lo;
-            lo.a0 = __shfl_up(incl.a0, o);
-            lo.a1 = __shfl_up(incl.a1, o);
-            if (lane >= o) incl = sr_compose(lo, incl);
-        }
+        const SrInc incl = sr_scan_inc_chain(mine);
+        // (this copy is written again two rounds on, behind a barrier that every reader of it has passed)
+        if (lane >= SR_WAVE - SR_SEQ_CHAINS) { sm.wa0[buf][wave][g] = incl.a0; sm.wa1[buf][wave][g] = incl.a1; }
         __syncthreads();
-        if (lane >= SR_WAVE - SR_SEQ_CHAINS) { sm.wa0[wave][g] = incl.a0; sm.wa1[wave][g] = incl.a1; }
-        if (tid == 0) sm.busy = 0u;
-        __syncthreads();
-        SrInc pre; pre.a0 = 0u; pre.a1 = 0u;
-        SrInc total; total.a0 = 0u; total.a1 = 0u;
-#pragma unroll
-        for (int w = 0; w < SR_SEQ_WAVES; w++) {
-            SrInc t; t.a0 = sm.wa0[w][g]; t.a1 = sm.wa1[w][g];
-            if (w < wave) pre = sr_compose(pre, t);
-            total = sr_compose(total, t);
+        // lane l holds, for chain l & 7, the totals of wave l >> 3 and of wave 8 + (l >> 3)
+        SrInc ta, tb;
+        ta.a0 = sm.wa0[buf][lane >> 3][g]; ta.a1 = sm.wa1[buf][lane >> 3][g];
+        tb.a0 = sm.wa0[buf][8 + (lane >> 3)][g]; tb.a1 = sm.wa1[buf][8 + (lane >> 3)][g];
+        ta = sr_scan_inc_chain(ta);
+        tb = sr_scan_inc_chain(tb);
+        SrInc half;
+        half.a0 = __shfl(ta.a0, SR_WAVE - SR_SEQ_CHAINS + g);
+        half.a1 = __shfl(ta.a1, SR_WAVE - SR_SEQ_CHAINS + g);
+        tb = sr_compose(half, tb);  // the chain's state function at the end of waves 8..15
+        const uint32_t t0 = __shfl(tb.a0, SR_WAVE - SR_SEQ_CHAINS + g), t1 = __shfl(tb.a1, SR_WAVE - SR_SEQ_CHAINS + g);
+        // the first wave at whose end the chain has left the binade (the running value never decreases)
+        const bool gone_a = !done && sr_sat_add(n_in, odd ? ta.a1 : ta.a0) >= (1u << 24);
+        const bool gone_b = !done && sr_sat_add(n_in, odd ? tb.a1 : tb.a0) >= (1u << 24);
+        const unsigned long long ba = __ballot(gone_a), bb = __ballot(gone_b);
+        if ((ba | bb) == 0ull) {
+            // no chain leaves its binade: settle every chain that is still open with its total
+            if (!done) s_in = sr_join(n_in + (odd ? t1 : t0), eb);
+            break;
         }
+        // (every lane takes part in the shuffles below: what differs per chain comes after them)
+        const unsigned long long ma = ba & chain_lanes, mb = bb & chain_lanes;
+        const int ev_wave = ma ? ((int)__ffsll((long long)ma) - 1) >> 3 : (mb ? 8 + (((int)__ffsll((long long)mb) - 1) >> 3) : -1);
+        // the chain's state function at the start of this wave
+        const int src_lane = ((wave - 1) & 7) * SR_SEQ_CHAINS + g;
+        SrInc pa, pb;
+        pa.a0 = __shfl(ta.a0, src_lane); pa.a1 = __shfl(ta.a1, src_lane);
+        pb.a0 = __shfl(tb.a0, src_lane); pb.a1 = __shfl(tb.a1, src_lane);
+        SrInc pre;
+        pre.a0 = wave == 0 ? 0u : (wave <= 8 ? pa.a0 : pb.a0);
+        pre.a1 = wave == 0 ? 0u : (wave <= 8 ? pa.a1 : pb.a1);
         SrInc ex;
         ex.a0 = __shfl_up(incl.a0, SR_SEQ_CHAINS);
         ex.a1 = __shfl_up(incl.a1, SR_SEQ_CHAINS);
         if (lane < SR_SEQ_CHAINS) { ex.a0 = 0u; ex.a1 = 0u; }
         ex = sr_compose(pre, ex);
-        const uint32_t before = sr_sat_add(n_in, (n_in & 1u) ? ex.a1 : ex.a0);
+        const uint32_t before = sr_sat_add(n_in, odd ? ex.a1 : ex.a0);
         const SrInc thr = sr_compose(ex, mine);
-        const uint32_t after = sr_sat_add(n_in, (n_in & 1u) ? thr.a1 : thr.a0);
-        const bool leaves = !done && lt >= start && after >= (1u << 24);
-        // first thread of the chain that leaves the binade
-        int cand = leaves ? lt : 0x7fffffff;
+        const uint32_t after = sr_sat_add(n_in, odd ? thr.a1 : thr.a0);
+        const bool leaves = !done && lt >= start && wave == ev_wave && after >= (1u << 24);
+        const unsigned long long bl = __ballot(leaves) & chain_lanes;
+        if (leaves && lane == (int)__ffsll((long long)bl) - 1) {
+            // the chain's first thread that leaves: replay its run with real float adds from its exact input
+            float acc = sr_join(before, eb);
 #pragma unroll
-        for (int o = SR_SEQ_CHAINS; o < SR_WAVE; o <<= 1) cand = min(cand, __shfl_xor(cand, o));
-        if (lane < SR_SEQ_CHAINS) sm.first[wave][g] = cand;
+            for (int j = 0; j < SR_SEQ_RUN8; j++) acc = __fadd_rn(acc, x[j]);
+            sm.acc[g] = sr_f2u(acc);
+            sm.first[g] = lt;
+        }
         __syncthreads();
-        int fst = 0x7fffffff;
-#pragma unroll
-        for (int w = 0; w < SR_SEQ_WAVES; w++) fst = min(fst, sm.first[w][g]);
         if (!done) {
-            if (fst == 0x7fffffff) {
-                // the chain's remainder stays in the binade: settle with the chain total
-                s_in = sr_join(n_in + ((n_in & 1u) ? total.a1 : total.a0), eb);
+            if (ev_wave < 0) {
+                s_in = sr_join(n_in + (odd ? t1 : t0), eb);  // this chain stays in its binade to the tile's end
                 done = true;
-            } else if (lt == fst) {
-                // replay this run with real float adds from its exact input
-                float acc = sr_join(before, eb);
-#pragma unroll
-                for (int j = 0; j < SR_SEQ_RUN8; j++) acc = __fadd_rn(acc, x[j]);
-                sm.acc[g] = sr_f2u(acc);
-                sm.busy = 1u;
+            } else {
+                s_in = sr_u2f(sm.acc[g]);
+                start = sm.first[g] + 1;
+                if (start >= SR_SEQ_CHAIN_THREADS) done = true;
             }
         }
-        __syncthreads();
-        const bool again = sm.busy != 0u;
-        if (!done) {
-            s_in = sr_u2f(sm.acc[g]);
-            start = fst + 1;
-            if (start >= SR_SEQ_CHAIN_THREADS) done = true;
-        }
-        if (!again) break;
     }
     *s = s_in;
 }
