@@ -555,6 +555,9 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
     const uint32_t mk = a.state[slot].maxkey;
     if (mk == 0xffffffffu || mk <= 0x007fffffu) return;  // NaN, or nothing above -inf: the row kernel makes it uniform
     const float m = sr_okey_inv(mk);
+    __shared__ uint64_t tab[32];  // the expf table: a lookup per element from global memory is a long dependent load
+    if (threadIdx.x < 32) tab[threadIdx.x] = sr_exp2f_tab[threadIdx.x];
+    __syncthreads();
     float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
     if (row_is_direct(rd)) {
         RowSource<ES> src;
@@ -565,7 +568,7 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
         stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c) {
             float e[16 / ES];
 #pragma unroll
-            for (int q = 0; q < 16 / ES; q++) e[q] = q < c ? sr_expf(__fsub_rn(x[q], m)) : 0.0f;
+            for (int q = 0; q < 16 / ES; q++) e[q] = q < c ? sr_expf_tab(__fsub_rn(x[q], m), tab) : 0.0f;
             store_run(w, i, e, c);
         });
     } else {
@@ -577,7 +580,7 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
         stream_row<4>(src, a.vocab, [&](int i, const float (&x)[4], int c) {
             float e[4];
 #pragma unroll
-            for (int q = 0; q < 4; q++) e[q] = q < c ? sr_expf(__fsub_rn(x[q], m)) : 0.0f;
+            for (int q = 0; q < 4; q++) e[q] = q < c ? sr_expf_tab(__fsub_rn(x[q], m), tab) : 0.0f;
             store_run(w, i, e, c);
         });
     }
