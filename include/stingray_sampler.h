@@ -159,6 +159,16 @@ SR_API int sr_sample_launch(sr_ctx* ctx, const sr_batch* batch, const void* logi
 
 /* Same, with the side inputs given directly and results in HOST buffers.  logits may be a device
  * (logits_on_device != 0) or a host tensor.  out_flags may be NULL. */
+/*
+ * SampleTopK (Sampler.cs:216-357) once more, by device-wide sorts of the whole row, for rows of a batch that
+ * sr_sample_launch reported with SR_OUT_ROW_UNSUPPORTED (any SampleTopK row may be given).  rows_host: HOST int32
+ * row indices into the batch; the same logits, outputs and uniforms as the launch before.  No counterpart in the
+ * reference, which has no row limit; sr_sample_batch calls it by itself.
+ */
+SR_API int sr_resample_rows_launch(sr_ctx* ctx, const sr_batch* batch, const void* logits_dev, int dtype,
+                                   int64_t row_stride_elems, const int32_t* rows_host, int32_t n_rows,
+                                   int32_t* out_tokens_dev, uint32_t* out_flags_dev);
+
 SR_API int sr_sample_batch(sr_ctx* ctx, const void* logits, int dtype, int logits_on_device,
                            int32_t rows, int32_t vocab, int64_t row_stride_elems,
                            const sr_row_params* params,

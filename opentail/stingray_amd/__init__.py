@@ -44,7 +44,7 @@ SR_OUT_ROW_UNSUPPORTED = 1 << 31
 EXPORTED_SYMBOLS = [
     "sr_create", "sr_destroy", "sr_bind_thread", "sr_set_stream", "sr_synchronize", "sr_last_error",
     "sr_version", "sr_batch_create", "sr_batch_destroy", "sr_batch_upload", "sr_batch_set_uniforms",
-    "sr_sample_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows",
+    "sr_sample_launch", "sr_resample_rows_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows",
     "sr_build_distribution_launch", "sr_sample_with_distribution_launch", "sr_sample_from_probs_launch",
     "sr_resample_residual_launch", "sr_spec_verify_launch", "sr_mtp_verify_launch", "sr_pack_allow_mask",
     "sr_build_distribution", "sr_sample_with_distribution", "sr_sample_from_probs", "sr_resample_residual",
@@ -138,6 +138,7 @@ def load_library():
                                   C.POINTER(C.c_uint8), f64p, i32]
     L.sr_batch_set_uniforms.argtypes = [vp, f64p]
     L.sr_sample_launch.argtypes = [vp, vp, vp, C.c_int, i64, vp, vp]
+    L.sr_resample_rows_launch.argtypes = [vp, vp, vp, C.c_int, i64, i32p, i32, vp, vp]
     L.sr_sample_batch.argtypes = [vp, vp, C.c_int, C.c_int, i32, i32, i64, rpp, i32p, i32p, i32p, f32p, i32p,
                                   u32p, i64, C.POINTER(C.c_uint8), f64p, i32p, u32p]
     L.sr_argmax_rows_launch.argtypes = [vp, vp, C.c_int, i32, i32, i64, vp, vp]
@@ -310,6 +311,15 @@ class SamplerContext:
             self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), self._row_stride(logits),
             C.c_void_p(out_tokens.data_ptr()), C.c_void_p(out_flags.data_ptr() if out_flags is not None else 0)))
 
+    def resample_rows_launch(self, batch: _Batch, logits, rows, out_tokens, out_flags=None):
+        """Async: SampleTopK by device-wide sorts for the given rows of the batch (those a launch flagged
+        SR_OUT_ROW_UNSUPPORTED); same tensors as sample_launch."""
+        r = np.ascontiguousarray(rows, dtype=np.int32)
+        self._check(self.L.sr_resample_rows_launch(
+            self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), self._row_stride(logits),
+            r.ctypes.data_as(C.POINTER(C.c_int32)), int(r.size),
+            C.c_void_p(out_tokens.data_ptr()), C.c_void_p(out_flags.data_ptr() if out_flags is not None else 0)))
+
     def sample_batch(self, logits, params: Sequence[SamplingParams], uniforms, allow_mask=None, mask_active=None,
                      return_flags: bool = False):
         """Sampler.Sample for every row (preceded by the row's mask). logits: CUDA tensor [rows, vocab].
@@ -323,6 +333,11 @@ class SamplerContext:
         self.sample_launch(batch, logits, toks, flags)
         self.synchronize()
         torch.cuda.synchronize()
+        redo = np.nonzero(flags.cpu().numpy().view(np.uint32) & np.uint32(SR_OUT_ROW_UNSUPPORTED))[0]
+        if redo.size:  # rows that overflowed the selection kernel's row tail: as sr_sample_batch does
+            self.resample_rows_launch(batch, logits, redo, toks, flags)
+            self.synchronize()
+            torch.cuda.synchronize()
         batch.close()
         t = toks.cpu().numpy()
         return (t, flags.cpu().numpy().view(np.uint32)) if return_flags else t

@@ -178,7 +178,7 @@ void sr_destroy(sr_ctx* ctx)
     DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best,
                          &ctx->work, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
-                         &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->spec_rows, &ctx->spec_probs};
+                         &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs};
     for (DeviceBuf* b : bufs) b->release();
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
     delete ctx;
@@ -487,10 +487,36 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         if (rc != SR_OK) return rc;
     }
     if (!b->h_wide_list.empty()) {
-        int rc = sr_wide_rows_launch(ctx, b, logits_dev, dtype, row_stride_elems, out_tokens_dev, out_flags_dev);
+        int rc = sr_wide_rows_launch(ctx, b, b->d_wide_list.as<int32_t>(), (int)b->h_wide_list.size(), logits_dev, dtype,
+                                     row_stride_elems, out_tokens_dev, out_flags_dev);
         if (rc != SR_OK) return rc;
     }
     return SR_OK;
+}
+
+int sr_resample_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride_elems,
+                            const int32_t* rows_host, int32_t n_rows, int32_t* out_tokens_dev, uint32_t* out_flags_dev)
+{
+    if (!ctx || !b) return SR_ERR_NULL_ARGUMENT;
+    if (n_rows == 0) return SR_OK;
+    if (!logits_dev || !out_tokens_dev || !rows_host)
+        return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_resample_rows_launch: null argument");
+    if (n_rows < 0 || (dtype != SR_DTYPE_F32 && dtype != SR_DTYPE_BF16) || row_stride_elems < b->vocab)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_resample_rows_launch: bad shape or dtype");
+    for (int32_t i = 0; i < n_rows; i++) {
+        const int32_t r = rows_host[i];
+        if (r < 0 || r >= b->rows) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_resample_rows_launch: row out of range");
+        const int32_t path = b->h_rows[(size_t)r].path;
+        if (path != SR_PATH_TOPK && path != SR_PATH_TOPK_WIDE)
+            return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_resample_rows_launch: not a SampleTopK row");
+    }
+    if (b->upr < 1) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_resample_rows_launch: a sampled row needs a uniform");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    SR_HIP(ctx, ctx->redo_list.reserve((size_t)n_rows * sizeof(int32_t), ctx->stream));
+    SR_HIP(ctx, hipMemcpyAsync(ctx->redo_list.p, rows_host, (size_t)n_rows * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the host array may go away
+    return sr_wide_rows_launch(ctx, b, ctx->redo_list.as<int32_t>(), n_rows, logits_dev, dtype, row_stride_elems,
+                               out_tokens_dev, out_flags_dev);
 }
 
 static int stage_logits(sr_ctx* ctx, const void* logits, int dtype, int on_device, int32_t rows, int32_t vocab,
@@ -534,10 +560,25 @@ int sr_sample_batch(sr_ctx* ctx, const void* logits, int dtype, int logits_on_de
     if (rc != SR_OK) return rc;
     SR_HIP(ctx, hipMemcpyAsync(out_tokens, ctx->out_tokens.p, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost,
                                ctx->stream));
-    if (out_flags)
-        SR_HIP(ctx, hipMemcpyAsync(out_flags, ctx->out_flags.p, (size_t)rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
-                                   ctx->stream));
+    std::vector<uint32_t> flags((size_t)rows);
+    SR_HIP(ctx, hipMemcpyAsync(flags.data(), ctx->out_flags.p, (size_t)rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                               ctx->stream));
     SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    // rows that overflowed the selection kernel's row tail (thousands of equal logits at the cut) take the sort path
+    std::vector<int32_t> redo;
+    for (int32_t r = 0; r < rows; r++)
+        if (flags[(size_t)r] & SR_KFLAG_UNSUPPORTED) redo.push_back(r);
+    if (!redo.empty()) {
+        rc = sr_resample_rows_launch(ctx, ctx->tmp_batch, dev, dtype, row_stride_elems, redo.data(), (int32_t)redo.size(),
+                                     ctx->out_tokens.as<int32_t>(), ctx->out_flags.as<uint32_t>());
+        if (rc != SR_OK) return rc;
+        SR_HIP(ctx, hipMemcpyAsync(out_tokens, ctx->out_tokens.p, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost,
+                                   ctx->stream));
+        SR_HIP(ctx, hipMemcpyAsync(flags.data(), ctx->out_flags.p, (size_t)rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                   ctx->stream));
+        SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    if (out_flags) memcpy(out_flags, flags.data(), (size_t)rows * sizeof(uint32_t));
     return SR_OK;
 }
 

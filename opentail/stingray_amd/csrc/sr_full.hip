@@ -870,6 +870,12 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
 // history penalties to those, orders them again (stable), and samples among the first k.  Here the whole row is
 // sorted device-wide by (raw logit descending, index ascending), the first `sel` entries are adjusted and sorted
 // again, and one workgroup per row walks the result.
+// the reference's selection size: k + history length when the row has history penalties (Sampler.cs:224-225)
+__device__ __forceinline__ int wide_sel(const SrRow& rd, int vocab)
+{
+    const long long s = (long long)rd.top_k + ((rd.flags & SR_ROWFLAG_HAS_PENALTY) ? (long long)rd.n_prev : 0ll);
+    return (int)(s < (long long)vocab ? s : (long long)vocab);
+}
 template <int ES>
 __global__ __launch_bounds__(256) void k_wide_keys(SrFullArgs a)
 {
@@ -903,7 +909,7 @@ __global__ __launch_bounds__(256) void k_wide_adjust(SrFullArgs a)
     const int32_t* sids = a.sort_vals_out + (size_t)slot * a.sort_stride;
     uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
     int32_t* ids = a.sort_vals_in + (size_t)slot * a.sort_stride;
-    const int sel = min(rd.sel, a.vocab);
+    const int sel = wide_sel(rd, a.vocab);
     if (blockIdx.x == 0 && threadIdx.x == 0) a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + sel;
     const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u && rd.edit_cnt > 0;
     const SrEdit* ed = a.edits + rd.edit_off;
@@ -940,7 +946,7 @@ __global__ __launch_bounds__(kT) void k_wide_tail(SrFullArgs a)
     const uint32_t* keys = a.sort_keys_out + (size_t)slot * a.sort_stride;
     const int32_t* ids = a.sort_vals_out + (size_t)slot * a.sort_stride;
     float* probs = a.work + (size_t)slot * a.work_stride;
-    const int k = min(rd.top_k, min(rd.sel, a.vocab));
+    const int k = min(rd.top_k, wide_sel(rd, a.vocab));
     const float v0 = sr_okey_inv(keys[0]);
     const int id0 = ids[0];
     if (id0 < 0 || sr_f2u(v0) == 0xff800000u) {

@@ -132,10 +132,9 @@ int sr_full_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, 
 
 // SampleTopK (Sampler.cs:216-357) for rows whose k + history length exceeds what the selection kernel's row tail
 // sorts: two device-wide segmented sorts and a walk by one workgroup per row.
-int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
-                        int32_t* out_tokens_dev, uint32_t* out_flags_dev)
+int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows, const void* logits_dev,
+                        int dtype, int64_t row_stride, int32_t* out_tokens_dev, uint32_t* out_flags_dev)
 {
-    const int n_rows = (int)b->h_wide_list.size();
     if (n_rows <= 0) return SR_OK;
     hipStream_t st = ctx->stream;
     const int vocab = b->vocab;
@@ -148,7 +147,7 @@ int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, 
     a.row_stride = row_stride;
     a.vocab = vocab;
     a.dtype = dtype;
-    a.row_list = b->d_wide_list.as<int32_t>();
+    a.row_list = list_dev;
     a.rows = b->d_rows.as<SrRow>();
     a.edits = b->d_edits.as<SrEdit>();
     a.mask = b->d_mask.as<uint32_t>();

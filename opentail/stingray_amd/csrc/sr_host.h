@@ -56,6 +56,7 @@ struct sr_ctx {
     DeviceBuf out_tokens, out_flags, out_val, uniforms_tmp;
     DeviceBuf seg, sort_k0, sort_k1, sort_v0, sort_v1, sort_tmp;  // device-wide sort of large nuclei
     DeviceBuf ident;         // identity row list
+    DeviceBuf redo_list;     // rows given to sr_resample_rows_launch
     int ident_rows = 0;
     DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
     sr_batch* tmp_batch = nullptr;
@@ -102,6 +103,6 @@ inline int sr_fail_hip(sr_ctx* ctx, hipError_t e, const char* what)
 // 2 = build distribution and sample from it.
 int sr_full_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
                         int32_t* out_tokens_dev, uint32_t* out_flags_dev);
-// SampleTopK for the rows of b->h_wide_list (sr_full_host.cpp)
-int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int dtype, int64_t row_stride,
-                        int32_t* out_tokens_dev, uint32_t* out_flags_dev);
+// SampleTopK by device-wide sorts for the SampleTopK rows in list_dev (sr_full_host.cpp)
+int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows, const void* logits_dev,
+                        int dtype, int64_t row_stride, int32_t* out_tokens_dev, uint32_t* out_flags_dev);

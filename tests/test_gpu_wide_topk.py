@@ -127,3 +127,34 @@ def test_bf16_rows_and_a_batch_that_mixes_every_path(ctx):
     dev = _cuda(bf.view(np.int16), torch.bfloat16)
     for _ in range(3):
         _check(ctx, logits, params, rng.random(rows), device_tensor=dev)
+
+
+def test_resampling_named_rows_agrees_with_the_selection_kernel_and_long_plateaus_at_the_cut(ctx):
+    import torch
+
+    rng = np.random.default_rng(75)
+    V, rows = 60_000, 6
+    logits = rng.normal(0, 1.0, (rows, V)).astype(np.float32)
+    # rows 0-2: a plateau of 5,000 to 30,000 equal logits right at the top-k cut, a few hundred larger values above it
+    for i, width in enumerate([5_000, 12_000, 30_000]):
+        where = rng.permutation(V)
+        logits[i, where[:width]] = np.float32(4.0)
+        logits[i, where[width:width + 300]] = (4.0 + rng.random(300) * 3).astype(np.float32)
+    params = [SamplingParams(Temperature=float(t), TopK=int(k), TopP=float(p), MinP=float(m), RepetitionPenalty=1.15,
+                             PreviousTokens=rng.integers(0, V, 100).tolist())
+              for t, k, p, m in [(0.8, 1000, 0.98, 0.0), (1.0, 2000, 1.0, 0.0), (0.7, 600, 0.9, 0.001),
+                                 (0.9, 40, 0.95, 0.02), (1.2, 700, 1.0, 0.0), (0.6, 5, 0.9, 0.0)]]
+    dev = _cuda(logits)
+    for _ in range(3):
+        u = rng.random(rows)
+        _check(ctx, logits, params, u, device_tensor=dev)      # sample_batch: overflowing rows are redone by itself
+        # every row once more through the sort path, named explicitly
+        batch = ctx.new_batch().upload(params, V, u)
+        toks = torch.full((rows,), -5, dtype=torch.int32, device="cuda")
+        flags = torch.zeros(rows, dtype=torch.int32, device="cuda")
+        ctx.resample_rows_launch(batch, dev, np.arange(rows), toks, flags)
+        ctx.synchronize()
+        torch.cuda.synchronize()
+        batch.close()
+        assert np.array_equal(toks.cpu().numpy(), oracle_tokens(logits, params, u))
+        assert np.all(flags.cpu().numpy().view(np.uint32) & OUT_TOPK)
