@@ -815,7 +815,32 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 }
             }
             if (ns > 0 && !closed) {
+                // the nucleus reaches past the candidates: the survivors, in index order (equal probabilities keep
+                // it through the stable sort), go to this row's segment of the device-wide sort
                 big = 1;
+                uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
+                int32_t* ids = a.sort_vals_in + (size_t)slot * a.sort_stride;
+                const bool aligned = ((uintptr_t)p & 15u) == 0u;
+                int base = 0;
+                for (int i0 = 0; i0 < n; i0 += 4 * kT) {
+                    const int i = i0 + 4 * tid;
+                    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (aligned && i + 4 <= n) {
+                        const float4 t = *(const float4*)(p + i);
+                        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                            if (i + q < n) v[q] = p[i + q];
+                    }
+                    const int mine = (v[0] > 0.0f ? 1 : 0) + (v[1] > 0.0f ? 1 : 0) + (v[2] > 0.0f ? 1 : 0) + (v[3] > 0.0f ? 1 : 0);
+                    int tot;
+                    int pos = base + blk_excl_scan(mine, &tot, sm);
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        if (v[q] > 0.0f) { keys[pos] = sr_f2u(v[q]); ids[pos] = i + q; pos++; }
+                    base += tot;
+                }
             }
             if (tid == 0) st->n_survivors = ns;
         }

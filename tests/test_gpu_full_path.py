@@ -290,3 +290,28 @@ def test_nucleus_finished_from_the_list_of_its_members(ctx):
         for u in ([0.0] * rows, [0.99999994] * rows, rng.random(rows).tolist()):
             _check_rows(ctx, logits, params, u)
         _check_distribution(ctx, logits, params)
+
+
+def test_nuclei_of_tens_of_thousands_of_members_take_the_device_wide_sort(ctx):
+    # Flat rows: the top-p nucleus does not close among the 4,096 largest probabilities, so the survivors are sorted
+    # device-wide (stable: equal probabilities in index order) and cut by the exact search.  Distributions must agree
+    # bit for bit -- the support is what the cut decides -- and so must the draws.
+    rng = np.random.default_rng(77)
+    V = 40_000
+    logits = np.stack([
+        rng.normal(0, 0.5, V),                               # ~ 80 % of the vocabulary inside a 0.95 nucleus
+        np.round(rng.normal(0, 0.7, V) * 8) / 8,             # a coarse grid: thousands of equal probabilities at the cut
+        rng.normal(0, 0.3, V),
+        rng.normal(0, 3.0, V),                               # a sharp row in the same batch: closes inside the kernel
+    ]).astype(np.float32)
+    params = [SamplingParams(Temperature=1.0, TopP=0.95), SamplingParams(Temperature=0.8, TopP=0.9),
+              SamplingParams(Temperature=1.3, TopP=0.5), SamplingParams(Temperature=1.0, TopP=0.95)]
+    _check_distribution(ctx, logits, params)
+    for _ in range(4):
+        _check_rows(ctx, logits, params, rng.random(4))
+    # the same under dense allow-masks and next to rows of the other paths
+    allowed = rng.random((4, V)) < np.array([0.6, 0.9, 0.5, 1.0])[:, None]
+    mask = pack_allow_mask(allowed)
+    active = np.ones(4, dtype=np.uint8)
+    _check_distribution(ctx, logits, params, mask, active)
+    _check_rows(ctx, logits, params, rng.random(4), mask, active)
