@@ -315,3 +315,83 @@ def test_nuclei_of_tens_of_thousands_of_members_take_the_device_wide_sort(ctx):
     active = np.ones(4, dtype=np.uint8)
     _check_distribution(ctx, logits, params, mask, active)
     _check_rows(ctx, logits, params, rng.random(4), mask, active)
+
+
+def _strided(a, pad, dtype=None):
+    """The rows of `a` inside a wider device tensor: row stride = a.shape[1] + pad elements."""
+    import torch
+
+    wide = np.zeros((a.shape[0], a.shape[1] + pad), dtype=a.dtype)
+    wide[:, :a.shape[1]] = a
+    t = torch.from_numpy(wide)
+    if dtype is not None:
+        t = t.view(dtype)
+    return t.cuda()[:, :a.shape[1]]
+
+
+def test_bf16_and_unaligned_rows_on_the_full_path(ctx):
+    import torch
+
+    rng = np.random.default_rng(78)
+    for V, pad in [(10_007, 3), (4_096, 0), (33_001, 6)]:
+        rows = 6
+        f32 = rng.normal(0, 2.0, (rows, V)).astype(np.float32)
+        bf = (f32.view(np.uint32) >> 16).astype(np.uint16)
+        exact = (bf.astype(np.uint32) << 16).view(np.float32)             # what the bf16 tensor holds
+        allowed = rng.random((rows, V)) < 0.7
+        mask = pack_allow_mask(allowed)
+        active = np.array([0, 1, 0, 1, 0, 0], dtype=np.uint8)
+        hist = rng.integers(0, V, 200).tolist()
+        params = [SamplingParams(Temperature=0.9, TopP=0.9),                                   # nothing edits the row
+                  SamplingParams(Temperature=1.0, TopP=0.95, MinP=0.001),
+                  SamplingParams(Temperature=0.7, LogitBias={5: 3.0, V - 1: -2.0, 17: 1.5}, TopK=50, TopP=0.9),
+                  SamplingParams(Temperature=1.2, RepetitionPenalty=1.3, FrequencyPenalty=0.2, PreviousTokens=hist),
+                  SamplingParams(Temperature=0.0, LogitBias={3: 100.0}),                        # greedy ignores the bias
+                  SamplingParams(Temperature=1.0)]
+        for logits, dev in [(exact, _strided(bf.view(np.int16), pad, torch.bfloat16)), (f32, _strided(f32, pad))]:
+            for _ in range(2):
+                u = rng.random(rows)
+                got, flags = ctx.sample_batch(dev, params, u, mask, active, return_flags=True)
+                assert np.array_equal(got, oracle_tokens(logits, params, u, mask, active)), (V, pad, dev.dtype)
+            got = ctx.build_distribution(dev, params, None, mask, active).cpu().numpy()
+            for r, p in enumerate(params):
+                row = orc.apply_allow_mask(logits[r], mask[r]) if active[r] else logits[r]
+                want = orc.build_filtered_distribution(row, to_oracle(p))
+                assert np.array_equal(got[r].view(np.uint32), want.view(np.uint32)), (V, pad, dev.dtype, r)
+
+
+def test_rows_without_a_finite_logit_and_rows_with_a_nan(ctx):
+    # Softmax falls back to the uniform distribution when the maximum is -inf or NaN (Sampler.cs:452-458)
+    rng = np.random.default_rng(79)
+    V = 3_000
+    logits = rng.normal(0, 1.0, (4, V)).astype(np.float32)
+    logits[0, :] = NEG_INF
+    logits[1, 1234] = np.float32("nan")
+    allowed = np.ones((4, V), dtype=bool)
+    allowed[2, :] = False                                                 # a dead mask: every id forbidden
+    mask = pack_allow_mask(allowed)
+    active = np.array([0, 0, 1, 0], dtype=np.uint8)
+    params = [SamplingParams(Temperature=1.0, TopP=0.9), SamplingParams(Temperature=0.8),
+              SamplingParams(Temperature=1.0, MinP=0.1), SamplingParams(Temperature=1.0, TopP=0.9)]
+    for _ in range(4):
+        u = rng.random(4)
+        got, flags = ctx.sample_batch(_cuda(logits), params, u, mask, active, return_flags=True)
+        assert np.array_equal(got, oracle_tokens(logits, params, u, mask, active)), (got, flags)
+        assert np.all(flags[:3] & 8) and not flags[3] & 8
+    _check_distribution(ctx, logits, params, mask, active)
+
+
+def test_sample_with_distribution_rows(ctx):
+    rng = np.random.default_rng(80)
+    V, rows = 20_000, 5
+    logits = rng.normal(0, 2.0, (rows, V)).astype(np.float32)
+    params = [SamplingParams(Temperature=1.0), SamplingParams(Temperature=0.7, TopK=40, TopP=0.9),
+              SamplingParams(Temperature=0.0), SamplingParams(Temperature=1.1, MinP=0.02),
+              SamplingParams(Temperature=0.9, TopP=0.8, RepetitionPenalty=1.2, PreviousTokens=rng.integers(0, V, 64).tolist())]
+    u = rng.random(rows)
+    toks, probs = ctx.sample_with_distribution(_cuda(logits), params, u)
+    probs = probs.cpu().numpy()
+    for r, p in enumerate(params):
+        t, d = orc.sample_with_distribution(logits[r], to_oracle(p), orc.Rng(replay=[u[r]]))
+        assert toks[r] == t, r
+        assert np.array_equal(probs[r].view(np.uint32), np.asarray(d, dtype=np.float32).view(np.uint32)), r
