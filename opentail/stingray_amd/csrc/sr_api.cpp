@@ -117,14 +117,14 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
             longest = std::max(longest, q.size() / 4);
         }
         // interleave the dies' queues; a die with fewer rows gets entries that end at once
-        std::vector<int32_t> sched(longest * (size_t)n_xcd * 4, -1);
+        std::vector<int32_t>& sched = b->h_sched;
+        sched.assign(longest * (size_t)n_xcd * 4, -1);
         for (int x = 0; x < n_xcd; x++)
             for (size_t i = 0; i < queue[(size_t)x].size() / 4; i++)
                 for (int w = 0; w < 4; w++) sched[(i * (size_t)n_xcd + (size_t)x) * 4 + (size_t)w] = queue[(size_t)x][i * 4 + (size_t)w];
         b->sched_len = (int32_t)(longest * (size_t)n_xcd);
         SR_HIP(ctx, b->d_sched.reserve(sched.size() * sizeof(int32_t), st));
         SR_HIP(ctx, hipMemcpyAsync(b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
-        SR_HIP(ctx, hipStreamSynchronize(st));
     }
     b->scan_stride = (int64_t)chunks * SR_TK_THREADS * SR_TK_MASK_WORDS;
     if (rows_changed)
@@ -263,8 +263,7 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
     b->mask_stride = allow_mask ? mask_stride_words : 0;
     b->max_sel = 0;
 
-    struct Occ { int32_t id; int32_t in_window; };
-    std::vector<Occ> occ;
+    std::vector<int32_t> slots;  // scratch of the history de-duplication
     for (int32_t r = 0; r < rows; r++) {
         const sr_row_params& p = params[r];
         SrRow& d = b->h_rows[(size_t)r];
@@ -308,26 +307,55 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         const bool want_hist = has_penalty;
         const bool want_bias = n_bias > 0 && !greedy;  // LogitBias is ignored by the greedy paths
         if (want_hist || want_bias) {
-            // occurrence counts of every in-range id: whole history and trailing repetition window
-            occ.clear();
+            // occurrence counts of every in-range id (whole history and trailing repetition window), one edit per
+            // distinct id in order of first appearance: an open-addressing table over the row's edits
+            std::vector<SrEdit>& ed = b->h_edits;
             if (want_hist) {
                 const int32_t ws = (p.repeat_last_n <= 0 || p.repeat_last_n >= n_prev) ? 0 : n_prev - p.repeat_last_n;
-                for (int32_t i = 0; i < n_prev; i++)
-                    if ((uint32_t)prev[i] < (uint32_t)vocab) occ.push_back({prev[i], i >= ws ? 1 : 0});
-                std::stable_sort(occ.begin(), occ.end(), [](const Occ& x, const Occ& y) { return x.id < y.id; });
+                size_t cap = 16;
+                while (cap < 2 * (size_t)n_prev) cap <<= 1;
+                slots.assign(cap, 0);  // 1 + index of the id's edit, 0 = free
+                for (int32_t i = 0; i < n_prev; i++) {
+                    const int32_t id = prev[i];
+                    if ((uint32_t)id >= (uint32_t)vocab) continue;
+                    size_t h = ((uint32_t)id * 2654435761u) & (cap - 1);
+                    while (slots[h] != 0 && ed[(size_t)slots[h] - 1].id != id) h = (h + 1) & (cap - 1);
+                    if (slots[h] == 0) {
+                        SrEdit e{};
+                        e.id = id;
+                        e.pen = 1.0f;
+                        ed.push_back(e);
+                        slots[h] = (int32_t)ed.size();
+                    }
+                    SrEdit& e = ed[(size_t)slots[h] - 1];
+                    e.occ_all++;
+                    if (i >= ws) e.occ_win++;
+                }
+                if (p.repetition_penalty != 1.0f) {
+                    // powf(repetition_penalty, occurrences in the window): the same few exponents over and over
+                    float pow_of[9];
+                    bool pow_known[9] = {false, false, false, false, false, false, false, false, false};
+                    for (size_t i = (size_t)d.edit_off; i < ed.size(); i++) {
+                        const int32_t win = ed[i].occ_win;
+                        if (win <= 0) continue;
+                        if (win < 9) {
+                            if (!pow_known[win]) { pow_of[win] = powf(p.repetition_penalty, (float)win); pow_known[win] = true; }
+                            ed[i].pen = pow_of[win];
+                        } else {
+                            ed[i].pen = powf(p.repetition_penalty, (float)win);
+                        }
+                    }
+                }
             }
-            std::vector<SrEdit>& ed = b->h_edits;
-            for (size_t i = 0; i < occ.size();) {
-                size_t j = i;
-                int32_t win = 0;
-                while (j < occ.size() && occ[j].id == occ[i].id) { win += occ[j].in_window; j++; }
-                SrEdit e{};
-                e.id = occ[i].id;
-                e.occ_all = (int32_t)(j - i);
-                e.occ_win = win;
-                e.pen = (p.repetition_penalty != 1.0f && win > 0) ? powf(p.repetition_penalty, (float)win) : 1.0f;
-                ed.push_back(e);
-                i = j;
+            // sorted by id where something searches them: the bias merge below, the rows whose penalties may raise a
+            // logit (the row tail looks candidates up) and the rows of the sort-based path
+            const bool lowering_only = p.repetition_penalty >= 1.0f && p.presence_penalty >= 0.0f && p.frequency_penalty >= 0.0f;
+            const bool searched = want_bias || (d.path == SR_PATH_TOPK && !lowering_only) ||
+                                  (d.path == SR_PATH_TOPK && (int64_t)p.top_k + (int64_t)(ed.size() - (size_t)d.edit_off) > SR_TK_SEL_MAX) ||
+                                  ed.size() - (size_t)d.edit_off > (size_t)SR_TK_SEL_MAX;
+            if (searched) {
+                std::sort(ed.begin() + d.edit_off, ed.end(), [](const SrEdit& x, const SrEdit& y) { return x.id < y.id; });
+                d.flags |= SR_ROWFLAG_EDITS_SORTED;
             }
             if (want_bias) {
                 for (int32_t i = b0; i < b1; i++) {
@@ -399,14 +427,14 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
     if (allow_mask) SR_HIP(ctx, up(b->d_mask, allow_mask, (size_t)rows * (size_t)mask_stride_words * sizeof(uint32_t)));
     if (uniforms_per_row > 0)
         SR_HIP(ctx, up(b->d_uniforms, uniforms, (size_t)rows * (size_t)uniforms_per_row * sizeof(double)));
-    // the host vectors are read by the async copies above
-    SR_HIP(ctx, hipStreamSynchronize(st));
     // scan masks for the layout of the last launch (16-byte aligned rows); a launch with another layout rebuilds
     if (!b->h_sel_list.empty()) {
         const int epv = ctx->last_epv;
         int rc = prepare_scan(b, epv, 0ull, 0ll);
         if (rc != SR_OK) return rc;
     }
+    // the host arrays (the batch's own and the caller's) are read by the async copies above
+    SR_HIP(ctx, hipStreamSynchronize(st));
     return SR_OK;
 }
 

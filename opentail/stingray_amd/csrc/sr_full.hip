@@ -944,10 +944,16 @@ __global__ __launch_bounds__(256) void k_wide_adjust(SrFullArgs a)
         if (sr_f2u(v) == 0xff800000u) {
             id = -1;
         } else if (pen) {
-            int lo = 0, hi = rd.edit_cnt;
-            while (lo < hi) {
-                const int mid = (lo + hi) >> 1;
-                if (ed[mid].id < id) lo = mid + 1; else hi = mid;
+            int lo = 0;
+            if (rd.flags & SR_ROWFLAG_EDITS_SORTED) {
+                int hi = rd.edit_cnt;
+                while (lo < hi) {
+                    const int mid = (lo + hi) >> 1;
+                    if (ed[mid].id < id) lo = mid + 1; else hi = mid;
+                }
+            } else {
+                // (a row that was meant for the selection kernel and is redone here: its few edits are unsorted)
+                while (lo < rd.edit_cnt && ed[lo].id != id) lo++;
             }
             if (lo < rd.edit_cnt && ed[lo].id == id && ed[lo].occ_all > 0) {
                 const SrEdit ee = ed[lo];

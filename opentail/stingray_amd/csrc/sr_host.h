@@ -71,6 +71,7 @@ struct sr_batch {
     std::vector<SrEdit> h_edits;
     std::vector<int32_t> h_sel_list;   // rows on the selection kernel: TOPK and plain GREEDY
     std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path
+    std::vector<int32_t> h_sched;     // the selection kernel's dispatch table (host copy, read by an async upload)
     int32_t sched_len = 0;             // workgroups of the selection kernel's grid (entries of d_sched)
     std::vector<int32_t> h_wide_list;  // SampleTopK rows too wide for the selection kernel
     std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel

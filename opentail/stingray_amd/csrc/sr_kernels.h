@@ -15,6 +15,8 @@
 // internal bit: the penalties can only lower a logit, so the scan skips the history ids (scan mask) and
 // the row tail fetches their logits by id instead of over-selecting by the history length
 #define SR_ROWFLAG_HIST_EXCL (1u << 9)
+// the row's edits are sorted by id (else they stand in order of first appearance in the history)
+#define SR_ROWFLAG_EDITS_SORTED (1u << 10)
 
 struct SrTopkArgs {
     const void* logits;

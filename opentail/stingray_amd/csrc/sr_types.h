@@ -30,7 +30,8 @@ struct SrRow {
     int32_t scan_row;   // row index into the scan-mask array (row edges, allow-mask, history ids)
 };
 
-// One distinct in-range token id that the row's history or logit bias touches; sorted by id per row.
+// One distinct in-range token id that the row's history or logit bias touches; sorted by id per row where a kernel
+// searches them (SR_ROWFLAG_EDITS_SORTED), else in order of first appearance in the history.
 struct SrEdit {
     int32_t id;
     float bias;         // LogitBias value (applied first); valid when has_bias
