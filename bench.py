@@ -71,7 +71,7 @@ def cpu_baseline(w, budget_s: float):
         done += w.rows
         passes += 1
         el = time.perf_counter() - t0
-        if el >= budget_s or passes >= 50:
+        if el >= budget_s or passes >= 400:
             break
     return done / el, done, el
 
