@@ -39,7 +39,20 @@ void topk_geometry(int vocab, int dtype, int n_rows, int cu_count, int* chunks, 
 // (Re)builds the scan masks of a batch for logits of the given vector width and alignment.  Rows without an
 // allow-mask and without excluded history ids share one mask row when every row starts at the same offset
 // inside its first vector.
-int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long stride_bytes)
+// Copies host data of a batch to the device on `st`: through the batch's pinned memory when `staged` (no wait
+// needed), else straight from `src`, which the caller then has to keep alive until the stream is synchronised.
+hipError_t batch_copy(sr_batch* b, bool staged, void* dst, const void* src, size_t bytes, hipStream_t st)
+{
+    if (bytes == 0) return hipSuccess;
+    const void* from = staged ? b->stage.put(src, bytes) : nullptr;
+    if (!from) {
+        from = src;
+        b->upload_must_wait = true;
+    }
+    return hipMemcpyAsync(dst, from, bytes, hipMemcpyHostToDevice, st);
+}
+
+int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long stride_bytes, bool staged = false)
 {
     sr_ctx* ctx = b->ctx;
     hipStream_t st = ctx->stream;
@@ -124,20 +137,20 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
                 for (int w = 0; w < 4; w++) sched[(i * (size_t)n_xcd + (size_t)x) * 4 + (size_t)w] = queue[(size_t)x][i * 4 + (size_t)w];
         b->sched_len = (int32_t)(longest * (size_t)n_xcd);
         SR_HIP(ctx, b->d_sched.reserve(sched.size() * sizeof(int32_t), st));
-        SR_HIP(ctx, hipMemcpyAsync(b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+        SR_HIP(ctx, batch_copy(b, staged, b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), st));
     }
     b->scan_stride = (int64_t)chunks * SR_TK_THREADS * SR_TK_MASK_WORDS;
     if (rows_changed)
-        SR_HIP(ctx, hipMemcpyAsync(b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), hipMemcpyHostToDevice, st));
+        SR_HIP(ctx, batch_copy(b, staged, b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), st));
     SR_HIP(ctx, b->d_scan_desc.reserve(b->h_scan.size() * sizeof(SrScanDesc), st));
-    SR_HIP(ctx, hipMemcpyAsync(b->d_scan_desc.p, b->h_scan.data(), b->h_scan.size() * sizeof(SrScanDesc), hipMemcpyHostToDevice, st));
+    SR_HIP(ctx, batch_copy(b, staged, b->d_scan_desc.p, b->h_scan.data(), b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, b->d_scan_mask.reserve(b->h_scan.size() * (size_t)b->scan_stride * sizeof(uint32_t), st));
     SR_HIP(ctx, sr_launch_build_scan_mask(b->d_scan_desc.as<SrScanDesc>(), (int)b->h_scan.size(), b->d_rows.as<SrRow>(),
                                           b->d_edits.as<SrEdit>(), b->d_mask.as<uint32_t>(), b->mask_stride,
                                           b->d_scan_mask.as<uint32_t>(), b->scan_stride, b->vocab, epv, chunks, chunk_vecs,
                                           base_addr, stride_bytes, st));
     // the host vectors are read by the async copies above
-    SR_HIP(ctx, hipStreamSynchronize(st));
+    if (!staged) SR_HIP(ctx, hipStreamSynchronize(st));
     return SR_OK;
 }
 
@@ -194,7 +207,11 @@ int sr_bind_thread(sr_ctx* ctx)
 int sr_set_stream(sr_ctx* ctx, void* hip_stream)
 {
     if (!ctx) return SR_ERR_NULL_ARGUMENT;
-    ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+    hipStream_t next = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+    // uploads of batches may still be running on the stream that is left: later launches are ordered behind them
+    // only on the same stream
+    if (next != ctx->stream) SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    ctx->stream = next;
     return SR_OK;
 }
 
@@ -224,6 +241,7 @@ void sr_batch_destroy(sr_batch* b)
     DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_wide_list, &b->d_scan_desc,
                          &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched};
     for (DeviceBuf* d : bufs) d->release();
+    b->stage.release();
     delete b;
 }
 
@@ -247,6 +265,8 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: uniforms is null");
     SR_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
+    SR_HIP(ctx, b->stage.begin());  // (waits for the copies of this batch's previous upload)
+    b->upload_must_wait = false;
 
     b->rows = rows;
     b->vocab = vocab;
@@ -417,24 +437,31 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         if (bytes == 0) return hipSuccess;
         hipError_t e = dst.reserve(bytes, st);
         if (e != hipSuccess) return e;
-        return hipMemcpyAsync(dst.p, src, bytes, hipMemcpyHostToDevice, st);
+        return batch_copy(b, true, dst.p, src, bytes, st);
     };
     SR_HIP(ctx, up(b->d_rows, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow)));
     SR_HIP(ctx, up(b->d_edits, b->h_edits.data(), b->h_edits.size() * sizeof(SrEdit)));
     SR_HIP(ctx, up(b->d_sel_list, b->h_sel_list.data(), b->h_sel_list.size() * sizeof(int32_t)));
     SR_HIP(ctx, up(b->d_full_list, b->h_full_list.data(), b->h_full_list.size() * sizeof(int32_t)));
     SR_HIP(ctx, up(b->d_wide_list, b->h_wide_list.data(), b->h_wide_list.size() * sizeof(int32_t)));
-    if (allow_mask) SR_HIP(ctx, up(b->d_mask, allow_mask, (size_t)rows * (size_t)mask_stride_words * sizeof(uint32_t)));
+    if (allow_mask) {  // large: straight from the caller's memory, which the wait at the end covers
+        const size_t bytes = (size_t)rows * (size_t)mask_stride_words * sizeof(uint32_t);
+        SR_HIP(ctx, b->d_mask.reserve(bytes, st));
+        SR_HIP(ctx, batch_copy(b, false, b->d_mask.p, allow_mask, bytes, st));
+    }
     if (uniforms_per_row > 0)
         SR_HIP(ctx, up(b->d_uniforms, uniforms, (size_t)rows * (size_t)uniforms_per_row * sizeof(double)));
     // scan masks for the layout of the last launch (16-byte aligned rows); a launch with another layout rebuilds
     if (!b->h_sel_list.empty()) {
         const int epv = ctx->last_epv;
-        int rc = prepare_scan(b, epv, 0ull, 0ll);
+        int rc = prepare_scan(b, epv, 0ull, 0ll, true);
         if (rc != SR_OK) return rc;
     }
-    // the host arrays (the batch's own and the caller's) are read by the async copies above
-    SR_HIP(ctx, hipStreamSynchronize(st));
+    // Everything small went through the batch's pinned memory: the copies and the scan-mask kernel run on while
+    // the caller goes on (launches on this stream are ordered behind them).  Pageable memory that a copy reads
+    // directly (the caller's allow-mask; anything the pinned memory had no room for yet) must be waited for.
+    if (b->upload_must_wait) SR_HIP(ctx, hipStreamSynchronize(st));
+    SR_HIP(ctx, b->stage.end(st));
     return SR_OK;
 }
 

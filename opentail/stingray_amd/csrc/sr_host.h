@@ -41,6 +41,65 @@ struct DeviceBuf {
     template <typename T> T* as() const { return (T*)p; }
 };
 
+// Pinned host memory that a batch packs its small uploads into, so that the copies to the device are truly
+// asynchronous and the upload need not wait for them.  An event marks the end of the copies of one upload; the next
+// upload waits for it before it overwrites the memory.
+struct HostStage {
+    char* p = nullptr;
+    size_t cap = 0, used = 0, wanted = 0;
+    hipEvent_t ev = nullptr;
+    bool busy = false;
+    hipError_t begin()
+    {
+        if (busy) {
+            hipError_t e = hipEventSynchronize(ev);
+            if (e != hipSuccess) return e;
+            busy = false;
+        }
+        if (wanted > cap) {
+            if (p) (void)hipHostFree(p);
+            p = nullptr;
+            cap = 0;
+            const size_t want = wanted + wanted / 2 + 4096;
+            hipError_t e = hipHostMalloc((void**)&p, want, hipHostMallocDefault);
+            if (e != hipSuccess) { p = nullptr; return e; }
+            cap = want;
+        }
+        used = wanted = 0;
+        return hipSuccess;
+    }
+    // a copy of src inside the pinned memory, or nullptr when it does not fit (it will the next time)
+    const void* put(const void* src, size_t bytes)
+    {
+        const size_t need = (bytes + 255) & ~(size_t)255;
+        wanted += need;
+        if (used + need > cap) return nullptr;
+        void* dst = p + used;
+        memcpy(dst, src, bytes);
+        used += need;
+        return dst;
+    }
+    hipError_t end(hipStream_t st)
+    {
+        if (!ev) {
+            hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+            if (e != hipSuccess) return e;
+        }
+        hipError_t e = hipEventRecord(ev, st);
+        if (e == hipSuccess) busy = true;
+        return e;
+    }
+    void release()
+    {
+        if (p) (void)hipHostFree(p);
+        if (ev) (void)hipEventDestroy(ev);
+        p = nullptr;
+        ev = nullptr;
+        cap = used = wanted = 0;
+        busy = false;
+    }
+};
+
 struct sr_ctx {
     int device = 0;
     hipStream_t own_stream = nullptr;
@@ -83,6 +142,8 @@ struct sr_batch {
     int32_t scan_epv = 0, scan_base_mod = -1, scan_stride_mod = -1;
     bool has_mask = false;
     int32_t max_sel = 0;
+    HostStage stage;          // pinned copies of what an upload sends to the device
+    bool upload_must_wait = false;  // some copy of the running upload reads pageable memory directly
 };
 
 inline int sr_fail(sr_ctx* ctx, int code, const std::string& msg)

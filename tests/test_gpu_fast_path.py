@@ -334,3 +334,39 @@ def test_vocabularies_of_more_than_four_chunks_per_row(ctx):
                          PreviousTokens=hb[i, :25].tolist() + rng.integers(0, Vb, 30).tolist())
           for i, k in enumerate([5, 1, 200, 900])]
     _check_rows(ctx, up, pb, rng.random(4), _cuda(bits.view(np.int16), torch.bfloat16))
+
+
+def test_decode_loop_that_uploads_the_batch_again_every_step_without_waiting(ctx):
+    # Each step's parameters (the histories grow by the sampled token) are uploaded through the same batch object
+    # right behind the previous step's launch; nothing is waited for until the end.
+    import torch
+
+    rng = np.random.default_rng(91)
+    rows, V, steps = 24, 20_000, 20
+    logits = [rng.normal(0, 2.0, (rows, V)).astype(np.float32) for _ in range(3)]
+    dev = [_cuda(x) for x in logits]
+    hist = [rng.integers(0, V, int(rng.integers(0, 30))).tolist() for _ in range(rows)]
+    base = [SamplingParams(Temperature=float(rng.choice([0.0, 0.7, 1.0])), TopK=int(rng.choice([1, 20, 200])),
+                           TopP=float(rng.choice([1.0, 0.9])), MinP=float(rng.choice([0.0, 0.02])),
+                           RepetitionPenalty=float(rng.choice([1.0, 1.3])), PresencePenalty=float(rng.choice([0.0, 0.4])),
+                           RepeatLastN=int(rng.choice([0, 8, 64]))) for _ in range(rows)]
+    uniforms = rng.random((steps, rows))
+    # the whole sequence from the oracle first
+    want, per_step_params = [], []
+    for s in range(steps):
+        ps = [SamplingParams(**{**p.__dict__, "PreviousTokens": list(hist[r])}) for r, p in enumerate(base)]
+        per_step_params.append(ps)
+        t = oracle_tokens(logits[s % 3], ps, uniforms[s])
+        want.append(t)
+        for r in range(rows):
+            hist[r].append(int(t[r]))
+    batch = ctx.new_batch()
+    outs = [torch.full((rows,), -9, dtype=torch.int32, device="cuda") for _ in range(steps)]
+    for s in range(steps):
+        batch.upload(per_step_params[s], V, uniforms[s])
+        ctx.sample_launch(batch, dev[s % 3], outs[s])
+    ctx.synchronize()
+    torch.cuda.synchronize()
+    batch.close()
+    for s in range(steps):
+        assert np.array_equal(outs[s].cpu().numpy(), want[s]), f"step {s}"
