@@ -132,6 +132,9 @@ SR_API void sr_batch_destroy(sr_batch* batch);
  *   mask_active   [rows] non-zero = row is constrained (ITokenConstraint.IsConstraining and Filter did
  *                 not return the input span); NULL = every row when allow_mask is given.
  *   uniforms      [rows x uniforms_per_row] NextDouble() values, consumed in order per row.
+ * Every host array may be reused when the call returns.  The copies to the device run on the context's stream
+ * and are not waited for (except for an allow-mask): launches that follow on the same stream see the batch
+ * complete; sr_set_stream synchronises the stream it leaves.
  */
 SR_API int sr_batch_upload(sr_batch* batch, int32_t rows, int32_t vocab,
                            const sr_row_params* params,
