@@ -187,8 +187,10 @@ __device__ __forceinline__ float seq_sum_tiles(Load load, int n, float s0, float
     return s;
 }
 
+// (every term is multiplied by m1 and then by m2 first: the two normalising factors of a row that was left unscaled)
 template <bool kSearch>
-__device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm)
+__device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm,
+                                             float m1 = 1.0f, float m2 = 1.0f)
 {
     static_assert(SR_SEQ_RUN % 4 == 0, "whole float4 per thread");
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
@@ -205,6 +207,8 @@ __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, fl
 #pragma unroll
             for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? p[i0 + j] : 0.0f;
         }
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = __fmul_rn(__fmul_rn(x[j], m1), m2);
     };
     return seq_sum_tiles<kSearch>(load, n, s0, target, found, sm);
 }
@@ -212,11 +216,11 @@ __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, fl
 // ... and over the positive part of the difference of two rows (residual resampling)
 template <bool kSearch>
 __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q, int n, float s0, float target, int* found,
-                                                  FullSmem& sm)
+                                                  FullSmem& sm, float m1 = 1.0f, float m2 = 1.0f)
 {
     const bool aligned = (((uintptr_t)p | (uintptr_t)q) & 15u) == 0u;
-    auto res = [](float a, float b) -> float {
-        const float r = __fsub_rn(a, b);
+    auto res = [&](float a, float b) -> float {
+        const float r = __fsub_rn(__fmul_rn(__fmul_rn(a, m1), m2), b);
         return r > 0.0f ? r : 0.0f;
     };
     auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
@@ -461,7 +465,10 @@ __global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
     src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
     src.scale = rd.temperature > 0.0f && rd.temperature != 1.0f;
     src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
-    if (blockIdx.x == 0 && threadIdx.x == 0) a.state[slot].maxkey = 0u;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        a.state[slot].maxkey = 0u;
+        a.state[slot].mul1 = a.state[slot].mul2 = 1.0f;
+    }
     if (row_is_direct(rd)) return;  // nothing edits this row: the kernels behind read the logits themselves
     stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c) { store_run(w, i, x, c); });
 }
@@ -602,11 +609,11 @@ __device__ __forceinline__ int row_argmax(const float* w, int n, FullSmem& sm)
 
 // first index whose running fp32 sum reaches r = (float)u; last index as the rounding fallback
 // (SampleFromDistribution, Sampler.cs:564-576)
-__device__ __forceinline__ int draw_from_row(const float* p, int n, double u, FullSmem& sm)
+__device__ __forceinline__ int draw_from_row(const float* p, int n, double u, FullSmem& sm, float m1 = 1.0f, float m2 = 1.0f)
 {
     const float r = __double2float_rn(u);
     int found;
-    seq_sum_row<true>(p, n, 0.0f, r, &found, sm);
+    seq_sum_row<true>(p, n, 0.0f, r, &found, sm, m1, m2);
     return found >= 0 ? found : n - 1;
 }
 
@@ -717,6 +724,24 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             FPROF(a, slot, 2);
             const bool do_scale = sum > 0.0f && sum != 1.0f;
             const float inv = do_scale ? __fdiv_rn(1.0f, sum) : 1.0f;
+            if (a.lazy_scale && a.mode == 1 && !(rd.top_k > 0 && rd.top_k < n) && !(rd.min_p > 0.0f) && !use_top_p) {
+                // No filter touches the row: its final entries are fmul(fmul(e, inv), inv2) with inv2 from the final
+                // Normalize (Sampler.cs:91-92) over the scaled values.  The reader applies the two factors; the row
+                // keeps e and is not written again.
+                const float sum2 = tp_sum([&](int i) -> float { return __fmul_rn(p[i], inv); }, n, sm);
+                const float inv2 = (sum2 > 0.0f && sum2 != 1.0f) ? __fdiv_rn(1.0f, sum2) : 1.0f;
+                if (tid == 0) {
+                    st->mul1 = inv;
+                    st->mul2 = inv2;
+                    st->n_survivors = 0;
+                    st->big = 0;
+                    st->flags = flags;
+                    st->pad = 1;  // finished in this phase
+                    a.seg_begin[slot] = a.seg_end[slot] = (int)((size_t)slot * a.sort_stride);
+                    if (a.out_flags) a.out_flags[row] = flags;
+                }
+                return;
+            }
             if (!(rd.top_k > 0 && rd.top_k < n) && (rd.min_p > 0.0f || use_top_p)) {
                 // No top-k stage in between: the scaling, the min-p cut (Sampler.cs:493-503) and the count of
                 // survivors that top-p starts from share one pass.  The largest probability needs no search: the
@@ -1042,15 +1067,16 @@ __global__ __launch_bounds__(kT) void k_draw_rows(const float* probs, int64_t st
 
 // residual = max(0, p - q): first the left-to-right sum of the positive residuals, then the first index
 // whose running residual reaches (float)u * sum; degenerate residual -> draw from p (Sampler.cs:587-618)
-__device__ __forceinline__ int resample_residual_row(const float* p, const float* q, int n, double u, FullSmem& sm)
+__device__ __forceinline__ int resample_residual_row(const float* p, const float* q, int n, double u, FullSmem& sm,
+                                                     float m1 = 1.0f, float m2 = 1.0f)
 {
     int dummy;
     auto res = [&](int i) -> float {
-        const float r = __fsub_rn(p[i], q[i]);
+        const float r = __fsub_rn(__fmul_rn(__fmul_rn(p[i], m1), m2), q[i]);
         return r > 0.0f ? r : 0.0f;
     };
-    const float sum = seq_sum_residual<false>(p, q, n, 0.0f, 0.0f, &dummy, sm);
-    if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm);  // sum <= 0 or NaN
+    const float sum = seq_sum_residual<false>(p, q, n, 0.0f, 0.0f, &dummy, sm, m1, m2);
+    if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm, m1, m2);  // sum <= 0 or NaN
     const float target = __fmul_rn(__double2float_rn(u), sum);
     // `target <= cum` is only tested on positive residuals: a zero target must not stop on a zero term
     int found;
@@ -1067,7 +1093,7 @@ __device__ __forceinline__ int resample_residual_row(const float* p, const float
         __syncthreads();
         return f;  // sum > 0 guarantees a positive residual exists
     }
-    seq_sum_residual<true>(p, q, n, 0.0f, target, &found, sm);
+    seq_sum_residual<true>(p, q, n, 0.0f, target, &found, sm, m1, m2);
     if (found >= 0) return found;
     // rounding fallback: the last index with a positive residual
     int last = -1;
@@ -1112,7 +1138,8 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
         const float* pd = pr + (size_t)i * n;
         const float* qd = a.draft_probs + ((size_t)row * L + i) * n;
         const int tok = a.draft_tokens[(size_t)row * L + i];
-        const float px = pd[tok];
+        const float m1 = a.state[(size_t)row * (L + 1) + i].mul1, m2 = a.state[(size_t)row * (L + 1) + i].mul2;
+        const float px = __fmul_rn(__fmul_rn(pd[tok], m1), m2);
         bool accept;
         if (true_spec) {
             const float qx = qd[tok];
@@ -1127,14 +1154,15 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
             accepted++;
             continue;
         }
-        correction = true_spec ? resample_residual_row(pd, qd, n, u[udraws++], sm)
-                               : draw_from_row(pd, n, u[udraws++], sm);
+        correction = true_spec ? resample_residual_row(pd, qd, n, u[udraws++], sm, m1, m2)
+                               : draw_from_row(pd, n, u[udraws++], sm, m1, m2);
         break;
     }
     if (correction < 0) {
         // every draft accepted: bonus token from the last position (greedy rows: its argmax, no draw)
         const float* pd = pr + (size_t)L * n;
-        correction = rd.temperature <= 0.0f ? row_argmax(pd, n, sm) : draw_from_row(pd, n, u[udraws++], sm);
+        const SrFullState* sl = a.state + (size_t)row * (L + 1) + L;
+        correction = rd.temperature <= 0.0f ? row_argmax(pd, n, sm) : draw_from_row(pd, n, u[udraws++], sm, sl->mul1, sl->mul2);
     }
     if (threadIdx.x == 0) {
         out[accepted] = correction;

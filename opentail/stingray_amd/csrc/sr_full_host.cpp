@@ -11,7 +11,7 @@ namespace {
 //   mode 0: work rows live in ctx scratch, tokens out.   mode 1/2: work rows ARE the caller's probs rows.
 int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows, bool any_top_p, const void* logits_dev,
              int dtype, int64_t row_stride, int mode, float* probs_dev, int64_t probs_stride, int32_t* out_tokens_dev,
-             uint32_t* out_flags_dev)
+             uint32_t* out_flags_dev, bool lazy_scale = false)
 {
     if (n_rows <= 0) return SR_OK;
     hipStream_t st = ctx->stream;
@@ -40,6 +40,7 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
         a.work_by_row = 1;
     }
     a.two_phase = any_top_p ? 1 : 0;
+    a.lazy_scale = lazy_scale ? 1 : 0;
     SR_HIP(ctx, ctx->full_state.reserve((size_t)n_rows * sizeof(SrFullState), st));
     a.state = ctx->full_state.as<SrFullState>();
     SR_HIP(ctx, ctx->seg.reserve((size_t)n_rows * 2 * sizeof(int32_t), st));
@@ -432,7 +433,7 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
     int rc = identity_list(ctx, rows * P, &list);
     if (rc == SR_OK)
         rc = run_full(ctx, &tmp, list, rows * P, any_top_p, target_logits_dev, SR_DTYPE_F32, V, 1, ctx->spec_probs.as<float>(), V,
-                      nullptr, nullptr);
+                      nullptr, nullptr, true);  // (the verifier applies the normalising factors of unfiltered rows itself)
     tmp.d_rows.p = nullptr;  // borrowed
     tmp.d_edits.p = nullptr;
     if (rc != SR_OK) return rc;
@@ -441,6 +442,7 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
     a.vocab = V;
     a.n_draft = n_draft;
     a.p_all = ctx->spec_probs.as<float>();
+    a.state = ctx->full_state.as<SrFullState>();
     a.target_logits = target_logits_dev;
     a.draft_probs = draft_probs_dev;
     a.draft_tokens = draft_tokens_dev;

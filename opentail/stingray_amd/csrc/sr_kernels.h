@@ -80,7 +80,8 @@ struct SrFullState {
     uint32_t flags;
     int32_t pad;          // 1 = the row was finished by the first phase
     uint32_t maxkey;      // ordered key of the row's largest adjusted logit (0xffffffff = the row holds a NaN)
-    int32_t pad2[3];
+    float mul1, mul2;     // the row's entries are to be multiplied by these two, in this order (1 unless lazy_scale)
+    int32_t pad2;
 };
 
 struct SrFullArgs {
@@ -98,6 +99,8 @@ struct SrFullArgs {
     int32_t work_by_row;
     int32_t mode;              // 0 = sample, 1 = distribution only, 2 = distribution and sample
     int32_t two_phase;         // a device-wide sort of large nuclei runs between phase 1 and phase 2
+    int32_t lazy_scale;        // mode 1 only: rows that no filter touches keep expf(x - max); their two normalising
+                               // factors go to state[slot].mul1 / mul2 for the reader to apply
     SrFullState* state;        // [slot]
     uint32_t* sort_keys_in;    // [slot][sort_stride]
     int32_t* sort_vals_in;
@@ -128,7 +131,8 @@ struct SrSpecArgs {
     const SrRow* rows;
     int32_t vocab;
     int32_t n_draft;
-    const float* p_all;          // [rows][n_draft + 1][vocab] filtered target distributions
+    const float* p_all;          // [rows][n_draft + 1][vocab] filtered target distributions, to be multiplied by ...
+    const SrFullState* state;    // ... mul1 and mul2 of [rows][n_draft + 1]
     const float* target_logits;  // [rows][n_draft + 1][vocab]
     const float* draft_probs;    // [rows][n_draft][vocab]
     const int32_t* draft_tokens; // [rows][n_draft]
