@@ -128,7 +128,8 @@ __device__ __forceinline__ SrInc sr_scan_inc(SrInc v)
 // A sum that starts small doubles within a few terms, again within twice as many, and so on: after a crossing at
 // thread f the next one is expected near thread 2f.  The round after a crossing therefore looks at the threads up to
 // 2f + 64 only (waves outside that window skip the arithmetic and the scan); a window that passes without a
-// crossing is settled like a whole tile and the rest of the tile follows in one more round.
+// crossing is settled like a whole tile and the rest of the tile follows in one more round.  The wave that holds a
+// crossing finishes all of its 64 threads by itself before the block goes on.
 template <bool kSearch>
 __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float* s, float target, int* found,
                                             SrSeqSmem& sm)
@@ -180,31 +181,60 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
                 pre.a0 = (uint32_t)__builtin_amdgcn_readlane((int)ti.a0, wave - 1);
                 pre.a1 = (uint32_t)__builtin_amdgcn_readlane((int)ti.a1, wave - 1);
             }
-            SrInc ex;
-            ex.a0 = __shfl_up(incl.a0, 1);
-            ex.a1 = __shfl_up(incl.a1, 1);
-            if (lane == 0) { ex.a0 = 0u; ex.a1 = 0u; }
-            ex = sr_compose(pre, ex);
-            // exact integer state before / after this thread's run, valid while below 2^24
-            const uint32_t before = sr_sat_add(n_in, (n_in & 1u) ? ex.a1 : ex.a0);
-            const SrInc thr = sr_compose(ex, mine);
-            const uint32_t after = sr_sat_add(n_in, (n_in & 1u) ? thr.a1 : thr.a0);
-            bool mine_ev = after >= (1u << 24);
-            if (kSearch) mine_ev = mine_ev || sr_join(after, eb) >= target;
-            const unsigned long long evl = __ballot(mine_ev && tid >= start);
-            const int fl = evl ? (int)__ffsll((long long)evl) - 1 : SR_WAVE - 1;  // evl != 0 by construction
-            if (lane == fl) {
-                // replay this run with real float adds from its exact input
-                float acc = sr_join(before, eb);
-                int where = -1;
+            // The exact state at this wave's first lane; from here the wave goes on alone, crossing after crossing
+            // (a sum that starts small crosses several binades inside one wave), and hands the block the state
+            // behind its last lane: no barrier and no shared memory per crossing.
+            uint32_t n_w = n_in + ((n_in & 1u) ? pre.a1 : pre.a0);
+            int eb_w = eb;
+            SrInc sc = incl;  // inclusive scan of the wave's increments in the binade eb_w, from n_w
+            int lstart = max(start - wave * SR_WAVE, 0);  // lanes below are settled
+            float s_w = 0.0f;
+            int where = -1, last = SR_WAVE - 1;
+            for (;;) {
+                SrInc ex;
+                ex.a0 = __shfl_up(sc.a0, 1);
+                ex.a1 = __shfl_up(sc.a1, 1);
+                if (lane == 0) { ex.a0 = 0u; ex.a1 = 0u; }
+                const bool odd = (n_w & 1u) != 0u;
+                // exact integer state before / after this thread's run, valid while below 2^24
+                const uint32_t before = sr_sat_add(n_w, odd ? ex.a1 : ex.a0);
+                const uint32_t after = sr_sat_add(n_w, odd ? sc.a1 : sc.a0);
+                bool mine_ev = after >= (1u << 24);
+                if (kSearch) mine_ev = mine_ev || sr_join(after, eb_w) >= target;
+                const unsigned long long evl = __ballot(mine_ev && lane >= lstart);
+                if (!evl) {
+                    // the rest of the wave stays in the binade
+                    const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)(odd ? sc.a1 : sc.a0), SR_WAVE - 1);
+                    s_w = sr_join(n_w + tot, eb_w);
+                    last = SR_WAVE - 1;
+                    break;
+                }
+                const int fl = (int)__ffsll((long long)evl) - 1;
+                // every lane replays its run with real float adds from its own input; the first event lane's counts
+                float acc = sr_join(before, eb_w);
+                int wj = -1;
 #pragma unroll
                 for (int j = 0; j < SR_SEQ_RUN; j++) {
                     acc = __fadd_rn(acc, x[j]);
-                    if (kSearch && where < 0 && acc >= target) where = tid * SR_SEQ_RUN + j;
+                    if (kSearch && wj < 0 && acc >= target) wj = j;
                 }
-                sm.misc[0] = sr_f2u(acc);
+                s_w = sr_u2f((uint32_t)__builtin_amdgcn_readlane((int)sr_f2u(acc), fl));
+                wj = __builtin_amdgcn_readlane(wj, fl);
+                last = fl;
+                if (kSearch && wj >= 0) { where = (wave * SR_WAVE + fl) * SR_SEQ_RUN + wj; break; }
+                lstart = fl + 1;
+                if (lstart >= SR_WAVE) break;
+                // the lanes behind it, scanned again in the binade the sum has reached
+                sr_split(s_w, &n_w, &eb_w);
+                SrInc m;
+                m.a0 = 0u; m.a1 = 0u;
+                if (lane >= lstart) m = sr_run_inc(x, eb_w);
+                sc = sr_scan_inc<false>(m);
+            }
+            if (lane == 0) {
+                sm.misc[0] = sr_f2u(s_w);
                 sm.misc[1] = (uint32_t)where;
-                sm.misc[2] = (uint32_t)tid;
+                sm.misc[2] = (uint32_t)(wave * SR_WAVE + last);
             }
         }
         __syncthreads();
