@@ -1134,17 +1134,36 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
     for (int i = threadIdx.x; i <= L; i += kT) out[i] = -1;
     __syncthreads();
     int accepted = 0, udraws = 0, correction = -1;
+    // What the accept tests need of every position -- the draft token, its target and draft probabilities -- is
+    // fetched for all positions at once: three dependent loads per position would otherwise line up one behind
+    // the other along the walk.
+    constexpr int kStage = 1024;
+    const bool staged = L <= kStage;
+    if (staged) {
+        for (int i = (int)threadIdx.x; i < L; i += kT) {
+            const int tok = a.draft_tokens[(size_t)row * L + i];
+            const SrFullState* sl = a.state + (size_t)row * (L + 1) + i;
+            sm.sprob[i] = __fmul_rn(__fmul_rn(pr[(size_t)i * n + tok], sl->mul1), sl->mul2);
+            sm.sprob[kStage + i] = true_spec ? a.draft_probs[((size_t)row * L + i) * n + tok] : 0.0f;
+            sm.sprob[2 * kStage + i] = __int_as_float(tok);
+        }
+        for (int i = (int)threadIdx.x; i <= L && i < a.uniforms_per_row; i += kT)
+            sm.sortbuf[i] = (unsigned long long)__double_as_longlong(u[i]);
+        __syncthreads();
+    }
     for (int i = 0; i < L; i++) {
         const float* pd = pr + (size_t)i * n;
         const float* qd = a.draft_probs + ((size_t)row * L + i) * n;
-        const int tok = a.draft_tokens[(size_t)row * L + i];
-        const float m1 = a.state[(size_t)row * (L + 1) + i].mul1, m2 = a.state[(size_t)row * (L + 1) + i].mul2;
-        const float px = __fmul_rn(__fmul_rn(pd[tok], m1), m2);
+        const int tok = staged ? __float_as_int(sm.sprob[2 * kStage + i]) : a.draft_tokens[(size_t)row * L + i];
+        const SrFullState* sl = a.state + (size_t)row * (L + 1) + i;
+        const float px = staged ? sm.sprob[i] : __fmul_rn(__fmul_rn(pd[tok], sl->mul1), sl->mul2);
         bool accept;
         if (true_spec) {
-            const float qx = qd[tok];
+            const float qx = staged ? sm.sprob[kStage + i] : qd[tok];
             const float acc = qx > 0.0f ? fminf(1.0f, __fdiv_rn(px, qx)) : (px > 0.0f ? 1.0f : 0.0f);
-            accept = u[udraws++] < (double)acc;
+            const double ui = staged ? __longlong_as_double((long long)sm.sortbuf[udraws]) : u[udraws];
+            udraws++;
+            accept = ui < (double)acc;
         } else {
             accept = px >= rd.p_min;
             if (!accept) accept = tok == row_argmax(lg + (size_t)i * n, n, sm);  // block-uniform branch
@@ -1154,6 +1173,7 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
             accepted++;
             continue;
         }
+        const float m1 = sl->mul1, m2 = sl->mul2;
         correction = true_spec ? resample_residual_row(pd, qd, n, u[udraws++], sm, m1, m2)
                                : draw_from_row(pd, n, u[udraws++], sm, m1, m2);
         break;
