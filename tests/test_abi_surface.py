@@ -17,6 +17,12 @@ def test_header_and_python_symbol_lists_agree():
     assert _declared_symbols() == sorted(sa.EXPORTED_SYMBOLS)
 
 
+def test_the_managed_binding_that_the_integration_notes_show_names_every_entry_point():
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    bound = sorted(set(re.findall(r'EntryPoint = "(sr_\w+)"', text)))
+    assert bound == _declared_symbols()
+
+
 def test_library_exports_every_declared_symbol():
     assert os.path.exists(sa.lib_path()), "build with: python -m opentail.stingray_amd.build"
     lib = ctypes.CDLL(sa.lib_path())
