@@ -712,6 +712,8 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         uint32_t flags = SR_KFLAG_FULL;
         bool fused = false;  // scaling, min-p and the count of survivors were done in one pass
         int survivors = 0;   // ... this thread's share of the count
+        int ns_listed = -1;  // >= 0: the block-wide count, and sm.sortbuf[0, ns_listed) holds the survivors
+        bool row_unwritten = false;  // the row still holds expf(x - max): it will be finished from the list
         if (any_nan || sr_f2u(m) == 0xff800000u) {
             const float uni = n > 0 ? __fdiv_rn(1.0f, (float)n) : 0.0f;
             row_pass<true>(p, n, [&](float, int) -> float { return uni; });
@@ -750,14 +752,44 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 const bool use_min_p = rd.min_p > 0.0f;
                 const float thr = use_min_p ? __fmul_rn(rd.min_p, mp) : 0.0f;
                 int c = 0;
-                row_pass<true>(p, n, [&](float x, int) -> float {
+                // A min-p cut leaves few survivors: they are listed while the row is read, which saves the pass that
+                // would collect them; a row that is only sampled from (no distribution out) and ends with at most
+                // 1,024 survivors is finished from that list and need not be written at all.
+                const bool list_now = use_min_p;
+                if (list_now) {
+                    if (tid == 0) sm.bc[4] = 0u;
+                    __syncthreads();
+                }
+                auto body = [&](float x, int i) -> float {
                     float y = do_scale ? __fmul_rn(x, inv) : x;
                     if (use_min_p && y < thr) y = 0.0f;
-                    c += y > 0.0f ? 1 : 0;
+                    if (y > 0.0f) {
+                        c++;
+                        if (list_now) {
+                            const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
+                            if (pos < (uint32_t)kSmall)
+                                sm.sortbuf[pos] = ((unsigned long long)sr_f2u(y) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+                        }
+                    }
                     return y;
-                });
+                };
+                const bool read_only = list_now && a.mode == 0 && n >= 8;
+                if (read_only) row_pass<false>(p, n, body); else row_pass<true>(p, n, body);
                 survivors = c;
                 fused = true;
+                if (list_now) {
+                    const int ns_now = blk_sum_i(c, sm);
+                    if (ns_now <= kSmall) ns_listed = ns_now;
+                    row_unwritten = read_only && ns_now > 0 && ns_now <= 1024;
+                    if (read_only && !row_unwritten) {
+                        // too many survivors to finish from the list: the scaled row is needed after all
+                        row_pass<true>(p, n, [&](float x, int) -> float {
+                            float y = do_scale ? __fmul_rn(x, inv) : x;
+                            if (use_min_p && y < thr) y = 0.0f;
+                            return y;
+                        });
+                    }
+                }
             } else if (do_scale) {
                 row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
             }
@@ -793,6 +825,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             // positions in index order (stable input for the device-wide sort)
             // each thread owns the strided indices tid, tid + kT, ...; a second pass assigns slots per tile
             ns = blk_sum_i(cnt, sm);
+            const bool have_list = ns_listed >= 0;  // (then ns == ns_listed <= kSmall)
             int nc = ns;           // candidates sorted inside the kernel
             float c_above = -1.0f;  // ... are the probabilities strictly above this value
             if (ns > kSmall) {
@@ -807,15 +840,17 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             }
             bool closed = false;
             if (nc > 0 && nc <= kSmall) {
-                if (tid == 0) sm.bc[4] = 0u;
-                __syncthreads();
-                row_pass<false>(p, n, [&](float v, int i) -> float {
-                    if (v > 0.0f && v > c_above) {
-                        const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
-                        sm.sortbuf[pos] = ((unsigned long long)sr_f2u(v) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
-                    }
-                    return v;
-                });
+                if (!have_list) {
+                    if (tid == 0) sm.bc[4] = 0u;
+                    __syncthreads();
+                    row_pass<false>(p, n, [&](float v, int i) -> float {
+                        if (v > 0.0f && v > c_above) {
+                            const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
+                            sm.sortbuf[pos] = ((unsigned long long)sr_f2u(v) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+                        }
+                        return v;
+                    });
+                }
                 __syncthreads();
                 int P = 2;
                 while (P < nc) P <<= 1;
@@ -829,8 +864,9 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 closed = found >= 0 || nc == ns;
                 if (closed) {
                     const int cutoff = found >= 0 ? found + 1 : nc;
-                    for (int i = cutoff + tid; i < nc; i += kT)
-                        p[0xffffffffu - (uint32_t)(sm.sortbuf[i] & 0xffffffffull)] = 0.0f;
+                    if (!row_unwritten)
+                        for (int i = cutoff + tid; i < nc; i += kT)
+                            p[0xffffffffu - (uint32_t)(sm.sortbuf[i] & 0xffffffffull)] = 0.0f;
                     __syncthreads();
                     if (nc < ns) {  // everything that was not a candidate comes later in the order
                         row_pass<true>(p, n, [&](float x, int) -> float { return x > c_above ? x : 0.0f; });
@@ -868,6 +904,8 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 }
             }
             if (tid == 0) st->n_survivors = ns;
+        } else if (ns_listed > 0 && ns_listed <= 1024 && n >= 8) {
+            listed = ns_listed;  // min-p alone: its survivors are the members
         }
         FPROF(a, slot, 6);
         // (up to a thousand members: beyond that the passes over the row are the faster way)

@@ -395,3 +395,21 @@ def test_sample_with_distribution_rows(ctx):
         t, d = orc.sample_with_distribution(logits[r], to_oracle(p), orc.Rng(replay=[u[r]]))
         assert toks[r] == t, r
         assert np.array_equal(probs[r].view(np.uint32), np.asarray(d, dtype=np.float32).view(np.uint32)), r
+
+
+def test_min_p_rows_with_few_and_with_thousands_of_survivors(ctx):
+    # min-p survivors are listed while the row is read: rows with up to 1,024 of them are finished from the list
+    # (sampled rows are then not written at all), rows with more take the passes over the row
+    rng = np.random.default_rng(81)
+    V = 50_000
+    logits = rng.normal(0, 1.5, (6, V)).astype(np.float32)
+    params = [SamplingParams(Temperature=1.0, MinP=0.05), SamplingParams(Temperature=0.8, MinP=0.05, TopP=0.9),
+              SamplingParams(Temperature=1.0, MinP=1e-3), SamplingParams(Temperature=1.2, MinP=1e-3, TopP=0.95),
+              SamplingParams(Temperature=1.0, MinP=1e-5, TopP=0.9), SamplingParams(Temperature=1.5, MinP=1e-6)]
+    _check_distribution(ctx, logits, params)
+    for _ in range(4):
+        _check_rows(ctx, logits, params, rng.random(6))
+    toks, probs = ctx.sample_with_distribution(_cuda(logits), params, np.full(6, 0.999999))
+    for r, p in enumerate(params):
+        t, d = orc.sample_with_distribution(logits[r], to_oracle(p), orc.Rng(replay=[0.999999]))
+        assert toks[r] == t and np.array_equal(probs[r].cpu().numpy().view(np.uint32), np.asarray(d, np.float32).view(np.uint32)), r
