@@ -13,6 +13,7 @@ back to, and loading fails loudly when the library has not been built.
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 import os
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence
@@ -178,6 +179,7 @@ class _Batch:
         self.ctx = ctx
         self.h = C.c_void_p()
         ctx._check(ctx.L.sr_batch_create(ctx.h, C.byref(self.h)))
+        ctx._batches.add(self)  # a batch must not outlive its context: the context closes what is left
         self.rows = 0
         self.vocab = 0
 
@@ -216,7 +218,7 @@ class _Batch:
                 act = np.ascontiguousarray(np.asarray(mask_active, dtype=np.uint8))
         u = None
         upr = 0
-        if uniforms is not None:
+        if uniforms is not None and rows > 0:
             u = np.ascontiguousarray(np.asarray(uniforms, dtype=np.float64)).reshape(rows, -1)
             upr = u.shape[1] if uniforms_per_row is None else uniforms_per_row
         self.ctx._check(self.ctx.L.sr_batch_upload(
@@ -232,7 +234,9 @@ class _Batch:
 
     def close(self):
         if self.h:
-            self.ctx.L.sr_batch_destroy(self.h)
+            self.ctx._batches.discard(self)
+            if self.ctx.h:
+                self.ctx.L.sr_batch_destroy(self.h)
             self.h = C.c_void_p()
 
     def __del__(self):  # pragma: no cover
@@ -248,6 +252,7 @@ class SamplerContext:
     def __init__(self, device: int = 0, use_torch_stream: bool = True):
         self.L = load_library()
         self.h = C.c_void_p()
+        self._batches = weakref.WeakSet()
         rc = self.L.sr_create(device, C.byref(self.h))
         if rc == SR_ERR_NO_DEVICE:
             raise NativeLibraryError("no HIP device: the sampler has no CPU path")
@@ -283,6 +288,8 @@ class SamplerContext:
 
     def close(self):
         if self.h:
+            for b in list(self._batches):
+                b.close()
             self.L.sr_destroy(self.h)
             self.h = C.c_void_p()
 
