@@ -1470,7 +1470,6 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     const int nvt = (V + mis + EPV - 1) / EPV;        // vectors of the row window
     const int f0 = c * a.chunk_vecs;                   // first vector of this chunk
     const int nv = min(a.chunk_vecs, nvt - f0);        // vectors of this chunk
-    const int wbase = f0 * EPV - mis;                  // row element index of the chunk's first window element
 
     if (nv > 0) {
         const u32x4* cp = (const u32x4*)(rowp - (size_t)mis * ES) + f0;
