@@ -1498,15 +1498,22 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         // three words (loaded ahead of the data), bit j * EPV + q = element q of its j-th vector.  They carry the
         // row's edges, its allow-mask and, when the row tail fetches them, its history ids: two operations per
         // element replace all per-element edge, allow-mask and history logic.
+        // A wave all of whose elements are kept (no edge, no allow-mask, no history id among them) skips them.
+        constexpr int kBits = kVec * EPV;
+        static_assert(kBits > 64 && kBits <= 96, "three keep-words per thread");
+        constexpr uint32_t kLast = kBits == 96 ? 0xffffffffu : ((1u << (kBits - 64)) - 1u);
+        const bool all_kept = (kw0 & kw1) == 0xffffffffu && (kw2 & kLast) == kLast;
+        if (__ballot(!all_kept) != 0ull) {
 #pragma unroll
-        for (int j = 0; j < kVec; j++)
+            for (int j = 0; j < kVec; j++)
 #pragma unroll
-            for (int q = 0; q < EPV; q++) {
-                const int bit = j * EPV + q;
-                const uint32_t w = bit < 32 ? kw0 : bit < 64 ? kw1 : kw2;
-                const uint32_t t = (uint32_t)((int)(w << (31 - (bit & 31))) >> 31);  // all ones = keep
-                xv[j * EPV + q] = sr_u2f((sr_f2u(xv[j * EPV + q]) & t) | (0xff800000u & ~t));
-            }
+                for (int q = 0; q < EPV; q++) {
+                    const int bit = j * EPV + q;
+                    const uint32_t w = bit < 32 ? kw0 : bit < 64 ? kw1 : kw2;
+                    const uint32_t t = (uint32_t)((int)(w << (31 - (bit & 31))) >> 31);  // all ones = keep
+                    xv[j * EPV + q] = sr_u2f((sr_f2u(xv[j * EPV + q]) & t) | (0xff800000u & ~t));
+                }
+        }
         if (a.prof) pt1 = wall_clock64();
 
         // Every lane owns four interleaved groups of vectors (j mod 4).  Of each group the row tail gets the largest
