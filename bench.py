@@ -236,6 +236,21 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     kern_us = dev_ms * 1e3 / args.steps  # device time per launch from HIP events on the launch stream
 
+    # a decode step that also uploads its batch again (histories change every step): host packing + copies + launch
+    step_with_upload_us = None
+    if args.workload.startswith("c3"):
+        n_up = max(10, args.steps // 4)
+        for i in range(3):
+            batches[i % n_buf].reupload()
+            step(i)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(n_up):
+            batches[i % n_buf].reupload()
+            step(i)
+        torch.cuda.synchronize()
+        step_with_upload_us = (time.perf_counter() - t1) * 1e6 / n_up
+
     # parity of the measured outputs against the oracle (outside the timed region)
     parity = None
     if not args.no_parity:
@@ -291,6 +306,7 @@ def main():
         "cpu_baseline": cpu,
         "parity": parity,
         "rows_unsupported": unsupported,
+        "us_per_step_with_batch_upload": step_with_upload_us,
     }
     print(json.dumps(out))
 

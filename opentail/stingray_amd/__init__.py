@@ -221,11 +221,18 @@ class _Batch:
         if uniforms is not None and rows > 0:
             u = np.ascontiguousarray(np.asarray(uniforms, dtype=np.float64)).reshape(rows, -1)
             upr = u.shape[1] if uniforms_per_row is None else uniforms_per_row
+        self._packed = (rows, vocab, arr, h_ids, h_off, b_ids, b_vals, b_off, m, stride, act, u, upr)
+        self.rows, self.vocab = rows, vocab
+        return self.reupload()
+
+    def reupload(self):
+        """sr_batch_upload once more with the arrays of the last upload(): what a decode step costs the host beyond
+        gathering its parameters."""
+        rows, vocab, arr, h_ids, h_off, b_ids, b_vals, b_off, m, stride, act, u, upr = self._packed
         self.ctx._check(self.ctx.L.sr_batch_upload(
             self.h, rows, vocab, arr, _ptr(h_ids, C.c_int32), _ptr(h_off, C.c_int32),
             _ptr(b_ids, C.c_int32), _ptr(b_vals, C.c_float), _ptr(b_off, C.c_int32),
             _ptr(m, C.c_uint32), stride, _ptr(act, C.c_uint8), _ptr(u, C.c_double), upr))
-        self.rows, self.vocab = rows, vocab
         return self
 
     def set_uniforms(self, uniforms):
