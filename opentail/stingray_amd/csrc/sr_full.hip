@@ -698,6 +698,10 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         if (tid == 0) {
             if (a.out_tokens) a.out_tokens[row] = am;
             if (a.out_flags) a.out_flags[row] = SR_KFLAG_GREEDY | SR_KFLAG_FULL;
+            // an empty segment for the device-wide sort that may follow (it reads every row's bounds)
+            a.seg_begin[slot] = a.seg_end[slot] = (int)((size_t)slot * a.sort_stride);
+            st->big = 0;
+            st->pad = 1;
         }
         return;
     }

@@ -309,6 +309,9 @@ def test_nuclei_of_tens_of_thousands_of_members_take_the_device_wide_sort(ctx):
     _check_distribution(ctx, logits, params)
     for _ in range(4):
         _check_rows(ctx, logits, params, rng.random(4))
+    # greedy rows in the same batch of distributions: their (empty) sort segments lie between the others'
+    mixed = [SamplingParams(Temperature=0.0), params[0], SamplingParams(Temperature=0.0, TopP=0.5), params[1]]
+    _check_distribution(ctx, logits[[3, 0, 2, 1]], mixed)
     # the same under dense allow-masks and next to rows of the other paths
     allowed = rng.random((4, V)) < np.array([0.6, 0.9, 0.5, 1.0])[:, None]
     mask = pack_allow_mask(allowed)
