@@ -100,7 +100,9 @@ SR_API void sr_destroy(sr_ctx* ctx);
 SR_API int sr_bind_thread(sr_ctx* ctx);
 /* Kernels are enqueued on this stream (a hipStream_t); NULL restores the context's own stream.  Lets
  * the forward pass that produced the logits and the sampler share one stream, so no event is needed
- * between them (the pattern of CudaBackend.cs:4119-4123). */
+ * between them (the pattern of CudaBackend.cs:4119-4123).  The context's own stream is non-blocking: it is
+ * not ordered with the device's default stream, so a caller whose tensors are produced there either passes
+ * hipStreamLegacy (the default stream by name) or synchronises before the launch. */
 SR_API int sr_set_stream(sr_ctx* ctx, void* hip_stream);
 SR_API int sr_synchronize(sr_ctx* ctx);
 /* Text of the last failure on this context (never NULL). */

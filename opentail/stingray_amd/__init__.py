@@ -26,6 +26,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "lib", "libstingray_sampler.so")
 
 SR_OK = 0
+HIP_STREAM_LEGACY = 1  # hipStreamLegacy: the device's default stream, named explicitly
 SR_ERR_INVALID_ARGUMENT = 1
 SR_ERR_NULL_ARGUMENT = 2
 SR_ERR_HIP = 3
@@ -269,7 +270,10 @@ class SamplerContext:
         if use_torch_stream:
             import torch
 
-            self.L.sr_set_stream(self.h, C.c_void_p(torch.cuda.current_stream(device).cuda_stream))
+            # torch's default stream has the handle 0, which sr_set_stream reads as "the context's own stream": a
+            # non-blocking stream that nothing orders behind torch's work.  The default stream is named explicitly.
+            handle = torch.cuda.current_stream(device).cuda_stream
+            self._check(self.L.sr_set_stream(self.h, C.c_void_p(handle or HIP_STREAM_LEGACY)))
 
     # -- plumbing ------------------------------------------------------------------------------
     def _check(self, rc: int):
@@ -285,6 +289,7 @@ class SamplerContext:
         raise RuntimeError(f"native sampler error {rc}: {msg}")
 
     def set_stream(self, stream_handle: Optional[int]):
+        """A hipStream_t handle; None or 0 = the context's own stream (HIP_STREAM_LEGACY names the default stream)."""
         self._check(self.L.sr_set_stream(self.h, C.c_void_p(stream_handle or 0)))
 
     def synchronize(self):

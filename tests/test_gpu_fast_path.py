@@ -370,3 +370,30 @@ def test_decode_loop_that_uploads_the_batch_again_every_step_without_waiting(ctx
     batch.close()
     for s in range(steps):
         assert np.array_equal(outs[s].cpu().numpy(), want[s]), f"step {s}"
+
+
+def test_launches_are_ordered_behind_torch_work_on_the_default_stream(ctx):
+    # torch's default stream has the handle 0; the context must still run on that stream, not on a stream of its
+    # own that nothing orders behind the kernels producing the logits.  The logits arrive behind some milliseconds
+    # of queued work and are sampled without a wait in between.
+    import torch
+
+    rng = np.random.default_rng(77)
+    rows, n = 8, 5000
+    lg = rng.normal(0, 3, (rows, n)).astype(np.float32)
+    params = [SamplingParams(Temperature=0.0) for _ in range(rows // 2)] + \
+             [SamplingParams(Temperature=0.7, TopK=40) for _ in range(rows - rows // 2)]
+    u = rng.random(rows)
+    want = oracle_tokens(lg, params, u)
+    src = _cuda(lg)
+    junk = torch.zeros(1 << 27, dtype=torch.float32, device="cuda")
+    for attempt in range(3):
+        dev = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        for _ in range(30):
+            junk.add_(1.0)
+        dev.copy_(src)
+        got = ctx.sample_batch(dev, params, u)
+        assert np.array_equal(got, want), attempt
+        probs = ctx.build_distribution(dev, params[rows // 2:] + params[:rows // 2])
+        assert float(probs.sum()) == pytest.approx(rows, rel=1e-4)
