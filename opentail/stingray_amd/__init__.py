@@ -117,6 +117,13 @@ def load_library():
         raise NativeLibraryError(
             f"{_LIB_PATH} is missing: build it with `python -m opentail.stingray_amd.build` "
             "(hipcc, gfx950). There is no CPU fallback.")
+    # torch brings its own copy of the HIP runtime.  It has to be the first one in the process: with the system's
+    # runtime loaded before it (by this library), torch finds no GPU afterwards.  Loaded second, this library binds
+    # to the runtime that is already there.
+    try:
+        import torch  # noqa: F401
+    except ImportError:  # pragma: no cover - the mirror allocates through torch, the library itself does not need it
+        pass
     try:
         L = C.CDLL(_LIB_PATH)
     except OSError as e:  # pragma: no cover - depends on the host
