@@ -238,7 +238,7 @@ def main():
 
     # a decode step that also uploads its batch again (histories change every step): host packing + copies + launch
     step_with_upload_us = None
-    if args.workload.startswith("c3"):
+    if args.workload.startswith("c3") and not os.environ.get("SR_BENCH_NO_UPLOAD_LEG"):
         n_up = max(10, args.steps // 4)
         for i in range(3):
             batches[i % n_buf].reupload()
