@@ -273,6 +273,30 @@ def main():
         torch.cuda.synchronize()
         step_with_upload_us = (time.perf_counter() - t1) * 1e6 / n_up
 
+    # a decode step that appends the sampled token to every history instead (sr_batch_append_tokens; random ids stand
+    # in for the sampled ones, so most are new to their history and every 16th step or so a row runs out of room and
+    # the batch is rebuilt).  Batches and outputs of their own: the measured ones stay as they are for the parity check.
+    step_with_append_us = None
+    if args.workload.startswith("c3") and not os.environ.get("SR_BENCH_NO_UPLOAD_LEG"):
+        n_up = max(10, args.steps // 4)
+        ab = [ctx.new_batch().upload(w.params, vocab, w.uniforms, w.allow_mask, w.mask_active) for _ in range(n_buf)]
+        atok = torch.empty(rows, dtype=torch.int32, device="cuda")
+        rng = np.random.default_rng(7)
+        ids = rng.integers(0, vocab, (n_up + 3, rows)).astype(np.int32)
+        un = rng.random((n_up + 3, rows))
+        for i in range(3):
+            ab[i % n_buf].append_tokens(ids[i], un[i])
+            ctx.sample_launch(ab[i % n_buf], bufs[i % n_buf], atok)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(n_up):
+            ab[i % n_buf].append_tokens(ids[i + 3], un[i + 3])
+            ctx.sample_launch(ab[i % n_buf], bufs[i % n_buf], atok)
+        torch.cuda.synchronize()
+        step_with_append_us = (time.perf_counter() - t1) * 1e6 / n_up
+        for b_ in ab:
+            b_.close()
+
     # parity of the measured outputs against the oracle (outside the timed region)
     parity = None
     if not args.no_parity:
@@ -330,6 +354,7 @@ def main():
         "parity": parity,
         "rows_unsupported": unsupported,
         "us_per_step_with_batch_upload": step_with_upload_us,
+        "us_per_step_with_token_append": step_with_append_us,
     }
     print(json.dumps(out))
 

@@ -145,6 +145,18 @@ SR_API int sr_batch_upload(sr_batch* batch, int32_t rows, int32_t vocab,
                            const uint32_t* allow_mask, int64_t mask_stride_words,
                            const uint8_t* mask_active,
                            const double* uniforms, int32_t uniforms_per_row);
+/* One more token at the end of every row's history, as the engine appends the sampled token to the sequence's
+ * RecentTokens after each step (src/OpenTail.Stingray.Engine/ContinuousBatchingEngine.cs:650, 1280): afterwards the
+ * batch is what sr_batch_upload would build from the longer histories and the same other inputs, for the cost of
+ * the few entries that change instead of a pass over every history.
+ *   tokens    [rows] host array; a negative entry leaves its row's history as it is.
+ *   uniforms  [rows x uniforms_per_row] for the next step, or NULL to keep those on the device.
+ * Rows the in-place update does not cover (the first history token of a row with penalties, rows with logit bias
+ * or with penalties that may raise a logit, a row that runs out of room) make the call rebuild the whole batch from
+ * the inputs it kept: same result, the cost of an upload.  A batch uploaded with allow-masks returns
+ * SR_ERR_UNSUPPORTED: its masks change with every step, so it is uploaded again anyway.  Copies run on the
+ * context's stream and are not waited for, as in sr_batch_upload. */
+SR_API int sr_batch_append_tokens(sr_batch* batch, const int32_t* tokens, const double* uniforms);
 /* Replaces only the uniforms of an uploaded batch (same rows and uniforms_per_row). */
 SR_API int sr_batch_set_uniforms(sr_batch* batch, const double* uniforms);
 

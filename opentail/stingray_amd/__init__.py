@@ -46,6 +46,7 @@ SR_OUT_ROW_UNSUPPORTED = 1 << 31
 EXPORTED_SYMBOLS = [
     "sr_create", "sr_destroy", "sr_bind_thread", "sr_set_stream", "sr_synchronize", "sr_last_error",
     "sr_version", "sr_batch_create", "sr_batch_destroy", "sr_batch_upload", "sr_batch_set_uniforms",
+    "sr_batch_append_tokens",
     "sr_sample_launch", "sr_resample_rows_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows",
     "sr_build_distribution_launch", "sr_sample_with_distribution_launch", "sr_sample_from_probs_launch",
     "sr_resample_residual_launch", "sr_spec_verify_launch", "sr_mtp_verify_launch", "sr_pack_allow_mask",
@@ -146,6 +147,7 @@ def load_library():
     L.sr_batch_upload.argtypes = [vp, i32, i32, rpp, i32p, i32p, i32p, f32p, i32p, u32p, i64,
                                   C.POINTER(C.c_uint8), f64p, i32]
     L.sr_batch_set_uniforms.argtypes = [vp, f64p]
+    L.sr_batch_append_tokens.argtypes = [vp, i32p, f64p]
     L.sr_sample_launch.argtypes = [vp, vp, vp, C.c_int, i64, vp, vp]
     L.sr_resample_rows_launch.argtypes = [vp, vp, vp, C.c_int, i64, i32p, i32, vp, vp]
     L.sr_sample_batch.argtypes = [vp, vp, C.c_int, C.c_int, i32, i32, i64, rpp, i32p, i32p, i32p, f32p, i32p,
@@ -241,6 +243,17 @@ class _Batch:
             self.h, rows, vocab, arr, _ptr(h_ids, C.c_int32), _ptr(h_off, C.c_int32),
             _ptr(b_ids, C.c_int32), _ptr(b_vals, C.c_float), _ptr(b_off, C.c_int32),
             _ptr(m, C.c_uint32), stride, _ptr(act, C.c_uint8), _ptr(u, C.c_double), upr))
+        return self
+
+    def append_tokens(self, tokens, uniforms=None):
+        """sr_batch_append_tokens: one more token per row (negative = none) at the end of the histories of the last
+        upload(), and optionally the uniforms of the next step."""
+        t = np.ascontiguousarray(np.asarray(tokens, dtype=np.int32))
+        assert t.shape == (self.rows,)
+        u = None
+        if uniforms is not None:
+            u = np.ascontiguousarray(np.asarray(uniforms, dtype=np.float64))
+        self.ctx._check(self.ctx.L.sr_batch_append_tokens(self.h, _ptr(t, C.c_int32), _ptr(u, C.c_double)))
         return self
 
     def set_uniforms(self, uniforms):

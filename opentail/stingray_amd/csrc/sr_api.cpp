@@ -140,6 +140,10 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
         SR_HIP(ctx, batch_copy(b, staged, b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), st));
     }
     b->scan_stride = (int64_t)chunks * SR_TK_THREADS * SR_TK_MASK_WORDS;
+    b->scan_chunks = chunks;
+    b->scan_chunk_vecs = chunk_vecs;
+    b->scan_base_addr = base_addr;
+    b->scan_stride_bytes = stride_bytes;
     if (rows_changed)
         SR_HIP(ctx, batch_copy(b, staged, b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), st));
     SR_HIP(ctx, b->d_scan_desc.reserve(b->h_scan.size() * sizeof(SrScanDesc), st));
@@ -239,17 +243,19 @@ void sr_batch_destroy(sr_batch* b)
     if (!b) return;
     if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
     DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_wide_list, &b->d_scan_desc,
-                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched};
+                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched, &b->d_patch};
     for (DeviceBuf* d : bufs) d->release();
     b->stage.release();
     delete b;
 }
 
-int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_params* params,
-                    const int32_t* hist_ids, const int32_t* hist_offsets,
-                    const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
-                    const uint32_t* allow_mask, int64_t mask_stride_words, const uint8_t* mask_active,
-                    const double* uniforms, int32_t uniforms_per_row)
+// sr_batch_upload.  retain: keep what sr_batch_append_tokens needs of the inputs; keep_uniforms: the uniforms on the
+// device stay as they are (uniforms is not read).
+static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_params* params,
+                             const int32_t* hist_ids, const int32_t* hist_offsets,
+                             const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                             const uint32_t* allow_mask, int64_t mask_stride_words, const uint8_t* mask_active,
+                             const double* uniforms, int32_t uniforms_per_row, bool retain, bool keep_uniforms)
 {
     if (!b || !b->ctx) return SR_ERR_NULL_ARGUMENT;
     sr_ctx* ctx = b->ctx;
@@ -261,7 +267,7 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: bias arrays are null");
     if (allow_mask && mask_stride_words < (vocab + 31) / 32)
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_upload: mask stride shorter than ceil(vocab/32)");
-    if (uniforms_per_row < 0 || (uniforms_per_row > 0 && !uniforms))
+    if (uniforms_per_row < 0 || (uniforms_per_row > 0 && !uniforms && !keep_uniforms))
         return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: uniforms is null");
     SR_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
@@ -282,6 +288,30 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
     b->has_mask = allow_mask != nullptr;
     b->mask_stride = allow_mask ? mask_stride_words : 0;
     b->max_sel = 0;
+    b->edit_cap.assign((size_t)rows, 0);
+    if (retain) {
+        b->can_append = allow_mask == nullptr;
+        b->hist_split = false;
+        b->keep_hist.clear();
+        if (b->can_append) {
+            b->keep_params.assign(params, params + rows);
+            const int32_t n_hist = hist_offsets ? hist_offsets[rows] : 0, n_bias = bias_offsets ? bias_offsets[rows] : 0;
+            b->keep_hist_off.assign((size_t)rows + 1, 0);
+            if (hist_offsets) b->keep_hist_off.assign(hist_offsets, hist_offsets + rows + 1);
+            b->keep_hist_ids.clear();
+            if (n_hist > 0) b->keep_hist_ids.assign(hist_ids, hist_ids + n_hist);
+            b->keep_bias_off.clear();
+            b->keep_bias_ids.clear();
+            b->keep_bias_vals.clear();
+            if (bias_offsets) {
+                b->keep_bias_off.assign(bias_offsets, bias_offsets + rows + 1);
+                if (n_bias > 0) {
+                    b->keep_bias_ids.assign(bias_ids, bias_ids + n_bias);
+                    b->keep_bias_vals.assign(bias_vals, bias_vals + n_bias);
+                }
+            }
+        }
+    }
 
     std::vector<int32_t> slots;  // scratch of the history de-duplication
     for (int32_t r = 0; r < rows; r++) {
@@ -394,6 +424,11 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
                 }
             }
             d.edit_cnt = (int32_t)ed.size() - d.edit_off;
+            b->edit_cap[(size_t)r] = d.edit_cnt;
+            if (want_hist && !searched && d.edit_cnt > 0) {  // room for the ids that appended tokens bring
+                ed.resize(ed.size() + SR_EDIT_SLACK);
+                b->edit_cap[(size_t)r] += SR_EDIT_SLACK;
+            }
         }
         // Penalties that can only lower a logit (Sampler.cs:281-286 with repetition >= 1, presence >= 0 and
         // frequency >= 0) cannot lift a history token past a token outside the history: the scan then skips
@@ -449,7 +484,7 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
         SR_HIP(ctx, b->d_mask.reserve(bytes, st));
         SR_HIP(ctx, batch_copy(b, false, b->d_mask.p, allow_mask, bytes, st));
     }
-    if (uniforms_per_row > 0)
+    if (uniforms_per_row > 0 && !keep_uniforms)
         SR_HIP(ctx, up(b->d_uniforms, uniforms, (size_t)rows * (size_t)uniforms_per_row * sizeof(double)));
     // scan masks for the layout of the last launch (16-byte aligned rows); a launch with another layout rebuilds
     if (!b->h_sel_list.empty()) {
@@ -460,6 +495,152 @@ int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_param
     // Everything small went through the batch's pinned memory: the copies and the scan-mask kernel run on while
     // the caller goes on (launches on this stream are ordered behind them).  Pageable memory that a copy reads
     // directly (the caller's allow-mask; anything the pinned memory had no room for yet) must be waited for.
+    if (b->upload_must_wait) SR_HIP(ctx, hipStreamSynchronize(st));
+    SR_HIP(ctx, b->stage.end(st));
+    return SR_OK;
+}
+
+int sr_batch_upload(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_params* params,
+                    const int32_t* hist_ids, const int32_t* hist_offsets,
+                    const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                    const uint32_t* allow_mask, int64_t mask_stride_words, const uint8_t* mask_active,
+                    const double* uniforms, int32_t uniforms_per_row)
+{
+    return batch_upload_impl(b, rows, vocab, params, hist_ids, hist_offsets, bias_ids, bias_vals, bias_offsets, allow_mask,
+                             mask_stride_words, mask_active, uniforms, uniforms_per_row, true, false);
+}
+
+// The batch as sr_batch_upload would build it for the histories as they are now (rows the in-place update does not
+// cover: a first history token, sorted edit lists, an edit range without room, a change of path).
+static int append_rebuild(sr_batch* b, const double* uniforms)
+{
+    const int32_t rows = b->rows;
+    std::vector<sr_row_params> params = b->keep_params;
+    std::vector<int32_t> ids, off((size_t)rows + 1, 0);
+    for (int32_t r = 0; r < rows; r++) {
+        ids.insert(ids.end(), b->keep_hist[(size_t)r].begin(), b->keep_hist[(size_t)r].end());
+        off[(size_t)r + 1] = (int32_t)ids.size();
+    }
+    const std::vector<int32_t> bias_ids = b->keep_bias_ids, bias_off = b->keep_bias_off;
+    const std::vector<float> bias_vals = b->keep_bias_vals;
+    return batch_upload_impl(b, rows, b->vocab, params.data(), ids.data(), off.data(),
+                             bias_off.empty() ? nullptr : bias_ids.data(), bias_off.empty() ? nullptr : bias_vals.data(),
+                             bias_off.empty() ? nullptr : bias_off.data(), nullptr, 0, nullptr, uniforms, b->upr, false,
+                             uniforms == nullptr);
+}
+
+int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uniforms)
+{
+    if (!b || !b->ctx) return SR_ERR_NULL_ARGUMENT;
+    sr_ctx* ctx = b->ctx;
+    if (!tokens) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_append_tokens: tokens is null");
+    if (!b->can_append)
+        return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_batch_append_tokens: the batch was not uploaded, or was uploaded with "
+                                                "allow-masks (upload it again with the new masks)");
+    const int32_t rows = b->rows, vocab = b->vocab;
+    if (rows == 0) return SR_OK;
+    if (!b->hist_split) {
+        b->keep_hist.assign((size_t)rows, std::vector<int32_t>());
+        for (int32_t r = 0; r < rows; r++) {
+            const int32_t h0 = b->keep_hist_off[(size_t)r], h1 = b->keep_hist_off[(size_t)r + 1];
+            if (h1 > h0) b->keep_hist[(size_t)r].assign(b->keep_hist_ids.begin() + h0, b->keep_hist_ids.begin() + h1);
+        }
+        b->hist_split = true;
+    }
+    for (int32_t r = 0; r < rows; r++)
+        if (tokens[r] >= 0) b->keep_hist[(size_t)r].push_back(tokens[r]);
+
+    // In place: one token more in the history of a row changes the occurrence counts of at most two ids (the one that
+    // enters, the one that leaves the repetition window, Sampler.cs:272-279) and may add one id.
+    std::vector<SrEditPatch> ep;
+    std::vector<SrMaskClear> mc;
+    std::vector<int32_t> touched;
+    bool rows_dirty = false, rebuild = false;
+    for (int32_t r = 0; r < rows && !rebuild; r++) {
+        if (tokens[r] < 0) continue;
+        const sr_row_params& p = b->keep_params[(size_t)r];
+        SrRow& d = b->h_rows[(size_t)r];
+        const std::vector<int32_t>& hist = b->keep_hist[(size_t)r];
+        const int32_t n_new = (int32_t)hist.size(), n_old = n_new - 1;
+        rows_dirty = true;
+        if (!has_history_penalty(p)) {  // the history is never looked at
+            d.n_prev = n_new;
+            continue;
+        }
+        if (n_old == 0 || d.edit_cnt == 0 || (d.flags & SR_ROWFLAG_EDITS_SORTED) || d.path == SR_PATH_TOPK_WIDE) {
+            rebuild = true;
+            break;
+        }
+        SrEdit* ed = b->h_edits.data() + d.edit_off;
+        auto find = [&](int32_t id) -> int32_t {
+            for (int32_t i = 0; i < d.edit_cnt; i++)
+                if (ed[i].id == id) return i;
+            return -1;
+        };
+        auto repow = [&](SrEdit& e) {
+            e.pen = (p.repetition_penalty != 1.0f && e.occ_win > 0) ? powf(p.repetition_penalty, (float)e.occ_win) : 1.0f;
+        };
+        touched.clear();
+        const int32_t rl = p.repeat_last_n;
+        const int32_t ws_old = (rl <= 0 || rl >= n_old) ? 0 : n_old - rl, ws_new = (rl <= 0 || rl >= n_new) ? 0 : n_new - rl;
+        for (int32_t i = ws_old; i < ws_new; i++) {  // leaves the window
+            const int32_t id = hist[(size_t)i];
+            if ((uint32_t)id >= (uint32_t)vocab) continue;
+            const int32_t k = find(id);
+            if (k < 0) { rebuild = true; break; }
+            ed[k].occ_win--;
+            repow(ed[k]);
+            touched.push_back(k);
+        }
+        if (rebuild) break;
+        const int32_t t = tokens[r];
+        if ((uint32_t)t < (uint32_t)vocab) {
+            int32_t k = find(t);
+            if (k < 0) {
+                const bool topk = d.path == SR_PATH_TOPK;
+                if (d.edit_cnt >= b->edit_cap[(size_t)r] || d.edit_cnt + 1 > SR_TK_SEL_MAX ||
+                    (topk && (int64_t)p.top_k + d.edit_cnt + 1 > SR_TK_SEL_MAX)) {
+                    rebuild = true;
+                    break;
+                }
+                k = d.edit_cnt++;
+                ed[k] = SrEdit{};
+                ed[k].id = t;
+                if (b->h_scan_need[(size_t)r] & SR_SCAN_HIST) mc.push_back(SrMaskClear{d.scan_row, r, t});
+            }
+            ed[k].occ_all++;
+            ed[k].occ_win++;
+            repow(ed[k]);
+            touched.push_back(k);
+        }
+        d.n_prev = n_new;
+        for (int32_t k : touched) ep.push_back(SrEditPatch{d.edit_off + k, ed[k]});
+    }
+    if (rebuild) {
+        b->append_rebuilds++;
+        return append_rebuild(b, uniforms);
+    }
+
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    SR_HIP(ctx, b->stage.begin());
+    b->upload_must_wait = false;
+    if (rows_dirty)
+        SR_HIP(ctx, batch_copy(b, true, b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), st));
+    if (!ep.empty() || !mc.empty()) {
+        const size_t eb = (ep.size() * sizeof(SrEditPatch) + 15) & ~(size_t)15, cb = mc.size() * sizeof(SrMaskClear);
+        SR_HIP(ctx, b->d_patch.reserve(eb + cb, st));
+        SR_HIP(ctx, batch_copy(b, true, b->d_patch.p, ep.data(), ep.size() * sizeof(SrEditPatch), st));
+        SR_HIP(ctx, batch_copy(b, true, (char*)b->d_patch.p + eb, mc.data(), cb, st));
+        // scan masks that are not built yet are built from the patched edits when they are needed
+        const bool masks = b->scan_epv != 0 && b->d_scan_mask.p != nullptr;
+        SR_HIP(ctx, sr_launch_apply_patches(b->d_edits.as<SrEdit>(), (const SrEditPatch*)b->d_patch.p, (int)ep.size(),
+                                            (const SrMaskClear*)((char*)b->d_patch.p + eb), masks ? (int)mc.size() : 0,
+                                            b->d_scan_mask.as<uint32_t>(), b->scan_stride, masks ? b->scan_epv : 4,
+                                            masks ? b->scan_chunk_vecs : 64, b->scan_base_addr, b->scan_stride_bytes, st));
+    }
+    if (uniforms && b->upr > 0)
+        SR_HIP(ctx, batch_copy(b, true, b->d_uniforms.p, uniforms, (size_t)rows * (size_t)b->upr * sizeof(double), st));
     if (b->upload_must_wait) SR_HIP(ctx, hipStreamSynchronize(st));
     SR_HIP(ctx, b->stage.end(st));
     return SR_OK;
@@ -709,6 +890,9 @@ int sr_pack_allow_mask(const float* masked_logits, int32_t vocab, uint32_t* out_
     }
     return SR_OK;
 }
+
+// Test hook (not part of the public header): how many sr_batch_append_tokens calls on this batch rebuilt it.
+SR_API int sr_debug_append_rebuilds(const sr_batch* b) { return b ? b->append_rebuilds : -1; }
 
 // Test hook: phase timestamps (wall_clock64, 100 MHz) of the selection kernel go to prof_dev[grid][16].
 SR_API int sr_debug_set_profile(sr_ctx* ctx, unsigned long long* prof_dev)

@@ -144,7 +144,25 @@ struct sr_batch {
     int32_t max_sel = 0;
     HostStage stage;          // pinned copies of what an upload sends to the device
     bool upload_must_wait = false;  // some copy of the running upload reads pageable memory directly
+    // geometry the scan masks were built with (sr_batch_append_tokens clears single bits in place)
+    int32_t scan_chunks = 0, scan_chunk_vecs = 0;
+    unsigned long long scan_base_addr = 0;
+    long long scan_stride_bytes = 0;
+    // What sr_batch_append_tokens needs of the last upload: the inputs of a batch without allow-masks (kept flat as
+    // they came; the histories are split per row by the first append) and the room each row's edit range has.
+    bool can_append = false, hist_split = false;
+    int32_t append_rebuilds = 0;  // calls of sr_batch_append_tokens that rebuilt the batch (test hook)
+    std::vector<sr_row_params> keep_params;
+    std::vector<int32_t> keep_hist_ids, keep_hist_off, keep_bias_ids, keep_bias_off;
+    std::vector<float> keep_bias_vals;
+    std::vector<std::vector<int32_t>> keep_hist;
+    std::vector<int32_t> edit_cap;
+    DeviceBuf d_patch;
 };
+
+// room left behind the edits of a row whose edits are kept in order of first appearance, for ids that
+// sr_batch_append_tokens adds
+#define SR_EDIT_SLACK 16
 
 inline int sr_fail(sr_ctx* ctx, int code, const std::string& msg)
 {

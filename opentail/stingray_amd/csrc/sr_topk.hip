@@ -1650,7 +1650,40 @@ __global__ __launch_bounds__(kThreads) void k_build_scan_mask(const SrScanDesc* 
     for (int i = t; i < kThreads * SR_TK_MASK_WORDS; i += kThreads) dst[i] = words[i];
 }
 
+// Applies what one appended token per row changes: whole edits at given positions of the edit array, and single
+// keep-bits of scan-mask rows cleared for ids that entered a history (same element -> bit mapping as above).
+__global__ __launch_bounds__(256) void k_apply_patches(SrEdit* edits, const SrEditPatch* ep, int n_edits,
+                                                       const SrMaskClear* mc, int n_clears, uint32_t* scan_mask,
+                                                       int64_t scan_stride, int epv, int es, int chunk_vecs,
+                                                       unsigned long long base_addr, long long stride_bytes)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_edits) edits[ep[i].index] = ep[i].edit;
+    if (i < n_clears) {
+        const SrMaskClear m = mc[i];
+        const int mis = (int)(((base_addr + (unsigned long long)m.row * (unsigned long long)stride_bytes) & 15ull) / (unsigned)es);
+        const int p = m.id + mis;
+        const int fv = p / epv, q = p - fv * epv;
+        const int c = fv / chunk_vecs, fl = fv - c * chunk_vecs;
+        const int j = fl / kThreads, tt = fl - j * kThreads;
+        const int b = j * epv + q;
+        atomicAnd(&scan_mask[(size_t)m.scan_row * scan_stride + ((size_t)c * kThreads + tt) * SR_TK_MASK_WORDS + (b >> 5)],
+                  ~(1u << (b & 31)));
+    }
+}
+
 }  // namespace
+
+hipError_t sr_launch_apply_patches(SrEdit* edits, const SrEditPatch* ep, int n_edits, const SrMaskClear* mc, int n_clears,
+                                   uint32_t* scan_mask, int64_t scan_stride, int epv, int chunk_vecs,
+                                   unsigned long long base_addr, long long stride_bytes, hipStream_t stream)
+{
+    const int n = n_edits > n_clears ? n_edits : n_clears;
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_apply_patches, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, edits, ep, n_edits, mc,
+                       n_clears, scan_mask, scan_stride, epv, epv == 8 ? 2 : 4, chunk_vecs, base_addr, stride_bytes);
+    return hipGetLastError();
+}
 
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
 {

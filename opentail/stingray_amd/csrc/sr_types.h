@@ -46,6 +46,17 @@ struct SrScanDesc {
     int32_t row;
     uint32_t flags;
 };
+// What sr_batch_append_tokens sends to the device: an edit to be written at a position of the edit array, and a
+// keep-bit of a scan-mask row to be cleared (the id entered the row's history).
+struct SrEditPatch {
+    int32_t index;
+    SrEdit edit;
+};
+struct SrMaskClear {
+    int32_t scan_row;
+    int32_t row;
+    int32_t id;
+};
 #define SR_SCAN_ALLOW 1u  // start from the row's allow-mask
 #define SR_SCAN_HIST 2u   // clear the row's history ids
 
