@@ -78,8 +78,8 @@ def cpu_baseline(w, budget_s: float):
 
 def prime_events(torch, stream):
     """Warm-up of the event machinery.  The first timing event that a process records on a stream has been seen to
-    make the launches queued behind it run one at a time (220 us instead of 53 us per launch for that first window
-    only, in any process but the first on a machine), so a pair is recorded and resolved before the warm-up steps."""
+    slow the launches queued behind it down (220 us instead of 53 us per launch for that first window only, in any
+    process but the first on a machine), so a pair is recorded and resolved before the warm-up steps."""
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     e1.record(stream)
