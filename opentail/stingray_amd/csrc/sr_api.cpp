@@ -243,7 +243,7 @@ void sr_batch_destroy(sr_batch* b)
     if (!b) return;
     if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
     DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_wide_list, &b->d_scan_desc,
-                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched, &b->d_patch};
+                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched};
     for (DeviceBuf* d : bufs) d->release();
     b->stage.release();
     delete b;
@@ -289,6 +289,7 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
     b->mask_stride = allow_mask ? mask_stride_words : 0;
     b->max_sel = 0;
     b->edit_cap.assign((size_t)rows, 0);
+    b->edit_ids.clear();
     if (retain) {
         b->can_append = allow_mask == nullptr;
         b->hist_split = false;
@@ -552,19 +553,39 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
 
     // In place: one token more in the history of a row changes the occurrence counts of at most two ids (the one that
     // enters, the one that leaves the repetition window, Sampler.cs:272-279) and may add one id.
+    if (b->edit_ids.size() != b->h_edits.size()) {
+        b->edit_ids.resize(b->h_edits.size());
+        for (size_t i = 0; i < b->h_edits.size(); i++) b->edit_ids[i] = b->h_edits[i].id;
+    }
+    // powf(repetition_penalty, occurrences): rows mostly share the penalty, and the counts are small
+    float pow_rep = 1.0f, pow_of[16];
+    bool pow_known[16] = {};
+    auto pow_cached = [&](float rep, int32_t occ) -> float {
+        if (occ >= 16) return powf(rep, (float)occ);
+        if (rep != pow_rep) {
+            pow_rep = rep;
+            for (bool& k : pow_known) k = false;
+        }
+        if (!pow_known[occ]) {
+            pow_of[occ] = powf(rep, (float)occ);
+            pow_known[occ] = true;
+        }
+        return pow_of[occ];
+    };
+    std::vector<SrRowPatch> rp;
     std::vector<SrEditPatch> ep;
     std::vector<SrMaskClear> mc;
     std::vector<int32_t> touched;
-    bool rows_dirty = false, rebuild = false;
+    bool rebuild = false;
     for (int32_t r = 0; r < rows && !rebuild; r++) {
         if (tokens[r] < 0) continue;
         const sr_row_params& p = b->keep_params[(size_t)r];
         SrRow& d = b->h_rows[(size_t)r];
         const std::vector<int32_t>& hist = b->keep_hist[(size_t)r];
         const int32_t n_new = (int32_t)hist.size(), n_old = n_new - 1;
-        rows_dirty = true;
         if (!has_history_penalty(p)) {  // the history is never looked at
             d.n_prev = n_new;
+            rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt});
             continue;
         }
         if (n_old == 0 || d.edit_cnt == 0 || (d.flags & SR_ROWFLAG_EDITS_SORTED) || d.path == SR_PATH_TOPK_WIDE) {
@@ -572,13 +593,13 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
             break;
         }
         SrEdit* ed = b->h_edits.data() + d.edit_off;
+        int32_t* eids = b->edit_ids.data() + d.edit_off;
         auto find = [&](int32_t id) -> int32_t {
-            for (int32_t i = 0; i < d.edit_cnt; i++)
-                if (ed[i].id == id) return i;
-            return -1;
+            const int32_t* f = std::find(eids, eids + d.edit_cnt, id);
+            return f == eids + d.edit_cnt ? -1 : (int32_t)(f - eids);
         };
         auto repow = [&](SrEdit& e) {
-            e.pen = (p.repetition_penalty != 1.0f && e.occ_win > 0) ? powf(p.repetition_penalty, (float)e.occ_win) : 1.0f;
+            e.pen = (p.repetition_penalty != 1.0f && e.occ_win > 0) ? pow_cached(p.repetition_penalty, e.occ_win) : 1.0f;
         };
         touched.clear();
         const int32_t rl = p.repeat_last_n;
@@ -606,6 +627,7 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
                 k = d.edit_cnt++;
                 ed[k] = SrEdit{};
                 ed[k].id = t;
+                eids[k] = t;
                 if (b->h_scan_need[(size_t)r] & SR_SCAN_HIST) mc.push_back(SrMaskClear{d.scan_row, r, t});
             }
             ed[k].occ_all++;
@@ -614,6 +636,7 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
             touched.push_back(k);
         }
         d.n_prev = n_new;
+        rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt});
         for (int32_t k : touched) ep.push_back(SrEditPatch{d.edit_off + k, ed[k]});
     }
     if (rebuild) {
@@ -621,27 +644,29 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
         return append_rebuild(b, uniforms);
     }
 
+    // One kernel applies everything, reading the lists straight from the batch's pinned memory: no copy calls.
     SR_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
+    const size_t n_uni = (uniforms && b->upr > 0) ? (size_t)rows * (size_t)b->upr : 0;
+    const size_t need = rp.size() * sizeof(SrRowPatch) + ep.size() * sizeof(SrEditPatch) + mc.size() * sizeof(SrMaskClear) +
+                        n_uni * sizeof(double) + 4 * 256;
     SR_HIP(ctx, b->stage.begin());
-    b->upload_must_wait = false;
-    if (rows_dirty)
-        SR_HIP(ctx, batch_copy(b, true, b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), st));
-    if (!ep.empty() || !mc.empty()) {
-        const size_t eb = (ep.size() * sizeof(SrEditPatch) + 15) & ~(size_t)15, cb = mc.size() * sizeof(SrMaskClear);
-        SR_HIP(ctx, b->d_patch.reserve(eb + cb, st));
-        SR_HIP(ctx, batch_copy(b, true, b->d_patch.p, ep.data(), ep.size() * sizeof(SrEditPatch), st));
-        SR_HIP(ctx, batch_copy(b, true, (char*)b->d_patch.p + eb, mc.data(), cb, st));
-        // scan masks that are not built yet are built from the patched edits when they are needed
-        const bool masks = b->scan_epv != 0 && b->d_scan_mask.p != nullptr;
-        SR_HIP(ctx, sr_launch_apply_patches(b->d_edits.as<SrEdit>(), (const SrEditPatch*)b->d_patch.p, (int)ep.size(),
-                                            (const SrMaskClear*)((char*)b->d_patch.p + eb), masks ? (int)mc.size() : 0,
-                                            b->d_scan_mask.as<uint32_t>(), b->scan_stride, masks ? b->scan_epv : 4,
-                                            masks ? b->scan_chunk_vecs : 64, b->scan_base_addr, b->scan_stride_bytes, st));
+    if (b->stage.cap < need) {  // grows at begin()
+        b->stage.wanted = need;
+        SR_HIP(ctx, b->stage.begin());
     }
-    if (uniforms && b->upr > 0)
-        SR_HIP(ctx, batch_copy(b, true, b->d_uniforms.p, uniforms, (size_t)rows * (size_t)b->upr * sizeof(double), st));
-    if (b->upload_must_wait) SR_HIP(ctx, hipStreamSynchronize(st));
+    const SrRowPatch* rp_d = (const SrRowPatch*)b->stage.put(rp.data(), rp.size() * sizeof(SrRowPatch));
+    const SrEditPatch* ep_d = (const SrEditPatch*)b->stage.put(ep.data(), ep.size() * sizeof(SrEditPatch));
+    const SrMaskClear* mc_d = (const SrMaskClear*)b->stage.put(mc.data(), mc.size() * sizeof(SrMaskClear));
+    const double* un_d = (const double*)b->stage.put(uniforms, n_uni * sizeof(double));
+    if (!rp_d || !ep_d || !mc_d || !un_d) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "sr_batch_append_tokens: no pinned memory");
+    // scan masks that are not built yet are built from the patched edits when they are needed
+    const bool masks = b->scan_epv != 0 && b->d_scan_mask.p != nullptr;
+    SR_HIP(ctx, sr_launch_apply_patches(b->d_rows.as<SrRow>(), rp_d, (int)rp.size(), b->d_edits.as<SrEdit>(), ep_d,
+                                        (int)ep.size(), mc_d, masks ? (int)mc.size() : 0, b->d_scan_mask.as<uint32_t>(),
+                                        b->scan_stride, masks ? b->scan_epv : 4, masks ? b->scan_chunk_vecs : 64,
+                                        b->scan_base_addr, b->scan_stride_bytes, b->d_uniforms.as<double>(), un_d,
+                                        (int)n_uni, st));
     SR_HIP(ctx, b->stage.end(st));
     return SR_OK;
 }

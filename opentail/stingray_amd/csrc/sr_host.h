@@ -157,7 +157,7 @@ struct sr_batch {
     std::vector<float> keep_bias_vals;
     std::vector<std::vector<int32_t>> keep_hist;
     std::vector<int32_t> edit_cap;
-    DeviceBuf d_patch;
+    std::vector<int32_t> edit_ids;  // the ids of h_edits, contiguous (searched by the append; made when first needed)
 };
 
 // room left behind the edits of a row whose edits are kept in order of first appearance, for ids that

@@ -57,11 +57,14 @@ hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, int n_scan, const 
                                      int vocab, int epv, int chunks, int chunk_vecs, unsigned long long base_addr,
                                      long long stride_bytes, hipStream_t stream);
 
-// Writes n_edits whole edits into the edit array and clears n_clears keep-bits of scan masks built with the given
-// geometry (sr_batch_append_tokens).
-hipError_t sr_launch_apply_patches(SrEdit* edits, const SrEditPatch* ep, int n_edits, const SrMaskClear* mc, int n_clears,
-                                   uint32_t* scan_mask, int64_t scan_stride, int epv, int chunk_vecs,
-                                   unsigned long long base_addr, long long stride_bytes, hipStream_t stream);
+// What one appended token per row changes (sr_batch_append_tokens): history length and edit count of n_rowp rows,
+// n_edits whole edits, n_clears keep-bits of scan masks built with the given geometry, n_uni uniforms.  The lists
+// may lie in pinned host memory.
+hipError_t sr_launch_apply_patches(SrRow* rows, const SrRowPatch* rp, int n_rowp, SrEdit* edits, const SrEditPatch* ep,
+                                   int n_edits, const SrMaskClear* mc, int n_clears, uint32_t* scan_mask,
+                                   int64_t scan_stride, int epv, int chunk_vecs, unsigned long long base_addr,
+                                   long long stride_bytes, double* uni_dst, const double* uni_src, int n_uni,
+                                   hipStream_t stream);
 
 struct SrArgmaxArgs {
     const void* logits;

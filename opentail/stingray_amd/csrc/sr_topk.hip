@@ -1650,14 +1650,23 @@ __global__ __launch_bounds__(kThreads) void k_build_scan_mask(const SrScanDesc* 
     for (int i = t; i < kThreads * SR_TK_MASK_WORDS; i += kThreads) dst[i] = words[i];
 }
 
-// Applies what one appended token per row changes: whole edits at given positions of the edit array, and single
-// keep-bits of scan-mask rows cleared for ids that entered a history (same element -> bit mapping as above).
-__global__ __launch_bounds__(256) void k_apply_patches(SrEdit* edits, const SrEditPatch* ep, int n_edits,
-                                                       const SrMaskClear* mc, int n_clears, uint32_t* scan_mask,
-                                                       int64_t scan_stride, int epv, int es, int chunk_vecs,
-                                                       unsigned long long base_addr, long long stride_bytes)
+// Applies what one appended token per row changes: history length and edit count of rows, whole edits at given
+// positions of the edit array, single keep-bits of scan-mask rows cleared for ids that entered a history (same
+// element -> bit mapping as above), and the uniforms of the next step.  The lists are read where the host wrote
+// them (pinned host memory).
+__global__ __launch_bounds__(256) void k_apply_patches(SrRow* rows, const SrRowPatch* rp, int n_rowp, SrEdit* edits,
+                                                       const SrEditPatch* ep, int n_edits, const SrMaskClear* mc,
+                                                       int n_clears, uint32_t* scan_mask, int64_t scan_stride, int epv,
+                                                       int es, int chunk_vecs, unsigned long long base_addr,
+                                                       long long stride_bytes, double* uni_dst, const double* uni_src,
+                                                       int n_uni)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_rowp) {
+        const SrRowPatch r = rp[i];
+        rows[r.row].n_prev = r.n_prev;
+        rows[r.row].edit_cnt = r.edit_cnt;
+    }
     if (i < n_edits) edits[ep[i].index] = ep[i].edit;
     if (i < n_clears) {
         const SrMaskClear m = mc[i];
@@ -1670,18 +1679,22 @@ __global__ __launch_bounds__(256) void k_apply_patches(SrEdit* edits, const SrEd
         atomicAnd(&scan_mask[(size_t)m.scan_row * scan_stride + ((size_t)c * kThreads + tt) * SR_TK_MASK_WORDS + (b >> 5)],
                   ~(1u << (b & 31)));
     }
+    if (i < n_uni) uni_dst[i] = uni_src[i];
 }
 
 }  // namespace
 
-hipError_t sr_launch_apply_patches(SrEdit* edits, const SrEditPatch* ep, int n_edits, const SrMaskClear* mc, int n_clears,
-                                   uint32_t* scan_mask, int64_t scan_stride, int epv, int chunk_vecs,
-                                   unsigned long long base_addr, long long stride_bytes, hipStream_t stream)
+hipError_t sr_launch_apply_patches(SrRow* rows, const SrRowPatch* rp, int n_rowp, SrEdit* edits, const SrEditPatch* ep,
+                                   int n_edits, const SrMaskClear* mc, int n_clears, uint32_t* scan_mask,
+                                   int64_t scan_stride, int epv, int chunk_vecs, unsigned long long base_addr,
+                                   long long stride_bytes, double* uni_dst, const double* uni_src, int n_uni,
+                                   hipStream_t stream)
 {
-    const int n = n_edits > n_clears ? n_edits : n_clears;
+    const int n = std::max(std::max(n_rowp, n_edits), std::max(n_clears, n_uni));
     if (n <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_apply_patches, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, edits, ep, n_edits, mc,
-                       n_clears, scan_mask, scan_stride, epv, epv == 8 ? 2 : 4, chunk_vecs, base_addr, stride_bytes);
+    hipLaunchKernelGGL(k_apply_patches, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, rows, rp, n_rowp, edits, ep,
+                       n_edits, mc, n_clears, scan_mask, scan_stride, epv, epv == 8 ? 2 : 4, chunk_vecs, base_addr,
+                       stride_bytes, uni_dst, uni_src, n_uni);
     return hipGetLastError();
 }
 

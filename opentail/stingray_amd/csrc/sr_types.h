@@ -52,6 +52,11 @@ struct SrEditPatch {
     int32_t index;
     SrEdit edit;
 };
+struct SrRowPatch {
+    int32_t row;
+    int32_t n_prev;
+    int32_t edit_cnt;
+};
 struct SrMaskClear {
     int32_t scan_row;
     int32_t row;
