@@ -202,6 +202,11 @@ def main():
     torch.cuda.set_stream(stream)           # so HIP events recorded here bracket the sampler's kernels
     ctx = SamplerContext(0)
     prime_events(torch, stream)
+    # no collector pauses inside the timed loops (as timeit does): a full collection of this process takes tens of
+    # milliseconds, which is hundreds of steps
+    import gc
+    gc.collect()
+    gc.disable()
 
     if args.workload == "c5":
         return bench_spec(args, w, ctx, stream)
