@@ -281,7 +281,9 @@ SR_API int sr_resample_residual(sr_ctx* ctx, const float* p, int32_t p_len, int6
  * The batch supplies the rows' parameters and n_draft+1 uniforms per row (accept draws in position
  * order, then the residual / bonus draw).  spec_draft_p_min in (0,1) selects the looser accept of
  * :546,552.  Outputs (DEVICE): out_accepted[rows]; out_tokens[rows x (n_draft+1)] = accepted drafts
- * followed by the correction or bonus token, the rest -1.
+ * followed by the correction or bonus token, the rest -1.  A draft id outside [0, vocab) ends its row at that
+ * position with -1 in place of the correction token (the managed loop throws IndexOutOfRangeException at
+ * pDist[x_i], :536); out_accepted counts the drafts accepted before it.
  */
 SR_API int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* batch, const float* target_logits_dev,
                                  const float* draft_probs_dev, const int32_t* draft_tokens_dev,

@@ -427,6 +427,22 @@ class SamplerContext:
             batch.close()
         return toks.cpu().numpy(), out
 
+    def sample_with_distribution_launch(self, batch: _Batch, logits, out_probs, out_tokens):
+        """Async: the draft side of StepSampled (SpeculativeDecoder.cs:509-513): distributions and drawn tokens of
+        every row stay on the device (out_probs [rows, vocab] fp32, out_tokens [rows] int32, CUDA tensors)."""
+        vocab = logits.shape[-1]
+        self._check(self.L.sr_sample_with_distribution_launch(
+            self.h, batch.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), self._row_stride(logits),
+            C.c_void_p(out_probs.data_ptr()), self._row_stride(out_probs), vocab, C.c_void_p(out_tokens.data_ptr())))
+
+    def spec_verify_launch(self, batch: _Batch, target_logits, draft_probs, draft_tokens, out_accepted, out_tokens):
+        """Async: sr_spec_verify_launch over device tensors (target [rows, L+1, V], q [rows, L, V], tokens [rows, L])."""
+        L = target_logits.shape[1] - 1
+        self._check(self.L.sr_spec_verify_launch(
+            self.h, batch.h, C.c_void_p(target_logits.data_ptr()), C.c_void_p(draft_probs.data_ptr()),
+            C.c_void_p(draft_tokens.data_ptr()), L, C.c_void_p(out_accepted.data_ptr()),
+            C.c_void_p(out_tokens.data_ptr())))
+
     def sample_from_probs(self, probs, uniforms):
         import torch
 

@@ -1176,6 +1176,7 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
     for (int i = threadIdx.x; i <= L; i += kT) out[i] = -1;
     __syncthreads();
     int accepted = 0, udraws = 0, correction = -1;
+    bool bad_id = false;
     // What the accept tests need of every position -- the draft token, its target and draft probabilities -- is
     // fetched for all positions at once: three dependent loads per position would otherwise line up one behind
     // the other along the walk.
@@ -1185,8 +1186,9 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
         for (int i = (int)threadIdx.x; i < L; i += kT) {
             const int tok = a.draft_tokens[(size_t)row * L + i];
             const SrFullState* sl = a.state + (size_t)row * (L + 1) + i;
-            sm.sprob[i] = __fmul_rn(__fmul_rn(pr[(size_t)i * n + tok], sl->mul1), sl->mul2);
-            sm.sprob[kStage + i] = true_spec ? a.draft_probs[((size_t)row * L + i) * n + tok] : 0.0f;
+            const bool in_range = (uint32_t)tok < (uint32_t)n;  // an id outside the vocabulary is never dereferenced
+            sm.sprob[i] = in_range ? __fmul_rn(__fmul_rn(pr[(size_t)i * n + tok], sl->mul1), sl->mul2) : 0.0f;
+            sm.sprob[kStage + i] = (true_spec && in_range) ? a.draft_probs[((size_t)row * L + i) * n + tok] : 0.0f;
             sm.sprob[2 * kStage + i] = __int_as_float(tok);
         }
         for (int i = (int)threadIdx.x; i <= L && i < a.uniforms_per_row; i += kT)
@@ -1198,6 +1200,9 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
         const float* qd = a.draft_probs + ((size_t)row * L + i) * n;
         const int tok = staged ? __float_as_int(sm.sprob[2 * kStage + i]) : a.draft_tokens[(size_t)row * L + i];
         const SrFullState* sl = a.state + (size_t)row * (L + 1) + i;
+        // The managed loop indexes pDist[x_i] (SpeculativeDecoder.cs:536) and throws on an id outside the
+        // vocabulary: the row ends here, with -1 where its correction token would stand.
+        if ((uint32_t)tok >= (uint32_t)n) { bad_id = true; break; }
         const float px = staged ? sm.sprob[i] : __fmul_rn(__fmul_rn(pd[tok], sl->mul1), sl->mul2);
         bool accept;
         if (true_spec) {
@@ -1220,7 +1225,7 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
                                : draw_from_row(pd, n, u[udraws++], sm, m1, m2);
         break;
     }
-    if (correction < 0) {
+    if (correction < 0 && !bad_id) {
         // every draft accepted: bonus token from the last position (greedy rows: its argmax, no draw)
         const float* pd = pr + (size_t)L * n;
         const SrFullState* sl = a.state + (size_t)row * (L + 1) + L;

@@ -627,6 +627,9 @@ int32_t oracle_spec_verify_row(const float* target_logits, const float* draft_pr
         const float* qd = draft_probs + (int64_t)i * n;
         int32_t tok = draft_tokens[i];
         oracle_build_filtered_distribution(tl, n, p, p_dist, n);
+        /* pDist[x_i] with x_i outside the vocabulary throws IndexOutOfRangeException (SpeculativeDecoder.cs:536):
+         * the row ends at this position, reported as -1 in place of its correction token */
+        if (tok < 0 || tok >= n) { out_tokens[accepted] = -1; return accepted; }
         float px = p_dist[tok];
         int accept;
         if (true_spec) {

@@ -234,6 +234,24 @@ def test_speculative_verification_rows(ctx):
     _check_spec(ctx, t, q, k, p3, u)
 
 
+def test_draft_ids_outside_the_vocabulary_end_their_row(ctx):
+    # SpeculativeDecoder.cs:536 indexes pDist[x_i]: an id outside the vocabulary throws there.  The device never
+    # dereferences it: the row ends at that position with -1 in place of the correction token.
+    V, L = 5_000, 4
+    params = [SamplingParams() for _ in range(4)]
+    t, q, k, u = _spec_case(4, L, V, params, 9, False)
+    u[:, :L] = 0.0            # every in-range draft is accepted (u < a for any a > 0)
+    k[0, 2] = V               # one past the end
+    k[1, 0] = -1
+    k[2, 3] = 2 ** 31 - 1
+    acc, out = ctx.spec_verify(_cuda(t), _cuda(q), _cuda(k), params, u)
+    for r in range(4):
+        wa, wt = orc.spec_verify_row(t[r], q[r], k[r], to_oracle(params[r]), orc.Rng(replay=u[r]))
+        assert acc[r] == wa and list(out[r][: wa + 1]) == list(wt), (r, acc[r], wa, out[r], wt)
+    assert (acc[0], out[0][2]) == (2, -1) and (acc[1], out[1][0]) == (0, -1) and (acc[2], out[2][3]) == (3, -1)
+    assert acc[3] == L and out[3][L] >= 0
+
+
 def test_reference_distribution_preservation_invariant(ctx):
     # SpeculativeSamplingTests.cs:21-50 at a GPU-sized batch: with fixed target/draft rows the emitted
     # histogram of (accepted drafts + correction) follows softmax(target) regardless of the draft.

@@ -235,6 +235,12 @@ def test_spec_accept_rule_closed_forms():
     assert orc.spec_verify_row(tl, q1, [2], pm, Rng(replay=[0.5]))[0] == 0   # .3 < .35, argmax is 3
     assert orc.spec_verify_row(tl, q1, [3], pm, Rng(replay=[0.5]))[0] == 1
     assert V == 4
+    # a draft id outside the vocabulary: pDist[x_i] throws in the managed loop (SpeculativeDecoder.cs:536); the
+    # restatement ends the row there with -1 and draws nothing
+    for bad in (-1, 4, 2 ** 31 - 1):
+        r = Rng(replay=[0.1, 0.1])
+        acc, toks = orc.spec_verify_row(tl, q1, [bad], p, r)
+        assert acc == 0 and list(toks) == [-1] and r.draws == 0
 
 
 def test_mtp_accept_draft_closed_form():
