@@ -23,7 +23,9 @@ import numpy as np
 __all__ = ["SamplingParams", "Sampler", "SamplerContext", "NativeLibraryError", "load_library", "lib_path"]
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "lib", "libstingray_sampler.so")
+# STINGRAY_SAMPLER_LIB names another build of the library (the profiling build, say), as the reference's resolver
+# probes an override before its default names (src/OpenTail.Stingray.Cuda/CudaLibraryResolver.cs:27-47)
+_LIB_PATH = os.environ.get("STINGRAY_SAMPLER_LIB") or os.path.join(_HERE, "lib", "libstingray_sampler.so")
 
 SR_OK = 0
 HIP_STREAM_LEGACY = 1  # hipStreamLegacy: the device's default stream, named explicitly

@@ -8,6 +8,7 @@
 #include <new>
 
 #include "sr_host.h"
+#include "../../../include/stingray_sampler_test.h"
 
 namespace {
 
@@ -83,59 +84,99 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     int chunks = 1, chunk_vecs = 0;
     topk_geometry(b->vocab, epv == 8 ? SR_DTYPE_BF16 : SR_DTYPE_F32, n_sel, ctx->cu_count, &chunks, &chunk_vecs);
     {
-        // Dispatch order.  Workgroups are dispatched in grid order, two resident per CU; a round is that many
-        // consecutive workgroups.  A row's tail goes to the middle of the round after the one that holds the row's
-        // last chunk: half of that round's workgroups have retired by the time it is dispatched, so its chunks have
-        // usually finished and it does not hold a slot while it waits, yet it does not queue behind all of the
-        // later rows' chunks either.  Every entry carries what its workgroup needs to find its data.
+        // The selection kernel's grid: workers with a program each -- chunk items to stream, then at most one row to
+        // finish.  A CU holds two workgroups of this kernel, so 2 x CUs workers are resident from the start and a
+        // later one starts when one of them ends.
+        //
+        // The programs are written by a simulation of the launch: the chunk items, rows in order of decreasing tail
+        // length, are dealt out one by one to the worker that will be free first; the worker that gets a row's last
+        // chunk also gets the row's tail, which ends its program, and frees a slot for the next worker of the grid
+        // when the tail is done.  The estimates (a chunk, a tail of a given size) only have to be roughly right: a
+        // tail that starts before its row's other chunks are in waits for them, a worker that is late delays nobody
+        // but its own items.
         //
         // The device's compute dies (XCDs, 32 CUs and one L2 each) take the workgroups of a grid in turn: workgroup i
-        // runs on die i mod n_xcd.  Row slot s is given to die s mod n_xcd and the order above is built per die, so
-        // that what a row's chunk workgroups write is in the L2 that its tail reads from.  Nothing depends on that
-        // placement for correctness.
-        const int n_xcd = std::max(1, ctx->cu_count / 32);
-        const int round = std::max(2, 2 * ctx->cu_count / n_xcd);
-        std::vector<std::vector<int32_t>> queue((size_t)n_xcd);
-        size_t longest = 0;
-        for (int x = 0; x < n_xcd; x++) {
-            std::vector<int32_t>& q = queue[(size_t)x];
-            auto push = [&](uint32_t item, int slot) {
-                const int32_t r = b->h_sel_list[(size_t)slot];
-                q.push_back((int32_t)item);
-                q.push_back(r);
-                q.push_back(b->h_rows[(size_t)r].scan_row);
-                q.push_back(b->h_rows[(size_t)r].sel);
-            };
-            const int n_mine = n_sel > x ? (n_sel - x + n_xcd - 1) / n_xcd : 0;  // slots x, x + n_xcd, ...
-            std::vector<int> ready_at((size_t)n_mine, 0);  // first position at which the row's tail may be placed
-            int next_tail = 0, row = 0, c = 0;
-            while (next_tail < n_mine) {
-                const int pos = (int)(q.size() / 4);
-                const int tail_slot = x + next_tail * n_xcd, row_slot = x + row * n_xcd;
-                if (next_tail < row && pos >= ready_at[(size_t)next_tail]) {
-                    push(0x80000000u | (uint32_t)tail_slot, tail_slot);
-                    next_tail++;
-                } else if (row < n_mine) {
-                    push(((uint32_t)c << 24) | (uint32_t)row_slot, row_slot);
-                    if (++c == chunks) {
-                        ready_at[(size_t)row] = (pos / round + 1) * round + round / 2;
-                        c = 0;
-                        row++;
-                    }
+        // runs on die i mod n_xcd.  Row slot s is given to die s mod n_xcd, and only workers of that die get its items,
+        // so that what a row's chunks write is in the L2 that its tail reads from.  Nothing depends on that placement
+        // for correctness.  A batch of few rows deals its items out to all dies instead.
+        const int n_xcd = std::min(SR_TK_MAX_XCD, std::max(1, ctx->cu_count / 32));
+        const int resident = 2 * std::max(ctx->cu_count, n_xcd);
+        const int total_items = n_sel * chunks;
+        const bool spread = n_sel < 2 * n_xcd;
+        const int n_pool = spread ? 1 : n_xcd;        // pools of workers that share a list of items
+        const int per_pool = resident / n_pool;         // resident workers of a pool
+        const double t_item = epv == 8 ? 6.0 : 9.0;     // microseconds: one chunk, streamed under the loads of the next
+        auto t_tail = [](const SrRow& d) { return d.sel <= 1 ? 8.0 : 11.0 + 0.0105 * (double)(d.sel + d.edit_cnt); };
+        struct Worker { double free_at; int id; };
+        auto later = [](const Worker& p, const Worker& q) { return p.free_at > q.free_at || (p.free_at == q.free_at && p.id > q.id); };
+        std::vector<std::vector<int32_t>> prog_items;   // per worker: indices into `entries`
+        std::vector<int32_t> prog_tail;
+        std::vector<int32_t> entries;                    // 4 ints per item, in list order
+        std::vector<std::vector<Worker>> heap((size_t)n_pool);
+        std::vector<std::vector<double>> slot_free((size_t)n_pool);  // when the slots of ended workers fall free
+        // worker ids: pool p owns the grid positions p, p + n_pool, ... (= die p when every die is a pool)
+        std::vector<int> next_id((size_t)n_pool);
+        auto new_worker = [&](int p, double at) {
+            const int id = next_id[(size_t)p];
+            next_id[(size_t)p] += n_pool;
+            if ((size_t)id >= prog_items.size()) { prog_items.resize((size_t)id + 1); prog_tail.resize((size_t)id + 1, -1); }
+            heap[(size_t)p].push_back(Worker{at, id});
+            std::push_heap(heap[(size_t)p].begin(), heap[(size_t)p].end(), later);
+        };
+        for (int p = 0; p < n_pool; p++) {
+            next_id[(size_t)p] = p;
+            const int n_first = std::min(per_pool, (total_items + n_pool - 1) / n_pool);
+            for (int w = 0; w < n_first; w++) new_worker(p, 0.0);
+        }
+        for (int slot = 0; slot < n_sel; slot++) {
+            const int32_t r = b->h_sel_list[(size_t)slot];
+            const SrRow& d = b->h_rows[(size_t)r];
+            const int p = spread ? 0 : slot % n_xcd;
+            for (int c = 0; c < chunks; c++) {
+                std::vector<Worker>& h = heap[(size_t)p];
+                if (h.empty()) {  // every worker of the pool has ended with a tail: the next one takes over its slot
+                    std::vector<double>& sf = slot_free[(size_t)p];
+                    std::sort(sf.begin(), sf.end());
+                    new_worker(p, sf.empty() ? 0.0 : sf.front());
+                    if (!sf.empty()) sf.erase(sf.begin());
+                }
+                std::pop_heap(h.begin(), h.end(), later);
+                Worker w = h.back();
+                h.pop_back();
+                prog_items[(size_t)w.id].push_back((int32_t)(entries.size() / 4));
+                entries.push_back((int32_t)(((uint32_t)c << 24) | (uint32_t)slot));
+                entries.push_back(r);
+                entries.push_back(d.scan_row);
+                entries.push_back(d.sel);
+                w.free_at += t_item;
+                if (c == chunks - 1) {
+                    prog_tail[(size_t)w.id] = slot;
+                    slot_free[(size_t)p].push_back(w.free_at + t_tail(d));
                 } else {
-                    push(0x80000000u | (uint32_t)tail_slot, tail_slot);  // nothing left to overlap with
-                    next_tail++;
+                    h.push_back(w);
+                    std::push_heap(h.begin(), h.end(), later);
                 }
             }
-            longest = std::max(longest, q.size() / 4);
         }
-        // interleave the dies' queues; a die with fewer rows gets entries that end at once
+        // the programs, each worker's items contiguous
+        const int n_workers = (int)prog_items.size();
         std::vector<int32_t>& sched = b->h_sched;
-        sched.assign(longest * (size_t)n_xcd * 4, -1);
-        for (int x = 0; x < n_xcd; x++)
-            for (size_t i = 0; i < queue[(size_t)x].size() / 4; i++)
-                for (int w = 0; w < 4; w++) sched[(i * (size_t)n_xcd + (size_t)x) * 4 + (size_t)w] = queue[(size_t)x][i * 4 + (size_t)w];
-        b->sched_len = (int32_t)(longest * (size_t)n_xcd);
+        sched.assign((size_t)n_workers * 4 + (size_t)total_items * 4, 0);
+        int32_t* progs = sched.data();
+        int32_t* items = sched.data() + (size_t)n_workers * 4;
+        int32_t at = 0;
+        for (int w = 0; w < n_workers; w++) {
+            progs[w * 4 + 0] = at;
+            progs[w * 4 + 1] = (int32_t)prog_items[(size_t)w].size();
+            progs[w * 4 + 2] = prog_tail[(size_t)w];
+            progs[w * 4 + 3] = 0;
+            for (int32_t e : prog_items[(size_t)w]) {
+                std::copy(entries.begin() + (size_t)e * 4, entries.begin() + (size_t)e * 4 + 4, items + (size_t)at * 4);
+                at++;
+            }
+        }
+        b->n_workers = n_workers;
+        b->n_items = total_items;
         SR_HIP(ctx, b->d_sched.reserve(sched.size() * sizeof(int32_t), st));
         SR_HIP(ctx, batch_copy(b, staged, b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), st));
     }
@@ -716,14 +757,23 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         topk_geometry(b->vocab, dtype, n_sel, ctx->cu_count, &a.chunks, &a.chunk_vecs);
         if (a.chunks > SR_TK_MAX_CHUNKS)
             return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_sample_launch: vocabulary too large for the selection kernel");
-        a.sched = b->d_sched.as<int4>();
-        a.n_wgs = b->sched_len;
+        a.progs = b->d_sched.as<int4>();
+        a.items = b->d_sched.as<int4>() + b->n_workers;
+        a.n_workers = b->n_workers;
+        a.n_items = b->n_items;
+        a.sel_list = b->d_sel_list.as<int32_t>();
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));
         SR_HIP(ctx, ctx->gmax.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
         SR_HIP(ctx, ctx->gmax2.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * 4 * sizeof(float), st));
         SR_HIP(ctx, ctx->gpos.reserve((size_t)n_sel * a.chunks * SR_TK_THREADS * sizeof(uint32_t), st));
         SR_HIP(ctx, ctx->gbound.reserve((size_t)n_sel * a.chunks * (SR_TK_THREADS / 64) * 2 * sizeof(uint32_t), st));
-        SR_HIP(ctx, ctx->row_done.reserve((size_t)std::max(n_sel, 1024) * sizeof(uint32_t), st, true));
+        // two sets of counters (see SrTopkArgs); a new allocation starts zeroed
+        if ((size_t)n_sel > ctx->done_cap || !ctx->row_done.p) {
+            const size_t cap = std::max((size_t)n_sel, (size_t)1024);
+            SR_HIP(ctx, ctx->row_done.reserve(2 * cap * sizeof(uint32_t), st, true));
+            ctx->done_cap = cap;
+            ctx->launch_no = 0;
+        }
         a.rows = b->d_rows.as<SrRow>();
         a.edits = b->d_edits.as<SrEdit>();
         a.mask = b->d_mask.as<uint32_t>();
@@ -736,6 +786,9 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.gpos = ctx->gpos.as<uint32_t>();
         a.gbound = ctx->gbound.as<uint32_t>();
         a.row_done = ctx->row_done.as<uint32_t>();
+        a.done_cap = (uint32_t)ctx->done_cap;
+        a.parity = (uint32_t)(ctx->launch_no++ & 1u);
+        a.spin_limit = ctx->spin_limit;
         a.uniforms = b->d_uniforms.as<double>();
         a.uniforms_per_row = b->upr;
         a.out_tokens = out_tokens_dev;
@@ -916,19 +969,30 @@ int sr_pack_allow_mask(const float* masked_logits, int32_t vocab, uint32_t* out_
     return SR_OK;
 }
 
-// Test hook (not part of the public header): how many sr_batch_append_tokens calls on this batch rebuilt it.
-SR_API int sr_debug_append_rebuilds(const sr_batch* b) { return b ? b->append_rebuilds : -1; }
+// ---- test and measurement hooks (include/stingray_sampler_test.h) ------------------------------------------
 
-// Test hook: phase timestamps (wall_clock64, 100 MHz) of the selection kernel go to prof_dev[grid][16].
-SR_API int sr_debug_set_profile(sr_ctx* ctx, unsigned long long* prof_dev)
+int sr_debug_append_rebuilds(const sr_batch* b) { return b ? b->append_rebuilds : -1; }
+
+int sr_debug_set_spin_limit(sr_ctx* ctx, uint32_t polls)
 {
     if (!ctx) return SR_ERR_NULL_ARGUMENT;
-    ctx->prof = prof_dev;
+    ctx->spin_limit = polls;
     return SR_OK;
 }
 
-// Test hook (not part of the public header): y[i] = the device expf for x[i], device pointers.
-SR_API int sr_selftest_expf(sr_ctx* ctx, const float* x_dev, float* y_dev, int64_t n)
+int sr_debug_set_profile(sr_ctx* ctx, unsigned long long* prof_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+#ifdef SR_PROFILE
+    ctx->prof = prof_dev;
+    return SR_OK;
+#else
+    (void)prof_dev;
+    return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_debug_set_profile: this library was built without -DSR_PROFILE");
+#endif
+}
+
+int sr_selftest_expf(sr_ctx* ctx, const float* x_dev, float* y_dev, int64_t n)
 {
     if (!ctx) return SR_ERR_NULL_ARGUMENT;
     SR_HIP(ctx, hipSetDevice(ctx->device));

@@ -24,6 +24,15 @@ __device__ __forceinline__ float sr_okey_inv(uint32_t k)
     return sr_u2f(b);
 }
 
+// The larger of two values that are not NaN, in one instruction (fmaxf first quiets a possible signalling NaN with
+// an instruction of its own).
+__device__ __forceinline__ float sr_max_f32(float a, float b)
+{
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 __device__ __forceinline__ float sr_bf16_to_f32(uint16_t h) { return sr_u2f(((uint32_t)h) << 16); }
 
 // glibc expf (2^(i/32) table, cubic in double, one rounding to float) with the FMA contractions of the

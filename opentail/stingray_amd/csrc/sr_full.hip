@@ -13,7 +13,11 @@
 
 namespace {
 
+#ifdef SR_PROFILE
 #define FPROF(a, slot_, i_) do { if ((a).prof && (slot_) == 0 && threadIdx.x == 0) (a).prof[(i_)] = (unsigned long long)wall_clock64(); } while (0)
+#else
+#define FPROF(a, slot_, i_) do { } while (0)
+#endif
 
 constexpr int kT = SR_SEQ_THREADS;
 constexpr int kW = SR_SEQ_WAVES;

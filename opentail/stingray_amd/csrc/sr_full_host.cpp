@@ -4,6 +4,7 @@
 #include <cstring>
 
 #include "sr_host.h"
+#include "../../../include/stingray_sampler_test.h"
 
 namespace {
 
@@ -471,8 +472,8 @@ int sr_mtp_verify_launch(sr_ctx* ctx, const float* logits_dev, int32_t rows, int
     return SR_OK;
 }
 
-// Test hook: exact left-to-right sum of x_dev[0..n) from s0; target = NaN disables the search.
-SR_API int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float s0, float target, float* out_sum_dev,
+// Test hook (include/stingray_sampler_test.h): exact left-to-right sum of x_dev[0..n) from s0
+int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float s0, float target, float* out_sum_dev,
                               int32_t* out_idx_dev)
 {
     if (!ctx) return SR_ERR_NULL_ARGUMENT;

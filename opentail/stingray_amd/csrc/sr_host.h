@@ -121,6 +121,11 @@ struct sr_ctx {
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
     int last_epv = 4;                    // vector width of the last launch: what an upload builds scan masks for
+    // selection kernel: entries per set of counters, launches so far (its parity picks the set), and how often a row
+    // tail polls its row's counter before it stops waiting and selects from the logits alone
+    size_t done_cap = 0;
+    unsigned launch_no = 0;
+    uint32_t spin_limit = 1u << 22;
 };
 
 struct sr_batch {
@@ -130,8 +135,9 @@ struct sr_batch {
     std::vector<SrEdit> h_edits;
     std::vector<int32_t> h_sel_list;   // rows on the selection kernel: TOPK and plain GREEDY
     std::vector<int32_t> h_full_list;  // rows on the full-vocabulary path
-    std::vector<int32_t> h_sched;     // the selection kernel's dispatch table (host copy, read by an async upload)
-    int32_t sched_len = 0;             // workgroups of the selection kernel's grid (entries of d_sched)
+    std::vector<int32_t> h_sched;     // the selection kernel's programs and chunk items (host copy, read by an async upload)
+    // the selection kernel's grid (see SrTopkArgs): workers (= programs at the head of d_sched) and chunk items
+    int32_t n_workers = 0, n_items = 0;
     std::vector<int32_t> h_wide_list;  // SampleTopK rows too wide for the selection kernel
     std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel
     std::vector<uint32_t> h_scan_need; // per batch row: SR_SCAN_* bits the row's scan mask must carry

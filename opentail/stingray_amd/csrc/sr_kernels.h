@@ -18,18 +18,22 @@
 // the row's edits are sorted by id (else they stand in order of first appearance in the history)
 #define SR_ROWFLAG_EDITS_SORTED (1u << 10)
 
+#define SR_TK_MAX_XCD 16
 struct SrTopkArgs {
     const void* logits;
     int64_t row_stride;      // elements
     int32_t vocab;
     int32_t dtype;           // 0 = f32, 1 = bf16
-    int32_t chunks;          // chunk workgroups per row
-    int32_t n_rows;          // rows in this launch: grid = n_rows * chunks chunk workgroups + n_rows tail workgroups
+    int32_t chunks;          // chunk items per row
+    int32_t n_rows;          // rows in this launch
     int32_t chunk_vecs;      // 16-byte vectors per chunk, a multiple of 64
-    // per workgroup in dispatch order: x = bit 31 row tail | bits 24..30 chunk | bits 0..23 launch slot of the row,
-    // y = batch row, z = scan-mask row, w = sel -- all a workgroup needs to find its data, in one 16-byte load
-    const int4* sched;
-    int32_t n_wgs;           // entries of sched = workgroups of the grid
+    // Workgroup b runs the program progs[b] = (first item, number of items, launch slot of the row it finishes at
+    // the end or -1, unused): it streams items[first .. first + n) in order.  An item is x = bits 24..30 chunk |
+    // bits 0..23 launch slot of the row, y = batch row, z = scan-mask row, w = sel.
+    const int4* items;
+    const int4* progs;
+    int32_t n_workers, n_items;
+    const int32_t* sel_list; // [n_rows] batch row of every launch slot
     const SrRow* rows;
     const SrEdit* edits;
     const uint32_t* mask;
@@ -42,12 +46,18 @@ struct SrTopkArgs {
     uint32_t* gbound;        // [n_rows][chunks][waves][2]: every chunk wave's share of the row's bound and its largest kept
                              // element (ordered keys)
     unsigned long long* cand; // [n_rows][SR_TK_ROW_CAP] (value bits << 32 | index), built by the row's tail
-    uint32_t* row_done;      // [n_rows], zero on entry, left zero on exit
+    // Counters, two sets of done_cap entries: a launch counts the chunks of slot s in row_done[parity * done_cap + s]
+    // and clears the other set for the launch after it, so that whatever a launch leaves behind never reaches a
+    // later one.
+    uint32_t* row_done;
+    uint32_t done_cap;
+    uint32_t parity;
+    uint32_t spin_limit;     // polls of a row's counter before its tail stops waiting and selects from the logits alone
     const double* uniforms;
     int32_t uniforms_per_row;
     int32_t* out_tokens;
     uint32_t* out_flags;     // may be null
-    unsigned long long* prof; // optional phase timestamps [grid][16] (test hook), normally null
+    unsigned long long* prof; // phase timestamps [chunk items + rows][16] in profiling builds, else unused
 };
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream);
 // Builds scan row i for descs[i]; base_addr / stride_bytes are those of the logits the mask is used with

@@ -1,15 +1,18 @@
 // Top-k-first sampling (the reference's SampleTopK, Sampler.cs:216-357) and the greedy rows.
 //
-// One launch, grid = rows x chunks chunk workgroups + one tail workgroup per row.  A chunk workgroup
-// loads one contiguous chunk of a row ONCE into registers (19 x 16 B per thread), applies the row's scan
-// mask, and leaves per lane and group of ~19 elements the largest element, its position and the second
-// largest, plus per wave a share of the row's bound.  Nothing is selected there: the workgroup streams.
+// One launch of persistent workgroups, each with a short list of chunks to stream and at most one row to finish.  A
+// chunk is a contiguous piece of a row that a workgroup holds in registers ONCE (19 x 16 B per thread); it applies
+// the row's scan mask and leaves, per lane and group of ~19 elements, the largest element, its position and the
+// second largest, plus per wave a share of the row's bound.  Nothing is selected there: the workgroup streams.
+// The worker that streams a row's last chunk then finishes the row (the row tail) and ends.
 //
 // The row tail derives a lower bound on the row's sel-th largest element from the waves' shares, takes the
 // largest element of every group whose second largest is below the bound directly, fetches the few groups
 // with more than one element above it again, and merges: penalties, pruning of candidates too small to
 // change any fp32 sum, an order by (value after penalties, value before, index), then the softmax / min-p /
-// top-p / draw arithmetic in the reference's sequential fp32 order.
+// top-p / draw arithmetic in the reference's sequential fp32 order.  A row whose candidates overflow the
+// tail's lists (thousands of equal logits at the cut), or whose chunks were not handed over in time, is selected
+// exactly from the logits themselves instead: every row gets its token in this launch.
 //
 // When the history penalties can only lower a logit (repetition >= 1, presence and frequency >= 0) the
 // scan skips the history ids (a per-row scan mask built when the batch is uploaded) and asks for the
@@ -24,7 +27,15 @@
 
 namespace {
 
-#define SR_PROF(a, slot_) do { if ((a).prof && threadIdx.x == 0) (a).prof[(size_t)blockIdx.x * 16 + (slot_)] = (unsigned long long)wall_clock64(); } while (0)
+// Phase timestamps exist in profiling builds only (-DSR_PROFILE); (a).prof then points at the 16 slots of the
+// unit (chunk item or row) at work.
+#ifdef SR_PROFILE
+#define SR_PROF(a, slot_) do { if ((a).prof && threadIdx.x == 0) (a).prof[(slot_)] = (unsigned long long)wall_clock64(); } while (0)
+#define SR_PROF_VAL(a, slot_, v_) do { if ((a).prof && threadIdx.x == 0) (a).prof[(slot_)] = (unsigned long long)(v_); } while (0)
+#else
+#define SR_PROF(a, slot_) do { } while (0)
+#define SR_PROF_VAL(a, slot_, v_) do { } while (0)
+#endif
 
 constexpr int kThreads = SR_TK_THREADS;
 constexpr int kWaves = kThreads / SR_WAVE;
@@ -391,11 +402,15 @@ __device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
 // slot = position of the row in this launch.
 template <int EPV, int kVec, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
-                                                float inv_temp, float* mx0_out, float* bscale_out, float* bound_out,
-                                                bool* binned, Early&& early, Late&& late, TopkSmem& sm);
+                                                bool force_exact, float inv_temp, float* mx0_out, float* bscale_out,
+                                                float* bound_out, bool* binned, Early&& early, Late&& late,
+                                                TopkSmem& sm);
 
+// force_exact: the chunk results of the row are not used, the candidates come from the logits themselves (what a row
+// whose candidates overflow the lists falls back to, and a row whose chunks were not handed over in time).
 template <int EPV, int kVec>
-__device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, TopkSmem& sm)
+__device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool force_exact,
+                                              TopkSmem& sm)
 {
     const int tid = threadIdx.x;
     const unsigned long long* cand = a.cand + (size_t)slot * kRowCap;
@@ -432,7 +447,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     bool binned = false;
     float mx0 = 0.0f, bscale0 = -56.0f, bound0 = 0.0f;
     const int n_c = build_candidates<EPV, kVec>(
-        a, slot, row, rd, want_bins, inv_temp, &mx0, &bscale0, &bound0, &binned,
+        a, slot, row, rd, want_bins, force_exact, inv_temp, &mx0, &bscale0, &bound0, &binned,
         [&]() SR_INL {
 #pragma unroll
             for (int r = 0; r < kHistRegs; r++) {
@@ -869,7 +884,8 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         // the first min(top_k, live) of the kept entries are the first of all live entries
         m2 = min(min(m2, max(rd.top_k, 0)), ms);
         sort_n = ms;
-        if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 13] = (unsigned long long)n_c; a.prof[(size_t)blockIdx.x * 16 + 14] = ((unsigned long long)n_live << 32) | (unsigned long long)ms; }
+        SR_PROF_VAL(a, 13, n_c);
+        SR_PROF_VAL(a, 14, ((unsigned long long)n_live << 32) | (unsigned long long)ms);
         if (by_bins) {
             // bins descend with the key, so an entry's rank is its bin's first position plus the entries of
             // the bin that precede it
@@ -1036,10 +1052,14 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 // the spot), and every candidate remembers its bin and its arrival number inside the bin (sm.probs, as integers):
 // the tail can then lay the candidates out bin by bin without another pass of atomics.  *binned tells whether
 // that happened (few chunks, a short enough list, a finite maximum); *mx0 is the maximum times inv_temp.
+// force_exact, and any row whose candidates overflow the lists: the row's sel-th largest kept element is found by a
+// radix select over the logits themselves, and the candidates are exactly the sel largest in (value desc, index asc)
+// order.  Slow (several passes over the row), exact for any data, and independent of the chunk results.
 template <int EPV, int kVec, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
-                                                float inv_temp, float* mx0_out, float* bscale_out, float* bound_out,
-                                                bool* binned, Early&& early, Late&& late, TopkSmem& sm)
+                                                bool force_exact, float inv_temp, float* mx0_out, float* bscale_out,
+                                                float* bound_out, bool* binned, Early&& early, Late&& late,
+                                                TopkSmem& sm)
 {
     *binned = false;
     *mx0_out = 0.0f;
@@ -1069,6 +1089,111 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         const int fv = c * a.chunk_vecs + (g + (int)(p / EPV) * SR_TK_GROUPS) * kThreads + tid;
         return fv * EPV + (int)(p % EPV) - mis;
     };
+    // wave-aggregated append to a list in LDS: one atomic per wave and call
+    auto wave_slot = [&](bool want, uint32_t* counter) SR_INL -> int {
+        const unsigned long long bal = __ballot(want);
+        if (bal == 0ull) return -1;
+        uint32_t base = 0u;
+        if (lane == (int)__ffsll((long long)bal) - 1) base = atomicAdd(counter, (uint32_t)__popcll(bal));
+        base = __shfl(base, (int)__ffsll((long long)bal) - 1);
+        return want ? (int)(base + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))) : -1;
+    };
+    auto append = [&](bool want, float x, int idx) SR_INL {
+        const int pos = wave_slot(want, &sm.bcast[12]);
+        if (pos >= 0) {
+            if (pos < kSelMax) {
+                sm.vals[pos] = x;
+                sm.idxs[pos] = idx;
+            } else if (pos < kRowCap) {
+                sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx);
+            }
+        }
+    };
+    // Of the kept elements equal to tx, the first need_eq by index join the candidates: a scan of the row in index
+    // order that stops as soon as it has them (equal values rank by ascending index, Sampler.cs:245-248).
+    auto take_ties = [&](float tx, int need_eq) SR_INL {
+        int emitted = 0;
+        for (int f_base = 0; f_base < nvt && emitted < need_eq; f_base += kThreads) {
+            const int fv = f_base + tid;
+            int ceq = 0;
+            bool is_eq[EPV];
+#pragma unroll
+            for (int q = 0; q < EPV; q++) is_eq[q] = false;
+            if (fv < nvt) {
+                const u32x4 v = wp[fv];
+                const int c = fv / a.chunk_vecs, fl = fv - c * a.chunk_vecs;
+                const uint32_t kb = keep_bits(c, fl / kThreads, fl % kThreads);
+#pragma unroll
+                for (int q = 0; q < EPV; q++) {
+                    is_eq[q] = VO::get(v, q) == tx && ((kb >> q) & 1u) != 0u;
+                    ceq += is_eq[q] ? 1 : 0;
+                }
+            }
+            int tile_total;
+            int rank = emitted + block_excl_scan(ceq, &tile_total, sm);
+#pragma unroll
+            for (int q = 0; q < EPV; q++) {
+                append(is_eq[q] && rank < need_eq, tx, fv * EPV + q - mis);
+                rank += is_eq[q] ? 1 : 0;
+            }
+            emitted += tile_total;
+        }
+    };
+    // The exact candidates of the row, from the logits alone.  Returns their number (at most sel).
+    auto exact_row = [&]() SR_INL -> int {
+        __syncthreads();
+        if (tid == 0) { sm.bcast[12] = 0u; sm.bcast[13] = 0u; }
+        // ordered key of every kept finite element, 0 for everything else
+        auto each_key = [&](auto&& body) SR_INL {
+            for (int f_base = 0; f_base < nvt; f_base += kThreads) {
+                const int fv = f_base + tid;
+                if (fv < nvt) {
+                    const u32x4 v = wp[fv];
+                    const int c = fv / a.chunk_vecs, fl = fv - c * a.chunk_vecs;
+                    const uint32_t kb = keep_bits(c, fl / kThreads, fl % kThreads);
+#pragma unroll
+                    for (int q = 0; q < EPV; q++) {
+                        const float x = VO::get(v, q);
+                        const bool ok = ((kb >> q) & 1u) != 0u && x == x && sr_f2u(x) != 0xff800000u;
+                        body(ok ? sr_okey(x) : 0u);
+                    }
+                }
+            }
+        };
+        // the sel-th largest key; 0 when the row has fewer than sel kept finite elements (all of them are taken)
+        const uint32_t tkey = block_radix_select(each_key, sel, sm);
+        __syncthreads();
+        for (int f_base = 0; f_base < nvt; f_base += kThreads) {
+            const int fv = f_base + tid;
+            u32x4 v = VO::neg_inf();
+            uint32_t kb = 0u;
+            if (fv < nvt) {
+                v = wp[fv];
+                const int c = fv / a.chunk_vecs, fl = fv - c * a.chunk_vecs;
+                kb = keep_bits(c, fl / kThreads, fl % kThreads);
+            }
+#pragma unroll
+            for (int q = 0; q < EPV; q++) {
+                const float x = VO::get(v, q);
+                const bool ok = ((kb >> q) & 1u) != 0u && x == x && sr_f2u(x) != 0xff800000u;
+                append(ok && sr_okey(x) > tkey, x, fv * EPV + q - mis);
+            }
+        }
+        __syncthreads();
+        const int n_gt = (int)sm.bcast[12];  // fewer than sel
+        if (tkey != 0u) take_ties(sr_okey_inv(tkey), sel - n_gt);
+        sr_drain_stores();
+        __syncthreads();
+        const int n = (int)sm.bcast[12];
+        __syncthreads();
+        return n;
+    };
+    if (force_exact) {
+        early();
+        late();
+        if (sel > kSelMax || sel < 1) return -1;
+        return exact_row();
+    }
     if (sel == 1) {
         // one candidate: the row's largest kept element, the first by index among equals -- the largest group
         // maximum, and of the groups that reach it the lowest position of their (first) largest element
@@ -1120,15 +1245,6 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
             if (c < S) f(c, gmr[c]);
         for (int c = kGmRegs; c < S; c++) f(c, gm_load(c));
     };
-    // wave-aggregated append to a list in LDS: one atomic per wave and call
-    auto wave_slot = [&](bool want, uint32_t* counter) SR_INL -> int {
-        const unsigned long long bal = __ballot(want);
-        if (bal == 0ull) return -1;
-        uint32_t base = 0u;
-        if (lane == (int)__ffsll((long long)bal) - 1) base = atomicAdd(counter, (uint32_t)__popcll(bal));
-        base = __shfl(base, (int)__ffsll((long long)bal) - 1);
-        return want ? (int)(base + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0u))) : -1;
-    };
     bool bins = false;
     float mx0 = 0.0f, bscale = -56.0f;
     uint32_t* meta = (uint32_t*)sm.probs;
@@ -1159,17 +1275,6 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         uint32_t base = 0u;
         if (total > 0 && lane == 0) base = atomicAdd(counter, (uint32_t)total);
         return (uint32_t)__builtin_amdgcn_readfirstlane((int)base) + (uint32_t)(incl - n_own);
-    };
-    auto append = [&](bool want, float x, int idx) SR_INL {
-        const int pos = wave_slot(want, &sm.bcast[12]);
-        if (pos >= 0) {
-            if (pos < kSelMax) {
-                sm.vals[pos] = x;
-                sm.idxs[pos] = idx;
-            } else if (pos < kRowCap) {
-                sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx);
-            }
-        }
     };
     auto list_group = [&](bool want, int c, int g) SR_INL {
         const int pos = wave_slot(want, &sm.bcast[13]);
@@ -1364,229 +1469,246 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         gather(nq, [&](float x) { return x > tx; });
         __syncthreads();
         const int n_gt = (int)sm.bcast[12];
-        const int need_eq = sel - n_gt;
-        int emitted = 0;
-        for (int f_base = 0; f_base < nvt && emitted < need_eq; f_base += kThreads) {
-            const int fv = f_base + tid;
-            int ceq = 0;
-            bool is_eq[EPV];
-#pragma unroll
-            for (int q = 0; q < EPV; q++) is_eq[q] = false;
-            if (fv < nvt) {
-                const u32x4 v = wp[fv];
-                const int c = fv / a.chunk_vecs, fl = fv - c * a.chunk_vecs;
-                const uint32_t kb = keep_bits(c, fl / kThreads, fl % kThreads);
-#pragma unroll
-                for (int q = 0; q < EPV; q++) {
-                    is_eq[q] = VO::get(v, q) == tx && ((kb >> q) & 1u) != 0u;
-                    ceq += is_eq[q] ? 1 : 0;
-                }
-            }
-            int tile_total;
-            int rank = emitted + block_excl_scan(ceq, &tile_total, sm);
-#pragma unroll
-            for (int q = 0; q < EPV; q++) {
-                append(is_eq[q] && rank < need_eq, tx, fv * EPV + q - mis);
-                rank += is_eq[q] ? 1 : 0;
-            }
-            emitted += tile_total;
-        }
+        take_ties(tx, sel - n_gt);
     }
     sr_drain_stores();
     __syncthreads();
     const uint32_t n_c = sm.bcast[12];
     __syncthreads();
+    if (n_c > (uint32_t)kRowCap) return exact_row();  // more candidates than the lists hold: the exact way
     *binned = bins && listed && n_c <= (uint32_t)kSelMax;
     *mx0_out = mx0;
     *bscale_out = bscale;
     *bound_out = tval;
-    return n_c > (uint32_t)kRowCap ? -1 : (int)n_c;
+    return (int)n_c;
 }
 
 // ---- the kernel --------------------------------------------------------------------------------------
+// Every workgroup is a worker with a short program that the host wrote when the batch was uploaded: a list of chunk
+// items, and possibly one row to finish at the end (the row tail) -- the row whose last chunk closes the list.  The
+// host deals the items out in order of decreasing tail length to whichever worker will be free first by its
+// estimate, so the rows with the longest tails are streamed first and finished while the others are still
+// streaming; a worker ends with its tail, and a worker of a grid larger than the device holds starts when one ends.
+// The row's other chunks were dealt out just before the last one, to workers that are running: the wait for them is
+// short and bounded, and a worker that waits is never waited for.
+//
+// A chunk is kVec 16-byte vectors per thread, each read once into registers and folded into the thread's four
+// groups.  When a vector has been folded, the load of the same vector of the worker's NEXT chunk is issued into its
+// registers, so every thread has up to kVec loads in flight from its first chunk to its last, and the stores, the
+// per-wave bound and the hand-off of a chunk run under the loads of the next one.
 template <int EPV, int kVec>
 __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 {
     __shared__ TopkSmem sm;
     using VO = VecOps<EPV>;
+    constexpr int ES = (EPV == 4) ? 4 : 2;  // element size in bytes
     const int tid = threadIdx.x, lane = sr_lane();
-    const int S = a.chunks;
-    // The host lays the workgroups out in dispatch order: chunk workgroups row by row, and the tail of a row
-    // about a round and a half of resident workgroups after the row's last chunk, so that a tail is dispatched
-    // after all chunk workgroups of its row (it waits, bounded, only on work that is already running) and
-    // rarely waits.  The entry is read through the constant address space (the host wrote it before the
-    // launch): one scalar 16-byte load.
+    const int S = a.chunks, V = a.vocab;
+    // programs and items are read through the constant address space (the host wrote them before the launch): one
+    // scalar 16-byte load each
     typedef int __attribute__((ext_vector_type(4))) i32x4;
     typedef const i32x4 __attribute__((address_space(4))) const_i32x4;
-    const i32x4 info = ((const_i32x4*)(uintptr_t)a.sched)[blockIdx.x];  // (item, row, scan-mask row, sel)
-    const uint32_t item = (uint32_t)info.x;
-    if (item == 0xffffffffu) return;  // padding entry
-    const bool is_tail = (item >> 31) != 0u;
-    const int slot_ = (int)(item & 0xffffffu), c_ = (int)((item >> 24) & 0x7fu);
-    if (is_tail) {
-        const int tslot = slot_;
-        // the row's descriptor does not depend on the chunks: fetched before the wait
-        const int trow = info.y;
-        SR_PROF(a, 0);
-        const SrRow trd = a.rows[trow];
-        if (tid == 0) {
-            uint32_t ok = 0u;
-            for (int it = 0; it < (1 << 22); it++) {
-                if (sr_load_agent(&a.row_done[tslot]) == (uint32_t)S) { ok = 1u; break; }
-                __builtin_amdgcn_s_sleep(4);
-            }
-            // the chunks' results were written through to L2: drop what this CU's L1 may hold of an earlier launch
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-            sr_store_agent(&a.row_done[tslot], 0u);  // ready for the next launch
-            sm.bcast[7] = ok;
-        }
-        __syncthreads();
-        if (!sm.bcast[7]) {
-            if (tid == 0) {
-                a.out_tokens[trow] = -1;
-                if (a.out_flags) a.out_flags[trow] = SR_KFLAG_UNSUPPORTED;
-            }
-            return;
-        }
-        SR_PROF(a, 4);
-        __builtin_amdgcn_s_setprio(3);  // the tail is the longer dependent chain: its waves go first
-        topk_row_tail<EPV, kVec>(a, tslot, trow, trd, sm);
-        SR_PROF(a, 15);
-        return;
+    const i32x4 prog = ((const const_i32x4*)(uintptr_t)a.progs)[blockIdx.x];  // (first item, items, row slot to finish or -1, -)
+    const const_i32x4* q = (const const_i32x4*)(uintptr_t)a.items + prog.x;
+    const int n_items = prog.y;
+    // this launch's counters: chunks counted in per row slot; the other set is cleared for the launch after this one,
+    // so that nothing a launch leaves behind reaches a later one
+    uint32_t* done = a.row_done + (size_t)a.parity * a.done_cap;
+    {
+        uint32_t* other = a.row_done + (size_t)(a.parity ^ 1u) * a.done_cap;
+        for (uint32_t e = blockIdx.x * kThreads + (uint32_t)tid; e < a.done_cap; e += gridDim.x * kThreads)
+            sr_store_agent(&other[e], 0u);
     }
-    const int slot = slot_, c = c_;
-    const int row = info.y;
-    const int V = a.vocab;
-    // phase timestamps stay in registers until the end: a store ahead of the scan-mask loads would keep the
-    // compiler from using scalar loads for them
-    unsigned long long pt0 = 0, pt1 = 0, pt2 = 0;
-    if (a.prof) pt0 = wall_clock64();
+    // Where an item's data lies.  The row is read as 16-byte vectors from the aligned address at or below its
+    // start: window element p is row element p - mis; chunks are whole multiples of 64 vectors of that window.
+    // Every load of a chunk is unconditional: a vector past the chunk's end (the last chunk of a row is ragged, and
+    // a row that starts late in its first vector may leave a chunk empty) is read from the last vector that exists
+    // instead -- the first vector of the row for an empty chunk -- and its keep-bits, all zero, turn it into -inf.
+    struct Geom {
+        const u32x4* cp;  // first vector of the chunk (of the row, for an empty chunk)
+        int last;         // index of the last vector that exists, relative to cp
+        int slot, c, sel, scan_row;
+    };
+    auto geom = [&](const i32x4& inf) SR_INL -> Geom {
+        Geom g;
+        g.slot = inf.x & 0xffffff;
+        g.c = (inf.x >> 24) & 0x7f;
+        g.sel = inf.w;
+        g.scan_row = inf.z;
+        const char* rowp = (const char*)a.logits + (size_t)inf.y * (size_t)a.row_stride * ES;
+        const int mis = (int)(((uintptr_t)rowp & 15u) / ES);
+        const int nvt = (V + mis + EPV - 1) / EPV;  // vectors of the row window
+        const int f0 = g.c * a.chunk_vecs;          // first vector of this chunk
+        const int nv = min(a.chunk_vecs, nvt - f0);  // vectors of this chunk that exist
+        g.cp = (const u32x4*)(rowp - (size_t)mis * ES) + (nv > 0 ? f0 : 0);
+        g.last = max(nv - 1, 0);
+        return g;
+    };
+    auto keep_words = [&](const Geom& g) SR_INL -> const uint32_t* {
+        return a.scan_mask + (size_t)g.scan_row * (size_t)a.scan_stride + ((size_t)g.c * kThreads + tid) * SR_TK_MASK_WORDS;
+    };
+    auto load_vec = [&](const Geom& g, int j) SR_INL -> u32x4 {
+        const uint32_t off = (uint32_t)min(j * kThreads + tid, g.last) * 16u;
+        return __builtin_nontemporal_load((const u32x4*)((const char*)g.cp + off));
+    };
 
-    // The row is read as 16-byte vectors from the aligned address at or below its start: window element
-    // p is row element p - mis.  Chunks are whole multiples of 64 vectors of that window.
-    constexpr int ES = (EPV == 4) ? 4 : 2;  // element size in bytes
-    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
-    const int mis = (int)(((uintptr_t)rowp & 15u) / ES);
-    const int nvt = (V + mis + EPV - 1) / EPV;        // vectors of the row window
-    const int f0 = c * a.chunk_vecs;                   // first vector of this chunk
-    const int nv = min(a.chunk_vecs, nvt - f0);        // vectors of this chunk
-
-    if (nv > 0) {
-        const u32x4* cp = (const u32x4*)(rowp - (size_t)mis * ES) + f0;
-        const uint32_t* mw = a.scan_mask + (size_t)info.z * (size_t)a.scan_stride + ((size_t)c * kThreads + tid) * SR_TK_MASK_WORDS;
-        const uint32_t kw0 = mw[0], kw1 = mw[1], kw2 = mw[2];
-        // the chunk as fp32 in registers (the upcast of bf16 is exact)
-        float xv[kVec * EPV];
+    if (n_items > 0) {
+        const i32x4 info = q[0];  // (chunk | launch slot of the row, batch row, scan-mask row, sel)
+        Geom cur = geom(info);
+        // The scan mask holds one keep-bit per window element in this kernel's access order: the thread's own three
+        // words, bit j * EPV + q = element q of its j-th vector.  They carry the row's edges, its allow-mask and, when
+        // the row tail fetches them, its history ids: two operations per element replace all of that logic.
+        uint32_t kw0, kw1, kw2;
         {
-            u32x4 t[kVec];
+            const uint32_t* mw = keep_words(cur);
+            kw0 = mw[0]; kw1 = mw[1]; kw2 = mw[2];
+        }
+        // A thread has kWin of its vectors in flight or in registers at a time: enough, over all workers, to keep the
+        // memory busy, and no more -- what is in flight beyond that only queues, and the row tails' few loads queue
+        // behind it.  Vector j passes through register slot j mod kWin; a chunk counts as kVecP vectors, a multiple
+        // of kWin, the ones past kVec being neither loaded nor folded.
+        constexpr int kWin = SR_TK_WINDOW < kVec ? SR_TK_WINDOW : kVec;
+        constexpr int kVecP = (kVec + kWin - 1) / kWin * kWin;
+        u32x4 t[kWin];
 #pragma unroll
-            for (int j = 0; j < kVec; j++) {
-                const int f = j * kThreads + tid;
-                t[j] = (f < nv) ? __builtin_nontemporal_load(&cp[f]) : VO::neg_inf();
+        for (int j = 0; j < kWin; j++) t[j] = load_vec(cur, j);
+
+        // One chunk per turn.  Behind the worker's last chunk the registers are refilled from that chunk's first
+        // vector, to no effect (one line, already in cache), so that the loop body is the same for every chunk: with
+        // two bodies, or a condition around the loads, the compiler keeps the incoming vectors in registers of their
+        // own and spills.
+        for (int k = 0; k < n_items; k++) {
+            const bool has_next = k + 1 < n_items;
+            Geom nxt = cur;
+            if (has_next) {
+                const i32x4 ninfo = q[k + 1];
+                nxt = geom(ninfo);
+            } else {
+                nxt.last = 0;
             }
-            // unpack in load order, one vector at a time, so that a packed vector's registers are free again
-            // before the next one is widened
+#ifdef SR_PROFILE
+            SrTopkArgs ap = a;
+            if (a.prof) ap.prof = a.prof + ((size_t)prog.x + (size_t)k) * 16;
+            SR_PROF(ap, 0);
+#endif
+            // Every lane owns four interleaved groups of vectors (j mod 4).  Of each group the row tail gets the
+            // largest element with its position inside the group, and the second largest: a group whose second
+            // largest is below the row's bound contributes its largest element directly and is never read again.
+            float gm1[SR_TK_GROUPS], gm2[SR_TK_GROUPS];
+            int gp1[SR_TK_GROUPS];
 #pragma unroll
-            for (int j = 0; j < kVec; j++) {
+            for (int g = 0; g < SR_TK_GROUPS; g++) { gm1[g] = SR_NEG_INF; gm2[g] = SR_NEG_INF; gp1[g] = 0; }
+#pragma unroll
+            for (int j = 0; j < kVecP; j++) {
+                const int g = j % SR_TK_GROUPS;
+                const int slot = j % kWin;
+                if (j < kVec) {
+#pragma unroll
+                    for (int e = 0; e < EPV; e++) {
+                        const int bit = j * EPV + e;
+                        const uint32_t wd = bit < 32 ? kw0 : bit < 64 ? kw1 : kw2;
+                        const uint32_t keep = (uint32_t)((int)(wd << (31 - (bit & 31))) >> 31);  // all ones = keep
+                        const float xe = sr_u2f((sr_f2u(VO::get(t[slot], e)) & keep) | (0xff800000u & ~keep));
+                        gp1[g] = xe > gm1[g] ? (j / SR_TK_GROUPS) * EPV + e : gp1[g];  // strict: the first of equal values stays
+                        gm2[g] = __builtin_amdgcn_fmed3f(gm1[g], gm2[g], xe);  // gm2 <= gm1: the median is the new second largest
+                        gm1[g] = sr_max_f32(gm1[g], xe);
+                    }
+                }
+                // The slot is free: the vector kWin places down the stream goes there -- of this chunk, or of the next.
+                // The empty statement pins the order (the group's results exist before it, the load is issued after
+                // it) and the scheduling barrier keeps the next vector's arithmetic behind this one's: left to itself
+                // the compiler issues the loads first, into registers of their own.
+                if (j + kWin < kVec) {
+                    asm volatile("" : "+v"(gm1[g]), "+v"(gm2[g]), "+v"(gp1[g]) : : "memory");
+                    t[slot] = load_vec(cur, j + kWin);
+                } else if (j + kWin >= kVecP) {
+                    asm volatile("" : "+v"(gm1[g]), "+v"(gm2[g]), "+v"(gp1[g]) : : "memory");
+                    t[slot] = load_vec(nxt, j + kWin - kVecP);
+                }
                 __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int q = 0; q < EPV; q++) xv[j * EPV + q] = VO::get(t[j], q);
             }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // The scan mask holds one keep-bit per window element in this kernel's access order: the thread's own
-        // three words (loaded ahead of the data), bit j * EPV + q = element q of its j-th vector.  They carry the
-        // row's edges, its allow-mask and, when the row tail fetches them, its history ids: two operations per
-        // element replace all per-element edge, allow-mask and history logic.
-        // A wave all of whose elements are kept (no edge, no allow-mask, no history id among them) skips them.
-        constexpr int kBits = kVec * EPV;
-        static_assert(kBits > 64 && kBits <= 96, "three keep-words per thread");
-        constexpr uint32_t kLast = kBits == 96 ? 0xffffffffu : ((1u << (kBits - 64)) - 1u);
-        const bool all_kept = (kw0 & kw1) == 0xffffffffu && (kw2 & kLast) == kLast;
-        if (__ballot(!all_kept) != 0ull) {
-#pragma unroll
-            for (int j = 0; j < kVec; j++)
-#pragma unroll
-                for (int q = 0; q < EPV; q++) {
-                    const int bit = j * EPV + q;
-                    const uint32_t w = bit < 32 ? kw0 : bit < 64 ? kw1 : kw2;
-                    const uint32_t t = (uint32_t)((int)(w << (31 - (bit & 31))) >> 31);  // all ones = keep
-                    xv[j * EPV + q] = sr_u2f((sr_f2u(xv[j * EPV + q]) & t) | (0xff800000u & ~t));
-                }
-        }
-        if (a.prof) pt1 = wall_clock64();
-
-        // Every lane owns four interleaved groups of vectors (j mod 4).  Of each group the row tail gets the largest
-        // element with its position inside the group, and the second largest: a group whose second largest is below
-        // the row's bound contributes its largest element directly and is never read again.
-        float gm1[SR_TK_GROUPS], gm2[SR_TK_GROUPS];
-        uint32_t gpk = 0u;
-#pragma unroll
-        for (int g = 0; g < SR_TK_GROUPS; g++) {
-            float m1 = SR_NEG_INF, m2 = SR_NEG_INF;
-            int p1 = 0;
-#pragma unroll
-            for (int j = g; j < kVec; j += SR_TK_GROUPS)
-#pragma unroll
-                for (int q = 0; q < EPV; q++) {
-                    const float x = xv[j * EPV + q];
-                    p1 = x > m1 ? (j / SR_TK_GROUPS) * EPV + q : p1;  // strict: the first of equal values stays
-                    m2 = __builtin_amdgcn_fmed3f(m1, m2, x);  // m2 <= m1: the median of the three is the new second largest
-                    m1 = fmaxf(m1, x);
-                }
-            gm1[g] = m1;
-            gm2[g] = m2;
-            gpk |= (uint32_t)p1 << (8 * g);
-        }
-        if (a.prof) pt2 = wall_clock64();
-        const size_t go = ((size_t)slot * S + c) * kThreads + tid;
-        float4* gout = a.gmax + go;
-        sr_store_agent_f4(gout, gm1[0], gm1[1], gm1[2], gm1[3]);
-        sr_store_agent_f4(a.gmax2 + go, gm2[0], gm2[1], gm2[2], gm2[3]);
-        __hip_atomic_store(a.gpos + go, gpk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // The wave's share of the row's bound: a value, to 16 bits and rounded down, with at least
-        // ceil(sel / (chunks x 8)) of the wave's 256 group maxima at or above it (found bit by bit with ballots).
-        // The smallest of all the row's waves' values then has at least sel group maxima at or above it.
-        __builtin_amdgcn_sched_barrier(0);  // after the stores: the chunk's registers are free by now
-        {
-            const int need = (info.w + S * kWaves - 1) / (S * kWaves);
-            uint32_t K = 0u;
+#ifdef SR_PROFILE
+            SR_PROF(ap, 1);
+#endif
+            // the next chunk's keep-words arrive under the stores and the bound loop
+            {
+                const uint32_t* mw = keep_words(nxt);
+                kw0 = mw[0]; kw1 = mw[1]; kw2 = mw[2];
+            }
+            const uint32_t gpk = (uint32_t)gp1[0] | ((uint32_t)gp1[1] << 8) | ((uint32_t)gp1[2] << 16) | ((uint32_t)gp1[3] << 24);
+            const size_t go = ((size_t)cur.slot * S + cur.c) * kThreads + tid;
+            sr_store_agent_f4(a.gmax + go, gm1[0], gm1[1], gm1[2], gm1[3]);
+            sr_store_agent_f4(a.gmax2 + go, gm2[0], gm2[1], gm2[2], gm2[3]);
+            __hip_atomic_store(a.gpos + go, gpk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // The wave's share of the row's bound: a value, to 16 bits and rounded down, with at least
+            // ceil(sel / (chunks x 8)) of the wave's 256 group maxima at or above it (found bit by bit with ballots).
+            // The smallest of all the row's waves' values then has at least sel group maxima at or above it.
+            {
+                const int need = (cur.sel + S * kWaves - 1) / (S * kWaves);
+                uint32_t K = 0u;
 #pragma unroll 1
-            for (int bit = 31; bit >= 16; bit--) {
-                const uint32_t cnd = K | (1u << bit);
-                const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
-                const int cge = __popcll(__ballot(gm1[0] >= fc)) + __popcll(__ballot(gm1[1] >= fc)) +
-                                __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc));
-                if (cge >= need) K = cnd;
+                for (int bit = 31; bit >= 16; bit--) {
+                    const uint32_t cnd = K | (1u << bit);
+                    const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
+                    const int cge = __popcll(__ballot(gm1[0] >= fc)) + __popcll(__ballot(gm1[1] >= fc)) +
+                                    __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc));
+                    if (cge >= need) K = cnd;
+                }
+                // ... and the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
+                const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(gm1[0], gm1[1]), fmaxf(gm1[2], gm1[3]))));
+                if (lane == 0) {
+                    uint32_t* gb = a.gbound + (((size_t)cur.slot * S + cur.c) * kWaves + (tid >> 6)) * 2;
+                    __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(gb + 1, wmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
-            // ... and the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
-            const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(gm1[0], gm1[1]), fmaxf(gm1[2], gm1[3]))));
-            if (lane == 0) {
-                uint32_t* gb = a.gbound + (((size_t)slot * S + c) * kWaves + (tid >> 6)) * 2;
-                __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(gb + 1, wmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-    } else {
-        float4* gout = a.gmax + ((size_t)slot * S + c) * kThreads + tid;
-        sr_store_agent_f4(gout, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
-        sr_store_agent_f4(a.gmax2 + ((size_t)slot * S + c) * kThreads + tid, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
-        __hip_atomic_store(a.gpos + ((size_t)slot * S + c) * kThreads + tid, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (lane == 0) {
-            uint32_t* gb = a.gbound + (((size_t)slot * S + c) * kWaves + (tid >> 6)) * 2;
-            __hip_atomic_store(gb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(gb + 1, kKeyNegInf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#ifdef SR_PROFILE
+            SR_PROF(ap, 2);
+            SR_PROF_VAL(ap, 13, cur.sel);
+            SR_PROF_VAL(ap, 14, cur.slot);
+#endif
+            // hand the chunk over: this wave's write-through stores (and, older than them, the loads of the next
+            // chunk) have completed, the workgroup meets, then the chunk is counted in
+            sr_drain_stores();
+            __syncthreads();
+            if (tid == 0) __hip_atomic_fetch_add(&done[cur.slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#ifdef SR_PROFILE
+            SR_PROF(ap, 5);
+#endif
+            cur = nxt;
         }
     }
-    SR_PROF(a, 3);
-    if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 0] = pt0; a.prof[(size_t)blockIdx.x * 16 + 1] = pt1; a.prof[(size_t)blockIdx.x * 16 + 2] = pt2; }
-    if (a.prof && tid == 0) { a.prof[(size_t)blockIdx.x * 16 + 13] = (unsigned long long)a.rows[row].sel; a.prof[(size_t)blockIdx.x * 16 + 14] = (unsigned long long)slot; }
+    if (prog.z < 0) return;
 
-    // hand the chunk over: drain this wave's write-through stores, meet, then count the chunk in
-    sr_drain_stores();
+    // ---- the row tail
+    const int tslot = prog.z;
+    const int trow = a.sel_list[tslot];
+    const SrRow trd = a.rows[trow];
+#ifdef SR_PROFILE
+    SrTopkArgs ap = a;
+    if (a.prof) ap.prof = a.prof + ((size_t)a.n_items + (size_t)tslot) * 16;
+    SR_PROF(ap, 0);
+#else
+    const SrTopkArgs& ap = a;
+#endif
+    // The row's other chunks are in the hands of workers that are running; they are nearly always in already.
+    // Should they not come (the wait is bounded), the row is selected from its logits alone.
+    if (tid == 0) {
+        uint32_t ok = 0u;
+        for (uint32_t it = 0; it < a.spin_limit; it++) {
+            if (sr_load_agent(&done[tslot]) == (uint32_t)S) { ok = 1u; break; }
+            __builtin_amdgcn_s_sleep(2);
+        }
+        // the chunks' results were written through to L2: drop what this CU's L1 may hold of an earlier launch
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        sm.bcast[7] = ok;
+    }
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_add(&a.row_done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    SR_PROF(a, 5);
+    const bool handed_over = sm.bcast[7] != 0u;
+    SR_PROF(ap, 4);
+    __builtin_amdgcn_s_setprio(3);  // the tail is the longer dependent chain: its waves go first
+    topk_row_tail<EPV, kVec>(ap, tslot, trow, trd, !handed_over, sm);
+    SR_PROF(ap, 15);
 }
 
 // ---- scan mask ---------------------------------------------------------------------------------------
@@ -1701,7 +1823,7 @@ hipError_t sr_launch_apply_patches(SrRow* rows, const SrRowPatch* rp, int n_rowp
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
 {
     if (n_rows <= 0) return hipSuccess;
-    dim3 grid((unsigned)a.n_wgs), block(kThreads);  // chunk workgroups + one tail per row (+ padding entries)
+    dim3 grid((unsigned)a.n_workers), block(kThreads);
     if (a.dtype == 1)
         hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16>), grid, block, 0, stream, a);
     else

@@ -13,6 +13,18 @@ def _declared_symbols():
     return sorted(set(re.findall(r"SR_API\s+[\w\s\*]+?\b(sr_\w+)\s*\(", text)))
 
 
+def _test_hook_symbols():
+    text = open(os.path.join(ROOT, "include", "stingray_sampler_test.h")).read()
+    return sorted(set(re.findall(r"SR_API\s+[\w\s\*]+?\b(sr_\w+)\s*\(", text)))
+
+
+def test_the_test_hooks_are_declared_apart_from_the_product_interface_and_exported():
+    hooks = _test_hook_symbols()
+    assert hooks and not set(hooks) & set(_declared_symbols())
+    lib = ctypes.CDLL(sa.lib_path())
+    assert not [s for s in hooks if not hasattr(lib, s)]
+
+
 def test_header_and_python_symbol_lists_agree():
     assert _declared_symbols() == sorted(sa.EXPORTED_SYMBOLS)
 
