@@ -383,14 +383,16 @@ class SamplerContext:
         t = toks.cpu().numpy()
         return (t, flags.cpu().numpy().view(np.uint32)) if return_flags else t
 
-    def argmax_rows(self, logits):
-        """(int Token, float Logit)[] per row -- BatchForwardMultiArgmax's result shape."""
+    def argmax_rows(self, logits, out=None):
+        """(int Token, float Logit)[] per row -- BatchForwardMultiArgmax's result shape.  out=(idx, val) device
+        tensors to write into."""
         import torch
 
         rows, vocab = logits.shape
-        idx = torch.empty(rows, dtype=torch.int32, device=logits.device)
-        val = torch.empty(rows, dtype=torch.float32, device=logits.device)
-        self._check(self.L.sr_argmax_rows_launch(
+        idx, val = out if out is not None else (torch.empty(rows, dtype=torch.int32, device=logits.device),
+                                                torch.empty(rows, dtype=torch.float32, device=logits.device))
+        fn = self.L.sr_argmax_rows_launch
+        self._check(fn(
             self.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), rows, vocab,
             self._row_stride(logits) if rows > 0 and vocab > 0 else vocab, C.c_void_p(idx.data_ptr()), C.c_void_p(val.data_ptr())))
         self.synchronize()

@@ -233,7 +233,7 @@ void sr_destroy(sr_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
-    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best,
+    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best, &ctx->argmax_done,
                          &ctx->work, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs};
@@ -896,32 +896,47 @@ int sr_sample_batch(sr_ctx* ctx, const void* logits, int dtype, int logits_on_de
     return SR_OK;
 }
 
-int sr_argmax_rows_launch(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows, int32_t vocab,
-                          int64_t row_stride_elems, int32_t* out_idx_dev, float* out_val_dev)
+static int argmax_check(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows, int32_t vocab, int64_t row_stride_elems,
+                        const int32_t* out_idx_dev)
 {
-    if (!ctx) return SR_ERR_NULL_ARGUMENT;
-    if (rows == 0) return SR_OK;
     if (!out_idx_dev || (!logits_dev && vocab > 0)) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_argmax_rows: null tensor");
     if (rows < 0 || vocab < 0 || (vocab > 0 && row_stride_elems < vocab))
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_argmax_rows: bad shape");
     if (dtype != SR_DTYPE_F32 && dtype != SR_DTYPE_BF16)
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_argmax_rows: unknown dtype");
-    SR_HIP(ctx, hipSetDevice(ctx->device));
-    SR_HIP(ctx, ctx->argmax_best.reserve((size_t)rows * sizeof(unsigned long long), ctx->stream));
+    return SR_OK;
+}
+
+static SrArgmaxArgs argmax_args(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows, int32_t vocab,
+                                int64_t row_stride_elems, int32_t* out_idx_dev, float* out_val_dev)
+{
     SrArgmaxArgs a{};
     a.logits = logits_dev;
     a.row_stride = row_stride_elems;
     a.vocab = vocab;
     a.dtype = dtype;
     a.rows = rows;
-    int s = std::max(1, std::min((4 * ctx->cu_count + rows - 1) / rows, std::max(1, vocab / 4096)));
-    a.chunk_len = (vocab + s - 1) / s;
-    if (a.chunk_len < 1) a.chunk_len = 1;
-    a.chunks = vocab > 0 ? (vocab + a.chunk_len - 1) / a.chunk_len : 1;
-    a.best = ctx->argmax_best.as<unsigned long long>();
     a.out_idx = out_idx_dev;
     a.out_val = out_val_dev;
-    SR_HIP(ctx, sr_launch_argmax_rows(a, ctx->stream));
+    sr_argmax_plan(a, ctx->cu_count);
+    return a;
+}
+
+int sr_argmax_rows_launch(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows, int32_t vocab,
+                          int64_t row_stride_elems, int32_t* out_idx_dev, float* out_val_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0) return SR_OK;
+    int rc = argmax_check(ctx, logits_dev, dtype, rows, vocab, row_stride_elems, out_idx_dev);
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    // slots and counters: zero when allocated, and every launch leaves them zero again
+    SR_HIP(ctx, ctx->argmax_best.reserve((size_t)rows * sizeof(unsigned long long), ctx->stream, true));
+    SR_HIP(ctx, ctx->argmax_done.reserve((size_t)rows * sizeof(uint32_t), ctx->stream, true));
+    SrArgmaxArgs a = argmax_args(ctx, logits_dev, dtype, rows, vocab, row_stride_elems, out_idx_dev, out_val_dev);
+    a.best = ctx->argmax_best.as<unsigned long long>();
+    a.done = ctx->argmax_done.as<uint32_t>();
+    SR_HIP(ctx, sr_launch_argmax_rows(a, false, ctx->stream));
     return SR_OK;
 }
 

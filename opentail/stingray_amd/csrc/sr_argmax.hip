@@ -2,62 +2,99 @@
 // the reference's llm_argmax_rows (CudaTextKernels.cs:465-479).  Lowest index wins on equal values; a NaN
 // element wins outright (first NaN), as TensorPrimitives.IndexOfMax documents.
 //
-// grid = rows x chunks; each workgroup reduces one chunk to a packed (key << 32 | ~index) and folds it
-// into the row's slot with a 64-bit atomic max, so no second pass is needed.
+// One launch, grid = rows x chunks.  A workgroup streams its chunk with 16-byte non-temporal loads (eight in
+// flight per thread), reduces it to a packed (key << 32 | ~index) and, when the row has more than one chunk,
+// folds that into the row's slot with a 64-bit atomic max and counts itself in; the workgroup that counts in
+// last writes the row's result and puts slot and counter back to zero, so the scratch of one launch is ready
+// for the next without a fill.  Rows of one chunk write their result directly.
+#include <algorithm>
+
 #include "sr_device.cuh"
 #include "sr_kernels.h"
+#include "sr_types.h"
 
 namespace {
 constexpr int kThreads = 256;
+constexpr int kUnroll = 8;
 
-__global__ void k_fill_u64(unsigned long long* p, int n, unsigned long long v)
+typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
+
+__global__ void k_fill_u32(uint32_t* p, int n, uint32_t v)
 {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
 }
 
-template <int ES>
-__device__ __forceinline__ float load_elem(const char* p, int64_t i)
+template <int ES> __device__ __forceinline__ float load_elem(const char* p, int64_t i)
 {
     if (ES == 4) return ((const float*)p)[i];
     return sr_bf16_to_f32(((const uint16_t*)p)[i]);
 }
 
-template <int ES>
-__global__ __launch_bounds__(kThreads) void k_argmax_chunks(SrArgmaxArgs a)
+__device__ __forceinline__ void fold(unsigned long long& best, float v, uint32_t i)
 {
-    __shared__ unsigned long long s_best[kThreads / SR_WAVE];
-    const int row = blockIdx.x / a.chunks, c = blockIdx.x - row * a.chunks;
-    const int lo = c * a.chunk_len, hi = min(a.vocab, lo + a.chunk_len);
-    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
-    unsigned long long best = 0ull;
-    for (int i = lo + (int)threadIdx.x; i < hi; i += kThreads) {
-        float v = load_elem<ES>(rowp, i);
-        uint32_t k = (v != v) ? 0xffffffffu : sr_okey(v);
-        unsigned long long e = ((unsigned long long)k << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
-        best = e > best ? e : best;
-    }
-    best = sr_wave_max_u64(best);
-    if (sr_lane() == 0) s_best[sr_wave_id()] = best;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < kThreads / SR_WAVE; w++) best = s_best[w] > best ? s_best[w] : best;
-        if (best) atomicMax(&a.best[row], best);
+    const uint32_t k = (v != v) ? 0xffffffffu : sr_okey(v);
+    const unsigned long long e = ((unsigned long long)k << 32) | (unsigned long long)(0xffffffffu - i);
+    best = e > best ? e : best;
+}
+
+template <int ES> __device__ __forceinline__ void fold_vec(unsigned long long& best, const u32x4 t, uint32_t first)
+{
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        if (ES == 4) {
+            fold(best, sr_u2f(t[w]), first + w);
+        } else {
+            fold(best, sr_u2f(t[w] << 16), first + 2 * w);
+            fold(best, sr_u2f(t[w] & 0xffff0000u), first + 2 * w + 1);
+        }
     }
 }
 
-template <int ES>
-__global__ void k_argmax_finish(SrArgmaxArgs a)
+// kVec: the rows start on 16-byte boundaries and chunk_len is a multiple of the elements of a vector
+template <int ES, bool kVec> __global__ __launch_bounds__(kThreads) void k_argmax_rows(SrArgmaxArgs a)
 {
-    int row = blockIdx.x * blockDim.x + threadIdx.x;
-    if (row >= a.rows) return;
-    unsigned long long e = a.best[row];
-    int idx = e ? (int)(0xffffffffu - (uint32_t)(e & 0xffffffffull)) : 0;  // empty row -> 0
-    a.out_idx[row] = idx;
-    if (a.out_val) {
-        const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
-        a.out_val[row] = a.vocab > 0 ? load_elem<ES>(rowp, idx) : 0.0f;  // the original bits, not a decode
+    __shared__ unsigned long long s_best[kThreads / SR_WAVE];
+    constexpr int EPV = 16 / ES;
+    const int row = __builtin_amdgcn_readfirstlane((int)(blockIdx.x / (unsigned)a.chunks));
+    const int c = (int)blockIdx.x - row * a.chunks;
+    const int lo = c * a.chunk_len, hi = min(a.vocab, lo + a.chunk_len);
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+    const int tid = (int)threadIdx.x;
+    unsigned long long best = 0ull;
+    int scalar_from = lo;
+    if (kVec) {
+        const u32x4* vp = (const u32x4*)rowp;
+        const int v_lo = lo / EPV, v_hi = hi / EPV;  // whole vectors; only the row's last chunk can leave elements over
+        int i = v_lo + tid;
+        for (; i + (kUnroll - 1) * kThreads < v_hi; i += kUnroll * kThreads) {
+            u32x4 t[kUnroll];
+#pragma unroll
+            for (int j = 0; j < kUnroll; j++) t[j] = __builtin_nontemporal_load(vp + i + j * kThreads);
+#pragma unroll
+            for (int j = 0; j < kUnroll; j++) fold_vec<ES>(best, t[j], (uint32_t)(i + j * kThreads) * EPV);
+        }
+        for (; i < v_hi; i += kThreads) fold_vec<ES>(best, __builtin_nontemporal_load(vp + i), (uint32_t)i * EPV);
+        scalar_from = max(lo, v_hi * EPV);
     }
+    for (int i = scalar_from + tid; i < hi; i += kThreads) fold(best, load_elem<ES>(rowp, i), (uint32_t)i);
+
+    best = sr_wave_max_u64(best);
+    if (sr_lane() == 0) s_best[sr_wave_id()] = best;
+    __syncthreads();
+    if (tid != 0) return;
+    for (int w = 1; w < kThreads / SR_WAVE; w++) best = s_best[w] > best ? s_best[w] : best;
+    if (a.chunks > 1) {
+        if (best) __hip_atomic_fetch_max(&a.best[row], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t before = __hip_atomic_fetch_add(&a.done[row], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (before != (uint32_t)a.chunks - 1u) return;
+        best = __hip_atomic_load(&a.best[row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&a.best[row], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&a.done[row], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const int idx = best ? (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull)) : 0;  // empty row -> 0
+    a.out_idx[row] = idx;
+    if (a.out_val) a.out_val[row] = a.vocab > 0 ? load_elem<ES>(rowp, idx) : 0.0f;  // the original bits, not a decode
 }
 
 __global__ void k_selftest_expf(const float* x, float* y, int64_t n)
@@ -67,17 +104,35 @@ __global__ void k_selftest_expf(const float* x, float* y, int64_t n)
 }
 }  // namespace
 
-hipError_t sr_launch_argmax_rows(const SrArgmaxArgs& a, hipStream_t stream)
+void sr_argmax_plan(SrArgmaxArgs& a, int cu_count)
+{
+    const int es = a.dtype == 1 ? 2 : 4, epv = 16 / es;
+    a.vec = ((uintptr_t)a.logits % 16 == 0 && ((size_t)a.row_stride * es) % 16 == 0) ? 1 : 0;
+    // enough workgroups for eight per compute unit, none with less than one unrolled pass of work
+    const int per_pass = kThreads * kUnroll * epv;
+    int s = std::max(1, std::min((8 * cu_count + a.rows - 1) / std::max(a.rows, 1), a.vocab / per_pass));
+    int len = (a.vocab + s - 1) / s;
+    len = (len + epv - 1) / epv * epv;
+    a.chunk_len = std::max(len, epv);
+    a.chunks = a.vocab > 0 ? (a.vocab + a.chunk_len - 1) / a.chunk_len : 1;
+}
+
+hipError_t sr_launch_argmax_rows(const SrArgmaxArgs& a, bool clear_first, hipStream_t stream)
 {
     if (a.rows <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_fill_u64, dim3((a.rows + 255) / 256), dim3(256), 0, stream, a.best, a.rows, 0ull);
-    if (a.vocab > 0) {
-        dim3 grid((unsigned)(a.rows * a.chunks));
-        if (a.dtype == 1) hipLaunchKernelGGL(k_argmax_chunks<2>, grid, dim3(kThreads), 0, stream, a);
-        else hipLaunchKernelGGL(k_argmax_chunks<4>, grid, dim3(kThreads), 0, stream, a);
+    if (clear_first && a.chunks > 1) {
+        // best and done are separate arrays: clear each where it is
+        hipLaunchKernelGGL(k_fill_u32, dim3((2 * a.rows + 255) / 256), dim3(256), 0, stream, (uint32_t*)a.best, 2 * a.rows, 0u);
+        hipLaunchKernelGGL(k_fill_u32, dim3((a.rows + 255) / 256), dim3(256), 0, stream, a.done, a.rows, 0u);
     }
-    if (a.dtype == 1) hipLaunchKernelGGL(k_argmax_finish<2>, dim3((a.rows + 255) / 256), dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL(k_argmax_finish<4>, dim3((a.rows + 255) / 256), dim3(256), 0, stream, a);
+    const dim3 grid((unsigned)a.rows * (unsigned)a.chunks), block(kThreads);
+    if (a.dtype == 1) {
+        if (a.vec) hipLaunchKernelGGL((k_argmax_rows<2, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((k_argmax_rows<2, false>), grid, block, 0, stream, a);
+    } else {
+        if (a.vec) hipLaunchKernelGGL((k_argmax_rows<4, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((k_argmax_rows<4, false>), grid, block, 0, stream, a);
+    }
     return hipGetLastError();
 }
 

@@ -107,7 +107,7 @@ struct sr_ctx {
     std::string err;
     int cu_count = 256;
     // scratch, lazily grown and reused across calls
-    DeviceBuf cand, gmax, gmax2, gpos, gbound, row_done, argmax_best;
+    DeviceBuf cand, gmax, gmax2, gpos, gbound, row_done, argmax_best, argmax_done;
     DeviceBuf work;          // fp32 rows of the full-vocabulary path
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits

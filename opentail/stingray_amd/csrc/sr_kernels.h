@@ -82,13 +82,20 @@ struct SrArgmaxArgs {
     int32_t vocab;
     int32_t dtype;
     int32_t rows;
-    int32_t chunks;
-    int32_t chunk_len;
-    unsigned long long* best; // [rows] packed (key << 32 | ~idx), zeroed by the launcher
+    int32_t chunks;           // workgroups per row
+    int32_t chunk_len;        // elements per chunk, a multiple of the elements of a 16-byte vector
+    int32_t vec;              // rows start on 16-byte boundaries: 16-byte loads
+    // rows of more than one chunk: [rows] packed (key << 32 | ~idx) and [rows] chunks counted in; both zero before
+    // the launch and zero again after it
+    unsigned long long* best;
+    uint32_t* done;
     int32_t* out_idx;
     float* out_val;           // may be null
 };
-hipError_t sr_launch_argmax_rows(const SrArgmaxArgs& a, hipStream_t stream);
+// fills chunks, chunk_len and vec from the other fields
+void sr_argmax_plan(SrArgmaxArgs& a, int cu_count);
+// clear_first: best and done may hold anything (a fill precedes the kernel)
+hipError_t sr_launch_argmax_rows(const SrArgmaxArgs& a, bool clear_first, hipStream_t stream);
 
 hipError_t sr_launch_selftest_expf(const float* x, float* y, int64_t n, hipStream_t stream);
 
