@@ -204,6 +204,19 @@ SR_API int sr_sample_batch(sr_ctx* ctx, const void* logits, int dtype, int logit
 SR_API int sr_argmax_rows_launch(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows,
                                  int32_t vocab, int64_t row_stride_elems,
                                  int32_t* out_idx_dev, float* out_val_dev);
+/*
+ * sr_argmax_rows_launch for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, results
+ * and errors; it calls no hipMalloc/hipFree: the per-row slots and counters that rows split over several
+ * workgroups need lie in a fixed array inside the library's code object (192 KiB per GPU, held until the
+ * process ends), whose part for this call a small fill kernel clears first.  At most SR_ARGMAX_NOALLOC_MAX_ROWS
+ * rows per call (SR_ERR_INVALID_ARGUMENT beyond).  All contexts of one GPU share the array: two calls that
+ * overlap on one GPU (different streams, different contexts) race; order them on one stream.
+ */
+#define SR_ARGMAX_NOALLOC_MAX_ROWS 16384
+SR_API int sr_argmax_rows_launch_noalloc(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows,
+                                         int32_t vocab, int64_t row_stride_elems,
+                                         int32_t* out_idx_dev, float* out_val_dev);
 /* Host-result form: (int Token, float Logit)[] as BatchForwardMultiArgmax returns it. */
 SR_API int sr_argmax_rows(sr_ctx* ctx, const void* logits, int dtype, int logits_on_device,
                           int32_t rows, int32_t vocab, int64_t row_stride_elems,

@@ -49,7 +49,8 @@ EXPORTED_SYMBOLS = [
     "sr_create", "sr_destroy", "sr_bind_thread", "sr_set_stream", "sr_synchronize", "sr_last_error",
     "sr_version", "sr_batch_create", "sr_batch_destroy", "sr_batch_upload", "sr_batch_set_uniforms",
     "sr_batch_append_tokens",
-    "sr_sample_launch", "sr_resample_rows_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows",
+    "sr_sample_launch", "sr_resample_rows_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows_launch_noalloc",
+    "sr_argmax_rows",
     "sr_build_distribution_launch", "sr_sample_with_distribution_launch", "sr_sample_from_probs_launch",
     "sr_resample_residual_launch", "sr_spec_verify_launch", "sr_mtp_verify_launch", "sr_pack_allow_mask",
     "sr_build_distribution", "sr_sample_with_distribution", "sr_sample_from_probs", "sr_resample_residual",
@@ -155,6 +156,7 @@ def load_library():
     L.sr_sample_batch.argtypes = [vp, vp, C.c_int, C.c_int, i32, i32, i64, rpp, i32p, i32p, i32p, f32p, i32p,
                                   u32p, i64, C.POINTER(C.c_uint8), f64p, i32p, u32p]
     L.sr_argmax_rows_launch.argtypes = [vp, vp, C.c_int, i32, i32, i64, vp, vp]
+    L.sr_argmax_rows_launch_noalloc.argtypes = [vp, vp, C.c_int, i32, i32, i64, vp, vp]
     L.sr_argmax_rows.argtypes = [vp, vp, C.c_int, C.c_int, i32, i32, i64, i32p, f32p]
     L.sr_build_distribution_launch.argtypes = [vp, vp, vp, C.c_int, i64, vp, i64, i32]
     L.sr_sample_with_distribution_launch.argtypes = [vp, vp, vp, C.c_int, i64, vp, i64, i32, vp]
@@ -383,15 +385,15 @@ class SamplerContext:
         t = toks.cpu().numpy()
         return (t, flags.cpu().numpy().view(np.uint32)) if return_flags else t
 
-    def argmax_rows(self, logits, out=None):
+    def argmax_rows(self, logits, out=None, noalloc=False):
         """(int Token, float Logit)[] per row -- BatchForwardMultiArgmax's result shape.  out=(idx, val) device
-        tensors to write into."""
+        tensors to write into; noalloc=True goes through the entry point that allocates no device memory."""
         import torch
 
         rows, vocab = logits.shape
         idx, val = out if out is not None else (torch.empty(rows, dtype=torch.int32, device=logits.device),
                                                 torch.empty(rows, dtype=torch.float32, device=logits.device))
-        fn = self.L.sr_argmax_rows_launch
+        fn = self.L.sr_argmax_rows_launch_noalloc if noalloc else self.L.sr_argmax_rows_launch
         self._check(fn(
             self.h, C.c_void_p(logits.data_ptr()), self._dtype_of(logits), rows, vocab,
             self._row_stride(logits) if rows > 0 and vocab > 0 else vocab, C.c_void_p(idx.data_ptr()), C.c_void_p(val.data_ptr())))

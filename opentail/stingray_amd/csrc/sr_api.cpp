@@ -223,6 +223,12 @@ int sr_create(int device_ordinal, sr_ctx** out)
         return SR_ERR_HIP;
     }
     ctx->stream = ctx->own_stream;
+    // where this device keeps its copy of the scratch that belongs to the library's code object
+    if (sr_argmax_static_scratch(device_ordinal, &ctx->static_best, &ctx->static_done) != hipSuccess) {
+        (void)hipStreamDestroy(ctx->own_stream);
+        delete ctx;
+        return SR_ERR_HIP;
+    }
     *out = ctx;
     return SR_OK;
 }
@@ -937,6 +943,29 @@ int sr_argmax_rows_launch(sr_ctx* ctx, const void* logits_dev, int dtype, int32_
     a.best = ctx->argmax_best.as<unsigned long long>();
     a.done = ctx->argmax_done.as<uint32_t>();
     SR_HIP(ctx, sr_launch_argmax_rows(a, false, ctx->stream));
+    return SR_OK;
+}
+
+static_assert(SR_ARGMAX_STATIC_ROWS == SR_ARGMAX_NOALLOC_MAX_ROWS, "the header states the size of the static scratch");
+
+int sr_argmax_rows_launch_noalloc(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows, int32_t vocab,
+                                  int64_t row_stride_elems, int32_t* out_idx_dev, float* out_val_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0) return SR_OK;
+    int rc = argmax_check(ctx, logits_dev, dtype, rows, vocab, row_stride_elems, out_idx_dev);
+    if (rc != SR_OK) return rc;
+    if (rows > SR_ARGMAX_STATIC_ROWS)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT,
+                       "sr_argmax_rows_launch_noalloc: " + std::to_string(rows) + " rows, the static scratch holds " +
+                           std::to_string(SR_ARGMAX_STATIC_ROWS) + " (use sr_argmax_rows_launch, or split the call)");
+    if (!ctx->static_best) return sr_fail(ctx, SR_ERR_HIP, "sr_argmax_rows_launch_noalloc: the static scratch was not found at sr_create");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    SrArgmaxArgs a = argmax_args(ctx, logits_dev, dtype, rows, vocab, row_stride_elems, out_idx_dev, out_val_dev);
+    a.best = ctx->static_best;
+    a.done = ctx->static_done;
+    // every caller on this device shares the array and it keeps what the last call left: clear the part this call uses
+    SR_HIP(ctx, sr_launch_argmax_rows(a, true, ctx->stream));
     return SR_OK;
 }
 

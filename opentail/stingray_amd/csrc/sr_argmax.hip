@@ -7,17 +7,27 @@
 // folds that into the row's slot with a 64-bit atomic max and counts itself in; the workgroup that counts in
 // last writes the row's result and puts slot and counter back to zero, so the scratch of one launch is ready
 // for the next without a fill.  Rows of one chunk write their result directly.
+//
+// This file also holds the scratch of the entry point that allocates nothing: a zero-initialised array in
+// device memory that belongs to the library's code object, one copy per GPU.
 #include <algorithm>
 
 #include "sr_device.cuh"
 #include "sr_kernels.h"
 #include "sr_types.h"
 
+// best[SR_ARGMAX_STATIC_ROWS] (8 bytes each) followed by done[SR_ARGMAX_STATIC_ROWS] (4 bytes each): 192 KiB.
+// In host code this name is only a handle for hipGetSymbolAddress, never an address to give a kernel.
+static __device__ __align__(256) unsigned long long scratch[SR_ARGMAX_STATIC_ROWS + SR_ARGMAX_STATIC_ROWS / 2];
+
 namespace {
 constexpr int kThreads = 256;
 constexpr int kUnroll = 8;
 
 typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // per device: where that device's copy of `scratch` lies
 
 __global__ void k_fill_u32(uint32_t* p, int n, uint32_t v)
 {
@@ -134,6 +144,22 @@ hipError_t sr_launch_argmax_rows(const SrArgmaxArgs& a, bool clear_first, hipStr
         else hipLaunchKernelGGL((k_argmax_rows<4, false>), grid, block, 0, stream, a);
     }
     return hipGetLastError();
+}
+
+// The address of the current device's copy of the static scratch, looked up once per device.
+hipError_t sr_argmax_static_scratch(int device, unsigned long long** best, uint32_t** done)
+{
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    void* p = __atomic_load_n(&g_scratch_ptr[device], __ATOMIC_ACQUIRE);
+    if (!p) {
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        __atomic_store_n(&g_scratch_ptr[device], p, __ATOMIC_RELEASE);
+    }
+    *best = (unsigned long long*)p;
+    *done = (uint32_t*)((unsigned long long*)p + SR_ARGMAX_STATIC_ROWS);
+    return hipSuccess;
 }
 
 hipError_t sr_launch_selftest_expf(const float* x, float* y, int64_t n, hipStream_t stream)

@@ -108,6 +108,9 @@ struct sr_ctx {
     int cu_count = 256;
     // scratch, lazily grown and reused across calls
     DeviceBuf cand, gmax, gmax2, gpos, gbound, row_done, argmax_best, argmax_done;
+    // this device's copy of the scratch inside the library's code object (looked up once, at sr_create)
+    unsigned long long* static_best = nullptr;
+    uint32_t* static_done = nullptr;
     DeviceBuf work;          // fp32 rows of the full-vocabulary path
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits

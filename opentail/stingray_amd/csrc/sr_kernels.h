@@ -96,6 +96,8 @@ struct SrArgmaxArgs {
 void sr_argmax_plan(SrArgmaxArgs& a, int cu_count);
 // clear_first: best and done may hold anything (a fill precedes the kernel)
 hipError_t sr_launch_argmax_rows(const SrArgmaxArgs& a, bool clear_first, hipStream_t stream);
+// the current device's copy of the scratch that belongs to the library's code object: SR_ARGMAX_STATIC_ROWS rows
+hipError_t sr_argmax_static_scratch(int device, unsigned long long** best, uint32_t** done);
 
 hipError_t sr_launch_selftest_expf(const float* x, float* y, int64_t n, hipStream_t stream);
 
