@@ -180,6 +180,7 @@ def main():
     ap.add_argument("--workload", default="c3_fp32_full")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget (0 = skip)")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--no-prime", action="store_true", help="skip the event warm-up (prime_events): for looking at it")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of one logits buffer (known size) so that a counter run\n"
                          "under rocprofv3 --pmc has a reference dispatch to scale FETCH_SIZE / WRITE_SIZE by")
@@ -201,7 +202,8 @@ def main():
     stream = torch.cuda.Stream()            # a real (non-null) stream shared by torch and the library,
     torch.cuda.set_stream(stream)           # so HIP events recorded here bracket the sampler's kernels
     ctx = SamplerContext(0)
-    prime_events(torch, stream)
+    if not args.no_prime:
+        prime_events(torch, stream)
     # no collector pauses inside the timed loops (as timeit does): a full collection of this process takes tens of
     # milliseconds, which is hundreds of steps
     import gc

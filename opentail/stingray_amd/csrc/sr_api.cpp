@@ -128,10 +128,29 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
             const int n_first = std::min(per_pool, (total_items + n_pool - 1) / n_pool);
             for (int w = 0; w < n_first; w++) new_worker(p, 0.0);
         }
+        // With a row or more per compute unit nothing is gained by spreading a row over workers (streaming alone
+        // already takes all the memory bandwidth, and tails that run beside it slow it down by more than they gain):
+        // every worker streams all chunks of one row and finishes it, waits for nobody and hands nothing over.
+        const bool affine = n_sel >= ctx->cu_count;
+        if (affine) {
+            prog_items.assign((size_t)n_sel, {});
+            prog_tail.assign((size_t)n_sel, -1);
+        }
         for (int slot = 0; slot < n_sel; slot++) {
             const int32_t r = b->h_sel_list[(size_t)slot];
             const SrRow& d = b->h_rows[(size_t)r];
             const int p = spread ? 0 : slot % n_xcd;
+            if (affine) {
+                for (int c = 0; c < chunks; c++) {
+                    prog_items[(size_t)slot].push_back((int32_t)(entries.size() / 4));
+                    entries.push_back((int32_t)(((uint32_t)c << 24) | (uint32_t)slot));
+                    entries.push_back(r);
+                    entries.push_back(d.scan_row);
+                    entries.push_back(d.sel);
+                }
+                prog_tail[(size_t)slot] = slot;
+                continue;
+            }
             for (int c = 0; c < chunks; c++) {
                 std::vector<Worker>& h = heap[(size_t)p];
                 if (h.empty()) {  // every worker of the pool has ended with a tail: the next one takes over its slot
@@ -169,7 +188,7 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
             progs[w * 4 + 0] = at;
             progs[w * 4 + 1] = (int32_t)prog_items[(size_t)w].size();
             progs[w * 4 + 2] = prog_tail[(size_t)w];
-            progs[w * 4 + 3] = 0;
+            progs[w * 4 + 3] = affine ? 1 : 0;
             for (int32_t e : prog_items[(size_t)w]) {
                 std::copy(entries.begin() + (size_t)e * 4, entries.begin() + (size_t)e * 4 + 4, items + (size_t)at * 4);
                 at++;
@@ -177,6 +196,7 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
         }
         b->n_workers = n_workers;
         b->n_items = total_items;
+        b->own_rows = affine;
         SR_HIP(ctx, b->d_sched.reserve(sched.size() * sizeof(int32_t), st));
         SR_HIP(ctx, batch_copy(b, staged, b->d_sched.p, sched.data(), sched.size() * sizeof(int32_t), st));
     }
@@ -766,6 +786,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.progs = b->d_sched.as<int4>();
         a.items = b->d_sched.as<int4>() + b->n_workers;
         a.n_workers = b->n_workers;
+        a.own_rows = b->own_rows ? 1 : 0;
         a.n_items = b->n_items;
         a.sel_list = b->d_sel_list.as<int32_t>();
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));

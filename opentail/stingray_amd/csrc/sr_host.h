@@ -141,6 +141,7 @@ struct sr_batch {
     std::vector<int32_t> h_sched;     // the selection kernel's programs and chunk items (host copy, read by an async upload)
     // the selection kernel's grid (see SrTopkArgs): workers (= programs at the head of d_sched) and chunk items
     int32_t n_workers = 0, n_items = 0;
+    bool own_rows = false;  // one worker per row
     std::vector<int32_t> h_wide_list;  // SampleTopK rows too wide for the selection kernel
     std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel
     std::vector<uint32_t> h_scan_need; // per batch row: SR_SCAN_* bits the row's scan mask must carry

@@ -28,11 +28,12 @@ struct SrTopkArgs {
     int32_t n_rows;          // rows in this launch
     int32_t chunk_vecs;      // 16-byte vectors per chunk, a multiple of 64
     // Workgroup b runs the program progs[b] = (first item, number of items, launch slot of the row it finishes at
-    // the end or -1, unused): it streams items[first .. first + n) in order.  An item is x = bits 24..30 chunk |
+    // the end or -1, 1 when its items are exactly that row's chunks): it streams items[first .. first + n) in order.  An item is x = bits 24..30 chunk |
     // bits 0..23 launch slot of the row, y = batch row, z = scan-mask row, w = sel.
     const int4* items;
     const int4* progs;
     int32_t n_workers, n_items;
+    int32_t own_rows;        // every worker's program is one whole row (all its chunks, then its tail)
     const int32_t* sel_list; // [n_rows] batch row of every launch slot
     const SrRow* rows;
     const SrEdit* edits;

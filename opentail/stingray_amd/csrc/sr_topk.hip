@@ -1496,7 +1496,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 // groups.  When a vector has been folded, the load of the same vector of the worker's NEXT chunk is issued into its
 // registers, so every thread has up to kVec loads in flight from its first chunk to its last, and the stores, the
 // per-wave bound and the hand-off of a chunk run under the loads of the next one.
-template <int EPV, int kVec>
+template <int EPV, int kVec, int kWindow>
 __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 {
     __shared__ TopkSmem sm;
@@ -1508,9 +1508,13 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
     // scalar 16-byte load each
     typedef int __attribute__((ext_vector_type(4))) i32x4;
     typedef const i32x4 __attribute__((address_space(4))) const_i32x4;
-    const i32x4 prog = ((const const_i32x4*)(uintptr_t)a.progs)[blockIdx.x];  // (first item, items, row slot to finish or -1, -)
+    // (first item, items, row slot to finish or -1, 1 = the items are all the chunks of that row and of no other)
+    const i32x4 prog = ((const const_i32x4*)(uintptr_t)a.progs)[blockIdx.x];
     const const_i32x4* q = (const const_i32x4*)(uintptr_t)a.items + prog.x;
     const int n_items = prog.y;
+    // A worker that streams all chunks of the one row it finishes hands nothing over: no other workgroup reads what
+    // its chunks leave, so the chunks are neither waited for one by one nor counted in.
+    const bool own_row = prog.w != 0;
     // this launch's counters: chunks counted in per row slot; the other set is cleared for the launch after this one,
     // so that nothing a launch leaves behind reaches a later one
     uint32_t* done = a.row_done + (size_t)a.parity * a.done_cap;
@@ -1567,7 +1571,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         // memory busy, and no more -- what is in flight beyond that only queues, and the row tails' few loads queue
         // behind it.  Vector j passes through register slot j mod kWin; a chunk counts as kVecP vectors, a multiple
         // of kWin, the ones past kVec being neither loaded nor folded.
-        constexpr int kWin = SR_TK_WINDOW < kVec ? SR_TK_WINDOW : kVec;
+        constexpr int kWin = kWindow < kVec ? kWindow : kVec;
         constexpr int kVecP = (kVec + kWin - 1) / kWin * kWin;
         u32x4 t[kWin];
 #pragma unroll
@@ -1669,9 +1673,11 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #endif
             // hand the chunk over: this wave's write-through stores (and, older than them, the loads of the next
             // chunk) have completed, the workgroup meets, then the chunk is counted in
-            sr_drain_stores();
-            __syncthreads();
-            if (tid == 0) __hip_atomic_fetch_add(&done[cur.slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (!own_row) {
+                sr_drain_stores();
+                __syncthreads();
+                if (tid == 0) __hip_atomic_fetch_add(&done[cur.slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
 #ifdef SR_PROFILE
             SR_PROF(ap, 5);
 #endif
@@ -1693,9 +1699,10 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #endif
     // The row's other chunks are in the hands of workers that are running; they are nearly always in already.
     // Should they not come (the wait is bounded), the row is selected from its logits alone.
+    if (own_row) sr_drain_stores();  // every wave's own stores; the barrier below joins them
     if (tid == 0) {
-        uint32_t ok = 0u;
-        for (uint32_t it = 0; it < a.spin_limit; it++) {
+        uint32_t ok = own_row && a.spin_limit != 0u ? 1u : 0u;
+        for (uint32_t it = 0; !own_row && it < a.spin_limit; it++) {
             if (sr_load_agent(&done[tslot]) == (uint32_t)S) { ok = 1u; break; }
             __builtin_amdgcn_s_sleep(2);
         }
@@ -1824,10 +1831,14 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
 {
     if (n_rows <= 0) return hipSuccess;
     dim3 grid((unsigned)a.n_workers), block(kThreads);
-    if (a.dtype == 1)
-        hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16>), grid, block, 0, stream, a);
-    else
-        hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC>), grid, block, 0, stream, a);
+    // workers with a row of their own are few per compute unit: each keeps more of its vectors in flight
+    if (a.dtype == 1) {
+        if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW_OWN>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW>), grid, block, 0, stream, a);
+    } else {
+        if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW_OWN>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW>), grid, block, 0, stream, a);
+    }
     return hipGetLastError();
 }
 
