@@ -6,6 +6,9 @@
 One "step" = one batched sampling call (sr_sample_launch / sr_spec_verify_launch) over a batch of
 seeded synthetic logits that are already resident in HBM.  Four distinct logits buffers are rotated so
 every step streams cold data (4 x 155.6 MB exceeds the 256 MB Infinity Cache).  Prints ONE JSON line.
+The default run times c3_fp32_full for K steps and then, in short windows of their own, the other
+configurations (c1, c2, c3_bf16, c4, c5): their figures are the "per_config" object of the same line.
+Every measured launch is checked against the CPU oracle outside the timed regions, every row of it.
 
 Workloads (opentail/stingray_amd/synthetic.py):
   c3_fp32_full  (default) batch 256 x vocab 151,936 fp32, heterogeneous top-k U{1..1000} / top-p / T,
@@ -87,7 +90,7 @@ def prime_events(torch, stream):
     e0.elapsed_time(e1)
 
 
-def bench_spec(args, w, ctx, stream):
+def bench_spec(args, w, ctx, stream) -> dict:
     """Speculative verification: target logits [rows, L+1, V], draft distributions [rows, L, V] and draft
     tokens resident; two distinct input sets are rotated (2 x 285 MB exceeds the Infinity Cache)."""
     import torch
@@ -134,7 +137,7 @@ def bench_spec(args, w, ctx, stream):
     acc_h, out_h = acc.cpu().numpy(), out.cpu().numpy()
     parity = None
     if not args.no_parity:
-        n_chk = 3
+        n_chk = rows
         tn, qn, kn = t[:n_chk].cpu().numpy(), q[:n_chk].cpu().numpy(), k[:n_chk].cpu().numpy()
         bad = 0
         for r in range(n_chk):
@@ -169,47 +172,17 @@ def bench_spec(args, w, ctx, stream):
                      "kernel": "k_full_row", "kernel_us": dev_us},
         "cpu_baseline": cpu, "parity": parity,
     }
-    print(json.dumps(out_j))
+    for _, _, _, b, _, _ in sets:
+        b.close()
+    return out_j
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=1000)
-    ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="c3_fp32_full")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget (0 = skip)")
-    ap.add_argument("--no-parity", action="store_true")
-    ap.add_argument("--no-prime", action="store_true", help="skip the event warm-up (prime_events): for looking at it")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run a plain device copy of one logits buffer (known size) so that a counter run\n"
-                         "under rocprofv3 --pmc has a reference dispatch to scale FETCH_SIZE / WRITE_SIZE by")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        raise SystemExit("bench.py: this build runs on one GPU (rows shard across GPUs without any exchange); "
-                         "run with --gpus 1")
-
+def run_workload(args, ctx, stream) -> dict:
+    """One workload (args.workload) for args.steps timed steps; the result as the dict that main() prints."""
     import torch
 
-    from opentail.stingray_amd import SamplerContext
-    from oracle import binding as orc  # checker + CPU baseline only
-
-    if not torch.cuda.is_available():
-        raise SystemExit("bench.py needs a GPU: the sampler has no CPU path")
-    torch.cuda.set_device(0)
     w = make_workload(args.workload)
     rows, vocab = w.rows, w.vocab
-    stream = torch.cuda.Stream()            # a real (non-null) stream shared by torch and the library,
-    torch.cuda.set_stream(stream)           # so HIP events recorded here bracket the sampler's kernels
-    ctx = SamplerContext(0)
-    if not args.no_prime:
-        prime_events(torch, stream)
-    # no collector pauses inside the timed loops (as timeit does): a full collection of this process takes tens of
-    # milliseconds, which is hundreds of steps
-    import gc
-    gc.collect()
-    gc.disable()
-
     if args.workload == "c5":
         return bench_spec(args, w, ctx, stream)
 
@@ -267,7 +240,8 @@ def main():
 
     # a decode step that also uploads its batch again (histories change every step): host packing + copies + launch
     step_with_upload_us = None
-    if args.workload.startswith("c3") and not os.environ.get("SR_BENCH_NO_UPLOAD_LEG"):
+    extra_legs = args.workload.startswith("c3") and not args.short and not os.environ.get("SR_BENCH_NO_UPLOAD_LEG")
+    if extra_legs:
         n_up = max(10, args.steps // 4)
         for i in range(3):
             batches[i % n_buf].reupload()
@@ -284,7 +258,7 @@ def main():
     # in for the sampled ones, so most are new to their history and every 16th step or so a row runs out of room and
     # the batch is rebuilt).  Batches and outputs of their own: the measured ones stay as they are for the parity check.
     step_with_append_us = None
-    if args.workload.startswith("c3") and not os.environ.get("SR_BENCH_NO_UPLOAD_LEG"):
+    if extra_legs:
         n_up = max(10, args.steps // 4)
         ab = [ctx.new_batch().upload(w.params, vocab, w.uniforms, w.allow_mask, w.mask_active) for _ in range(n_buf)]
         atok = torch.empty(rows, dtype=torch.int32, device="cuda")
@@ -309,7 +283,7 @@ def main():
     if not args.no_parity:
         from tests.helpers import oracle_tokens
 
-        n_chk = min(rows, 24)
+        n_chk = rows  # every row of the measured launch
         got = toks[0].cpu().numpy()[:n_chk]
         want = oracle_tokens(host_logits[0][:n_chk], w.params[:n_chk], np.asarray(w.uniforms)[:n_chk],
                              None if w.allow_mask is None else w.allow_mask[:n_chk],
@@ -353,7 +327,10 @@ def main():
         "config": {"workload": args.workload, "rows": rows, "vocab": vocab,
                    "chain": "penalties+top-k+top-p+min-p" if args.workload == "c3_fp32_full" else args.workload},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "frac_with_token_append": (None if step_with_append_us is None else
+                                                alg_bytes / (step_with_append_us * 1e-6) / 1e9 / HBM_PEAK_GBS),
+                     "traffic": traffic,
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "kernel": "k_topk_rows" if args.workload.startswith(("c1", "c3")) else "k_full_row",
                      "kernel_us": kern_us},
@@ -363,6 +340,74 @@ def main():
         "us_per_step_with_batch_upload": step_with_upload_us,
         "us_per_step_with_token_append": step_with_append_us,
     }
+    for b_ in batches:
+        b_.close()
+    return out
+
+
+# The other configurations of the benchmark, each for a short window of its own inside the default run:
+# (workload, timed steps, warm-up steps, seconds of CPU baseline)
+PER_CONFIG = [("c1", 400, 40, 1.5), ("c2", 60, 6, 1.5), ("c3_bf16", 200, 20, 1.5), ("c4", 30, 4, 1.5), ("c5", 20, 3, 1.5)]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--workload", default="c3_fp32_full")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget (0 = skip)")
+    ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--no-prime", action="store_true", help="skip the event warm-up (prime_events): for looking at it")
+    ap.add_argument("--no-per-config", action="store_true",
+                    help="the default workload alone, without the short windows of the other configurations")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain device copy of one logits buffer (known size) so that a counter run\n"
+                         "under rocprofv3 --pmc has a reference dispatch to scale FETCH_SIZE / WRITE_SIZE by")
+    args = ap.parse_args()
+    args.short = False
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on one GPU (rows shard across GPUs without any exchange); "
+                         "run with --gpus 1")
+
+    import torch
+
+    from opentail.stingray_amd import SamplerContext
+    from oracle import binding as orc  # noqa: F401  (checker + CPU baseline only; loaded before the timed regions)
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU: the sampler has no CPU path")
+    torch.cuda.set_device(0)
+    stream = torch.cuda.Stream()            # a real (non-null) stream shared by torch and the library,
+    torch.cuda.set_stream(stream)           # so HIP events recorded here bracket the sampler's kernels
+    ctx = SamplerContext(0)
+    if not args.no_prime:
+        prime_events(torch, stream)
+    # no collector pauses inside the timed loops (as timeit does): a full collection of this process takes tens of
+    # milliseconds, which is hundreds of steps
+    import gc
+    gc.collect()
+    gc.disable()
+
+    out = run_workload(args, ctx, stream)
+    if args.workload == "c3_fp32_full" and not args.no_per_config and not args.copy_probe:
+        per = {}
+        for name, steps, warmup, cpu_s in PER_CONFIG:
+            gc.collect()
+            torch.cuda.empty_cache()
+            sub = argparse.Namespace(**vars(args))
+            sub.workload, sub.steps, sub.warmup, sub.short = name, steps, warmup, True
+            sub.cpu_seconds = min(cpu_s, args.cpu_seconds)
+            r = run_workload(sub, ctx, stream)
+            per[name] = {
+                "us_per_step": r["us_per_step_device"], "steps": steps, "value": r["value"], "unit": r["unit"],
+                "frac": r["roofline"]["frac"], "achieved_gbs": r["roofline"]["achieved"], "kernel": r["roofline"]["kernel"],
+                "algorithmic_bytes_per_launch": r["roofline"]["algorithmic_bytes_per_launch"],
+                "cpu_baseline": None if r["cpu_baseline"] is None else
+                {k: r["cpu_baseline"][k] for k in ("value", "unit", "cores", "kind")},
+                "parity": r["parity"], "config": r["config"],
+            }
+        out["per_config"] = per
     print(json.dumps(out))
 
 
