@@ -153,9 +153,9 @@ SR_API int sr_batch_upload(sr_batch* batch, int32_t rows, int32_t vocab,
  *   uniforms  [rows x uniforms_per_row] for the next step, or NULL to keep those on the device.
  * Rows the in-place update does not cover (the first history token of a row with penalties, rows with logit bias
  * or with penalties that may raise a logit, a row that runs out of room) make the call rebuild the whole batch from
- * the inputs it kept: same result, the cost of an upload.  A batch uploaded with allow-masks returns
- * SR_ERR_UNSUPPORTED: its masks change with every step, so it is uploaded again anyway.  Copies run on the
- * context's stream and are not waited for, as in sr_batch_upload. */
+ * the inputs it kept: same result, the cost of an upload.  A batch uploaded with allow-masks of its own returns
+ * SR_ERR_UNSUPPORTED (its masks change with every step: register them and use sr_batch_upload_mask_ids /
+ * sr_batch_append_tokens_masks).  Copies run on the context's stream and are not waited for, as in sr_batch_upload. */
 SR_API int sr_batch_append_tokens(sr_batch* batch, const int32_t* tokens, const double* uniforms);
 /* Replaces only the uniforms of an uploaded batch (same rows and uniforms_per_row). */
 SR_API int sr_batch_set_uniforms(sr_batch* batch, const double* uniforms);
@@ -317,6 +317,38 @@ SR_API int sr_mtp_verify_launch(sr_ctx* ctx, const float* logits_dev, int32_t ro
  * (bit set iff the entry is not negative infinity).  ceil(vocab / 32) words are written.
  */
 SR_API int sr_pack_allow_mask(const float* masked_logits, int32_t vocab, uint32_t* out_words);
+/* The same for `rows` masked rows that are already on the device (fp32 or bf16): out_words_dev is a DEVICE array
+ * [rows x out_stride_words], out_stride_words >= ceil(vocab / 32).  Asynchronous on the context's stream. */
+SR_API int sr_pack_allow_mask_launch(sr_ctx* ctx, const void* masked_logits_dev, int dtype, int32_t rows, int32_t vocab,
+                                     int64_t row_stride_elems, uint32_t* out_words_dev, int64_t out_stride_words);
+
+/*
+ * Registered allow-masks.  A grammar constraint has few distinct masks -- one per automaton state
+ * (JsonToolArgumentConstraint.ComputeMask, src/OpenTail.Stingray.Core/Grammar/JsonToolArgumentConstraint.cs:434-478,
+ * computes the mask of a state by walking the vocabulary; JsonSchemaGrammarMasker.Filter :55-103) -- and meets them
+ * again and again.  sr_mask_register copies the packed bits of one mask (ceil(vocab / 32) words, the format of
+ * sr_batch_upload's allow_mask; host memory, or device memory when words_on_device is non-zero, e.g. what
+ * sr_pack_allow_mask_launch wrote) into device memory once and returns its id; batches then name masks by id
+ * (sr_batch_upload_mask_ids, sr_batch_append_tokens_masks) and a constrained decode step uploads 4 bytes per row
+ * instead of 19 KB.  A context holds masks of one vocabulary size at a time.  sr_mask_release frees an id for
+ * reuse; the caller must not release a mask that an uploaded batch still names.
+ */
+SR_API int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, int32_t vocab, int32_t* out_id);
+SR_API int sr_mask_release(sr_ctx* ctx, int32_t mask_id);
+/* sr_batch_upload with the allow-mask of every row named by id: mask_ids [rows], -1 = the row is not constrained
+ * (ITokenConstraint.Filter returned its input, ITokenConstraint.cs:36-41).  No copy is waited for. */
+SR_API int sr_batch_upload_mask_ids(sr_batch* batch, int32_t rows, int32_t vocab,
+                                    const sr_row_params* params,
+                                    const int32_t* hist_ids, const int32_t* hist_offsets,
+                                    const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                                    const int32_t* mask_ids,
+                                    const double* uniforms, int32_t uniforms_per_row);
+/* sr_batch_append_tokens for a batch uploaded with mask ids: every row also gets the mask of its constraint's next
+ * state (mask_ids [rows], -1 = none), as the engine filters with the advanced constraint before the next Sample
+ * (ContinuousBatchingEngine.cs:635-650: Filter -> Sample -> Accept -> RecentTokens.Add).  In place: a changed id is
+ * 4 bytes in the row's descriptor, plus one rebuilt row of keep-bits for rows of the selection kernel. */
+SR_API int sr_batch_append_tokens_masks(sr_batch* batch, const int32_t* tokens, const double* uniforms,
+                                        const int32_t* mask_ids);
 
 #ifdef __cplusplus
 }

@@ -48,7 +48,8 @@ SR_OUT_ROW_UNSUPPORTED = 1 << 31
 EXPORTED_SYMBOLS = [
     "sr_create", "sr_destroy", "sr_bind_thread", "sr_set_stream", "sr_synchronize", "sr_last_error",
     "sr_version", "sr_batch_create", "sr_batch_destroy", "sr_batch_upload", "sr_batch_set_uniforms",
-    "sr_batch_append_tokens",
+    "sr_batch_append_tokens", "sr_batch_append_tokens_masks", "sr_batch_upload_mask_ids", "sr_mask_register",
+    "sr_mask_release", "sr_pack_allow_mask_launch",
     "sr_sample_launch", "sr_resample_rows_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows_launch_noalloc",
     "sr_argmax_rows",
     "sr_build_distribution_launch", "sr_sample_with_distribution_launch", "sr_sample_from_probs_launch",
@@ -151,6 +152,11 @@ def load_library():
                                   C.POINTER(C.c_uint8), f64p, i32]
     L.sr_batch_set_uniforms.argtypes = [vp, f64p]
     L.sr_batch_append_tokens.argtypes = [vp, i32p, f64p]
+    L.sr_batch_append_tokens_masks.argtypes = [vp, i32p, f64p, i32p]
+    L.sr_batch_upload_mask_ids.argtypes = [vp, i32, i32, rpp, i32p, i32p, i32p, f32p, i32p, i32p, f64p, i32]
+    L.sr_mask_register.argtypes = [vp, vp, C.c_int, i32, i32p]
+    L.sr_mask_release.argtypes = [vp, i32]
+    L.sr_pack_allow_mask_launch.argtypes = [vp, vp, C.c_int, i32, i32, i64, vp, i64]
     L.sr_sample_launch.argtypes = [vp, vp, vp, C.c_int, i64, vp, vp]
     L.sr_resample_rows_launch.argtypes = [vp, vp, vp, C.c_int, i64, i32p, i32, vp, vp]
     L.sr_sample_batch.argtypes = [vp, vp, C.c_int, C.c_int, i32, i32, i64, rpp, i32p, i32p, i32p, f32p, i32p,
@@ -198,7 +204,9 @@ class _Batch:
         self.vocab = 0
 
     def upload(self, params: Sequence[SamplingParams], vocab: int, uniforms=None, allow_mask=None,
-               mask_active=None, uniforms_per_row: Optional[int] = None):
+               mask_active=None, uniforms_per_row: Optional[int] = None, mask_ids=None):
+        """mask_ids: per row the id of a registered allow-mask (SamplerContext.register_mask), -1 for none, instead
+        of allow_mask / mask_active."""
         rows = len(params)
         arr = (RowParams * max(rows, 1))()
         hist: List[int] = []
@@ -237,6 +245,14 @@ class _Batch:
             upr = u.shape[1] if uniforms_per_row is None else uniforms_per_row
         self._packed = (rows, vocab, arr, h_ids, h_off, b_ids, b_vals, b_off, m, stride, act, u, upr)
         self.rows, self.vocab = rows, vocab
+        if mask_ids is not None:
+            assert allow_mask is None
+            ids = np.ascontiguousarray(np.asarray(mask_ids, dtype=np.int32))
+            assert ids.shape == (rows,)
+            self.ctx._check(self.ctx.L.sr_batch_upload_mask_ids(
+                self.h, rows, vocab, arr, _ptr(h_ids, C.c_int32), _ptr(h_off, C.c_int32), _ptr(b_ids, C.c_int32),
+                _ptr(b_vals, C.c_float), _ptr(b_off, C.c_int32), _ptr(ids, C.c_int32), _ptr(u, C.c_double), upr))
+            return self
         return self.reupload()
 
     def reupload(self):
@@ -249,14 +265,21 @@ class _Batch:
             _ptr(m, C.c_uint32), stride, _ptr(act, C.c_uint8), _ptr(u, C.c_double), upr))
         return self
 
-    def append_tokens(self, tokens, uniforms=None):
+    def append_tokens(self, tokens, uniforms=None, mask_ids=None):
         """sr_batch_append_tokens: one more token per row (negative = none) at the end of the histories of the last
-        upload(), and optionally the uniforms of the next step."""
+        upload(), and optionally the uniforms of the next step.  mask_ids (batches uploaded with mask ids): the
+        registered allow-mask of every row for the next step (sr_batch_append_tokens_masks)."""
         t = np.ascontiguousarray(np.asarray(tokens, dtype=np.int32))
         assert t.shape == (self.rows,)
         u = None
         if uniforms is not None:
             u = np.ascontiguousarray(np.asarray(uniforms, dtype=np.float64))
+        if mask_ids is not None:
+            ids = np.ascontiguousarray(np.asarray(mask_ids, dtype=np.int32))
+            assert ids.shape == (self.rows,)
+            self.ctx._check(self.ctx.L.sr_batch_append_tokens_masks(self.h, _ptr(t, C.c_int32), _ptr(u, C.c_double),
+                                                                    _ptr(ids, C.c_int32)))
+            return self
         self.ctx._check(self.ctx.L.sr_batch_append_tokens(self.h, _ptr(t, C.c_int32), _ptr(u, C.c_double)))
         return self
 
@@ -321,6 +344,33 @@ class SamplerContext:
 
     def new_batch(self) -> _Batch:
         return _Batch(self)
+
+    def register_mask(self, words, vocab: int) -> int:
+        """sr_mask_register: packed allow-bits (numpy uint32 array, or a CUDA int32/uint32 tensor) -> mask id."""
+        out = C.c_int32(-1)
+        if isinstance(words, np.ndarray):
+            w = np.ascontiguousarray(words, dtype=np.uint32)
+            assert w.size >= (vocab + 31) // 32
+            self._check(self.L.sr_mask_register(self.h, w.ctypes.data_as(C.c_void_p), 0, vocab, C.byref(out)))
+        else:
+            assert words.is_cuda and words.numel() >= (vocab + 31) // 32
+            self._check(self.L.sr_mask_register(self.h, C.c_void_p(words.data_ptr()), 1, vocab, C.byref(out)))
+        return int(out.value)
+
+    def release_mask(self, mask_id: int) -> None:
+        self._check(self.L.sr_mask_release(self.h, int(mask_id)))
+
+    def pack_allow_mask_launch(self, masked_logits):
+        """Packed allow-bits [rows, ceil(vocab / 32)] (a CUDA int32 tensor holding the uint32 words) of masked rows
+        that are on the device: bit set iff the element is not -inf."""
+        import torch
+
+        rows, vocab = masked_logits.shape
+        out = torch.zeros((rows, (vocab + 31) // 32), dtype=torch.int32, device=masked_logits.device)
+        self._check(self.L.sr_pack_allow_mask_launch(
+            self.h, C.c_void_p(masked_logits.data_ptr()), self._dtype_of(masked_logits), rows, vocab,
+            self._row_stride(masked_logits), C.c_void_p(out.data_ptr()), out.shape[1]))
+        return out
 
     def close(self):
         if self.h:

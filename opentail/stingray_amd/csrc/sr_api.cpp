@@ -10,6 +10,10 @@
 #include "sr_host.h"
 #include "../../../include/stingray_sampler_test.h"
 
+// where a batch's allow-masks lie: its own upload, or the context's registered masks
+const uint32_t* sr_batch_mask_ptr(const sr_batch* b) { return b->mask_ids ? b->ctx->mask_pool.as<uint32_t>() : b->d_mask.as<uint32_t>(); }
+int64_t sr_batch_mask_stride(const sr_batch* b) { return b->mask_ids ? (int64_t)b->ctx->pool_words : b->mask_stride; }
+
 namespace {
 
 inline bool has_history_penalty(const sr_row_params& p)
@@ -210,8 +214,8 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     SR_HIP(ctx, b->d_scan_desc.reserve(b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, batch_copy(b, staged, b->d_scan_desc.p, b->h_scan.data(), b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, b->d_scan_mask.reserve(b->h_scan.size() * (size_t)b->scan_stride * sizeof(uint32_t), st));
-    SR_HIP(ctx, sr_launch_build_scan_mask(b->d_scan_desc.as<SrScanDesc>(), (int)b->h_scan.size(), b->d_rows.as<SrRow>(),
-                                          b->d_edits.as<SrEdit>(), b->d_mask.as<uint32_t>(), b->mask_stride,
+    SR_HIP(ctx, sr_launch_build_scan_mask(b->d_scan_desc.as<SrScanDesc>(), nullptr, (int)b->h_scan.size(), b->d_rows.as<SrRow>(),
+                                          b->d_edits.as<SrEdit>(), sr_batch_mask_ptr(b), sr_batch_mask_stride(b),
                                           b->d_scan_mask.as<uint32_t>(), b->scan_stride, b->vocab, epv, chunks, chunk_vecs,
                                           base_addr, stride_bytes, st));
     // the host vectors are read by the async copies above
@@ -259,7 +263,7 @@ void sr_destroy(sr_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
-    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best, &ctx->argmax_done,
+    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best, &ctx->argmax_done, &ctx->mask_pool,
                          &ctx->work, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs};
@@ -322,7 +326,8 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
                              const int32_t* hist_ids, const int32_t* hist_offsets,
                              const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
                              const uint32_t* allow_mask, int64_t mask_stride_words, const uint8_t* mask_active,
-                             const double* uniforms, int32_t uniforms_per_row, bool retain, bool keep_uniforms)
+                             const double* uniforms, int32_t uniforms_per_row, bool retain, bool keep_uniforms,
+                             const int32_t* mask_ids = nullptr)
 {
     if (!b || !b->ctx) return SR_ERR_NULL_ARGUMENT;
     sr_ctx* ctx = b->ctx;
@@ -336,6 +341,17 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_upload: mask stride shorter than ceil(vocab/32)");
     if (uniforms_per_row < 0 || (uniforms_per_row > 0 && !uniforms && !keep_uniforms))
         return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload: uniforms is null");
+    if (mask_ids) {
+        if (allow_mask) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_upload: allow-masks and mask ids are exclusive");
+        for (int32_t r = 0; r < rows; r++) {
+            const int32_t id = mask_ids[r];
+            if (id < -1 || (id >= 0 && (id >= ctx->pool_cap || !ctx->pool_used[(size_t)id])))
+                return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_upload_mask_ids: row " + std::to_string(r) + " names mask " +
+                                                                 std::to_string(id) + ", which is not registered");
+            if (id >= 0 && ctx->pool_vocab != vocab)
+                return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_upload_mask_ids: the masks were registered for another vocabulary size");
+        }
+    }
     SR_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
     SR_HIP(ctx, b->stage.begin());  // (waits for the copies of this batch's previous upload)
@@ -352,8 +368,10 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
     b->h_scan.clear();
     b->h_scan_need.assign((size_t)rows, 0u);
     b->scan_epv = 0;
-    b->has_mask = allow_mask != nullptr;
+    b->has_mask = allow_mask != nullptr || mask_ids != nullptr;
     b->mask_stride = allow_mask ? mask_stride_words : 0;
+    b->mask_ids = mask_ids != nullptr;
+    if (mask_ids) b->keep_mask_ids.assign(mask_ids, mask_ids + rows); else b->keep_mask_ids.clear();
     b->max_sel = 0;
     b->edit_cap.assign((size_t)rows, 0);
     b->edit_ids.clear();
@@ -405,7 +423,7 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
         d.n_prev = n_prev;
         d.flags = (p.flags & 0xffu) | (has_bias ? (uint32_t)SR_ROW_HAS_LOGIT_BIAS : 0u) |
                   (has_penalty ? SR_ROWFLAG_HAS_PENALTY : 0u);
-        d.mask_row = (allow_mask && (!mask_active || mask_active[r])) ? r : -1;
+        d.mask_row = mask_ids ? mask_ids[r] : (allow_mask && (!mask_active || mask_active[r])) ? r : -1;
         d.edit_off = (int32_t)b->h_edits.size();
         d.edit_cnt = 0;
         d.scan_row = -1;
@@ -522,7 +540,8 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
         if (d.path == SR_PATH_TOPK_WIDE) {
             b->h_wide_list.push_back(r);
         } else if (d.path != SR_PATH_FULL) {
-            if (d.mask_row >= 0) b->h_scan_need[(size_t)r] |= SR_SCAN_ALLOW;
+            // (with registered masks every row gets a scan-mask row of its own: its mask may come, go and change in place)
+            if (d.mask_row >= 0 || mask_ids) b->h_scan_need[(size_t)r] |= SR_SCAN_ALLOW;
             b->h_sel_list.push_back(r);
             b->max_sel = std::max(b->max_sel, d.sel);
         } else {
@@ -591,22 +610,35 @@ static int append_rebuild(sr_batch* b, const double* uniforms)
     }
     const std::vector<int32_t> bias_ids = b->keep_bias_ids, bias_off = b->keep_bias_off;
     const std::vector<float> bias_vals = b->keep_bias_vals;
+    const std::vector<int32_t> mids = b->keep_mask_ids;
     return batch_upload_impl(b, rows, b->vocab, params.data(), ids.data(), off.data(),
                              bias_off.empty() ? nullptr : bias_ids.data(), bias_off.empty() ? nullptr : bias_vals.data(),
                              bias_off.empty() ? nullptr : bias_off.data(), nullptr, 0, nullptr, uniforms, b->upr, false,
-                             uniforms == nullptr);
+                             uniforms == nullptr, b->mask_ids ? mids.data() : nullptr);
 }
 
-int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uniforms)
+static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniforms, const int32_t* new_mask_ids)
 {
     if (!b || !b->ctx) return SR_ERR_NULL_ARGUMENT;
     sr_ctx* ctx = b->ctx;
     if (!tokens) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_append_tokens: tokens is null");
     if (!b->can_append)
         return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_batch_append_tokens: the batch was not uploaded, or was uploaded with "
-                                                "allow-masks (upload it again with the new masks)");
+                                                "allow-masks of its own (register the masks and upload their ids, or "
+                                                "upload it again with the new masks)");
+    if (new_mask_ids && !b->mask_ids)
+        return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_batch_append_tokens_masks: the batch was not uploaded with mask ids");
     const int32_t rows = b->rows, vocab = b->vocab;
     if (rows == 0) return SR_OK;
+    std::vector<int32_t> scan_again;  // scan-mask rows whose allow-mask changes
+    if (new_mask_ids) {
+        for (int32_t r = 0; r < rows; r++) {
+            const int32_t id = new_mask_ids[r];
+            if (id < -1 || (id >= 0 && (id >= ctx->pool_cap || !ctx->pool_used[(size_t)id] || ctx->pool_vocab != vocab)))
+                return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_append_tokens_masks: row " + std::to_string(r) +
+                                                                 " names mask " + std::to_string(id) + ", which is not registered");
+        }
+    }
     if (!b->hist_split) {
         b->keep_hist.assign((size_t)rows, std::vector<int32_t>());
         for (int32_t r = 0; r < rows; r++) {
@@ -645,14 +677,24 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
     std::vector<int32_t> touched;
     bool rebuild = false;
     for (int32_t r = 0; r < rows && !rebuild; r++) {
-        if (tokens[r] < 0) continue;
-        const sr_row_params& p = b->keep_params[(size_t)r];
         SrRow& d = b->h_rows[(size_t)r];
+        bool mask_changed = false;
+        if (new_mask_ids && new_mask_ids[r] != d.mask_row) {
+            d.mask_row = new_mask_ids[r];
+            b->keep_mask_ids[(size_t)r] = new_mask_ids[r];
+            mask_changed = true;
+            if (d.scan_row >= 0 && (b->h_scan_need[(size_t)r] & SR_SCAN_ALLOW)) scan_again.push_back(d.scan_row);
+        }
+        if (tokens[r] < 0) {
+            if (mask_changed) rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row});
+            continue;
+        }
+        const sr_row_params& p = b->keep_params[(size_t)r];
         const std::vector<int32_t>& hist = b->keep_hist[(size_t)r];
         const int32_t n_new = (int32_t)hist.size(), n_old = n_new - 1;
         if (!has_history_penalty(p)) {  // the history is never looked at
             d.n_prev = n_new;
-            rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt});
+            rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row});
             continue;
         }
         if (n_old == 0 || d.edit_cnt == 0 || (d.flags & SR_ROWFLAG_EDITS_SORTED) || d.path == SR_PATH_TOPK_WIDE) {
@@ -703,11 +745,12 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
             touched.push_back(k);
         }
         d.n_prev = n_new;
-        rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt});
+        rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row});
         for (int32_t k : touched) ep.push_back(SrEditPatch{d.edit_off + k, ed[k]});
     }
     if (rebuild) {
         b->append_rebuilds++;
+        if (new_mask_ids) b->keep_mask_ids.assign(new_mask_ids, new_mask_ids + rows);  // (the loop above stopped early)
         return append_rebuild(b, uniforms);
     }
 
@@ -716,7 +759,7 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
     hipStream_t st = ctx->stream;
     const size_t n_uni = (uniforms && b->upr > 0) ? (size_t)rows * (size_t)b->upr : 0;
     const size_t need = rp.size() * sizeof(SrRowPatch) + ep.size() * sizeof(SrEditPatch) + mc.size() * sizeof(SrMaskClear) +
-                        n_uni * sizeof(double) + 4 * 256;
+                        n_uni * sizeof(double) + scan_again.size() * sizeof(int32_t) + 5 * 256;
     SR_HIP(ctx, b->stage.begin());
     if (b->stage.cap < need) {  // grows at begin()
         b->stage.wanted = need;
@@ -726,7 +769,8 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
     const SrEditPatch* ep_d = (const SrEditPatch*)b->stage.put(ep.data(), ep.size() * sizeof(SrEditPatch));
     const SrMaskClear* mc_d = (const SrMaskClear*)b->stage.put(mc.data(), mc.size() * sizeof(SrMaskClear));
     const double* un_d = (const double*)b->stage.put(uniforms, n_uni * sizeof(double));
-    if (!rp_d || !ep_d || !mc_d || !un_d) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "sr_batch_append_tokens: no pinned memory");
+    const int32_t* sa_d = (const int32_t*)b->stage.put(scan_again.data(), scan_again.size() * sizeof(int32_t));
+    if (!rp_d || !ep_d || !mc_d || !un_d || !sa_d) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "sr_batch_append_tokens: no pinned memory");
     // scan masks that are not built yet are built from the patched edits when they are needed
     const bool masks = b->scan_epv != 0 && b->d_scan_mask.p != nullptr;
     SR_HIP(ctx, sr_launch_apply_patches(b->d_rows.as<SrRow>(), rp_d, (int)rp.size(), b->d_edits.as<SrEdit>(), ep_d,
@@ -734,7 +778,111 @@ int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uni
                                         b->scan_stride, masks ? b->scan_epv : 4, masks ? b->scan_chunk_vecs : 64,
                                         b->scan_base_addr, b->scan_stride_bytes, b->d_uniforms.as<double>(), un_d,
                                         (int)n_uni, st));
+    // rows whose allow-mask changed: their scan-mask rows are built again, from the new mask and the patched history
+    if (masks && !scan_again.empty())
+        SR_HIP(ctx, sr_launch_build_scan_mask(b->d_scan_desc.as<SrScanDesc>(), sa_d, (int)scan_again.size(), b->d_rows.as<SrRow>(),
+                                              b->d_edits.as<SrEdit>(), sr_batch_mask_ptr(b), sr_batch_mask_stride(b),
+                                              b->d_scan_mask.as<uint32_t>(), b->scan_stride, b->vocab, b->scan_epv,
+                                              b->scan_chunks, b->scan_chunk_vecs, b->scan_base_addr, b->scan_stride_bytes, st));
     SR_HIP(ctx, b->stage.end(st));
+    return SR_OK;
+}
+
+int sr_batch_append_tokens(sr_batch* b, const int32_t* tokens, const double* uniforms)
+{
+    return append_impl(b, tokens, uniforms, nullptr);
+}
+
+int sr_batch_append_tokens_masks(sr_batch* b, const int32_t* tokens, const double* uniforms, const int32_t* mask_ids)
+{
+    if (b && b->ctx && !mask_ids) return sr_fail(b->ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_append_tokens_masks: mask_ids is null");
+    return append_impl(b, tokens, uniforms, mask_ids);
+}
+
+int sr_batch_upload_mask_ids(sr_batch* b, int32_t rows, int32_t vocab, const sr_row_params* params,
+                             const int32_t* hist_ids, const int32_t* hist_offsets,
+                             const int32_t* bias_ids, const float* bias_vals, const int32_t* bias_offsets,
+                             const int32_t* mask_ids, const double* uniforms, int32_t uniforms_per_row)
+{
+    if (b && b->ctx && !mask_ids) return sr_fail(b->ctx, SR_ERR_NULL_ARGUMENT, "sr_batch_upload_mask_ids: mask_ids is null");
+    return batch_upload_impl(b, rows, vocab, params, hist_ids, hist_offsets, bias_ids, bias_vals, bias_offsets, nullptr, 0,
+                             nullptr, uniforms, uniforms_per_row, true, false, mask_ids);
+}
+
+// ---- registered allow-masks ---------------------------------------------------------------------------
+int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, int32_t vocab, int32_t* out_id)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (!words || !out_id) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_mask_register: null argument");
+    if (vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_register: empty vocabulary");
+    *out_id = -1;
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    const bool any_used = std::find(ctx->pool_used.begin(), ctx->pool_used.end(), (uint8_t)1) != ctx->pool_used.end();
+    if (any_used && vocab != ctx->pool_vocab)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_register: a context holds masks of one vocabulary size at a time (" +
+                                                         std::to_string(ctx->pool_vocab) + " now); release them first");
+    const int32_t nw = (vocab + 31) / 32;
+    if (!any_used && vocab != ctx->pool_vocab) {  // a new vocabulary: the pool starts again
+        SR_HIP(ctx, hipStreamSynchronize(st));
+        ctx->mask_pool.release();
+        ctx->pool_cap = 0;
+        ctx->pool_used.clear();
+        ctx->pool_vocab = vocab;
+        ctx->pool_words = (nw + 3) & ~3;  // rows of the pool start on 16 bytes
+    }
+    int32_t id = -1;
+    for (int32_t i = 0; i < ctx->pool_cap; i++)
+        if (!ctx->pool_used[(size_t)i]) { id = i; break; }
+    if (id < 0) {  // grow: a larger array, the masks moved over on the stream, the old one freed when that is done
+        const int32_t cap = std::max(16, ctx->pool_cap * 2);
+        void* bigger = nullptr;
+        SR_HIP(ctx, hipMalloc(&bigger, (size_t)cap * (size_t)ctx->pool_words * sizeof(uint32_t)));
+        if (ctx->pool_cap > 0) {
+            hipError_t e = hipMemcpyAsync(bigger, ctx->mask_pool.p, (size_t)ctx->pool_cap * (size_t)ctx->pool_words * sizeof(uint32_t),
+                                          hipMemcpyDeviceToDevice, st);
+            if (e == hipSuccess) e = hipStreamSynchronize(st);
+            if (e != hipSuccess) { (void)hipFree(bigger); return sr_fail_hip(ctx, e, "sr_mask_register: moving the masks"); }
+        }
+        ctx->mask_pool.release();
+        ctx->mask_pool.p = bigger;
+        ctx->mask_pool.cap = (size_t)cap * (size_t)ctx->pool_words * sizeof(uint32_t);
+        id = ctx->pool_cap;
+        ctx->pool_cap = cap;
+        ctx->pool_used.resize((size_t)cap, 0);
+    }
+    uint32_t* dst = ctx->mask_pool.as<uint32_t>() + (size_t)id * (size_t)ctx->pool_words;
+    SR_HIP(ctx, hipMemcpyAsync(dst, words, (size_t)nw * sizeof(uint32_t),
+                               words_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, st));
+    // the caller's array may be reused when the call returns (a mask is registered once per grammar state, not per step)
+    if (!words_on_device) SR_HIP(ctx, hipStreamSynchronize(st));
+    ctx->pool_used[(size_t)id] = 1;
+    *out_id = id;
+    return SR_OK;
+}
+
+int sr_mask_release(sr_ctx* ctx, int32_t id)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (id < 0 || id >= ctx->pool_cap || !ctx->pool_used[(size_t)id])
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_release: mask " + std::to_string(id) + " is not registered");
+    ctx->pool_used[(size_t)id] = 0;
+    return SR_OK;
+}
+
+int sr_pack_allow_mask_launch(sr_ctx* ctx, const void* masked_logits_dev, int dtype, int32_t rows, int32_t vocab,
+                              int64_t row_stride_elems, uint32_t* out_words_dev, int64_t out_stride_words)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (rows == 0 || vocab == 0) return SR_OK;
+    if (!masked_logits_dev || !out_words_dev) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_pack_allow_mask_launch: null tensor");
+    if (rows < 0 || vocab < 0 || row_stride_elems < vocab || out_stride_words < (vocab + 31) / 32)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_pack_allow_mask_launch: bad shape");
+    if (dtype != SR_DTYPE_F32 && dtype != SR_DTYPE_BF16)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_pack_allow_mask_launch: unknown dtype");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    SR_HIP(ctx, sr_launch_pack_allow_mask(masked_logits_dev, dtype, rows, vocab, row_stride_elems, out_words_dev,
+                                          out_stride_words, ctx->stream));
     return SR_OK;
 }
 
@@ -803,8 +951,8 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         }
         a.rows = b->d_rows.as<SrRow>();
         a.edits = b->d_edits.as<SrEdit>();
-        a.mask = b->d_mask.as<uint32_t>();
-        a.mask_stride = b->mask_stride;
+        a.mask = sr_batch_mask_ptr(b);
+        a.mask_stride = sr_batch_mask_stride(b);
         a.scan_mask = b->d_scan_mask.as<uint32_t>();
         a.scan_stride = b->scan_stride;
         a.cand = ctx->cand.as<unsigned long long>();

@@ -25,8 +25,8 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     a.row_list = list_dev;
     a.rows = b->d_rows.as<SrRow>();
     a.edits = b->d_edits.as<SrEdit>();
-    a.mask = b->d_mask.as<uint32_t>();
-    a.mask_stride = b->mask_stride;
+    a.mask = sr_batch_mask_ptr(b);
+    a.mask_stride = sr_batch_mask_stride(b);
     a.mode = mode;
     a.prof = ctx->prof;
     if (mode == 0) {
@@ -152,8 +152,8 @@ int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev,
     a.row_list = list_dev;
     a.rows = b->d_rows.as<SrRow>();
     a.edits = b->d_edits.as<SrEdit>();
-    a.mask = b->d_mask.as<uint32_t>();
-    a.mask_stride = b->mask_stride;
+    a.mask = sr_batch_mask_ptr(b);
+    a.mask_stride = sr_batch_mask_stride(b);
     SR_HIP(ctx, ctx->work.reserve(items * sizeof(float), st));
     a.work = ctx->work.as<float>();
     a.work_stride = stride;

@@ -124,6 +124,11 @@ struct sr_ctx {
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
     int last_epv = 4;                    // vector width of the last launch: what an upload builds scan masks for
+    // Registered allow-masks (sr_mask_register): one device array of `pool_cap` slots of `pool_words` words each, the
+    // id of a mask is its slot.  One vocabulary size per context at a time.
+    DeviceBuf mask_pool;
+    int32_t pool_vocab = 0, pool_words = 0, pool_cap = 0;
+    std::vector<uint8_t> pool_used;
     // selection kernel: entries per set of counters, launches so far (its parity picks the set), and how often a row
     // tail polls its row's counter before it stops waiting and selects from the logits alone
     size_t done_cap = 0;
@@ -151,6 +156,8 @@ struct sr_batch {
     // the row stride in bytes modulo 16 (rows share a mask row only when all start at the same offset)
     int32_t scan_epv = 0, scan_base_mod = -1, scan_stride_mod = -1;
     bool has_mask = false;
+    bool mask_ids = false;               // the rows' allow-masks are registered masks of the context (mask_row = id)
+    std::vector<int32_t> keep_mask_ids;  // ... per row, -1 none
     int32_t max_sel = 0;
     HostStage stage;          // pinned copies of what an upload sends to the device
     bool upload_must_wait = false;  // some copy of the running upload reads pageable memory directly
@@ -188,6 +195,10 @@ inline int sr_fail_hip(sr_ctx* ctx, hipError_t e, const char* what)
         hipError_t _e = (call);                                       \
         if (_e != hipSuccess) return sr_fail_hip((ctx), _e, #call);   \
     } while (0)
+
+// where a batch's allow-masks lie: its own upload, or the context's registered masks (sr_api.cpp)
+const uint32_t* sr_batch_mask_ptr(const sr_batch* b);
+int64_t sr_batch_mask_stride(const sr_batch* b);
 
 // Full-vocabulary rows of a batch (sr_full_host.cpp).  mode: 0 = sample, 1 = build distribution,
 // 2 = build distribution and sample from it.

@@ -63,7 +63,10 @@ struct SrTopkArgs {
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream);
 // Builds scan row i for descs[i]; base_addr / stride_bytes are those of the logits the mask is used with
 // (they decide where a row starts inside its first 16-byte vector), epv = 4 (fp32) or 8 (bf16).
-hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, int n_scan, const SrRow* rows, const SrEdit* edits,
+// scan_ids: the n_scan scan rows to build (NULL: rows 0 .. n_scan - 1)
+hipError_t sr_launch_pack_allow_mask(const void* logits, int dtype, int rows, int vocab, int64_t row_stride, uint32_t* out,
+                                     int64_t out_stride, hipStream_t stream);
+hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, const int32_t* scan_ids, int n_scan, const SrRow* rows, const SrEdit* edits,
                                      const uint32_t* mask, int64_t mask_stride, uint32_t* scan_mask, int64_t scan_stride,
                                      int vocab, int epv, int chunks, int chunk_vecs, unsigned long long base_addr,
                                      long long stride_bytes, hipStream_t stream);

@@ -1724,14 +1724,16 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 // lies inside the row, its allow-mask (if any) admits it and, for rows whose tail fetches the history logits by
 // id, it is not a history id.  One workgroup per (scan row, chunk): the words are built in LDS, the history ids
 // that fall into the chunk are cleared there, then the words are written out.
-__global__ __launch_bounds__(kThreads) void k_build_scan_mask(const SrScanDesc* descs, const SrRow* rows, const SrEdit* edits,
+__global__ __launch_bounds__(kThreads) void k_build_scan_mask(const SrScanDesc* descs, const int32_t* scan_ids,
+                                                              const SrRow* rows, const SrEdit* edits,
                                                               const uint32_t* mask, int64_t mask_stride, uint32_t* scan_mask,
                                                               int64_t scan_stride, int vocab, int epv, int es, int chunks,
                                                               int chunk_vecs, int vecs_per_thread,
                                                               unsigned long long base_addr, long long stride_bytes)
 {
     __shared__ uint32_t words[kThreads * SR_TK_MASK_WORDS];
-    const int srow = blockIdx.x / chunks, c = blockIdx.x - srow * chunks;
+    const int nth = blockIdx.x / chunks, c = blockIdx.x - nth * chunks;
+    const int srow = scan_ids ? scan_ids[nth] : nth;  // a list of scan rows to build again, or all of them
     const int t = threadIdx.x;
     const SrScanDesc d = descs[srow];
     const SrRow rd = rows[d.row];
@@ -1795,6 +1797,7 @@ __global__ __launch_bounds__(256) void k_apply_patches(SrRow* rows, const SrRowP
         const SrRowPatch r = rp[i];
         rows[r.row].n_prev = r.n_prev;
         rows[r.row].edit_cnt = r.edit_cnt;
+        rows[r.row].mask_row = r.mask_row;
     }
     if (i < n_edits) edits[ep[i].index] = ep[i].edit;
     if (i < n_clears) {
@@ -1811,7 +1814,42 @@ __global__ __launch_bounds__(256) void k_apply_patches(SrRow* rows, const SrRowP
     if (i < n_uni) uni_dst[i] = uni_src[i];
 }
 
+// Packed allow-bits of rows that hold -inf where a token is not allowed (ITokenConstraint.Filter's output,
+// ITokenConstraint.cs:31-42): bit (i & 31) of word (i >> 5) = the row's element i is not -inf.  One wave per 64
+// elements: a coalesced load, one ballot, two words.
+template <int ES>
+__global__ __launch_bounds__(256) void k_pack_allow_mask(const void* logits, int64_t row_stride, int vocab, uint32_t* out,
+                                                         int64_t out_stride)
+{
+    const int row = blockIdx.y;
+    const char* rowp = (const char*)logits + (size_t)row * (size_t)row_stride * ES;
+    const int n64 = (vocab + 63) / 64;
+    const int wave = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6), lane = sr_lane();
+    const int n_waves = (int)((gridDim.x * blockDim.x) >> 6);
+    for (int g = wave; g < n64; g += n_waves) {
+        const int i = g * 64 + lane;
+        bool allowed = false;
+        if (i < vocab) {
+            const uint32_t bits = ES == 4 ? ((const uint32_t*)rowp)[i] : ((uint32_t)((const uint16_t*)rowp)[i] << 16);
+            allowed = bits != 0xff800000u;
+        }
+        const unsigned long long bal = __ballot(allowed);
+        if (lane < 2 && g * 2 + lane < (vocab + 31) / 32)
+            out[(size_t)row * out_stride + g * 2 + lane] = (uint32_t)(bal >> (32 * lane));
+    }
+}
 }  // namespace
+
+hipError_t sr_launch_pack_allow_mask(const void* logits, int dtype, int rows, int vocab, int64_t row_stride, uint32_t* out,
+                                     int64_t out_stride, hipStream_t stream)
+{
+    if (rows <= 0 || vocab <= 0) return hipSuccess;
+    const int n64 = (vocab + 63) / 64;
+    const dim3 grid((unsigned)std::min((n64 + 3) / 4, 1024), (unsigned)rows), block(256);
+    if (dtype == 1) hipLaunchKernelGGL(k_pack_allow_mask<2>, grid, block, 0, stream, logits, row_stride, vocab, out, out_stride);
+    else hipLaunchKernelGGL(k_pack_allow_mask<4>, grid, block, 0, stream, logits, row_stride, vocab, out, out_stride);
+    return hipGetLastError();
+}
 
 hipError_t sr_launch_apply_patches(SrRow* rows, const SrRowPatch* rp, int n_rowp, SrEdit* edits, const SrEditPatch* ep,
                                    int n_edits, const SrMaskClear* mc, int n_clears, uint32_t* scan_mask,
@@ -1842,13 +1880,13 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
     return hipGetLastError();
 }
 
-hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, int n_scan, const SrRow* rows, const SrEdit* edits,
+hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, const int32_t* scan_ids, int n_scan, const SrRow* rows, const SrEdit* edits,
                                      const uint32_t* mask, int64_t mask_stride, uint32_t* scan_mask, int64_t scan_stride,
                                      int vocab, int epv, int chunks, int chunk_vecs, unsigned long long base_addr,
                                      long long stride_bytes, hipStream_t stream)
 {
     if (n_scan <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_build_scan_mask, dim3((unsigned)(n_scan * chunks)), dim3(kThreads), 0, stream, descs, rows, edits,
+    hipLaunchKernelGGL(k_build_scan_mask, dim3((unsigned)(n_scan * chunks)), dim3(kThreads), 0, stream, descs, scan_ids, rows, edits,
                        mask, mask_stride, scan_mask, scan_stride, vocab, epv, epv == 8 ? 2 : 4, chunks, chunk_vecs,
                        epv == 8 ? SR_TK_VEC_BF16 : SR_TK_VEC, base_addr, stride_bytes);
     return hipGetLastError();
