@@ -29,10 +29,16 @@ def test_header_and_python_symbol_lists_agree():
     assert _declared_symbols() == sorted(sa.EXPORTED_SYMBOLS)
 
 
-def test_the_managed_binding_that_the_integration_notes_show_names_every_entry_point():
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+def test_the_managed_binding_names_every_entry_point():
+    text = open(os.path.join(ROOT, "opentail", "stingray_amd", "managed", "StingraySamplerInterop.cs")).read()
     bound = sorted(set(re.findall(r'EntryPoint = "(sr_\w+)"', text)))
     assert bound == _declared_symbols()
+    # ... and the managed sampler calls only bindings that exist
+    calls = set()
+    for f in ("RocmBatchSampler.cs", "EngineSeam.cs"):
+        calls |= set(re.findall(r"StingraySamplerInterop\.(\w+)\(", open(os.path.join(ROOT, "opentail", "stingray_amd", "managed", f)).read()))
+    declared = set(re.findall(r"internal static (?:partial )?\w+ (\w+)\(", text))
+    assert calls and calls <= declared, calls - declared
 
 
 def test_library_exports_every_declared_symbol():
