@@ -98,12 +98,14 @@ SR_API void sr_destroy(sr_ctx* ctx);
 /* IThreadAffineBackend.BindToCurrentThread (IThreadAffineBackend.cs:9-21): makes the context's device
  * current on the calling thread. */
 SR_API int sr_bind_thread(sr_ctx* ctx);
-/* Kernels are enqueued on this stream (a hipStream_t); NULL restores the context's own stream.  Lets
- * the forward pass that produced the logits and the sampler share one stream, so no event is needed
- * between them (the pattern of CudaBackend.cs:4119-4123).  The context's own stream is non-blocking: it is
- * not ordered with the device's default stream, so a caller whose tensors are produced there either passes
- * hipStreamLegacy (the default stream by name) or synchronises before the launch. */
+/* Kernels are enqueued on this stream (a hipStream_t).  Lets the forward pass that produced the logits and the
+ * sampler share one stream, so no event is needed between them (the pattern of CudaBackend.cs:4119-4123).
+ * NULL means what it means everywhere in HIP: the device's default stream -- a managed caller that passes a zero
+ * handle is ordered behind work on the default stream, not silently beside it.  A new context runs on a stream of
+ * its own, which is non-blocking (not ordered with the default stream); sr_use_own_stream goes back to it.
+ * Either call first waits for what the context has in flight on the stream it leaves. */
 SR_API int sr_set_stream(sr_ctx* ctx, void* hip_stream);
+SR_API int sr_use_own_stream(sr_ctx* ctx);
 SR_API int sr_synchronize(sr_ctx* ctx);
 /* Text of the last failure on this context (never NULL). */
 SR_API const char* sr_last_error(sr_ctx* ctx);

@@ -46,7 +46,7 @@ SR_OUT_ROW_UNSUPPORTED = 1 << 31
 
 # every symbol include/stingray_sampler.h declares
 EXPORTED_SYMBOLS = [
-    "sr_create", "sr_destroy", "sr_bind_thread", "sr_set_stream", "sr_synchronize", "sr_last_error",
+    "sr_create", "sr_destroy", "sr_bind_thread", "sr_set_stream", "sr_use_own_stream", "sr_synchronize", "sr_last_error",
     "sr_version", "sr_batch_create", "sr_batch_destroy", "sr_batch_upload", "sr_batch_set_uniforms",
     "sr_batch_append_tokens", "sr_batch_append_tokens_masks", "sr_batch_upload_mask_ids", "sr_mask_register",
     "sr_mask_release", "sr_pack_allow_mask_launch",
@@ -141,6 +141,7 @@ def load_library():
     L.sr_destroy.restype = None
     L.sr_bind_thread.argtypes = [vp]
     L.sr_set_stream.argtypes = [vp, vp]
+    L.sr_use_own_stream.argtypes = [vp]
     L.sr_synchronize.argtypes = [vp]
     L.sr_last_error.argtypes = [vp]
     L.sr_last_error.restype = C.c_char_p
@@ -317,10 +318,9 @@ class SamplerContext:
         if use_torch_stream:
             import torch
 
-            # torch's default stream has the handle 0, which sr_set_stream reads as "the context's own stream": a
-            # non-blocking stream that nothing orders behind torch's work.  The default stream is named explicitly.
+            # torch's current stream; its default stream has the handle 0, which is HIP's default stream here too
             handle = torch.cuda.current_stream(device).cuda_stream
-            self._check(self.L.sr_set_stream(self.h, C.c_void_p(handle or HIP_STREAM_LEGACY)))
+            self._check(self.L.sr_set_stream(self.h, C.c_void_p(handle)))
 
     # -- plumbing ------------------------------------------------------------------------------
     def _check(self, rc: int):
@@ -336,8 +336,11 @@ class SamplerContext:
         raise RuntimeError(f"native sampler error {rc}: {msg}")
 
     def set_stream(self, stream_handle: Optional[int]):
-        """A hipStream_t handle; None or 0 = the context's own stream (HIP_STREAM_LEGACY names the default stream)."""
-        self._check(self.L.sr_set_stream(self.h, C.c_void_p(stream_handle or 0)))
+        """A hipStream_t handle (0 = the device's default stream); None = the context's own stream."""
+        if stream_handle is None:
+            self._check(self.L.sr_use_own_stream(self.h))
+        else:
+            self._check(self.L.sr_set_stream(self.h, C.c_void_p(stream_handle)))
 
     def synchronize(self):
         self._check(self.L.sr_synchronize(self.h))

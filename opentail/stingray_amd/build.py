@@ -27,7 +27,7 @@ SOURCES = ["sr_api.cpp", "sr_full_host.cpp", "sr_topk.hip", "sr_argmax.hip", "sr
 
 
 def _deps():
-    return [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".cuh"))] + [
+    return [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")] + [
         os.path.join(HERE, "..", "..", "include", "stingray_sampler.h")]
 
 

@@ -279,15 +279,25 @@ int sr_bind_thread(sr_ctx* ctx)
     return SR_OK;
 }
 
-int sr_set_stream(sr_ctx* ctx, void* hip_stream)
+static int switch_stream(sr_ctx* ctx, hipStream_t next)
 {
-    if (!ctx) return SR_ERR_NULL_ARGUMENT;
-    hipStream_t next = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
     // uploads of batches may still be running on the stream that is left: later launches are ordered behind them
     // only on the same stream
     if (next != ctx->stream) SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
     ctx->stream = next;
     return SR_OK;
+}
+
+int sr_set_stream(sr_ctx* ctx, void* hip_stream)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    return switch_stream(ctx, (hipStream_t)hip_stream);  // NULL is HIP's default stream, as everywhere in HIP
+}
+
+int sr_use_own_stream(sr_ctx* ctx)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    return switch_stream(ctx, ctx->own_stream);
 }
 
 int sr_synchronize(sr_ctx* ctx)

@@ -12,7 +12,7 @@
 // device memory that belongs to the library's code object, one copy per GPU.
 #include <algorithm>
 
-#include "sr_device.cuh"
+#include "sr_device.h"
 #include "sr_kernels.h"
 #include "sr_types.h"
 

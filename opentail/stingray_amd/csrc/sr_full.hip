@@ -4,11 +4,11 @@
 //
 // The row is materialised in an fp32 work row exactly as the reference copies it, and every stage is
 // one pass of a 1024-thread workgroup over that row.  All running sums that the reference evaluates
-// left to right go through the exact evaluator in sr_seqsum.cuh, so probabilities, cut-offs and draws
+// left to right go through the exact evaluator in sr_seqsum.h, so probabilities, cut-offs and draws
 // carry the reference's bits.
-#include "sr_device.cuh"
+#include "sr_device.h"
 #include "sr_kernels.h"
-#include "sr_seqsum.cuh"
+#include "sr_seqsum.h"
 #include "sr_types.h"
 
 namespace {

@@ -18,7 +18,7 @@
 // Block size: SR_SEQ_THREADS threads, SR_SEQ_RUN consecutive terms per thread, so one tile covers
 // SR_SEQ_THREADS * SR_SEQ_RUN terms.  All threads of the block must call.
 #pragma once
-#include "sr_device.cuh"
+#include "sr_device.h"
 
 #define SR_SEQ_THREADS 1024
 #define SR_SEQ_RUN 16

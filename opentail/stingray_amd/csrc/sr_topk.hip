@@ -21,7 +21,7 @@
 // history is in the final k only if it is among the k best outside the history, and a history token
 // that the reference's over-selection misses has more than k unpenalised tokens above it.  Penalties
 // that can raise a logit keep the reference's literal over-selection.
-#include "sr_device.cuh"
+#include "sr_device.h"
 #include "sr_types.h"
 #include "sr_kernels.h"
 

@@ -23,6 +23,7 @@ internal static unsafe partial class StingraySamplerInterop
     [LibraryImport(Lib, EntryPoint = "sr_destroy")]       internal static partial void Destroy(nint ctx);
     [LibraryImport(Lib, EntryPoint = "sr_bind_thread")]   internal static partial int BindThread(nint ctx);
     [LibraryImport(Lib, EntryPoint = "sr_set_stream")]    internal static partial int SetStream(nint ctx, nint hipStream);
+    [LibraryImport(Lib, EntryPoint = "sr_use_own_stream")] internal static partial int UseOwnStream(nint ctx);
     [LibraryImport(Lib, EntryPoint = "sr_synchronize")]   internal static partial int Synchronize(nint ctx);
     [LibraryImport(Lib, EntryPoint = "sr_last_error")]    internal static partial nint LastError(nint ctx);
 
