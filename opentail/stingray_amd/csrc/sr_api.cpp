@@ -41,22 +41,49 @@ void topk_geometry(int vocab, int dtype, int n_rows, int cu_count, int* chunks, 
     *chunk_vecs = cv;
 }
 
-// (Re)builds the scan masks of a batch for logits of the given vector width and alignment.  Rows without an
-// allow-mask and without excluded history ids share one mask row when every row starts at the same offset
-// inside its first vector.
+// Sends the packed pieces: one kernel reads them from the pinned memory and writes them where they belong.  To be
+// called before anything that reads the destinations is enqueued.
+hipError_t batch_flush(sr_batch* b, hipStream_t st)
+{
+    if (b->segs.empty()) return hipSuccess;
+    const SrCopySeg* table = (const SrCopySeg*)b->stage.put(b->segs.data(), b->segs.size() * sizeof(SrCopySeg));
+    hipError_t e = hipSuccess;
+    if (table) {
+        e = sr_launch_scatter(table, (int)b->segs.size(), st);
+    } else {  // no room for the list (the pinned memory grows for the next upload): one copy per piece
+        for (const SrCopySeg& s : b->segs) {
+            e = hipMemcpyAsync(s.dst, s.src, (size_t)s.bytes, hipMemcpyHostToDevice, st);
+            if (e != hipSuccess) break;
+        }
+    }
+    b->segs.clear();
+    return e;
+}
+
 // Copies host data of a batch to the device on `st`: through the batch's pinned memory when `staged` (no wait
 // needed), else straight from `src`, which the caller then has to keep alive until the stream is synchronised.
 hipError_t batch_copy(sr_batch* b, bool staged, void* dst, const void* src, size_t bytes, hipStream_t st)
 {
     if (bytes == 0) return hipSuccess;
     const void* from = staged ? b->stage.put(src, bytes) : nullptr;
-    if (!from) {
-        from = src;
-        b->upload_must_wait = true;
+    if (from) {  // packed: sent with the other pieces by batch_flush; a later version of the same array replaces the earlier
+        for (SrCopySeg& s : b->segs)
+            if (s.dst == dst) { s.src = from; s.bytes = (unsigned long long)bytes; return hipSuccess; }
+        b->segs.push_back(SrCopySeg{from, dst, (unsigned long long)bytes});
+        return hipSuccess;
     }
-    return hipMemcpyAsync(dst, from, bytes, hipMemcpyHostToDevice, st);
+    // Straight from the caller's memory.  The packed pieces go first: one of them may be an earlier version of this
+    // very array (the row descriptors are sent again once their scan-mask rows are known), and the order of the
+    // two must stay the order of the calls.
+    hipError_t e = batch_flush(b, st);
+    if (e != hipSuccess) return e;
+    b->upload_must_wait = true;
+    return hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, st);
 }
 
+// (Re)builds the scan masks of a batch for logits of the given vector width and alignment.  Rows without an
+// allow-mask and without excluded history ids share one mask row when every row starts at the same offset
+// inside its first vector.
 int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long stride_bytes, bool staged = false)
 {
     sr_ctx* ctx = b->ctx;
@@ -214,6 +241,7 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     SR_HIP(ctx, b->d_scan_desc.reserve(b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, batch_copy(b, staged, b->d_scan_desc.p, b->h_scan.data(), b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, b->d_scan_mask.reserve(b->h_scan.size() * (size_t)b->scan_stride * sizeof(uint32_t), st));
+    SR_HIP(ctx, batch_flush(b, st));
     SR_HIP(ctx, sr_launch_build_scan_mask(b->d_scan_desc.as<SrScanDesc>(), nullptr, (int)b->h_scan.size(), b->d_rows.as<SrRow>(),
                                           b->d_edits.as<SrEdit>(), sr_batch_mask_ptr(b), sr_batch_mask_stride(b),
                                           b->d_scan_mask.as<uint32_t>(), b->scan_stride, b->vocab, epv, chunks, chunk_vecs,
@@ -365,6 +393,7 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
     SR_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
     SR_HIP(ctx, b->stage.begin());  // (waits for the copies of this batch's previous upload)
+    b->segs.clear();
     b->upload_must_wait = false;
 
     b->rows = rows;
@@ -521,9 +550,12 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
             }
             d.edit_cnt = (int32_t)ed.size() - d.edit_off;
             b->edit_cap[(size_t)r] = d.edit_cnt;
-            if (want_hist && !searched && d.edit_cnt > 0) {  // room for the ids that appended tokens bring
-                ed.resize(ed.size() + SR_EDIT_SLACK);
-                b->edit_cap[(size_t)r] += SR_EDIT_SLACK;
+            if (want_hist && !searched && d.edit_cnt > 0) {
+                // room for the ids that appended tokens bring: a fixed minimum, and half as much again as the row has
+                // (a batch that was rebuilt because a row ran out of room is not rebuilt again soon)
+                const int32_t slack = std::max(SR_EDIT_SLACK, d.edit_cnt / 2);
+                ed.resize(ed.size() + (size_t)slack);
+                b->edit_cap[(size_t)r] += slack;
             }
         }
         // Penalties that can only lower a logit (Sampler.cs:281-286 with repetition >= 1, presence >= 0 and
@@ -572,6 +604,10 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
         return batch_copy(b, true, dst.p, src, bytes, st);
     };
     SR_HIP(ctx, up(b->d_rows, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow)));
+    // (the edit lists of a batch that tokens are appended to grow with every rebuild: room for four times their size, so
+    // that a rebuild finds its device memory in place)
+    if (b->can_append && b->d_edits.cap < b->h_edits.size() * sizeof(SrEdit))
+        SR_HIP(ctx, b->d_edits.reserve(4 * b->h_edits.size() * sizeof(SrEdit), st));
     SR_HIP(ctx, up(b->d_edits, b->h_edits.data(), b->h_edits.size() * sizeof(SrEdit)));
     SR_HIP(ctx, up(b->d_sel_list, b->h_sel_list.data(), b->h_sel_list.size() * sizeof(int32_t)));
     SR_HIP(ctx, up(b->d_full_list, b->h_full_list.data(), b->h_full_list.size() * sizeof(int32_t)));
@@ -592,6 +628,7 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
     // Everything small went through the batch's pinned memory: the copies and the scan-mask kernel run on while
     // the caller goes on (launches on this stream are ordered behind them).  Pageable memory that a copy reads
     // directly (the caller's allow-mask; anything the pinned memory had no room for yet) must be waited for.
+    SR_HIP(ctx, batch_flush(b, st));
     if (b->upload_must_wait) SR_HIP(ctx, hipStreamSynchronize(st));
     SR_HIP(ctx, b->stage.end(st));
     return SR_OK;

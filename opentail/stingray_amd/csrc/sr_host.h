@@ -14,10 +14,12 @@
 struct DeviceBuf {
     void* p = nullptr;
     size_t cap = 0;
-    // Grows (never shrinks).  zero_new clears a newly allocated buffer on `stream`.
+    // Grows (never shrinks), by half at least: a buffer that grows a little with every call (the edit lists of a
+    // decode loop) is not allocated anew every time.  zero_new clears a newly allocated buffer on `stream`.
     hipError_t reserve(size_t bytes, hipStream_t stream, bool zero_new = false)
     {
         if (bytes <= cap) return hipSuccess;
+        if (p) bytes = std::max(bytes, cap + cap / 2);
         if (p) {
             hipError_t e = hipStreamSynchronize(stream);
             if (e != hipSuccess) return e;
@@ -60,7 +62,8 @@ struct HostStage {
             if (p) (void)hipHostFree(p);
             p = nullptr;
             cap = 0;
-            const size_t want = wanted + wanted / 2 + 4096;
+            // roomy (a decode loop's edit lists grow; an upload that does not fit sends pieces unpacked and waits)
+            const size_t want = 4 * wanted + 65536;
             hipError_t e = hipHostMalloc((void**)&p, want, hipHostMallocDefault);
             if (e != hipSuccess) { p = nullptr; return e; }
             cap = want;
@@ -160,6 +163,7 @@ struct sr_batch {
     std::vector<int32_t> keep_mask_ids;  // ... per row, -1 none
     int32_t max_sel = 0;
     HostStage stage;          // pinned copies of what an upload sends to the device
+    std::vector<SrCopySeg> segs;  // ... the pieces that are packed and not yet sent
     bool upload_must_wait = false;  // some copy of the running upload reads pageable memory directly
     // geometry the scan masks were built with (sr_batch_append_tokens clears single bits in place)
     int32_t scan_chunks = 0, scan_chunk_vecs = 0;
@@ -179,7 +183,7 @@ struct sr_batch {
 
 // room left behind the edits of a row whose edits are kept in order of first appearance, for ids that
 // sr_batch_append_tokens adds
-#define SR_EDIT_SLACK 16
+#define SR_EDIT_SLACK 32
 
 inline int sr_fail(sr_ctx* ctx, int code, const std::string& msg)
 {

@@ -63,6 +63,8 @@ struct SrTopkArgs {
 hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream);
 // Builds scan row i for descs[i]; base_addr / stride_bytes are those of the logits the mask is used with
 // (they decide where a row starts inside its first 16-byte vector), epv = 4 (fp32) or 8 (bf16).
+// all pieces of an upload in one launch: segs (itself in pinned host memory) lists n pieces
+hipError_t sr_launch_scatter(const SrCopySeg* segs, int n, hipStream_t stream);
 // scan_ids: the n_scan scan rows to build (NULL: rows 0 .. n_scan - 1)
 hipError_t sr_launch_pack_allow_mask(const void* logits, int dtype, int rows, int vocab, int64_t row_stride, uint32_t* out,
                                      int64_t out_stride, hipStream_t stream);

@@ -52,6 +52,12 @@ struct SrEditPatch {
     int32_t index;
     SrEdit edit;
 };
+// one piece of an upload: bytes that lie in pinned host memory and belong at a device address
+struct SrCopySeg {
+    const void* src;
+    void* dst;
+    unsigned long long bytes;
+};
 struct SrRowPatch {
     int32_t row;
     int32_t n_prev;
