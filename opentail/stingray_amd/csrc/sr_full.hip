@@ -159,36 +159,60 @@ __device__ __forceinline__ float seq_sum(Term term, int n, float s0, float targe
     return s;
 }
 
-// The same over a row in memory: a thread's SR_SEQ_RUN consecutive terms come in with four 16-byte loads when the
-// row is 16-byte aligned (one 4-byte load per term makes every load instruction of a wave touch 64 cache lines),
-// and the loads of the next tile are in flight while the current one is scanned.
-template <bool kSearch, typename Load>
-__device__ __forceinline__ float seq_sum_tiles(Load load, int n, float s0, float target, int* found, FullSmem& sm)
+// The same over rows in memory.  A thread's SR_SEQ_RUN consecutive terms come in with four 16-byte loads when the
+// row is 16-byte aligned (one 4-byte load per term makes every load instruction of a wave touch 64 cache lines).
+// The loads run kDepth - 1 tiles ahead of the tile that is scanned, into register sets that take turns: one
+// workgroup has to keep that much in flight to cover the latency of memory, or every tile waits for its loads
+// (what is loaded is turned into terms only when its tile is up, so that nothing waits for a load early).
+//   issue(base, raw)   starts the loads of the tile whose first term is `base`
+//   finish(raw, x)     the tile's terms from what was loaded
+template <bool kSearch, int kDepth, typename Raw, typename Issue, typename Finish>
+__device__ __forceinline__ float seq_sum_tiles(Issue issue, Finish finish, int n, float s0, float target, int* found, FullSmem& sm)
 {
     float s = s0;
     *found = -1;
-    // two register sets take turns, so that no copy (which would wait for the loads) sits between the tiles
-    float xa[SR_SEQ_RUN], xb[SR_SEQ_RUN];
+    Raw r[kDepth];
+    const int n_tiles = (n + SR_SEQ_TILE - 1) / SR_SEQ_TILE;
 #pragma unroll
-    for (int j = 0; j < SR_SEQ_RUN; j++) xa[j] = xb[j] = 0.0f;
-    if (n > 0) load(0, xa);
-    for (int base = 0; base < n; base += 2 * SR_SEQ_TILE) {
-        int f;
-        if (base + SR_SEQ_TILE < n) load(base + SR_SEQ_TILE, xb);
-        sr_seq_tile<kSearch>(xa, &s, target, &f, sm.seq);
-        if (kSearch && f >= 0) {
-            *found = base + f;
-            return s;
-        }
-        if (base + SR_SEQ_TILE >= n) break;
-        if (base + 2 * SR_SEQ_TILE < n) load(base + 2 * SR_SEQ_TILE, xa);
-        sr_seq_tile<kSearch>(xb, &s, target, &f, sm.seq);
-        if (kSearch && f >= 0) {
-            *found = base + SR_SEQ_TILE + f;
-            return s;
+    for (int k = 0; k < kDepth - 1; k++)
+        if (k < n_tiles) issue(k * SR_SEQ_TILE, r[k]);
+    for (int t0 = 0; t0 < n_tiles; t0 += kDepth) {
+#pragma unroll
+        for (int k = 0; k < kDepth; k++) {
+            const int t = t0 + k;
+            if (t >= n_tiles) return s;
+            if (t + kDepth - 1 < n_tiles) issue((t + kDepth - 1) * SR_SEQ_TILE, r[(k + kDepth - 1) % kDepth]);
+            float x[SR_SEQ_RUN];
+            finish(r[k], x);
+            int f;
+            sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+            if (kSearch && f >= 0) {
+                *found = t * SR_SEQ_TILE + f;
+                return s;
+            }
         }
     }
     return s;
+}
+
+struct SeqRaw1 { float v[SR_SEQ_RUN]; };
+struct SeqRaw2 { float p[SR_SEQ_RUN], q[SR_SEQ_RUN]; };
+
+// SR_SEQ_RUN consecutive elements of a row from index i0 on, zeros past the row's end
+__device__ __forceinline__ void seq_load_run(const float* p, bool aligned, int i0, int n, float (&v)[SR_SEQ_RUN])
+{
+    static_assert(SR_SEQ_RUN % 4 == 0, "whole float4 per thread");
+    if (aligned && i0 + SR_SEQ_RUN <= n) {
+        const float4* vp = (const float4*)(p + i0);
+#pragma unroll
+        for (int k = 0; k < SR_SEQ_RUN / 4; k++) {
+            const float4 a = vp[k];
+            v[4 * k] = a.x; v[4 * k + 1] = a.y; v[4 * k + 2] = a.z; v[4 * k + 3] = a.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) v[j] = (i0 + j < n) ? p[i0 + j] : 0.0f;
+    }
 }
 
 // (every term is multiplied by m1 and then by m2 first: the two normalising factors of a row that was left unscaled)
@@ -196,25 +220,15 @@ template <bool kSearch>
 __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm,
                                              float m1 = 1.0f, float m2 = 1.0f)
 {
-    static_assert(SR_SEQ_RUN % 4 == 0, "whole float4 per thread");
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
-    auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
-        const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
-        if (aligned && i0 + SR_SEQ_RUN <= n) {
-            const float4* v = (const float4*)(p + i0);
-#pragma unroll
-            for (int k = 0; k < SR_SEQ_RUN / 4; k++) {
-                const float4 a = v[k];
-                x[4 * k] = a.x; x[4 * k + 1] = a.y; x[4 * k + 2] = a.z; x[4 * k + 3] = a.w;
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? p[i0 + j] : 0.0f;
-        }
-#pragma unroll
-        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = __fmul_rn(__fmul_rn(x[j], m1), m2);
+    auto issue = [&](int base, SeqRaw1& r) __attribute__((always_inline)) {
+        seq_load_run(p, aligned, base + (int)threadIdx.x * SR_SEQ_RUN, n, r.v);
     };
-    return seq_sum_tiles<kSearch>(load, n, s0, target, found, sm);
+    auto finish = [&](const SeqRaw1& r, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = __fmul_rn(__fmul_rn(r.v[j], m1), m2);
+    };
+    return seq_sum_tiles<kSearch, 3, SeqRaw1>(issue, finish, n, s0, target, found, sm);
 }
 
 // ... and over the positive part of the difference of two rows (residual resampling)
@@ -223,27 +237,19 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
                                                   FullSmem& sm, float m1 = 1.0f, float m2 = 1.0f)
 {
     const bool aligned = (((uintptr_t)p | (uintptr_t)q) & 15u) == 0u;
-    auto res = [&](float a, float b) -> float {
-        const float r = __fsub_rn(__fmul_rn(__fmul_rn(a, m1), m2), b);
-        return r > 0.0f ? r : 0.0f;
-    };
-    auto load = [&](int base, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
+    auto issue = [&](int base, SeqRaw2& r) __attribute__((always_inline)) {
         const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
-        if (aligned && i0 + SR_SEQ_RUN <= n) {
-            const float4* vp = (const float4*)(p + i0);
-            const float4* vq = (const float4*)(q + i0);
+        seq_load_run(p, aligned, i0, n, r.p);
+        seq_load_run(q, aligned, i0, n, r.q);
+    };
+    auto finish = [&](const SeqRaw2& r, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int k = 0; k < SR_SEQ_RUN / 4; k++) {
-                const float4 a = vp[k], b = vq[k];
-                x[4 * k] = res(a.x, b.x); x[4 * k + 1] = res(a.y, b.y);
-                x[4 * k + 2] = res(a.z, b.z); x[4 * k + 3] = res(a.w, b.w);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? res(p[i0 + j], q[i0 + j]) : 0.0f;
+        for (int j = 0; j < SR_SEQ_RUN; j++) {
+            const float d = __fsub_rn(__fmul_rn(__fmul_rn(r.p[j], m1), m2), r.q[j]);
+            x[j] = d > 0.0f ? d : 0.0f;
         }
     };
-    return seq_sum_tiles<kSearch>(load, n, s0, target, found, sm);
+    return seq_sum_tiles<kSearch, 2, SeqRaw2>(issue, finish, n, s0, target, found, sm);
 }
 
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
@@ -322,16 +328,20 @@ __device__ __forceinline__ void normalize_row(float* p, int n, FullSmem& sm)
 // k-th largest value of p[0..n) (1-based), p >= 0: FindKthLargest (Sampler.cs:624-645).
 // With last_shift = 16 only the upper 16 bits are resolved: the result is then the smallest value of the
 // 65536-value bucket that holds the k-th largest.
-__device__ __forceinline__ float kth_largest(const float* p, int n, int k, FullSmem& sm, int last_shift = 0)
+// Keys above hi_key are left out (they count as absent).
+__device__ __forceinline__ float kth_largest(const float* p, int n, int k, FullSmem& sm, int last_shift = 0,
+                                             uint32_t hi_key = 0xffffffffu)
 {
     uint32_t prefix = 0u, pmask = 0u;
     int need = k;
     for (int shift = 24; shift >= last_shift; shift -= 8) {
         if (threadIdx.x < 256) sm.hist[threadIdx.x] = 0u;
         __syncthreads();
+        // Zeros (masked or filtered entries, often most of the row) are left out: they are the smallest keys and
+        // only matter when fewer than k entries are positive, and then the answer is zero either way.
         row_pass<false>(const_cast<float*>(p), n, [&](float x, int) -> float {
             const uint32_t key = sr_f2u(x);
-            if ((key & pmask) == prefix) atomicAdd(&sm.hist[(key >> shift) & 0xffu], 1u);
+            if (key != 0u && (key & pmask) == prefix && key <= hi_key) atomicAdd(&sm.hist[(key >> shift) & 0xffu], 1u);
             return x;
         });
         __syncthreads();
@@ -834,32 +844,40 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             // each thread owns the strided indices tid, tid + kT, ...; a second pass assigns slots per tile
             ns = blk_sum_i(cnt, sm);
             const bool have_list = ns_listed >= 0;  // (then ns == ns_listed <= kSmall)
-            int nc = ns;           // candidates sorted inside the kernel
-            float c_above = -1.0f;  // ... are the probabilities strictly above this value
-            if (ns > kSmall) {
-                // Many survivors (a masked row without min-p): the nucleus is still short.  Take the largest
-                // probabilities -- everything above the 65536-value bucket that holds the kSmall-th largest --
-                // and look for the cut-off among them; only if the nucleus does not close there is the whole row
-                // sorted.
-                c_above = sr_u2f(sr_f2u(kth_largest(p, n, kSmall, sm, 16)) | 0xffffu);
-                int cg = 0;
-                row_pass<false>(p, n, [&](float x, int) -> float { cg += x > c_above ? 1 : 0; return x; });
-                nc = blk_sum_i(cg, sm);  // < kSmall
-            }
+            // The nucleus is walked in descending order, a slab of at most kSmall probabilities at a time: the slab
+            // is everything above the 65536-value bucket that holds the kSmall-th largest of what is left, it is
+            // sorted here and the exact running sum goes on through it from where the slab before ended.  Most
+            // nuclei close in the first slab; a masked row without min-p (tens of thousands of survivors) takes a
+            // few.  Only a row that makes no progress (more than kSmall probabilities inside one bucket) or needs
+            // more than kMaxSlabs slabs has its survivors sorted device-wide.
+            constexpr int kMaxSlabs = 24;
             bool closed = false;
-            if (nc > 0 && nc <= kSmall) {
-                if (!have_list) {
+            float run = 0.0f;                  // exact running sum behind the slabs taken so far
+            int taken = 0;                     // survivors in those slabs
+            uint32_t hi_key = 0xffffffffu;     // what is left are the probabilities with keys <= hi_key
+            float c_above = -1.0f;             // the current slab: probabilities strictly above this value ...
+            for (int slab = 0; slab < kMaxSlabs && ns > 0 && !closed; slab++) {
+                const bool last_slab = ns - taken <= kSmall;  // everything that is left fits
+                c_above = last_slab ? 0.0f : sr_u2f(sr_f2u(kth_largest(p, n, kSmall, sm, 16, hi_key)) | 0xffffu);
+                int nc;
+                if (have_list) {
+                    nc = ns;  // (ns <= kSmall: the survivors were listed while the row was scaled)
+                } else {
                     if (tid == 0) sm.bc[4] = 0u;
                     __syncthreads();
                     row_pass<false>(p, n, [&](float v, int i) -> float {
-                        if (v > 0.0f && v > c_above) {
+                        if (v > c_above && sr_f2u(v) <= hi_key) {
                             const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
-                            sm.sortbuf[pos] = ((unsigned long long)sr_f2u(v) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+                            if (pos < (uint32_t)kSmall)
+                                sm.sortbuf[pos] = ((unsigned long long)sr_f2u(v) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
                         }
                         return v;
                     });
+                    __syncthreads();
+                    nc = (int)sm.bc[4];
+                    __syncthreads();
                 }
-                __syncthreads();
+                if (nc <= 0 || nc > kSmall) break;  // no progress: the device-wide sort takes the row
                 int P = 2;
                 while (P < nc) P <<= 1;
                 for (int i = nc + tid; i < P; i += kT) sm.sortbuf[i] = 0ull;
@@ -868,19 +886,22 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 for (int i = tid; i < nc; i += kT) sm.sprob[i] = sr_u2f((uint32_t)(sm.sortbuf[i] >> 32));
                 __syncthreads();
                 int found;
-                seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, 0.0f, rd.top_p, &found, sm);
-                closed = found >= 0 || nc == ns;
+                run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, rd.top_p, &found, sm);
+                taken += nc;
+                closed = found >= 0 || taken == ns;
                 if (closed) {
                     const int cutoff = found >= 0 ? found + 1 : nc;
                     if (!row_unwritten)
                         for (int i = cutoff + tid; i < nc; i += kT)
                             p[0xffffffffu - (uint32_t)(sm.sortbuf[i] & 0xffffffffull)] = 0.0f;
                     __syncthreads();
-                    if (nc < ns) {  // everything that was not a candidate comes later in the order
+                    if (taken < ns) {  // everything that was in no slab comes later in the order
                         row_pass<true>(p, n, [&](float x, int) -> float { return x > c_above ? x : 0.0f; });
                         __syncthreads();
                     }
-                    listed = cutoff;
+                    if (slab == 0) listed = cutoff;  // the members are all at hand
+                } else {
+                    hi_key = sr_f2u(c_above);
                 }
             }
             if (ns > 0 && !closed) {
