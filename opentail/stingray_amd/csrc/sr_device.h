@@ -109,6 +109,11 @@ __device__ __forceinline__ void sr_store_agent_f4(float4* p, float x, float y, f
 }
 __device__ __forceinline__ void sr_drain_stores() { __builtin_amdgcn_s_waitcnt(0); }
 
+// A workgroup barrier for data exchanged through LDS only: waits for this wave's LDS operations, not for its loads
+// from memory.  __syncthreads() carries a fence that also waits for every load in flight, which throws away
+// whatever a loop has prefetched for its next turn.
+__device__ __forceinline__ void sr_barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ---- wave / block primitives --------------------------------------------------------------------
 __device__ __forceinline__ int sr_lane() { return (int)(threadIdx.x & (SR_WAVE - 1)); }
 __device__ __forceinline__ int sr_wave_id() { return (int)(threadIdx.x >> 6); }

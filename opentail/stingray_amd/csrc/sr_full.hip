@@ -148,7 +148,7 @@ __device__ __forceinline__ float seq_sum(Term term, int n, float s0, float targe
         float x[SR_SEQ_RUN];
         const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
 #pragma unroll
-        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (i0 + j < n) ? term(i0 + j) : 0.0f;
+        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = (threadIdx.x < SR_SEQ_ACTIVE && i0 + j < n) ? term(i0 + j) : 0.0f;
         int f;
         sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
         if (kSearch && f >= 0) {
@@ -159,37 +159,54 @@ __device__ __forceinline__ float seq_sum(Term term, int n, float s0, float targe
     return s;
 }
 
-// The same over rows in memory.  A thread's SR_SEQ_RUN consecutive terms come in with four 16-byte loads when the
-// row is 16-byte aligned (one 4-byte load per term makes every load instruction of a wave touch 64 cache lines).
-// The loads run kDepth - 1 tiles ahead of the tile that is scanned, into register sets that take turns: one
-// workgroup has to keep that much in flight to cover the latency of memory, or every tile waits for its loads
-// (what is loaded is turned into terms only when its tile is up, so that nothing waits for a load early).
-//   issue(base, raw)   starts the loads of the tile whose first term is `base`
-//   finish(raw, x)     the tile's terms from what was loaded
-template <bool kSearch, int kDepth, typename Raw, typename Issue, typename Finish>
-__device__ __forceinline__ float seq_sum_tiles(Issue issue, Finish finish, int n, float s0, float target, int* found, FullSmem& sm)
+// The same over rows in memory.  A thread's SR_SEQ_RUN consecutive terms come in with 16-byte loads when the row
+// is 16-byte aligned (one 4-byte load per term makes every load instruction of a wave touch 64 cache lines).
+// The whole tiles of an aligned row are loaded kDepth - 1 tiles ahead of the tile that is scanned, into register
+// sets that take turns: one workgroup has to keep that much in flight to cover the latency of memory.  Two things
+// keep the loads in flight: what is loaded is turned into terms only when its tile is up, and the loop issues the
+// same number of loads on every path -- behind the last tile it loads that tile again, to no effect -- because the
+// compiler can wait for "all but the newest n loads" only where it can count them, and otherwise waits for all.
+//   issue_fast(base, raw)  starts the loads of the whole tile whose first term is `base`, no conditions
+//   issue_any(base, raw)   the same for any tile of any row (ragged end, unaligned row)
+//   finish(raw, x)         the tile's terms from what was loaded
+template <bool kSearch, int kDepth, typename Raw, typename IssueFast, typename IssueAny, typename Finish>
+__device__ __forceinline__ float seq_sum_tiles(IssueFast issue_fast, IssueAny issue_any, Finish finish, bool fast_ok, int n,
+                                               float s0, float target, int* found, FullSmem& sm)
 {
     float s = s0;
     *found = -1;
-    Raw r[kDepth];
-    const int n_tiles = (n + SR_SEQ_TILE - 1) / SR_SEQ_TILE;
+    const int n_full = fast_ok ? n / SR_SEQ_TILE : 0;  // whole tiles, taken by the pipelined loop
+    if (n_full > 0) {
+        Raw r[kDepth];
 #pragma unroll
-    for (int k = 0; k < kDepth - 1; k++)
-        if (k < n_tiles) issue(k * SR_SEQ_TILE, r[k]);
-    for (int t0 = 0; t0 < n_tiles; t0 += kDepth) {
+        for (int k = 0; k < kDepth - 1; k++) issue_fast(min(k, n_full - 1) * SR_SEQ_TILE, r[k]);
+        for (int t0 = 0; t0 < n_full; t0 += kDepth) {
 #pragma unroll
-        for (int k = 0; k < kDepth; k++) {
-            const int t = t0 + k;
-            if (t >= n_tiles) return s;
-            if (t + kDepth - 1 < n_tiles) issue((t + kDepth - 1) * SR_SEQ_TILE, r[(k + kDepth - 1) % kDepth]);
-            float x[SR_SEQ_RUN];
-            finish(r[k], x);
-            int f;
-            sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
-            if (kSearch && f >= 0) {
-                *found = t * SR_SEQ_TILE + f;
-                return s;
+            for (int k = 0; k < kDepth; k++) {
+                const int t = t0 + k;
+                if (t >= n_full) break;
+                issue_fast(min(t + kDepth - 1, n_full - 1) * SR_SEQ_TILE, r[(k + kDepth - 1) % kDepth]);
+                float x[SR_SEQ_RUN];
+                finish(r[k], x);
+                int f;
+                sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+                if (kSearch && f >= 0) {
+                    *found = t * SR_SEQ_TILE + f;
+                    return s;
+                }
             }
+        }
+    }
+    for (int base = n_full * SR_SEQ_TILE; base < n; base += SR_SEQ_TILE) {
+        Raw r;
+        issue_any(base, r);
+        float x[SR_SEQ_RUN];
+        finish(r, x);
+        int f;
+        sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
+        if (kSearch && f >= 0) {
+            *found = base + f;
+            return s;
         }
     }
     return s;
@@ -198,17 +215,25 @@ __device__ __forceinline__ float seq_sum_tiles(Issue issue, Finish finish, int n
 struct SeqRaw1 { float v[SR_SEQ_RUN]; };
 struct SeqRaw2 { float p[SR_SEQ_RUN], q[SR_SEQ_RUN]; };
 
-// SR_SEQ_RUN consecutive elements of a row from index i0 on, zeros past the row's end
-__device__ __forceinline__ void seq_load_run(const float* p, bool aligned, int i0, int n, float (&v)[SR_SEQ_RUN])
+// SR_SEQ_RUN consecutive elements of an aligned row from index i0 on, all inside the row
+__device__ __forceinline__ void seq_load_run_fast(const float* p, int i0, float (&v)[SR_SEQ_RUN])
 {
     static_assert(SR_SEQ_RUN % 4 == 0, "whole float4 per thread");
-    if (aligned && i0 + SR_SEQ_RUN <= n) {
-        const float4* vp = (const float4*)(p + i0);
+    const float4* vp = (const float4*)(p + i0);
 #pragma unroll
-        for (int k = 0; k < SR_SEQ_RUN / 4; k++) {
-            const float4 a = vp[k];
-            v[4 * k] = a.x; v[4 * k + 1] = a.y; v[4 * k + 2] = a.z; v[4 * k + 3] = a.w;
-        }
+    for (int k = 0; k < SR_SEQ_RUN / 4; k++) {
+        const float4 a = vp[k];
+        v[4 * k] = a.x; v[4 * k + 1] = a.y; v[4 * k + 2] = a.z; v[4 * k + 3] = a.w;
+    }
+}
+// ... of any row, zeros past the row's end
+__device__ __forceinline__ void seq_load_run(const float* p, bool aligned, int i0, int n, float (&v)[SR_SEQ_RUN])
+{
+    if (threadIdx.x >= SR_SEQ_ACTIVE) {  // (these threads carry no terms)
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) v[j] = 0.0f;
+    } else if (aligned && i0 + SR_SEQ_RUN <= n) {
+        seq_load_run_fast(p, i0, v);
     } else {
 #pragma unroll
         for (int j = 0; j < SR_SEQ_RUN; j++) v[j] = (i0 + j < n) ? p[i0 + j] : 0.0f;
@@ -220,15 +245,19 @@ template <bool kSearch>
 __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm,
                                              float m1 = 1.0f, float m2 = 1.0f)
 {
+    static_assert(SR_SEQ_ACTIVE == SR_SEQ_THREADS, "every thread of the block loads a run");
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
-    auto issue = [&](int base, SeqRaw1& r) __attribute__((always_inline)) {
+    auto issue_fast = [&](int base, SeqRaw1& r) __attribute__((always_inline)) {
+        seq_load_run_fast(p, base + (int)threadIdx.x * SR_SEQ_RUN, r.v);
+    };
+    auto issue_any = [&](int base, SeqRaw1& r) __attribute__((always_inline)) {
         seq_load_run(p, aligned, base + (int)threadIdx.x * SR_SEQ_RUN, n, r.v);
     };
     auto finish = [&](const SeqRaw1& r, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = __fmul_rn(__fmul_rn(r.v[j], m1), m2);
     };
-    return seq_sum_tiles<kSearch, 3, SeqRaw1>(issue, finish, n, s0, target, found, sm);
+    return seq_sum_tiles<kSearch, 3, SeqRaw1>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm);
 }
 
 // ... and over the positive part of the difference of two rows (residual resampling)
@@ -237,7 +266,12 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
                                                   FullSmem& sm, float m1 = 1.0f, float m2 = 1.0f)
 {
     const bool aligned = (((uintptr_t)p | (uintptr_t)q) & 15u) == 0u;
-    auto issue = [&](int base, SeqRaw2& r) __attribute__((always_inline)) {
+    auto issue_fast = [&](int base, SeqRaw2& r) __attribute__((always_inline)) {
+        const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
+        seq_load_run_fast(p, i0, r.p);
+        seq_load_run_fast(q, i0, r.q);
+    };
+    auto issue_any = [&](int base, SeqRaw2& r) __attribute__((always_inline)) {
         const int i0 = base + (int)threadIdx.x * SR_SEQ_RUN;
         seq_load_run(p, aligned, i0, n, r.p);
         seq_load_run(q, aligned, i0, n, r.q);
@@ -249,7 +283,7 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
             x[j] = d > 0.0f ? d : 0.0f;
         }
     };
-    return seq_sum_tiles<kSearch, 2, SeqRaw2>(issue, finish, n, s0, target, found, sm);
+    return seq_sum_tiles<kSearch, 2, SeqRaw2>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm);
 }
 
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the

@@ -15,15 +15,18 @@
 //     input, and the rest of the tile is rescanned in the new binade.  A sum crosses at most ~150
 //     binades, in practice a handful.
 //
-// Block size: SR_SEQ_THREADS threads, SR_SEQ_RUN consecutive terms per thread, so one tile covers
-// SR_SEQ_THREADS * SR_SEQ_RUN terms.  All threads of the block must call.
+// Block size: SR_SEQ_THREADS threads, of which the first SR_SEQ_ACTIVE carry SR_SEQ_RUN consecutive terms each, so
+// one tile covers SR_SEQ_ACTIVE * SR_SEQ_RUN terms (a round of the tile costs what its waves' scans cost: with the
+// terms in half as many waves, twice as many each, a round takes about half the time).  All threads of the block
+// must call.
 #pragma once
 #include "sr_device.h"
 
 #define SR_SEQ_THREADS 1024
+#define SR_SEQ_ACTIVE 1024  // threads that carry terms in sr_seq_tile: the first eight waves (the others only meet at the barriers)
 #define SR_SEQ_RUN 16
 #define SR_SEQ_RUN8 16  // terms per thread of the eight-chain tile
-#define SR_SEQ_TILE (SR_SEQ_THREADS * SR_SEQ_RUN)
+#define SR_SEQ_TILE (SR_SEQ_ACTIVE * SR_SEQ_RUN)
 #define SR_SEQ_WAVES (SR_SEQ_THREADS / SR_WAVE)
 #define SR_SEQ_SAT (1u << 26)  // saturated increment: "this run leaves the binade"
 
@@ -89,6 +92,24 @@ template <int N> __device__ __forceinline__ SrInc sr_run_inc(const float (&x)[N]
 template <bool kRowOnly>
 __device__ __forceinline__ SrInc sr_scan_inc(SrInc v)
 {
+    // Nearly always every lane's increment is the same for both parities (they differ only behind an add that fell
+    // exactly half way between two values): the functions are then plain numbers and their composition is a sum.
+    if (__ballot(v.a0 != v.a1) == 0ull) {
+        uint32_t t = v.a0;
+        t = sr_sat_add(t, sr_dpp_u32<0x111>(t));
+        t = sr_sat_add(t, sr_dpp_u32<0x112>(t));
+        t = sr_sat_add(t, sr_dpp_u32<0x114>(t));
+        t = sr_sat_add(t, sr_dpp_u32<0x118>(t));
+        if (!kRowOnly) {
+            const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)t, 15);
+            const uint32_t r1 = sr_sat_add(r0, (uint32_t)__builtin_amdgcn_readlane((int)t, 31));
+            const uint32_t r2 = sr_sat_add(r1, (uint32_t)__builtin_amdgcn_readlane((int)t, 47));
+            const int row = sr_lane() >> 4;
+            t = sr_sat_add(row == 1 ? r0 : row == 2 ? r1 : row == 3 ? r2 : 0u, t);
+        }
+        v.a0 = v.a1 = t;
+        return v;
+    }
     auto step = [&](auto ctrl) {
         constexpr int kC = decltype(ctrl)::value;
         SrInc lo;
@@ -137,10 +158,10 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
     const int tid = threadIdx.x, lane = sr_lane();
     const int wave = __builtin_amdgcn_readfirstlane(sr_wave_id());
     int start = 0;             // threads below `start` are settled
-    int wend = SR_SEQ_THREADS;  // this round looks at the threads [start, wend); a multiple of the wave size
+    int wend = SR_SEQ_ACTIVE;  // this round looks at the threads [start, wend); a multiple of the wave size
     float s_in = *s;
     *found = -1;
-    __syncthreads();  // the previous call's readers are done with the arrays below
+    sr_barrier_lds();  // the previous call's readers are done with the arrays below
     for (int round = 0;; round++) {
         const int buf = round & 1;
         uint32_t n_in;
@@ -155,7 +176,7 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
         }
         // (this copy is written again two rounds on, behind a barrier that every reader of it has passed)
         if (lane == SR_WAVE - 1) { sm.wa0[buf][wave] = incl.a0; sm.wa1[buf][wave] = incl.a1; }
-        __syncthreads();
+        sr_barrier_lds();
         SrInc ti; ti.a0 = 0u; ti.a1 = 0u;
         if (lane < SR_SEQ_WAVES) { ti.a0 = sm.wa0[buf][lane]; ti.a1 = sm.wa1[buf][lane]; }
         ti = sr_scan_inc<true>(ti);  // lanes 0..15: the state function at the end of every wave
@@ -169,9 +190,9 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
             // everything up to the window's end stays in the binade: settle with the total
             const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)((n_in & 1u) ? ti.a1 : ti.a0), SR_SEQ_WAVES - 1);
             s_in = sr_join(n_in + tot, eb);
-            if (wend >= SR_SEQ_THREADS) { *s = s_in; return; }
+            if (wend >= SR_SEQ_ACTIVE) { *s = s_in; return; }
             start = wend;
-            wend = SR_SEQ_THREADS;
+            wend = SR_SEQ_ACTIVE;
             continue;
         }
         const int ev_wave = (int)__ffsll((long long)ev) - 1;
@@ -237,14 +258,16 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
                 sm.misc[2] = (uint32_t)(wave * SR_WAVE + last);
             }
         }
-        __syncthreads();
+        sr_barrier_lds();
         s_in = sr_u2f(sm.misc[0]);
         const int where = (int)sm.misc[1];
         const int fst = (int)sm.misc[2];
         if (kSearch && where >= 0) { *found = where; *s = s_in; return; }
         start = fst + 1;
-        if (start >= SR_SEQ_THREADS) { *s = s_in; return; }
-        wend = min(SR_SEQ_THREADS, (2 * start + 2 * SR_WAVE - 1) & ~(SR_WAVE - 1));
+        if (start >= SR_SEQ_ACTIVE) { *s = s_in; return; }
+        // (a tile's first crossing is mostly its only one -- a sum that has grown doubles once in many tiles --, so the
+        // round after it takes the whole rest; from the second crossing on the sum is doubling fast)
+        wend = round == 0 ? SR_SEQ_ACTIVE : min(SR_SEQ_ACTIVE, (2 * start + 2 * SR_WAVE - 1) & ~(SR_WAVE - 1));
     }
 }
 
@@ -294,7 +317,7 @@ __device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN8], floa
     int start = 0;     // chain threads below `start` are settled
     bool done = false; // this chain has finished the tile
     float s_in = *s;
-    __syncthreads();  // the previous call's readers are done with the arrays below
+    sr_barrier_lds();  // the previous call's readers are done with the arrays below
     for (int round = 0;; round++) {
         const int buf = round & 1;
         uint32_t n_in;
@@ -307,7 +330,7 @@ __device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN8], floa
         const SrInc incl = sr_scan_inc_chain(mine);
         // (this copy is written again two rounds on, behind a barrier that every reader of it has passed)
         if (lane >= SR_WAVE - SR_SEQ_CHAINS) { sm.wa0[buf][wave][g] = incl.a0; sm.wa1[buf][wave][g] = incl.a1; }
-        __syncthreads();
+        sr_barrier_lds();
         // lane l holds, for chain l & 7, the totals of wave l >> 3 and of wave 8 + (l >> 3)
         SrInc ta, tb;
         ta.a0 = sm.wa0[buf][lane >> 3][g]; ta.a1 = sm.wa1[buf][lane >> 3][g];
@@ -357,7 +380,7 @@ __device__ __forceinline__ void sr_seq_tile8(const float (&x)[SR_SEQ_RUN8], floa
             sm.acc[g] = sr_f2u(acc);
             sm.first[g] = lt;
         }
-        __syncthreads();
+        sr_barrier_lds();
         if (!done) {
             if (ev_wave < 0) {
                 s_in = sr_join(n_in + (odd ? t1 : t0), eb);  // this chain stays in its binade to the tile's end
