@@ -19,6 +19,7 @@ Workloads (opentail/stingray_amd/synthetic.py):
   c1            batch 1 x vocab 49,152 (us/step is the figure of interest)
   c2, c4        full-vocabulary path (batch 64 / batch 32 with allow-masks)
   c5            speculative verification, batch 16 x 8 drafts x vocab 262,144 (sr_spec_verify_launch)
+  argmax        Sampler.Greedy per row of 256 x 151,936 fp32 (sr_argmax_rows_launch)
 """
 from __future__ import annotations
 
@@ -177,10 +178,64 @@ def bench_spec(args, w, ctx, stream) -> dict:
     return out_j
 
 
+def bench_argmax(args, ctx, stream) -> dict:
+    """Row argmax (sr_argmax_rows_launch) of 256 x 151,936 fp32 logits, four rotated resident buffers."""
+    import torch
+
+    from opentail.stingray_amd import synthetic
+
+    w = synthetic.config3(rows=256, bf16=False)
+    rows, vocab = w.rows, w.vocab
+    bufs = [torch.from_numpy(np.roll(w.logits, (i * 7) % rows, axis=0)).cuda() for i in range(4)]
+    idx = torch.empty(rows, dtype=torch.int32, device="cuda")
+    val = torch.empty(rows, dtype=torch.float32, device="cuda")
+    import ctypes as C
+
+    def step(i):
+        t = bufs[i % 4]
+        ctx._check(ctx.L.sr_argmax_rows_launch(ctx.h, C.c_void_p(t.data_ptr()), 0, rows, vocab, vocab,
+                                               C.c_void_p(idx.data_ptr()), C.c_void_p(val.data_ptr())))
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for i in range(args.steps):
+        step(i)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_us = ev0.elapsed_time(ev1) * 1e3 / args.steps
+    parity = None
+    if not args.no_parity:
+        from oracle import binding as orc
+
+        last = np.roll(w.logits, (((args.steps - 1) % 4) * 7) % rows, axis=0)
+        want = np.array([orc.greedy(r) for r in last])
+        parity = {"rows_checked": rows, "mismatches": int((idx.cpu().numpy() != want).sum())}
+    alg_bytes = rows * vocab * 4 + rows * 8
+    achieved = alg_bytes / (dev_us * 1e-6) / 1e9
+    return {
+        "metric": f"greedy rows/sec at B={rows}x{vocab} vocab", "value": rows * args.steps / wall, "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps,
+        "us_per_step_device": dev_us, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (seeded Gaussian + Zipf-head logits, 4 rotated resident buffers)",
+        "config": {"workload": "argmax", "rows": rows, "vocab": vocab},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                     "kernel": "k_argmax_rows", "kernel_us": dev_us},
+        "cpu_baseline": None, "parity": parity,
+    }
+
+
 def run_workload(args, ctx, stream) -> dict:
     """One workload (args.workload) for args.steps timed steps; the result as the dict that main() prints."""
     import torch
 
+    if args.workload == "argmax":
+        return bench_argmax(args, ctx, stream)
     w = make_workload(args.workload)
     rows, vocab = w.rows, w.vocab
     if args.workload == "c5":

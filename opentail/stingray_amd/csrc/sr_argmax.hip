@@ -41,14 +41,20 @@ template <int ES> __device__ __forceinline__ float load_elem(const char* p, int6
     return sr_bf16_to_f32(((const uint16_t*)p)[i]);
 }
 
-__device__ __forceinline__ void fold(unsigned long long& best, float v, uint32_t i)
+// A thread's best element so far: key (NaN above everything) and index.  A thread meets its elements in ascending
+// index order, so "strictly larger" keeps the first of equal keys.
+struct Best {
+    uint32_t key, idx;
+};
+__device__ __forceinline__ void fold(Best& b, float v, uint32_t i)
 {
     const uint32_t k = (v != v) ? 0xffffffffu : sr_okey(v);
-    const unsigned long long e = ((unsigned long long)k << 32) | (unsigned long long)(0xffffffffu - i);
-    best = e > best ? e : best;
+    const bool up = k > b.key;
+    b.idx = up ? i : b.idx;
+    b.key = up ? k : b.key;
 }
 
-template <int ES> __device__ __forceinline__ void fold_vec(unsigned long long& best, const u32x4 t, uint32_t first)
+template <int ES> __device__ __forceinline__ void fold_vec(Best& best, const u32x4 t, uint32_t first)
 {
 #pragma unroll
     for (int w = 0; w < 4; w++) {
@@ -71,7 +77,9 @@ template <int ES, bool kVec> __global__ __launch_bounds__(kThreads) void k_argma
     const int lo = c * a.chunk_len, hi = min(a.vocab, lo + a.chunk_len);
     const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
     const int tid = (int)threadIdx.x;
-    unsigned long long best = 0ull;
+    Best tb;
+    tb.key = 0u;  // (no element has the key 0: an empty chunk leaves it)
+    tb.idx = 0u;
     int scalar_from = lo;
     if (kVec) {
         const u32x4* vp = (const u32x4*)rowp;
@@ -82,21 +90,27 @@ template <int ES, bool kVec> __global__ __launch_bounds__(kThreads) void k_argma
 #pragma unroll
             for (int j = 0; j < kUnroll; j++) t[j] = __builtin_nontemporal_load(vp + i + j * kThreads);
 #pragma unroll
-            for (int j = 0; j < kUnroll; j++) fold_vec<ES>(best, t[j], (uint32_t)(i + j * kThreads) * EPV);
+            for (int j = 0; j < kUnroll; j++) fold_vec<ES>(tb, t[j], (uint32_t)(i + j * kThreads) * EPV);
         }
-        for (; i < v_hi; i += kThreads) fold_vec<ES>(best, __builtin_nontemporal_load(vp + i), (uint32_t)i * EPV);
+        for (; i < v_hi; i += kThreads) fold_vec<ES>(tb, __builtin_nontemporal_load(vp + i), (uint32_t)i * EPV);
         scalar_from = max(lo, v_hi * EPV);
     }
-    for (int i = scalar_from + tid; i < hi; i += kThreads) fold(best, load_elem<ES>(rowp, i), (uint32_t)i);
+    for (int i = scalar_from + tid; i < hi; i += kThreads) fold(tb, load_elem<ES>(rowp, i), (uint32_t)i);
 
+    // (key << 32 | ~index): the largest key wins, among equal keys the lowest index
+    unsigned long long best = tb.key ? ((unsigned long long)tb.key << 32) | (unsigned long long)(0xffffffffu - tb.idx) : 0ull;
     best = sr_wave_max_u64(best);
     if (sr_lane() == 0) s_best[sr_wave_id()] = best;
     __syncthreads();
     if (tid != 0) return;
     for (int w = 1; w < kThreads / SR_WAVE; w++) best = s_best[w] > best ? s_best[w] : best;
     if (a.chunks > 1) {
-        if (best) __hip_atomic_fetch_max(&a.best[row], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t before = __hip_atomic_fetch_add(&a.done[row], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        // Both are device-scope atomics without a fence (a release fence would write back the whole L2): the maximum
+        // is waited for -- its old value comes back -- before the chunk is counted in, so whoever counts in last
+        // finds every chunk's maximum in the slot.
+        const unsigned long long seen = __hip_atomic_fetch_max(&a.best[row], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("" : : "v"(seen) : "memory");
+        const uint32_t before = __hip_atomic_fetch_add(&a.done[row], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (before != (uint32_t)a.chunks - 1u) return;
         best = __hip_atomic_load(&a.best[row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&a.best[row], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
