@@ -55,8 +55,13 @@ enum { SR_DTYPE_F32 = 0, SR_DTYPE_BF16 = 1 };
 
 /* per-row flags in sr_row_params.flags */
 enum {
-    SR_ROW_HAS_LOGIT_BIAS = 1u << 0 /* LogitBias.Count > 0: selects the full-vocabulary path even when
-                                       every id is out of range (Sampler.cs:27,38)                      */
+    SR_ROW_HAS_LOGIT_BIAS = 1u << 0, /* LogitBias.Count > 0: selects the full-vocabulary path even when
+                                        every id is out of range (Sampler.cs:27,38)                      */
+    SR_ROW_DRAFT_FROM_LOOKUP = 1u << 1 /* sr_spec_verify_launch: the row's draft tokens came from prompt lookup
+                                          (usedPld, SpeculativeDecoder.cs:488-501): there are no draft
+                                          distributions, the accept rule is px >= spec_draft_p_min or the
+                                          draft is the argmax, a rejection draws from p (:538-552), whatever
+                                          spec_draft_p_min is; draft_probs_dev is not read for the row     */
 };
 
 /* bits reported per row in out_flags */
@@ -294,9 +299,10 @@ SR_API int sr_resample_residual(sr_ctx* ctx, const float* p, int32_t p_len, int6
  *   draft_probs_dev   [rows x n_draft x vocab]       q_i, as SampleWithDistribution left them (:509-513)
  *   draft_tokens_dev  [rows x n_draft]
  * The batch supplies the rows' parameters and n_draft+1 uniforms per row (accept draws in position
- * order, then the residual / bonus draw).  spec_draft_p_min in (0,1) selects the looser accept of
- * :546,552.  Outputs (DEVICE): out_accepted[rows]; out_tokens[rows x (n_draft+1)] = accepted drafts
- * followed by the correction or bonus token, the rest -1.  A draft id outside [0, vocab) ends its row at that
+ * order, then the residual / bonus draw).  spec_draft_p_min in (0,1), or SR_ROW_DRAFT_FROM_LOOKUP in the
+ * row's flags, selects the looser accept of :546,552; draft_probs_dev may be NULL when every row does.
+ * Outputs (DEVICE): out_accepted[rows]; out_tokens[rows x (n_draft+1)] = accepted drafts followed by the
+ * correction or bonus token, the rest -1.  A draft id outside [0, vocab) ends its row at that
  * position with -1 in place of the correction token (the managed loop throws IndexOutOfRangeException at
  * pDist[x_i], :536); out_accepted counts the drafts accepted before it.
  */

@@ -57,6 +57,9 @@ struct SamplingParams {
     std::map<int, float> LogitBias;
     std::vector<int> PreviousTokens;
     float SpecDraftPMin = 1.0f;
+    // not a field of the managed class: the step's `usedPld` (SpeculativeDecoder.cs:488-501), read beside the
+    // parameters by the accept loop (:538, :549)
+    bool SpecDraftFromLookup = false;
 
     bool HasHistoryPenalty() const
     {
@@ -189,7 +192,8 @@ private:
             row.presence_penalty = p.PresencePenalty;
             row.frequency_penalty = p.FrequencyPenalty;
             row.spec_draft_p_min = p.SpecDraftPMin;
-            row.flags = p.LogitBias.empty() ? 0u : (uint32_t)SR_ROW_HAS_LOGIT_BIAS;
+            row.flags = (p.LogitBias.empty() ? 0u : (uint32_t)SR_ROW_HAS_LOGIT_BIAS) |
+                        (p.SpecDraftFromLookup ? (uint32_t)SR_ROW_DRAFT_FROM_LOOKUP : 0u);
             h.assign(p.PreviousTokens.begin(), p.PreviousTokens.end());
             for (const auto& kv : p.LogitBias) { bi.push_back(kv.first); bv.push_back(kv.second); }
             hist_off[1] = (int32_t)h.size();

@@ -38,6 +38,7 @@ SR_ERR_NO_DEVICE = 6
 SR_DTYPE_F32 = 0
 SR_DTYPE_BF16 = 1
 SR_ROW_HAS_LOGIT_BIAS = 1
+SR_ROW_DRAFT_FROM_LOOKUP = 2
 SR_OUT_PATH_GREEDY = 1
 SR_OUT_PATH_TOPK_FAST = 2
 SR_OUT_PATH_FULL_VOCAB = 4
@@ -94,6 +95,9 @@ class SamplingParams:
     LogitBias: Optional[Dict[int, float]] = None
     PreviousTokens: Optional[Sequence[int]] = None
     SpecDraftPMin: float = 1.0
+    # not a field of the reference's SamplingParams: the step's `usedPld` (SpeculativeDecoder.cs:488-501), which the
+    # accept loop reads beside them (:538, :549)
+    SpecDraftFromLookup: bool = False
 
     @property
     def HasHistoryPenalty(self) -> bool:
@@ -102,7 +106,8 @@ class SamplingParams:
     def to_row(self) -> RowParams:
         return RowParams(self.Temperature, self.TopK, self.TopP, self.MinP, self.RepetitionPenalty,
                          self.RepeatLastN, self.PresencePenalty, self.FrequencyPenalty, self.SpecDraftPMin,
-                         SR_ROW_HAS_LOGIT_BIAS if self.LogitBias else 0)
+                         (SR_ROW_HAS_LOGIT_BIAS if self.LogitBias else 0)
+                         | (SR_ROW_DRAFT_FROM_LOOKUP if self.SpecDraftFromLookup else 0))
 
 
 _lib = None
@@ -498,7 +503,8 @@ class SamplerContext:
         """Async: sr_spec_verify_launch over device tensors (target [rows, L+1, V], q [rows, L, V], tokens [rows, L])."""
         L = target_logits.shape[1] - 1
         self._check(self.L.sr_spec_verify_launch(
-            self.h, batch.h, C.c_void_p(target_logits.data_ptr()), C.c_void_p(draft_probs.data_ptr()),
+            self.h, batch.h, C.c_void_p(target_logits.data_ptr()),
+            C.c_void_p(None if draft_probs is None else draft_probs.data_ptr()),
             C.c_void_p(draft_tokens.data_ptr()), L, C.c_void_p(out_accepted.data_ptr()),
             C.c_void_p(out_tokens.data_ptr())))
 
@@ -538,7 +544,8 @@ class SamplerContext:
         toks = torch.empty((rows, L + 1), dtype=torch.int32, device=target_logits.device)
         try:
             self._check(self.L.sr_spec_verify_launch(
-                self.h, batch.h, C.c_void_p(target_logits.data_ptr()), C.c_void_p(draft_probs.data_ptr()),
+                self.h, batch.h, C.c_void_p(target_logits.data_ptr()),
+            C.c_void_p(None if draft_probs is None else draft_probs.data_ptr()),
                 C.c_void_p(draft_tokens.data_ptr()), L, C.c_void_p(acc.data_ptr()), C.c_void_p(toks.data_ptr())))
             self.synchronize()
         finally:

@@ -1163,6 +1163,8 @@ int sr_argmax_rows_launch(sr_ctx* ctx, const void* logits_dev, int dtype, int32_
 }
 
 static_assert(SR_ARGMAX_STATIC_ROWS == SR_ARGMAX_NOALLOC_MAX_ROWS, "the header states the size of the static scratch");
+static_assert(SR_ROWBIT_HAS_LOGIT_BIAS == SR_ROW_HAS_LOGIT_BIAS && SR_ROWBIT_DRAFT_FROM_LOOKUP == SR_ROW_DRAFT_FROM_LOOKUP,
+              "the kernels' names for the public flag bits");
 
 int sr_argmax_rows_launch_noalloc(sr_ctx* ctx, const void* logits_dev, int dtype, int32_t rows, int32_t vocab,
                                   int64_t row_stride_elems, int32_t* out_idx_dev, float* out_val_dev)

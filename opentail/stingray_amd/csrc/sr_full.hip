@@ -1231,7 +1231,8 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
     const float* lg = a.target_logits + (size_t)row * (L + 1) * n;
     const double* u = a.uniforms + (size_t)row * a.uniforms_per_row;
     int* out = a.out_tokens + (size_t)row * (L + 1);
-    const bool true_spec = !(rd.p_min > 0.0f && rd.p_min < 1.0f);  // SpeculativeDecoder.cs:192
+    // SpeculativeDecoder.cs:192 and :538, :549 (`_trueSpecSampling && !usedPld`)
+    const bool true_spec = !(rd.p_min > 0.0f && rd.p_min < 1.0f) && (rd.flags & SR_ROWBIT_DRAFT_FROM_LOOKUP) == 0u;
     for (int i = threadIdx.x; i <= L; i += kT) out[i] = -1;
     __syncthreads();
     int accepted = 0, udraws = 0, correction = -1;

@@ -397,8 +397,16 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
     if (!ctx || !b) return SR_ERR_NULL_ARGUMENT;
     if (b->rows == 0) return SR_OK;
     if (n_draft < 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_spec_verify_launch: negative draft length");
-    if (!target_logits_dev || !out_accepted_dev || !out_tokens_dev || (n_draft > 0 && (!draft_probs_dev || !draft_tokens_dev)))
+    if (!target_logits_dev || !out_accepted_dev || !out_tokens_dev || (n_draft > 0 && !draft_tokens_dev))
         return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_spec_verify_launch: null tensor");
+    if (n_draft > 0 && !draft_probs_dev) {
+        // only rows under the ratio test read q (SpeculativeDecoder.cs:538-543)
+        for (int r = 0; r < b->rows; r++) {
+            const SrRow& d = b->h_rows[(size_t)r];
+            if (!(d.p_min > 0.0f && d.p_min < 1.0f) && !(d.flags & SR_ROW_DRAFT_FROM_LOOKUP))
+                return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_spec_verify_launch: a row under the ratio test needs the draft distributions");
+        }
+    }
     if (b->vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_spec_verify_launch: empty vocabulary");
     if (b->upr < n_draft + 1) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_spec_verify_launch: needs n_draft + 1 uniforms per row");
     if (b->has_mask) return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_spec_verify_launch: allow-masks are not part of speculative verification");

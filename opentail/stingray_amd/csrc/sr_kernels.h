@@ -10,6 +10,9 @@
 #define SR_KFLAG_FULL (1u << 2)
 #define SR_KFLAG_DEGENERATE (1u << 3)
 #define SR_KFLAG_UNSUPPORTED (1u << 31)
+// the public bits of SrRow.flags as device code sees them (the public header is not included on the device side)
+#define SR_ROWBIT_HAS_LOGIT_BIAS (1u << 0)
+#define SR_ROWBIT_DRAFT_FROM_LOOKUP (1u << 1)
 // internal bit of SrRow.flags: the row has a history and at least one active penalty
 #define SR_ROWFLAG_HAS_PENALTY (1u << 8)
 // internal bit: the penalties can only lower a logit, so the scan skips the history ids (scan mask) and

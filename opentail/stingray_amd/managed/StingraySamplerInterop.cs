@@ -12,7 +12,7 @@ internal struct SrRowParams            // sr_row_params
 {
     public float Temperature; public int TopK; public float TopP; public float MinP;
     public float RepetitionPenalty; public int RepeatLastN; public float PresencePenalty; public float FrequencyPenalty;
-    public float SpecDraftPMin; public uint Flags;      // bit 0: LogitBias.Count > 0
+    public float SpecDraftPMin; public uint Flags;      // bit 0: LogitBias.Count > 0; bit 1: drafts from prompt lookup
 }
 
 internal static unsafe partial class StingraySamplerInterop

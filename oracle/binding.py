@@ -40,6 +40,7 @@ class CParams(C.Structure):
         ("bias_vals", C.POINTER(C.c_float)),
         ("n_bias", C.c_int32),
         ("spec_draft_p_min", C.c_float),
+        ("draft_from_lookup", C.c_int32),
     ]
 
 
@@ -69,6 +70,7 @@ class Params:
     previous_tokens: Optional[Sequence[int]] = None
     logit_bias: Optional[dict] = None
     spec_draft_p_min: float = 1.0
+    draft_from_lookup: bool = False
     _keep: list = field(default_factory=list, repr=False)
 
     def to_c(self) -> CParams:
@@ -82,6 +84,7 @@ class Params:
         cp.presence_penalty = self.presence_penalty
         cp.frequency_penalty = self.frequency_penalty
         cp.spec_draft_p_min = self.spec_draft_p_min
+        cp.draft_from_lookup = 1 if self.draft_from_lookup else 0
         self._keep = []
         if self.previous_tokens is not None and len(self.previous_tokens) > 0:
             prev = np.ascontiguousarray(np.asarray(self.previous_tokens, dtype=np.int32))

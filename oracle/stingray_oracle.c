@@ -222,6 +222,7 @@ void oracle_params_default(oracle_params* p)
     p->repetition_penalty = 1.0f;
     p->repeat_last_n = 64;
     p->spec_draft_p_min = 1.0f;
+    p->draft_from_lookup = 0;
 }
 
 static inline int has_history_penalty(const oracle_params* p) /* Sampler.cs:686 */
@@ -620,6 +621,8 @@ int32_t oracle_spec_verify_row(const float* target_logits, const float* draft_pr
 {
     /* SpeculativeDecoder.cs:192 */
     int true_spec = !(p->spec_draft_p_min > 0.0f && p->spec_draft_p_min < 1.0f);
+    /* :538, :549: `_trueSpecSampling && !usedPld` -- lookup drafts have no q, so they take the other rule */
+    if (p->draft_from_lookup) true_spec = 0;
     int32_t accepted = 0;
     int32_t correction = -1;
     for (int32_t i = 0; i < n_draft; i++) {

@@ -54,6 +54,8 @@ typedef struct oracle_params {
     const float* bias_vals;     /*   every id is out of range (SamplerTests.cs:215-216)           */
     int32_t n_bias;
     float spec_draft_p_min;     /* 1.0 */
+    int32_t draft_from_lookup;  /* the step's draft tokens came from prompt lookup: no draft distributions exist
+                                   (usedPld, SpeculativeDecoder.cs:488-501, 538, 549) */
 } oracle_params;
 
 void oracle_params_default(oracle_params* p);

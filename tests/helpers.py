@@ -12,7 +12,7 @@ def to_oracle(p: SamplingParams) -> orc.Params:
                       repetition_penalty=p.RepetitionPenalty, repeat_last_n=p.RepeatLastN,
                       presence_penalty=p.PresencePenalty, frequency_penalty=p.FrequencyPenalty,
                       previous_tokens=p.PreviousTokens, logit_bias=p.LogitBias,
-                      spec_draft_p_min=p.SpecDraftPMin)
+                      spec_draft_p_min=p.SpecDraftPMin, draft_from_lookup=p.SpecDraftFromLookup)
 
 
 def oracle_tokens(logits: np.ndarray, params, uniforms, allow_mask=None, mask_active=None) -> np.ndarray:

@@ -234,6 +234,34 @@ def test_speculative_verification_rows(ctx):
     _check_spec(ctx, t, q, k, p3, u)
 
 
+def test_drafts_from_prompt_lookup_take_the_p_min_rule_whatever_p_min_is(ctx):
+    # usedPld (SpeculativeDecoder.cs:488-501, 538-552): no draft distributions exist; accept iff px >= SpecDraftPMin or the
+    # draft is the argmax, a rejection draws from p.  Rows of both kinds in one launch; then lookup rows alone with no q.
+    V, L = 20_000, 5
+    kinds = [SamplingParams(SpecDraftFromLookup=True),
+             SamplingParams(Temperature=0.7, TopK=40, TopP=0.95, SpecDraftFromLookup=True),
+             SamplingParams(Temperature=0.8, SpecDraftPMin=0.05, SpecDraftFromLookup=True),
+             SamplingParams(Temperature=0.0, SpecDraftFromLookup=True),
+             SamplingParams(Temperature=0.9, TopP=0.9)]
+    params = [kinds[r % len(kinds)] for r in range(10)]
+    t, q, k, u = _spec_case(10, L, V, params, 5, True)
+    rng = np.random.default_rng(6)
+    for r in range(10):                                           # lookup drafts: a mix of likely and arbitrary continuations
+        if params[r].SpecDraftFromLookup:
+            q[r] = np.nan                                         # must not be read
+            for i in range(L):
+                k[r, i] = int(np.argmax(t[r, i])) if rng.random() < 0.6 else int(rng.integers(0, V))
+    _check_spec(ctx, t, q, k, params, u)
+    only = [p for p in params if p.SpecDraftFromLookup]
+    idx = [r for r, p in enumerate(params) if p.SpecDraftFromLookup]
+    acc, out = ctx.spec_verify(_cuda(t[idx]), None, _cuda(k[idx]), only, u[idx])
+    for j, r in enumerate(idx):
+        wa, wt = orc.spec_verify_row(t[r], q[r], k[r], to_oracle(params[r]), orc.Rng(replay=u[r]))
+        assert acc[j] == wa and list(out[j][: wa + 1]) == list(wt), r
+    with pytest.raises(TypeError):                                # a row under the ratio test needs q (a null argument)
+        ctx.spec_verify(_cuda(t), None, _cuda(k), params, u)
+
+
 def test_draft_ids_outside_the_vocabulary_end_their_row(ctx):
     # SpeculativeDecoder.cs:536 indexes pDist[x_i]: an id outside the vocabulary throws there.  The device never
     # dereferences it: the row ends at that position with -1 in place of the correction token.

@@ -235,6 +235,19 @@ def test_spec_accept_rule_closed_forms():
     assert orc.spec_verify_row(tl, q1, [2], pm, Rng(replay=[0.5]))[0] == 0   # .3 < .35, argmax is 3
     assert orc.spec_verify_row(tl, q1, [3], pm, Rng(replay=[0.5]))[0] == 1
     assert V == 4
+    # drafts from prompt lookup (usedPld, SpeculativeDecoder.cs:538-552): the p-min rule and a draw from p itself, also
+    # with the default SpecDraftPMin = 1 that selects the ratio test otherwise; q is never read, one draw on a rejection
+    pl = Params(draft_from_lookup=True)
+    qbad = np.full((1, 4), np.nan, dtype=np.float32)
+    r = Rng(replay=[0.55, 0.9])
+    acc, toks = orc.spec_verify_row(tl, qbad, [2], pl, r)           # .3 < 1 and the argmax is 3: rejected,
+    assert acc == 0 and list(toks) == [2] and r.draws == 1          # p: cum .1,.3,.6 -> u=.55 -> token 2 (not removed)
+    r = Rng(replay=[0.6])
+    acc, toks = orc.spec_verify_row(tl, qbad, [3], pl, r)           # the argmax is accepted; bonus from the uniform row
+    assert acc == 1 and list(toks) == [3, 2] and r.draws == 1
+    pl2 = Params(draft_from_lookup=True, spec_draft_p_min=0.25)
+    assert orc.spec_verify_row(tl, qbad, [2], pl2, Rng(replay=[0.5]))[0] == 1   # .3 >= .25
+    assert orc.spec_verify_row(tl, qbad, [1], pl2, Rng(replay=[0.5]))[0] == 0   # .2 < .25, not the argmax
     # a draft id outside the vocabulary: pDist[x_i] throws in the managed loop (SpeculativeDecoder.cs:536); the
     # restatement ends the row there with -1 and draws nothing
     for bad in (-1, 4, 2 ** 31 - 1):
