@@ -982,6 +982,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.items = b->d_sched.as<int4>() + b->n_workers;
         a.n_workers = b->n_workers;
         a.own_rows = b->own_rows ? 1 : 0;
+        a.kept = (b->own_rows && b->n_workers <= ctx->cu_count) ? 1 : 0;
         a.n_items = b->n_items;
         a.sel_list = b->d_sel_list.as<int32_t>();
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));

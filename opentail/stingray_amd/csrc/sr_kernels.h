@@ -37,6 +37,7 @@ struct SrTopkArgs {
     const int4* progs;
     int32_t n_workers, n_items;
     int32_t own_rows;        // every worker's program is one whole row (all its chunks, then its tail)
+    int32_t kept;            // ... and there is at most one worker per compute unit
     const int32_t* sel_list; // [n_rows] batch row of every launch slot
     const SrRow* rows;
     const SrEdit* edits;

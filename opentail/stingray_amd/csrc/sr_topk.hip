@@ -400,17 +400,26 @@ __device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
 // ---- the row tail ----------------------------------------------------------------------------------
 // Called by every thread of the tail workgroup of a row once all chunks of the row have been counted in.
 // slot = position of the row in this launch.
-template <int EPV, int kVec, typename Early, typename Late>
+// What a worker that streams all chunks of its own row keeps of them in registers instead of writing it out: per
+// chunk (at most kKeptChunks) the thread's four group maxima, second maxima and packed positions.  The waves' shares
+// of the row's bound and their largest kept elements lie in sm.hist, two words per (chunk, wave).
+constexpr int kKeptChunks = 4;
+struct KeptGroups {
+    float4 g1[kKeptChunks], g2[kKeptChunks];
+    uint32_t gp[kKeptChunks];
+};
+
+template <int EPV, int kVec, bool kKept, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
                                                 bool force_exact, float inv_temp, float* mx0_out, float* bscale_out,
-                                                float* bound_out, bool* binned, Early&& early, Late&& late,
-                                                TopkSmem& sm);
+                                                float* bound_out, bool* binned, const KeptGroups& kept, Early&& early,
+                                                Late&& late, TopkSmem& sm);
 
 // force_exact: the chunk results of the row are not used, the candidates come from the logits themselves (what a row
 // whose candidates overflow the lists falls back to, and a row whose chunks were not handed over in time).
-template <int EPV, int kVec>
+template <int EPV, int kVec, bool kKept>
 __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool force_exact,
-                                              TopkSmem& sm)
+                                              const KeptGroups& kept, TopkSmem& sm)
 {
     const int tid = threadIdx.x;
     const unsigned long long* cand = a.cand + (size_t)slot * kRowCap;
@@ -446,8 +455,8 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     const bool want_bins = rd.path == SR_PATH_TOPK && (!use_edits || hist_regs);
     bool binned = false;
     float mx0 = 0.0f, bscale0 = -56.0f, bound0 = 0.0f;
-    const int n_c = build_candidates<EPV, kVec>(
-        a, slot, row, rd, want_bins, force_exact, inv_temp, &mx0, &bscale0, &bound0, &binned,
+    const int n_c = build_candidates<EPV, kVec, kKept>(
+        a, slot, row, rd, want_bins, force_exact, inv_temp, &mx0, &bscale0, &bound0, &binned, kept,
         [&]() SR_INL {
 #pragma unroll
             for (int r = 0; r < kHistRegs; r++) {
@@ -1055,11 +1064,11 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 // force_exact, and any row whose candidates overflow the lists: the row's sel-th largest kept element is found by a
 // radix select over the logits themselves, and the candidates are exactly the sel largest in (value desc, index asc)
 // order.  Slow (several passes over the row), exact for any data, and independent of the chunk results.
-template <int EPV, int kVec, typename Early, typename Late>
+template <int EPV, int kVec, bool kKept, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
                                                 bool force_exact, float inv_temp, float* mx0_out, float* bscale_out,
-                                                float* bound_out, bool* binned, Early&& early, Late&& late,
-                                                TopkSmem& sm)
+                                                float* bound_out, bool* binned, const KeptGroups& kept, Early&& early,
+                                                Late&& late, TopkSmem& sm)
 {
     *binned = false;
     *mx0_out = 0.0f;
@@ -1199,22 +1208,35 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         // maximum, and of the groups that reach it the lowest position of their (first) largest element
         early();
         uint32_t km = 0u;
-        for (int c = 0; c < S; c++) {
-            const float4 m = gm_load(c);
+        auto fold_max = [&](const float4& m) SR_INL {
             km = max(max(max(km, sr_okey(m.x)), max(sr_okey(m.y), sr_okey(m.z))), sr_okey(m.w));
+        };
+        if constexpr (kKept) {
+#pragma unroll
+            for (int c = 0; c < kKeptChunks; c++)
+                if (c < S) fold_max(kept.g1[c]);
+        } else {
+            for (int c = 0; c < S; c++) fold_max(gm_load(c));
         }
         late();
         km = block_max_u32(km, sm);
         const bool any = km > kKeyNegInf;
         int best = 0x7fffffff;
-        for (int c = 0; c < S && any; c++) {
-            const float4 m = gm_load(c);
-            if (max(max(sr_okey(m.x), sr_okey(m.y)), max(sr_okey(m.z), sr_okey(m.w))) != km) continue;
-            const uint32_t gp = a.gpos[((size_t)slot * S + c) * kThreads + tid];
+        auto fold_best = [&](int c, const float4& m, auto&& gpos_of) SR_INL {
+            if (max(max(sr_okey(m.x), sr_okey(m.y)), max(sr_okey(m.z), sr_okey(m.w))) != km) return;
+            const uint32_t gp = gpos_of();
             const float m1[4] = {m.x, m.y, m.z, m.w};
 #pragma unroll
             for (int g = 0; g < 4; g++)
                 if (sr_okey(m1[g]) == km) best = min(best, idx_of(c, g, (gp >> (8 * g)) & 0xffu));
+        };
+        if constexpr (kKept) {
+#pragma unroll
+            for (int c = 0; c < kKeptChunks; c++)
+                if (c < S && any) fold_best(c, kept.g1[c], [&]() SR_INL { return kept.gp[c]; });
+        } else {
+            for (int c = 0; c < S && any; c++)
+                fold_best(c, gm_load(c), [&]() SR_INL { return a.gpos[((size_t)slot * S + c) * kThreads + tid]; });
         }
         best = block_min_i32(best, sm);
         if (tid == 0 && any) {
@@ -1226,7 +1248,11 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     }
     float4 gmr[kGmRegs];
 #pragma unroll
-    for (int c = 0; c < kGmRegs; c++) gmr[c] = c < S ? gm_load(c) : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+    for (int c = 0; c < kGmRegs; c++) {
+        if constexpr (kKept) gmr[c] = c < S ? kept.g1[c] : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+        else gmr[c] = c < S ? gm_load(c) : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+    }
+    static_assert(kGmRegs == kKeptChunks, "kept chunks fill the direct path's registers");
     // with few chunks the second maxima and the positions of the maxima come along in the same batch of loads
     constexpr int kG2Regs = 4;
     const bool direct = S <= kG2Regs;  // a group whose second largest is below the bound hands over its largest directly
@@ -1235,8 +1261,13 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 #pragma unroll
     for (int c = 0; c < kG2Regs; c++) {
         const bool in = direct && c < S;
-        g2r[c] = in ? a.gmax2[((size_t)slot * S + c) * kThreads + tid] : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
-        gpr[c] = in ? a.gpos[((size_t)slot * S + c) * kThreads + tid] : 0u;
+        if constexpr (kKept) {
+            g2r[c] = in ? kept.g2[c] : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+            gpr[c] = in ? kept.gp[c] : 0u;
+        } else {
+            g2r[c] = in ? a.gmax2[((size_t)slot * S + c) * kThreads + tid] : make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+            gpr[c] = in ? a.gpos[((size_t)slot * S + c) * kThreads + tid] : 0u;
+        }
     }
     early();
     auto each_gm = [&](auto&& f) SR_INL {
@@ -1338,11 +1369,18 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     {
         const int nb = S * kWaves;
         uint32_t k = 0xffffffffu, km = 0u;
-        const uint2* gb = (const uint2*)a.gbound + (size_t)slot * nb;
-        for (int i = lane; i < nb; i += SR_WAVE) {
-            const uint2 b = gb[i];
-            k = min(k, b.x);
-            km = max(km, b.y);
+        if constexpr (kKept) {
+            if (lane < nb) {  // nb <= kKeptChunks * kWaves
+                k = sm.hist[2 * lane];
+                km = sm.hist[2 * lane + 1];
+            }
+        } else {
+            const uint2* gb = (const uint2*)a.gbound + (size_t)slot * nb;
+            for (int i = lane; i < nb; i += SR_WAVE) {
+                const uint2 b = gb[i];
+                k = min(k, b.x);
+                km = max(km, b.y);
+            }
         }
         k = sr_wave_min_u32(k);
         km = sr_wave_max_u32(km);
@@ -1496,8 +1534,13 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 // groups.  When a vector has been folded, the load of the same vector of the worker's NEXT chunk is issued into its
 // registers, so every thread has up to kVec loads in flight from its first chunk to its last, and the stores, the
 // per-wave bound and the hand-off of a chunk run under the loads of the next one.
-template <int EPV, int kVec, int kWindow>
-__global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
+//
+// kKept: every worker streams all chunks (at most kKeptChunks) of the one row it finishes and there is at most one
+// worker per compute unit.  Nothing is handed over then, so nothing is written out: the group results of all chunks
+// stay in the thread's registers (the workgroup has the register file of its compute unit to itself) and the waves'
+// shares of the bound go through LDS.
+template <int EPV, int kVec, int kWindow, bool kKept>
+__global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArgs a)
 {
     __shared__ TopkSmem sm;
     using VO = VecOps<EPV>;
@@ -1556,6 +1599,15 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
         return __builtin_nontemporal_load((const u32x4*)((const char*)g.cp + off));
     };
 
+    KeptGroups kept;
+    if constexpr (kKept) {
+#pragma unroll
+        for (int c = 0; c < kKeptChunks; c++) {
+            kept.g1[c] = make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
+            kept.g2[c] = kept.g1[c];
+            kept.gp[c] = 0u;
+        }
+    }
     if (n_items > 0) {
         const i32x4 info = q[0];  // (chunk | launch slot of the row, batch row, scan-mask row, sel)
         Geom cur = geom(info);
@@ -1640,10 +1692,22 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 kw0 = mw[0]; kw1 = mw[1]; kw2 = mw[2];
             }
             const uint32_t gpk = (uint32_t)gp1[0] | ((uint32_t)gp1[1] << 8) | ((uint32_t)gp1[2] << 16) | ((uint32_t)gp1[3] << 24);
-            const size_t go = ((size_t)cur.slot * S + cur.c) * kThreads + tid;
-            sr_store_agent_f4(a.gmax + go, gm1[0], gm1[1], gm1[2], gm1[3]);
-            sr_store_agent_f4(a.gmax2 + go, gm2[0], gm2[1], gm2[2], gm2[3]);
-            __hip_atomic_store(a.gpos + go, gpk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if constexpr (kKept) {
+#pragma unroll
+                for (int c = 0; c < kKeptChunks; c++) {
+                    const bool on = cur.c == c;
+                    kept.g1[c].x = on ? gm1[0] : kept.g1[c].x; kept.g1[c].y = on ? gm1[1] : kept.g1[c].y;
+                    kept.g1[c].z = on ? gm1[2] : kept.g1[c].z; kept.g1[c].w = on ? gm1[3] : kept.g1[c].w;
+                    kept.g2[c].x = on ? gm2[0] : kept.g2[c].x; kept.g2[c].y = on ? gm2[1] : kept.g2[c].y;
+                    kept.g2[c].z = on ? gm2[2] : kept.g2[c].z; kept.g2[c].w = on ? gm2[3] : kept.g2[c].w;
+                    kept.gp[c] = on ? gpk : kept.gp[c];
+                }
+            } else {
+                const size_t go = ((size_t)cur.slot * S + cur.c) * kThreads + tid;
+                sr_store_agent_f4(a.gmax + go, gm1[0], gm1[1], gm1[2], gm1[3]);
+                sr_store_agent_f4(a.gmax2 + go, gm2[0], gm2[1], gm2[2], gm2[3]);
+                __hip_atomic_store(a.gpos + go, gpk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             // The wave's share of the row's bound: a value, to 16 bits and rounded down, with at least
             // ceil(sel / (chunks x 8)) of the wave's 256 group maxima at or above it (found bit by bit with ballots).
             // The smallest of all the row's waves' values then has at least sel group maxima at or above it.
@@ -1661,9 +1725,15 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
                 // ... and the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
                 const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(gm1[0], gm1[1]), fmaxf(gm1[2], gm1[3]))));
                 if (lane == 0) {
-                    uint32_t* gb = a.gbound + (((size_t)cur.slot * S + cur.c) * kWaves + (tid >> 6)) * 2;
-                    __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(gb + 1, wmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if constexpr (kKept) {
+                        const int w = (min(cur.c, kKeptChunks - 1) * kWaves + (tid >> 6)) * 2;
+                        sm.hist[w] = K;
+                        sm.hist[w + 1] = wmax;
+                    } else {
+                        uint32_t* gb = a.gbound + (((size_t)cur.slot * S + cur.c) * kWaves + (tid >> 6)) * 2;
+                        __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(gb + 1, wmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
             }
 #ifdef SR_PROFILE
@@ -1673,7 +1743,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #endif
             // hand the chunk over: this wave's write-through stores (and, older than them, the loads of the next
             // chunk) have completed, the workgroup meets, then the chunk is counted in
-            if (!own_row) {
+            if (!kKept && !own_row) {
                 sr_drain_stores();
                 __syncthreads();
                 if (tid == 0) __hip_atomic_fetch_add(&done[cur.slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1699,22 +1769,30 @@ __global__ __launch_bounds__(kThreads, 4) void k_topk_rows(SrTopkArgs a)
 #endif
     // The row's other chunks are in the hands of workers that are running; they are nearly always in already.
     // Should they not come (the wait is bounded), the row is selected from its logits alone.
-    if (own_row) sr_drain_stores();  // every wave's own stores; the barrier below joins them
-    if (tid == 0) {
-        uint32_t ok = own_row && a.spin_limit != 0u ? 1u : 0u;
-        for (uint32_t it = 0; !own_row && it < a.spin_limit; it++) {
-            if (sr_load_agent(&done[tslot]) == (uint32_t)S) { ok = 1u; break; }
-            __builtin_amdgcn_s_sleep(2);
+    bool handed_over;
+    if constexpr (kKept) {
+        // the row's results are in this workgroup's registers and LDS; a worker whose program is not of that kind (the
+        // host writes none for this kernel) selects its row from the logits alone
+        __syncthreads();  // the waves' shares of the bound
+        handed_over = own_row && S <= kKeptChunks && a.spin_limit != 0u;
+    } else {
+        if (own_row) sr_drain_stores();  // every wave's own stores; the barrier below joins them
+        if (tid == 0) {
+            uint32_t ok = own_row && a.spin_limit != 0u ? 1u : 0u;
+            for (uint32_t it = 0; !own_row && it < a.spin_limit; it++) {
+                if (sr_load_agent(&done[tslot]) == (uint32_t)S) { ok = 1u; break; }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            // the chunks' results were written through to L2: drop what this CU's L1 may hold of an earlier launch
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            sm.bcast[7] = ok;
         }
-        // the chunks' results were written through to L2: drop what this CU's L1 may hold of an earlier launch
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        sm.bcast[7] = ok;
+        __syncthreads();
+        handed_over = sm.bcast[7] != 0u;
     }
-    __syncthreads();
-    const bool handed_over = sm.bcast[7] != 0u;
     SR_PROF(ap, 4);
     __builtin_amdgcn_s_setprio(3);  // the tail is the longer dependent chain: its waves go first
-    topk_row_tail<EPV, kVec>(ap, tslot, trow, trd, !handed_over, sm);
+    topk_row_tail<EPV, kVec, kKept>(ap, tslot, trow, trd, !handed_over, kept, sm);
     SR_PROF(ap, 15);
 }
 
@@ -1894,12 +1972,16 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
     if (n_rows <= 0) return hipSuccess;
     dim3 grid((unsigned)a.n_workers), block(kThreads);
     // workers with a row of their own are few per compute unit: each keeps more of its vectors in flight
+    // ... and where there is at most one of them per compute unit, the results of its chunks stay in its registers
+    const bool kept = a.own_rows && a.kept && a.chunks <= kKeptChunks;
     if (a.dtype == 1) {
-        if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW_OWN>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW>), grid, block, 0, stream, a);
+        if (kept) hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW_KEPT, true>), grid, block, 0, stream, a);
+        else if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW_OWN, false>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW, false>), grid, block, 0, stream, a);
     } else {
-        if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW_OWN>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW>), grid, block, 0, stream, a);
+        if (kept) hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW_KEPT, true>), grid, block, 0, stream, a);
+        else if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW_OWN, false>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW, false>), grid, block, 0, stream, a);
     }
     return hipGetLastError();
 }
