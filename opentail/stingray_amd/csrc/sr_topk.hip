@@ -408,6 +408,38 @@ struct KeptGroups {
     float4 g1[kKeptChunks], g2[kKeptChunks];
     uint32_t gp[kKeptChunks];
 };
+// ... and what it fetches of its row's history before it starts to stream: the thread's history ids with their
+// counts, and their (masked) logits
+struct KeptHistory {
+    SrEdit hee[kHistRegs];
+    float hx[kHistRegs];
+};
+// The masked logit of one token id of a row.
+__device__ __forceinline__ float row_logit(const SrTopkArgs& a, int row, const SrRow& rd, int id)
+{
+    const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * (a.dtype == 1 ? 2 : 4);
+    float x = (a.dtype == 1) ? sr_bf16_to_f32(((const uint16_t*)rowp)[id]) : ((const float*)rowp)[id];
+    if (rd.mask_row >= 0 && !mask_bit(a.mask + (size_t)rd.mask_row * a.mask_stride, id)) x = SR_NEG_INF;
+    return x;
+}
+// A row descriptor read through the constant address space: one scalar load for the whole workgroup, in nobody's way
+// (the descriptors were written before the launch).
+__device__ __forceinline__ SrRow load_row_uniform(const SrRow* p)
+{
+    static_assert(sizeof(SrRow) == 64, "four 16-byte loads");
+    typedef int __attribute__((ext_vector_type(4))) i32x4;
+    typedef const i32x4 __attribute__((address_space(4))) const_i32x4;
+    const const_i32x4* q = (const const_i32x4*)(uintptr_t)p;
+    union { SrRow r; i32x4 v[4]; } u;
+    u.v[0] = q[0]; u.v[1] = q[1]; u.v[2] = q[2]; u.v[3] = q[3];
+    return u.r;
+}
+// Whether the row tail holds the row's history ids in registers (penalties that only lower, few enough ids).
+__device__ __forceinline__ bool row_history_in_registers(const SrRow& rd)
+{
+    const bool use_edits = (rd.flags & kRowHasPenalty) != 0u && rd.edit_cnt > 0;
+    return use_edits && (rd.flags & kRowHistExcl) != 0u && rd.path == SR_PATH_TOPK && rd.edit_cnt <= kHistRegs * kThreads;
+}
 
 template <int EPV, int kVec, bool kKept, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
@@ -419,7 +451,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 // whose candidates overflow the lists falls back to, and a row whose chunks were not handed over in time).
 template <int EPV, int kVec, bool kKept>
 __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool force_exact,
-                                              const KeptGroups& kept, TopkSmem& sm)
+                                              const KeptGroups& kept, const KeptHistory& kept_hist, TopkSmem& sm)
 {
     const int tid = threadIdx.x;
     const unsigned long long* cand = a.cand + (size_t)slot * kRowCap;
@@ -445,11 +477,14 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 
     // The history ids and their logits are fetched behind the candidate builder's own loads, so that neither
     // waits for the other.
-    const bool hist_regs = excl && rd.path == SR_PATH_TOPK && ne <= kHistRegs * kThreads;
+    const bool hist_regs = row_history_in_registers(rd);
     SrEdit hee[kHistRegs];
     float hx[kHistRegs];
 #pragma unroll
-    for (int r = 0; r < kHistRegs; r++) { hee[r] = SrEdit{}; hx[r] = SR_NEG_INF; }
+    for (int r = 0; r < kHistRegs; r++) {
+        if constexpr (kKept) { hee[r] = kept_hist.hee[r]; hx[r] = kept_hist.hx[r]; }
+        else { hee[r] = SrEdit{}; hx[r] = SR_NEG_INF; }
+    }
     const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
     // rows without penalties that may raise a logit have their candidates binned while they are collected
     const bool want_bins = rd.path == SR_PATH_TOPK && (!use_edits || hist_regs);
@@ -458,17 +493,21 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     const int n_c = build_candidates<EPV, kVec, kKept>(
         a, slot, row, rd, want_bins, force_exact, inv_temp, &mx0, &bscale0, &bound0, &binned, kept,
         [&]() SR_INL {
+            if constexpr (!(kKept)) {
 #pragma unroll
-            for (int r = 0; r < kHistRegs; r++) {
-                const int e = r * kThreads + tid;
-                if (hist_regs && e < ne) hee[r] = ed[e];
+                for (int r = 0; r < kHistRegs; r++) {
+                    const int e = r * kThreads + tid;
+                    if (hist_regs && e < ne) hee[r] = ed[e];
+                }
             }
         },
         [&]() SR_INL {
+            if constexpr (!(kKept)) {
 #pragma unroll
-            for (int r = 0; r < kHistRegs; r++) {
-                const int e = r * kThreads + tid;
-                if (hist_regs && e < ne) hx[r] = hist_logit(hee[r].id);
+                for (int r = 0; r < kHistRegs; r++) {
+                    const int e = r * kThreads + tid;
+                    if (hist_regs && e < ne) hx[r] = hist_logit(hee[r].id);
+                }
             }
         },
         sm);
@@ -1402,11 +1441,12 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     }
     late();
     SR_PROF(a, 1);
+    uint32_t mq1 = 0u, base_a = 0u;
     if (direct) {
         // The thread's 16 groups as two bit masks -- largest element at or above the bound with the second largest
         // below it (handed over directly), second largest at or above it (listed, fetched below) --, one
         // reservation per wave and list, then every lane places its own.
-        uint32_t mq1 = 0u, mq2 = 0u;
+        uint32_t mq2 = 0u;
 #pragma unroll
         for (int c = 0; c < kG2Regs; c++) {
             if (c < S) {
@@ -1424,7 +1464,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         const int n_own = __popc(mq1) | (__popc(mq2) << 16);
         const int incl = sr_wave_incl_scan_i32(n_own);
         const int total = __builtin_amdgcn_readlane(incl, SR_WAVE - 1);
-        uint32_t base_a = 0u, base_l = 0u;
+        uint32_t base_l = 0u;
         if (lane == 0) {
             if ((total & 0xffff) > 0) base_a = atomicAdd(&sm.bcast[12], (uint32_t)(total & 0xffff));
             if ((total >> 16) > 0) base_l = atomicAdd(&sm.bcast[13], (uint32_t)(total >> 16));
@@ -1432,31 +1472,10 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         base_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)base_a) + (uint32_t)((incl - n_own) & 0xffff);
         base_l = (uint32_t)__builtin_amdgcn_readfirstlane((int)base_l) + (uint32_t)((incl - n_own) >> 16);
         // Every lane walks its own set bits, lowest first: the wave makes as many rounds as its busiest lane has
-        // groups to hand over (a handful) instead of one per group of the thread (16).  The group's largest
-        // element and its position are picked out of the thread's registers by the bit number.
-        // selects written as mask arithmetic: as conditionals the compiler may turn them into branches
-        auto sel = [](uint32_t x0, uint32_t x1, int bit) SR_INL -> uint32_t {
-            const uint32_t m = 0u - (uint32_t)(bit & 1);
-            return (x0 & ~m) | (x1 & m);
-        };
-        auto pick4 = [&](const float4& v, int g) SR_INL -> uint32_t {
-            return sel(sel(sr_f2u(v.x), sr_f2u(v.y), g), sel(sr_f2u(v.z), sr_f2u(v.w), g), g >> 1);
-        };
-        {
-            uint32_t m = mq1, pos = base_a;
-            while (__ballot(m != 0u) != 0ull) {
-                const bool on = m != 0u;
-                const int bit = on ? __ffs((int)m) - 1 : 0;
-                m &= m - 1u;
-                const int c = bit >> 2, g = bit & 3;
-                const float x = sr_u2f(sel(sel(pick4(gmr[0], g), pick4(gmr[1], g), c), sel(pick4(gmr[2], g), pick4(gmr[3], g), c), c >> 1));
-                const uint32_t gp = sel(sel(gpr[0], gpr[1], c), sel(gpr[2], gpr[3], c), c >> 1);
-                if (on) place(pos++, x, idx_of(c, g, (gp >> (8 * g)) & 0xffu));
-            }
-        }
+        // groups (a handful) instead of one per group of the thread (16).
         {
             uint32_t m = mq2, pos = base_l;
-            while (__ballot(m != 0u) != 0ull) {  // groups that may hold more than one: fetched below
+            while (__ballot(m != 0u) != 0ull) {
                 const bool on = m != 0u;
                 const int bit = on ? __ffs((int)m) - 1 : 0;
                 m &= m - 1u;
@@ -1475,9 +1494,32 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     __syncthreads();
     const int n_q = (int)sm.bcast[13];
     SR_PROF(a, 2);
+    // The largest element of every group with one element at or above the bound, picked out of the thread's registers
+    // by the bit number and handed over as it is.  Selects written as mask arithmetic: as conditionals the compiler
+    // may turn them into branches.
+    auto hand_over_direct = [&]() SR_INL {
+        auto sel = [](uint32_t x0, uint32_t x1, int bit) SR_INL -> uint32_t {
+            const uint32_t m = 0u - (uint32_t)(bit & 1);
+            return (x0 & ~m) | (x1 & m);
+        };
+        auto pick4 = [&](const float4& v, int g) SR_INL -> uint32_t {
+            return sel(sel(sr_f2u(v.x), sr_f2u(v.y), g), sel(sr_f2u(v.z), sr_f2u(v.w), g), g >> 1);
+        };
+        uint32_t m = mq1, pos = base_a;
+        while (__ballot(m != 0u) != 0ull) {
+            const bool on = m != 0u;
+            const int bit = on ? __ffs((int)m) - 1 : 0;
+            m &= m - 1u;
+            const int c = bit >> 2, g = bit & 3;
+            const float x = sr_u2f(sel(sel(pick4(gmr[0], g), pick4(gmr[1], g), c), sel(pick4(gmr[2], g), pick4(gmr[3], g), c), c >> 1));
+            const uint32_t gp = sel(sel(gpr[0], gpr[1], c), sel(gpr[2], gpr[3], c), c >> 1);
+            if (on) place(pos++, x, idx_of(c, g, (gp >> (8 * g)) & 0xffu));
+        }
+    };
     bool listed = false;
     if (n_q <= kQCap) {
         SR_PROF(a, 3);
+        hand_over_direct();  // (no bits set unless direct)
         gather(n_q, [&](float x) { return x >= tval; });
         listed = true;
     } else {
@@ -1600,12 +1642,30 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
     };
 
     KeptGroups kept;
+    KeptHistory kept_hist;
+    int trow = 0;
+    SrRow trd;
     if constexpr (kKept) {
 #pragma unroll
         for (int c = 0; c < kKeptChunks; c++) {
             kept.g1[c] = make_float4(SR_NEG_INF, SR_NEG_INF, SR_NEG_INF, SR_NEG_INF);
             kept.g2[c] = kept.g1[c];
             kept.gp[c] = 0u;
+        }
+        // the row to finish is known from the start: its descriptor, and the history ids with their logits, are
+        // fetched now and wait in registers while the row streams
+        if (prog.z >= 0) {
+            typedef const int __attribute__((address_space(4))) const_i32;
+            trow = ((const_i32*)(uintptr_t)a.sel_list)[prog.z];
+            trd = load_row_uniform(a.rows + trow);
+            const bool hist_regs = row_history_in_registers(trd);
+#pragma unroll
+            for (int r = 0; r < kHistRegs; r++) {
+                const int e = r * kThreads + tid;
+                const bool in = hist_regs && e < trd.edit_cnt;
+                kept_hist.hee[r] = in ? a.edits[trd.edit_off + e] : SrEdit{};
+                kept_hist.hx[r] = in ? row_logit(a, trow, trd, kept_hist.hee[r].id) : SR_NEG_INF;
+            }
         }
     }
     if (n_items > 0) {
@@ -1758,8 +1818,10 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
 
     // ---- the row tail
     const int tslot = prog.z;
-    const int trow = a.sel_list[tslot];
-    const SrRow trd = a.rows[trow];
+    if constexpr (!kKept) {
+        trow = a.sel_list[tslot];
+        trd = a.rows[trow];
+    }
 #ifdef SR_PROFILE
     SrTopkArgs ap = a;
     if (a.prof) ap.prof = a.prof + ((size_t)a.n_items + (size_t)tslot) * 16;
@@ -1792,7 +1854,7 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
     }
     SR_PROF(ap, 4);
     __builtin_amdgcn_s_setprio(3);  // the tail is the longer dependent chain: its waves go first
-    topk_row_tail<EPV, kVec, kKept>(ap, tslot, trow, trd, !handed_over, kept, sm);
+    topk_row_tail<EPV, kVec, kKept>(ap, tslot, trow, trd, !handed_over, kept, kept_hist, sm);
     SR_PROF(ap, 15);
 }
 
