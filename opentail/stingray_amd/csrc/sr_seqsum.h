@@ -271,6 +271,60 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
     }
 }
 
+// ---- one wave by itself --------------------------------------------------------------------------------
+// The running sum s of the wave's 64 x N terms (lane order = term order, N consecutive terms per lane), crossing after
+// crossing, with no barrier and no shared memory: what a short list needs (a row tail's few hundred probabilities).
+// When kSearch, stops at the first term at which the running sum reaches `target`: *found = its index (lane * N + j,
+// else -1) and the returned value is the running sum AT that term.  Terms past the end must be 0.  All 64 lanes call.
+template <int N, bool kSearch>
+__device__ __forceinline__ float sr_seq_wave(const float (&x)[N], float s, float target, int* found)
+{
+    const int lane = sr_lane();
+    int lstart = 0;  // lanes below are settled
+    *found = -1;
+    for (;;) {
+        uint32_t n_w;
+        int eb_w;
+        sr_split(s, &n_w, &eb_w);
+        SrInc m;
+        m.a0 = 0u; m.a1 = 0u;
+        if (lane >= lstart) m = sr_run_inc(x, eb_w);
+        const SrInc sc = sr_scan_inc<false>(m);
+        SrInc ex;
+        ex.a0 = __shfl_up(sc.a0, 1);
+        ex.a1 = __shfl_up(sc.a1, 1);
+        if (lane == 0) { ex.a0 = 0u; ex.a1 = 0u; }
+        const bool odd = (n_w & 1u) != 0u;
+        // exact integer state before / after this lane's run, valid while below 2^24
+        const uint32_t before = sr_sat_add(n_w, odd ? ex.a1 : ex.a0);
+        const uint32_t after = sr_sat_add(n_w, odd ? sc.a1 : sc.a0);
+        bool ev = after >= (1u << 24);
+        if (kSearch) ev = ev || sr_join(after, eb_w) >= target;
+        const unsigned long long evl = __ballot(ev && lane >= lstart);
+        if (!evl) {  // the rest of the wave stays in the binade and below the target
+            const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)(odd ? sc.a1 : sc.a0), SR_WAVE - 1);
+            return sr_join(n_w + tot, eb_w);
+        }
+        const int fl = (int)__ffsll((long long)evl) - 1;
+        // the first such lane's run, replayed with real float adds from its exact input (every lane replays its own)
+        float acc = sr_join(before, eb_w), hit = 0.0f;
+        int wj = -1;
+#pragma unroll
+        for (int j = 0; j < N; j++) {
+            acc = __fadd_rn(acc, x[j]);
+            if (kSearch && wj < 0 && acc >= target) { wj = j; hit = acc; }
+        }
+        wj = __builtin_amdgcn_readlane(wj, fl);
+        if (kSearch && wj >= 0) {
+            *found = fl * N + wj;
+            return sr_u2f((uint32_t)__builtin_amdgcn_readlane((int)sr_f2u(hit), fl));
+        }
+        s = sr_u2f((uint32_t)__builtin_amdgcn_readlane((int)sr_f2u(acc), fl));
+        lstart = fl + 1;
+        if (lstart >= SR_WAVE) return s;
+    }
+}
+
 // ---- eight independent chains at once -----------------------------------------------------------------
 // Thread t serves chain (t & 7) with the SR_SEQ_RUN8 terms number (t >> 3) * SR_SEQ_RUN8 ... of that chain's
 // tile, so one tile covers SR_SEQ_THREADS / 8 * SR_SEQ_RUN8 terms of every chain.  *s is the running sum

@@ -24,6 +24,7 @@
 #include "sr_device.h"
 #include "sr_types.h"
 #include "sr_kernels.h"
+#include "sr_seqsum.h"
 
 namespace {
 
@@ -55,6 +56,31 @@ constexpr int kBinsPerLane = kBins / SR_WAVE;
 // further than a multiple of the strip length, so that the 64 lanes of a wave fall on different LDS banks.
 constexpr int kBinsPad = kBins + SR_WAVE + 1;
 __device__ __forceinline__ int bin_word(int b) { return b + b / kBinsPerLane; }
+// The bin of an entry of the row tail, from xs = (its value) x (1 / temperature): 0 .. kBins - 1, never decreasing as
+// the value falls (all that the ranking needs of it).  Two maps.  The plain one: equal steps of xs down from the
+// origin.  The other one, when the candidates' lower bound is known: steps that grow with the distance u above that
+// bound like the bit pattern of the float u + c does (128 bins per doubling, c = span / 256: eight doublings, all
+// the bins), so that the crowd just above the bound is spread over many bins and the few entries far above it share
+// few.
+constexpr int kBinShift = 16;               // 2^(23 - 16) bins per doubling
+constexpr float kBinOffset = 0.00390625f;   // c / span
+struct BinMap {
+    float mx = 0.0f;        // the origin: the largest kept element, scaled
+    float bscale = -56.0f;  // plain map: bins per unit, negated
+    float span = 0.0f;      // the other map: origin minus bound (scaled), the offset c and its bits, the bin of u = 0
+    float c = 0.0f;
+    uint32_t cbits = 0u;
+    int ftop = 0;
+    bool by_bits = false;
+    __device__ __forceinline__ int of(float xs) const
+    {
+        const float d = __fsub_rn(xs, mx);
+        if (!by_bits) return min(max((int)__fmul_rn(d, bscale), 0), kBins - 1);
+        const float u = fmaxf(__fadd_rn(d, span), 0.0f);
+        const int f = (int)((sr_f2u(__fadd_rn(u, c)) - cbits) >> kBinShift);
+        return min(max(ftop - f, 0), kBins - 1);
+    }
+};
 
 struct TopkSmem {
     uint32_t xa[kSelMax];  // list of groups to fetch (xa and xb), then the kept entries by bin / the sort exchange
@@ -443,7 +469,7 @@ __device__ __forceinline__ bool row_history_in_registers(const SrRow& rd)
 
 template <int EPV, int kVec, bool kKept, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
-                                                bool force_exact, float inv_temp, float* mx0_out, float* bscale_out,
+                                                bool force_exact, float inv_temp, BinMap* map_out,
                                                 float* bound_out, bool* binned, const KeptGroups& kept, Early&& early,
                                                 Late&& late, TopkSmem& sm);
 
@@ -489,9 +515,10 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     // rows without penalties that may raise a logit have their candidates binned while they are collected
     const bool want_bins = rd.path == SR_PATH_TOPK && (!use_edits || hist_regs);
     bool binned = false;
-    float mx0 = 0.0f, bscale0 = -56.0f, bound0 = 0.0f;
+    BinMap map0;
+    float bound0 = 0.0f;
     const int n_c = build_candidates<EPV, kVec, kKept>(
-        a, slot, row, rd, want_bins, force_exact, inv_temp, &mx0, &bscale0, &bound0, &binned, kept,
+        a, slot, row, rd, want_bins, force_exact, inv_temp, &map0, &bound0, &binned, kept,
         [&]() SR_INL {
             if constexpr (!(kKept)) {
 #pragma unroll
@@ -620,8 +647,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     };
 
     float mx;
-    float mx_bins = 0.0f;  // what the bins are measured from: mx, or the largest kept element outside the history
-    float bscale = -56.0f;  // bins per unit of (v / T), negated
+    BinMap bmap;  // its origin: mx, or the largest kept element outside the history
     // Candidates whose e = expf(v / T - max) is below 2^-26 are dropped before the sort: with e_0 = 1
     // they change neither running sum (they are under half an ulp of a sum >= 1, and of a cumulative
     // probability >= probs[0]) and the draw can never stop on them, so the result is bit-identical.
@@ -753,14 +779,13 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         // 0..1023.  Never increasing with the key, so "bin <= b" is a prefix of the descending order.
         auto bin_of = [&](uint32_t key) SR_INL -> int {
             if (key == 0u) return -1;
-            const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx_bins);
-            if (x < -18.1f) return -1;
-            return min(max((int)__fmul_rn(x, bscale), 0), kBins - 1);
+            const float xs = __fmul_rn(sr_okey_inv(key), inv_temp);
+            if (__fsub_rn(xs, bmap.mx) < -18.1f) return -1;
+            return bmap.of(xs);
         };
         // the bin of an entry that was kept (binned candidates are never dropped once they are on the list)
         auto bin_kept = [&](uint32_t key) SR_INL -> int {
-            const float x = __fsub_rn(__fmul_rn(sr_okey_inv(key), inv_temp), mx_bins);
-            return min(max((int)__fmul_rn(x, bscale), 0), kBins - 1);
+            return bmap.of(__fmul_rn(sr_okey_inv(key), inv_temp));
         };
         int bstar = kBins - 1, n_live = 0, n_keep = 0, max_bin = 0;
         // every wave reads the histogram: live entries, and the first bin at which the k best are complete;
@@ -798,8 +823,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         bool by_bins = true;  // kept entries are laid out bin by bin and ranked inside their bin
         if (binned) {
             // The candidates were counted into the histogram as they were collected; the history ids join them.
-            mx_bins = mx0;
-            bscale = bscale0;
+            bmap = map0;
             // a history id whose adjusted logit is below the candidates' bound has at least top_k candidates above
             // it, or lies too far below the maximum to matter
             const uint32_t bound_key = sr_okey(bound0);
@@ -842,7 +866,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 placed = true;
             } else {
                 load_cands();  // a flat or heavily tied row: the general way below
-                bscale = -56.0f;
+                bmap = BinMap{};
             }
         }
         if (!placed) {
@@ -856,7 +880,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
         if (kmaxn == 0u) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
         mx = __fmul_rn(sr_okey_inv(kmaxn), inv_temp);
-        mx_bins = mx;
+        bmap.mx = mx;
 #pragma unroll
         for (int r = 0; r < kCandRegs; r++)
             if (r < nr) { const int b = bin_of(kreg[r]); if (b >= 0) atomicAdd(&sm.bhist[bin_word(b)], 1u); }
@@ -944,7 +968,18 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 const int b = bin_kept(mh);
                 const int p0 = (int)sm.boff[bin_word(b)], p1 = p0 + (int)sm.bhist[bin_word(b)];
                 int rank = p0;
-                for (int j = p0; j < p1; j++) rank += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
+                // four entries of the bin per step, their twelve words fetched together (an index past the bin's end
+                // reads the bin's last entry and does not count)
+                for (int j = p0; j < p1; j += 4) {
+                    uint32_t eh[4], em[4], el[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const int jj = min(j + q, p1 - 1);
+                        eh[q] = sm.xa[jj]; em[q] = sm.xb[jj]; el[q] = sm.xc[jj];
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; q++) rank += (j + q < p1 && key3_less(mh, mm, ml, eh[q], em[q], el[q])) ? 1 : 0;
+                }
                 if (rank < kk) {
                     sm.vals[rank] = sr_okey_inv(mh);
                     sm.idxs[rank] = (int)(0xffffffffu - ml);
@@ -999,14 +1034,47 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     }
     if (tid < 8) sm.probs[k + tid] = 0.0f;
     live = (int)block_max_u32((uint32_t)live, sm);
-    if (tid == 0) {
-        // e_0 = expf(0) = 1, so from t = 1 on the running sum is >= 1 and terms below 2^-24 leave it
-        // unchanged: stopping at `live` gives the same bits as running to k
-        const int n = max(live, 1);
+    // The left-to-right sum of a long list, bit for bit, by one wave: every lane takes kRun consecutive entries, the
+    // wave composes their increment functions and replays only the runs in which the sum changes binade -- a few
+    // rounds (0.4 us each) instead of a chain of a thousand dependent additions (4 us); a short list is quicker
+    // summed by one lane.
+    constexpr int kRun = 16;
+#ifndef SR_AB_KSUM
+#define SR_AB_KSUM 384
+#endif
+    constexpr int kSumByOneLane = SR_AB_KSUM;
+    auto load_run = [&](int base, int limit, float (&x)[kRun]) SR_INL {
+        const float4* p4 = (const float4*)(sm.probs + base) + sr_lane() * (kRun / 4);
+#pragma unroll
+        for (int j4 = 0; j4 < kRun / 4; j4++) {
+            const int i = base + sr_lane() * kRun + j4 * 4;
+            float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (i < limit) v = p4[j4];  // (the array is longer than any list by two such vectors)
+            x[j4 * 4 + 0] = v.x;
+            x[j4 * 4 + 1] = i + 1 < limit ? v.y : 0.0f;
+            x[j4 * 4 + 2] = i + 2 < limit ? v.z : 0.0f;
+            x[j4 * 4 + 3] = i + 3 < limit ? v.w : 0.0f;
+        }
+    };
+    // e_0 = expf(0) = 1, so from t = 1 on the running sum is >= 1 and terms below 2^-24 leave it
+    // unchanged: stopping at `live` gives the same bits as running to k
+    const int n_sum = max(live, 1);
+    if (n_sum > kSumByOneLane) {
+        if (sr_wave_id() == 0) {
+            float sum = 0.0f;
+            for (int base = 0; base < n_sum; base += SR_WAVE * kRun) {
+                float x[kRun];
+                load_run(base, n_sum, x);
+                int unused;
+                sum = sr_seq_wave<kRun, false>(x, sum, 0.0f, &unused);
+            }
+            if (sr_lane() == 0) sm.bcast[5] = sr_f2u(sum);
+        }
+    } else if (tid == 0) {
         float sum = 0.0f;
         const float4* p4 = (const float4*)sm.probs;
         float4 cur = p4[0];
-        for (int t = 0; t < n; t += 4) {
+        for (int t = 0; t < n_sum; t += 4) {
             const float4 nxt = p4[(t >> 2) + 1];
             sum = __fadd_rn(sum, cur.x); sum = __fadd_rn(sum, cur.y);
             sum = __fadd_rn(sum, cur.z); sum = __fadd_rn(sum, cur.w);
@@ -1095,23 +1163,22 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 // SR_TK_SEL_MAX in sm.vals / sm.idxs, the rest of an unusually long list in a.cand.  Returns the number of
 // candidates, or -1 when the row cannot be handled.  Called by every thread of the tail workgroup; the two
 // hooks let the caller issue loads of its own behind the group maxima's (early) and after the first wait (late).
-// With want_bins the candidates are also counted into the tail's histogram of distances below the row's largest
-// kept element (sm.bhist, bins of 1/56 in units of the temperature; entries more than 18.1 below it are dropped on
-// the spot), and every candidate remembers its bin and its arrival number inside the bin (sm.probs, as integers):
-// the tail can then lay the candidates out bin by bin without another pass of atomics.  *binned tells whether
-// that happened (few chunks, a short enough list, a finite maximum); *mx0 is the maximum times inv_temp.
+// With want_bins the candidates are also counted into the tail's histogram (sm.bhist; the bins run from the row's
+// largest kept element down to the bound, see BinMap), and every candidate remembers its bin and its arrival number
+// inside the bin (sm.probs, as integers): the tail can then lay the candidates out bin by bin without another pass
+// of atomics.  *binned tells whether that happened (few chunks, a short enough list, a finite maximum); *map_out
+// is the map that was used.
 // force_exact, and any row whose candidates overflow the lists: the row's sel-th largest kept element is found by a
 // radix select over the logits themselves, and the candidates are exactly the sel largest in (value desc, index asc)
 // order.  Slow (several passes over the row), exact for any data, and independent of the chunk results.
 template <int EPV, int kVec, bool kKept, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
-                                                bool force_exact, float inv_temp, float* mx0_out, float* bscale_out,
+                                                bool force_exact, float inv_temp, BinMap* map_out,
                                                 float* bound_out, bool* binned, const KeptGroups& kept, Early&& early,
                                                 Late&& late, TopkSmem& sm)
 {
     *binned = false;
-    *mx0_out = 0.0f;
-    *bscale_out = -56.0f;
+    *map_out = BinMap{};
     *bound_out = -3.402823466e38f;
     using VO = VecOps<EPV>;
     constexpr int ES = (EPV == 4) ? 4 : 2;
@@ -1316,14 +1383,11 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         for (int c = kGmRegs; c < S; c++) f(c, gm_load(c));
     };
     bool bins = false;
-    float mx0 = 0.0f, bscale = -56.0f;
+    BinMap map;
     uint32_t* meta = (uint32_t*)sm.probs;
     // the bin of a candidate: 0 .. kBins - 1, never increasing with the value (what lies too far below the maximum
     // to matter never gets here: the bound is at least the maximum minus 18 T, see below)
-    auto bin0 = [&](float x) SR_INL -> int {
-        const float d = __fsub_rn(__fmul_rn(x, inv_temp), mx0);
-        return min(max((int)__fmul_rn(d, bscale), 0), kBins - 1);
-    };
+    auto bin0 = [&](float x) SR_INL -> int { return map.of(__fmul_rn(x, inv_temp)); };
     // one candidate at list position pos
     auto place = [&](uint32_t pos, float x, int idx) SR_INL {
         if (pos < (uint32_t)kSelMax) {
@@ -1434,10 +1498,16 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
             tval = fmaxf(tval, tdead);
         }
         bins = want_bins && direct && km > kKeyNegInf;
-        mx0 = __fmul_rn(sr_okey_inv(km), inv_temp);
+        map.mx = __fmul_rn(sr_okey_inv(km), inv_temp);
         // the bins span what can become a candidate: from the maximum down to the bound
-        const float span = __fsub_rn(mx0, __fmul_rn(tval, inv_temp));
-        if (bins && span > 1e-3f && span < 1e30f) bscale = -fminf(__fdiv_rn((float)(kBins - 1), span), 65536.0f);
+        const float span = __fsub_rn(map.mx, __fmul_rn(tval, inv_temp));
+        if (bins && span > 1e-3f && span < 1e30f) {
+            map.by_bits = true;
+            map.span = span;
+            map.c = __fmul_rn(span, kBinOffset);
+            map.cbits = sr_f2u(map.c);
+            map.ftop = (int)((sr_f2u(__fadd_rn(span, map.c)) - map.cbits) >> kBinShift);
+        }
     }
     late();
     SR_PROF(a, 1);
@@ -1557,8 +1627,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     __syncthreads();
     if (n_c > (uint32_t)kRowCap) return exact_row();  // more candidates than the lists hold: the exact way
     *binned = bins && listed && n_c <= (uint32_t)kSelMax;
-    *mx0_out = mx0;
-    *bscale_out = bscale;
+    *map_out = map;
     *bound_out = tval;
     return (int)n_c;
 }

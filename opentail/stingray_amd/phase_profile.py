@@ -77,6 +77,11 @@ def main(argv):
                 parts.append("%s %.1f" % (nm, us(pt[ok, b_] - pt[ok, a_]).mean()))
         print("tails with %4d..%4d candidates: n %3d, start %.1f, end %.1f, total %.1f us | %s" % (
             lo, hi, m.sum(), us(pt[m, 4] - t0).mean(), us(pt[m, 15] - t0).mean(), total[m].mean(), ", ".join(parts)))
+    print("the longest tails:")
+    for i in np.argsort(-total)[:6]:
+        parts = ["%s %.1f" % (nm, us(pt[i, b_] - pt[i, a_])) for nm, a_, b_ in phases if pt[i, a_] > 0 and pt[i, b_] > 0]
+        print("  candidates %5d, start %.1f, end %.1f, total %.1f us | %s" % (
+            n_c[i], us(pt[i, 4] - t0), us(pt[i, 15] - t0), total[i], ", ".join(parts)))
     print("time (us)  chunks running  tails running")
     for b0 in np.arange(0, us(pt[:, 15].max() - t0) + 5, 5.0):
         ac = ((us(pc[:, 0] - t0) < b0 + 5) & (us(pc[:, 5] - t0) > b0)).sum()
