@@ -1099,17 +1099,20 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         count = min(count, block_min_i32(first, sm));
     }
     // Sampler.cs:326-349: running sum; top-p cuts after the first cum >= TopP.  Then the draw (:351-357): the first
-    // entry whose running sum reaches r = u * (sum of the kept entries).  One lane runs both chains and nothing is
-    // stored in between: the second chain repeats the additions of the first (same operands, same order, same
-    // bits) up to where the draw stops.  The sums never decrease, so whole blocks of 32 entries are added without
-    // a look (eight loads in flight, one chain of 32 additions) until a block's last sum has reached the target;
-    // only that block, or the remainder of the list, is walked entry by entry.
-    if (tid == 0) {
+    // entry whose running sum reaches r = u * (sum of the kept entries).  One wave runs both searches and nothing is
+    // stored in between: the second repeats the additions of the first (same operands, same order, same bits) up to
+    // where the draw stops.  A search mostly ends early in the list, so its first kChainFirst entries are walked as
+    // one chain of additions (every lane the same one): whole blocks of 32 entries without a look (eight loads in
+    // flight, the sums never decrease) until a block's last sum has reached the target, then that block entry by
+    // entry.  A search that goes on from there takes the wave's exact scan.
+    constexpr int kChainFirst = 256;
+    if (sr_wave_id() == 0) {
         const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
         const float top_p = use_top_p ? rd.top_p : __uint_as_float(0x7f800000u);  // +inf: never reached
         const float4* p4 = (const float4*)sm.probs;
         // first t < limit whose running sum is >= target (else -1); *val = that sum, or the sum of all `limit` entries
-        auto first_reach = [&](float target, int limit, float* val) SR_INL -> int {
+        auto first_reach = [&](float target, int limit_all, float* val) SR_INL -> int {
+            const int limit = min(limit_all, kChainFirst);
             float cum = 0.0f;
             int t = 0;
             while (t + 32 <= limit) {
@@ -1139,6 +1142,13 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 if (cw >= target) { *val = cw; return t + 3; }
                 cum = cw;
             }
+            for (int base = kChainFirst; base < limit_all; base += SR_WAVE * kRun) {
+                float x[kRun];
+                load_run(base, limit_all, x);
+                int f;
+                cum = sr_seq_wave<kRun, true>(x, cum, target, &f);
+                if (f >= 0) { *val = cum; return base + f; }
+            }
             *val = cum;
             return -1;
         };
@@ -1149,8 +1159,10 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept_sum);
         float unused;
         const int first = first_reach(r, cnt, &unused);
-        a.out_tokens[row] = sm.idxs[first >= 0 ? first : 0];
-        if (a.out_flags) a.out_flags[row] = out_flag;
+        if (sr_lane() == 0) {
+            a.out_tokens[row] = sm.idxs[first >= 0 ? first : 0];
+            if (a.out_flags) a.out_flags[row] = out_flag;
+        }
     }
 }
 
