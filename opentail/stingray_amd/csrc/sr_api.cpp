@@ -159,10 +159,13 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
             const int n_first = std::min(per_pool, (total_items + n_pool - 1) / n_pool);
             for (int w = 0; w < n_first; w++) new_worker(p, 0.0);
         }
-        // With a row or more per compute unit nothing is gained by spreading a row over workers (streaming alone
-        // already takes all the memory bandwidth, and tails that run beside it slow it down by more than they gain):
-        // every worker streams all chunks of one row and finishes it, waits for nobody and hands nothing over.
-        const bool affine = n_sel >= ctx->cu_count;
+        // With rows for more than about half the compute units nothing is gained by spreading a row over workers
+        // (a compute unit streams at little more than its share of the memory bandwidth anyway, and tails that run
+        // beside the streaming slow it down by more than they gain): every worker streams all chunks of one row and
+        // finishes it, waits for nobody and hands nothing over.  (Measured on 256 compute units, 151,936 fp32 logits
+        // a row: the two ways cost the same at 136 rows; at 192 rows 37.8 against 45.9 us, at 128 rows 36.0 against
+        // 33.2 us.)
+        const bool affine = n_sel * 32 >= ctx->cu_count * 17;
         if (affine) {
             prog_items.assign((size_t)n_sel, {});
             prog_tail.assign((size_t)n_sel, -1);

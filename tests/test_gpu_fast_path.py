@@ -185,6 +185,48 @@ def test_config3_full_chain_with_penalties(ctx):
     _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits))
 
 
+@pytest.mark.parametrize("rows,vocab", [(120, 20_011), (150, 20_011), (200, 151_936), (256, 20_011), (300, 20_011), (520, 9_973)])
+def test_every_shape_of_the_launch_gives_the_oracles_tokens(ctx, rows, vocab):
+    # The host picks the launch's shape from the number of rows: rows dealt out chunk by chunk over all workers (few
+    # rows), one worker per row that keeps the chunk results in its registers (from about half the compute units'
+    # number of rows up to one row per compute unit), one worker per row that writes them out (more rows).  Rows of
+    # every kind in each: greedy with and without penalties, top-k 1 .. 1000 with top-p / min-p, histories that lower
+    # and that raise, coarse values (ties at every cut), rows with a handful of finite logits.
+    import torch
+
+    rng = np.random.default_rng(rows * 7 + vocab)
+    logits = synthetic.zipf_head_logits(rng, rows, vocab)
+    logits[1::5] = np.round(logits[1::5] * 4) / 4                      # quantised rows: ties
+    logits[2::17, :] = NEG_INF
+    for r in range(2, rows, 17):
+        logits[r, rng.integers(0, vocab, 5)] = rng.normal(0, 1, 5).astype(np.float32)
+    params = []
+    for r in range(rows):
+        hist = rng.integers(0, vocab, int(rng.integers(1, 70))).tolist()
+        kind = r % 6
+        k = int(rng.integers(1, min(1001, vocab)))
+        if kind == 0:
+            p = SamplingParams(Temperature=0.0)
+        elif kind == 1:
+            p = SamplingParams(Temperature=0.0, RepetitionPenalty=1.3, FrequencyPenalty=0.2, PreviousTokens=hist)
+        elif kind == 2:
+            p = SamplingParams(Temperature=float(rng.uniform(0.3, 1.5)), TopK=k, TopP=float(rng.uniform(0.5, 1.0)))
+        elif kind == 3:
+            p = SamplingParams(Temperature=float(rng.uniform(0.3, 1.5)), TopK=k, TopP=0.9, MinP=0.02, RepetitionPenalty=1.1,
+                               PresencePenalty=0.3, FrequencyPenalty=0.1, PreviousTokens=hist)
+        elif kind == 4:
+            p = SamplingParams(Temperature=0.8, TopK=min(k, 200), RepetitionPenalty=0.8, PresencePenalty=-0.2,
+                               PreviousTokens=hist)               # penalties that raise: the literal over-selection
+        else:
+            p = SamplingParams(Temperature=1.0, TopK=k, MinP=0.1)
+        params.append(p)
+    u = rng.random(rows)
+    flags = _check_rows(ctx, logits, params, u, _cuda(logits))
+    assert np.all(flags & 3)                                          # greedy or top-k-first: the selection kernel
+    bits = synthetic.to_bf16_bits(logits)
+    _check_rows(ctx, synthetic.bf16_bits_to_f32(bits), params, u, _cuda(bits.view(np.int16), torch.bfloat16))
+
+
 def test_top_k_under_an_allow_mask_and_unaligned_rows(ctx):
     import torch
 
