@@ -358,6 +358,7 @@ void sr_batch_destroy(sr_batch* b)
                          &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched};
     for (DeviceBuf* d : bufs) d->release();
     b->stage.release();
+    b->patch_ring.release();
     delete b;
 }
 
@@ -810,16 +811,12 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     const size_t n_uni = (uniforms && b->upr > 0) ? (size_t)rows * (size_t)b->upr : 0;
     const size_t need = rp.size() * sizeof(SrRowPatch) + ep.size() * sizeof(SrEditPatch) + mc.size() * sizeof(SrMaskClear) +
                         n_uni * sizeof(double) + scan_again.size() * sizeof(int32_t) + 5 * 256;
-    SR_HIP(ctx, b->stage.begin());
-    if (b->stage.cap < need) {  // grows at begin()
-        b->stage.wanted = need;
-        SR_HIP(ctx, b->stage.begin());
-    }
-    const SrRowPatch* rp_d = (const SrRowPatch*)b->stage.put(rp.data(), rp.size() * sizeof(SrRowPatch));
-    const SrEditPatch* ep_d = (const SrEditPatch*)b->stage.put(ep.data(), ep.size() * sizeof(SrEditPatch));
-    const SrMaskClear* mc_d = (const SrMaskClear*)b->stage.put(mc.data(), mc.size() * sizeof(SrMaskClear));
-    const double* un_d = (const double*)b->stage.put(uniforms, n_uni * sizeof(double));
-    const int32_t* sa_d = (const int32_t*)b->stage.put(scan_again.data(), scan_again.size() * sizeof(int32_t));
+    SR_HIP(ctx, b->patch_ring.begin(need, st));
+    const SrRowPatch* rp_d = (const SrRowPatch*)b->patch_ring.put(rp.data(), rp.size() * sizeof(SrRowPatch));
+    const SrEditPatch* ep_d = (const SrEditPatch*)b->patch_ring.put(ep.data(), ep.size() * sizeof(SrEditPatch));
+    const SrMaskClear* mc_d = (const SrMaskClear*)b->patch_ring.put(mc.data(), mc.size() * sizeof(SrMaskClear));
+    const double* un_d = (const double*)b->patch_ring.put(uniforms, n_uni * sizeof(double));
+    const int32_t* sa_d = (const int32_t*)b->patch_ring.put(scan_again.data(), scan_again.size() * sizeof(int32_t));
     if (!rp_d || !ep_d || !mc_d || !un_d || !sa_d) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "sr_batch_append_tokens: no pinned memory");
     // scan masks that are not built yet are built from the patched edits when they are needed
     const bool masks = b->scan_epv != 0 && b->d_scan_mask.p != nullptr;
@@ -834,7 +831,6 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
                                               b->d_edits.as<SrEdit>(), sr_batch_mask_ptr(b), sr_batch_mask_stride(b),
                                               b->d_scan_mask.as<uint32_t>(), b->scan_stride, b->vocab, b->scan_epv,
                                               b->scan_chunks, b->scan_chunk_vecs, b->scan_base_addr, b->scan_stride_bytes, st));
-    SR_HIP(ctx, b->stage.end(st));
     return SR_OK;
 }
 

@@ -103,6 +103,77 @@ struct HostStage {
     }
 };
 
+// Pinned host memory for the short lists of a decode step (the changes of one appended token per row), which a
+// kernel reads in place.  An event after every step's kernel would tell when its piece may be overwritten, but an
+// event between two kernels of a stream costs about 4 us of device time here; so the memory is two halves, each filled
+// piece by piece over many steps, and only the change of halves records an event (for everything enqueued so far) and
+// waits for the one recorded when the other half was left, many steps ago.
+struct HostRing {
+    char* p = nullptr;
+    size_t half = 0, used = 0;
+    int cur = 0;
+    hipEvent_t ev[2] = {nullptr, nullptr};
+    bool pending[2] = {false, false};
+    bool dirty = false;             // pieces handed out since the last wait for a whole stream
+    hipStream_t last = nullptr;     // the stream of those pieces' kernels
+    // room for `need` bytes in the present half (its pieces are handed out by put)
+    hipError_t begin(size_t need, hipStream_t st)
+    {
+        hipError_t e = hipSuccess;
+        if (dirty && st != last) {  // the caller changed streams: nothing orders the old stream's readers before new events
+            if ((e = hipStreamSynchronize(last)) != hipSuccess) return e;
+            pending[0] = pending[1] = dirty = false;
+            used = 0;
+        }
+        last = st;
+        if (need > half) {  // grow: nothing may still be reading the old memory
+            if (dirty && (e = hipStreamSynchronize(st)) != hipSuccess) return e;
+            if (p) (void)hipHostFree(p);
+            p = nullptr;
+            half = used = 0;
+            pending[0] = pending[1] = dirty = false;
+            const size_t want = 16 * need + 65536;
+            if ((e = hipHostMalloc((void**)&p, 2 * want, hipHostMallocDefault)) != hipSuccess) { p = nullptr; return e; }
+            half = want;
+            cur = 0;
+        }
+        if (used + need > half) {
+            for (int h = 0; h < 2; h++)
+                if (!ev[h] && (e = hipEventCreateWithFlags(&ev[h], hipEventDisableTiming)) != hipSuccess) return e;
+            if ((e = hipEventRecord(ev[cur], st)) != hipSuccess) return e;
+            pending[cur] = true;
+            cur ^= 1;
+            if (pending[cur]) {
+                if ((e = hipEventSynchronize(ev[cur])) != hipSuccess) return e;
+                pending[cur] = false;
+            }
+            used = 0;
+        }
+        return hipSuccess;
+    }
+    // a copy of src inside the present half (begin made the room); nullptr when it does not fit after all
+    const void* put(const void* src, size_t bytes)
+    {
+        const size_t need = std::max((bytes + 255) & ~(size_t)255, (size_t)256);  // (an empty list has an address too)
+        if (!p || used + need > half) return nullptr;
+        void* dst = p + (size_t)cur * half + used;
+        if (bytes) memcpy(dst, src, bytes);
+        used += need;
+        dirty = true;
+        return dst;
+    }
+    void release()  // (the owner has waited for the stream)
+    {
+        if (p) (void)hipHostFree(p);
+        for (int h = 0; h < 2; h++)
+            if (ev[h]) (void)hipEventDestroy(ev[h]);
+        p = nullptr;
+        ev[0] = ev[1] = nullptr;
+        half = used = 0;
+        pending[0] = pending[1] = dirty = false;
+    }
+};
+
 struct sr_ctx {
     int device = 0;
     hipStream_t own_stream = nullptr;
@@ -162,7 +233,8 @@ struct sr_batch {
     bool mask_ids = false;               // the rows' allow-masks are registered masks of the context (mask_row = id)
     std::vector<int32_t> keep_mask_ids;  // ... per row, -1 none
     int32_t max_sel = 0;
-    HostStage stage;          // pinned copies of what an upload sends to the device
+    HostStage stage;
+    HostRing patch_ring;  // the lists of sr_batch_append_tokens          // pinned copies of what an upload sends to the device
     std::vector<SrCopySeg> segs;  // ... the pieces that are packed and not yet sent
     bool upload_must_wait = false;  // some copy of the running upload reads pageable memory directly
     // geometry the scan masks were built with (sr_batch_append_tokens clears single bits in place)

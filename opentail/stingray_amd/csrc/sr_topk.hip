@@ -2014,15 +2014,20 @@ __global__ __launch_bounds__(256) void k_apply_patches(SrRow* rows, const SrRowP
                                                        int n_uni)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    // The lists lie in pinned host memory: every read is a trip over the bus.  All four are read first, without
+    // conditions (a thread past a list's end reads the list's last entry, or whatever stands at the head of an empty
+    // list's 256 bytes), so that the trips run side by side; then the changes are applied.
+    const SrRowPatch r = rp[min(i, max(n_rowp, 1) - 1)];
+    const SrEditPatch e = ep[min(i, max(n_edits, 1) - 1)];
+    const SrMaskClear m = mc[min(i, max(n_clears, 1) - 1)];
+    const double u = uni_src[min(i, max(n_uni, 1) - 1)];
     if (i < n_rowp) {
-        const SrRowPatch r = rp[i];
         rows[r.row].n_prev = r.n_prev;
         rows[r.row].edit_cnt = r.edit_cnt;
         rows[r.row].mask_row = r.mask_row;
     }
-    if (i < n_edits) edits[ep[i].index] = ep[i].edit;
+    if (i < n_edits) edits[e.index] = e.edit;
     if (i < n_clears) {
-        const SrMaskClear m = mc[i];
         const int mis = (int)(((base_addr + (unsigned long long)m.row * (unsigned long long)stride_bytes) & 15ull) / (unsigned)es);
         const int p = m.id + mis;
         const int fv = p / epv, q = p - fv * epv;
@@ -2032,7 +2037,7 @@ __global__ __launch_bounds__(256) void k_apply_patches(SrRow* rows, const SrRowP
         atomicAnd(&scan_mask[(size_t)m.scan_row * scan_stride + ((size_t)c * kThreads + tt) * SR_TK_MASK_WORDS + (b >> 5)],
                   ~(1u << (b & 31)));
     }
-    if (i < n_uni) uni_dst[i] = uni_src[i];
+    if (i < n_uni) uni_dst[i] = u;
 }
 
 // The pieces of a batch upload, read where the host packed them (pinned host memory, over the bus) and written
