@@ -158,9 +158,9 @@ SR_API int sr_batch_upload(sr_batch* batch, int32_t rows, int32_t vocab,
  * the few entries that change instead of a pass over every history.
  *   tokens    [rows] host array; a negative entry leaves its row's history as it is.
  *   uniforms  [rows x uniforms_per_row] for the next step, or NULL to keep those on the device.
- * Rows the in-place update does not cover (the first history token of a row with penalties, rows with logit bias
- * or with penalties that may raise a logit, a row that runs out of room) make the call rebuild the whole batch from
- * the inputs it kept: same result, the cost of an upload.  A batch uploaded with allow-masks of its own returns
+ * Rows the in-place update does not cover (the first history token of a row with penalties, a row that runs out of
+ * the room it was given for new ids -- 32 and more per row --, a top-k beyond 2,048 entries) make the call rebuild the
+ * whole batch from the inputs it kept: same result, the cost of an upload.  A batch uploaded with allow-masks of its own returns
  * SR_ERR_UNSUPPORTED (its masks change with every step: register them and use sr_batch_upload_mask_ids /
  * sr_batch_append_tokens_masks).  Copies run on the context's stream and are not waited for, as in sr_batch_upload. */
 SR_API int sr_batch_append_tokens(sr_batch* batch, const int32_t* tokens, const double* uniforms);

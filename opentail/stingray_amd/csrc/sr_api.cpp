@@ -180,7 +180,7 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
                     entries.push_back((int32_t)(((uint32_t)c << 24) | (uint32_t)slot));
                     entries.push_back(r);
                     entries.push_back(d.scan_row);
-                    entries.push_back(d.sel);
+                    entries.push_back(b->sel_cap[(size_t)r]);
                 }
                 prog_tail[(size_t)slot] = slot;
                 continue;
@@ -200,7 +200,7 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
                 entries.push_back((int32_t)(((uint32_t)c << 24) | (uint32_t)slot));
                 entries.push_back(r);
                 entries.push_back(d.scan_row);
-                entries.push_back(d.sel);
+                entries.push_back(b->sel_cap[(size_t)r]);
                 w.free_at += t_item;
                 if (c == chunks - 1) {
                     prog_tail[(size_t)w.id] = slot;
@@ -417,6 +417,7 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
     if (mask_ids) b->keep_mask_ids.assign(mask_ids, mask_ids + rows); else b->keep_mask_ids.clear();
     b->max_sel = 0;
     b->edit_cap.assign((size_t)rows, 0);
+    b->sel_cap.assign((size_t)rows, 0);
     b->edit_ids.clear();
     if (retain) {
         b->can_append = allow_mask == nullptr;
@@ -554,7 +555,7 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
             }
             d.edit_cnt = (int32_t)ed.size() - d.edit_off;
             b->edit_cap[(size_t)r] = d.edit_cnt;
-            if (want_hist && !searched && d.edit_cnt > 0) {
+            if (want_hist && d.edit_cnt > 0) {
                 // room for the ids that appended tokens bring: a fixed minimum, and half as much again as the row has
                 // (a batch that was rebuilt because a row ran out of room is not rebuilt again soon)
                 const int32_t slack = std::max(SR_EDIT_SLACK, d.edit_cnt / 2);
@@ -583,6 +584,12 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
         } else if (d.path == SR_PATH_TOPK && d.edit_cnt == 0) {
             d.sel = p.top_k;  // no history id inside the vocabulary: nothing is ever penalised
         }
+        // A row that over-selects by its history length asks for one more with every appended token: the chunk items
+        // of the launch (which carry sel for the waves' shares of the bound) are written for a little more, so that
+        // appended tokens need no new items; any value with that many group maxima above it is a bound for less too.
+        b->sel_cap[(size_t)r] = d.sel;
+        if (d.path == SR_PATH_TOPK && has_penalty && d.edit_cnt > 0 && !lowering)
+            b->sel_cap[(size_t)r] = (int32_t)std::min<int64_t>((int64_t)d.sel + (b->edit_cap[(size_t)r] - d.edit_cnt), vocab);
         if (d.path == SR_PATH_TOPK_WIDE) {
             b->h_wide_list.push_back(r);
         } else if (d.path != SR_PATH_FULL) {
@@ -737,7 +744,7 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
             if (d.scan_row >= 0 && (b->h_scan_need[(size_t)r] & SR_SCAN_ALLOW)) scan_again.push_back(d.scan_row);
         }
         if (tokens[r] < 0) {
-            if (mask_changed) rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row});
+            if (mask_changed) rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel});
             continue;
         }
         const sr_row_params& p = b->keep_params[(size_t)r];
@@ -745,13 +752,16 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
         const int32_t n_new = (int32_t)hist.size(), n_old = n_new - 1;
         if (!has_history_penalty(p)) {  // the history is never looked at
             d.n_prev = n_new;
-            rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row});
+            rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel});
             continue;
         }
-        if (n_old == 0 || d.edit_cnt == 0 || (d.flags & SR_ROWFLAG_EDITS_SORTED) || d.path == SR_PATH_TOPK_WIDE) {
+        if (n_old == 0 || d.edit_cnt == 0 || d.path == SR_PATH_TOPK_WIDE) {
             rebuild = true;
             break;
         }
+        const bool sorted = (d.flags & SR_ROWFLAG_EDITS_SORTED) != 0u;
+        // a row that over-selects by its history length (penalties that may raise a logit, Sampler.cs:224-225)
+        const bool literal = d.path == SR_PATH_TOPK && (d.flags & SR_ROWFLAG_HIST_EXCL) == 0u;
         SrEdit* ed = b->h_edits.data() + d.edit_off;
         int32_t* eids = b->edit_ids.data() + d.edit_off;
         auto find = [&](int32_t id) -> int32_t {
@@ -784,9 +794,20 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
                     rebuild = true;
                     break;
                 }
-                k = d.edit_cnt++;
+                if (sorted) {
+                    // the edits stay in order of their ids (a kernel searches them): the new one goes where it
+                    // belongs, the ones behind it move up by one and are sent again
+                    k = (int32_t)(std::lower_bound(eids, eids + d.edit_cnt, t) - eids);
+                    for (int32_t j = d.edit_cnt; j > k; j--) { ed[j] = ed[j - 1]; eids[j] = eids[j - 1]; }
+                    for (int32_t& j : touched) j += j >= k ? 1 : 0;
+                    d.edit_cnt++;
+                    for (int32_t j = k + 1; j < d.edit_cnt; j++) touched.push_back(j);
+                } else {
+                    k = d.edit_cnt++;
+                }
                 ed[k] = SrEdit{};
                 ed[k].id = t;
+                ed[k].pen = 1.0f;
                 eids[k] = t;
                 if (b->h_scan_need[(size_t)r] & SR_SCAN_HIST) mc.push_back(SrMaskClear{d.scan_row, r, t});
             }
@@ -796,7 +817,17 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
             touched.push_back(k);
         }
         d.n_prev = n_new;
-        rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row});
+        if (literal) {
+            const int64_t sel = std::min<int64_t>((int64_t)p.top_k + n_new, vocab);
+            if (sel > b->sel_cap[(size_t)r] || sel > SR_TK_SEL_MAX) {  // new chunk items, or the sort-based path
+                rebuild = true;
+                break;
+            }
+            d.sel = (int32_t)sel;
+        }
+        rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel});
+        std::sort(touched.begin(), touched.end());
+        touched.erase(std::unique(touched.begin(), touched.end()), touched.end());
         for (int32_t k : touched) ep.push_back(SrEditPatch{d.edit_off + k, ed[k]});
     }
     if (rebuild) {

@@ -250,6 +250,7 @@ struct sr_batch {
     std::vector<float> keep_bias_vals;
     std::vector<std::vector<int32_t>> keep_hist;
     std::vector<int32_t> edit_cap;
+    std::vector<int32_t> sel_cap;   // per row: the sel that the launch's chunk items were written for (>= the row's sel)
     std::vector<int32_t> edit_ids;  // the ids of h_edits, contiguous (searched by the append; made when first needed)
 };
 

@@ -63,6 +63,7 @@ struct SrRowPatch {
     int32_t n_prev;
     int32_t edit_cnt;
     int32_t mask_row;  // the row's allow-mask from now on (-1 none); rows of batches without registered masks keep theirs
+    int32_t sel;
 };
 struct SrMaskClear {
     int32_t scan_row;

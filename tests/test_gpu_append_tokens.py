@@ -41,12 +41,17 @@ def _rows(rng, vocab):
         # no penalties at all: the history is never read
         P(Temperature=0.8, TopK=20, TopP=0.9, PreviousTokens=hist(5)),
         P(Temperature=0.0, PreviousTokens=None),
-        # rows that make the call rebuild the batch: empty history with penalties, penalties that may raise a
-        # logit (sorted edits, over-selection by the history length), logit bias
+        # rows whose first history token makes the call rebuild the batch (once): empty history with penalties
         P(Temperature=0.8, TopK=10, RepetitionPenalty=1.2, PreviousTokens=None),
         P(Temperature=0.0, PresencePenalty=1.0, PreviousTokens=[]),
+        # penalties that may raise a logit (edits sorted by id, over-selection by the history length, which grows with
+        # every token) and logit bias (edits sorted by id): in place, the edits behind a new id move up
         P(Temperature=0.9, TopK=12, RepetitionPenalty=0.8, PresencePenalty=-0.3, PreviousTokens=hist(7)),
         P(Temperature=1.0, TopP=0.8, PresencePenalty=0.5, LogitBias={3: 2.0, 11: -1.0}, PreviousTokens=hist(4)),
+        P(Temperature=0.7, TopK=300, TopP=0.9, FrequencyPenalty=-0.2, RepeatLastN=16, RepetitionPenalty=1.3,
+          PreviousTokens=hist(90)),
+        P(Temperature=0.8, MinP=0.01, RepetitionPenalty=1.2, RepeatLastN=10,
+          LogitBias={i * 37 % 2000: (i % 5) - 2.0 for i in range(40)}, PreviousTokens=hist(30)),
     ]
 
 
@@ -125,10 +130,8 @@ def test_decode_loop_with_appended_tokens_matches_oracle_and_fresh_upload(ctx, v
             if app[r] >= 0:
                 hists[r].append(int(app[r]))
     n_rebuilt = _rebuilds(ctx, inc)
-    if in_place_only:  # only a row that ran out of room rebuilds: most calls must have been in place
-        assert n_rebuilt <= steps // 4, n_rebuilt
-    else:
-        assert n_rebuilt == steps
+    # only a row that ran out of room (or got its first history token) rebuilds: most calls must have been in place
+    assert n_rebuilt <= steps // 4, n_rebuilt
     inc.close()
 
 

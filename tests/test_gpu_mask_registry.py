@@ -47,8 +47,15 @@ def _mixed_params(rng, rows, vocab, hist_len):
     params = []
     for r in range(rows):
         hist = rng.integers(0, vocab, hist_len).tolist()
-        kind = r % 6
-        if kind == 0:
+        kind = r % 8
+        if kind == 6:                                                                  # penalties that raise: literal set
+            p = SamplingParams(Temperature=0.9, TopK=int(rng.integers(1, 80)), TopP=0.95, RepetitionPenalty=0.85,
+                               PresencePenalty=-0.2, PreviousTokens=hist)
+        elif kind == 7:                                                                # logit bias: full path, sorted edits
+            p = SamplingParams(Temperature=0.8, TopP=0.9, FrequencyPenalty=0.3,
+                               LogitBias={int(i): float(rng.normal(0, 2)) for i in rng.integers(0, vocab, 6)},
+                               PreviousTokens=hist)
+        elif kind == 0:
             p = SamplingParams(Temperature=0.0)                                        # Greedy(masked)
         elif kind == 1:
             p = SamplingParams(Temperature=0.6, TopP=0.95)                             # full path
