@@ -50,6 +50,7 @@ constexpr int kQCap = 2 * kSelMax;            // groups of a row whose elements 
 constexpr int kCandRegs = kRowCap / kThreads;   // candidates a thread holds in the row tail (16)
 constexpr int kSortRegs = kSelMax / kThreads;   // sort elements per thread (4)
 constexpr int kHistRegs = kSelMax / kThreads;   // history ids per thread (4)
+constexpr int kShortList = 128;                 // most entries (candidates + history ids) ranked by counting
 constexpr int kBins = 1024;                     // histogram bins of the row tail
 constexpr int kBinsPerLane = kBins / SR_WAVE;
 // Bin b lives at word b + b / kBinsPerLane: the strip of kBinsPerLane bins that a lane scans starts one word
@@ -787,6 +788,61 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         auto bin_kept = [&](uint32_t key) SR_INL -> int {
             return bmap.of(__fmul_rn(sr_okey_inv(key), inv_temp));
         };
+        // A short list (top-k of a few dozen) is ranked by counting: every entry against every other, four threads to
+        // an entry.  No histogram, no layout by bins.  A history id whose adjusted logit is below the candidates' bound
+        // stays out (it has at least top_k candidates above it, or lies too far below the maximum to matter); entries
+        // too small to matter are not dropped here: they rank last and change no sum (see above), as in the
+        // reference, which keeps them too.
+        bool short_list = false;
+        if (n_c <= kShortList && ne <= kThreads) {
+            const uint32_t bound_key = sr_okey(bound0);
+            __syncthreads();
+            if (tid == 0) sm.bcast[4] = 0u;
+            __syncthreads();
+            if (tid < n_c) {  // (candidates of a list this short: the first register slot, or the head of the list in LDS)
+                const uint32_t key = binned ? sr_okey(sm.vals[tid]) : kreg[0];
+                const int id = binned ? sm.idxs[tid] : kid[0];
+                sm.xa[tid] = key;
+                sm.xb[tid] = key;
+                sm.xc[tid] = 0xffffffffu - (uint32_t)id;
+            }
+            if (hraw[0] != 0u && hadj[0] >= bound_key) {  // (this thread's history id, if its logit is finite)
+                const int pos = n_c + (int)atomicAdd(&sm.bcast[4], 1u);
+                sm.xa[pos] = hadj[0];
+                sm.xb[pos] = hraw[0];
+                sm.xc[pos] = 0xffffffffu - (uint32_t)hee[0].id;
+            }
+            __syncthreads();
+            const int n_all = n_c + (int)sm.bcast[4];
+            short_list = n_all <= kShortList;
+            __syncthreads();  // (every thread has read the count: the other way may use the word again)
+            // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
+            if (n_all == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
+            if (short_list) {
+                const int kk = min(rd.top_k, n_all);
+                const int e = tid >> 2, part = tid & 3;
+                static_assert(kShortList * 4 <= kThreads, "four threads to an entry");
+                uint32_t mh = 0u, mm = 0u, ml = 0u;
+                int ahead = 0;
+                if (e < n_all) {
+                    mh = sm.xa[e]; mm = sm.xb[e]; ml = sm.xc[e];
+                    for (int j = part; j < n_all; j += 4) ahead += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
+                }
+                ahead += __shfl_xor(ahead, 1);
+                ahead += __shfl_xor(ahead, 2);
+                if (e < n_all && part == 0 && ahead < kk) {
+                    sm.vals[ahead] = sr_okey_inv(mh);
+                    sm.idxs[ahead] = (int)(0xffffffffu - ml);
+                }
+                ranked = true;
+                placed = true;  // the maximum is the first ranked entry
+                m2 = n_all;
+                sort_n = n_all;
+                SR_PROF(a, 6);
+                SR_PROF(a, 7);
+            }
+        }
+        if (!short_list) {
         int bstar = kBins - 1, n_live = 0, n_keep = 0, max_bin = 0;
         // every wave reads the histogram: live entries, and the first bin at which the k best are complete;
         // wave 0 leaves every bin's first list position in sm.boff
@@ -995,6 +1051,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             }
         }
         SR_PROF(a, 7);
+        }  // !short_list
     }
 
     // the k best that are still alive
