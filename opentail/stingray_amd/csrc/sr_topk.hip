@@ -1554,8 +1554,26 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                 km = max(km, b.y);
             }
         }
+        // Every wave's pair stands for distinct group maxima of the row: one that equals its second word and (its
+        // share - 1) that are at least its first.  The largest value with sel of all those at or above it is a bound
+        // too, and a much closer one than the smallest first word when sel is small (a top-k of 40 asks every wave
+        // for its second largest: the smallest of 32 of those has some 250 elements above it, the 40th largest of the
+        // 64 words about 50).  With one pair per lane it is found bit by bit with ballots, to 16 bits, rounded down.
+        // (Worth its 32 ballots, about 1 us, only where the shares are that small.)
+        uint32_t k_close = 0u;
+        const int share = (sel + nb - 1) / nb;  // (the waves' share was this or more)
+        if (nb <= SR_WAVE && share <= 2) {
+            const bool in = lane < nb;
+#pragma unroll 1
+            for (int bit = 31; bit >= 16; bit--) {
+                const uint32_t cnd = k_close | (1u << bit);
+                const int w = __popcll(__ballot(in && k >= cnd)) * (share - 1) + __popcll(__ballot(in && km >= cnd));
+                if (w >= sel) k_close = cnd;
+            }
+        }
         k = sr_wave_min_u32(k);
         km = sr_wave_max_u32(km);
+        k = max(k, k_close);
         if (k > kKeyNegInf) tval = sr_okey_inv(k);
         // An element 19 T below the row's largest kept element has expf((v - max) / T) < 2^-26 whatever else
         // joins the row (penalties that only lower cannot raise the maximum's rivals above it, and the maximum of
