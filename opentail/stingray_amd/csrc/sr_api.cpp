@@ -824,6 +824,7 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
                 break;
             }
             d.sel = (int32_t)sel;
+            b->max_sel = std::max(b->max_sel, d.sel);
         }
         rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel});
         std::sort(touched.begin(), touched.end());
@@ -1013,6 +1014,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.n_workers = b->n_workers;
         a.own_rows = b->own_rows ? 1 : 0;
         a.kept = (b->own_rows && b->n_workers <= ctx->cu_count) ? 1 : 0;
+        a.short_lists = b->max_sel <= SR_TK_SHORT_SEL ? 1 : 0;
         a.n_items = b->n_items;
         a.sel_list = b->d_sel_list.as<int32_t>();
         SR_HIP(ctx, ctx->cand.reserve((size_t)n_sel * SR_TK_ROW_CAP * sizeof(unsigned long long), st));

@@ -38,6 +38,7 @@ struct SrTopkArgs {
     int32_t n_workers, n_items;
     int32_t own_rows;        // every worker's program is one whole row (all its chunks, then its tail)
     int32_t kept;            // ... and there is at most one worker per compute unit
+    int32_t short_lists;     // no row of the launch asks for more than SR_TK_SHORT_SEL entries
     const int32_t* sel_list; // [n_rows] batch row of every launch slot
     const SrRow* rows;
     const SrEdit* edits;

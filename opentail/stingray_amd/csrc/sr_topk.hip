@@ -51,6 +51,7 @@ constexpr int kCandRegs = kRowCap / kThreads;   // candidates a thread holds in 
 constexpr int kSortRegs = kSelMax / kThreads;   // sort elements per thread (4)
 constexpr int kHistRegs = kSelMax / kThreads;   // history ids per thread (4)
 constexpr int kShortList = 128;                 // most entries (candidates + history ids) ranked by counting
+constexpr int kShortSel = SR_TK_SHORT_SEL;      // launches whose rows all ask for at most this many take the steps for short lists
 constexpr int kBins = 1024;                     // histogram bins of the row tail
 constexpr int kBinsPerLane = kBins / SR_WAVE;
 // Bin b lives at word b + b / kBinsPerLane: the strip of kBinsPerLane bins that a lane scans starts one word
@@ -468,7 +469,7 @@ __device__ __forceinline__ bool row_history_in_registers(const SrRow& rd)
     return use_edits && (rd.flags & kRowHistExcl) != 0u && rd.path == SR_PATH_TOPK && rd.edit_cnt <= kHistRegs * kThreads;
 }
 
-template <int EPV, int kVec, bool kKept, typename Early, typename Late>
+template <int EPV, int kVec, bool kKept, bool kShort, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
                                                 bool force_exact, float inv_temp, BinMap* map_out,
                                                 float* bound_out, bool* binned, const KeptGroups& kept, Early&& early,
@@ -476,7 +477,10 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 
 // force_exact: the chunk results of the row are not used, the candidates come from the logits themselves (what a row
 // whose candidates overflow the lists falls back to, and a row whose chunks were not handed over in time).
-template <int EPV, int kVec, bool kKept>
+// kShort: the launch holds no row that asks for more than kShortSel entries; the tail then carries the two steps that
+// pay for such rows only (a closer bound from the waves' pairs, ranking a short list by counting).  They are compiled
+// into launches of their own because their mere presence costs the long tails of other launches 0.6 us.
+template <int EPV, int kVec, bool kKept, bool kShort>
 __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool force_exact,
                                               const KeptGroups& kept, const KeptHistory& kept_hist, TopkSmem& sm)
 {
@@ -516,9 +520,10 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     // rows without penalties that may raise a logit have their candidates binned while they are collected
     const bool want_bins = rd.path == SR_PATH_TOPK && (!use_edits || hist_regs);
     bool binned = false;
+    if (tid == 0) sm.bcast[4] = 0u;  // the short list's count of history entries (the barriers of the next call publish it)
     BinMap map0;
     float bound0 = 0.0f;
-    const int n_c = build_candidates<EPV, kVec, kKept>(
+    const int n_c = build_candidates<EPV, kVec, kKept, kShort>(
         a, slot, row, rd, want_bins, force_exact, inv_temp, &map0, &bound0, &binned, kept,
         [&]() SR_INL {
             if constexpr (!(kKept)) {
@@ -794,11 +799,9 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         // too small to matter are not dropped here: they rank last and change no sum (see above), as in the
         // reference, which keeps them too.
         bool short_list = false;
-        if (n_c <= kShortList && ne <= kThreads) {
+        if (kShort && n_c <= kShortList && ne <= kThreads) {
             const uint32_t bound_key = sr_okey(bound0);
-            __syncthreads();
-            if (tid == 0) sm.bcast[4] = 0u;
-            __syncthreads();
+            // (xa .. xc are free and the counter is zero: see where the candidates are built)
             if (tid < n_c) {  // (candidates of a list this short: the first register slot, or the head of the list in LDS)
                 const uint32_t key = binned ? sr_okey(sm.vals[tid]) : kreg[0];
                 const int id = binned ? sm.idxs[tid] : kid[0];
@@ -815,7 +818,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             __syncthreads();
             const int n_all = n_c + (int)sm.bcast[4];
             short_list = n_all <= kShortList;
-            __syncthreads();  // (every thread has read the count: the other way may use the word again)
+            if (!short_list) __syncthreads();  // (every thread has read the count: the other way uses the word again)
             // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
             if (n_all == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
             if (short_list) {
@@ -1240,7 +1243,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 // force_exact, and any row whose candidates overflow the lists: the row's sel-th largest kept element is found by a
 // radix select over the logits themselves, and the candidates are exactly the sel largest in (value desc, index asc)
 // order.  Slow (several passes over the row), exact for any data, and independent of the chunk results.
-template <int EPV, int kVec, bool kKept, typename Early, typename Late>
+template <int EPV, int kVec, bool kKept, bool kShort, typename Early, typename Late>
 __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, int row, const SrRow& rd, bool want_bins,
                                                 bool force_exact, float inv_temp, BinMap* map_out,
                                                 float* bound_out, bool* binned, const KeptGroups& kept, Early&& early,
@@ -1562,7 +1565,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         // (Worth its 32 ballots, about 1 us, only where the shares are that small.)
         uint32_t k_close = 0u;
         const int share = (sel + nb - 1) / nb;  // (the waves' share was this or more)
-        if (nb <= SR_WAVE && share <= 2) {
+        if (kShort && nb <= SR_WAVE && share <= 2) {
             const bool in = lane < nb;
 #pragma unroll 1
             for (int bit = 31; bit >= 16; bit--) {
@@ -1737,7 +1740,7 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 // worker per compute unit.  Nothing is handed over then, so nothing is written out: the group results of all chunks
 // stay in the thread's registers (the workgroup has the register file of its compute unit to itself) and the waves'
 // shares of the bound go through LDS.
-template <int EPV, int kVec, int kWindow, bool kKept>
+template <int EPV, int kVec, int kWindow, bool kKept, bool kShort>
 __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArgs a)
 {
     __shared__ TopkSmem sm;
@@ -2010,7 +2013,7 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
     }
     SR_PROF(ap, 4);
     __builtin_amdgcn_s_setprio(3);  // the tail is the longer dependent chain: its waves go first
-    topk_row_tail<EPV, kVec, kKept>(ap, tslot, trow, trd, !handed_over, kept, kept_hist, sm);
+    topk_row_tail<EPV, kVec, kKept, kShort>(ap, tslot, trow, trd, !handed_over, kept, kept_hist, sm);
     SR_PROF(ap, 15);
 }
 
@@ -2198,14 +2201,21 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
     // workers with a row of their own are few per compute unit: each keeps more of its vectors in flight
     // ... and where there is at most one of them per compute unit, the results of its chunks stay in its registers
     const bool kept = a.own_rows && a.kept && a.chunks <= kKeptChunks;
+    // ... and a launch whose rows all ask for few entries carries the steps that pay for such rows only
+    auto launch = [&](auto epv, auto vec, auto shrt) {
+        constexpr int kE = decltype(epv)::value, kV = decltype(vec)::value;
+        constexpr bool kS = decltype(shrt)::value;
+        if (kept) hipLaunchKernelGGL((k_topk_rows<kE, kV, SR_TK_WINDOW_KEPT, true, kS>), grid, block, 0, stream, a);
+        else if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<kE, kV, SR_TK_WINDOW_OWN, false, kS>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((k_topk_rows<kE, kV, SR_TK_WINDOW, false, kS>), grid, block, 0, stream, a);
+    };
+    using std::integral_constant;
     if (a.dtype == 1) {
-        if (kept) hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW_KEPT, true>), grid, block, 0, stream, a);
-        else if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW_OWN, false>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((k_topk_rows<8, SR_TK_VEC_BF16, SR_TK_WINDOW, false>), grid, block, 0, stream, a);
+        if (a.short_lists) launch(integral_constant<int, 8>{}, integral_constant<int, SR_TK_VEC_BF16>{}, std::true_type{});
+        else launch(integral_constant<int, 8>{}, integral_constant<int, SR_TK_VEC_BF16>{}, std::false_type{});
     } else {
-        if (kept) hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW_KEPT, true>), grid, block, 0, stream, a);
-        else if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW_OWN, false>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((k_topk_rows<4, SR_TK_VEC, SR_TK_WINDOW, false>), grid, block, 0, stream, a);
+        if (a.short_lists) launch(integral_constant<int, 4>{}, integral_constant<int, SR_TK_VEC>{}, std::true_type{});
+        else launch(integral_constant<int, 4>{}, integral_constant<int, SR_TK_VEC>{}, std::false_type{});
     }
     return hipGetLastError();
 }

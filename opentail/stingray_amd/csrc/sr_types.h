@@ -83,6 +83,7 @@ struct SrMaskClear {
 #define SR_TK_WINDOW_KEPT 19               // ... and has a compute unit to itself
 #define SR_TK_MASK_WORDS 3                 // 32-bit keep-words per chunk thread: 19 x 4 and 10 x 8 bits both fit 96
 #define SR_TK_GROUPS 4                     // group maxima per thread
+#define SR_TK_SHORT_SEL 64                 // a launch whose rows all ask for at most this many entries: see k_topk_rows
 #define SR_TK_SEL_MAX 2048                 // most entries (candidates + history ids) the row tail sorts
 #define SR_TK_ROW_CAP 8192                 // candidates all chunks of a row may hand to its tail (16 per thread)
 #define SR_TK_MAX_CHUNKS 128               // most workgroups one row is split over

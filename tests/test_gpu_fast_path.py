@@ -185,13 +185,16 @@ def test_config3_full_chain_with_penalties(ctx):
     _check_rows(ctx, w.logits, w.params, w.uniforms, _cuda(w.logits))
 
 
-@pytest.mark.parametrize("rows,vocab", [(120, 20_011), (150, 20_011), (200, 151_936), (256, 20_011), (300, 20_011), (520, 9_973)])
-def test_every_shape_of_the_launch_gives_the_oracles_tokens(ctx, rows, vocab):
+@pytest.mark.parametrize("rows,vocab,kmax", [(120, 20_011, 1000), (150, 20_011, 1000), (200, 151_936, 1000), (256, 20_011, 1000),
+                                             (300, 20_011, 1000), (520, 9_973, 1000),
+                                             (3, 49_152, 50), (120, 20_011, 64), (150, 20_011, 30), (256, 151_936, 64), (300, 20_011, 8)])
+def test_every_shape_of_the_launch_gives_the_oracles_tokens(ctx, rows, vocab, kmax):
     # The host picks the launch's shape from the number of rows: rows dealt out chunk by chunk over all workers (few
     # rows), one worker per row that keeps the chunk results in its registers (from about half the compute units'
     # number of rows up to one row per compute unit), one worker per row that writes them out (more rows).  Rows of
     # every kind in each: greedy with and without penalties, top-k 1 .. 1000 with top-p / min-p, histories that lower
-    # and that raise, coarse values (ties at every cut), rows with a handful of finite logits.
+    # and that raise, coarse values (ties at every cut), rows with a handful of finite logits.  A batch whose rows all
+    # ask for at most 64 entries (kmax) takes the launches that carry the steps for short lists.
     import torch
 
     rng = np.random.default_rng(rows * 7 + vocab)
@@ -204,7 +207,7 @@ def test_every_shape_of_the_launch_gives_the_oracles_tokens(ctx, rows, vocab):
     for r in range(rows):
         hist = rng.integers(0, vocab, int(rng.integers(1, 70))).tolist()
         kind = r % 6
-        k = int(rng.integers(1, min(1001, vocab)))
+        k = int(rng.integers(1, min(kmax + 1, vocab)))
         if kind == 0:
             p = SamplingParams(Temperature=0.0)
         elif kind == 1:
@@ -216,7 +219,7 @@ def test_every_shape_of_the_launch_gives_the_oracles_tokens(ctx, rows, vocab):
                                PresencePenalty=0.3, FrequencyPenalty=0.1, PreviousTokens=hist)
         elif kind == 4:
             p = SamplingParams(Temperature=0.8, TopK=min(k, 200), RepetitionPenalty=0.8, PresencePenalty=-0.2,
-                               PreviousTokens=hist)               # penalties that raise: the literal over-selection
+                               PreviousTokens=hist if kmax > 64 else hist[:3])  # penalties that raise: the literal over-selection
         else:
             p = SamplingParams(Temperature=1.0, TopK=k, MinP=0.1)
         params.append(p)
