@@ -421,9 +421,35 @@ __device__ __forceinline__ float load_logit(const char* rowp, int i)
     return sr_bf16_to_f32(((const uint16_t*)rowp)[i]);
 }
 
-// A sampled row that no logit bias and no history penalty touches needs no adjusted copy: the masked, scaled logit
-// is recomputed from the input where it is read (the row maximum and the expf pass), which saves one pass.
-__device__ __forceinline__ bool row_is_direct(const SrRow& rd) { return rd.temperature > 0.0f && rd.edit_cnt <= 0; }
+// A sampled row needs no adjusted copy: the masked, scaled logit is recomputed from the input where it is read (the
+// row maximum and the expf pass), which saves one pass over the row and one write of it.  The few ids that a logit
+// bias or a history penalty touches are left out of those two passes -- a bitmap of the vocabulary, read beside the
+// logits like an allow-mask, names them -- and handled by the kernels that run one workgroup per row: k_full_edits
+// computes their adjusted values, keeps them (a.edit_tab: the bitmap, then one float per edit) and folds them into the
+// row's maximum; k_full_row writes their expf before it reads the row.  Without the table (the host gives it when the
+// batch holds such a row), and for a row with more edits than it takes, the row keeps its adjusted copy.
+__device__ __forceinline__ bool row_edits_on_the_fly(const SrRow& rd, const SrFullArgs& a)
+{
+    return a.edit_tab != nullptr && sr_row_edits_on_the_fly(rd, a.vocab);
+}
+__device__ __forceinline__ bool row_is_direct(const SrRow& rd, const SrFullArgs& a)
+{
+    return rd.temperature > 0.0f && (rd.edit_cnt <= 0 || row_edits_on_the_fly(rd, a));
+}
+
+// The value of an edited id before the temperature: LogitBias (Sampler.cs:51-58), then the history penalties
+// (:367-419), on the masked logit.
+__device__ __forceinline__ float edited_logit(float x, const SrEdit& e, const SrRow& rd, bool sampled, bool pen)
+{
+    if (sampled && e.has_bias) x = __fadd_rn(x, e.bias);
+    if (pen && e.occ_all > 0) {
+        if (rd.rep != 1.0f)
+            for (int o = 0; o < e.occ_win; o++) x = x > 0.0f ? __fdiv_rn(x, rd.rep) : __fmul_rn(x, rd.rep);
+        if (rd.presence != 0.0f || rd.frequency != 0.0f)
+            x = __fsub_rn(x, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)e.occ_all)));
+    }
+    return x;
+}
 
 // ---- one pass of the grid's x dimension over a row of logits ---------------------------------------------
 // The masked (and temperature-scaled) logits of a row, sixteen input bytes per thread and load, four loads in flight;
@@ -435,6 +461,7 @@ struct RowSource {
     const uint32_t* mrow;
     bool scale;
     float inv_temp;
+    const uint32_t* erow = nullptr;  // bitmap of the ids the row's edits touch (body gets the bits of its run), or null
     __device__ __forceinline__ float fix(float x, uint32_t keep) const
     {
         if (!keep) x = SR_NEG_INF;
@@ -449,15 +476,17 @@ __device__ __forceinline__ void stream_row(const RowSource<ES>& src, int n, Body
     const int step = (int)gridDim.x * 256;
     for (int v0 = (int)blockIdx.x * 256 + (int)threadIdx.x; v0 < nv; v0 += step * kU) {
         uint4 raw[kU];
-        uint32_t keep[kU];
+        uint32_t keep[kU], hit[kU];
 #pragma unroll
         for (int u = 0; u < kU; u++) {
             const int v = v0 + u * step;
             raw[u] = make_uint4(0u, 0u, 0u, 0u);
             keep[u] = 0xffu;
+            hit[u] = 0u;
             if (v < nv) {
                 raw[u] = ((const uint4*)src.rowp)[v];
                 if (src.mrow) keep[u] = src.mrow[(v * E) >> 5] >> ((v * E) & 31);
+                if (src.erow) hit[u] = (src.erow[(v * E) >> 5] >> ((v * E) & 31)) & ((1u << E) - 1u);
             }
         }
 #pragma unroll
@@ -477,13 +506,13 @@ __device__ __forceinline__ void stream_row(const RowSource<ES>& src, int n, Body
             }
 #pragma unroll
             for (int q = 0; q < E; q++) x[q] = src.fix(x[q], (keep[u] >> q) & 1u);
-            body(v * E, x, E);
+            body(v * E, x, E, hit[u]);
         }
     }
     for (int i = nv * E + (int)blockIdx.x * 256 + (int)threadIdx.x; i < n; i += step) {
         float x[E];
         x[0] = src.fix(load_logit<ES>(src.rowp, i), src.mrow ? (src.mrow[i >> 5] >> (i & 31)) & 1u : 1u);
-        body(i, x, 1);
+        body(i, x, 1, src.erow ? (src.erow[i >> 5] >> (i & 31)) & 1u : 0u);
     }
 }
 // stores c values (c = 1, 4 or 8) at w + i, with 16-byte stores where the address allows
@@ -513,12 +542,8 @@ __global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
     src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
     src.scale = rd.temperature > 0.0f && rd.temperature != 1.0f;
     src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-        a.state[slot].maxkey = 0u;
-        a.state[slot].mul1 = a.state[slot].mul2 = 1.0f;
-    }
-    if (row_is_direct(rd)) return;  // nothing edits this row: the kernels behind read the logits themselves
-    stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c) { store_run(w, i, x, c); });
+    if (row_is_direct(rd, a)) return;  // the kernels behind read the logits themselves
+    stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c, uint32_t) { store_run(w, i, x, c); });
 }
 
 // ---- stage 2: logit bias and history penalties on the few ids they touch (Sampler.cs:51-58, :367-419)
@@ -528,7 +553,42 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
     const int slot = blockIdx.x;
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
+    if (threadIdx.x == 0) {  // (the first kernel of the pipeline that runs for every row)
+        a.state[slot].maxkey = 0u;
+        a.state[slot].mul1 = a.state[slot].mul2 = 1.0f;
+    }
     if (rd.edit_cnt <= 0) return;
+    const SrEdit* ed = a.edits + rd.edit_off;
+    if (row_edits_on_the_fly(rd, a)) {
+        // the row's bitmap (cleared first: the barrier's wait for the stores stands between them and the atomics on
+        // the same words), the adjusted and scaled values of its edits, and their share of the row's maximum
+        const int words = (a.vocab + 31) / 32;
+        uint32_t* tab = a.edit_tab + (size_t)slot * (size_t)a.edit_tab_stride;
+        float* vals = (float*)(tab + words);
+        for (int i = threadIdx.x; i < words; i += 256) tab[i] = 0u;
+        sr_drain_stores();  // (not a fence: a release at device scope writes the whole L2 back)
+        __syncthreads();
+        const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+        const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+        const bool scale = rd.temperature != 1.0f;
+        const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+        const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u;
+        uint32_t k = 0u;
+        for (int e = threadIdx.x; e < rd.edit_cnt; e += 256) {
+            const int id = ed[e].id;
+            atomicOr(&tab[id >> 5], 1u << (id & 31));
+            float x = load_logit<ES>(rowp, id);
+            if (mrow && !((mrow[id >> 5] >> (id & 31)) & 1u)) x = SR_NEG_INF;
+            x = edited_logit(x, ed[e], rd, true, pen);
+            if (scale) x = __fmul_rn(x, inv_temp);
+            vals[e] = x;
+            const uint32_t kv = (x != x) ? 0xffffffffu : sr_okey(x);  // NaN propagates (TensorPrimitives.Max)
+            k = kv > k ? kv : k;
+        }
+        k = sr_wave_max_u32(k);
+        if (sr_lane() == 0 && k != 0u) atomicMax(&a.state[slot].maxkey, k);
+        return;
+    }
     const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
     float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
     const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
@@ -536,18 +596,11 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
     const bool scale = sampled && rd.temperature != 1.0f;
     const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
     const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u;
-    const SrEdit* ed = a.edits + rd.edit_off;
     for (int e = threadIdx.x; e < rd.edit_cnt; e += 256) {
         const int id = ed[e].id;
         float x = load_logit<ES>(rowp, id);
         if (mrow && !((mrow[id >> 5] >> (id & 31)) & 1u)) x = SR_NEG_INF;
-        if (sampled && ed[e].has_bias) x = __fadd_rn(x, ed[e].bias);
-        if (pen && ed[e].occ_all > 0) {
-            if (rd.rep != 1.0f)
-                for (int o = 0; o < ed[e].occ_win; o++) x = x > 0.0f ? __fdiv_rn(x, rd.rep) : __fmul_rn(x, rd.rep);
-            if (rd.presence != 0.0f || rd.frequency != 0.0f)
-                x = __fsub_rn(x, __fadd_rn(rd.presence, __fmul_rn(rd.frequency, (float)ed[e].occ_all)));
-        }
+        x = edited_logit(x, ed[e], rd, sampled, pen);
         if (scale) x = __fmul_rn(x, inv_temp);
         w[id] = x;
     }
@@ -569,16 +622,18 @@ __global__ __launch_bounds__(256) void k_full_max(SrFullArgs a)
         const uint32_t kv = (v != v) ? 0xffffffffu : sr_okey(v);  // NaN propagates (TensorPrimitives.Max)
         k = kv > k ? kv : k;
     };
-    if (row_is_direct(rd)) {
+    if (row_is_direct(rd, a)) {
         RowSource<ES> src;
         src.rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
         src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
         src.scale = rd.temperature != 1.0f;
         src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
-        stream_row<ES>(src, a.vocab, [&](int, const float (&x)[16 / ES], int c) {
+        // (ids that the row's edits touch are not looked at: k_full_edits has folded their adjusted values in)
+        src.erow = rd.edit_cnt > 0 ? a.edit_tab + (size_t)slot * (size_t)a.edit_tab_stride : nullptr;
+        stream_row<ES>(src, a.vocab, [&](int, const float (&x)[16 / ES], int c, uint32_t hit) {
 #pragma unroll
             for (int q = 0; q < 16 / ES; q++)
-                if (q < c) fold(x[q]);
+                if (q < c && ((hit >> q) & 1u) == 0u) fold(x[q]);
         });
     } else {
         RowSource<4> src;  // the adjusted copy
@@ -586,7 +641,7 @@ __global__ __launch_bounds__(256) void k_full_max(SrFullArgs a)
         src.mrow = nullptr;
         src.scale = false;
         src.inv_temp = 1.0f;
-        stream_row<4>(src, a.vocab, [&](int, const float (&x)[4], int c) {
+        stream_row<4>(src, a.vocab, [&](int, const float (&x)[4], int c, uint32_t) {
 #pragma unroll
             for (int q = 0; q < 4; q++)
                 if (q < c) fold(x[q]);
@@ -614,13 +669,14 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
     if (threadIdx.x < 32) tab[threadIdx.x] = sr_exp2f_tab[threadIdx.x];
     __syncthreads();
     float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
-    if (row_is_direct(rd)) {
+    if (row_is_direct(rd, a)) {
         RowSource<ES> src;
         src.rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
         src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
         src.scale = rd.temperature != 1.0f;
         src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
-        stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c) {
+        // (what is written for an id that the row's edits touch does not matter: k_full_row writes it again)
+        stream_row<ES>(src, a.vocab, [&](int i, const float (&x)[16 / ES], int c, uint32_t) {
             float e[16 / ES];
 #pragma unroll
             for (int q = 0; q < 16 / ES; q++) e[q] = q < c ? sr_expf_tab(__fsub_rn(x[q], m), tab) : 0.0f;
@@ -632,7 +688,7 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
         src.mrow = nullptr;
         src.scale = false;
         src.inv_temp = 1.0f;
-        stream_row<4>(src, a.vocab, [&](int i, const float (&x)[4], int c) {
+        stream_row<4>(src, a.vocab, [&](int i, const float (&x)[4], int c, uint32_t) {
             float e[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) e[q] = q < c ? sr_expf_tab(__fsub_rn(x[q], m), tab) : 0.0f;
@@ -772,6 +828,15 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             flags |= SR_KFLAG_DEGENERATE;
             __syncthreads();
         } else {
+            if (row_edits_on_the_fly(rd, a)) {
+                // the ids that the row's edits touch were left out of the expf pass: their e, from the adjusted values
+                // that k_full_edits kept
+                const float* vals = (const float*)(a.edit_tab + (size_t)slot * (size_t)a.edit_tab_stride + (n + 31) / 32);
+                const SrEdit* ed = a.edits + rd.edit_off;
+                for (int e = tid; e < rd.edit_cnt; e += kT) p[ed[e].id] = sr_expf(__fsub_rn(vals[e], m));
+                sr_drain_stores();  // (this compute unit has not read these lines before: the loads below find them in L2)
+                __syncthreads();
+            }
             int dummy;
             const float sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm);
             __syncthreads();
@@ -1356,11 +1421,12 @@ hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
     if (n_rows <= 0) return hipSuccess;
     const int bx = max(1, min(64, (a.vocab + 256 * 16 - 1) / (256 * 16)));
     dim3 grid(bx, n_rows);
+    // (the adjusted copy only where some row keeps one: the host knows)
     if (a.dtype == 1) {
-        hipLaunchKernelGGL(k_full_prep<2>, grid, dim3(256), 0, st, a);
+        if (a.any_copy) hipLaunchKernelGGL(k_full_prep<2>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(k_full_edits<2>, dim3(n_rows), dim3(256), 0, st, a);
     } else {
-        hipLaunchKernelGGL(k_full_prep<4>, grid, dim3(256), 0, st, a);
+        if (a.any_copy) hipLaunchKernelGGL(k_full_prep<4>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(k_full_edits<4>, dim3(n_rows), dim3(256), 0, st, a);
     }
     if (a.dtype == 1) {

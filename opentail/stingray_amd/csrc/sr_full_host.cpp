@@ -12,7 +12,7 @@ namespace {
 //   mode 0: work rows live in ctx scratch, tokens out.   mode 1/2: work rows ARE the caller's probs rows.
 int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows, bool any_top_p, const void* logits_dev,
              int dtype, int64_t row_stride, int mode, float* probs_dev, int64_t probs_stride, int32_t* out_tokens_dev,
-             uint32_t* out_flags_dev, bool lazy_scale = false)
+             uint32_t* out_flags_dev, bool lazy_scale = false, const std::vector<SrRow>* host_rows = nullptr)
 {
     if (n_rows <= 0) return SR_OK;
     hipStream_t st = ctx->stream;
@@ -42,6 +42,22 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     }
     a.two_phase = any_top_p ? 1 : 0;
     a.lazy_scale = lazy_scale ? 1 : 0;
+    // Which of the rows that come here keep an adjusted copy, and which have their edits applied where they are read
+    // (the rows of the batch that take this path: every row in modes 1 / 2).
+    bool any_table = false, any_copy = false;
+    for (const SrRow& r : (host_rows ? *host_rows : b->h_rows)) {
+        if (mode == 0 && r.path != SR_PATH_FULL) continue;
+        const bool on_the_fly = sr_row_edits_on_the_fly(r, vocab);
+        any_table = any_table || on_the_fly;
+        any_copy = any_copy || !(r.temperature > 0.0f && (r.edit_cnt <= 0 || on_the_fly));
+    }
+    a.any_copy = any_copy ? 1 : 0;
+    a.edit_tab = nullptr;
+    a.edit_tab_stride = (((int64_t)vocab + 31) / 32 + SR_FULL_EDIT_VALUES + 3) & ~(int64_t)3;
+    if (any_table) {
+        SR_HIP(ctx, ctx->edit_tab.reserve((size_t)n_rows * (size_t)a.edit_tab_stride * sizeof(uint32_t), st));
+        a.edit_tab = ctx->edit_tab.as<uint32_t>();
+    }
     SR_HIP(ctx, ctx->full_state.reserve((size_t)n_rows * sizeof(SrFullState), st));
     a.state = ctx->full_state.as<SrFullState>();
     SR_HIP(ctx, ctx->seg.reserve((size_t)n_rows * 2 * sizeof(int32_t), st));
@@ -442,7 +458,7 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
     int rc = identity_list(ctx, rows * P, &list);
     if (rc == SR_OK)
         rc = run_full(ctx, &tmp, list, rows * P, any_top_p, target_logits_dev, SR_DTYPE_F32, V, 1, ctx->spec_probs.as<float>(), V,
-                      nullptr, nullptr, true);  // (the verifier applies the normalising factors of unfiltered rows itself)
+                      nullptr, nullptr, true, &b->h_rows);  // (the verifier applies the normalising factors of unfiltered rows itself)
     tmp.d_rows.p = nullptr;  // borrowed
     tmp.d_edits.p = nullptr;
     if (rc != SR_OK) return rc;

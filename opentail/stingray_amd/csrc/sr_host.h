@@ -186,6 +186,7 @@ struct sr_ctx {
     unsigned long long* static_best = nullptr;
     uint32_t* static_done = nullptr;
     DeviceBuf work;          // fp32 rows of the full-vocabulary path
+    DeviceBuf edit_tab;      // per row: the table of its edits (bitmap of the vocabulary + slots)
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits
     DeviceBuf stage_probs;   // staging for host-resident distributions

@@ -21,6 +21,14 @@
 // the row's edits are sorted by id (else they stand in order of first appearance in the history)
 #define SR_ROWFLAG_EDITS_SORTED (1u << 10)
 
+// A sampled full-vocabulary row that keeps no adjusted copy of its logits although bias or penalties touch some ids
+// (host and device agree on this: the host provides the rows' tables when a batch holds such a row).
+#define SR_FULL_EDIT_VALUES 2048
+static inline __host__ __device__ bool sr_row_edits_on_the_fly(const SrRow& rd, int)
+{
+    return rd.temperature > 0.0f && rd.edit_cnt > 0 && rd.edit_cnt <= SR_FULL_EDIT_VALUES;
+}
+
 #define SR_TK_MAX_XCD 16
 struct SrTopkArgs {
     const void* logits;
@@ -140,6 +148,9 @@ struct SrFullArgs {
     int32_t two_phase;         // a device-wide sort of large nuclei runs between phase 1 and phase 2
     int32_t lazy_scale;        // mode 1 only: rows that no filter touches keep expf(x - max); their two normalising
                                // factors go to state[slot].mul1 / mul2 for the reader to apply
+    uint32_t* edit_tab;        // [slot][edit_tab_stride]: per row a bitmap of the ids its edits touch and one float per
+    int64_t edit_tab_stride;   // edit (the adjusted value), for sampled rows that keep no adjusted copy; or null
+    int32_t any_copy;          // some row keeps an adjusted copy of its logits (greedy rows, rows the table does not take)
     SrFullState* state;        // [slot]
     uint32_t* sort_keys_in;    // [slot][sort_stride]
     int32_t* sort_vals_in;
