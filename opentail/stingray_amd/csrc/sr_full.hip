@@ -187,7 +187,7 @@ __device__ __forceinline__ float seq_sum_tiles(IssueFast issue_fast, IssueAny is
                 if (t >= n_full) break;
                 issue_fast(min(t + kDepth - 1, n_full - 1) * SR_SEQ_TILE, r[(k + kDepth - 1) % kDepth]);
                 float x[SR_SEQ_RUN];
-                finish(r[k], x);
+                finish(r[k], x, t * SR_SEQ_TILE);
                 int f;
                 sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
                 if (kSearch && f >= 0) {
@@ -201,7 +201,7 @@ __device__ __forceinline__ float seq_sum_tiles(IssueFast issue_fast, IssueAny is
         Raw r;
         issue_any(base, r);
         float x[SR_SEQ_RUN];
-        finish(r, x);
+        finish(r, x, base);
         int f;
         sr_seq_tile<kSearch>(x, &s, target, &f, sm.seq);
         if (kSearch && f >= 0) {
@@ -241,9 +241,13 @@ __device__ __forceinline__ void seq_load_run(const float* p, bool aligned, int i
 }
 
 // (every term is multiplied by m1 and then by m2 first: the two normalising factors of a row that was left unscaled)
-template <bool kSearch>
+struct SeqNoWatch {
+    __device__ __forceinline__ void operator()(float, int) const {}
+};
+// watch(x, i) sees every term with its index as it passes (the terms of a tile are looked at before the tile is added)
+template <bool kSearch, typename Watch = SeqNoWatch>
 __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm,
-                                             float m1 = 1.0f, float m2 = 1.0f)
+                                             float m1 = 1.0f, float m2 = 1.0f, Watch watch = Watch())
 {
     static_assert(SR_SEQ_ACTIVE == SR_SEQ_THREADS, "every thread of the block loads a run");
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
@@ -253,9 +257,12 @@ __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, fl
     auto issue_any = [&](int base, SeqRaw1& r) __attribute__((always_inline)) {
         seq_load_run(p, aligned, base + (int)threadIdx.x * SR_SEQ_RUN, n, r.v);
     };
-    auto finish = [&](const SeqRaw1& r, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
+    auto finish = [&](const SeqRaw1& r, float (&x)[SR_SEQ_RUN], int base) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < SR_SEQ_RUN; j++) x[j] = __fmul_rn(__fmul_rn(r.v[j], m1), m2);
+        for (int j = 0; j < SR_SEQ_RUN; j++) {
+            x[j] = __fmul_rn(__fmul_rn(r.v[j], m1), m2);
+            watch(x[j], base + (int)threadIdx.x * SR_SEQ_RUN + j);
+        }
     };
     return seq_sum_tiles<kSearch, 3, SeqRaw1>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm);
 }
@@ -276,7 +283,7 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
         seq_load_run(p, aligned, i0, n, r.p);
         seq_load_run(q, aligned, i0, n, r.q);
     };
-    auto finish = [&](const SeqRaw2& r, float (&x)[SR_SEQ_RUN]) __attribute__((always_inline)) {
+    auto finish = [&](const SeqRaw2& r, float (&x)[SR_SEQ_RUN], int) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < SR_SEQ_RUN; j++) {
             const float d = __fsub_rn(__fmul_rn(__fmul_rn(r.p[j], m1), m2), r.q[j]);
@@ -838,8 +845,30 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 __syncthreads();
             }
             int dummy;
-            const float sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm);
+            // A row that min-p cuts, with no top-k stage before the cut and no distribution to hand out, is not read a
+            // second time for the cut: a survivor has fl(e * inv) >= fl(min_p * inv), so e >= min_p * (1 - 2^-22), and
+            // the few entries that large are listed while the sum passes over them; the exact test follows below.
+            const bool watch_min_p = rd.min_p > 0.0f && !(rd.top_k > 0 && rd.top_k < n) && a.mode == 0 && n >= 8;
+            const float e_low = __fmul_rn(rd.min_p, 0.999999f);
+            if (watch_min_p) {
+                if (tid == 0) sm.bc[4] = 0u;
+                __syncthreads();
+            }
+            float sum;
+            if (watch_min_p) {
+                sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm, 1.0f, 1.0f, [&](float x, int i) {
+                    if (x >= e_low) {
+                        const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
+                        if (pos < (uint32_t)kSmall)
+                            sm.sortbuf[pos] = ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+                    }
+                });
+            } else {
+                sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm);
+            }
             __syncthreads();
+            const int n_watched = watch_min_p ? (int)sm.bc[4] : -1;
+            const bool from_watch = n_watched >= 0 && n_watched <= kSmall;  // (else the row is read again, as before)
             FPROF(a, slot, 2);
             const bool do_scale = sum > 0.0f && sum != 1.0f;
             const float inv = do_scale ? __fdiv_rn(1.0f, sum) : 1.0f;
@@ -891,7 +920,24 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                     return y;
                 };
                 const bool read_only = list_now && a.mode == 0 && n >= 8;
-                if (read_only) row_pass<false>(p, n, body); else row_pass<true>(p, n, body);
+                if (from_watch) {
+                    // the entries listed during the sum, put to the exact test; the survivors are listed again
+                    static_assert(kSmall % kT == 0, "whole candidates per thread");
+                    unsigned long long cand[kSmall / kT];
+#pragma unroll
+                    for (int r = 0; r < kSmall / kT; r++) cand[r] = (r * kT + tid < n_watched) ? sm.sortbuf[r * kT + tid] : 0ull;
+                    __syncthreads();
+                    if (tid == 0) sm.bc[4] = 0u;
+                    __syncthreads();
+#pragma unroll
+                    for (int r = 0; r < kSmall / kT; r++)
+                        if (r * kT + tid < n_watched)
+                            (void)body(sr_u2f((uint32_t)(cand[r] >> 32)), (int)(0xffffffffu - (uint32_t)cand[r]));
+                } else if (read_only) {
+                    row_pass<false>(p, n, body);
+                } else {
+                    row_pass<true>(p, n, body);
+                }
                 survivors = c;
                 fused = true;
                 if (list_now) {
