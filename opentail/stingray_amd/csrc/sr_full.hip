@@ -996,6 +996,43 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             // few.  Only a row that makes no progress (more than kSmall probabilities inside one bucket) or needs
             // more than kMaxSlabs slabs has its survivors sorted device-wide.
             constexpr int kMaxSlabs = 24;
+            // A row that needs several slabs has all their bounds from one histogram of its probabilities' 16-bit keys
+            // instead of two select passes per slab.  The histogram is counted in LDS (the slabs' sort buffer, free
+            // until the first slab): position d = 0x3fff - key, so that positions ascend as the values fall; 8,192
+            // positions reach down to 2^-63, what lies below shares the last one.  Its running sums go to the row's
+            // segment of the sort buffers: sums[d] = survivors at positions <= d, and the position that holds the
+            // kSmall-th largest of what is left is the first d with sums[d] >= taken + kSmall.
+            constexpr int kPos = 8192;
+            static_assert(kPos * 4 <= kSmall * 8 && kPos % kT == 0, "the histogram fits the sort buffer");
+            constexpr int kPer = kPos / kT;
+            uint32_t* sums = a.sort_keys_in + (size_t)slot * a.sort_stride;
+            bool use_hist = !have_list && ns > kSmall && a.sort_stride >= kPos;
+            if (use_hist) {
+                uint32_t* cnt = (uint32_t*)sm.sortbuf;
+                for (int i = tid; i < kPos; i += kT) cnt[i] = 0u;
+                if (tid == 0) sm.bc[5] = 0u;
+                __syncthreads();
+                row_pass<false>(p, n, [&](float v, int) -> float {
+                    if (v > 0.0f) {
+                        const uint32_t key = sr_f2u(v) >> 16;
+                        if (key <= 0x3fffu) atomicAdd(&cnt[min(0x3fffu - key, (uint32_t)(kPos - 1))], 1u);
+                        else sm.bc[5] = 1u;  // (no probability is 2 or more; if one is, the slabs take the other way)
+                    }
+                    return v;
+                });
+                __syncthreads();
+                use_hist = sm.bc[5] == 0u;
+                uint32_t mine[kPer];
+                int own = 0;
+#pragma unroll
+                for (int q = 0; q < kPer; q++) { mine[q] = cnt[tid * kPer + q]; own += (int)mine[q]; }
+                int tot;
+                int upto = blk_excl_scan(own, &tot, sm);
+#pragma unroll
+                for (int q = 0; q < kPer; q++) { upto += (int)mine[q]; sums[tid * kPer + q] = (uint32_t)upto; }
+                sr_drain_stores();
+                __syncthreads();
+            }
             bool closed = false;
             float run = 0.0f;                  // exact running sum behind the slabs taken so far
             int taken = 0;                     // survivors in those slabs
@@ -1003,7 +1040,31 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             float c_above = -1.0f;             // the current slab: probabilities strictly above this value ...
             for (int slab = 0; slab < kMaxSlabs && ns > 0 && !closed; slab++) {
                 const bool last_slab = ns - taken <= kSmall;  // everything that is left fits
-                c_above = last_slab ? 0.0f : sr_u2f(sr_f2u(kth_largest(p, n, kSmall, sm, 16, hi_key)) | 0xffffu);
+                if (last_slab) {
+                    c_above = 0.0f;
+                } else if (use_hist) {
+                    const uint32_t target = (uint32_t)(taken + kSmall);
+                    // the one thread whose positions hold the first d with sums[d] >= target names it
+                    const uint32_t last = sums[tid * kPer + kPer - 1], before = tid > 0 ? sums[tid * kPer - 1] : 0u;
+                    if (last >= target && before < target) {
+                        int d = tid * kPer + kPer - 1;
+#pragma unroll
+                        for (int q = kPer - 2; q >= 0; q--)
+                            if (sums[tid * kPer + q] >= target) d = tid * kPer + q;
+                        sm.bc[5] = (uint32_t)d;
+                    }
+                    __syncthreads();
+                    const uint32_t d = sm.bc[5];
+                    __syncthreads();
+                    if (d < (uint32_t)(kPos - 1)) {
+                        c_above = sr_u2f(((0x3fffu - d) << 16) | 0xffffu);
+                    } else {  // (the shared last position: its keys are not one bucket)
+                        use_hist = false;
+                        c_above = sr_u2f(sr_f2u(kth_largest(p, n, kSmall, sm, 16, hi_key)) | 0xffffu);
+                    }
+                } else {
+                    c_above = sr_u2f(sr_f2u(kth_largest(p, n, kSmall, sm, 16, hi_key)) | 0xffffu);
+                }
                 int nc;
                 if (have_list) {
                     nc = ns;  // (ns <= kSmall: the survivors were listed while the row was scaled)
