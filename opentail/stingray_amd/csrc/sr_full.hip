@@ -15,8 +15,11 @@ namespace {
 
 #ifdef SR_PROFILE
 #define FPROF(a, slot_, i_) do { if ((a).prof && (slot_) == 0 && threadIdx.x == 0) (a).prof[(i_)] = (unsigned long long)wall_clock64(); } while (0)
+// (adds the time since *t_ to stamp i_ and moves *t_ on: for the steps of a loop)
+#define FPROF_ADD(a, slot_, i_, t_) do { if ((a).prof && (slot_) == 0 && threadIdx.x == 0) { const unsigned long long now_ = (unsigned long long)wall_clock64(); (a).prof[(i_)] += now_ - (t_); (t_) = now_; } } while (0)
 #else
 #define FPROF(a, slot_, i_) do { } while (0)
+#define FPROF_ADD(a, slot_, i_, t_) do { } while (0)
 #endif
 
 constexpr int kT = SR_SEQ_THREADS;
@@ -34,6 +37,7 @@ struct FullSmem {
     uint32_t bc[16];
     unsigned long long sortbuf[kSmall];
     float sprob[kSmall];
+    uint32_t tags[kSmall];
 };
 
 // ---- block reductions ------------------------------------------------------------------------------
@@ -245,9 +249,13 @@ struct SeqNoWatch {
     __device__ __forceinline__ void operator()(float, int) const {}
 };
 // watch(x, i) sees every term with its index as it passes (the terms of a tile are looked at before the tile is added)
-template <bool kSearch, typename Watch = SeqNoWatch>
+struct SeqNoMap {
+    __device__ __forceinline__ float operator()(float x, int) const { return x; }
+};
+// map(x, i) stands between a scaled term and the sum: the term that is added (and watched) is what it returns
+template <bool kSearch, typename Watch = SeqNoWatch, typename Map = SeqNoMap>
 __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm,
-                                             float m1 = 1.0f, float m2 = 1.0f, Watch watch = Watch())
+                                             float m1 = 1.0f, float m2 = 1.0f, Watch watch = Watch(), Map map = Map())
 {
     static_assert(SR_SEQ_ACTIVE == SR_SEQ_THREADS, "every thread of the block loads a run");
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
@@ -260,7 +268,7 @@ __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, fl
     auto finish = [&](const SeqRaw1& r, float (&x)[SR_SEQ_RUN], int base) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < SR_SEQ_RUN; j++) {
-            x[j] = __fmul_rn(__fmul_rn(r.v[j], m1), m2);
+            x[j] = map(__fmul_rn(__fmul_rn(r.v[j], m1), m2), base + (int)threadIdx.x * SR_SEQ_RUN + j);
             watch(x[j], base + (int)threadIdx.x * SR_SEQ_RUN + j);
         }
     };
@@ -404,22 +412,138 @@ __device__ __forceinline__ float kth_largest(const float* p, int n, int k, FullS
     return sr_u2f(prefix);
 }
 
-// bitonic sort (descending) of sm.sortbuf[0 .. n_pow2)
-__device__ __forceinline__ void sort_small_desc(FullSmem& sm, int n_pow2)
+// The value of lane (lane ^ kMask), moved by the vector unit alone (no LDS): DPP inside rows of 16 lanes, the swaps of
+// rows and of wave halves beyond.  Every lane of the wave must be active.
+template <int kMask> __device__ __forceinline__ uint32_t lane_xor_u32(uint32_t v)
 {
-    for (int k2 = 2; k2 <= n_pow2; k2 <<= 1) {
-        for (int j2 = k2 >> 1; j2 > 0; j2 >>= 1) {
-            for (int i = threadIdx.x; i < n_pow2; i += kT) {
-                const int ixj = i ^ j2;
-                if (ixj > i) {
-                    const unsigned long long a = sm.sortbuf[i], b = sm.sortbuf[ixj];
-                    if ((a < b) == ((i & k2) == 0)) { sm.sortbuf[i] = b; sm.sortbuf[ixj] = a; }
+    static_assert(kMask == 1 || kMask == 2 || kMask == 4 || kMask == 8 || kMask == 16 || kMask == 32, "one bit of the lane number");
+    if (kMask == 1) return sr_dpp_u32<0xB1>(v);                        // quad_perm [1, 0, 3, 2]
+    if (kMask == 2) return sr_dpp_u32<0x4E>(v);                        // quad_perm [2, 3, 0, 1]
+    if (kMask == 4) return sr_dpp_u32<0x1B>(sr_dpp_u32<0x141>(v));     // 7 - l inside eight lanes, then 3 - l inside four
+    if (kMask == 8) return sr_dpp_u32<0x128>(v);                       // a row rotated by half its length
+    if (kMask == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+        return (sr_lane() & 16) ? r[0] : r[1];
+    }
+    const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return (sr_lane() & 32) ? r[0] : r[1];
+}
+template <int kMask> __device__ __forceinline__ unsigned long long lane_xor_key(unsigned long long v)
+{
+    return ((unsigned long long)lane_xor_u32<kMask>((uint32_t)(v >> 32)) << 32) | (unsigned long long)lane_xor_u32<kMask>((uint32_t)v);
+}
+template <int kMask> __device__ __forceinline__ uint32_t lane_xor_key(uint32_t v) { return lane_xor_u32<kMask>(v); }
+
+// Bitonic sort (descending) of buf[0 .. n_pow2) in LDS, n_pow2 a power of two <= kSmall, keys of 32 or 64 bits; entries
+// that must come last are zero.  All threads call, behind a barrier that follows the last write of the entries.
+//
+// The entries live in registers, four consecutive ones per thread (a wave holds 256 consecutive entries): strides 1 and
+// 2 pair registers of one thread, strides 4..128 pair lanes of one wave, and LDS is needed only for the strides of 256
+// and more.  Those come at the start of the last merges (sizes 512 and up); all of them of one merge are done in one
+// visit to LDS, by 256 threads that each hold one column (entries c, c + 256, c + 512, ...).
+template <typename K>
+__device__ __forceinline__ void sort_lds_desc(K* buf, int n_pow2)
+{
+    constexpr int kRow = 256;                 // entries of one wave
+    constexpr int kCols = kSmall / kRow;      // most entries of one column
+    static_assert(kRow == 4 * SR_WAVE && kRow * kW >= kSmall && kCols == 16, "the layout described above");
+    const int tid = threadIdx.x, wave = sr_wave_id();
+    if (n_pow2 <= kRow) {
+        // A short list: every entry counts the entries that come before it (equal ones by their place).
+        K key = 0;
+        int rank = 0;
+        if (tid < n_pow2) {
+            key = buf[tid];
+            for (int j = 0; j < n_pow2; j++) {
+                const K o = buf[j];
+                rank += (o > key || (o == key && j < tid)) ? 1 : 0;
+            }
+        }
+        __syncthreads();
+        if (tid < n_pow2) buf[rank] = key;
+        __syncthreads();
+        return;
+    }
+    const int base = 4 * tid;
+    const int pe = max(n_pow2, 4);
+    const bool wave_has = wave * kRow < pe;   // (the other waves only meet at the barriers)
+    K v[4];
+    auto load_rows = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = (base + r < n_pow2) ? buf[base + r] : (K)0;
+    };
+    auto store_rows = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            if (base + r < n_pow2) buf[base + r] = v[r];
+    };
+    auto cx = [&](K& lo_i, K& hi_i, bool desc) __attribute__((always_inline)) {  // lo_i is the entry with the smaller index
+        const K mx = lo_i > hi_i ? lo_i : hi_i, mn = lo_i > hi_i ? hi_i : lo_i;
+        lo_i = desc ? mx : mn;
+        hi_i = desc ? mn : mx;
+    };
+    auto lane_step = [&](auto mask, bool want_max) __attribute__((always_inline)) {
+        constexpr int kM = decltype(mask)::value;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const K o = lane_xor_key<kM>(v[r]);
+            const K mx = v[r] > o ? v[r] : o, mn = v[r] > o ? o : v[r];
+            v[r] = want_max ? mx : mn;
+        }
+    };
+    // the steps of merge size k2 with strides j_first, j_first / 2, ..., 1 (j_first <= 128)
+    auto row_steps = [&](int k2, int j_first) __attribute__((always_inline)) {
+        const bool desc = (base & k2) == 0;  // (k2 >= 4: the four entries share it; k2 == 2 is handled below)
+        if (j_first >= 128) lane_step(std::integral_constant<int, 32>{}, desc == ((base & 128) == 0));
+        if (j_first >= 64) lane_step(std::integral_constant<int, 16>{}, desc == ((base & 64) == 0));
+        if (j_first >= 32) lane_step(std::integral_constant<int, 8>{}, desc == ((base & 32) == 0));
+        if (j_first >= 16) lane_step(std::integral_constant<int, 4>{}, desc == ((base & 16) == 0));
+        if (j_first >= 8) lane_step(std::integral_constant<int, 2>{}, desc == ((base & 8) == 0));
+        if (j_first >= 4) lane_step(std::integral_constant<int, 1>{}, desc == ((base & 4) == 0));
+        if (k2 == 2) {
+            cx(v[0], v[1], true);
+            cx(v[2], v[3], false);
+        } else {
+            cx(v[0], v[2], desc);
+            cx(v[1], v[3], desc);
+            cx(v[0], v[1], desc);
+            cx(v[2], v[3], desc);
+        }
+    };
+    if (wave_has) {
+        load_rows();
+        for (int k2 = 2; k2 <= min(pe, kRow); k2 <<= 1) row_steps(k2, k2 >> 1);
+    }
+    for (int k2 = 2 * kRow; k2 <= pe; k2 <<= 1) {
+        if (wave_has) store_rows();
+        __syncthreads();
+        if (tid < kRow) {
+            const int cols = pe / kRow;  // 2, 4, 8 or 16 entries in this thread's column
+            K c[kCols];
+#pragma unroll
+            for (int a2 = 0; a2 < kCols; a2++) c[a2] = a2 < cols ? buf[tid + a2 * kRow] : (K)0;
+#pragma unroll
+            for (int ja = kCols / 2; ja >= 1; ja >>= 1) {
+                if (ja * kRow * 2 <= k2) {
+#pragma unroll
+                    for (int a2 = 0; a2 < kCols; a2++)
+                        if ((a2 & ja) == 0 && (a2 | ja) < cols) cx(c[a2], c[a2 | ja], ((a2 * kRow) & k2) == 0);
                 }
             }
-            __syncthreads();
+#pragma unroll
+            for (int a2 = 0; a2 < kCols; a2++)
+                if (a2 < cols) buf[tid + a2 * kRow] = c[a2];
+        }
+        __syncthreads();
+        if (wave_has) {
+            load_rows();
+            row_steps(k2, kRow / 2);
         }
     }
+    if (wave_has) store_rows();
+    __syncthreads();
 }
+__device__ __forceinline__ void sort_small_desc(FullSmem& sm, int n_pow2) { sort_lds_desc(sm.sortbuf, n_pow2); }
 
 template <int ES>
 __device__ __forceinline__ float load_logit(const char* rowp, int i)
@@ -728,11 +852,136 @@ __device__ __forceinline__ int draw_from_row(const float* p, int n, double u, Fu
     return found >= 0 ? found : n - 1;
 }
 
-// Final Normalize (Sampler.cs:91-92, :553-562) and draw (:564-576) of a row whose m survivors are listed in
-// sm.sortbuf (probability bits << 32 | ~index) and whose other entries are all zero.  Adding zero changes no
-// running sum, so the eight strided chains of TensorPrimitives.Sum (plus its overlapped tail) and the running sum
-// of the draw are taken over the survivors alone, in index order: a chain's terms are the survivors whose index
-// falls on it, and the tail's indices lie behind every body index, so one order serves all eight chains.
+// Final Normalize (Sampler.cs:91-92, :553-562) and draw (:564-576) of a row whose survivors are listed in index order
+// in sm.sortbuf[0, m) (~index << 32 | probability bits; an entry with probability bits of zero is no survivor) and
+// whose other entries are all zero.  Adding zero changes no running sum, so the eight strided chains of
+// TensorPrimitives.Sum (plus its overlapped tail) and the running sum of the draw are taken over the survivors alone,
+// in index order: a chain's terms are the survivors whose index falls on it, and the tail's indices lie behind every
+// body index, so one order serves all eight chains.  Behind a barrier that follows the last write of the list.
+// A list of more than kSmall entries comes through sm.sortbuf a block of kSmall at a time: fill(first, count), called
+// by all threads between two barriers, puts the entries [first, first + count) at sm.sortbuf[0, count).  A list that is
+// in sm.sortbuf already has m <= kSmall and a fill that does nothing.
+struct NoFill {
+    __device__ __forceinline__ void operator()(int, int) const {}
+};
+template <typename Fill = NoFill>
+__device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, float* p, int n, int m, int row, FullSmem& sm,
+                                                         Fill fill = Fill())
+{
+    constexpr bool kResident = std::is_same<Fill, NoFill>::value;
+    const int nv8 = (n / 8) * 8;
+    const int lane = sr_lane(), wave = sr_wave_id();
+    // One wave per chain: it passes over the whole list in index order, sixteen entries per lane at a time, with the
+    // entries of the other chains as zeros.
+    auto load_terms = [&](int i0, int cnt, int chain, float mul, bool scale, float (&x)[16]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int i = i0 + j;
+            const unsigned long long v = i < cnt ? sm.sortbuf[i] : 0ull;
+            const int e = (int)(0xffffffffu - (uint32_t)(v >> 32));
+            const bool mine = chain < 0 || (e < nv8 ? (e & 7) : e - (n - 8)) == chain;
+            const float t = sr_u2f((uint32_t)v);
+            x[j] = (i < cnt && mine) ? (scale ? __fmul_rn(t, mul) : t) : 0.0f;
+        }
+    };
+    if (kResident && m <= SR_WAVE) {
+        // A short list: one thread per chain adds its members as they come, and one thread draws.
+        const int tid = threadIdx.x;
+        if (tid < SR_SEQ_CHAINS) {
+            float s = 0.0f;
+            for (int i = 0; i < m; i++) {
+                const unsigned long long v = sm.sortbuf[i];
+                const int e = (int)(0xffffffffu - (uint32_t)(v >> 32));
+                const int chain = e < nv8 ? (e & 7) : e - (n - 8);
+                if (chain == tid) s = __fadd_rn(s, sr_u2f((uint32_t)v));
+            }
+            sm.lane_sum[tid] = s;
+        }
+        __syncthreads();
+        const float l0 = sm.lane_sum[0], l1 = sm.lane_sum[1], l2 = sm.lane_sum[2], l3 = sm.lane_sum[3],
+                    l4 = sm.lane_sum[4], l5 = sm.lane_sum[5], l6 = sm.lane_sum[6], l7 = sm.lane_sum[7];
+        const float sum = __fadd_rn(__fadd_rn(__fadd_rn(l0, l1), __fadd_rn(l2, l3)), __fadd_rn(__fadd_rn(l4, l5), __fadd_rn(l6, l7)));
+        const bool scale = sum > 0.0f && sum != 1.0f;
+        const float inv = scale ? __fdiv_rn(1.0f, sum) : 1.0f;
+        if (a.mode != 0 && scale) row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
+        if (a.mode != 1 && tid == 0) {
+            const float r = __double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]);
+            int token = n - 1;
+            if (!(r > 0.0f)) {
+                token = 0;  // the running sum starts at p[0] >= 0: index 0 reaches a target of zero whatever it holds
+            } else {
+                float acc = 0.0f;
+                for (int i = 0; i < m; i++) {
+                    const unsigned long long v = sm.sortbuf[i];
+                    const float x = sr_u2f((uint32_t)v);
+                    acc = __fadd_rn(acc, scale ? __fmul_rn(x, inv) : x);
+                    if (acc >= r) { token = (int)(0xffffffffu - (uint32_t)(v >> 32)); break; }
+                }
+            }
+            if (a.out_tokens) a.out_tokens[row] = token;
+        }
+        return;
+    }
+    float sc = 0.0f;
+    for (int first = 0; first < m; first += kSmall) {
+        const int cnt = min(kSmall, m - first);
+        if (!kResident) {
+            __syncthreads();
+            fill(first, cnt);
+            __syncthreads();
+        }
+        if (wave < SR_SEQ_CHAINS) {
+            for (int b0 = 0; b0 < cnt; b0 += 16 * SR_WAVE) {
+                float x[16];
+                load_terms(b0 + 16 * lane, cnt, wave, 1.0f, false, x);
+                int dummy;
+                sc = sr_seq_wave<16, false>(x, sc, 0.0f, &dummy);
+            }
+        }
+    }
+    if (wave < SR_SEQ_CHAINS && lane == 0) sm.lane_sum[wave] = sc;
+    __syncthreads();
+    const float l0 = sm.lane_sum[0], l1 = sm.lane_sum[1], l2 = sm.lane_sum[2], l3 = sm.lane_sum[3],
+                l4 = sm.lane_sum[4], l5 = sm.lane_sum[5], l6 = sm.lane_sum[6], l7 = sm.lane_sum[7];
+    const float sum = __fadd_rn(__fadd_rn(__fadd_rn(l0, l1), __fadd_rn(l2, l3)), __fadd_rn(__fadd_rn(l4, l5), __fadd_rn(l6, l7)));
+    const bool scale = sum > 0.0f && sum != 1.0f;
+    const float inv = scale ? __fdiv_rn(1.0f, sum) : 1.0f;
+    if (a.mode != 0 && scale) row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
+    if (a.mode == 1) return;
+    const float r = __double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]);
+    int token = n - 1;
+    bool done = false;  // (what wave 0 knows)
+    if (!(r > 0.0f)) {
+        token = 0;  // the running sum starts at p[0] >= 0: index 0 reaches a target of zero whatever it holds
+        done = true;
+    }
+    float acc = 0.0f;
+    for (int first = 0; first < m; first += kSmall) {
+        const int cnt = min(kSmall, m - first);
+        if (!kResident) {
+            if (wave == 0 && lane == 0) sm.bc[10] = done ? 1u : 0u;
+            __syncthreads();
+            if (sm.bc[10] != 0u) break;
+            fill(first, cnt);
+            __syncthreads();
+        }
+        if (wave == 0 && !done) {
+            for (int b0 = 0; b0 < cnt; b0 += 16 * SR_WAVE) {
+                float x[16];
+                load_terms(b0 + 16 * lane, cnt, -1, inv, scale, x);
+                int f;
+                acc = sr_seq_wave<16, true>(x, acc, r, &f);
+                if (f >= 0) {
+                    token = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[b0 + f] >> 32));
+                    done = true;
+                    break;
+                }
+            }
+        }
+    }
+    if (wave == 0 && lane == 0 && a.out_tokens) a.out_tokens[row] = token;
+}
+// ... of a list in any order, its entries as probability bits << 32 | ~index
 __device__ __forceinline__ void finish_from_list(const SrFullArgs& a, float* p, int n, int m, int row, FullSmem& sm)
 {
     const int tid = threadIdx.x;
@@ -745,40 +994,315 @@ __device__ __forceinline__ void finish_from_list(const SrFullArgs& a, float* p, 
     }
     __syncthreads();
     sort_small_desc(sm, P);
-    const int nv8 = (n / 8) * 8;
-    if (tid < SR_SEQ_CHAINS) {
-        float s = 0.0f;
-        for (int i = 0; i < m; i++) {
-            const unsigned long long v = sm.sortbuf[i];
-            const int e = (int)(0xffffffffu - (uint32_t)(v >> 32));
-            const int chain = e < nv8 ? (e & 7) : e - (n - 8);
-            if (chain == tid) s = __fadd_rn(s, sr_u2f((uint32_t)v));
-        }
-        sm.lane_sum[tid] = s;
+    finish_from_ordered_list(a, p, n, m, row, sm);
+}
+
+// Every wave passes over its stretch [w0, w1) of a row (w0 a multiple of 4) and hands the entries for which pred(y, i)
+// holds to a sink, in index order -- y being the entry times inv (the entry itself without do_scale).  Returns the
+// wave's count.  The loads of the next thousand entries are on their way while a thousand are looked at.
+//   sink.reserve(before, count)   room for `count` more finds of this wave, `before` found so far: the first one's place
+//   sink.put(place, rank, y bits, index)   rank = the find's number within the wave
+// The pass is bound by its instructions, not by memory: about 8 us for a row of 151,936 entries with few finds, 30 us
+// when every 256 entries hold some.
+struct StretchToSegment {  // at the stretch's own positions of the row's sort segment
+    uint32_t* gk;
+    int32_t* gi;
+    int w0;
+    __device__ __forceinline__ int reserve(int before, int) const { return w0 + before; }
+    __device__ __forceinline__ void put(int place, int, uint32_t ybits, int i) const { gk[place] = ybits; gi[place] = i; }
+};
+constexpr int kTagIndexBits = 19;  // a find's tag: rank << 19 | index
+struct StretchToPool {  // appended to a pool in LDS that all waves share: values to vals, tags to tags
+    uint32_t* counter;
+    uint32_t* vals;
+    uint32_t* tags;
+    __device__ __forceinline__ int reserve(int, int count) const
+    {
+        int b = 0;
+        if (sr_lane() == 0) b = (int)atomicAdd(counter, (uint32_t)count);
+        return __builtin_amdgcn_readfirstlane(b);
     }
-    __syncthreads();
-    const float l0 = sm.lane_sum[0], l1 = sm.lane_sum[1], l2 = sm.lane_sum[2], l3 = sm.lane_sum[3],
-                l4 = sm.lane_sum[4], l5 = sm.lane_sum[5], l6 = sm.lane_sum[6], l7 = sm.lane_sum[7];
-    const float sum = __fadd_rn(__fadd_rn(__fadd_rn(l0, l1), __fadd_rn(l2, l3)), __fadd_rn(__fadd_rn(l4, l5), __fadd_rn(l6, l7)));
-    const bool scale = sum > 0.0f && sum != 1.0f;
-    const float inv = scale ? __fdiv_rn(1.0f, sum) : 1.0f;
-    if (a.mode != 0 && scale) row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
-    if (a.mode != 1 && tid == 0) {
-        const float r = __double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]);
-        int token = n - 1;
-        if (!(r > 0.0f)) {
-            token = 0;  // the running sum starts at p[0] >= 0: index 0 reaches a target of zero whatever it holds
-        } else {
-            float acc = 0.0f;
-            for (int i = 0; i < m; i++) {
-                const unsigned long long v = sm.sortbuf[i];
-                const float x = sr_u2f((uint32_t)v);
-                acc = __fadd_rn(acc, scale ? __fmul_rn(x, inv) : x);
-                if (acc >= r) { token = (int)(0xffffffffu - (uint32_t)(v >> 32)); break; }
+    __device__ __forceinline__ void put(int place, int rank, uint32_t ybits, int i) const
+    {
+        if (place < kSmall) { vals[place] = ybits; tags[place] = ((uint32_t)rank << kTagIndexBits) | (uint32_t)i; }
+    }
+};
+template <typename Sink, typename Pred>
+__device__ __forceinline__ int list_stretch(const float* p, int w0, int w1, bool do_scale, float inv, Sink sink, Pred pred)
+{
+    const int lane = sr_lane();
+    const bool aligned = ((uintptr_t)p & 15u) == 0u;
+    int cw = 0;
+    auto load = [&](int i0, float (&v)[4][4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = i0 + u * 256 + 4 * lane;
+            if (aligned && i + 4 <= w1) {
+                const float4 t = *(const float4*)(p + i);
+                v[u][0] = t.x; v[u][1] = t.y; v[u][2] = t.z; v[u][3] = t.w;
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; k++) v[u][k] = (i + k < w1) ? p[i + k] : 0.0f;
             }
         }
-        if (a.out_tokens) a.out_tokens[row] = token;
+    };
+    auto look = [&](int i0, const float (&v)[4][4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = i0 + u * 256 + 4 * lane;
+            float y[4];
+            bool pr[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                y[k] = do_scale ? __fmul_rn(v[u][k], inv) : v[u][k];
+                pr[k] = i + k < w1 && pred(y[k], i + k);
+            }
+            if (__ballot(pr[0] || pr[1] || pr[2] || pr[3]) == 0ull) continue;
+            int before = 0, total = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const unsigned long long b = __ballot(pr[k]);
+                before += (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
+                total += __popcll(b);
+            }
+            int place = sink.reserve(cw, total) + before, rank = cw + before;
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                if (pr[k]) { sink.put(place, rank, sr_f2u(y[k]), i + k); place++; rank++; }
+            cw += total;
+        }
+    };
+    if (w0 >= w1) return 0;
+    float va[4][4], vb[4][4];
+    load(w0, va);
+    for (int i0 = w0; i0 < w1; i0 += 2048) {
+        if (i0 + 1024 < w1) load(i0 + 1024, vb);
+        look(i0, va);
+        if (i0 + 1024 >= w1) break;
+        if (i0 + 2048 < w1) load(i0 + 2048, va);
+        look(i0 + 1024, vb);
     }
+    return cw;
+}
+
+// ---- the nucleus of a row that only top-p cuts, without a pass that writes the row ---------------------------------
+// The row holds e = expf(x - max); its probabilities are y = fl(e * inv) (y = e when the sum is 1), which rise with e.
+// While the exact sum passed over the row, the caller counted the e by their upper 16 bits in hcnt (LDS, kHistPos
+// positions: position d holds the keys 0x3f80 - d, position 0 is e = 1, the last position everything below).  From the
+// counts: the longest run of positions from the top that holds at most kSmall entries, shortened to where a lower bound
+// of its probability mass (count x the position's smallest value) passes top_p with a margin.  One read of the row lists
+// the entries above that bound in index order (every wave takes a stretch of the row and writes its finds to the same
+// stretch of the row's sort segment, then the stretches are joined in LDS); their values alone are sorted, the exact
+// running sum finds the cut, and the members -- the values above the cut value and the first few equal to it -- are
+// marked in the index-ordered list, from which the row is finished.  Returns false when the row has to go the general
+// way (nothing is written then but LDS and the row's sort segment).
+constexpr int kHistPos = 8192;
+constexpr uint32_t kHistTopKey = 0x3f80u;
+__device__ __forceinline__ void hist_count(uint32_t* hcnt, uint32_t* bad, float e)
+{
+    if (e > 0.0f) {
+        const uint32_t key = sr_f2u(e) >> 16;
+        if (key <= kHistTopKey) atomicAdd(&hcnt[min(kHistTopKey - key, (uint32_t)(kHistPos - 1))], 1u);
+        else *bad = 1u;  // (no e exceeds 1; if one does, the general way takes the row)
+    }
+}
+enum NucleusWay : int { kNucleusDone = 0, kNucleusGeneral = 1, kNucleusGeneralNoSlabs = 2 };
+constexpr int kNucleusMaxSlabs = 24;
+__device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float top_p, const float* p, int n, int slot,
+                                                      int row, bool do_scale, float inv, FullSmem& sm)
+{
+    constexpr int kPer = kHistPos / kT;
+    static_assert(kHistPos * 4 <= kSmall * 8 && kHistPos % kT == 0, "the histogram fits the sort buffer");
+    const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
+    const uint32_t* hcnt = (const uint32_t*)sm.sortbuf;
+    uint32_t* sval = (uint32_t*)sm.sprob;
+    unsigned long long t_step = 0ull;
+    FPROF_ADD(a, slot, 16, t_step);
+    if (sm.bc[5] != 0u) return kNucleusGeneral;
+    // counts and mass bounds (in units of 2^-28) of this thread's positions
+    uint32_t mine[kPer], mq[kPer];
+    int own = 0;
+    uint32_t ownq = 0u;
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        const int d = tid * kPer + j;
+        mine[j] = hcnt[d];
+        const float e_low = d < kHistPos - 1 ? sr_u2f((kHistTopKey - (uint32_t)d) << 16) : 0.0f;
+        const float y_low = do_scale ? __fmul_rn(e_low, inv) : e_low;
+        mq[j] = (uint32_t)fminf((float)mine[j] * y_low * 268435456.0f, 268435456.0f);
+        own += (int)mine[j];
+        ownq += mq[j];
+    }
+    int tot, totq;
+    const int c0 = blk_excl_scan(own, &tot, sm);
+    const uint32_t q0 = (uint32_t)blk_excl_scan((int)ownq, &totq, sm);
+    if (tid == 0) { sm.bc[7] = (uint32_t)kHistPos; sm.bc[11] = (uint32_t)tot; }
+    __syncthreads();
+    {
+        const uint32_t target_q = (uint32_t)(top_p * 1.001f * 268435456.0f) + 64u;
+        uint32_t q = q0;
+        int c = c0, d_first = kHistPos, c_first = 0;
+#pragma unroll
+        for (int j = 0; j < kPer; j++) {
+            q += mq[j];
+            c += (int)mine[j];
+            if (q >= target_q && d_first == kHistPos) { d_first = tid * kPer + j; c_first = c; }
+        }
+        if (d_first < kHistPos) {
+            atomicMin(&sm.bc[7], (uint32_t)d_first);
+            atomicMin(&sm.bc[11], (uint32_t)c_first);  // (counts rise with the positions: the least belongs to the first)
+        }
+    }
+    const int chunk = ((n + kW * 256 - 1) / (kW * 256)) * 256;
+    const int w0 = min(n, wave * chunk), w1 = min(n, w0 + chunk);
+    uint32_t* gk = a.sort_keys_in + (size_t)slot * a.sort_stride;
+    int32_t* gi = a.sort_vals_in + (size_t)slot * a.sort_stride;
+    FPROF_ADD(a, slot, 11, t_step);
+
+    // The nucleus is walked from the top, a slab of at most kSmall entries at a time: the positions [d_prev, d_end).
+    constexpr int kMaxSlabs = kNucleusMaxSlabs;
+    float run = 0.0f;      // exact running sum behind the slabs before
+    float hi_y = 0.0f;     // what is left has y <= hi_y (from the second slab on)
+    int d_prev = 0;
+    int taken = 0;         // entries that the histogram holds at the positions before d_prev
+    int found = -1, nc = 0, slab = 0;
+    bool all_in = false;
+    for (;; slab++) {
+        if (slab >= kMaxSlabs) return kNucleusGeneralNoSlabs;  // (the general way would walk the same slabs)
+        if (tid == 0) sm.bc[6] = (uint32_t)kHistPos;
+        __syncthreads();
+        {
+            int c = c0, d_first = kHistPos;
+#pragma unroll
+            for (int j = 0; j < kPer; j++) {
+                c += (int)mine[j];
+                if (tid * kPer + j >= d_prev && c - taken > kSmall && d_first == kHistPos) d_first = tid * kPer + j;
+            }
+            if (d_first < kHistPos) atomicMin(&sm.bc[6], (uint32_t)d_first);
+        }
+        __syncthreads();
+        // about how many entries the nucleus holds: a row that would need more slabs than are walked goes the general
+        // way at once (its survivors are sorted device-wide)
+        if (slab == 0 && (int)sm.bc[11] > (kMaxSlabs - 2) * kSmall) return kNucleusGeneralNoSlabs;
+        const int d_cnt = (int)sm.bc[6], d_mass = (int)sm.bc[7];
+        const int d_end = d_mass + 1 > d_prev ? min(d_cnt, d_mass + 1) : d_cnt;
+        if (d_end <= d_prev) return kNucleusGeneralNoSlabs;  // (one position alone holds more than a slab: no walk by slabs passes it)
+        {
+            int c = c0;
+#pragma unroll
+            for (int j = 0; j < kPer; j++) {
+                c += (int)mine[j];
+                if (tid * kPer + j == d_end - 1) sm.bc[8] = (uint32_t)c;
+            }
+        }
+        all_in = d_end >= kHistPos;
+        const float c_e = all_in ? 0.0f : sr_u2f(((kHistTopKey - (uint32_t)d_end) << 16) | 0xffffu);
+        const float c_y = do_scale ? __fmul_rn(c_e, inv) : c_e;  // taken: y > c_y, which e > c_e follows from
+        const bool capped = slab > 0;
+
+        // the slab's entries: every wave lists those of its stretch of the row in a pool in LDS, each with its number
+        // within the wave, from which its place in index order follows once all waves' counts are known
+        if (tid == 0) sm.bc[4] = 0u;
+        __syncthreads();
+        const int cw = list_stretch(p, w0, w1, do_scale, inv, StretchToPool{&sm.bc[4], sval, sm.tags},
+                                    [&](float y, int) -> bool { return y > c_y && !(capped && y > hi_y); });
+        if (lane == 0) sm.redi[wave] = cw;
+        __syncthreads();
+        taken = (int)sm.bc[8];
+        nc = (int)sm.bc[4];
+        if (nc > kSmall) return kNucleusGeneral;
+        FPROF_ADD(a, slot, 12, t_step);
+        if (nc > 0) {
+            int P = 2;
+            while (P < nc) P <<= 1;
+            for (int e = tid; e < P; e += kT) {
+                if (e < nc) {
+                    const uint32_t tag = sm.tags[e];
+                    const int i = (int)(tag & ((1u << kTagIndexBits) - 1u)), w = i / chunk;
+                    int off = (int)(tag >> kTagIndexBits);
+#pragma unroll
+                    for (int k = 0; k < kW - 1; k++) off += k < w ? sm.redi[k] : 0;
+                    sm.sortbuf[off] = ((unsigned long long)(0xffffffffu - (uint32_t)i) << 32) | (unsigned long long)sval[e];
+                } else {
+                    sval[e] = 0u;
+                }
+            }
+            __syncthreads();
+            sort_lds_desc(sval, P);
+            FPROF_ADD(a, slot, 13, t_step);
+            run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, top_p, &found, sm);
+            FPROF_ADD(a, slot, 14, t_step);
+        }
+        if (a.prof && slot == 0 && tid == 0) a.prof[15] += 1ull;
+        if (found >= 0 || all_in) break;
+        hi_y = c_y;
+        d_prev = d_end;
+    }
+
+    // Members: everything above the value at the cut, and of the entries equal to it the first ones by index.
+    uint32_t ycut = 0u;
+    int idx_last = -1;  // the last member among the entries equal to the cut value
+    if (found >= 0) {
+        ycut = sval[found];
+        int gt = 0;
+        for (int e = tid; e < nc; e += kT) gt += sval[e] > ycut ? 1 : 0;
+        const int keep_eq = found + 1 - blk_sum_i(gt, sm);
+        unsigned long long ent[4];
+        int eqc = 0;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int e = 4 * tid + r;
+            ent[r] = e < nc ? sm.sortbuf[e] : 0ull;
+            eqc += (e < nc && (uint32_t)ent[r] == ycut) ? 1 : 0;
+        }
+        int tot_eq;
+        int rank = blk_excl_scan(eqc, &tot_eq, sm);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int e = 4 * tid + r;
+            if (e < nc) {
+                const uint32_t yb = (uint32_t)ent[r];
+                const bool keep = yb > ycut || (yb == ycut && rank < keep_eq);
+                if (yb == ycut && rank == keep_eq - 1) sm.bc[9] = 0xffffffffu - (uint32_t)(ent[r] >> 32);
+                if (yb == ycut) rank++;
+                if (!keep) sm.sortbuf[e] = ent[r] & 0xffffffff00000000ull;
+            }
+        }
+        __syncthreads();
+        idx_last = (int)sm.bc[9];
+    }
+    if (slab == 0) {
+        finish_from_ordered_list(a, const_cast<float*>(p), n, nc, row, sm);
+        return kNucleusDone;
+    }
+    // Several slabs: the members -- known by value and, at the cut value, by index -- are listed by one more read of
+    // the row, again in index order in the waves' stretches of the sort segment, and the final Normalize and the draw
+    // take them from there a block at a time.
+    const float ycut_f = sr_u2f(ycut);
+    const int cm = list_stretch(p, w0, w1, do_scale, inv, StretchToSegment{gk, gi, w0},
+                                [&](float y, int i) -> bool { return y > ycut_f || (y == ycut_f && i <= idx_last); });
+    sr_drain_stores();
+    __syncthreads();  // (the last readers of sm.hist are long past; this one orders the stretches' stores before the fills)
+    if (lane == 0) sm.hist[wave] = (uint32_t)cm;
+    __syncthreads();
+    int members = 0;
+#pragma unroll
+    for (int w = 0; w < kW; w++) members += (int)sm.hist[w];
+    FPROF_ADD(a, slot, 17, t_step);
+    finish_from_ordered_list(a, const_cast<float*>(p), n, members, row, sm, [&](int first, int cnt) {
+        for (int e = tid; e < cnt; e += kT) {
+            const int g = first + e;
+            int w = 0, off = 0;
+#pragma unroll
+            for (int k = 0; k < kW - 1; k++) {
+                const int ck = (int)sm.hist[k];
+                if (w == k && g >= off + ck) { off += ck; w = k + 1; }
+            }
+            const int src = min(n, w * chunk) + (g - off);
+            sm.sortbuf[e] = ((unsigned long long)(0xffffffffu - (uint32_t)gi[src]) << 32) | (unsigned long long)gk[src];
+        }
+    });
+    return kNucleusDone;
 }
 
 // ---- stage 3: softmax, top-k, min-p, top-p on the work row --------------------------------------------
@@ -829,6 +1353,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         int survivors = 0;   // ... this thread's share of the count
         int ns_listed = -1;  // >= 0: the block-wide count, and sm.sortbuf[0, ns_listed) holds the survivors
         bool row_unwritten = false;  // the row still holds expf(x - max): it will be finished from the list
+        bool no_slabs = false;       // the nucleus is known to be too large for the walk by slabs
         if (any_nan || sr_f2u(m) == 0xff800000u) {
             const float uni = n > 0 ? __fdiv_rn(1.0f, (float)n) : 0.0f;
             row_pass<true>(p, n, [&](float, int) -> float { return uni; });
@@ -854,8 +1379,20 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 if (tid == 0) sm.bc[4] = 0u;
                 __syncthreads();
             }
+            // A row that only top-p cuts and that is only sampled from: see nucleus_from_histogram
+            const bool fast_nucleus = use_top_p && !(rd.top_k > 0 && rd.top_k < n) && !(rd.min_p > 0.0f) && a.mode == 0 &&
+                                      n >= 8 && n <= (1 << kTagIndexBits) && a.sort_stride >= n;
+            if (fast_nucleus) {
+                uint32_t* hcnt = (uint32_t*)sm.sortbuf;
+                for (int i = tid; i < kHistPos; i += kT) hcnt[i] = 0u;
+                if (tid == 0) sm.bc[5] = 0u;
+                __syncthreads();
+            }
             float sum;
-            if (watch_min_p) {
+            if (fast_nucleus) {
+                uint32_t* hcnt = (uint32_t*)sm.sortbuf;
+                sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm, 1.0f, 1.0f, [&](float x, int) { hist_count(hcnt, &sm.bc[5], x); });
+            } else if (watch_min_p) {
                 sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm, 1.0f, 1.0f, [&](float x, int i) {
                     if (x >= e_low) {
                         const uint32_t pos = atomicAdd(&sm.bc[4], 1u);
@@ -890,6 +1427,20 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 }
                 return;
             }
+            const int way = fast_nucleus ? nucleus_from_histogram(a, rd.top_p, p, n, slot, row, do_scale, inv, sm) : kNucleusGeneral;
+            no_slabs = way == kNucleusGeneralNoSlabs;
+            if (way == kNucleusDone) {
+                FPROF(a, slot, 9);
+                if (tid == 0) {
+                    st->n_survivors = 0;
+                    st->big = 0;
+                    st->flags = flags;
+                    st->pad = 1;  // finished in this phase
+                    a.seg_begin[slot] = a.seg_end[slot] = (int)((size_t)slot * a.sort_stride);
+                    if (a.out_flags) a.out_flags[row] = flags;
+                }
+                return;
+            }
             if (!(rd.top_k > 0 && rd.top_k < n) && (rd.min_p > 0.0f || use_top_p)) {
                 // No top-k stage in between: the scaling, the min-p cut (Sampler.cs:493-503) and the count of
                 // survivors that top-p starts from share one pass.  The largest probability needs no search: the
@@ -900,7 +1451,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 int c = 0;
                 // A min-p cut leaves few survivors: they are listed while the row is read, which saves the pass that
                 // would collect them; a row that is only sampled from (no distribution out) and ends with at most
-                // 1,024 survivors is finished from that list and need not be written at all.
+                // 4,096 survivors is finished from that list and need not be written at all.
                 const bool list_now = use_min_p;
                 if (list_now) {
                     if (tid == 0) sm.bc[4] = 0u;
@@ -943,7 +1494,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 if (list_now) {
                     const int ns_now = blk_sum_i(c, sm);
                     if (ns_now <= kSmall) ns_listed = ns_now;
-                    row_unwritten = read_only && ns_now > 0 && ns_now <= 1024;
+                    row_unwritten = read_only && ns_now > 0 && ns_now <= kSmall;
                     if (read_only && !row_unwritten) {
                         // too many survivors to finish from the list: the scaled row is needed after all
                         row_pass<true>(p, n, [&](float x, int) -> float {
@@ -1006,7 +1557,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             static_assert(kPos * 4 <= kSmall * 8 && kPos % kT == 0, "the histogram fits the sort buffer");
             constexpr int kPer = kPos / kT;
             uint32_t* sums = a.sort_keys_in + (size_t)slot * a.sort_stride;
-            bool use_hist = !have_list && ns > kSmall && a.sort_stride >= kPos;
+            bool use_hist = !have_list && ns > kSmall && a.sort_stride >= kPos && !no_slabs;
             if (use_hist) {
                 uint32_t* cnt = (uint32_t*)sm.sortbuf;
                 for (int i = tid; i < kPos; i += kT) cnt[i] = 0u;
@@ -1033,12 +1584,15 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 sr_drain_stores();
                 __syncthreads();
             }
+            FPROF(a, slot, 10);
+            unsigned long long t_step = 0ull;
+            FPROF_ADD(a, slot, 16, t_step);
             bool closed = false;
             float run = 0.0f;                  // exact running sum behind the slabs taken so far
             int taken = 0;                     // survivors in those slabs
             uint32_t hi_key = 0xffffffffu;     // what is left are the probabilities with keys <= hi_key
             float c_above = -1.0f;             // the current slab: probabilities strictly above this value ...
-            for (int slab = 0; slab < kMaxSlabs && ns > 0 && !closed; slab++) {
+            for (int slab = 0; slab < kMaxSlabs && ns > 0 && !closed && !no_slabs; slab++) {
                 const bool last_slab = ns - taken <= kSmall;  // everything that is left fits
                 if (last_slab) {
                     c_above = 0.0f;
@@ -1065,6 +1619,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 } else {
                     c_above = sr_u2f(sr_f2u(kth_largest(p, n, kSmall, sm, 16, hi_key)) | 0xffffu);
                 }
+                FPROF_ADD(a, slot, 11, t_step);
                 int nc;
                 if (have_list) {
                     nc = ns;  // (ns <= kSmall: the survivors were listed while the row was scaled)
@@ -1083,16 +1638,20 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                     nc = (int)sm.bc[4];
                     __syncthreads();
                 }
+                FPROF_ADD(a, slot, 12, t_step);
                 if (nc <= 0 || nc > kSmall) break;  // no progress: the device-wide sort takes the row
                 int P = 2;
                 while (P < nc) P <<= 1;
                 for (int i = nc + tid; i < P; i += kT) sm.sortbuf[i] = 0ull;
                 __syncthreads();
                 sort_small_desc(sm, P);
+                FPROF_ADD(a, slot, 13, t_step);
                 for (int i = tid; i < nc; i += kT) sm.sprob[i] = sr_u2f((uint32_t)(sm.sortbuf[i] >> 32));
                 __syncthreads();
                 int found;
                 run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, rd.top_p, &found, sm);
+                FPROF_ADD(a, slot, 14, t_step);
+                if (a.prof && slot == 0 && tid == 0) a.prof[15] += 1ull;
                 taken += nc;
                 closed = found >= 0 || taken == ns;
                 if (closed) {
@@ -1139,12 +1698,11 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 }
             }
             if (tid == 0) st->n_survivors = ns;
-        } else if (ns_listed > 0 && ns_listed <= 1024 && n >= 8) {
+        } else if (ns_listed > 0 && ns_listed <= kSmall && n >= 8) {
             listed = ns_listed;  // min-p alone: its survivors are the members
         }
         FPROF(a, slot, 6);
-        // (up to a thousand members: beyond that the passes over the row are the faster way)
-        const bool finish_here = listed > 0 && listed <= 1024 && n >= 8;
+        const bool finish_here = listed > 0 && listed <= kSmall && n >= 8;
         if (tid == 0) {
             st->big = big;
             st->flags = flags;
@@ -1155,6 +1713,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         if (finish_here) {
             // the nucleus closed inside the kernel and its members are at hand: no pass over the row is needed
             finish_from_list(a, p, n, listed, row, sm);
+            FPROF(a, slot, 9);
             if (tid == 0 && a.out_flags) a.out_flags[row] = flags;
             return;
         }

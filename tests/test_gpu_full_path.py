@@ -366,6 +366,40 @@ def test_nuclei_of_tens_of_thousands_of_members_take_the_device_wide_sort(ctx):
     _check_rows(ctx, logits, params, rng.random(4), mask, active)
 
 
+def test_rows_that_only_top_p_cuts_at_every_size_of_nucleus(ctx):
+    # A sampled row with top-p alone is cut without being rewritten: a histogram of its exponentials bounds the slabs
+    # that are sorted, the members come from reads of the row in index order.  Nuclei that close in the first slab,
+    # that take several slabs (their members then pass through the kernel a block at a time), that are larger than the
+    # walk goes (device-wide sort), equal probabilities at the cut (the first ones by index stay), under allow-masks,
+    # with uniforms at both ends of the range (a draw near 1 lands among the last members).
+    rng = np.random.default_rng(4242)
+    V = synthetic.QWEN_VOCAB
+    logits = np.stack([
+        rng.normal(0, 3.0, V),                               # sharp: a few hundred members
+        rng.normal(0, 1.6, V),                               # some thousands
+        rng.normal(0, 1.2, V),                               # several slabs
+        np.round(rng.normal(0, 1.2, V) * 4) / 4,             # ... with hundreds of equal probabilities at the cut
+        np.round(rng.normal(0, 2.5, V) * 2) / 2,             # equal probabilities at a cut inside the first slab
+        rng.normal(0, 0.4, V),                               # most of the vocabulary: beyond the walk
+    ]).astype(np.float32)
+    params = [SamplingParams(Temperature=1.0, TopP=0.95), SamplingParams(Temperature=1.0, TopP=0.9),
+              SamplingParams(Temperature=1.0, TopP=0.9), SamplingParams(Temperature=0.9, TopP=0.8),
+              SamplingParams(Temperature=1.1, TopP=0.7), SamplingParams(Temperature=1.0, TopP=0.95)]
+    rows = len(params)
+    for u in ([0.99999994] * rows, [0.0] * rows, [0.9995] * rows, rng.random(rows).tolist(), rng.random(rows).tolist()):
+        _check_rows(ctx, logits, params, u)
+    allowed = rng.random((rows, V)) < np.array([0.5, 0.3, 0.9, 0.7, 0.2, 0.8])[:, None]
+    mask = pack_allow_mask(allowed)
+    active = np.ones(rows, dtype=np.uint8)
+    for u in ([0.99999994] * rows, rng.random(rows).tolist()):
+        _check_rows(ctx, logits, params, u, mask, active)
+    # shorter rows, lengths off the multiples of 4 and 8
+    for n in (4097, 20_001, 65_539):
+        sub = np.ascontiguousarray(logits[:, :n])
+        for u in ([0.99999994] * rows, rng.random(rows).tolist()):
+            _check_rows(ctx, sub, params, u)
+
+
 def _strided(a, pad, dtype=None):
     """The rows of `a` inside a wider device tensor: row stride = a.shape[1] + pad elements."""
     import torch
