@@ -873,11 +873,24 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
     const int lane = sr_lane(), wave = sr_wave_id();
     // One wave per chain: it passes over the whole list in index order, sixteen entries per lane at a time, with the
     // entries of the other chains as zeros.
+    // A lane's sixteen consecutive entries would all lie in the same LDS banks as every other lane's: inside each
+    // thousand entries the list is laid out anew, entry 16 l + j at place 64 j + l.
+    auto place_of = [](int i) -> int { return (i & ~1023) | ((i & 15) << 6) | ((i >> 4) & 63); };
+    auto lay_out = [&]() __attribute__((always_inline)) {
+        static_assert(kSmall == 4 * kT, "four entries per thread");
+        unsigned long long t[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) t[r] = sm.sortbuf[4 * (int)threadIdx.x + r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 4; r++) sm.sortbuf[place_of(4 * (int)threadIdx.x + r)] = t[r];
+        __syncthreads();
+    };
     auto load_terms = [&](int i0, int cnt, int chain, float mul, bool scale, float (&x)[16]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             const int i = i0 + j;
-            const unsigned long long v = i < cnt ? sm.sortbuf[i] : 0ull;
+            const unsigned long long v = i < cnt ? sm.sortbuf[place_of(i)] : 0ull;
             const int e = (int)(0xffffffffu - (uint32_t)(v >> 32));
             const bool mine = chain < 0 || (e < nv8 ? (e & 7) : e - (n - 8)) == chain;
             const float t = sr_u2f((uint32_t)v);
@@ -923,12 +936,14 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
         return;
     }
     float sc = 0.0f;
+    if (kResident) lay_out();
     for (int first = 0; first < m; first += kSmall) {
         const int cnt = min(kSmall, m - first);
         if (!kResident) {
             __syncthreads();
             fill(first, cnt);
             __syncthreads();
+            lay_out();
         }
         if (wave < SR_SEQ_CHAINS) {
             for (int b0 = 0; b0 < cnt; b0 += 16 * SR_WAVE) {
@@ -941,6 +956,7 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
     }
     if (wave < SR_SEQ_CHAINS && lane == 0) sm.lane_sum[wave] = sc;
     __syncthreads();
+    FPROF(a, blockIdx.x, 18);
     const float l0 = sm.lane_sum[0], l1 = sm.lane_sum[1], l2 = sm.lane_sum[2], l3 = sm.lane_sum[3],
                 l4 = sm.lane_sum[4], l5 = sm.lane_sum[5], l6 = sm.lane_sum[6], l7 = sm.lane_sum[7];
     const float sum = __fadd_rn(__fadd_rn(__fadd_rn(l0, l1), __fadd_rn(l2, l3)), __fadd_rn(__fadd_rn(l4, l5), __fadd_rn(l6, l7)));
@@ -964,6 +980,7 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
             if (sm.bc[10] != 0u) break;
             fill(first, cnt);
             __syncthreads();
+            lay_out();
         }
         if (wave == 0 && !done) {
             for (int b0 = 0; b0 < cnt; b0 += 16 * SR_WAVE) {
@@ -972,7 +989,7 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
                 int f;
                 acc = sr_seq_wave<16, true>(x, acc, r, &f);
                 if (f >= 0) {
-                    token = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[b0 + f] >> 32));
+                    token = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[place_of(b0 + f)] >> 32));
                     done = true;
                     break;
                 }
@@ -1290,17 +1307,26 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     for (int w = 0; w < kW; w++) members += (int)sm.hist[w];
     FPROF_ADD(a, slot, 17, t_step);
     finish_from_ordered_list(a, const_cast<float*>(p), n, members, row, sm, [&](int first, int cnt) {
-        for (int e = tid; e < cnt; e += kT) {
-            const int g = first + e;
+        // (all of a thread's loads are on their way before the first of them is waited for)
+        int src[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int g = first + min(r * kT + tid, cnt - 1);
             int w = 0, off = 0;
 #pragma unroll
             for (int k = 0; k < kW - 1; k++) {
                 const int ck = (int)sm.hist[k];
                 if (w == k && g >= off + ck) { off += ck; w = k + 1; }
             }
-            const int src = min(n, w * chunk) + (g - off);
-            sm.sortbuf[e] = ((unsigned long long)(0xffffffffu - (uint32_t)gi[src]) << 32) | (unsigned long long)gk[src];
+            src[r] = min(n, w * chunk) + (g - off);
         }
+        uint32_t yb[4];
+        int32_t ix[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) { yb[r] = gk[src[r]]; ix[r] = gi[src[r]]; }
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            if (r * kT + tid < cnt) sm.sortbuf[r * kT + tid] = ((unsigned long long)(0xffffffffu - (uint32_t)ix[r]) << 32) | (unsigned long long)yb[r];
     });
     return kNucleusDone;
 }
