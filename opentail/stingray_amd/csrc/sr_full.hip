@@ -1093,10 +1093,14 @@ __device__ __forceinline__ int list_stretch(const float* p, int w0, int w1, bool
     float va[4][4], vb[4][4];
     load(w0, va);
     for (int i0 = w0; i0 < w1; i0 += 2048) {
+        // (the scheduling barriers keep the loads where they are written: left alone, the compiler moves them down
+        // to where their values are used, and every thousand entries wait for memory once more)
         if (i0 + 1024 < w1) load(i0 + 1024, vb);
+        __builtin_amdgcn_sched_barrier(0);
         look(i0, va);
         if (i0 + 1024 >= w1) break;
         if (i0 + 2048 < w1) load(i0 + 2048, va);
+        __builtin_amdgcn_sched_barrier(0);
         look(i0 + 1024, vb);
     }
     return cw;
@@ -1184,6 +1188,9 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     int taken = 0;         // entries that the histogram holds at the positions before d_prev
     int found = -1, nc = 0, slab = 0;
     bool all_in = false;
+    uint32_t pv[4] = {0u, 0u, 0u, 0u};  // the last slab's entries that this thread read from the pool: values,
+    int pi[4] = {0, 0, 0, 0};            // indices
+    int lpos[4] = {0, 0, 0, 0};          // and places in index order
     for (;; slab++) {
         if (slab >= kMaxSlabs) return kNucleusGeneralNoSlabs;  // (the general way would walk the same slabs)
         if (tid == 0) sm.bc[6] = (uint32_t)kHistPos;
@@ -1230,22 +1237,87 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         if (nc > kSmall) return kNucleusGeneral;
         FPROF_ADD(a, slot, 12, t_step);
         if (nc > 0) {
-            int P = 2;
-            while (P < nc) P <<= 1;
-            for (int e = tid; e < P; e += kT) {
-                if (e < nc) {
-                    const uint32_t tag = sm.tags[e];
-                    const int i = (int)(tag & ((1u << kTagIndexBits) - 1u)), w = i / chunk;
-                    int off = (int)(tag >> kTagIndexBits);
+            // this thread's four entries of the pool, and their places in index order
 #pragma unroll
-                    for (int k = 0; k < kW - 1; k++) off += k < w ? sm.redi[k] : 0;
-                    sm.sortbuf[off] = ((unsigned long long)(0xffffffffu - (uint32_t)i) << 32) | (unsigned long long)sval[e];
-                } else {
-                    sval[e] = 0u;
+            for (int r = 0; r < 4; r++) {
+                const int e = r * kT + tid;
+                pv[r] = e < nc ? sval[e] : 0u;
+                const uint32_t tag = e < nc ? sm.tags[e] : 0u;
+                const int i = (int)(tag & ((1u << kTagIndexBits) - 1u)), w = i / chunk;
+                int off = (int)(tag >> kTagIndexBits);
+#pragma unroll
+                for (int k = 0; k < kW - 1; k++) off += k < w ? sm.redi[k] : 0;
+                pi[r] = i;
+                lpos[r] = off;
+            }
+            // The values are sorted.  A long list is first cut into 4,096 groups of equal width in the values' bit
+            // patterns between the slab's bounds -- counted, the counts summed, the values put group by group -- and
+            // then every value finds its rank among the values of its group (equal values are interchangeable in the
+            // sum that follows): far fewer steps than the sorting network, unless a group holds more than a few dozen.
+            const uint32_t bhi = sr_f2u(capped ? hi_y : (do_scale ? __fmul_rn(1.0f, inv) : 1.0f)), blo = sr_f2u(c_y);
+            const uint32_t span = bhi >= blo ? bhi - blo : 0xffffffffu;
+            const int gshift = span < (uint32_t)kSmall ? 0 : 20 - __clz((int)span);  // (span >> gshift) < kSmall
+            auto group_of = [&](uint32_t v) -> uint32_t { return min((bhi - v) >> gshift, (uint32_t)(kSmall - 1)); };
+            bool counted = false;
+            if (nc > 1024 && bhi >= blo) {
+                uint32_t* cur = (uint32_t*)sm.sortbuf;
+                uint32_t* grp = cur + kSmall;
+                __syncthreads();  // (sval and the tags have been read)
+#pragma unroll
+                for (int r = 0; r < 4; r++) cur[r * kT + tid] = 0u;
+                if (tid == 0) sm.bc[12] = 0u;
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (r * kT + tid < nc) atomicAdd(&cur[group_of(pv[r])], 1u);
+                __syncthreads();
+                uint32_t c4[4];
+                int own = 0;
+                uint32_t big = 0u;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    c4[r] = cur[4 * tid + r];
+                    own += (int)c4[r];
+                    big = max(big, c4[r]);
+                }
+                if (big > 128u) sm.bc[12] = 1u;
+                int tot_c;
+                int at = blk_excl_scan(own, &tot_c, sm);
+                counted = sm.bc[12] == 0u;  // (the scan's barriers lie between the store and this load)
+                if (counted) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) { cur[4 * tid + r] = (uint32_t)at; at += (int)c4[r]; }
+                    __syncthreads();
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (r * kT + tid < nc) grp[atomicAdd(&cur[group_of(pv[r])], 1u)] = pv[r];
+                    __syncthreads();  // cur[g] is now where group g ends
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int i = r * kT + tid;
+                        if (i < nc) {
+                            const uint32_t v = grp[i];
+                            const uint32_t g = group_of(v);
+                            const int from = g > 0u ? (int)cur[g - 1u] : 0, to = (int)cur[g];
+                            int rank = from;
+                            for (int j = from; j < to; j++) {
+                                const uint32_t o = grp[j];
+                                rank += (o > v || (o == v && j < i)) ? 1 : 0;
+                            }
+                            sval[rank] = v;
+                        }
+                    }
+                    __syncthreads();
                 }
             }
-            __syncthreads();
-            sort_lds_desc(sval, P);
+            if (!counted) {
+                int P = 2;
+                while (P < nc) P <<= 1;
+                __syncthreads();
+                for (int e = nc + tid; e < P; e += kT) sval[e] = 0u;
+                __syncthreads();
+                sort_lds_desc(sval, P);
+            }
             FPROF_ADD(a, slot, 13, t_step);
             run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, top_p, &found, sm);
             FPROF_ADD(a, slot, 14, t_step);
@@ -1256,6 +1328,12 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         d_prev = d_end;
     }
 
+    // the last slab's entries in index order (the sort's scratch memory is free again)
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+        if (r * kT + tid < nc) sm.sortbuf[lpos[r]] = ((unsigned long long)(0xffffffffu - (uint32_t)pi[r]) << 32) | (unsigned long long)pv[r];
+    __syncthreads();
     // Members: everything above the value at the cut, and of the entries equal to it the first ones by index.
     uint32_t ycut = 0u;
     int idx_last = -1;  // the last member among the entries equal to the cut value
