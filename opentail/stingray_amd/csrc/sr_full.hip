@@ -363,10 +363,105 @@ __device__ __forceinline__ float tp_sum(Term term, int n, FullSmem& sm)
     return __fadd_rn(__fadd_rn(lane_sum[0], lane_sum[1]), __fadd_rn(lane_sum[2], lane_sum[3]));
 }
 
+// The same sum over a long row in memory (times mul when do_mul), one wave per lane accumulator.  The row comes in
+// through LDS 8,192 entries at a time -- every thread brings two 16-byte pieces, two rounds ahead of the round that is
+// added --, laid out chain by chain, and the wave of a chain adds its 1,024 terms of the round with the wave's own
+// exact scan (sr_seq_wave): no block-wide step but one barrier per round, so a round costs what its 32 KB take to
+// arrive.  The place of term v = 16 l + j of chain g is g * 1024 + 64 j + (l + 2 j) mod 64: the 64 lanes of a wave
+// read a term from 64 consecutive places, and the stores of a piece's four entries fall two to a bank.
+__device__ __forceinline__ float tp_sum_row(const float* p, int n, float mul, bool do_mul, FullSmem& sm)
+{
+    constexpr int kRound = 8192;
+    static_assert(offsetof(FullSmem, sprob) == offsetof(FullSmem, sortbuf) + sizeof(FullSmem::sortbuf) &&
+                  offsetof(FullSmem, tags) == offsetof(FullSmem, sprob) + sizeof(FullSmem::sprob) &&
+                  sizeof(FullSmem::sortbuf) + sizeof(FullSmem::sprob) + sizeof(FullSmem::tags) >= 2 * kRound * sizeof(float),
+                  "two rounds fit the three arrays, which lie one behind the other");
+    static_assert(kRound == 8 * kT, "two 16-byte pieces per thread and round");
+    if (n < 2 * kRound || ((uintptr_t)p & 15u) != 0u) {
+        if (do_mul) return tp_sum([&](int i) -> float { return __fmul_rn(p[i], mul); }, n, sm);
+        return tp_sum([&](int i) -> float { return p[i]; }, n, sm);
+    }
+    float* buf = (float*)sm.sortbuf;
+    const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
+    const int nv = n / 8, rem = n - nv * 8, body = nv * 8;
+    const int rounds = (body + kRound - 1) / kRound;
+    auto fetch = [&](int r, float4 (&v)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int x0 = r * kRound + 4 * (tid + h * kT);
+            if (x0 + 4 <= body) {
+                v[h] = *(const float4*)(p + x0);
+            } else {
+                v[h].x = x0 < body ? p[x0] : 0.0f;
+                v[h].y = x0 + 1 < body ? p[x0 + 1] : 0.0f;
+                v[h].z = x0 + 2 < body ? p[x0 + 2] : 0.0f;
+                v[h].w = 0.0f;  // (x0 + 3 < body would have taken the other way)
+            }
+        }
+    };
+    auto stash = [&](int r, const float4 (&v)[2]) __attribute__((always_inline)) {
+        float* b = buf + (r & 1) * kRound;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int t2 = tid + h * kT;  // the piece's number within the round
+            const int vec = t2 >> 1, j = vec & 15, l = vec >> 4;
+            float* at = b + (4 * (t2 & 1)) * 1024 + 64 * j + ((l + 2 * j) & 63);
+            at[0] = do_mul ? __fmul_rn(v[h].x, mul) : v[h].x;
+            at[1024] = do_mul ? __fmul_rn(v[h].y, mul) : v[h].y;
+            at[2048] = do_mul ? __fmul_rn(v[h].z, mul) : v[h].z;
+            at[3072] = do_mul ? __fmul_rn(v[h].w, mul) : v[h].w;
+        }
+    };
+    float sc = 0.0f;
+    auto add_round = [&](int r) __attribute__((always_inline)) {
+        if (wave < SR_SEQ_CHAINS) {
+            const float* b = buf + (r & 1) * kRound + wave * 1024;
+            float x[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) x[j] = b[64 * j + ((lane + 2 * j) & 63)];
+            int dummy;
+            sc = sr_seq_wave<16, false>(x, sc, 0.0f, &dummy);
+        }
+    };
+    // (behind the last round the loop fetches that round again, to no effect: the compiler can wait for "all but the
+    // newest loads" only where it can count them)
+    float4 va[2], vb[2];
+    __syncthreads();  // (whoever used the arrays before is done)
+    fetch(0, va);
+    fetch(min(1, rounds - 1), vb);
+    stash(0, va);
+    for (int r = 0; r < rounds; r += 2) {
+        fetch(min(r + 2, rounds - 1), va);
+        __syncthreads();
+        add_round(r);
+        if (r + 1 >= rounds) break;
+        stash(r + 1, vb);
+        fetch(min(r + 3, rounds - 1), vb);
+        __syncthreads();
+        add_round(r + 1);
+        if (r + 2 < rounds) stash(r + 2, va);
+    }
+    if (wave < SR_SEQ_CHAINS) {
+        if (rem > 0 && wave >= 8 - rem) {  // the overlapped last vector's entry of this chain
+            float x[1];
+            const float t = p[n - 8 + wave];
+            x[0] = lane == 0 ? (do_mul ? __fmul_rn(t, mul) : t) : 0.0f;
+            int dummy;
+            sc = sr_seq_wave<1, false>(x, sc, 0.0f, &dummy);
+        }
+        if (lane == 0) sm.lane_sum[wave] = sc;
+    }
+    __syncthreads();
+    const float l0 = sm.lane_sum[0], l1 = sm.lane_sum[1], l2 = sm.lane_sum[2], l3 = sm.lane_sum[3],
+                l4 = sm.lane_sum[4], l5 = sm.lane_sum[5], l6 = sm.lane_sum[6], l7 = sm.lane_sum[7];
+    __syncthreads();
+    return __fadd_rn(__fadd_rn(__fadd_rn(l0, l1), __fadd_rn(l2, l3)), __fadd_rn(__fadd_rn(l4, l5), __fadd_rn(l6, l7)));
+}
+
 // Normalize (Sampler.cs:553-562)
 __device__ __forceinline__ void normalize_row(float* p, int n, FullSmem& sm)
 {
-    const float sum = tp_sum([&](int i) -> float { return p[i]; }, n, sm);
+    const float sum = tp_sum_row(p, n, 1.0f, false, sm);
     if (sum > 0.0f && sum != 1.0f) {
         const float inv = __fdiv_rn(1.0f, sum);
         row_pass<true>(p, n, [&](float x, int) -> float { return __fmul_rn(x, inv); });
@@ -1517,7 +1612,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 // No filter touches the row: its final entries are fmul(fmul(e, inv), inv2) with inv2 from the final
                 // Normalize (Sampler.cs:91-92) over the scaled values.  The reader applies the two factors; the row
                 // keeps e and is not written again.
-                const float sum2 = tp_sum([&](int i) -> float { return __fmul_rn(p[i], inv); }, n, sm);
+                const float sum2 = tp_sum_row(p, n, inv, true, sm);
                 const float inv2 = (sum2 > 0.0f && sum2 != 1.0f) ? __fdiv_rn(1.0f, sum2) : 1.0f;
                 if (tid == 0) {
                     st->mul1 = inv;
