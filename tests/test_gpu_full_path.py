@@ -400,6 +400,20 @@ def test_rows_that_only_top_p_cuts_at_every_size_of_nucleus(ctx):
             _check_rows(ctx, sub, params, u)
 
 
+def test_final_normalize_of_long_rows_at_ragged_lengths(ctx):
+    # The eight-lane sum of a long row is taken by one wave per lane over blocks of 8,192 entries; lengths that leave
+    # one to seven entries for the overlapped last vector, a last block that is nearly empty or nearly full, rows
+    # that top-k cuts to a few entries and rows that keep half of theirs.  The distributions must agree bit for bit.
+    rng = np.random.default_rng(909)
+    for n in (16_384, 16_385, 16_391, 24_575, 24_577, 65_539, 151_937):
+        logits = rng.normal(0, 2.0, (4, n)).astype(np.float32)
+        params = [SamplingParams(Temperature=1.0, TopK=40), SamplingParams(Temperature=0.8, TopK=3000),
+                  SamplingParams(Temperature=1.2, TopK=5000, TopP=0.99),
+                  SamplingParams(Temperature=1.0, TopK=n // 2 if n < 30_000 else 1000, MinP=1e-6)]
+        _check_distribution(ctx, logits, params)
+        _check_rows(ctx, logits, params, rng.random(4))
+
+
 def _strided(a, pad, dtype=None):
     """The rows of `a` inside a wider device tensor: row stride = a.shape[1] + pad elements."""
     import torch
