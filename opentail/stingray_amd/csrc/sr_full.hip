@@ -2149,6 +2149,107 @@ __global__ __launch_bounds__(kT) void k_residual_rows(const float* p, int64_t ps
     if (threadIdx.x == 0) out_tokens[row] = t;
 }
 
+// ... from the residual row itself (res[i] = max(0, fl(fl(p[i] m1) m2) - q[i]), written by k_spec_residual): the same
+// terms in the same order, read from one row instead of computed from two
+__device__ __forceinline__ int resample_residual_stored(const float* res, const float* p, int n, double u, FullSmem& sm,
+                                                        float m1, float m2)
+{
+    int dummy;
+    const float sum = seq_sum_row<false>(res, n, 0.0f, 0.0f, &dummy, sm);
+    if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm, m1, m2);  // sum <= 0 or NaN
+    const float target = __fmul_rn(__double2float_rn(u), sum);
+    auto edge = [&](bool first_one) -> int {  // the first / the last index with a positive residual
+        int at = first_one ? 0x7fffffff : -1;
+        for (int i = threadIdx.x; i < n; i += kT)
+            if (res[i] > 0.0f) {
+                at = i;
+                if (first_one) break;
+            }
+        at = first_one ? sr_wave_min_i32(at) : -sr_wave_min_i32(-at);
+        __syncthreads();
+        if (sr_lane() == 0) sm.redi[sr_wave_id()] = at;
+        __syncthreads();
+        int f = first_one ? 0x7fffffff : -1;
+        for (int w = 0; w < kW; w++) f = first_one ? min(f, sm.redi[w]) : max(f, sm.redi[w]);
+        __syncthreads();
+        return f;
+    };
+    if (target <= 0.0f) return edge(true);  // a zero target must not stop on a zero term
+    int found;
+    seq_sum_row<true>(res, n, 0.0f, target, &found, sm);
+    return found >= 0 ? found : edge(false);  // (rounding: the sum of the search fell short of the target)
+}
+
+// The accept loop of a row under the ratio test needs one element of p and of q per position, no pass over a row:
+// one wave walks it ahead of everything else and names the first rejected position, so that the residual row of
+// that position -- which the row's workgroup would otherwise compute twice, from two rows, at the rate of one compute
+// unit -- can be written by the whole device (k_spec_residual) before k_spec_verify reads it.
+__global__ __launch_bounds__(SR_WAVE) void k_spec_walk(SrSpecArgs a)
+{
+    const int row = blockIdx.x, lane = sr_lane();
+    const SrRow rd = a.rows[row];
+    const int n = a.vocab, L = a.n_draft;
+    const bool true_spec = !(rd.p_min > 0.0f && rd.p_min < 1.0f) && (rd.flags & SR_ROWBIT_DRAFT_FROM_LOOKUP) == 0u;
+    int reject = -1;
+    if (true_spec) {
+        const float* pr = a.p_all + (size_t)row * (L + 1) * n;
+        const double* u = a.uniforms + (size_t)row * a.uniforms_per_row;
+        for (int i0 = 0; i0 < L; i0 += SR_WAVE) {
+            const int i = i0 + lane;
+            bool stop = false, bad = false;
+            if (i < L) {
+                const int tok = a.draft_tokens[(size_t)row * L + i];
+                bad = (uint32_t)tok >= (uint32_t)n;
+                if (!bad) {
+                    const SrFullState* sl = a.state + (size_t)row * (L + 1) + i;
+                    const float px = __fmul_rn(__fmul_rn(pr[(size_t)i * n + tok], sl->mul1), sl->mul2);
+                    const float qx = a.draft_probs[((size_t)row * L + i) * n + tok];
+                    const float acc = qx > 0.0f ? fminf(1.0f, __fdiv_rn(px, qx)) : (px > 0.0f ? 1.0f : 0.0f);
+                    stop = !(u[i] < (double)acc);  // (every position before it was accepted and drew one uniform)
+                }
+            }
+            const unsigned long long ends = __ballot(stop || bad);
+            if (ends != 0ull) {
+                const int l = (int)__ffsll((long long)ends) - 1;
+                const bool is_bad = ((__ballot(bad) >> l) & 1ull) != 0ull;
+                reject = is_bad ? -1 : i0 + l;  // (an id outside the vocabulary ends the row without a correction)
+                break;
+            }
+        }
+    }
+    if (lane == 0) a.reject[row] = reject;
+}
+
+__global__ __launch_bounds__(256) void k_spec_residual(SrSpecArgs a)
+{
+    const int row = blockIdx.y;
+    const int i = a.reject[row];
+    if (i < 0) return;
+    const int n = a.vocab, L = a.n_draft;
+    const float* pd = a.p_all + ((size_t)row * (L + 1) + i) * n;
+    const float* qd = a.draft_probs + ((size_t)row * L + i) * n;
+    const SrFullState* sl = a.state + (size_t)row * (L + 1) + i;
+    const float m1 = sl->mul1, m2 = sl->mul2;
+    float* out = a.resid + (size_t)row * (size_t)a.resid_stride;
+    auto res = [&](float pv, float qv) -> float {
+        const float r = __fsub_rn(__fmul_rn(__fmul_rn(pv, m1), m2), qv);
+        return r > 0.0f ? r : 0.0f;
+    };
+    const int t = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
+    if (((((uintptr_t)pd) | ((uintptr_t)qd)) & 15u) == 0u) {
+        const int nv = n / 4;
+        for (int v = t; v < nv; v += nt) {
+            const float4 pv = ((const float4*)pd)[v], qv = ((const float4*)qd)[v];
+            float4 o;
+            o.x = res(pv.x, qv.x); o.y = res(pv.y, qv.y); o.z = res(pv.z, qv.z); o.w = res(pv.w, qv.w);
+            ((float4*)out)[v] = o;
+        }
+        for (int x = nv * 4 + t; x < n; x += nt) out[x] = res(pd[x], qd[x]);
+    } else {
+        for (int x = t; x < n; x += nt) out[x] = res(pd[x], qd[x]);
+    }
+}
+
 // ---- speculative verification: the accept loop of StepSampled (SpeculativeDecoder.cs:530-559) ---------
 // p_all holds the filtered target distributions of every position, [rows][n_draft + 1][n].
 __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
@@ -2211,8 +2312,11 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
             continue;
         }
         const float m1 = sl->mul1, m2 = sl->mul2;
-        correction = true_spec ? resample_residual_row(pd, qd, n, u[udraws++], sm, m1, m2)
-                               : draw_from_row(pd, n, u[udraws++], sm, m1, m2);
+        const double uc = u[udraws++];
+        if (true_spec && a.reject && a.reject[row] == i)  // the residual row is there already
+            correction = resample_residual_stored(a.resid + (size_t)row * (size_t)a.resid_stride, pd, n, uc, sm, m1, m2);
+        else
+            correction = true_spec ? resample_residual_row(pd, qd, n, uc, sm, m1, m2) : draw_from_row(pd, n, uc, sm, m1, m2);
         break;
     }
     if (correction < 0 && !bad_id) {
@@ -2346,7 +2450,15 @@ hipError_t sr_launch_residual_rows(const float* p, int64_t ps, const float* q, i
 hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st)
 {
     if (rows <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_spec_verify, dim3(rows), dim3(kT), 0, st, a);
+    SrSpecArgs b = a;
+    if (!(b.resid && b.reject && b.n_draft > 0 && b.draft_probs)) {
+        b.resid = nullptr;
+        b.reject = nullptr;
+    } else {
+        hipLaunchKernelGGL(k_spec_walk, dim3(rows), dim3(SR_WAVE), 0, st, b);
+        hipLaunchKernelGGL(k_spec_residual, dim3(64, rows), dim3(256), 0, st, b);
+    }
+    hipLaunchKernelGGL(k_spec_verify, dim3(rows), dim3(kT), 0, st, b);
     return hipGetLastError();
 }
 hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int rows, const int* draft, float p_min,

@@ -475,6 +475,11 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
     a.uniforms_per_row = b->upr;
     a.out_accepted = out_accepted_dev;
     a.out_tokens = out_tokens_dev;
+    a.resid_stride = ((int64_t)V + 3) & ~(int64_t)3;
+    SR_HIP(ctx, ctx->spec_resid.reserve((size_t)rows * (size_t)a.resid_stride * sizeof(float), st));
+    SR_HIP(ctx, ctx->spec_reject.reserve((size_t)rows * sizeof(int32_t), st));
+    a.resid = ctx->spec_resid.as<float>();
+    a.reject = ctx->spec_reject.as<int32_t>();
     SR_HIP(ctx, sr_launch_spec_verify(a, rows, st));
     return SR_OK;
 }

@@ -196,6 +196,7 @@ struct sr_ctx {
     DeviceBuf redo_list;     // rows given to sr_resample_rows_launch
     int ident_rows = 0;
     DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
+    DeviceBuf spec_resid, spec_reject;  // ... the residual row of every row's first rejected position, that position
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
     int last_epv = 4;                    // vector width of the last launch: what an upload builds scan masks for

@@ -190,6 +190,9 @@ struct SrSpecArgs {
     int32_t uniforms_per_row;
     int32_t* out_accepted;       // [rows]
     int32_t* out_tokens;         // [rows][n_draft + 1]
+    float* resid;                // [rows][resid_stride]: max(0, p - q) of the row's first rejected position
+    int64_t resid_stride;
+    int32_t* reject;             // [rows]: that position, or -1 (none, or a row that does not take the ratio test)
 };
 hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st);
 hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int rows, const int* draft, float p_min,
