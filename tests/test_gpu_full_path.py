@@ -234,6 +234,24 @@ def test_speculative_verification_rows(ctx):
     _check_spec(ctx, t, q, k, p3, u)
 
 
+def test_corrections_drawn_at_both_ends_of_the_residual(ctx):
+    # The residual row of a row's first rejected position is written ahead of the verifier and read back by it.  Rows
+    # whose lengths leave the distributions at any alignment; a first uniform just below 1 (rejected unless the ratio is
+    # 1) or 0 (accepted wherever p > 0), so that rejections fall on the first and on later positions; corrections drawn
+    # with a uniform of 0 (the first positive residual), of the smallest positive double and of nearly 1 (the last
+    # entries of the running sum).
+    for V, seed in ((20_000, 11), (20_001, 12), (20_003, 13)):
+        rows, L = 8, 3
+        params = [SamplingParams() if r % 2 == 0 else SamplingParams(Temperature=0.8, TopK=60, TopP=0.9) for r in range(rows)]
+        t, q, k, u = _spec_case(rows, L, V, params, seed, True)
+        for first, corr in ((0.99999994, 0.0), (0.99999994, 0.99999994), (0.99999994, 5e-324), (0.0, 0.99999994), (0.3, 0.0)):
+            uu = u.copy()
+            uu[:, 0] = first
+            uu[:, 1:] = np.where(np.arange(rows)[:, None] % 3 == 0, corr, uu[:, 1:])  # every third row: all later draws
+            uu[1::3, 1] = corr                                                       # the others: the draw behind position 0
+            _check_spec(ctx, t, q, k, params, uu)
+
+
 def test_drafts_from_prompt_lookup_take_the_p_min_rule_whatever_p_min_is(ctx):
     # usedPld (SpeculativeDecoder.cs:488-501, 538-552): no draft distributions exist; accept iff px >= SpecDraftPMin or the
     # draft is the argmax, a rejection draws from p.  Rows of both kinds in one launch; then lookup rows alone with no q.
