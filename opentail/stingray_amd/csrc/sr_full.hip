@@ -1780,9 +1780,33 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 int upto = blk_excl_scan(own, &tot, sm);
 #pragma unroll
                 for (int q = 0; q < kPer; q++) { upto += (int)mine[q]; sums[tid * kPer + q] = (uint32_t)upto; }
+                // The first slab need not be full: count x the position's smallest value bounds the mass of the
+                // positions from below (in units of 2^-28), and the slab ends where that bound passes top-p (+ 0.1 %) --
+                // a few hundred entries for a sharp row instead of 4,096 to gather and sort.
+                uint32_t ownq = 0u, mq[kPer];
+#pragma unroll
+                for (int q = 0; q < kPer; q++) {
+                    const int d = tid * kPer + q;
+                    const float y_low = d < kPos - 1 ? sr_u2f((0x3fffu - (uint32_t)d) << 16) : 0.0f;
+                    mq[q] = (uint32_t)fminf((float)mine[q] * y_low * 268435456.0f, 268435456.0f);
+                    ownq += mq[q];
+                }
+                int totq;
+                uint32_t uptoq = (uint32_t)blk_excl_scan((int)ownq, &totq, sm);
+                if (tid == 0) sm.bc[7] = (uint32_t)kPos;
+                __syncthreads();
+                const uint32_t target_q = (uint32_t)(rd.top_p * 1.001f * 268435456.0f) + 64u;
+                int d_first = kPos;
+#pragma unroll
+                for (int q = 0; q < kPer; q++) {
+                    uptoq += mq[q];
+                    if (uptoq >= target_q && d_first == kPos) d_first = tid * kPer + q;
+                }
+                if (d_first < kPos) atomicMin(&sm.bc[7], (uint32_t)d_first);
                 sr_drain_stores();
                 __syncthreads();
             }
+            const uint32_t d_mass = use_hist ? sm.bc[7] : (uint32_t)kPos;
             FPROF(a, slot, 10);
             unsigned long long t_step = 0ull;
             FPROF_ADD(a, slot, 16, t_step);
@@ -1807,8 +1831,9 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                         sm.bc[5] = (uint32_t)d;
                     }
                     __syncthreads();
-                    const uint32_t d = sm.bc[5];
+                    uint32_t d = sm.bc[5];
                     __syncthreads();
+                    if (slab == 0) d = min(d, d_mass + 1u);
                     if (d < (uint32_t)(kPos - 1)) {
                         c_above = sr_u2f(((0x3fffu - d) << 16) | 0xffffu);
                     } else {  // (the shared last position: its keys are not one bucket)

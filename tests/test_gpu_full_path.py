@@ -406,6 +406,9 @@ def test_rows_that_only_top_p_cuts_at_every_size_of_nucleus(ctx):
     rows = len(params)
     for u in ([0.99999994] * rows, [0.0] * rows, [0.9995] * rows, rng.random(rows).tolist(), rng.random(rows).tolist()):
         _check_rows(ctx, logits, params, u)
+    # the same rows as distributions (written rows: the walk by slabs of the general way, its first slab ended by the
+    # bound on its mass)
+    _check_distribution(ctx, logits, params)
     allowed = rng.random((rows, V)) < np.array([0.5, 0.3, 0.9, 0.7, 0.2, 0.8])[:, None]
     mask = pack_allow_mask(allowed)
     active = np.ones(rows, dtype=np.uint8)
