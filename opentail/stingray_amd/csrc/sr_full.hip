@@ -1205,13 +1205,15 @@ __device__ __forceinline__ int list_stretch(const float* p, int w0, int w1, bool
 // The row holds e = expf(x - max); its probabilities are y = fl(e * inv) (y = e when the sum is 1), which rise with e.
 // While the exact sum passed over the row, the caller counted the e by their upper 16 bits in hcnt (LDS, kHistPos
 // positions: position d holds the keys 0x3f80 - d, position 0 is e = 1, the last position everything below).  From the
-// counts: the longest run of positions from the top that holds at most kSmall entries, shortened to where a lower bound
-// of its probability mass (count x the position's smallest value) passes top_p with a margin.  One read of the row lists
-// the entries above that bound in index order (every wave takes a stretch of the row and writes its finds to the same
-// stretch of the row's sort segment, then the stretches are joined in LDS); their values alone are sorted, the exact
-// running sum finds the cut, and the members -- the values above the cut value and the first few equal to it -- are
-// marked in the index-ordered list, from which the row is finished.  Returns false when the row has to go the general
-// way (nothing is written then but LDS and the row's sort segment).
+// counts: the longest run of positions from the top that holds at most kSmall entries (a slab), the first one shortened
+// to where a lower bound of its probability mass (count x the position's smallest value) passes top_p with a margin.
+// One read of the row lists a slab's entries (every wave takes a stretch of the row; the finds go to a pool in LDS
+// with their number within the wave, from which their places in index order follow); their values alone are sorted,
+// the exact running sum goes on through them, and slab follows slab until it reaches top_p.  The members -- the values
+// above the value at the cut and the first few equal to it by index -- are marked in the last slab's index-ordered
+// list, from which a nucleus of one slab is finished; one of several slabs has its members listed by one more read
+// of the row into the row's sort segment and is finished from there a block at a time.  Returns kNucleusDone, or
+// which general way the row has to go (nothing is written then but LDS and the row's sort segment).
 constexpr int kHistPos = 8192;
 constexpr uint32_t kHistTopKey = 0x3f80u;
 __device__ __forceinline__ void hist_count(uint32_t* hcnt, uint32_t* bad, float e)
