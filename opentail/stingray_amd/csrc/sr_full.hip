@@ -2478,7 +2478,7 @@ hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st)
 {
     if (rows <= 0) return hipSuccess;
     SrSpecArgs b = a;
-    if (!(b.resid && b.reject && b.n_draft > 0 && b.draft_probs)) {
+    if (!(b.resid && b.reject && b.n_draft > 0 && b.draft_probs && rows <= 65535)) {  // (rows are the grid's second dimension)
         b.resid = nullptr;
         b.reject = nullptr;
     } else {
