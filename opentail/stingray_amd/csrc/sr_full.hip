@@ -2207,6 +2207,17 @@ __device__ __forceinline__ int resample_residual_stored(const float* res, const 
     return found >= 0 ? found : edge(false);  // (rounding: the sum of the search fell short of the target)
 }
 
+// Every position of a row is filtered with the row's own parameters (SpeculativeDecoder.cs:535): the batch's row
+// descriptors, one copy per position, without their allow-masks
+__global__ __launch_bounds__(256) void k_expand_rows(const SrRow* src, SrRow* dst, int rows, int positions)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * positions) return;
+    SrRow d = src[i / positions];
+    d.mask_row = -1;
+    dst[i] = d;
+}
+
 // The accept loop of a row under the ratio test needs one element of p and of q per position, no pass over a row:
 // one wave walks it ahead of everything else and names the first rejected position, so that the residual row of
 // that position -- which the row's workgroup would otherwise compute twice, from two rows, at the rate of one compute
@@ -2472,6 +2483,12 @@ hipError_t sr_launch_residual_rows(const float* p, int64_t ps, const float* q, i
 {
     if (rows <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_residual_rows, dim3(rows), dim3(kT), 0, st, p, ps, q, qs, n, u, out);
+    return hipGetLastError();
+}
+hipError_t sr_launch_expand_rows(const SrRow* src, SrRow* dst, int rows, int positions, hipStream_t st)
+{
+    if (rows <= 0 || positions <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_expand_rows, dim3((unsigned)((rows * positions + 255) / 256)), dim3(256), 0, st, src, dst, rows, positions);
     return hipGetLastError();
 }
 hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st)

@@ -433,18 +433,10 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
     // batch's row descriptors to rows x positions and build all distributions in one pass.
     if ((int64_t)rows * P * V >= (int64_t)1 << 31)
         return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_spec_verify_launch: rows x positions x vocab exceeds 2^31 entries");
-    std::vector<SrRow> exp_rows((size_t)rows * P);
     bool any_top_p = false;
-    for (int r = 0; r < rows; r++)
-        for (int i = 0; i < P; i++) {
-            SrRow d = b->h_rows[(size_t)r];
-            d.mask_row = -1;
-            exp_rows[(size_t)r * P + i] = d;
-            any_top_p = any_top_p || row_uses_top_p(d);
-        }
-    SR_HIP(ctx, ctx->spec_rows.reserve(exp_rows.size() * sizeof(SrRow), st));
-    SR_HIP(ctx, hipMemcpyAsync(ctx->spec_rows.p, exp_rows.data(), exp_rows.size() * sizeof(SrRow), hipMemcpyHostToDevice, st));
-    SR_HIP(ctx, hipStreamSynchronize(st));
+    for (int r = 0; r < rows; r++) any_top_p = any_top_p || row_uses_top_p(b->h_rows[(size_t)r]);
+    SR_HIP(ctx, ctx->spec_rows.reserve((size_t)rows * P * sizeof(SrRow), st));
+    SR_HIP(ctx, sr_launch_expand_rows(b->d_rows.as<SrRow>(), ctx->spec_rows.as<SrRow>(), rows, P, st));  // (no wait for the host)
     SR_HIP(ctx, ctx->spec_probs.reserve((size_t)rows * P * V * sizeof(float), st));
     sr_batch tmp;  // a view: expanded rows, the original edits
     tmp.ctx = ctx;

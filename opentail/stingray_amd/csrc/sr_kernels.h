@@ -195,6 +195,7 @@ struct SrSpecArgs {
     int32_t* reject;             // [rows]: that position, or -1 (none, or a row that does not take the ratio test)
 };
 hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st);
+hipError_t sr_launch_expand_rows(const SrRow* src, SrRow* dst, int rows, int positions, hipStream_t st);
 hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int rows, const int* draft, float p_min,
                                 int* out_argmax, int* out_accept, float* out_prob, hipStream_t st);
 hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum, int* out_idx,
