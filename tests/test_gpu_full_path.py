@@ -252,6 +252,37 @@ def test_corrections_drawn_at_both_ends_of_the_residual(ctx):
             _check_spec(ctx, t, q, k, params, uu)
 
 
+def test_verification_after_tokens_were_appended_to_the_batch(ctx):
+    # The verifier copies the batch's row descriptors on the device: rows with penalties whose histories grew by
+    # sr_batch_append_tokens (in place, no new upload) must be verified with the histories as they are now.
+    import torch
+
+    V, L, rows = 20_000, 3, 6
+    rng = np.random.default_rng(515)
+    hist = [rng.integers(0, V, 40).tolist() for _ in range(rows)]
+    def params_of(h):
+        return [SamplingParams(Temperature=0.9, TopP=0.95, FrequencyPenalty=0.4, PresencePenalty=0.2, RepetitionPenalty=1.1,
+                               PreviousTokens=list(h[r])) for r in range(rows)]
+    t, q, k, u = _spec_case(rows, L, V, params_of(hist), 21, True)
+    batch = ctx.new_batch().upload(params_of(hist), V, u)
+    for step in range(3):
+        new = rng.integers(0, V, rows)
+        for r in range(rows):
+            hist[r].append(int(new[r]))
+        u = rng.random((rows, L + 1))
+        batch.append_tokens(new, u)
+    acc = torch.zeros(rows, dtype=torch.int32, device="cuda")
+    out = torch.zeros((rows, L + 1), dtype=torch.int32, device="cuda")
+    ctx.spec_verify_launch(batch, _cuda(t), _cuda(q), _cuda(k), acc, out)
+    ctx.synchronize()
+    acc, out = acc.cpu().numpy(), out.cpu().numpy()
+    now = params_of(hist)
+    for r in range(rows):
+        wa, wt = orc.spec_verify_row(t[r], q[r], k[r], to_oracle(now[r]), orc.Rng(replay=u[r]))
+        assert acc[r] == wa and list(out[r][: wa + 1]) == list(wt), (r, acc[r], wa, out[r], wt)
+    batch.close()
+
+
 def test_drafts_from_prompt_lookup_take_the_p_min_rule_whatever_p_min_is(ctx):
     # usedPld (SpeculativeDecoder.cs:488-501, 538-552): no draft distributions exist; accept iff px >= SpecDraftPMin or the
     # draft is the argmax, a rejection draws from p.  Rows of both kinds in one launch; then lookup rows alone with no q.
