@@ -305,6 +305,7 @@ SR_API int sr_resample_residual(sr_ctx* ctx, const float* p, int32_t p_len, int6
  * correction or bonus token, the rest -1.  A draft id outside [0, vocab) ends its row at that
  * position with -1 in place of the correction token (the managed loop throws IndexOutOfRangeException at
  * pDist[x_i], :536); out_accepted counts the drafts accepted before it.
+ * The call enqueues its kernels on the context's stream and returns without waiting for them.
  */
 SR_API int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* batch, const float* target_logits_dev,
                                  const float* draft_probs_dev, const int32_t* draft_tokens_dev,
