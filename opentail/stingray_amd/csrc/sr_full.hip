@@ -1234,7 +1234,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
     const uint32_t* hcnt = (const uint32_t*)sm.sortbuf;
     uint32_t* sval = (uint32_t*)sm.sprob;
-    unsigned long long t_step = 0ull;
+    [[maybe_unused]] unsigned long long t_step = 0ull;
     FPROF_ADD(a, slot, 16, t_step);
     if (sm.bc[5] != 0u) return kNucleusGeneral;
     // counts and mass bounds (in units of 2^-28) of this thread's positions
@@ -1810,7 +1810,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             }
             const uint32_t d_mass = use_hist ? sm.bc[7] : (uint32_t)kPos;
             FPROF(a, slot, 10);
-            unsigned long long t_step = 0ull;
+            [[maybe_unused]] unsigned long long t_step = 0ull;
             FPROF_ADD(a, slot, 16, t_step);
             bool closed = false;
             float run = 0.0f;                  // exact running sum behind the slabs taken so far
