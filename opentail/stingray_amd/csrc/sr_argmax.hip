@@ -84,15 +84,26 @@ template <int ES, bool kVec> __global__ __launch_bounds__(kThreads) void k_argma
     if (kVec) {
         const u32x4* vp = (const u32x4*)rowp;
         const int v_lo = lo / EPV, v_hi = hi / EPV;  // whole vectors; only the row's last chunk can leave elements over
-        int i = v_lo + tid;
-        for (; i + (kUnroll - 1) * kThreads < v_hi; i += kUnroll * kThreads) {
+        // Sets of kUnroll vectors per thread, all of a set's loads issued before the first is folded.  The chunk's last
+        // set is loaded whole too -- a vector past the chunk's end is the chunk's last one again and is not folded --
+        // rather than vector by vector, each of which would be a trip to memory of its own.
+        const int last = v_hi - 1;
+        for (int base = v_lo; base < v_hi; base += kUnroll * kThreads) {
+            const int i = base + tid;
             u32x4 t[kUnroll];
+            if (base + kUnroll * kThreads <= v_hi) {
 #pragma unroll
-            for (int j = 0; j < kUnroll; j++) t[j] = __builtin_nontemporal_load(vp + i + j * kThreads);
+                for (int j = 0; j < kUnroll; j++) t[j] = __builtin_nontemporal_load(vp + i + j * kThreads);
 #pragma unroll
-            for (int j = 0; j < kUnroll; j++) fold_vec<ES>(tb, t[j], (uint32_t)(i + j * kThreads) * EPV);
+                for (int j = 0; j < kUnroll; j++) fold_vec<ES>(tb, t[j], (uint32_t)(i + j * kThreads) * EPV);
+            } else {
+#pragma unroll
+                for (int j = 0; j < kUnroll; j++) t[j] = __builtin_nontemporal_load(vp + min(i + j * kThreads, last));
+#pragma unroll
+                for (int j = 0; j < kUnroll; j++)
+                    if (i + j * kThreads < v_hi) fold_vec<ES>(tb, t[j], (uint32_t)(i + j * kThreads) * EPV);
+            }
         }
-        for (; i < v_hi; i += kThreads) fold_vec<ES>(tb, __builtin_nontemporal_load(vp + i), (uint32_t)i * EPV);
         scalar_from = max(lo, v_hi * EPV);
     }
     for (int i = scalar_from + tid; i < hi; i += kThreads) fold(tb, load_elem<ES>(rowp, i), (uint32_t)i);
@@ -132,9 +143,11 @@ void sr_argmax_plan(SrArgmaxArgs& a, int cu_count)
 {
     const int es = a.dtype == 1 ? 2 : 4, epv = 16 / es;
     a.vec = ((uintptr_t)a.logits % 16 == 0 && ((size_t)a.row_stride * es) % 16 == 0) ? 1 : 0;
-    // enough workgroups for eight per compute unit, none with less than one unrolled pass of work
+    // enough workgroups for two per compute unit (64 KB of loads in flight on each: what the memory's latency takes at
+    // the machine's rate; eight per compute unit, with their dispatch and their atomics, were 5 us slower on 256 rows of
+    // 151,936), none with less than one unrolled pass of work
     const int per_pass = kThreads * kUnroll * epv;
-    int s = std::max(1, std::min((8 * cu_count + a.rows - 1) / std::max(a.rows, 1), a.vocab / per_pass));
+    int s = std::max(1, std::min((2 * cu_count + a.rows - 1) / std::max(a.rows, 1), a.vocab / per_pass));
     int len = (a.vocab + s - 1) / s;
     len = (len + epv - 1) / epv * epv;
     a.chunk_len = std::max(len, epv);
