@@ -1506,11 +1506,82 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     return kNucleusDone;
 }
 
+// ---- the survivors of a row sorted where they lie -------------------------------------------------------------------
+// keys[i] (probability bits) and ids[i] (indices) of ns entries in device memory, sorted by descending key, equal keys
+// by ascending index, by this workgroup alone: a bitonic network whose comparators all point the same way (a merge
+// starts by comparing every entry with its mirror image in the block, then halves), so that a length that is no power of
+// two needs no padding in memory -- the entries past the end count as the smallest and never move.  Tiles of kSmall
+// entries are sorted and merged in LDS; only the steps that reach across tiles go through memory.  For the rare row
+// whose nucleus the walk by slabs cannot close: about 2 ms for 130 thousand survivors.
+__device__ __forceinline__ void sort_survivors_in_place(uint32_t* keys, int32_t* ids, int ns, FullSmem& sm)
+{
+    typedef unsigned long long u64;
+    const int tid = threadIdx.x;
+    auto ld = [&](int i) -> u64 { return ((u64)keys[i] << 32) | (u64)(0xffffffffu - (uint32_t)ids[i]); };
+    auto st = [&](int i, u64 v) { keys[i] = (uint32_t)(v >> 32); ids[i] = (int32_t)(0xffffffffu - (uint32_t)v); };
+    auto tile_in = [&](int t0) {
+        for (int e = tid; e < kSmall; e += kT) sm.sortbuf[e] = t0 + e < ns ? ld(t0 + e) : 0ull;
+        __syncthreads();
+    };
+    auto tile_out = [&](int t0) {
+        for (int e = tid; e < kSmall; e += kT)
+            if (t0 + e < ns) st(t0 + e, sm.sortbuf[e]);
+        sr_drain_stores();
+        __syncthreads();
+    };
+    __syncthreads();
+    for (int t0 = 0; t0 < ns; t0 += kSmall) {
+        tile_in(t0);
+        sort_lds_desc(sm.sortbuf, kSmall);
+        tile_out(t0);
+    }
+    int total = kSmall;  // the power of two that the network is laid out for
+    while (total < ns) total <<= 1;
+    for (int k2 = 2 * kSmall; k2 <= total; k2 <<= 1) {
+        // every entry of a block's first half against its mirror image in the second
+        for (int pr = tid; pr < total / 2; pr += kT) {
+            const int blk = pr / (k2 / 2), off = pr - blk * (k2 / 2);
+            const int i = blk * k2 + off, j = blk * k2 + k2 - 1 - off;
+            if (j < ns) {
+                const u64 x = ld(i), y = ld(j);
+                if (x < y) { st(i, y); st(j, x); }
+            }
+        }
+        sr_drain_stores();
+        __syncthreads();
+        // halves, quarters, ... of the block down to the size of a tile
+        for (int j2 = k2 / 4; j2 >= kSmall; j2 >>= 1) {
+            for (int pr = tid; pr < total / 2; pr += kT) {
+                const int i = ((pr & ~(j2 - 1)) << 1) | (pr & (j2 - 1)), j = i | j2;
+                if (j < ns) {
+                    const u64 x = ld(i), y = ld(j);
+                    if (x < y) { st(i, y); st(j, x); }
+                }
+            }
+            sr_drain_stores();
+            __syncthreads();
+        }
+        // the rest of the merge inside every tile
+        for (int t0 = 0; t0 < ns; t0 += kSmall) {
+            tile_in(t0);
+            for (int j2 = kSmall / 2; j2 >= 1; j2 >>= 1) {
+                for (int pr = tid; pr < kSmall / 2; pr += kT) {
+                    const int i = ((pr & ~(j2 - 1)) << 1) | (pr & (j2 - 1)), j = i | j2;
+                    const u64 x = sm.sortbuf[i], y = sm.sortbuf[j];
+                    if (x < y) { sm.sortbuf[i] = y; sm.sortbuf[j] = x; }
+                }
+                __syncthreads();
+            }
+            tile_out(t0);
+        }
+    }
+}
+
 // ---- stage 3: softmax, top-k, min-p, top-p on the work row --------------------------------------------
 // phase 1 ends after top-p for rows whose nucleus candidates fit the kernel (<= kSmall survivors), or
 // after compacting the survivors for the device-wide sort otherwise; phase 2 finishes those rows and
 // then normalises, draws and writes results for every row.
-__global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
+__global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
 {
     __shared__ FullSmem sm;
     const int tid = threadIdx.x;
@@ -1524,7 +1595,6 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
     const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
 
     if (greedy) {
-        if (phase == 2) return;
         // Greedy / GreedyWithHistoryPenalties on the adjusted row; distributions become one-hot
         const int am = row_argmax(p, n, sm);
         if (a.mode != 0) {
@@ -1534,15 +1604,11 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         if (tid == 0) {
             if (a.out_tokens) a.out_tokens[row] = am;
             if (a.out_flags) a.out_flags[row] = SR_KFLAG_GREEDY | SR_KFLAG_FULL;
-            // an empty segment for the device-wide sort that may follow (it reads every row's bounds)
-            a.seg_begin[slot] = a.seg_end[slot] = (int)((size_t)slot * a.sort_stride);
-            st->big = 0;
-            st->pad = 1;
         }
         return;
     }
 
-    if (phase == 1) {
+    {
         FPROF(a, slot, 0);
         // Softmax (Sampler.cs:448-472): the maximum and e = expf(x - max) were computed by the kernels before
         const uint32_t mk = st->maxkey;
@@ -1620,10 +1686,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                     st->mul1 = inv;
                     st->mul2 = inv2;
                     st->n_survivors = 0;
-                    st->big = 0;
                     st->flags = flags;
-                    st->pad = 1;  // finished in this phase
-                    a.seg_begin[slot] = a.seg_end[slot] = (int)((size_t)slot * a.sort_stride);
                     if (a.out_flags) a.out_flags[row] = flags;
                 }
                 return;
@@ -1634,10 +1697,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 FPROF(a, slot, 9);
                 if (tid == 0) {
                     st->n_survivors = 0;
-                    st->big = 0;
                     st->flags = flags;
-                    st->pad = 1;  // finished in this phase
-                    a.seg_begin[slot] = a.seg_end[slot] = (int)((size_t)slot * a.sort_stride);
                     if (a.out_flags) a.out_flags[row] = flags;
                 }
                 return;
@@ -1731,7 +1791,6 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         }
         FPROF(a, slot, 5);
         // ApplyTopP (Sampler.cs:516-551)
-        int big = 0;
         int listed = -1;  // the row's survivors are sm.sortbuf[0, listed)
         if (use_top_p) {
             int cnt = survivors;
@@ -1896,9 +1955,8 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                 }
             }
             if (ns > 0 && !closed) {
-                // the nucleus reaches past the candidates: the survivors, in index order (equal probabilities keep
-                // it through the stable sort), go to this row's segment of the device-wide sort
-                big = 1;
+                // the nucleus reaches past what the walk by slabs takes: the survivors go to the row's sort segment and
+                // are sorted there
                 uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
                 int32_t* ids = a.sort_vals_in + (size_t)slot * a.sort_stride;
                 const bool aligned = ((uintptr_t)p & 15u) == 0u;
@@ -1922,6 +1980,14 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
                         if (v[q] > 0.0f) { keys[pos] = sr_f2u(v[q]); ids[pos] = i + q; pos++; }
                     base += tot;
                 }
+                sr_drain_stores();
+                sort_survivors_in_place(keys, ids, ns, sm);
+                // the nucleus over the sorted survivors (descending probability, ascending index among equal ones)
+                int found;
+                seq_sum<true>([&](int i) -> float { return sr_u2f(keys[i]); }, ns, 0.0f, rd.top_p, &found, sm);
+                const int cutoff = found >= 0 ? found + 1 : ns;
+                for (int i = cutoff + tid; i < ns; i += kT) p[ids[i]] = 0.0f;
+                __syncthreads();
             }
             if (tid == 0) st->n_survivors = ns;
         } else if (ns_listed > 0 && ns_listed <= kSmall && n >= 8) {
@@ -1930,11 +1996,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
         FPROF(a, slot, 6);
         const bool finish_here = listed > 0 && listed <= kSmall && n >= 8;
         if (tid == 0) {
-            st->big = big;
             st->flags = flags;
-            st->pad = finish_here ? 1 : 0;  // 1 = the row is finished in this phase
-            a.seg_begin[slot] = (int)((size_t)slot * a.sort_stride);
-            a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + (big ? st->n_survivors : 0);
         }
         if (finish_here) {
             // the nucleus closed inside the kernel and its members are at hand: no pass over the row is needed
@@ -1943,21 +2005,6 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a, int phase)
             if (tid == 0 && a.out_flags) a.out_flags[row] = flags;
             return;
         }
-        if (a.two_phase) return;
-        __syncthreads();
-    }
-    if (a.two_phase && st->pad == 1) return;  // finished in phase 1
-
-    // ---- phase 2 --------------------------------------------------------------------------------------
-    if (a.two_phase && st->big) {
-        // nucleus over the device-sorted survivors (descending probability, ascending index on ties)
-        const uint32_t* keys = a.sort_keys_out + (size_t)slot * a.sort_stride;
-        const int* vals = a.sort_vals_out + (size_t)slot * a.sort_stride;
-        const int ns = st->n_survivors;
-        int found;
-        seq_sum<true>([&](int i) -> float { return sr_u2f(keys[i]); }, ns, 0.0f, rd.top_p, &found, sm);
-        const int cutoff = found >= 0 ? found + 1 : ns;
-        for (int i = cutoff + tid; i < ns; i += kT) p[vals[i]] = 0.0f;
         __syncthreads();
     }
     FPROF(a, slot, 7);
@@ -2465,10 +2512,10 @@ hipError_t sr_launch_wide_tail(const SrFullArgs& a, int n_rows, hipStream_t st)
     hipLaunchKernelGGL(k_wide_tail, dim3(n_rows), dim3(kT), 0, st, a);
     return hipGetLastError();
 }
-hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st)
+hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, hipStream_t st)
 {
     if (n_rows <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_full_row, dim3(n_rows), dim3(kT), 0, st, a, phase);
+    hipLaunchKernelGGL(k_full_row, dim3(n_rows), dim3(kT), 0, st, a);
     return hipGetLastError();
 }
 hipError_t sr_launch_draw_rows(const float* probs, int64_t stride, int n, int rows, const double* u, int* out,

@@ -40,7 +40,6 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
         a.work_stride = probs_stride;
         a.work_by_row = 1;
     }
-    a.two_phase = any_top_p ? 1 : 0;
     a.lazy_scale = lazy_scale ? 1 : 0;
     // Which of the rows that come here keep an adjusted copy, and which have their edits applied where they are read
     // (the rows of the batch that take this path: every row in modes 1 / 2).
@@ -60,27 +59,18 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     }
     SR_HIP(ctx, ctx->full_state.reserve((size_t)n_rows * sizeof(SrFullState), st));
     a.state = ctx->full_state.as<SrFullState>();
-    SR_HIP(ctx, ctx->seg.reserve((size_t)n_rows * 2 * sizeof(int32_t), st));
-    a.seg_begin = ctx->seg.as<int32_t>();
-    a.seg_end = a.seg_begin + n_rows;
     // sort segments are laid out with the work stride of mode 0; in modes 1/2 use a private stride
     const int64_t seg_stride = (vocab + 3) & ~3;
     if ((int64_t)n_rows * seg_stride >= (int64_t)1 << 31)
         return sr_fail(ctx, SR_ERR_UNSUPPORTED, "full-vocabulary path: rows x vocab exceeds 2^31 entries");
-    size_t tmp_bytes = 0;
-    if (a.two_phase) {
+    if (any_top_p) {
+        // a row's segment: scratch of its top-p stage (histogram sums, the members of a long nucleus, and the survivors
+        // of a row that the walk by slabs cannot close, sorted there by the row's workgroup)
         const size_t items = (size_t)n_rows * seg_stride;
         SR_HIP(ctx, ctx->sort_k0.reserve(items * 4, st));
-        SR_HIP(ctx, ctx->sort_k1.reserve(items * 4, st));
         SR_HIP(ctx, ctx->sort_v0.reserve(items * 4, st));
-        SR_HIP(ctx, ctx->sort_v1.reserve(items * 4, st));
         a.sort_keys_in = ctx->sort_k0.as<uint32_t>();
         a.sort_vals_in = ctx->sort_v0.as<int32_t>();
-        a.sort_keys_out = ctx->sort_k1.as<uint32_t>();
-        a.sort_vals_out = ctx->sort_v1.as<int32_t>();
-        SR_HIP(ctx, sr_segmented_sort_desc(nullptr, &tmp_bytes, a.sort_keys_in, ctx->sort_k1.as<uint32_t>(), a.sort_vals_in,
-                                           ctx->sort_v1.as<int32_t>(), (int64_t)items, n_rows, a.seg_begin, a.seg_end, st));
-        SR_HIP(ctx, ctx->sort_tmp.reserve(tmp_bytes + 256, st));
     }
     // the kernels index sort segments with work_stride; keep both strides equal in mode 0 and pass the
     // segment stride separately otherwise
@@ -91,14 +81,7 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     a.out_flags = out_flags_dev;
 
     SR_HIP(ctx, sr_launch_full_prep(a, n_rows, st));
-    SR_HIP(ctx, sr_launch_full_row(a, n_rows, 1, st));
-    if (a.two_phase) {
-        const size_t items = (size_t)n_rows * seg_stride;
-        SR_HIP(ctx, sr_segmented_sort_desc(ctx->sort_tmp.p, &tmp_bytes, a.sort_keys_in, ctx->sort_k1.as<uint32_t>(),
-                                           a.sort_vals_in, ctx->sort_v1.as<int32_t>(), (int64_t)items, n_rows, a.seg_begin,
-                                           a.seg_end, st));
-        SR_HIP(ctx, sr_launch_full_row(a, n_rows, 2, st));
-    }
+    SR_HIP(ctx, sr_launch_full_row(a, n_rows, st));  // (every row is finished by this one launch)
     return SR_OK;
 }
 

@@ -123,9 +123,9 @@ hipError_t sr_launch_selftest_expf(const float* x, float* y, int64_t n, hipStrea
 // ---- full-vocabulary path (sr_full.hip) ---------------------------------------------------------------
 struct SrFullState {
     int32_t n_survivors;  // entries with probability > 0 when top-p starts
-    int32_t big;          // survivors exceed what the row kernel sorts itself: device-wide sort needed
+    int32_t unused0;
     uint32_t flags;
-    int32_t pad;          // 1 = the row was finished by the first phase
+    int32_t unused1;
     uint32_t maxkey;      // ordered key of the row's largest adjusted logit (0xffffffff = the row holds a NaN)
     float mul1, mul2;     // the row's entries are to be multiplied by these two, in this order (1 unless lazy_scale)
     int32_t pad2;
@@ -145,7 +145,6 @@ struct SrFullArgs {
     int64_t work_stride;
     int32_t work_by_row;
     int32_t mode;              // 0 = sample, 1 = distribution only, 2 = distribution and sample
-    int32_t two_phase;         // a device-wide sort of large nuclei runs between phase 1 and phase 2
     int32_t lazy_scale;        // mode 1 only: rows that no filter touches keep expf(x - max); their two normalising
                                // factors go to state[slot].mul1 / mul2 for the reader to apply
     uint32_t* edit_tab;        // [slot][edit_tab_stride]: per row a bitmap of the ids its edits touch and one float per
@@ -166,7 +165,7 @@ struct SrFullArgs {
     unsigned long long* prof;  // optional phase timestamps of slot 0 [32] (test hook), normally null
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
-hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, int phase, hipStream_t st);
+hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, hipStream_t st);
 // SampleTopK by device-wide sorts (rows beyond the selection kernel's limits): keys of the whole row, the adjusted
 // first `sel` entries, the walk over the sorted result
 hipError_t sr_launch_wide_keys(const SrFullArgs& a, int n_rows, hipStream_t st);
