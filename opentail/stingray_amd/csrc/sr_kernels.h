@@ -200,7 +200,7 @@ hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int 
 hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum, int* out_idx,
                                      hipStream_t st);
 
-// Stable descending segmented sort of (probability bits, index) pairs (sr_sort.hip, rocPRIM/hipCUB).
+// Stable descending segmented sort of (key, index) pairs (sr_sort.hip, rocPRIM/hipCUB): the wide top-k rows.
 // With tmp == nullptr only *tmp_bytes is set.
 hipError_t sr_segmented_sort_desc(void* tmp, size_t* tmp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
                                   const int32_t* vals_in, int32_t* vals_out, int64_t n_items, int n_segments,

@@ -1,5 +1,5 @@
-// Device-wide stable segmented radix sort (descending) for nuclei too large to sort inside one
-// workgroup.  Equal probabilities keep their input order, which is ascending token index.
+// Device-wide stable segmented radix sort (descending) of whole rows: SampleTopK beyond the selection kernel's limits
+// (sr_wide_rows_launch).  Equal keys keep their input order, which is ascending token index.
 #include <hip/hip_runtime.h>
 #include <hipcub/hipcub.hpp>
 
