@@ -1226,6 +1226,7 @@ __device__ __forceinline__ void hist_count(uint32_t* hcnt, uint32_t* bad, float 
 }
 enum NucleusWay : int { kNucleusDone = 0, kNucleusGeneral = 1, kNucleusGeneralNoSlabs = 2 };
 constexpr int kNucleusMaxSlabs = 24;
+constexpr int kNucleusRowFinish = 4;  // a nucleus that took more slabs than this is finished by passes over the row
 __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float top_p, const float* p, int n, int slot,
                                                       int row, bool do_scale, float inv, FullSmem& sm)
 {
@@ -1471,6 +1472,23 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     // the row, again in index order in the waves' stretches of the sort segment, and the final Normalize and the draw
     // take them from there a block at a time.
     const float ycut_f = sr_u2f(ycut);
+    if (slab >= kNucleusRowFinish) {
+        // A nucleus of many thousands of members: listing them and passing over the list, 5 us per thousand, costs more
+        // than writing the row -- scaled, everything outside the nucleus zero -- and the two passes over it of the
+        // final Normalize and the pass of the draw (about 70 us for 151,936 entries).
+        float* w = const_cast<float*>(p);
+        row_pass<true>(w, n, [&](float e, int i) -> float {
+            const float y = do_scale ? __fmul_rn(e, inv) : e;
+            return (y > ycut_f || (y == ycut_f && i <= idx_last)) ? y : 0.0f;
+        });
+        __syncthreads();
+        normalize_row(w, n, sm);
+        if (a.mode != 1) {
+            const int token = draw_from_row(w, n, a.uniforms[(size_t)row * a.uniforms_per_row], sm);
+            if (tid == 0 && a.out_tokens) a.out_tokens[row] = token;
+        }
+        return kNucleusDone;
+    }
     const int cm = list_stretch(p, w0, w1, do_scale, inv, StretchToSegment{gk, gi, w0},
                                 [&](float y, int i) -> bool { return y > ycut_f || (y == ycut_f && i <= idx_last); });
     sr_drain_stores();
