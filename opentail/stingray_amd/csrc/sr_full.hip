@@ -1139,6 +1139,19 @@ struct StretchToPool {  // appended to a pool in LDS that all waves share: value
         if (place < kSmall) { vals[place] = ybits; tags[place] = ((uint32_t)rank << kTagIndexBits) | (uint32_t)i; }
     }
 };
+struct StretchCount {  // nothing is kept: the wave's count is what list_stretch returns
+    __device__ __forceinline__ int reserve(int, int) const { return 0; }
+    __device__ __forceinline__ void put(int, int, uint32_t, int) const {}
+};
+struct StretchFind {  // the index of the wave's find number `target` (none for a negative target)
+    int target;
+    uint32_t* out;
+    __device__ __forceinline__ int reserve(int, int) const { return 0; }
+    __device__ __forceinline__ void put(int, int rank, uint32_t, int i) const
+    {
+        if (rank == target) *out = (uint32_t)i;
+    }
+};
 template <typename Sink, typename Pred>
 __device__ __forceinline__ int list_stretch(const float* p, int w0, int w1, bool do_scale, float inv, Sink sink, Pred pred)
 {
@@ -1225,7 +1238,7 @@ __device__ __forceinline__ void hist_count(uint32_t* hcnt, uint32_t* bad, float 
     }
 }
 enum NucleusWay : int { kNucleusDone = 0, kNucleusGeneral = 1, kNucleusGeneralNoSlabs = 2 };
-constexpr int kNucleusMaxSlabs = 24;
+constexpr int kNucleusMaxSlabs = 40;
 constexpr int kNucleusRowFinish = 4;  // a nucleus that took more slabs than this is finished by passes over the row
 __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float top_p, const float* p, int n, int slot,
                                                       int row, bool do_scale, float inv, FullSmem& sm)
@@ -1255,6 +1268,10 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     int tot, totq;
     const int c0 = blk_excl_scan(own, &tot, sm);
     const uint32_t q0 = (uint32_t)blk_excl_scan((int)ownq, &totq, sm);
+    int crowd = 0;  // entries at positions that hold more than a slab (runs of one value, if the row can be walked at all)
+#pragma unroll
+    for (int j = 0; j < kPer; j++) crowd += mine[j] > (uint32_t)kSmall ? (int)mine[j] : 0;
+    const int crowded_total = blk_sum_i(crowd, sm);
     if (tid == 0) { sm.bc[7] = (uint32_t)kHistPos; sm.bc[11] = (uint32_t)tot; }
     __syncthreads();
     {
@@ -1286,6 +1303,11 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     int taken = 0;         // entries that the histogram holds at the positions before d_prev
     int found = -1, nc = 0, slab = 0;
     bool all_in = false;
+    int runs = 0;              // positions passed as runs of one value
+    bool was_capped = false;   // ... after which what is left is bounded from above too
+    bool cut_in_run = false;   // the cut fell inside such a run: ycut / idx_last are set by the walk
+    uint32_t ycut = 0u;
+    int idx_last = -1;         // the last member among the entries equal to the cut value
     uint32_t pv[4] = {0u, 0u, 0u, 0u};  // the last slab's entries that this thread read from the pool: values,
     int pi[4] = {0, 0, 0, 0};            // indices
     int lpos[4] = {0, 0, 0, 0};          // and places in index order
@@ -1305,10 +1327,101 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         __syncthreads();
         // about how many entries the nucleus holds: a row that would need more slabs than are walked goes the general
         // way at once (its survivors are sorted device-wide)
-        if (slab == 0 && (int)sm.bc[11] > (kMaxSlabs - 2) * kSmall) return kNucleusGeneralNoSlabs;
+        if (slab == 0 && runs == 0 && (int)sm.bc[11] - min((int)sm.bc[11], crowded_total) > (kMaxSlabs - 2) * kSmall)
+            return kNucleusGeneralNoSlabs;
         const int d_cnt = (int)sm.bc[6], d_mass = (int)sm.bc[7];
         const int d_end = d_mass + 1 > d_prev ? min(d_cnt, d_mass + 1) : d_cnt;
-        if (d_end <= d_prev) return kNucleusGeneralNoSlabs;  // (one position alone holds more than a slab: no walk by slabs passes it)
+        if (d_end <= d_prev) {
+            // One position alone holds more than a slab.  Where all its entries share one probability -- the equal
+            // logits of a coarse grid, of bf16 -- no order among them is needed: the running sum goes through them
+            // as through so many equal terms, and if the cut falls among them, the members are the first ones by
+            // index.  Anything else is left to the general way's sort.
+            if (++runs > 256) return kNucleusGeneralNoSlabs;
+            const uint32_t key_d = kHistTopKey - (uint32_t)d_prev;
+            const bool last_pos = d_prev == kHistPos - 1;
+            // the position's distinct probabilities (a few at most, or the row is left to the sort) and their counts
+            constexpr int kDistinct = 16;
+            uint32_t* dval = sm.hist + 32;
+            uint32_t* dcnt = sm.hist + 32 + kDistinct;
+            __syncthreads();
+            if (tid < 2 * kDistinct) sm.hist[32 + tid] = 0u;
+            if (tid == 0) sm.bc[12] = 0u;
+            __syncthreads();
+            row_pass<false>(const_cast<float*>(p), n, [&](float e, int) -> float {
+                const uint32_t k16 = sr_f2u(e) >> 16;
+                if (e > 0.0f && (last_pos ? k16 <= key_d : k16 == key_d)) {
+                    const uint32_t yb = sr_f2u(do_scale ? __fmul_rn(e, inv) : e);
+                    bool placed = false;
+                    for (int sl = 0; sl < kDistinct && !placed; sl++) {
+                        const uint32_t old = atomicCAS(&dval[sl], 0u, yb);
+                        if (old == 0u || old == yb) {
+                            atomicAdd(&dcnt[sl], 1u);
+                            placed = true;
+                        }
+                    }
+                    if (!placed || yb < 0x00800000u) sm.bc[12] = 1u;  // (too many values, or one below the normal range)
+                }
+                return e;
+            });
+            __syncthreads();
+            if (sm.bc[12] != 0u) return kNucleusGeneralNoSlabs;
+            // from the largest value down (every thread finds the same order)
+            uint32_t below = 0xffffffffu;  // values at or above this one are done
+            bool cut_here = false;
+            for (int round = 0; round < kDistinct; round++) {
+                uint32_t mn = 0u;
+                int c_run = 0;
+                for (int sl = 0; sl < kDistinct; sl++) {
+                    const uint32_t v = dval[sl];
+                    if (v != 0u && v < below && v > mn) { mn = v; c_run = (int)dcnt[sl]; }
+                }
+                if (mn == 0u) break;  // all of the position's values are done
+                below = mn;
+                const float yv = sr_u2f(mn);
+                int f;
+                run = seq_sum<true>([&](int) -> float { return yv; }, c_run, run, top_p, &f, sm);
+                if (f < 0) continue;
+                // the cut falls inside this run: its first f + 1 entries by index are members
+                const int cw = list_stretch(p, w0, w1, do_scale, inv, StretchCount{}, [&](float y, int) -> bool { return sr_f2u(y) == mn; });
+                __syncthreads();
+                if (lane == 0) sm.redi[wave] = cw;
+                if (tid == 0) sm.bc[9] = 0xffffffffu;
+                __syncthreads();
+                int before_w = 0;
+#pragma unroll
+                for (int w = 0; w < kW; w++) before_w += w < wave ? sm.redi[w] : 0;
+                const int target = (f >= before_w && f < before_w + cw) ? f - before_w : -1;
+                __syncthreads();
+                (void)list_stretch(p, w0, w1, do_scale, inv, StretchFind{target, &sm.bc[9]}, [&](float y, int) -> bool { return sr_f2u(y) == mn; });
+                __syncthreads();
+                if (sm.bc[9] == 0xffffffffu) return kNucleusGeneralNoSlabs;  // (the counts of the two reads differ: not possible)
+                ycut = mn;
+                idx_last = (int)sm.bc[9];
+                cut_in_run = true;
+                cut_here = true;
+                break;
+            }
+            if (cut_here) { nc = 0; break; }
+            const uint32_t mn = below;  // the position's smallest value: what is left of the row lies below it
+            // the whole run lies inside the nucleus: on to the position behind it
+            {
+                int c = c0;
+#pragma unroll
+                for (int j = 0; j < kPer; j++) {
+                    c += (int)mine[j];
+                    if (tid * kPer + j == d_prev) sm.bc[8] = (uint32_t)c;
+                }
+            }
+            __syncthreads();
+            taken = (int)sm.bc[8];
+            hi_y = sr_u2f(mn - 1u);  // what is left lies below the run's value
+            d_prev = d_prev + 1;
+            __syncthreads();
+            if (d_prev >= kHistPos) { all_in = true; nc = 0; break; }
+            slab--;  // (a run is not one of the slabs that the limit counts; the for's increment puts it back)
+            was_capped = true;
+            continue;
+        }
         {
             int c = c0;
 #pragma unroll
@@ -1320,7 +1433,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         all_in = d_end >= kHistPos;
         const float c_e = all_in ? 0.0f : sr_u2f(((kHistTopKey - (uint32_t)d_end) << 16) | 0xffffu);
         const float c_y = do_scale ? __fmul_rn(c_e, inv) : c_e;  // taken: y > c_y, which e > c_e follows from
-        const bool capped = slab > 0;
+        const bool capped = slab > 0 || was_capped;
 
         // the slab's entries: every wave lists those of its stretch of the row in a pool in LDS, each with its number
         // within the wave, from which its place in index order follows once all waves' counts are known
@@ -1433,9 +1546,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         if (r * kT + tid < nc) sm.sortbuf[lpos[r]] = ((unsigned long long)(0xffffffffu - (uint32_t)pi[r]) << 32) | (unsigned long long)pv[r];
     __syncthreads();
     // Members: everything above the value at the cut, and of the entries equal to it the first ones by index.
-    uint32_t ycut = 0u;
-    int idx_last = -1;  // the last member among the entries equal to the cut value
-    if (found >= 0) {
+    if (found >= 0 && !cut_in_run) {
         ycut = sval[found];
         int gt = 0;
         for (int e = tid; e < nc; e += kT) gt += sval[e] > ycut ? 1 : 0;
@@ -1464,7 +1575,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         __syncthreads();
         idx_last = (int)sm.bc[9];
     }
-    if (slab == 0) {
+    if (slab == 0 && runs == 0) {
         finish_from_ordered_list(a, const_cast<float*>(p), n, nc, row, sm);
         return kNucleusDone;
     }
@@ -1472,7 +1583,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     // the row, again in index order in the waves' stretches of the sort segment, and the final Normalize and the draw
     // take them from there a block at a time.
     const float ycut_f = sr_u2f(ycut);
-    if (slab >= kNucleusRowFinish) {
+    if (slab >= kNucleusRowFinish || runs > 0) {
         // A nucleus of many thousands of members: listing them and passing over the list, 5 us per thousand, costs more
         // than writing the row -- scaled, everything outside the nucleus zero -- and the two passes over it of the
         // final Normalize and the pass of the draw (about 70 us for 151,936 entries).

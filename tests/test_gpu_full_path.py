@@ -466,6 +466,33 @@ def test_final_normalize_of_long_rows_at_ragged_lengths(ctx):
         _check_rows(ctx, logits, params, rng.random(4))
 
 
+def test_top_p_over_thousands_of_equal_logits(ctx):
+    # Logits on a grid (as bf16 gives them) put thousands of entries on one probability.  The walk through the nucleus
+    # takes such a value as a run of equal terms -- no order among them is needed for the running sum -- and if the cut
+    # falls inside the run, the members are its first entries by index.  Rows: a coarse grid (one value per crowded
+    # position of the histogram), a cluster of three values so close that they share a position, bf16-rounded logits
+    # at a high temperature; uniforms at both ends, and the same under allow-masks.
+    rng = np.random.default_rng(2024)
+    V = synthetic.QWEN_VOCAB
+    grid = np.round(rng.normal(0, 1.0, V) * 8) / 8
+    cluster = rng.normal(0, 2.0, V)
+    pick = rng.random(V) < 0.6
+    cluster[pick] = rng.choice(np.array([1.0, 1.002, 1.004]), size=int(pick.sum()))
+    bf = synthetic.bf16_bits_to_f32(synthetic.to_bf16_bits(rng.normal(0, 1.5, (1, V)).astype(np.float32)))[0]
+    logits = np.stack([grid, cluster, cluster, bf, grid]).astype(np.float32)
+    params = [SamplingParams(Temperature=1.0, TopP=0.9), SamplingParams(Temperature=1.0, TopP=0.6),
+              SamplingParams(Temperature=0.8, TopP=0.95), SamplingParams(Temperature=1.3, TopP=0.9),
+              SamplingParams(Temperature=2.0, TopP=0.5)]
+    rows = len(params)
+    for u in ([0.99999994] * rows, [0.0] * rows, rng.random(rows).tolist(), rng.random(rows).tolist()):
+        _check_rows(ctx, logits, params, u)
+    allowed = rng.random((rows, V)) < np.array([0.5, 0.9, 0.3, 0.8, 0.7])[:, None]
+    mask = pack_allow_mask(allowed)
+    active = np.ones(rows, dtype=np.uint8)
+    for u in ([0.99999994] * rows, rng.random(rows).tolist()):
+        _check_rows(ctx, logits, params, u, mask, active)
+
+
 def _strided(a, pad, dtype=None):
     """The rows of `a` inside a wider device tensor: row stride = a.shape[1] + pad elements."""
     import torch
