@@ -1326,7 +1326,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         }
         __syncthreads();
         // about how many entries the nucleus holds: a row that would need more slabs than are walked goes the general
-        // way at once (its survivors are sorted device-wide)
+        // way at once (its survivors are sorted where they lie)
         if (slab == 0 && runs == 0 && (int)sm.bc[11] - min((int)sm.bc[11], crowded_total) > (kMaxSlabs - 2) * kSmall)
             return kNucleusGeneralNoSlabs;
         const int d_cnt = (int)sm.bc[6], d_mass = (int)sm.bc[7];
@@ -1707,9 +1707,8 @@ __device__ __forceinline__ void sort_survivors_in_place(uint32_t* keys, int32_t*
 }
 
 // ---- stage 3: softmax, top-k, min-p, top-p on the work row --------------------------------------------
-// phase 1 ends after top-p for rows whose nucleus candidates fit the kernel (<= kSmall survivors), or
-// after compacting the survivors for the device-wide sort otherwise; phase 2 finishes those rows and
-// then normalises, draws and writes results for every row.
+// One workgroup per row, one launch: the row is cut, normalised and drawn from here.  A nucleus that the walk by
+// slabs cannot close has its survivors compacted into the row's sort segment and sorted there by this workgroup.
 __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
 {
     __shared__ FullSmem sm;
@@ -1925,8 +1924,6 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             int cnt = survivors;
             if (!fused) row_pass<false>(p, n, [&](float x, int) -> float { cnt += x > 0.0f ? 1 : 0; return x; });
             int ns;
-            // positions in index order (stable input for the device-wide sort)
-            // each thread owns the strided indices tid, tid + kT, ...; a second pass assigns slots per tile
             ns = blk_sum_i(cnt, sm);
             const bool have_list = ns_listed >= 0;  // (then ns == ns_listed <= kSmall)
             // The nucleus is walked in descending order, a slab of at most kSmall probabilities at a time: the slab
@@ -1934,7 +1931,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             // sorted here and the exact running sum goes on through it from where the slab before ended.  Most
             // nuclei close in the first slab; a masked row without min-p (tens of thousands of survivors) takes a
             // few.  Only a row that makes no progress (more than kSmall probabilities inside one bucket) or needs
-            // more than kMaxSlabs slabs has its survivors sorted device-wide.
+            // more than kMaxSlabs slabs has all its survivors sorted (sort_survivors_in_place).
             constexpr int kMaxSlabs = 24;
             // A row that needs several slabs has all their bounds from one histogram of its probabilities' 16-bit keys
             // instead of two select passes per slab.  The histogram is counted in LDS (the slabs' sort buffer, free
@@ -2053,7 +2050,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                     __syncthreads();
                 }
                 FPROF_ADD(a, slot, 12, t_step);
-                if (nc <= 0 || nc > kSmall) break;  // no progress: the device-wide sort takes the row
+                if (nc <= 0 || nc > kSmall) break;  // no progress: the row's survivors are sorted as a whole
                 int P = 2;
                 while (P < nc) P <<= 1;
                 for (int i = nc + tid; i < P; i += kT) sm.sortbuf[i] = 0ull;
