@@ -70,7 +70,14 @@ enum {
     SR_OUT_PATH_TOPK_FAST = 1u << 1,   /* SampleTopK (Sampler.cs:216-357)                       */
     SR_OUT_PATH_FULL_VOCAB = 1u << 2,  /* slow path (Sampler.cs:41-95)                          */
     SR_OUT_DEGENERATE = 1u << 3,       /* all -inf row: greedy / uniform fallback was taken     */
-    SR_OUT_ROW_UNSUPPORTED = 1u << 31  /* thousands of equal logits at the top-k cut: token is -1 */
+    SR_OUT_AMBIGUOUS = 1u << 4,        /* the token depends on a convention the managed runtime leaves open: a cut or the
+                                          draw fell within a few ulp of a boundary of the running sum, or a top-p cut
+                                          split a run of equal probabilities (Sampler.cs:533 unstable sort, :555 lane
+                                          order of TensorPrimitives.Sum).  The token is still the one the documented
+                                          conventions give; a caller that wants certainty re-runs the row on the CPU  */
+    SR_OUT_ROW_UNSUPPORTED = 1u << 31  /* an internal limit of the selection kernel was met although sr_batch_upload
+                                          routes every row by those limits: token is -1.  No input is known to set it;
+                                          sr_sample_batch finishes such a row with sr_resample_rows_launch            */
 };
 
 /*
@@ -177,22 +184,24 @@ SR_API int sr_batch_set_uniforms(sr_batch* batch, const double* uniforms);
  * uint32[rows] (out_flags may be NULL).  One uniform per row is consumed by non-greedy rows.
  * This is the batched sibling of IBatchedForwardPass.BatchForwardMultiArgmax
  * (src/OpenTail.Stingray.Engine/IBatchedForwardPass.cs:105-117) for rows that are not greedy.
+ * The call keeps host-side state per launch (which of two sets of hand-over counters the launch uses): it must not be
+ * recorded into a HIP graph and replayed; sr_argmax_rows_launch_noalloc is the entry point made for that.
  */
 SR_API int sr_sample_launch(sr_ctx* ctx, const sr_batch* batch, const void* logits_dev, int dtype,
                             int64_t row_stride_elems, int32_t* out_tokens_dev, uint32_t* out_flags_dev);
 
-/* Same, with the side inputs given directly and results in HOST buffers.  logits may be a device
- * (logits_on_device != 0) or a host tensor.  out_flags may be NULL. */
 /*
- * SampleTopK (Sampler.cs:216-357) once more, by device-wide sorts of the whole row, for rows of a batch that
- * sr_sample_launch reported with SR_OUT_ROW_UNSUPPORTED (any SampleTopK row may be given).  rows_host: HOST int32
- * row indices into the batch; the same logits, outputs and uniforms as the launch before.  No counterpart in the
- * reference, which has no row limit; sr_sample_batch calls it by itself.
+ * SampleTopK (Sampler.cs:216-357) once more, by device-wide sorts of the whole row, for the SampleTopK rows of a batch
+ * named in rows_host (HOST int32 row indices into the batch); the same logits, outputs and uniforms as the launch
+ * before.  The finisher for rows flagged SR_OUT_ROW_UNSUPPORTED, and an independent second way to the same answer
+ * for any SampleTopK row.  No counterpart in the reference, which has no row limit.
  */
 SR_API int sr_resample_rows_launch(sr_ctx* ctx, const sr_batch* batch, const void* logits_dev, int dtype,
                                    int64_t row_stride_elems, const int32_t* rows_host, int32_t n_rows,
                                    int32_t* out_tokens_dev, uint32_t* out_flags_dev);
 
+/* sr_sample_launch with the side inputs given directly and results in HOST buffers.  logits may be a device
+ * (logits_on_device != 0) or a host tensor.  out_flags may be NULL. */
 SR_API int sr_sample_batch(sr_ctx* ctx, const void* logits, int dtype, int logits_on_device,
                            int32_t rows, int32_t vocab, int64_t row_stride_elems,
                            const sr_row_params* params,
@@ -269,7 +278,8 @@ SR_API int sr_sample_with_distribution(sr_ctx* ctx, const float* logits, int32_t
 /*
  * int Sampler.SampleFromProbs(ReadOnlySpan<float> probs, Random rng) per row (Sampler.cs:195-199):
  * first index whose running fp32 sum reaches (float)u, last index as the rounding fallback.
- * uniforms: HOST double[rows] (NULL -> SR_ERR_NULL_ARGUMENT, the ArgumentNullException of :197).
+ * uniforms: HOST double[rows] (NULL -> SR_ERR_NULL_ARGUMENT, the ArgumentNullException of :197); they are copied
+ * into pinned memory of the context, so the array may be reused at once and the call does not wait for the device.
  */
 SR_API int sr_sample_from_probs_launch(sr_ctx* ctx, const float* probs_dev, int32_t rows, int32_t vocab,
                                        int64_t probs_stride_elems, const double* uniforms,
@@ -340,10 +350,21 @@ SR_API int sr_pack_allow_mask_launch(sr_ctx* ctx, const void* masked_logits_dev,
  * sr_pack_allow_mask_launch wrote) into device memory once and returns its id; batches then name masks by id
  * (sr_batch_upload_mask_ids, sr_batch_append_tokens_masks) and a constrained decode step uploads 4 bytes per row
  * instead of 19 KB.  A context holds masks of one vocabulary size at a time.  sr_mask_release frees an id for
- * reuse; the caller must not release a mask that an uploaded batch still names.
+ * reuse.  A batch that still names a released id (or an id of a pool that was started again for another vocabulary) is
+ * stale: every launch with it returns SR_ERR_INVALID_ARGUMENT until it is uploaded again or the row is given a
+ * registered id by sr_batch_append_tokens_masks.
  */
 SR_API int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, int32_t vocab, int32_t* out_id);
 SR_API int sr_mask_release(sr_ctx* ctx, int32_t mask_id);
+/*
+ * AndTokenConstraint.Filter (src/OpenTail.Stingray.Core/Grammar/AndTokenConstraint.cs:44-86) over registered masks: the
+ * intersection of mask_ids[0..n) is written into a NEW registered mask whose id is returned in *out_id (released like any
+ * other).  An entry of -1 (an inner constraint in its dead state, :74) is skipped.  *out_id is -1 -- "no mask", the row
+ * goes unmasked -- when nothing is left to intersect, and when the intersection allows no token of the vocabulary (the
+ * dead-intersection rule, :80-85).  At most 8 ids per call.  The call waits for the 4-byte answer "any token left";
+ * a constraint pair meets the same pair of states again and again, so callers keep the result per tuple of ids.
+ */
+SR_API int sr_mask_and(sr_ctx* ctx, const int32_t* mask_ids, int32_t n, int32_t* out_id);
 /* sr_batch_upload with the allow-mask of every row named by id: mask_ids [rows], -1 = the row is not constrained
  * (ITokenConstraint.Filter returned its input, ITokenConstraint.cs:36-41).  No copy is waited for. */
 SR_API int sr_batch_upload_mask_ids(sr_batch* batch, int32_t rows, int32_t vocab,

@@ -43,6 +43,7 @@ SR_OUT_PATH_GREEDY = 1
 SR_OUT_PATH_TOPK_FAST = 2
 SR_OUT_PATH_FULL_VOCAB = 4
 SR_OUT_DEGENERATE = 8
+SR_OUT_AMBIGUOUS = 16
 SR_OUT_ROW_UNSUPPORTED = 1 << 31
 
 # every symbol include/stingray_sampler.h declares
@@ -50,7 +51,7 @@ EXPORTED_SYMBOLS = [
     "sr_create", "sr_destroy", "sr_bind_thread", "sr_set_stream", "sr_use_own_stream", "sr_synchronize", "sr_last_error",
     "sr_version", "sr_batch_create", "sr_batch_destroy", "sr_batch_upload", "sr_batch_set_uniforms",
     "sr_batch_append_tokens", "sr_batch_append_tokens_masks", "sr_batch_upload_mask_ids", "sr_mask_register",
-    "sr_mask_release", "sr_pack_allow_mask_launch",
+    "sr_mask_release", "sr_mask_and", "sr_pack_allow_mask_launch",
     "sr_sample_launch", "sr_resample_rows_launch", "sr_sample_batch", "sr_argmax_rows_launch", "sr_argmax_rows_launch_noalloc",
     "sr_argmax_rows",
     "sr_build_distribution_launch", "sr_sample_with_distribution_launch", "sr_sample_from_probs_launch",
@@ -162,6 +163,7 @@ def load_library():
     L.sr_batch_upload_mask_ids.argtypes = [vp, i32, i32, rpp, i32p, i32p, i32p, f32p, i32p, i32p, f64p, i32]
     L.sr_mask_register.argtypes = [vp, vp, C.c_int, i32, i32p]
     L.sr_mask_release.argtypes = [vp, i32]
+    L.sr_mask_and.argtypes = [vp, i32p, i32, i32p]
     L.sr_pack_allow_mask_launch.argtypes = [vp, vp, C.c_int, i32, i32, i64, vp, i64]
     L.sr_sample_launch.argtypes = [vp, vp, vp, C.c_int, i64, vp, vp]
     L.sr_resample_rows_launch.argtypes = [vp, vp, vp, C.c_int, i64, i32p, i32, vp, vp]
@@ -363,6 +365,14 @@ class SamplerContext:
         else:
             assert words.is_cuda and words.numel() >= (vocab + 31) // 32
             self._check(self.L.sr_mask_register(self.h, C.c_void_p(words.data_ptr()), 1, vocab, C.byref(out)))
+        return int(out.value)
+
+    def mask_and(self, mask_ids) -> int:
+        """sr_mask_and: the registered intersection of the given masks (-1 entries skipped), or -1 when nothing is
+        left to intersect or the intersection allows no token (the row then goes unmasked)."""
+        ids = np.ascontiguousarray(np.asarray(mask_ids, dtype=np.int32))
+        out = C.c_int32(-1)
+        self._check(self.L.sr_mask_and(self.h, _ptr(ids, C.c_int32), int(ids.size), C.byref(out)))
         return int(out.value)
 
     def release_mask(self, mask_id: int) -> None:

@@ -69,6 +69,7 @@ def build_cpp_test(oracle_lib: str) -> str:
     root = os.path.normpath(os.path.join(HERE, "..", ".."))
     cmd = ["g++", "-std=c++17", "-O1", "-o", os.path.normpath(CPP_TEST_BIN), os.path.normpath(CPP_TEST_SRC),
            "-I" + os.path.join(root, "include"), "-I" + os.path.join(root, "oracle"),
+           "-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__", "-L/opt/rocm/lib", "-lamdhip64",
            "-L" + LIB_DIR, "-lstingray_sampler", "-L" + os.path.dirname(os.path.abspath(oracle_lib)), "-lstingray_oracle",
            "-Wl,-rpath,$ORIGIN/../../opentail/stingray_amd/lib", "-Wl,-rpath,$ORIGIN/../../oracle/_build",
            "-Wl,-rpath,/opt/rocm/lib"]

@@ -14,6 +14,22 @@
 const uint32_t* sr_batch_mask_ptr(const sr_batch* b) { return b->mask_ids ? b->ctx->mask_pool.as<uint32_t>() : b->d_mask.as<uint32_t>(); }
 int64_t sr_batch_mask_stride(const sr_batch* b) { return b->mask_ids ? (int64_t)b->ctx->pool_words : b->mask_stride; }
 
+int sr_batch_masks_valid(sr_ctx* ctx, const sr_batch* b, const char* who)
+{
+    if (!b->mask_ids) return SR_OK;
+    bool stale = b->mask_pool_gen != ctx->pool_gen || ctx->pool_vocab != b->vocab || b->keep_mask_ids.size() != (size_t)b->rows;
+    for (int32_t r = 0; r < b->rows && !stale; r++) {
+        const int32_t id = b->keep_mask_ids[(size_t)r];
+        if (id < 0) continue;
+        stale = id >= ctx->pool_cap || !ctx->pool_used[(size_t)id] || ctx->pool_slot_gen[(size_t)id] != b->keep_mask_gen[(size_t)r];
+    }
+    if (stale)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": the batch names a registered mask that was released, or whose "
+                                                         "pool was started again for another vocabulary, after the batch took its id; "
+                                                         "upload the batch again");
+    return SR_OK;
+}
+
 namespace {
 
 inline bool has_history_penalty(const sr_row_params& p)
@@ -294,11 +310,12 @@ void sr_destroy(sr_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
-    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best, &ctx->argmax_done, &ctx->mask_pool,
+    DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best, &ctx->argmax_done, &ctx->mask_pool, &ctx->mask_any,
                          &ctx->work, &ctx->edit_tab, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
-                         &ctx->uniforms_tmp, &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
+                         &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs, &ctx->spec_resid, &ctx->spec_reject};
     for (DeviceBuf* b : bufs) b->release();
+    ctx->uni_ring.release();
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
     delete ctx;
 }
@@ -415,6 +432,11 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
     b->mask_stride = allow_mask ? mask_stride_words : 0;
     b->mask_ids = mask_ids != nullptr;
     if (mask_ids) b->keep_mask_ids.assign(mask_ids, mask_ids + rows); else b->keep_mask_ids.clear();
+    b->keep_mask_gen.assign(mask_ids ? (size_t)rows : 0, 0u);
+    b->mask_pool_gen = ctx->pool_gen;
+    if (mask_ids)
+        for (int32_t r = 0; r < rows; r++)
+            if (mask_ids[r] >= 0) b->keep_mask_gen[(size_t)r] = ctx->pool_slot_gen[(size_t)mask_ids[r]];
     b->max_sel = 0;
     b->edit_cap.assign((size_t)rows, 0);
     b->sel_cap.assign((size_t)rows, 0);
@@ -689,6 +711,9 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     const int32_t rows = b->rows, vocab = b->vocab;
     if (rows == 0) return SR_OK;
     std::vector<int32_t> scan_again;  // scan-mask rows whose allow-mask changes
+    if (new_mask_ids && b->mask_pool_gen != ctx->pool_gen)
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_append_tokens_masks: the registered masks were started again for another "
+                                                         "vocabulary since the batch was uploaded; upload the batch again");
     if (new_mask_ids) {
         for (int32_t r = 0; r < rows; r++) {
             const int32_t id = new_mask_ids[r];
@@ -737,9 +762,12 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     for (int32_t r = 0; r < rows && !rebuild; r++) {
         SrRow& d = b->h_rows[(size_t)r];
         bool mask_changed = false;
-        if (new_mask_ids && new_mask_ids[r] != d.mask_row) {
+        // (an id that was released and registered again since the row took it names another mask now)
+        const uint32_t slot_gen = (new_mask_ids && new_mask_ids[r] >= 0) ? ctx->pool_slot_gen[(size_t)new_mask_ids[r]] : 0u;
+        if (new_mask_ids && (new_mask_ids[r] != d.mask_row || slot_gen != b->keep_mask_gen[(size_t)r])) {
             d.mask_row = new_mask_ids[r];
             b->keep_mask_ids[(size_t)r] = new_mask_ids[r];
+            b->keep_mask_gen[(size_t)r] = slot_gen;
             mask_changed = true;
             if (d.scan_row >= 0 && (b->h_scan_need[(size_t)r] & SR_SCAN_ALLOW)) scan_again.push_back(d.scan_row);
         }
@@ -888,17 +916,14 @@ int sr_batch_upload_mask_ids(sr_batch* b, int32_t rows, int32_t vocab, const sr_
 }
 
 // ---- registered allow-masks ---------------------------------------------------------------------------
-int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, int32_t vocab, int32_t* out_id)
+// A free slot of the pool of registered masks for vocabulary `vocab` (the pool starts again for a new vocabulary
+// when no mask is held, and grows when it is full).  The slot is not marked used yet.
+static int pool_take_slot(sr_ctx* ctx, int32_t vocab, const char* who, int32_t* out_slot)
 {
-    if (!ctx) return SR_ERR_NULL_ARGUMENT;
-    if (!words || !out_id) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_mask_register: null argument");
-    if (vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_register: empty vocabulary");
-    *out_id = -1;
-    SR_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
     const bool any_used = std::find(ctx->pool_used.begin(), ctx->pool_used.end(), (uint8_t)1) != ctx->pool_used.end();
     if (any_used && vocab != ctx->pool_vocab)
-        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_register: a context holds masks of one vocabulary size at a time (" +
+        return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": a context holds masks of one vocabulary size at a time (" +
                                                          std::to_string(ctx->pool_vocab) + " now); release them first");
     const int32_t nw = (vocab + 31) / 32;
     if (!any_used && vocab != ctx->pool_vocab) {  // a new vocabulary: the pool starts again
@@ -906,8 +931,10 @@ int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, in
         ctx->mask_pool.release();
         ctx->pool_cap = 0;
         ctx->pool_used.clear();
+        ctx->pool_slot_gen.clear();
         ctx->pool_vocab = vocab;
         ctx->pool_words = (nw + 3) & ~3;  // rows of the pool start on 16 bytes
+        ctx->pool_gen++;                  // batches that name masks of the old pool are stale from here on
     }
     int32_t id = -1;
     for (int32_t i = 0; i < ctx->pool_cap; i++)
@@ -920,7 +947,7 @@ int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, in
             hipError_t e = hipMemcpyAsync(bigger, ctx->mask_pool.p, (size_t)ctx->pool_cap * (size_t)ctx->pool_words * sizeof(uint32_t),
                                           hipMemcpyDeviceToDevice, st);
             if (e == hipSuccess) e = hipStreamSynchronize(st);
-            if (e != hipSuccess) { (void)hipFree(bigger); return sr_fail_hip(ctx, e, "sr_mask_register: moving the masks"); }
+            if (e != hipSuccess) { (void)hipFree(bigger); return sr_fail_hip(ctx, e, "moving the registered masks"); }
         }
         ctx->mask_pool.release();
         ctx->mask_pool.p = bigger;
@@ -928,7 +955,24 @@ int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, in
         id = ctx->pool_cap;
         ctx->pool_cap = cap;
         ctx->pool_used.resize((size_t)cap, 0);
+        ctx->pool_slot_gen.resize((size_t)cap, 0u);
     }
+    *out_slot = id;
+    return SR_OK;
+}
+
+int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, int32_t vocab, int32_t* out_id)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (!words || !out_id) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_mask_register: null argument");
+    if (vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_register: empty vocabulary");
+    *out_id = -1;
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    int32_t id = -1;
+    int rc = pool_take_slot(ctx, vocab, "sr_mask_register", &id);
+    if (rc != SR_OK) return rc;
+    const int32_t nw = (vocab + 31) / 32;
     uint32_t* dst = ctx->mask_pool.as<uint32_t>() + (size_t)id * (size_t)ctx->pool_words;
     SR_HIP(ctx, hipMemcpyAsync(dst, words, (size_t)nw * sizeof(uint32_t),
                                words_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, st));
@@ -939,12 +983,49 @@ int sr_mask_register(sr_ctx* ctx, const uint32_t* words, int words_on_device, in
     return SR_OK;
 }
 
+int sr_mask_and(sr_ctx* ctx, const int32_t* mask_ids, int32_t n, int32_t* out_id)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (!out_id || (!mask_ids && n > 0)) return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_mask_and: null argument");
+    *out_id = -1;
+    if (n < 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_and: negative count");
+    int32_t ids[SR_MASK_AND_MAX];
+    int32_t m = 0;
+    for (int32_t i = 0; i < n; i++) {
+        const int32_t id = mask_ids[i];
+        if (id == -1) continue;  // an inner constraint in its dead state contributes nothing (AndTokenConstraint.cs:74)
+        if (id < -1 || id >= ctx->pool_cap || !ctx->pool_used[(size_t)id])
+            return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_and: mask " + std::to_string(id) + " is not registered");
+        if (m == SR_MASK_AND_MAX)
+            return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_mask_and: at most " + std::to_string(SR_MASK_AND_MAX) + " masks per call (combine in steps)");
+        ids[m++] = id;
+    }
+    if (m == 0) return SR_OK;  // nothing constrains: no mask
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    int32_t slot = -1;
+    int rc = pool_take_slot(ctx, ctx->pool_vocab, "sr_mask_and", &slot);
+    if (rc != SR_OK) return rc;
+    SR_HIP(ctx, ctx->mask_any.reserve(sizeof(uint32_t), st));
+    SR_HIP(ctx, hipMemsetAsync(ctx->mask_any.p, 0, sizeof(uint32_t), st));
+    SR_HIP(ctx, sr_launch_mask_and(ctx->mask_pool.as<uint32_t>(), ctx->pool_words, ids, m, slot, ctx->pool_vocab,
+                                   ctx->mask_any.as<uint32_t>(), st));
+    uint32_t any = 0u;
+    SR_HIP(ctx, hipMemcpyAsync(&any, ctx->mask_any.p, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    SR_HIP(ctx, hipStreamSynchronize(st));
+    if (!any) return SR_OK;  // dead intersection: never wedge, the row goes unmasked (AndTokenConstraint.cs:80-85); the slot stays free
+    ctx->pool_used[(size_t)slot] = 1;
+    *out_id = slot;
+    return SR_OK;
+}
+
 int sr_mask_release(sr_ctx* ctx, int32_t id)
 {
     if (!ctx) return SR_ERR_NULL_ARGUMENT;
     if (id < 0 || id >= ctx->pool_cap || !ctx->pool_used[(size_t)id])
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_mask_release: mask " + std::to_string(id) + " is not registered");
     ctx->pool_used[(size_t)id] = 0;
+    ctx->pool_slot_gen[(size_t)id]++;  // a batch that still names the id is stale from here on
     return SR_OK;
 }
 
@@ -987,6 +1068,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_launch: unknown dtype");
     if (row_stride_elems < b->vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_launch: row stride < vocab");
     if (b->vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_sample_launch: empty vocabulary");
+    if (int rc = sr_batch_masks_valid(ctx, b, "sr_sample_launch")) return rc;
     for (const SrRow& r : b->h_rows)
         if (r.path != SR_PATH_GREEDY && r.path != SR_PATH_GREEDY_PEN && b->upr < 1)
             return sr_fail(ctx, SR_ERR_NULL_ARGUMENT, "sr_sample_launch: a sampled row needs a uniform");

@@ -93,7 +93,7 @@ int check_batch_call(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
     if (dtype != SR_DTYPE_F32 && dtype != SR_DTYPE_BF16) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": unknown dtype");
     if (b->vocab <= 0) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": empty vocabulary");
     if (row_stride < b->vocab) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": row stride < vocab");
-    return SR_OK;
+    return sr_batch_masks_valid(ctx, b, who);
 }
 
 // identity row list [0, rows) on the device
@@ -111,12 +111,15 @@ int identity_list(sr_ctx* ctx, int rows, const int32_t** out)
     return SR_OK;
 }
 
+// The caller's uniforms for a kernel enqueued on the context's stream: copied into pinned memory of the context, which
+// the kernel reads in place, so the call neither waits nor depends on the caller's array afterwards.
 int upload_uniforms(sr_ctx* ctx, const double* uniforms, int rows, const double** dev)
 {
-    SR_HIP(ctx, ctx->uniforms_tmp.reserve((size_t)rows * sizeof(double), ctx->stream));
-    SR_HIP(ctx, hipMemcpyAsync(ctx->uniforms_tmp.p, uniforms, (size_t)rows * sizeof(double), hipMemcpyHostToDevice, ctx->stream));
-    SR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the host array may go away
-    *dev = ctx->uniforms_tmp.as<double>();
+    const size_t bytes = (size_t)rows * sizeof(double);
+    SR_HIP(ctx, ctx->uni_ring.begin(bytes + 256, ctx->stream));
+    const void* at = ctx->uni_ring.put(uniforms, bytes);
+    if (!at) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "no pinned memory for the uniforms");
+    *dev = (const double*)at;
     return SR_OK;
 }
 

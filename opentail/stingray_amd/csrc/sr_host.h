@@ -190,7 +190,8 @@ struct sr_ctx {
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
     DeviceBuf host_logits;   // staging for host-resident logits
     DeviceBuf stage_probs;   // staging for host-resident distributions
-    DeviceBuf out_tokens, out_flags, out_val, uniforms_tmp;
+    DeviceBuf out_tokens, out_flags, out_val;
+    HostRing uni_ring;       // uniforms of the calls that take them as host arrays and enqueue a kernel (read in place)
     DeviceBuf seg, sort_k0, sort_k1, sort_v0, sort_v1, sort_tmp;  // device-wide sort of large nuclei
     DeviceBuf ident;         // identity row list
     DeviceBuf redo_list;     // rows given to sr_resample_rows_launch
@@ -205,6 +206,11 @@ struct sr_ctx {
     DeviceBuf mask_pool;
     int32_t pool_vocab = 0, pool_words = 0, pool_cap = 0;
     std::vector<uint8_t> pool_used;
+    // pool_gen counts the times the pool started again (another vocabulary), pool_slot_gen[id] the releases of a slot:
+    // a batch remembers both for the ids it names, and a launch refuses a batch whose ids have changed hands since
+    unsigned pool_gen = 0;
+    std::vector<uint32_t> pool_slot_gen;
+    DeviceBuf mask_any;      // sr_mask_and: "a bit is left" word
     // selection kernel: entries per set of counters, launches so far (its parity picks the set), and how often a row
     // tail polls its row's counter before it stops waiting and selects from the logits alone
     size_t done_cap = 0;
@@ -234,6 +240,8 @@ struct sr_batch {
     bool has_mask = false;
     bool mask_ids = false;               // the rows' allow-masks are registered masks of the context (mask_row = id)
     std::vector<int32_t> keep_mask_ids;  // ... per row, -1 none
+    std::vector<uint32_t> keep_mask_gen; // ... the release count of the row's slot when the row took the id
+    unsigned mask_pool_gen = 0;          // ... the pool's generation at that time
     int32_t max_sel = 0;
     HostStage stage;
     HostRing patch_ring;  // the lists of sr_batch_append_tokens          // pinned copies of what an upload sends to the device
@@ -275,6 +283,9 @@ inline int sr_fail_hip(sr_ctx* ctx, hipError_t e, const char* what)
         if (_e != hipSuccess) return sr_fail_hip((ctx), _e, #call);   \
     } while (0)
 
+// SR_OK, or SR_ERR_INVALID_ARGUMENT when the batch names a registered mask that was released (or whose pool was
+// started again for another vocabulary) after the batch took the id: to be called before every launch that reads masks
+int sr_batch_masks_valid(sr_ctx* ctx, const sr_batch* b, const char* who);
 // where a batch's allow-masks lie: its own upload, or the context's registered masks (sr_api.cpp)
 const uint32_t* sr_batch_mask_ptr(const sr_batch* b);
 int64_t sr_batch_mask_stride(const sr_batch* b);

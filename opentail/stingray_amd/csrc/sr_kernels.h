@@ -81,6 +81,11 @@ hipError_t sr_launch_scatter(const SrCopySeg* segs, int n, hipStream_t stream);
 // scan_ids: the n_scan scan rows to build (NULL: rows 0 .. n_scan - 1)
 hipError_t sr_launch_pack_allow_mask(const void* logits, int dtype, int rows, int vocab, int64_t row_stride, uint32_t* out,
                                      int64_t out_stride, hipStream_t stream);
+// AND of the n (<= SR_MASK_AND_MAX) registered masks ids_host[] into slot dst of the pool; *any (zero before) becomes 1
+// when a bit inside the vocabulary is left
+#define SR_MASK_AND_MAX 8
+hipError_t sr_launch_mask_and(uint32_t* pool, int64_t pool_words, const int32_t* ids_host, int n, int dst, int vocab, uint32_t* any,
+                              hipStream_t stream);
 hipError_t sr_launch_build_scan_mask(const SrScanDesc* descs, const int32_t* scan_ids, int n_scan, const SrRow* rows, const SrEdit* edits,
                                      const uint32_t* mask, int64_t mask_stride, uint32_t* scan_mask, int64_t scan_stride,
                                      int vocab, int epv, int chunks, int chunk_vecs, unsigned long long base_addr,

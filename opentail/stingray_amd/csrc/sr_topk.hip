@@ -2160,6 +2160,27 @@ __global__ __launch_bounds__(256) void k_pack_allow_mask(const void* logits, int
             out[(size_t)row * out_stride + g * 2 + lane] = (uint32_t)(bal >> (32 * lane));
     }
 }
+
+// AND of n registered masks (slots ids[0..n) of the pool) into slot `dst`; *any is set when a bit of the vocabulary
+// is left.  ids lie in the kernel's arguments (few constraints are ever combined).
+struct SrMaskAndIds { int32_t id[SR_MASK_AND_MAX]; };
+__global__ __launch_bounds__(256) void k_mask_and(uint32_t* pool, int64_t pool_words, SrMaskAndIds ids, int n, int dst, int vocab,
+                                                  uint32_t* any)
+{
+    const int nw = (vocab + 31) / 32;
+    uint32_t seen = 0u;
+    for (int w = blockIdx.x * blockDim.x + threadIdx.x; w < (int)pool_words; w += gridDim.x * blockDim.x) {
+        uint32_t v = 0u;
+        if (w < nw) {
+            v = 0xffffffffu;
+            for (int k = 0; k < n; k++) v &= pool[(size_t)ids.id[k] * (size_t)pool_words + w];
+            if (w == nw - 1 && (vocab & 31)) v &= (1u << (vocab & 31)) - 1u;  // bits beyond the vocabulary never count
+        }
+        pool[(size_t)dst * (size_t)pool_words + w] = v;
+        seen |= v;
+    }
+    if (__ballot(seen != 0u) != 0ull && sr_lane() == 0) atomicOr(any, 1u);
+}
 }  // namespace
 
 hipError_t sr_launch_scatter(const SrCopySeg* segs, int n, hipStream_t stream)
@@ -2177,6 +2198,16 @@ hipError_t sr_launch_pack_allow_mask(const void* logits, int dtype, int rows, in
     const dim3 grid((unsigned)std::min((n64 + 3) / 4, 1024), (unsigned)rows), block(256);
     if (dtype == 1) hipLaunchKernelGGL(k_pack_allow_mask<2>, grid, block, 0, stream, logits, row_stride, vocab, out, out_stride);
     else hipLaunchKernelGGL(k_pack_allow_mask<4>, grid, block, 0, stream, logits, row_stride, vocab, out, out_stride);
+    return hipGetLastError();
+}
+
+hipError_t sr_launch_mask_and(uint32_t* pool, int64_t pool_words, const int32_t* ids_host, int n, int dst, int vocab, uint32_t* any,
+                              hipStream_t stream)
+{
+    SrMaskAndIds ids{};
+    for (int k = 0; k < n && k < SR_MASK_AND_MAX; k++) ids.id[k] = ids_host[k];
+    const int blocks = (int)std::min<int64_t>((pool_words + 255) / 256, 64);
+    hipLaunchKernelGGL(k_mask_and, dim3((unsigned)std::max(blocks, 1)), dim3(256), 0, stream, pool, pool_words, ids, n, dst, vocab, any);
     return hipGetLastError();
 }
 

@@ -31,6 +31,9 @@ public sealed unsafe class RocmBatchSampler : IDisposable
     private readonly nint _ctx;
     private nint _batch;
     private int _rows = -1, _vocab;
+    // the library's copy of the histories is what the engine's RecentTokens are: true after a step that went through
+    // Sample, false after any step that did not
+    private bool _historyValid;
 
     public static bool IsAvailable => StingraySamplerInterop.IsAvailable;
 
@@ -70,6 +73,20 @@ public sealed unsafe class RocmBatchSampler : IDisposable
         }
     }
 
+    /// <summary>AndTokenConstraint.Filter over registered masks (AndTokenConstraint.cs:44-86): the id of the intersection,
+    /// or -1 (no mask) when no id is left to intersect or no token survives.</summary>
+    public int MaskAnd(ReadOnlySpan<int> ids)
+    {
+        fixed (int* p = ids)
+        {
+            StingraySamplerInterop.Check(_ctx, StingraySamplerInterop.MaskAnd(_ctx, p, ids.Length, out int id), "sr_mask_and");
+            return id;
+        }
+    }
+
+    /// <summary>A decode step did not go through Sample: the next one uploads, whatever the caller says about its rows.</summary>
+    public void InvalidateHistory() => _historyValid = false;
+
     public void ReleaseMask(int id) =>
         StingraySamplerInterop.Check(_ctx, StingraySamplerInterop.MaskRelease(_ctx, id), "sr_mask_release");
 
@@ -82,9 +99,9 @@ public sealed unsafe class RocmBatchSampler : IDisposable
     /// (CudaForwardPass.cs:5229-5232).
     /// </summary>
     public void Sample(nint logitsDev, int dtype, int rows, int vocab, long rowStrideElems,
-                       nint tokensDev, in BatchedSamplingInputs inputs, bool sameRowsAsLastStep)
+                       nint tokensDev, nint flagsDev, in BatchedSamplingInputs inputs, bool sameRowsAsLastStep)
     {
-        if (sameRowsAsLastStep && rows == _rows && vocab == _vocab && inputs.PreviousTokens.Length == rows)
+        if (sameRowsAsLastStep && _historyValid && rows == _rows && vocab == _vocab && inputs.PreviousTokens.Length == rows)
         {
             fixed (int* t = inputs.PreviousTokens)
             fixed (double* u = inputs.Uniforms)
@@ -97,7 +114,8 @@ public sealed unsafe class RocmBatchSampler : IDisposable
             Upload(rows, vocab, inputs);
         }
         StingraySamplerInterop.Check(_ctx, StingraySamplerInterop.SampleLaunch(_ctx, _batch, logitsDev, dtype, rowStrideElems,
-                                                                             tokensDev, 0), "sr_sample_launch");
+                                                                             tokensDev, flagsDev), "sr_sample_launch");
+        _historyValid = true;
     }
 
     private void Upload(int rows, int vocab, in BatchedSamplingInputs inputs)

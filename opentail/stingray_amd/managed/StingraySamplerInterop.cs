@@ -19,6 +19,10 @@ internal static unsafe partial class StingraySamplerInterop
 {
     private const string Lib = "stingray_sampler";
 
+    // SR_OUT_* bits of the per-row flags
+    internal const uint OutPathGreedy = 1u << 0, OutPathTopKFast = 1u << 1, OutPathFullVocab = 1u << 2,
+                        OutDegenerate = 1u << 3, OutAmbiguous = 1u << 4;
+
     [LibraryImport(Lib, EntryPoint = "sr_create")]        internal static partial int Create(int deviceOrdinal, out nint ctx);
     [LibraryImport(Lib, EntryPoint = "sr_destroy")]       internal static partial void Destroy(nint ctx);
     [LibraryImport(Lib, EntryPoint = "sr_bind_thread")]   internal static partial int BindThread(nint ctx);
@@ -75,6 +79,8 @@ internal static unsafe partial class StingraySamplerInterop
     internal static partial int MaskRegister(nint ctx, uint* words, int wordsOnDevice, int vocab, out int maskId);
     [LibraryImport(Lib, EntryPoint = "sr_mask_release")]
     internal static partial int MaskRelease(nint ctx, int maskId);
+    [LibraryImport(Lib, EntryPoint = "sr_mask_and")]
+    internal static partial int MaskAnd(nint ctx, int* maskIds, int n, out int maskId);
     [LibraryImport(Lib, EntryPoint = "sr_pack_allow_mask_launch")]
     internal static partial int PackAllowMaskLaunch(nint ctx, nint maskedLogitsDev, int dtype, int rows, int vocab,
         long rowStrideElems, nint outWordsDev, long outStrideWords);

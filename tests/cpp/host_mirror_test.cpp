@@ -7,6 +7,8 @@
 #include <limits>
 #include <random>
 
+#include <hip/hip_runtime_api.h>
+
 #include "stingray_oracle.h"
 #include "stingray_sampler.hpp"
 
@@ -193,6 +195,139 @@ int main()
         CHECK(threw, "a sampled row without rng must throw ArgumentNullException");
     }
     std::printf("error behaviour done\n");
+
+    // The gate of the batcher loop (ContinuousBatchingEngine.cs:580-650) against the loop's own way (full logits on
+    // the host, the oracle sampling): a step that is skipped, a forced token in the middle, the draws per sequence.
+    {
+        const int rows = 3, n = 6007, steps = 16;
+        struct Seq {
+            SamplingParams Sp;
+            std::vector<int> hist;
+            std::vector<int>* RecentTokens = nullptr;
+            PeekableRandom* Rng = nullptr;
+            bool ForcedClose = false;
+            int MaskId = -1;
+            int Id = 0;
+        };
+        struct SeededRandom : Random {  // any generator will do: both engines replay the same values
+            std::mt19937_64 g;
+            std::uniform_real_distribution<double> d{0.0, 1.0};
+            explicit SeededRandom(unsigned s) : g(s) {}
+            double NextDouble() override { return d(g); }
+        };
+        struct Fwd {
+            BatchSampler* sampler;
+            const std::vector<float>* host_rows;
+            float* dev = nullptr;
+            int32_t* tok = nullptr;
+            uint32_t* flg = nullptr;
+            int rows, n, sample_calls = 0;
+            bool SupportsBatchedGpuSampling() { return true; }
+            void InvalidateSamplingState() { sampler->InvalidateHistory(); }
+            void BatchForwardMultiSample(const std::vector<int>&, const BatchedSamplingInputs& in, bool same, std::vector<int>& out,
+                                         std::vector<uint32_t>& flags)
+            {
+                sample_calls++;
+                (void)hipMemcpy(dev, host_rows->data(), (size_t)rows * n * sizeof(float), hipMemcpyHostToDevice);
+                sampler->Sample(dev, SR_DTYPE_F32, rows, n, n, tok, flg, in, same);
+                sampler->Synchronize();
+                std::vector<int32_t> t((size_t)rows);
+                flags.assign((size_t)rows, 0u);
+                (void)hipMemcpy(t.data(), tok, (size_t)rows * 4, hipMemcpyDeviceToHost);
+                (void)hipMemcpy(flags.data(), flg, (size_t)rows * 4, hipMemcpyDeviceToHost);
+                out.assign(t.begin(), t.end());
+            }
+        };
+        BatchSampler bs(0);
+        std::vector<float> host_rows((size_t)rows * n);
+        Fwd fwd{&bs, &host_rows};
+        fwd.rows = rows;
+        fwd.n = n;
+        (void)hipMalloc((void**)&fwd.dev, (size_t)rows * n * sizeof(float));
+        (void)hipMalloc((void**)&fwd.tok, (size_t)rows * 4);
+        (void)hipMalloc((void**)&fwd.flg, (size_t)rows * 4);
+        std::vector<Seq> dev_seqs((size_t)rows), ref_seqs((size_t)rows);
+        std::vector<SeededRandom> dev_src, ref_src;
+        std::vector<PeekableRandom> dev_rng, ref_rng;
+        for (int r = 0; r < rows; r++) { dev_src.emplace_back(77u + (unsigned)r); ref_src.emplace_back(77u + (unsigned)r); }
+        for (int r = 0; r < rows; r++) { dev_rng.emplace_back(&dev_src[(size_t)r]); ref_rng.emplace_back(&ref_src[(size_t)r]); }
+        for (int r = 0; r < rows; r++) {
+            SamplingParams p;
+            if (r == 0) { p.Temperature = 0.8f; p.TopK = 40; p.TopP = 0.95f; p.RepetitionPenalty = 1.15f; p.FrequencyPenalty = 0.3f; }
+            if (r == 1) { p.Temperature = 0.7f; p.TopP = 0.9f; p.PresencePenalty = 0.6f; }
+            if (r == 2) { p.Temperature = 1.0f; p.TopK = 12; }
+            for (auto* v : {&dev_seqs, &ref_seqs}) {
+                Seq& q = (*v)[(size_t)r];
+                q.Sp = p;
+                q.Id = r;
+                q.RecentTokens = p.HasHistoryPenalty() ? &q.hist : nullptr;
+            }
+            dev_seqs[(size_t)r].Rng = &dev_rng[(size_t)r];
+            ref_seqs[(size_t)r].Rng = &ref_rng[(size_t)r];
+        }
+        DeviceSamplingGate gate;
+        std::vector<int> cur((size_t)rows, 1);
+        int host_steps = 0;
+        for (int step = 0; step < steps; step++) {
+            for (int r = 0; r < rows; r++) {
+                auto row = make_logits(g, (size_t)n, 1.5f);
+                if (step == 9 && r == 2) std::fill(row.begin(), row.end(), -std::numeric_limits<float>::infinity());  // draws nothing
+                std::copy(row.begin(), row.end(), host_rows.begin() + (size_t)r * n);
+            }
+            // the reference's way for every row
+            std::vector<int> want((size_t)rows);
+            for (int r = 0; r < rows; r++) {
+                Seq& q = ref_seqs[(size_t)r];
+                SamplingParams sp = q.Sp;
+                if (q.RecentTokens) sp.PreviousTokens = *q.RecentTokens;
+                OracleParams op(sp);
+                const double u = q.Rng->Peek();
+                oracle_rng orng;
+                oracle_rng_replay(&orng, &u, 1);
+                want[(size_t)r] = (step == 5 && r == 1) ? 90 : oracle_sample(host_rows.data() + (size_t)r * n, n, &op.p, &orng);
+                if (!(step == 5 && r == 1) && orng.pos > 0) q.Rng->Commit();
+            }
+            // the device engine: step 5 has a forced token in the middle row, step 11 is skipped by the engine (sampled on the host)
+            dev_seqs[1].ForcedClose = step == 5;
+            std::vector<int> got;
+            const size_t draws_before = dev_rng[0].draws + dev_rng[1].draws + dev_rng[2].draws;
+            const bool on_device = step != 11 && gate.TrySample(fwd, dev_seqs, cur, step, got);
+            if (!on_device) {
+                host_steps++;
+                if (step == 5) CHECK(dev_rng[0].draws + dev_rng[1].draws + dev_rng[2].draws == draws_before, "the refused step consumed a uniform");
+                if (step == 11) bs.InvalidateHistory();
+                got.assign((size_t)rows, 0);
+                for (int r = 0; r < rows; r++) {
+                    Seq& q = dev_seqs[(size_t)r];
+                    if (q.ForcedClose) { got[(size_t)r] = 90; continue; }
+                    SamplingParams sp = q.Sp;
+                    if (q.RecentTokens) sp.PreviousTokens = *q.RecentTokens;
+                    OracleParams op(sp);
+                    const double u = q.Rng->Peek();
+                    oracle_rng orng;
+                    oracle_rng_replay(&orng, &u, 1);
+                    got[(size_t)r] = oracle_sample(host_rows.data() + (size_t)r * n, n, &op.p, &orng);
+                    if (orng.pos > 0) q.Rng->Commit();
+                }
+            }
+            for (int r = 0; r < rows; r++) {
+                CHECK(got[(size_t)r] == want[(size_t)r], "gate step %d row %d: device engine %d, reference %d", step, r, got[(size_t)r], want[(size_t)r]);
+                if (dev_seqs[(size_t)r].RecentTokens) dev_seqs[(size_t)r].hist.push_back(want[(size_t)r]);
+                if (ref_seqs[(size_t)r].RecentTokens) ref_seqs[(size_t)r].hist.push_back(want[(size_t)r]);
+                cur[(size_t)r] = want[(size_t)r];
+            }
+        }
+        for (int r = 0; r < rows; r++)
+            CHECK(dev_rng[(size_t)r].draws == ref_rng[(size_t)r].draws, "row %d drew %zu values, the reference %zu", r, dev_rng[(size_t)r].draws,
+                  ref_rng[(size_t)r].draws);
+        CHECK(ref_rng[2].draws == (size_t)steps - 1, "the row without a finite logit must not draw");
+        CHECK(host_steps == 2 && fwd.sample_calls == steps - 2, "two steps on the host, the others on the device");
+        CHECK(bs.uploads == 3 && bs.appends == steps - 2 - 3, "uploads %d appends %d: the first step and the step after each host step upload", bs.uploads, bs.appends);
+        (void)hipFree(fwd.dev);
+        (void)hipFree(fwd.tok);
+        (void)hipFree(fwd.flg);
+    }
+    std::printf("engine gate done\n");
 
     if (g_failed) {
         std::printf("FAILED %d of %d checks\n", g_failed, g_checks);

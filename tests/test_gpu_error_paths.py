@@ -81,3 +81,44 @@ def test_empty_batches_and_a_single_token_vocabulary(ctx):
     one = _cuda(np.array([[0.5], [-2.0]], dtype=np.float32))
     params = [SamplingParams(Temperature=1.0, TopP=0.5), SamplingParams(Temperature=0.7, TopK=1)]
     assert ctx.sample_batch(one, params, [0.3, 0.9]).tolist() == [0, 0]
+
+
+def test_a_batch_that_names_a_released_or_restarted_mask_is_refused_before_any_launch(ctx):
+    """Only status codes are looked at: a launch with a stale id would read outside the pool of masks."""
+    import torch
+
+    rng = np.random.default_rng(5)
+    V = 3_001
+    L, h = ctx.L, ctx.h
+    p = lambda t: C.c_void_p(t.data_ptr())
+    dev = _cuda(rng.normal(0, 1, (2, V)).astype(np.float32))
+    toks = torch.empty(2, dtype=torch.int32, device="cuda")
+    probs = torch.empty((2, V), dtype=torch.float32, device="cuda")
+    words = rng.integers(1, 2**32, (2, (V + 31) // 32), dtype=np.uint64).astype(np.uint32)
+    ids = [ctx.register_mask(words[i], V) for i in range(2)]
+    params = [SamplingParams(Temperature=0.8, TopK=20), SamplingParams(Temperature=0.9, TopP=0.9)]
+    b = ctx.new_batch().upload(params, V, rng.random(2), mask_ids=ids)
+    assert L.sr_sample_launch(h, b.h, p(dev), sa.SR_DTYPE_F32, V, p(toks), None) == sa.SR_OK
+    ctx.synchronize()
+    # released, and registered again with other bits: the id is the same, the mask is not
+    ctx.release_mask(ids[1])
+    assert L.sr_sample_launch(h, b.h, p(dev), sa.SR_DTYPE_F32, V, p(toks), None) == sa.SR_ERR_INVALID_ARGUMENT
+    assert b"released" in L.sr_last_error(h)
+    assert ctx.register_mask(words[0], V) == ids[1]
+    assert L.sr_sample_launch(h, b.h, p(dev), sa.SR_DTYPE_F32, V, p(toks), None) == sa.SR_ERR_INVALID_ARGUMENT
+    assert L.sr_build_distribution_launch(h, b.h, p(dev), sa.SR_DTYPE_F32, V, p(probs), V, V) == sa.SR_ERR_INVALID_ARGUMENT
+    # naming the id again (the caller states which mask the row has now) makes the batch good again
+    b.append_tokens([-1, -1], rng.random(2), mask_ids=ids)
+    assert L.sr_sample_launch(h, b.h, p(dev), sa.SR_DTYPE_F32, V, p(toks), None) == sa.SR_OK
+    ctx.synchronize()
+    # every mask released and one registered for another vocabulary: the pool starts again, the old batch is stale for good
+    for i in ids:
+        ctx.release_mask(i)
+    other = ctx.register_mask(np.full(40, 0xffffffff, np.uint32), 1_000)
+    assert L.sr_sample_launch(h, b.h, p(dev), sa.SR_DTYPE_F32, V, p(toks), None) == sa.SR_ERR_INVALID_ARGUMENT
+    t = np.array([-1, -1], dtype=np.int32)
+    m = np.array([0, 0], dtype=np.int32)
+    assert L.sr_batch_append_tokens_masks(b.h, t.ctypes.data_as(C.POINTER(C.c_int32)), None,
+                                          m.ctypes.data_as(C.POINTER(C.c_int32))) == sa.SR_ERR_INVALID_ARGUMENT
+    ctx.release_mask(other)
+    b.close()

@@ -169,3 +169,79 @@ def test_constrained_decode_loop_over_registered_states(ctx, vocab, rows, steps)
     batch.close()
     for i in ids:
         ctx.release_mask(i)
+
+
+def _allowed_on_device(ctx, mask_id, vocab):
+    """Which tokens a registered mask lets through, asked of the sampler itself: row t prefers token t by a wide margin,
+    so Greedy(masked row t) == t exactly when t is allowed (the probe of ForcedToolCallConstraintTests.AllowedMask and
+    AndTokenConstraintTests.Allowed, through the device)."""
+    import torch
+
+    logits = np.zeros((vocab, vocab), dtype=np.float32)
+    logits[np.arange(vocab), np.arange(vocab)] = 50.0
+    dev = _cuda(logits)
+    params = [SamplingParams(Temperature=0.0) for _ in range(vocab)]
+    batch = ctx.new_batch().upload(params, vocab, None, mask_ids=[mask_id] * vocab)
+    got = _launch(ctx, batch, dev, vocab)
+    batch.close()
+    return got == np.arange(vocab)
+
+
+def _one_hot_words(vocab, allow):
+    a = np.zeros(vocab, dtype=bool)
+    a[list(allow)] = True
+    return pack_allow_mask(a)
+
+
+def test_mask_and_follows_the_and_constraint(ctx):
+    """AndTokenConstraintTests.cs: shared token survives, an empty intersection falls back unmasked, dead inners are
+    skipped, four inners all contribute (AndTokenConstraint.cs:44-86)."""
+    V = 8
+    ids = {t: ctx.register_mask(_one_hot_words(V, [t]), V) for t in (0, 1, 2, 3, 4)}
+    both = ctx.register_mask(_one_hot_words(V, [2, 4, 5]), V)
+    # OverlappingWindows_SharedAllowedToken_Survives
+    m = ctx.mask_and([ids[4], ids[4]])
+    assert m >= 0 and _allowed_on_device(ctx, m, V).tolist() == [t == 4 for t in range(V)]
+    # OverlappingWindows_EmptyIntersection_FallsBackUnmasked / CombineParams_FourSurvivors: no mask at all
+    assert ctx.mask_and([ids[2], ids[3]]) == -1
+    assert ctx.mask_and([ids[0], ids[1], ids[2], ids[3]]) == -1
+    # a dead inner (its Filter returned the input: id -1) is skipped, the others still intersect
+    m2 = ctx.mask_and([-1, both, ids[2], -1])
+    assert m2 >= 0 and _allowed_on_device(ctx, m2, V).tolist() == [t == 2 for t in range(V)]
+    # nothing constraining: no mask; a single survivor: a copy of it
+    assert ctx.mask_and([-1, -1]) == -1 and ctx.mask_and([]) == -1
+    m3 = ctx.mask_and([both])
+    assert m3 not in (both, -1) and _allowed_on_device(ctx, m3, V).tolist() == [t in (2, 4, 5) for t in range(V)]
+    with pytest.raises(ValueError):
+        ctx.mask_and([ids[0], 99])
+    # a wide vocabulary with bits set beyond it: they never count as "a token is left"
+    V2_words = np.full((151_936 + 31) // 32, 0, dtype=np.uint32)
+    for i in list(ids.values()) + [both, m, m2, m3]:
+        ctx.release_mask(i)
+    a = V2_words.copy(); a[-1] = 0xffffffff; a[5] = 1 << 7
+    b = V2_words.copy(); b[-1] = 0xffff0000; b[5] = 1 << 9
+    ia, ib = ctx.register_mask(a, 151_936 - 17), ctx.register_mask(b, 151_936 - 17)
+    assert ctx.mask_and([ia, ib]) == -1          # word 4747 overlaps only in bits >= 15, beyond vocab 151,919
+    ctx.release_mask(ia)
+    ctx.release_mask(ib)
+
+
+def test_forced_marker_and_trie_masks_through_the_registry(ctx):
+    """ForcedToolCallConstraintTests.cs (only the marker is samplable before it), ConstrainedChoiceSamplingTests.cs
+    Test16 (:365-378: only token 10 stays legal) and Test2 (:41-64: the illegal top logit 99 loses to token 10)."""
+    V = 32
+    forced = ctx.register_mask(_one_hot_words(V, [1]), V)
+    allowed = _allowed_on_device(ctx, forced, V)
+    assert allowed[1] and allowed.sum() == 1
+    ctx.release_mask(forced)
+    V = 100
+    yes = ctx.register_mask(_one_hot_words(V, [10]), V)      # children of the trie's root for AllowedChoices = ["YES"]
+    allowed = _allowed_on_device(ctx, yes, V)
+    assert allowed[10] and not allowed[0] and not allowed[99] and allowed.sum() == 1
+    logits = np.zeros((2, V), dtype=np.float32)
+    logits[:, 99] = 9.0                                          # MockHighestLogitForwardPass(99)
+    params = [SamplingParams(Temperature=0.0), SamplingParams(Temperature=0.8, TopK=40, TopP=0.95)]
+    batch = ctx.new_batch().upload(params, V, [0.0, 0.77], mask_ids=[yes, yes])
+    assert _launch(ctx, batch, _cuda(logits), 2).tolist() == [10, 10]
+    batch.close()
+    ctx.release_mask(yes)
