@@ -4,8 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 One "step" = one batched sampling call (sr_sample_launch / sr_spec_verify_launch) over a batch of
-seeded synthetic logits that are already resident in HBM.  Four distinct logits buffers are rotated so
-every step streams cold data (4 x 155.6 MB exceeds the 256 MB Infinity Cache).  Prints ONE JSON line.
+seeded synthetic logits that are already resident in HBM.  Distinct logits buffers are rotated, enough of them to
+exceed the 256 MB Infinity Cache (4 x 155.6 MB for the headline; 8 for c2, 16 for c4; c1 is measured warm and the line
+says so), so every step streams cold data.  Prints ONE JSON line.
 The default run times c3_fp32_full for K steps and then, in short windows of their own, the other
 configurations (c1, c2, c3_bf16, c4, c5): their figures are the "per_config" object of the same line.
 Every measured launch is checked against the CPU oracle outside the timed regions, every row of it.
@@ -37,15 +38,15 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 
 
-def make_workload(name: str):
+def make_workload(name: str, rows: int = 256):
     from opentail.stingray_amd import synthetic
 
     if name == "c3_fp32_full":
-        return synthetic.config3(rows=256, bf16=False, full_chain=True)
+        return synthetic.config3(rows=rows, bf16=False, full_chain=True)
     if name == "c3_fp32":
-        return synthetic.config3(rows=256, bf16=False)
+        return synthetic.config3(rows=rows, bf16=False)
     if name == "c3_bf16":
-        return synthetic.config3(rows=256, bf16=True)
+        return synthetic.config3(rows=rows, bf16=True)
     if name == "c1":
         return synthetic.config1(steps=1)
     if name == "c2":
@@ -57,27 +58,49 @@ def make_workload(name: str):
     raise SystemExit(f"unknown workload {name}")
 
 
+def host_description() -> dict:
+    """CPU model and core count of the box the baseline runs on, and whether a .NET runtime is there."""
+    import shutil
+
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    dotnet = shutil.which("dotnet")
+    return {"cpu_model": model, "nproc": os.cpu_count(), "dotnet": dotnet,
+            "note": ("dotnet found at %s, but the managed shim is not built here" % dotnet) if dotnet else
+                    "no .NET runtime on this box: the C restatement of the reference sampler is the baseline"}
+
+
 def cpu_baseline(w, budget_s: float):
-    """The CPU oracle (a port of the reference sampler) on one core, rows in order, same inputs."""
+    """The CPU oracle (a C restatement of the reference sampler) on one core, rows in order, same inputs.  A step is
+    the whole batch.  At least 10 warm-up steps (fewer only when they alone would take longer than the budget), then
+    the median of at least 5 timed steps, as many as the budget allows."""
     from oracle import binding as orc
     from tests.helpers import to_oracle
 
     params = [to_oracle(p) for p in w.params]
     u = np.asarray(w.uniforms, dtype=np.float64).reshape(w.rows, -1)[:, 0].copy()
-    orc.sample_batch(w.logits[:2], params[:2], u[:2],
-                     None if w.allow_mask is None else w.allow_mask[:2],
-                     None if w.mask_active is None else w.mask_active[:2])  # warm-up
-    done = 0
-    t0 = time.perf_counter()
-    passes = 0
-    while True:
+
+    def one_step():
+        t0 = time.perf_counter()
         orc.sample_batch(w.logits, params, u, w.allow_mask, w.mask_active)
-        done += w.rows
-        passes += 1
-        el = time.perf_counter() - t0
-        if el >= budget_s or passes >= 400:
-            break
-    return done / el, done, el
+        return time.perf_counter() - t0
+
+    first = one_step()
+    n_warm = 10 if first * 10 <= budget_s else max(1, int(budget_s / max(first, 1e-9)) // 2)
+    for _ in range(n_warm - 1):
+        one_step()
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 or (time.perf_counter() - t_all < budget_s and len(times) < 2000):
+        times.append(one_step())
+    med = float(np.median(times))
+    return w.rows / med, n_warm, len(times), med
 
 
 def prime_events(torch, stream):
@@ -157,9 +180,11 @@ def bench_spec(args, w, ctx, stream) -> dict:
         el = time.perf_counter() - c0
         cpu = {"value": done / el, "unit": "rows/s", "cores": 1, "kind": "port",
                "sample": f"{done} row verifications (8 drafts each) of the same workload on one thread, {el:.1f} s"}
-    # every target position is read for its distribution; the draft distribution of the rejected position
-    # and the bonus / residual pass add one more row each
-    alg_bytes = rows * (L + 1) * V * 4 + rows * V * 4 + rows * L * 8
+    # the target logits of the L verified positions once, one draft distribution per row (the position of the first
+    # rejection) and the gathers of q at the draft tokens
+    alg_bytes = rows * L * V * 4 + rows * V * 4 + rows * L * 4
+    bytes_with_bonus = rows * (L + 1) * V * 4 + rows * V * 4 + rows * L * 8   # ... the bonus position counted for every row
+    bytes_everything = rows * (L + 1) * V * 4 + rows * L * V * 4              # ... every input tensor in full
     achieved = alg_bytes / (dev_us * 1e-6) / 1e9
     emitted = float((acc_h + 1).mean())
     out_j = {
@@ -170,6 +195,7 @@ def bench_spec(args, w, ctx, stream) -> dict:
         "config": {"workload": "c5", "rows": rows, "n_draft": L, "vocab": V, "mean_tokens_emitted_per_row": emitted},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                     "bytes_with_bonus_position_for_every_row": bytes_with_bonus, "bytes_reading_every_input": bytes_everything,
                      "kernel": "k_full_row", "kernel_us": dev_us},
         "cpu_baseline": cpu, "parity": parity,
     }
@@ -236,16 +262,20 @@ def run_workload(args, ctx, stream) -> dict:
 
     if args.workload == "argmax":
         return bench_argmax(args, ctx, stream)
-    w = make_workload(args.workload)
+    w = make_workload(args.workload, getattr(args, "rows", 256))
     rows, vocab = w.rows, w.vocab
     if args.workload == "c5":
         return bench_spec(args, w, ctx, stream)
 
-    # four distinct resident logits buffers (row-rotated copies of the seeded tensor) + their batches
-    n_buf = 4
+    # distinct resident logits buffers (row-rotated copies of the seeded tensor) + their batches: four, or as many as
+    # it takes to exceed the 256 MB Infinity Cache (16 at most: a smaller workload is measured warm and says so)
+    elem = 2 if w.logits_bf16 is not None else 4
+    buf_bytes = rows * vocab * elem
+    n_buf = int(min(16, max(4, -(-300_000_000 // buf_bytes))))
+    cold = n_buf * buf_bytes > 268_435_456
     bufs, batches, host_logits = [], [], []
     for i in range(n_buf):
-        sh = (i * 7) % rows
+        sh = (i * 7) % rows if rows > 1 else 0
         lg = np.roll(w.logits, sh, axis=0)
         host_logits.append(lg)
         if w.logits_bf16 is not None:
@@ -297,7 +327,7 @@ def run_workload(args, ctx, stream) -> dict:
     step_with_upload_us = None
     extra_legs = args.workload.startswith("c3") and not args.short and not os.environ.get("SR_BENCH_NO_UPLOAD_LEG")
     if extra_legs:
-        n_up = max(10, args.steps // 4)
+        n_up = max(100, args.steps // 4)
         for i in range(3):
             batches[i % n_buf].reupload()
             step(i)
@@ -314,7 +344,7 @@ def run_workload(args, ctx, stream) -> dict:
     # the batch is rebuilt).  Batches and outputs of their own: the measured ones stay as they are for the parity check.
     step_with_append_us = None
     if extra_legs:
-        n_up = max(10, args.steps // 4)
+        n_up = max(100, args.steps // 4)
         ab = [ctx.new_batch().upload(w.params, vocab, w.uniforms, w.allow_mask, w.mask_active) for _ in range(n_buf)]
         atok = torch.empty(rows, dtype=torch.int32, device="cuda")
         rng = np.random.default_rng(7)
@@ -346,12 +376,11 @@ def run_workload(args, ctx, stream) -> dict:
         parity = {"rows_checked": int(n_chk), "mismatches": int((got != want).sum())}
     unsupported = int(sum(int((f.cpu().numpy().view(np.uint32) >> 31).sum()) for f in flags))
 
-    elem = 2 if w.logits_bf16 is not None else 4
     alg_bytes = rows * vocab * elem + (0 if w.allow_mask is None else w.allow_mask.nbytes) + rows * 8
     achieved = alg_bytes / (kern_us * 1e-6) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", f"traffic_{args.workload}.json.txt")
-    if os.path.exists(tpath):
+    if os.path.exists(tpath) and rows == 256:
         try:
             traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
         except Exception:
@@ -359,10 +388,12 @@ def run_workload(args, ctx, stream) -> dict:
 
     cpu = None
     if args.cpu_seconds > 0:
-        tps, n_done, el = cpu_baseline(w, args.cpu_seconds)
-        cpu = {"value": tps, "unit": "tokens/s", "cores": 1, "kind": "port",
-               "sample": f"{n_done} rows of the same workload ({args.workload}), rows in order on one thread, "
-                         f"{el:.1f} s; oracle = C port of the reference sampler (no .NET runtime on this box)"}
+        tps, n_warm, n_rep, med = cpu_baseline(w, args.cpu_seconds)
+        host = host_description()
+        cpu = {"value": tps, "unit": "tokens/s", "cores": 1, "kind": "port", "us_per_step": med * 1e6,
+               "cpu_model": host["cpu_model"], "nproc": host["nproc"],
+               "sample": f"one step = the {rows} rows of the same workload ({args.workload}), rows in order on one thread of "
+                         f"{host['nproc']}; {n_warm} warm-up steps, median of {n_rep} timed steps; {host['note']}"}
 
     out = {
         "metric": "sampled tokens/sec at B=256x152k vocab" if rows == 256 else f"sampled tokens/sec at B={rows}x{vocab} vocab",
@@ -378,7 +409,8 @@ def run_workload(args, ctx, stream) -> dict:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32" if elem == 4 else "bf16->f32",
-        "data": "synthetic (seeded Gaussian + Zipf-head logits, 4 rotated resident buffers)",
+        "data": f"synthetic (seeded Gaussian + Zipf-head logits, {n_buf} rotated resident buffers = "
+                f"{n_buf * buf_bytes / 1e6:.0f} MB: {'cold reads' if cold else 'WARM: fits the 256 MB Infinity Cache'})",
         "config": {"workload": args.workload, "rows": rows, "vocab": vocab,
                    "chain": "penalties+top-k+top-p+min-p" if args.workload == "c3_fp32_full" else args.workload},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -386,6 +418,8 @@ def run_workload(args, ctx, stream) -> dict:
                      "frac_with_token_append": (None if step_with_append_us is None else
                                                 alg_bytes / (step_with_append_us * 1e-6) / 1e9 / HBM_PEAK_GBS),
                      "traffic": traffic,
+                     "traffic_source": None if traffic is None else
+                     f"profiles/{os.path.basename(tpath)}: rocprofv3 --pmc runs of this command, committed; not measured by this run",
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "kernel": "k_topk_rows" if args.workload.startswith(("c1", "c3")) else "k_full_row",
                      "kernel_us": kern_us},
@@ -411,6 +445,7 @@ def main():
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="c3_fp32_full")
+    ap.add_argument("--rows", type=int, default=256, help="batch rows of the c3_* workloads (the benchmark's point is 256)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget (0 = skip)")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--no-prime", action="store_true", help="skip the event warm-up (prime_events): for looking at it")
@@ -463,6 +498,17 @@ def main():
                 "parity": r["parity"], "config": r["config"],
             }
         out["per_config"] = per
+        # the headline kernel at other batch sizes (same row width and chain): the curve around the benchmark's point
+        sweep = {}
+        for n_rows in (64, 128, 192, 320, 512):
+            gc.collect()
+            torch.cuda.empty_cache()
+            sub = argparse.Namespace(**vars(args))
+            sub.workload, sub.steps, sub.warmup, sub.short, sub.rows, sub.cpu_seconds = "c3_fp32_full", 200, 20, True, n_rows, 0.0
+            r = run_workload(sub, ctx, stream)
+            sweep[str(n_rows)] = {"us_per_step": r["us_per_step_device"], "frac": r["roofline"]["frac"], "value": r["value"],
+                                  "parity": r["parity"]}
+        out["rows_sweep_c3_fp32_full"] = sweep
     print(json.dumps(out))
 
 

@@ -17,11 +17,12 @@ int64_t sr_batch_mask_stride(const sr_batch* b) { return b->mask_ids ? (int64_t)
 int sr_batch_masks_valid(sr_ctx* ctx, const sr_batch* b, const char* who)
 {
     if (!b->mask_ids) return SR_OK;
-    bool stale = b->mask_pool_gen != ctx->pool_gen || ctx->pool_vocab != b->vocab || b->keep_mask_ids.size() != (size_t)b->rows;
+    bool stale = b->keep_mask_ids.size() != (size_t)b->rows;
     for (int32_t r = 0; r < b->rows && !stale; r++) {
         const int32_t id = b->keep_mask_ids[(size_t)r];
-        if (id < 0) continue;
-        stale = id >= ctx->pool_cap || !ctx->pool_used[(size_t)id] || ctx->pool_slot_gen[(size_t)id] != b->keep_mask_gen[(size_t)r];
+        if (id < 0) continue;  // (a batch whose rows name no mask reads none)
+        stale = b->mask_pool_gen != ctx->pool_gen || ctx->pool_vocab != b->vocab || id >= ctx->pool_cap ||
+                !ctx->pool_used[(size_t)id] || ctx->pool_slot_gen[(size_t)id] != b->keep_mask_gen[(size_t)r];
     }
     if (stale)
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, std::string(who) + ": the batch names a registered mask that was released, or whose "
@@ -711,6 +712,9 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     const int32_t rows = b->rows, vocab = b->vocab;
     if (rows == 0) return SR_OK;
     std::vector<int32_t> scan_again;  // scan-mask rows whose allow-mask changes
+    bool names_mask = false;
+    for (int32_t r = 0; new_mask_ids && r < b->rows && !names_mask; r++) names_mask = b->keep_mask_ids[(size_t)r] >= 0;
+    if (new_mask_ids && !names_mask) b->mask_pool_gen = ctx->pool_gen;  // no row held an id of an older pool
     if (new_mask_ids && b->mask_pool_gen != ctx->pool_gen)
         return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_batch_append_tokens_masks: the registered masks were started again for another "
                                                          "vocabulary since the batch was uploaded; upload the batch again");
