@@ -886,6 +886,15 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             // a history id whose adjusted logit is below the candidates' bound has at least top_k candidates above
             // it, or lies too far below the maximum to matter
             const uint32_t bound_key = sr_okey(bound0);
+            // (here and not where the candidates are collected: a thread's few atomics are in flight together, where
+            // each candidate handed over waited for the one before it)
+            {
+                uint32_t* meta_w = (uint32_t*)sm.probs;
+                for (int i = tid; i < n_c; i += kThreads) {
+                    const int b = bmap.of(__fmul_rn(sm.vals[i], inv_temp));
+                    meta_w[i] = ((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u);
+                }
+            }
             uint32_t hmeta[kHistRegs];
 #pragma unroll
             for (int r = 0; r < kHistRegs; r++) {
@@ -1235,11 +1244,11 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 // SR_TK_SEL_MAX in sm.vals / sm.idxs, the rest of an unusually long list in a.cand.  Returns the number of
 // candidates, or -1 when the row cannot be handled.  Called by every thread of the tail workgroup; the two
 // hooks let the caller issue loads of its own behind the group maxima's (early) and after the first wait (late).
-// With want_bins the candidates are also counted into the tail's histogram (sm.bhist; the bins run from the row's
-// largest kept element down to the bound, see BinMap), and every candidate remembers its bin and its arrival number
-// inside the bin (sm.probs, as integers): the tail can then lay the candidates out bin by bin without another pass
-// of atomics.  *binned tells whether that happened (few chunks, a short enough list, a finite maximum); *map_out
-// is the map that was used.
+// With want_bins the tail's histogram (sm.bhist) is cleared and the map of its bins is made (the bins run from the
+// row's largest kept element down to the bound, see BinMap); the caller then counts the candidates into it, each
+// remembering its bin and its arrival number inside the bin (sm.probs, as integers), and lays them out bin by bin.
+// *binned tells whether the list is fit for that (few chunks, a short enough list, a finite maximum); *map_out is
+// the map.
 // force_exact, and any row whose candidates overflow the lists: the row's sel-th largest kept element is found by a
 // radix select over the logits themselves, and the candidates are exactly the sel largest in (value desc, index asc)
 // order.  Slow (several passes over the row), exact for any data, and independent of the chunk results.
@@ -1456,19 +1465,12 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     };
     bool bins = false;
     BinMap map;
-    uint32_t* meta = (uint32_t*)sm.probs;
-    // the bin of a candidate: 0 .. kBins - 1, never increasing with the value (what lies too far below the maximum
-    // to matter never gets here: the bound is at least the maximum minus 18 T, see below)
-    auto bin0 = [&](float x) SR_INL -> int { return map.of(__fmul_rn(x, inv_temp)); };
     // one candidate at list position pos
     auto place = [&](uint32_t pos, float x, int idx) SR_INL {
         if (pos < (uint32_t)kSelMax) {
             sm.vals[pos] = x;
             sm.idxs[pos] = idx;
-            if (bins) {
-                const int b = bin0(x);
-                meta[pos] = ((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u);
-            }
+
         } else if (pos < (uint32_t)kRowCap) {
             sr_store_agent(&crow[pos], ((unsigned long long)sr_f2u(x) << 32) | (unsigned long long)(uint32_t)idx);
         }
