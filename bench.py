@@ -375,6 +375,10 @@ def run_workload(args, ctx, stream) -> dict:
                              None if w.mask_active is None else w.mask_active[:n_chk])
         parity = {"rows_checked": int(n_chk), "mismatches": int((got != want).sum())}
     unsupported = int(sum(int((f.cpu().numpy().view(np.uint32) >> 31).sum()) for f in flags))
+    # rows whose token rests on a convention the managed runtime leaves open (SR_OUT_AMBIGUOUS, bit 4), over the
+    # buffers the run touched
+    used = flags[: min(n_buf, args.steps + args.warmup)]
+    ambiguous = int(sum(int(((f.cpu().numpy().view(np.uint32) >> 4) & 1).sum()) for f in used))
 
     alg_bytes = rows * vocab * elem + (0 if w.allow_mask is None else w.allow_mask.nbytes) + rows * 8
     achieved = alg_bytes / (kern_us * 1e-6) / 1e9
@@ -426,6 +430,7 @@ def run_workload(args, ctx, stream) -> dict:
         "cpu_baseline": cpu,
         "parity": parity,
         "rows_unsupported": unsupported,
+        "rows_flagged_ambiguous": {"rows": ambiguous, "of": rows * len(used)},
         "us_per_step_with_batch_upload": step_with_upload_us,
         "us_per_step_with_token_append": step_with_append_us,
     }

@@ -40,6 +40,11 @@ struct FullSmem {
     uint32_t tags[kSmall];
 };
 
+// SR_OUT_AMBIGUOUS of the row at work: any thread that sees a cut or the draw land on its boundary (sr_near /
+// sr_stop_near) stores here; the row's flags are written behind a barrier that follows.
+#define SR_AMB_WORD 15
+#define SR_AMB_IF(cond_) do { if (cond_) sm.bc[SR_AMB_WORD] = 1u; } while (0)
+
 // ---- block reductions ------------------------------------------------------------------------------
 __device__ __forceinline__ float blk_max_f(float v, bool* any_nan, FullSmem& sm)
 {
@@ -943,7 +948,9 @@ __device__ __forceinline__ int draw_from_row(const float* p, int n, double u, Fu
 {
     const float r = __double2float_rn(u);
     int found;
-    seq_sum_row<true>(p, n, 0.0f, r, &found, sm, m1, m2);
+    const float at = seq_sum_row<true>(p, n, 0.0f, r, &found, sm, m1, m2);
+    if (threadIdx.x == 0)
+        SR_AMB_IF(found >= 0 ? sr_stop_near(at, __fmul_rn(__fmul_rn(p[found], m1), m2), r) : sr_near(at, r));
     return found >= 0 ? found : n - 1;
 }
 
@@ -1019,12 +1026,18 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
                 token = 0;  // the running sum starts at p[0] >= 0: index 0 reaches a target of zero whatever it holds
             } else {
                 float acc = 0.0f;
-                for (int i = 0; i < m; i++) {
+                bool hit = false;
+                for (int i = 0; i < m && !hit; i++) {
                     const unsigned long long v = sm.sortbuf[i];
-                    const float x = sr_u2f((uint32_t)v);
-                    acc = __fadd_rn(acc, scale ? __fmul_rn(x, inv) : x);
-                    if (acc >= r) { token = (int)(0xffffffffu - (uint32_t)(v >> 32)); break; }
+                    const float x = sr_u2f((uint32_t)v), xs = scale ? __fmul_rn(x, inv) : x;
+                    acc = __fadd_rn(acc, xs);
+                    if (acc >= r) {
+                        token = (int)(0xffffffffu - (uint32_t)(v >> 32));
+                        hit = true;
+                        SR_AMB_IF(sr_stop_near(acc, xs, r));
+                    }
                 }
+                if (!hit) SR_AMB_IF(sr_near(acc, r));
             }
             if (a.out_tokens) a.out_tokens[row] = token;
         }
@@ -1084,14 +1097,20 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
                 int f;
                 acc = sr_seq_wave<16, true>(x, acc, r, &f);
                 if (f >= 0) {
-                    token = (int)(0xffffffffu - (uint32_t)(sm.sortbuf[place_of(b0 + f)] >> 32));
+                    const unsigned long long v = sm.sortbuf[place_of(b0 + f)];
+                    token = (int)(0xffffffffu - (uint32_t)(v >> 32));
                     done = true;
+                    const float t = sr_u2f((uint32_t)v);
+                    SR_AMB_IF(lane == 0 && sr_stop_near(acc, scale ? __fmul_rn(t, inv) : t, r));
                     break;
                 }
             }
         }
     }
-    if (wave == 0 && lane == 0 && a.out_tokens) a.out_tokens[row] = token;
+    if (wave == 0 && lane == 0) {
+        SR_AMB_IF(!done && sr_near(acc, r));  // (the draw ran off the end of the list: the last index, by the rounding fallback)
+        if (a.out_tokens) a.out_tokens[row] = token;
+    }
 }
 // ... of a list in any order, its entries as probability bits << 32 | ~index
 __device__ __forceinline__ void finish_from_list(const SrFullArgs& a, float* p, int n, int m, int row, FullSmem& sm)
@@ -1381,6 +1400,9 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
                 int f;
                 run = seq_sum<true>([&](int) -> float { return yv; }, c_run, run, top_p, &f, sm);
                 if (f < 0) continue;
+                // (a cut inside a run of equal probabilities keeps the first ones by index: the managed sort leaves
+                // their order open)
+                SR_AMB_IF(f + 1 < c_run || sr_stop_near(run, yv, top_p));
                 // the cut falls inside this run: its first f + 1 entries by index are members
                 const int cw = list_stretch(p, w0, w1, do_scale, inv, StretchCount{}, [&](float y, int) -> bool { return sr_f2u(y) == mn; });
                 __syncthreads();
@@ -1531,6 +1553,8 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
             }
             FPROF_ADD(a, slot, 13, t_step);
             run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, top_p, &found, sm);
+            if (found >= 0)
+                SR_AMB_IF(sr_stop_near(run, sm.sprob[found], top_p) || (found + 1 < nc && sm.sprob[found + 1] == sm.sprob[found]));
             FPROF_ADD(a, slot, 14, t_step);
         }
         if (a.prof && slot == 0 && tid == 0) a.prof[15] += 1ull;
@@ -1538,6 +1562,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         hi_y = c_y;
         d_prev = d_end;
     }
+    if (found < 0 && !cut_in_run) SR_AMB_IF(sr_near(run, top_p));  // the whole row is the nucleus: barely?
 
     // the last slab's entries in index order (the sort's scratch memory is free again)
     __syncthreads();
@@ -1721,6 +1746,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
     SrFullState* st = a.state + slot;
     const bool greedy = rd.temperature <= 0.0f;
     const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
+    if (tid == 0) sm.bc[SR_AMB_WORD] = 0u;  // (every path that can set it passes a barrier first)
 
     if (greedy) {
         // Greedy / GreedyWithHistoryPenalties on the adjusted row; distributions become one-hot
@@ -1823,10 +1849,11 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             no_slabs = way == kNucleusGeneralNoSlabs;
             if (way == kNucleusDone) {
                 FPROF(a, slot, 9);
+                __syncthreads();
                 if (tid == 0) {
                     st->n_survivors = 0;
                     st->flags = flags;
-                    if (a.out_flags) a.out_flags[row] = flags;
+                    if (a.out_flags) a.out_flags[row] = flags | (sm.bc[SR_AMB_WORD] ? SR_KFLAG_AMBIGUOUS : 0u);
                 }
                 return;
             }
@@ -1848,6 +1875,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                 }
                 auto body = [&](float x, int i) -> float {
                     float y = do_scale ? __fmul_rn(x, inv) : x;
+                    if (use_min_p) SR_AMB_IF(sr_near(y, thr));  // an entry on the threshold
                     if (use_min_p && y < thr) y = 0.0f;
                     if (y > 0.0f) {
                         c++;
@@ -1914,7 +1942,10 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             bool nn;
             mp = blk_max_f(mp, &nn, sm);
             const float thr = __fmul_rn(rd.min_p, mp);
-            row_pass<true>(p, n, [&](float x, int) -> float { return x < thr ? 0.0f : x; });
+            row_pass<true>(p, n, [&](float x, int) -> float {
+                SR_AMB_IF(x > 0.0f && sr_near(x, thr));
+                return x < thr ? 0.0f : x;
+            });
             __syncthreads();
         }
         FPROF(a, slot, 5);
@@ -2061,6 +2092,10 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                 __syncthreads();
                 int found;
                 run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, rd.top_p, &found, sm);
+                if (found >= 0)
+                    SR_AMB_IF(sr_stop_near(run, sm.sprob[found], rd.top_p) || (found + 1 < nc && sm.sprob[found + 1] == sm.sprob[found]));
+                else if (taken + nc == ns)
+                    SR_AMB_IF(sr_near(run, rd.top_p));
                 FPROF_ADD(a, slot, 14, t_step);
                 if (a.prof && slot == 0 && tid == 0) a.prof[15] += 1ull;
                 taken += nc;
@@ -2110,7 +2145,10 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                 sort_survivors_in_place(keys, ids, ns, sm);
                 // the nucleus over the sorted survivors (descending probability, ascending index among equal ones)
                 int found;
-                seq_sum<true>([&](int i) -> float { return sr_u2f(keys[i]); }, ns, 0.0f, rd.top_p, &found, sm);
+                const float at = seq_sum<true>([&](int i) -> float { return sr_u2f(keys[i]); }, ns, 0.0f, rd.top_p, &found, sm);
+                if (tid == 0)
+                    SR_AMB_IF(found >= 0 ? (sr_stop_near(at, sr_u2f(keys[found]), rd.top_p) || (found + 1 < ns && keys[found + 1] == keys[found]))
+                                         : sr_near(at, rd.top_p));
                 const int cutoff = found >= 0 ? found + 1 : ns;
                 for (int i = cutoff + tid; i < ns; i += kT) p[ids[i]] = 0.0f;
                 __syncthreads();
@@ -2128,7 +2166,8 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             // the nucleus closed inside the kernel and its members are at hand: no pass over the row is needed
             finish_from_list(a, p, n, listed, row, sm);
             FPROF(a, slot, 9);
-            if (tid == 0 && a.out_flags) a.out_flags[row] = flags;
+            __syncthreads();
+            if (tid == 0 && a.out_flags) a.out_flags[row] = flags | (sm.bc[SR_AMB_WORD] ? SR_KFLAG_AMBIGUOUS : 0u);
             return;
         }
         __syncthreads();
@@ -2143,7 +2182,8 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
         if (tid == 0 && a.out_tokens) a.out_tokens[row] = token;
     }
     FPROF(a, slot, 9);
-    if (tid == 0 && a.out_flags) a.out_flags[row] = st->flags;
+    __syncthreads();
+    if (tid == 0 && a.out_flags) a.out_flags[row] = st->flags | (sm.bc[SR_AMB_WORD] ? SR_KFLAG_AMBIGUOUS : 0u);
 }
 
 // ---- SampleTopK (Sampler.cs:216-357) for rows wider than the selection kernel takes -----------------------
@@ -2258,6 +2298,7 @@ __global__ __launch_bounds__(kT) void k_wide_tail(SrFullArgs a)
     row_pass<true>(probs, k, [&](float x, int) -> float { return __fmul_rn(x, inv_sum); });
     __syncthreads();
     int count = k;
+    bool amb = false;  // SR_OUT_AMBIGUOUS: a cut or the draw lies on its boundary
     if (rd.min_p > 0.0f) {
         const float thr = __fmul_rn(rd.min_p, probs[0]);
         unsigned long long first = 0ull;  // ~index of the first entry below the threshold
@@ -2270,19 +2311,22 @@ __global__ __launch_bounds__(kT) void k_wide_tail(SrFullArgs a)
         });
         first = blk_max_u64(first, sm);
         if (first) count = (int)(0xffffffffull - first);
+        amb = (count > 0 && sr_near(probs[count - 1], thr)) || (count < k && sr_near(probs[count], thr));
     }
     if (rd.top_p < 1.0f && rd.top_p > 0.0f) {
-        seq_sum_row<true>(probs, count, 0.0f, rd.top_p, &found, sm);
+        const float at = seq_sum_row<true>(probs, count, 0.0f, rd.top_p, &found, sm);
+        amb = amb || (found >= 0 ? sr_stop_near(at, probs[found], rd.top_p) : sr_near(at, rd.top_p));
         if (found >= 0) count = found + 1;
     }
     const float kept = seq_sum_row<false>(probs, count, 0.0f, 0.0f, &found, sm);
     const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept);
-    seq_sum_row<true>(probs, count, 0.0f, r, &found, sm);
+    const float at = seq_sum_row<true>(probs, count, 0.0f, r, &found, sm);
+    amb = amb || (found >= 0 ? sr_stop_near(at, probs[found], r) : sr_near(at, r));
     if (tid == 0) {
         int token = id0;
         if (found >= 0 && ids[found] >= 0) token = ids[found];
         a.out_tokens[row] = token;
-        if (a.out_flags) a.out_flags[row] = SR_KFLAG_TOPK;
+        if (a.out_flags) a.out_flags[row] = SR_KFLAG_TOPK | (amb ? SR_KFLAG_AMBIGUOUS : 0u);
     }
 }
 

@@ -9,6 +9,7 @@
 #define SR_KFLAG_TOPK (1u << 1)
 #define SR_KFLAG_FULL (1u << 2)
 #define SR_KFLAG_DEGENERATE (1u << 3)
+#define SR_KFLAG_AMBIGUOUS (1u << 4)
 #define SR_KFLAG_UNSUPPORTED (1u << 31)
 // the public bits of SrRow.flags as device code sees them (the public header is not included on the device side)
 #define SR_ROWBIT_HAS_LOGIT_BIAS (1u << 0)

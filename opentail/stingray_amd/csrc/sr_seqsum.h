@@ -30,6 +30,19 @@
 #define SR_SEQ_WAVES (SR_SEQ_THREADS / SR_WAVE)
 #define SR_SEQ_SAT (1u << 26)  // saturated increment: "this run leaves the binade"
 
+// The guard band behind SR_OUT_AMBIGUOUS: two values count as "on the same boundary" when they are within about four
+// ulps of each other.  The managed runtime leaves three things open that can move a running sum by an ulp or two --
+// the lane order of TensorPrimitives.Sum, the last bit of expf, the order of equal keys in its sort --; a draw or a
+// cut that clears its boundary by more than this band comes out the same whichever way those fall.
+#define SR_AMBIG_REL 4.8e-7f
+__device__ __forceinline__ bool sr_near(float a, float b) { return fabsf(a - b) <= fmaxf(fabsf(a), fabsf(b)) * SR_AMBIG_REL; }
+// A search stopped at a term of size `term` where the running sum `at` reached `target`: the stop is on a boundary
+// when the sum barely reached the target, or the sum before the term (at - term) barely missed it.
+__device__ __forceinline__ bool sr_stop_near(float at, float term, float target)
+{
+    return sr_near(at, target) || (term - (at - target)) <= at * SR_AMBIG_REL;
+}
+
 struct SrSeqSmem {
     uint32_t wa0[2][SR_SEQ_WAVES];  // every wave's increment function, rounds alternate between the two copies
     uint32_t wa1[2][SR_SEQ_WAVES];
@@ -139,7 +152,8 @@ __device__ __forceinline__ SrInc sr_scan_inc(SrInc v)
 // One tile: adds this thread's SR_SEQ_RUN terms (thread order = term order) to the running sum *s
 // (uniform across the block on entry and exit).  When kSearch, also looks for the first term index at
 // which the running sum reaches `target` (fl(s) >= target); on success returns its tile-local index
-// (thread * SR_SEQ_RUN + j) in *found (uniform), else leaves -1.  Terms past the end must be 0.
+// (thread * SR_SEQ_RUN + j) in *found (uniform) and *s is the running sum at that term; else leaves -1.  Terms
+// past the end must be 0.
 //
 // Per round: every wave scans its threads' increment functions and publishes its total; every wave then scans the
 // sixteen totals itself, which also shows the first wave in which the sum leaves the binade (or reaches the
@@ -232,17 +246,21 @@ __device__ __forceinline__ void sr_seq_tile(const float (&x)[SR_SEQ_RUN], float*
                 }
                 const int fl = (int)__ffsll((long long)evl) - 1;
                 // every lane replays its run with real float adds from its own input; the first event lane's counts
-                float acc = sr_join(before, eb_w);
+                float acc = sr_join(before, eb_w), hit = 0.0f;
                 int wj = -1;
 #pragma unroll
                 for (int j = 0; j < SR_SEQ_RUN; j++) {
                     acc = __fadd_rn(acc, x[j]);
-                    if (kSearch && wj < 0 && acc >= target) wj = j;
+                    if (kSearch && wj < 0 && acc >= target) { wj = j; hit = acc; }
                 }
                 s_w = sr_u2f((uint32_t)__builtin_amdgcn_readlane((int)sr_f2u(acc), fl));
                 wj = __builtin_amdgcn_readlane(wj, fl);
                 last = fl;
-                if (kSearch && wj >= 0) { where = (wave * SR_WAVE + fl) * SR_SEQ_RUN + wj; break; }
+                if (kSearch && wj >= 0) {  // (the sum handed back is the running sum AT the term that reached the target)
+                    s_w = sr_u2f((uint32_t)__builtin_amdgcn_readlane((int)sr_f2u(hit), fl));
+                    where = (wave * SR_WAVE + fl) * SR_SEQ_RUN + wj;
+                    break;
+                }
                 lstart = fl + 1;
                 if (lstart >= SR_WAVE) break;
                 // the lanes behind it, scanned again in the binade the sum has reached

@@ -1160,12 +1160,15 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 
     // Sampler.cs:315-324 min-p: the first probs[t] < thr bounds the survivors
     int count = k;
+    bool amb = false;  // SR_OUT_AMBIGUOUS: a cut or the draw lies on its boundary (what wave 0's first lane knows)
     if (rd.min_p > 0.0f) {
         const float thr = __fmul_rn(rd.min_p, sm.probs[0]);
         int first = k;
         for (int t = tid; t < k; t += kThreads)
             if (sm.probs[t] < thr) { first = t; break; }
         count = min(count, block_min_i32(first, sm));
+        // the entries on either side of the cut (the list descends): on the threshold?
+        amb = (count > 0 && sr_near(sm.probs[count - 1], thr)) || (count < k && sr_near(sm.probs[count], thr));
     }
     // Sampler.cs:326-349: running sum; top-p cuts after the first cum >= TopP.  Then the draw (:351-357): the first
     // entry whose running sum reaches r = u * (sum of the kept entries).  One wave runs both searches and nothing is
@@ -1224,13 +1227,15 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         float kept_sum = 0.0f;
         const int hit = first_reach(top_p, count, &kept_sum);
         const int cnt = hit >= 0 ? hit + 1 : count;
+        if (use_top_p) amb = amb || (hit >= 0 ? sr_stop_near(kept_sum, sm.probs[hit], top_p) : sr_near(kept_sum, top_p));
         SR_PROF(a, 10);
         const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept_sum);
-        float unused;
-        const int first = first_reach(r, cnt, &unused);
+        float at = 0.0f;
+        const int first = first_reach(r, cnt, &at);
+        amb = amb || (first >= 0 ? sr_stop_near(at, sm.probs[first], r) : sr_near(at, r));
         if (sr_lane() == 0) {
             a.out_tokens[row] = sm.idxs[first >= 0 ? first : 0];
-            if (a.out_flags) a.out_flags[row] = out_flag;
+            if (a.out_flags) a.out_flags[row] = out_flag | (amb ? SR_KFLAG_AMBIGUOUS : 0u);
         }
     }
 }
