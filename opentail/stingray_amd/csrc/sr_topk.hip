@@ -74,6 +74,13 @@ struct BinMap {
     uint32_t cbits = 0u;
     int ftop = 0;
     bool by_bits = false;
+    // A third map, for rows of bf16 logits that no penalty touches: one bin per distinct value (the upper 16 bits of the
+    // ordered key are the whole value), counted down from the row's largest.  Entries of one bin are then equal, no
+    // order among them is needed for any sum, and the one entry whose index matters -- the draw's -- is picked from its
+    // bin at the end: see topk_row_tail.
+    bool exact = false;
+    uint32_t ktop = 0u;     // ordered key of the row's largest kept element >> 16
+    __device__ __forceinline__ int of_raw(float x) const { return min(max((int)(ktop - (sr_okey(x) >> 16)), 0), kBins - 1); }
     __device__ __forceinline__ int of(float xs) const
     {
         const float d = __fsub_rn(xs, mx);
@@ -669,6 +676,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     int sort_n = 0;  // entries handed to the sort
     bool ranked = false;  // sm.vals / sm.idxs already hold the k first entries
     bool placed = false;  // ... laid out from the binned candidate list: the maximum is the first ranked entry
+    bool exact_bins = false;  // ... one bin per distinct value: entries of a bin stand in no order (see BinMap::exact)
 
     if (use_edits && !excl) {
         // ---- penalties that may raise a logit: the reference's literal top-(k + history length) set ------
@@ -891,7 +899,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             {
                 uint32_t* meta_w = (uint32_t*)sm.probs;
                 for (int i = tid; i < n_c; i += kThreads) {
-                    const int b = bmap.of(__fmul_rn(sm.vals[i], inv_temp));
+                    const int b = bmap.exact ? bmap.of_raw(sm.vals[i]) : bmap.of(__fmul_rn(sm.vals[i], inv_temp));
                     meta_w[i] = ((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u);
                 }
             }
@@ -907,7 +915,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             if (n_live == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
             __syncthreads();  // sm.boff written, every wave done with the histogram
             SR_PROF(a, 6);
-            if (n_keep <= kSelMax && max_bin <= 96) {
+            if (n_keep <= kSelMax && max_bin <= (bmap.exact ? 256 : 96)) {
                 const uint32_t* meta = (const uint32_t*)sm.probs;
                 for (int i = tid; i < n_c; i += kThreads) {
                     const uint32_t mt = meta[i];
@@ -936,6 +944,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 load_cands();  // a flat or heavily tied row: the general way below
                 bmap = BinMap{};
             }
+            exact_bins = placed && bmap.exact;
         }
         if (!placed) {
         uint32_t lmaxk = 0u;
@@ -1031,7 +1040,15 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             // the bin that precede it
             ranked = true;
             const int kk = min(rd.top_k, m2);
-            for (int i = tid; i < ms; i += kThreads) {
+            if (exact_bins) {
+                // every bin holds one value: the layout is the order by value already, and which of a bin's equal
+                // entries stands where makes no difference to any sum
+                for (int i = tid; i < kk; i += kThreads) {
+                    sm.vals[i] = sr_okey_inv(sm.xa[i]);
+                    sm.idxs[i] = (int)(0xffffffffu - sm.xc[i]);
+                }
+            }
+            for (int i = tid; i < (exact_bins ? 0 : ms); i += kThreads) {
                 const uint32_t mh = sm.xa[i], mm = sm.xb[i], ml = sm.xc[i];
                 const int b = bin_kept(mh);
                 const int p0 = (int)sm.boff[bin_word(b)], p1 = p0 + (int)sm.bhist[bin_word(b)];
@@ -1233,8 +1250,26 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         float at = 0.0f;
         const int first = first_reach(r, cnt, &at);
         amb = amb || (first >= 0 ? sr_stop_near(at, sm.probs[first], r) : sr_near(at, r));
+        int token = sm.idxs[first >= 0 ? first : 0];
+        if (exact_bins) {
+            // The draw stopped at place t of the order by value; the entries of that value -- all of them, also those
+            // that the top-k cut left out -- lie side by side in the laid-out list, in no order.  The reference orders
+            // equal values by index (Sampler.cs:245-248): the token is the one with as many smaller indices in its bin
+            // as t has places before it in the bin.
+            const int t = first >= 0 ? first : 0;
+            const int b = bmap.of_raw(sm.vals[t]);
+            const int p0 = (int)sm.boff[bin_word(b)], m = (int)sm.bhist[bin_word(b)], j = t - p0;
+            for (int e0 = 0; e0 < m; e0 += SR_WAVE) {
+                const int e = e0 + sr_lane();
+                const uint32_t mine = e < m ? sm.xc[p0 + e] : 0u;  // ~index: a smaller index is a larger word
+                int before = 0;
+                for (int q = 0; q < m; q++) before += sm.xc[p0 + q] > mine ? 1 : 0;
+                const unsigned long long is = __ballot(e < m && before == j);
+                if (is != 0ull) token = (int)(0xffffffffu - (uint32_t)__shfl((int)mine, (int)__ffsll((long long)is) - 1));
+            }
+        }
         if (sr_lane() == 0) {
-            a.out_tokens[row] = sm.idxs[first >= 0 ? first : 0];
+            a.out_tokens[row] = token;
             if (a.out_flags) a.out_flags[row] = out_flag | (amb ? SR_KFLAG_AMBIGUOUS : 0u);
         }
     }
@@ -1598,7 +1633,11 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         map.mx = __fmul_rn(sr_okey_inv(km), inv_temp);
         // the bins span what can become a candidate: from the maximum down to the bound
         const float span = __fsub_rn(map.mx, __fmul_rn(tval, inv_temp));
-        if (bins && span > 1e-3f && span < 1e30f) {
+        if (EPV == 8 && bins && ((rd.flags & kRowHasPenalty) == 0u || rd.edit_cnt <= 0) && tval > -3.0e38f &&
+            (km >> 16) - (sr_okey(tval) >> 16) < (uint32_t)kBins) {
+            map.exact = true;
+            map.ktop = km >> 16;
+        } else if (bins && span > 1e-3f && span < 1e30f) {
             map.by_bits = true;
             map.span = span;
             map.c = __fmul_rn(span, kBinOffset);

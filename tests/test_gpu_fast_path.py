@@ -442,3 +442,33 @@ def test_launches_are_ordered_behind_torch_work_on_the_default_stream(ctx):
         assert np.array_equal(got, want), attempt
         probs = ctx.build_distribution(dev, params[rows // 2:] + params[:rows // 2])
         assert float(probs.sum()) == pytest.approx(rows, rel=1e-4)
+
+
+def test_bf16_rows_of_few_distinct_values_draw_the_right_index_inside_a_run(ctx):
+    """bf16 rows that no penalty touches are ranked by value only (one bin per distinct value) and the draw's entry is
+    picked from its run of equal values by index at the end: rows of 12 to 200 distinct values, so that the top-k cut,
+    the top-p cut and the draw all fall inside runs of dozens of equal logits; also 160 rows (one worker per row with
+    its results in registers), masks, and -0 beside +0."""
+    import torch
+
+    rng = np.random.default_rng(77)
+    V = 60_000
+    for rows, n_vals in ((40, 12), (40, 200), (160, 60)):
+        levels = np.sort(rng.normal(0, 2.0, n_vals)).astype(np.float32)
+        # few entries at the top levels, many below: a run at the cut holds dozens of entries
+        pick = np.minimum((rng.exponential(0.12, (rows, V)) * n_vals).astype(np.int64), n_vals - 1)
+        logits = levels[n_vals - 1 - pick]
+        if n_vals == 12:
+            logits[0, :5000] = np.float32(-0.0)
+            logits[0, 5000:9000] = np.float32(0.0)
+        bits = synthetic.to_bf16_bits(logits)
+        up = synthetic.bf16_bits_to_f32(bits)
+        params = [SamplingParams(Temperature=float(rng.uniform(0.5, 1.6)), TopK=int(rng.integers(1, 1000)),
+                                 TopP=float(rng.choice([1.0, 0.9, 0.6])), MinP=float(rng.choice([0.0, 0.0, 0.02])))
+                  for _ in range(rows)]
+        allowed = rng.random((rows, V)) < 0.7
+        mask = pack_allow_mask(allowed)
+        active = (np.arange(rows) % 3 == 0).astype(np.uint8)
+        for rep in range(3):
+            u = rng.random(rows)
+            _check_rows(ctx, up, params, u, _cuda(bits.view(np.int16), torch.bfloat16), mask, active)
