@@ -899,7 +899,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             {
                 uint32_t* meta_w = (uint32_t*)sm.probs;
                 for (int i = tid; i < n_c; i += kThreads) {
-                    const int b = bmap.exact ? bmap.of_raw(sm.vals[i]) : bmap.of(__fmul_rn(sm.vals[i], inv_temp));
+                    const int b = (EPV == 8 && bmap.exact) ? bmap.of_raw(sm.vals[i]) : bmap.of(__fmul_rn(sm.vals[i], inv_temp));
                     meta_w[i] = ((uint32_t)b << 16) | atomicAdd(&sm.bhist[bin_word(b)], 1u);
                 }
             }
@@ -915,7 +915,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             if (n_live == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
             __syncthreads();  // sm.boff written, every wave done with the histogram
             SR_PROF(a, 6);
-            if (n_keep <= kSelMax && max_bin <= (bmap.exact ? 256 : 96)) {
+            if (n_keep <= kSelMax && max_bin <= ((EPV == 8 && bmap.exact) ? 256 : 96)) {
                 const uint32_t* meta = (const uint32_t*)sm.probs;
                 for (int i = tid; i < n_c; i += kThreads) {
                     const uint32_t mt = meta[i];
@@ -944,7 +944,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                 load_cands();  // a flat or heavily tied row: the general way below
                 bmap = BinMap{};
             }
-            exact_bins = placed && bmap.exact;
+            if constexpr (EPV == 8) exact_bins = placed && bmap.exact;
         }
         if (!placed) {
         uint32_t lmaxk = 0u;
@@ -1040,7 +1040,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             // the bin that precede it
             ranked = true;
             const int kk = min(rd.top_k, m2);
-            if (exact_bins) {
+            if (EPV == 8 && exact_bins) {
                 // every bin holds one value: the layout is the order by value already, and which of a bin's equal
                 // entries stands where makes no difference to any sum
                 for (int i = tid; i < kk; i += kThreads) {
@@ -1048,7 +1048,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
                     sm.idxs[i] = (int)(0xffffffffu - sm.xc[i]);
                 }
             }
-            for (int i = tid; i < (exact_bins ? 0 : ms); i += kThreads) {
+            for (int i = tid; i < ((EPV == 8 && exact_bins) ? 0 : ms); i += kThreads) {
                 const uint32_t mh = sm.xa[i], mm = sm.xb[i], ml = sm.xc[i];
                 const int b = bin_kept(mh);
                 const int p0 = (int)sm.boff[bin_word(b)], p1 = p0 + (int)sm.bhist[bin_word(b)];
@@ -1177,15 +1177,12 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
 
     // Sampler.cs:315-324 min-p: the first probs[t] < thr bounds the survivors
     int count = k;
-    bool amb = false;  // SR_OUT_AMBIGUOUS: a cut or the draw lies on its boundary (what wave 0's first lane knows)
     if (rd.min_p > 0.0f) {
         const float thr = __fmul_rn(rd.min_p, sm.probs[0]);
         int first = k;
         for (int t = tid; t < k; t += kThreads)
             if (sm.probs[t] < thr) { first = t; break; }
         count = min(count, block_min_i32(first, sm));
-        // the entries on either side of the cut (the list descends): on the threshold?
-        amb = (count > 0 && sr_near(sm.probs[count - 1], thr)) || (count < k && sr_near(sm.probs[count], thr));
     }
     // Sampler.cs:326-349: running sum; top-p cuts after the first cum >= TopP.  Then the draw (:351-357): the first
     // entry whose running sum reaches r = u * (sum of the kept entries).  One wave runs both searches and nothing is
@@ -1244,14 +1241,12 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         float kept_sum = 0.0f;
         const int hit = first_reach(top_p, count, &kept_sum);
         const int cnt = hit >= 0 ? hit + 1 : count;
-        if (use_top_p) amb = amb || (hit >= 0 ? sr_stop_near(kept_sum, sm.probs[hit], top_p) : sr_near(kept_sum, top_p));
         SR_PROF(a, 10);
         const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept_sum);
         float at = 0.0f;
         const int first = first_reach(r, cnt, &at);
-        amb = amb || (first >= 0 ? sr_stop_near(at, sm.probs[first], r) : sr_near(at, r));
         int token = sm.idxs[first >= 0 ? first : 0];
-        if (exact_bins) {
+        if (EPV == 8 && exact_bins) {
             // The draw stopped at place t of the order by value; the entries of that value -- all of them, also those
             // that the top-k cut left out -- lie side by side in the laid-out list, in no order.  The reference orders
             // equal values by index (Sampler.cs:245-248): the token is the one with as many smaller indices in its bin
@@ -1270,7 +1265,17 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         }
         if (sr_lane() == 0) {
             a.out_tokens[row] = token;
-            if (a.out_flags) a.out_flags[row] = out_flag | (amb ? SR_KFLAG_AMBIGUOUS : 0u);
+            if (a.out_flags) {
+                // SR_OUT_AMBIGUOUS (behind the token, for callers that ask for flags): the draw, the top-p cut or the
+                // min-p cut lies on its boundary -- the entries on either side of the min-p cut (the list descends) on
+                // the threshold, the running sum at the top-p cut or at the draw barely past its target, or the sum
+                // before it barely short of it
+                const float thr = __fmul_rn(rd.min_p, sm.probs[0]);
+                bool amb = rd.min_p > 0.0f && ((count > 0 && sr_near(sm.probs[count - 1], thr)) || (count < k && sr_near(sm.probs[count], thr)));
+                if (use_top_p) amb = amb || (hit >= 0 ? sr_stop_near(kept_sum, sm.probs[hit], top_p) : sr_near(kept_sum, top_p));
+                amb = amb || (first >= 0 ? sr_stop_near(at, sm.probs[first], r) : sr_near(at, r));
+                a.out_flags[row] = out_flag | (amb ? SR_KFLAG_AMBIGUOUS : 0u);
+            }
         }
     }
 }
