@@ -23,7 +23,7 @@ FLAGS = [
     "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-SOURCES = ["sr_api.cpp", "sr_full_host.cpp", "sr_topk.hip", "sr_argmax.hip", "sr_full.hip", "sr_sort.hip"]
+SOURCES = ["sr_api.cpp", "sr_full_host.cpp", "sr_topk.hip", "sr_argmax.hip", "sr_full.hip"]
 
 
 def _deps():

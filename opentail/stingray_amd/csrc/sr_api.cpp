@@ -313,8 +313,8 @@ void sr_destroy(sr_ctx* ctx)
     if (ctx->tmp_batch) sr_batch_destroy(ctx->tmp_batch);
     DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best, &ctx->argmax_done, &ctx->mask_pool, &ctx->mask_any,
                          &ctx->work, &ctx->edit_tab, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
-                         &ctx->full_state, &ctx->seg, &ctx->sort_k0, &ctx->sort_k1, &ctx->sort_v0,
-                         &ctx->sort_v1, &ctx->sort_tmp, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs, &ctx->spec_resid, &ctx->spec_reject};
+                         &ctx->full_state, &ctx->sort_k0, &ctx->sort_v0,
+                         &ctx->sort_v1, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs, &ctx->spec_resid, &ctx->spec_reject};
     for (DeviceBuf* b : bufs) b->release();
     ctx->uni_ring.release();
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);

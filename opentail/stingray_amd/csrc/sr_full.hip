@@ -2207,10 +2207,6 @@ __global__ __launch_bounds__(256) void k_wide_keys(SrFullArgs a)
     const uint32_t* mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
     uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
     int32_t* ids = a.sort_vals_in + (size_t)slot * a.sort_stride;
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-        a.seg_begin[slot] = (int)((size_t)slot * a.sort_stride);
-        a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + a.vocab;
-    }
     for (int i = blockIdx.x * 256 + threadIdx.x; i < a.vocab; i += gridDim.x * 256) {
         float x = load_logit<ES>(rowp, i);
         if (mrow && !((mrow[i >> 5] >> (i & 31)) & 1u)) x = SR_NEG_INF;
@@ -2226,12 +2222,15 @@ __global__ __launch_bounds__(256) void k_wide_adjust(SrFullArgs a)
     const int slot = blockIdx.y;
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
-    const uint32_t* skeys = a.sort_keys_out + (size_t)slot * a.sort_stride;
-    const int32_t* sids = a.sort_vals_out + (size_t)slot * a.sort_stride;
+    // In place: entry t of the sorted row becomes (adjusted key, t) -- the place in the first order is what the second
+    // sort breaks ties by, which makes it the stable sort that the reference's insertion is (Sampler.cs:289-294) --
+    // and its token id goes to wide_ids[t].
     uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
     int32_t* ids = a.sort_vals_in + (size_t)slot * a.sort_stride;
+    const uint32_t* skeys = keys;
+    const int32_t* sids = ids;
+    int32_t* tok = a.wide_ids + (size_t)slot * a.sort_stride;
     const int sel = wide_sel(rd, a.vocab);
-    if (blockIdx.x == 0 && threadIdx.x == 0) a.seg_end[slot] = (int)((size_t)slot * a.sort_stride) + sel;
     const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u && rd.edit_cnt > 0;
     const SrEdit* ed = a.edits + rd.edit_off;
     for (int t = blockIdx.x * 256 + threadIdx.x; t < sel; t += gridDim.x * 256) {
@@ -2258,8 +2257,21 @@ __global__ __launch_bounds__(256) void k_wide_adjust(SrFullArgs a)
             }
         }
         keys[t] = sr_okey(v);
-        ids[t] = id;
+        ids[t] = t;
+        tok[t] = id;
     }
+}
+
+// One row's (key, id) pairs sorted where they lie by the row's workgroup: descending key, ascending id among equal
+// keys.  first != 0: the whole row (ids = token indices: the order the reference's selection keeps, Sampler.cs:232-247);
+// else its first `sel` entries after the penalties (ids = places in the first order).
+__global__ __launch_bounds__(kT) void k_wide_sort(SrFullArgs a, int first)
+{
+    __shared__ FullSmem sm;
+    const int slot = blockIdx.x;
+    const SrRow rd = a.rows[a.row_list[slot]];
+    sort_survivors_in_place(a.sort_keys_in + (size_t)slot * a.sort_stride, a.sort_vals_in + (size_t)slot * a.sort_stride,
+                            first ? a.vocab : wide_sel(rd, a.vocab), sm);
 }
 
 // temperature softmax over the first k entries, min-p, top-p and the draw, all left to right (Sampler.cs:299-356)
@@ -2270,12 +2282,13 @@ __global__ __launch_bounds__(kT) void k_wide_tail(SrFullArgs a)
     const int slot = blockIdx.x;
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
-    const uint32_t* keys = a.sort_keys_out + (size_t)slot * a.sort_stride;
-    const int32_t* ids = a.sort_vals_out + (size_t)slot * a.sort_stride;
+    const uint32_t* keys = a.sort_keys_in + (size_t)slot * a.sort_stride;
+    const int32_t* pos = a.sort_vals_in + (size_t)slot * a.sort_stride;   // an entry's place in the first order ...
+    const int32_t* tok = a.wide_ids + (size_t)slot * a.sort_stride;       // ... names its token id
     float* probs = a.work + (size_t)slot * a.work_stride;
     const int k = min(rd.top_k, wide_sel(rd, a.vocab));
     const float v0 = sr_okey_inv(keys[0]);
-    const int id0 = ids[0];
+    const int id0 = tok[pos[0]];
     if (id0 < 0 || sr_f2u(v0) == 0xff800000u) {
         // nothing above -inf (Sampler.cs:254-255): Greedy over a row of -inf returns index 0
         if (tid == 0) {
@@ -2324,7 +2337,7 @@ __global__ __launch_bounds__(kT) void k_wide_tail(SrFullArgs a)
     amb = amb || (found >= 0 ? sr_stop_near(at, probs[found], r) : sr_near(at, r));
     if (tid == 0) {
         int token = id0;
-        if (found >= 0 && ids[found] >= 0) token = ids[found];
+        if (found >= 0 && tok[pos[found]] >= 0) token = tok[pos[found]];
         a.out_tokens[row] = token;
         if (a.out_flags) a.out_flags[row] = SR_KFLAG_TOPK | (amb ? SR_KFLAG_AMBIGUOUS : 0u);
     }
@@ -2674,6 +2687,11 @@ hipError_t sr_launch_wide_adjust(const SrFullArgs& a, int n_rows, hipStream_t st
 {
     if (n_rows <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_wide_adjust, dim3(32, n_rows), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+hipError_t sr_launch_wide_sort(const SrFullArgs& a, int n_rows, int first, hipStream_t st)
+{
+    hipLaunchKernelGGL(k_wide_sort, dim3((unsigned)n_rows), dim3(kT), 0, st, a, first);
     return hipGetLastError();
 }
 hipError_t sr_launch_wide_tail(const SrFullArgs& a, int n_rows, hipStream_t st)

@@ -135,7 +135,8 @@ int sr_full_rows_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, 
 }
 
 // SampleTopK (Sampler.cs:216-357) for rows whose k + history length exceeds what the selection kernel's row tail
-// sorts: two device-wide segmented sorts and a walk by one workgroup per row.
+// sorts: the row sorted where it lies by one workgroup, its first k + history-length entries adjusted and sorted
+// again, and a walk over the result by the same workgroup.
 int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows, const void* logits_dev,
                         int dtype, int64_t row_stride, int32_t* out_tokens_dev, uint32_t* out_flags_dev)
 {
@@ -159,34 +160,22 @@ int sr_wide_rows_launch(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev,
     SR_HIP(ctx, ctx->work.reserve(items * sizeof(float), st));
     a.work = ctx->work.as<float>();
     a.work_stride = stride;
-    SR_HIP(ctx, ctx->seg.reserve((size_t)n_rows * 2 * sizeof(int32_t), st));
-    a.seg_begin = ctx->seg.as<int32_t>();
-    a.seg_end = a.seg_begin + n_rows;
     SR_HIP(ctx, ctx->sort_k0.reserve(items * 4, st));
-    SR_HIP(ctx, ctx->sort_k1.reserve(items * 4, st));
     SR_HIP(ctx, ctx->sort_v0.reserve(items * 4, st));
     SR_HIP(ctx, ctx->sort_v1.reserve(items * 4, st));
     a.sort_keys_in = ctx->sort_k0.as<uint32_t>();
     a.sort_vals_in = ctx->sort_v0.as<int32_t>();
-    a.sort_keys_out = ctx->sort_k1.as<uint32_t>();
-    a.sort_vals_out = ctx->sort_v1.as<int32_t>();
+    a.wide_ids = ctx->sort_v1.as<int32_t>();
     a.sort_stride = stride;
-    size_t tmp_bytes = 0;
-    SR_HIP(ctx, sr_segmented_sort_desc(nullptr, &tmp_bytes, a.sort_keys_in, ctx->sort_k1.as<uint32_t>(), a.sort_vals_in,
-                                       ctx->sort_v1.as<int32_t>(), (int64_t)items, n_rows, a.seg_begin, a.seg_end, st));
-    SR_HIP(ctx, ctx->sort_tmp.reserve(tmp_bytes + 256, st));
     a.uniforms = b->d_uniforms.as<double>();
     a.uniforms_per_row = b->upr;
     a.out_tokens = out_tokens_dev;
     a.out_flags = out_flags_dev;
 
     SR_HIP(ctx, sr_launch_wide_keys(a, n_rows, st));
-    for (int pass = 0; pass < 2; pass++) {
-        SR_HIP(ctx, sr_segmented_sort_desc(ctx->sort_tmp.p, &tmp_bytes, a.sort_keys_in, ctx->sort_k1.as<uint32_t>(),
-                                           a.sort_vals_in, ctx->sort_v1.as<int32_t>(), (int64_t)items, n_rows, a.seg_begin,
-                                           a.seg_end, st));
-        if (pass == 0) SR_HIP(ctx, sr_launch_wide_adjust(a, n_rows, st));
-    }
+    SR_HIP(ctx, sr_launch_wide_sort(a, n_rows, 1, st));
+    SR_HIP(ctx, sr_launch_wide_adjust(a, n_rows, st));
+    SR_HIP(ctx, sr_launch_wide_sort(a, n_rows, 0, st));
     SR_HIP(ctx, sr_launch_wide_tail(a, n_rows, st));
     return SR_OK;
 }

@@ -192,7 +192,7 @@ struct sr_ctx {
     DeviceBuf stage_probs;   // staging for host-resident distributions
     DeviceBuf out_tokens, out_flags, out_val;
     HostRing uni_ring;       // uniforms of the calls that take them as host arrays and enqueue a kernel (read in place)
-    DeviceBuf seg, sort_k0, sort_k1, sort_v0, sort_v1, sort_tmp;  // device-wide sort of large nuclei
+    DeviceBuf sort_k0, sort_v0, sort_v1;  // sort segments of rows: top-p survivors, wide top-k rows (and their token ids)
     DeviceBuf ident;         // identity row list
     DeviceBuf redo_list;     // rows given to sr_resample_rows_launch
     int ident_rows = 0;

@@ -159,11 +159,8 @@ struct SrFullArgs {
     SrFullState* state;        // [slot]
     uint32_t* sort_keys_in;    // [slot][sort_stride]
     int32_t* sort_vals_in;
-    const uint32_t* sort_keys_out;
-    const int32_t* sort_vals_out;
     int64_t sort_stride;       // entries per row segment in the sort buffers
-    int32_t* seg_begin;        // [slot]
-    int32_t* seg_end;
+    int32_t* wide_ids;         // [slot][sort_stride]: wide top-k rows, the token id of every place of the first order
     const double* uniforms;
     int32_t uniforms_per_row;
     int32_t* out_tokens;       // [row], may be null in mode 1
@@ -172,10 +169,12 @@ struct SrFullArgs {
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, hipStream_t st);
-// SampleTopK by device-wide sorts (rows beyond the selection kernel's limits): keys of the whole row, the adjusted
-// first `sel` entries, the walk over the sorted result
+// SampleTopK by sorts of the whole row (rows beyond the selection kernel's limits): keys of the whole row, the row's
+// sort by its own workgroup (first != 0) or that of its adjusted first `sel` entries, the adjustment, the walk over
+// the sorted result
 hipError_t sr_launch_wide_keys(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_wide_adjust(const SrFullArgs& a, int n_rows, hipStream_t st);
+hipError_t sr_launch_wide_sort(const SrFullArgs& a, int n_rows, int first, hipStream_t st);
 hipError_t sr_launch_wide_tail(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_draw_rows(const float* probs, int64_t stride, int n, int rows, const double* u, int* out,
                                hipStream_t st);
@@ -205,9 +204,3 @@ hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int 
                                 int* out_argmax, int* out_accept, float* out_prob, hipStream_t st);
 hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum, int* out_idx,
                                      hipStream_t st);
-
-// Stable descending segmented sort of (key, index) pairs (sr_sort.hip, rocPRIM/hipCUB): the wide top-k rows.
-// With tmp == nullptr only *tmp_bytes is set.
-hipError_t sr_segmented_sort_desc(void* tmp, size_t* tmp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
-                                  const int32_t* vals_in, int32_t* vals_out, int64_t n_items, int n_segments,
-                                  const int32_t* seg_begin, const int32_t* seg_end, hipStream_t st);

@@ -2,7 +2,7 @@
 
     python -m opentail.stingray_amd.build --profile
     STINGRAY_SAMPLER_LIB=opentail/stingray_amd/lib/libstingray_sampler_prof.so \\
-        python -m opentail.stingray_amd.phase_profile [full|fp32|bf16] [rows]
+        python phase_profile.py [full|fp32|bf16] [rows]
 
 The profiling build (-DSR_PROFILE) stamps wall_clock64 (100 MHz) at the phase boundaries of every chunk item and of
 every row tail of k_topk_rows; sr_debug_set_profile hands it the array.  This prints, for one launch over the
@@ -15,6 +15,10 @@ import ctypes as C
 import sys
 
 import numpy as np
+
+import os
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 
 def main(argv):
