@@ -179,8 +179,6 @@ def load_library():
     L.sr_spec_verify_launch.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp]
     L.sr_mtp_verify_launch.argtypes = [vp, vp, i32, i32, i64, vp, C.c_float, vp, vp, vp]
     L.sr_pack_allow_mask.argtypes = [f32p, i32, u32p]
-    if hasattr(L, "sr_selftest_expf"):
-        L.sr_selftest_expf.argtypes = [vp, vp, vp, i64]
     _lib = L
     return L
 

@@ -1,6 +1,6 @@
 """Builds libstingray_sampler.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
-Usage: python -m opentail.stingray_amd.build [--force] [--profile]
+Usage: python -m opentail.stingray_amd.build [--force] [--hooks | --profile]
 """
 from __future__ import annotations
 
@@ -31,27 +31,36 @@ def _deps():
         os.path.join(HERE, "..", "..", "include", "stingray_sampler.h")]
 
 
-def _compile(src: str, force: bool, profile: bool = False) -> str:
-    obj = os.path.join(OBJ + ("_prof" if profile else ""), os.path.splitext(src)[0] + ".o")
+def _variant(profile: bool, hooks: bool) -> str:
+    return "_prof" if profile else ("_hooks" if hooks else "")
+
+
+def _compile(src: str, force: bool, profile: bool = False, hooks: bool = False) -> str:
+    obj = os.path.join(OBJ + _variant(profile, hooks), os.path.splitext(src)[0] + ".o")
     path = os.path.join(CSRC, src)
     newest = max(os.path.getmtime(p) for p in [path] + _deps())
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
         return obj
-    cmd = [HIPCC] + FLAGS + (["-DSR_PROFILE"] if profile else []) + ["-x", "hip", "-c", path, "-o", obj]
+    defs = (["-DSR_PROFILE"] if profile else []) + (["-DSR_TEST_HOOKS"] if (hooks or profile) else [])
+    cmd = [HIPCC] + FLAGS + defs + ["-x", "hip", "-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
     return obj
 
 
-def build(force: bool = False, profile: bool = False) -> str:
-    """profile=True builds libstingray_sampler_prof.so instead: the same library with the kernels' phase timestamps
-    compiled in (-DSR_PROFILE; sr_debug_set_profile).  STINGRAY_SAMPLER_LIB=<path> makes the Python mirror load it."""
-    os.makedirs(OBJ + ("_prof" if profile else ""), exist_ok=True)
+def build(force: bool = False, profile: bool = False, hooks: bool = False) -> str:
+    """The product library exports the entry points of include/stingray_sampler.h and nothing else.
+    hooks=True builds libstingray_sampler_hooks.so instead: the same sources with the test and measurement hooks of
+    include/stingray_sampler_test.h compiled in (-DSR_TEST_HOOKS); the tests call its hooks on contexts and batches of
+    the product library (tests/helpers.py).  profile=True builds libstingray_sampler_prof.so: the hooks plus the
+    kernels' phase timestamps (-DSR_PROFILE; sr_debug_set_profile).  STINGRAY_SAMPLER_LIB=<path> makes the Python
+    mirror load another build."""
+    os.makedirs(OBJ + _variant(profile, hooks), exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
-    lib = LIB.replace(".so", "_prof.so") if profile else LIB
+    lib = LIB.replace(".so", "_prof.so") if profile else (LIB.replace(".so", "_hooks.so") if hooks else LIB)
     with ThreadPoolExecutor(max_workers=4) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force, profile), SOURCES))
+        objs = list(ex.map(lambda s: _compile(s, force, profile, hooks), SOURCES))
     if force or not os.path.exists(lib) or any(os.path.getmtime(o) > os.path.getmtime(lib) for o in objs):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs
         r = subprocess.run(cmd, capture_output=True, text=True)
@@ -80,4 +89,4 @@ def build_cpp_test(oracle_lib: str) -> str:
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv, profile="--profile" in sys.argv))
+    print(build(force="--force" in sys.argv, profile="--profile" in sys.argv, hooks="--hooks" in sys.argv))

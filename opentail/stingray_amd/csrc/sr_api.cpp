@@ -1350,6 +1350,7 @@ int sr_pack_allow_mask(const float* masked_logits, int32_t vocab, uint32_t* out_
     return SR_OK;
 }
 
+#ifdef SR_TEST_HOOKS
 // ---- test and measurement hooks (include/stingray_sampler_test.h) ------------------------------------------
 
 int sr_debug_append_rebuilds(const sr_batch* b) { return b ? b->append_rebuilds : -1; }
@@ -1380,5 +1381,7 @@ int sr_selftest_expf(sr_ctx* ctx, const float* x_dev, float* y_dev, int64_t n)
     SR_HIP(ctx, sr_launch_selftest_expf(x_dev, y_dev, n, ctx->stream));
     return SR_OK;
 }
+
+#endif  // SR_TEST_HOOKS
 
 }  // extern "C"

@@ -132,11 +132,13 @@ template <int ES, bool kVec> __global__ __launch_bounds__(kThreads) void k_argma
     if (a.out_val) a.out_val[row] = a.vocab > 0 ? load_elem<ES>(rowp, idx) : 0.0f;  // the original bits, not a decode
 }
 
+#ifdef SR_TEST_HOOKS
 __global__ void k_selftest_expf(const float* x, float* y, int64_t n)
 {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) y[i] = sr_expf(x[i]);
 }
+#endif
 }  // namespace
 
 void sr_argmax_plan(SrArgmaxArgs& a, int cu_count)
@@ -189,9 +191,11 @@ hipError_t sr_argmax_static_scratch(int device, unsigned long long** best, uint3
     return hipSuccess;
 }
 
+#ifdef SR_TEST_HOOKS
 hipError_t sr_launch_selftest_expf(const float* x, float* y, int64_t n, hipStream_t stream)
 {
     if (n <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_selftest_expf, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, y, n);
     return hipGetLastError();
 }
+#endif

@@ -2638,6 +2638,7 @@ __global__ __launch_bounds__(kT) void k_mtp_verify(const float* logits, int64_t 
     }
 }
 
+#ifdef SR_TEST_HOOKS
 __global__ __launch_bounds__(kT) void k_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum,
                                                          int* out_idx)
 {
@@ -2650,6 +2651,7 @@ __global__ __launch_bounds__(kT) void k_selftest_seqsum(const float* x, int n, f
         s = seq_sum_row<false>(x, n, s0, 0.0f, &found, sm);
     if (threadIdx.x == 0) { *out_sum = s; *out_idx = found; }
 }
+#endif
 
 }  // namespace
 
@@ -2748,9 +2750,11 @@ hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int 
                        out_accept, out_prob);
     return hipGetLastError();
 }
+#ifdef SR_TEST_HOOKS
 hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum, int* out_idx,
                                      hipStream_t st)
 {
     hipLaunchKernelGGL(k_selftest_seqsum, dim3(1), dim3(kT), 0, st, x, n, s0, target, out_sum, out_idx);
     return hipGetLastError();
 }
+#endif

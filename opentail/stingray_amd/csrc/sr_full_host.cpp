@@ -468,6 +468,7 @@ int sr_mtp_verify_launch(sr_ctx* ctx, const float* logits_dev, int32_t rows, int
     return SR_OK;
 }
 
+#ifdef SR_TEST_HOOKS
 // Test hook (include/stingray_sampler_test.h): exact left-to-right sum of x_dev[0..n) from s0
 int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float s0, float target, float* out_sum_dev,
                               int32_t* out_idx_dev)
@@ -477,5 +478,6 @@ int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float s0, flo
     SR_HIP(ctx, sr_launch_selftest_seqsum(x_dev, n, s0, target, out_sum_dev, out_idx_dev, ctx->stream));
     return SR_OK;
 }
+#endif  // SR_TEST_HOOKS
 
 }  // extern "C"

@@ -21,6 +21,35 @@ def oracle_tokens(logits: np.ndarray, params, uniforms, allow_mask=None, mask_ac
                             allow_mask, mask_active)
 
 
+_hooks = None
+
+
+def hooks_lib():
+    """libstingray_sampler_hooks.so: the library once more with the test and measurement hooks of
+    include/stingray_sampler_test.h compiled in (the product library exports none of them).  Its hooks are called on
+    contexts and batches of the product library -- both are built from the same sources, so a hook that sets a field of a
+    context or launches a routine on its stream works on either's."""
+    global _hooks
+    if _hooks is None:
+        import ctypes as C
+        import os
+
+        import opentail.stingray_amd as sa
+
+        sa.load_library()  # (the product library, and with it torch's HIP runtime, first)
+        path = sa.lib_path().replace("libstingray_sampler.so", "libstingray_sampler_hooks.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python -m opentail.stingray_amd.build --hooks`")
+        H = C.CDLL(path)
+        vp = C.c_void_p
+        H.sr_selftest_expf.argtypes = [vp, vp, vp, C.c_int64]
+        H.sr_selftest_seqsum.argtypes = [vp, vp, C.c_int32, C.c_float, C.c_float, vp, vp]
+        H.sr_debug_append_rebuilds.argtypes = [vp]
+        H.sr_debug_set_spin_limit.argtypes = [vp, C.c_uint32]
+        _hooks = H
+    return _hooks
+
+
 class ReplayRandom:
     """Stands in for System.Random: hands out the given NextDouble() values and counts the draws."""
 

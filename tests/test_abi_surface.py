@@ -18,11 +18,14 @@ def _test_hook_symbols():
     return sorted(set(re.findall(r"SR_API\s+[\w\s\*]+?\b(sr_\w+)\s*\(", text)))
 
 
-def test_the_test_hooks_are_declared_apart_from_the_product_interface_and_exported():
+def test_the_test_hooks_are_declared_apart_and_exported_by_the_hooks_build_only():
     hooks = _test_hook_symbols()
     assert hooks and not set(hooks) & set(_declared_symbols())
     lib = ctypes.CDLL(sa.lib_path())
-    assert not [s for s in hooks if not hasattr(lib, s)]
+    assert not [s for s in hooks if hasattr(lib, s)], "the product library ships a test hook"
+    with_hooks = ctypes.CDLL(sa.lib_path().replace("libstingray_sampler.so", "libstingray_sampler_hooks.so"))
+    assert not [s for s in hooks if not hasattr(with_hooks, s)]
+    assert not [s for s in _declared_symbols() if not hasattr(with_hooks, s)]
 
 
 def test_header_and_python_symbol_lists_agree():

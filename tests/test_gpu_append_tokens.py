@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from opentail.stingray_amd import SamplerContext, SamplingParams, pack_allow_mask
-from tests.helpers import oracle_tokens
+from tests.helpers import hooks_lib, oracle_tokens
 
 pytestmark = pytest.mark.gpu
 
@@ -65,8 +65,7 @@ def _peaked_logits(rng, rows, vocab, hot):
 def _rebuilds(ctx, batch):
     import ctypes as C
 
-    ctx.L.sr_debug_append_rebuilds.argtypes = [C.c_void_p]
-    return int(ctx.L.sr_debug_append_rebuilds(batch.h))
+    return int(hooks_lib().sr_debug_append_rebuilds(batch.h))
 
 
 @pytest.mark.parametrize("vocab,dtype_bf16,pad,in_place_only",

@@ -7,7 +7,7 @@ import pytest
 
 from oracle import binding as orc
 from opentail.stingray_amd import Sampler, SamplerContext, SamplingParams, pack_allow_mask, synthetic
-from tests.helpers import DotnetRandom, ReplayRandom, oracle_tokens
+from tests.helpers import DotnetRandom, ReplayRandom, hooks_lib, oracle_tokens
 
 pytestmark = pytest.mark.gpu
 NEG_INF = np.float32("-inf")
@@ -39,7 +39,7 @@ def test_device_expf_is_bit_identical_to_the_oracle(ctx):
     ]).astype(np.float32)
     x = _cuda(xs)
     y = torch.empty_like(x)
-    ctx._check(ctx.L.sr_selftest_expf(ctx.h, C.c_void_p(x.data_ptr()), C.c_void_p(y.data_ptr()), xs.size))
+    ctx._check(hooks_lib().sr_selftest_expf(ctx.h, C.c_void_p(x.data_ptr()), C.c_void_p(y.data_ptr()), xs.size))
     ctx.synchronize()
     got = y.cpu().numpy()
     lib = orc.lib()

@@ -8,7 +8,7 @@ import pytest
 
 from oracle import binding as orc
 from opentail.stingray_amd import Sampler, SamplerContext, SamplingParams, pack_allow_mask, synthetic
-from tests.helpers import DotnetRandom, ReplayRandom, oracle_tokens, to_oracle
+from tests.helpers import DotnetRandom, ReplayRandom, hooks_lib, oracle_tokens, to_oracle
 
 pytestmark = pytest.mark.gpu
 NEG_INF = np.float32("-inf")
@@ -17,7 +17,6 @@ NEG_INF = np.float32("-inf")
 @pytest.fixture(scope="module")
 def ctx():
     c = SamplerContext(0)
-    c.L.sr_selftest_seqsum.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_void_p]
     yield c
     c.close()
 
@@ -34,7 +33,7 @@ def _gpu_seq_sum(ctx, x, s0=0.0, target=float("nan")):
     xd = _cuda(np.asarray(x, dtype=np.float32))
     s = torch.zeros(1, dtype=torch.float32, device="cuda")
     idx = torch.zeros(1, dtype=torch.int32, device="cuda")
-    ctx._check(ctx.L.sr_selftest_seqsum(ctx.h, C.c_void_p(xd.data_ptr()), len(x), s0, target,
+    ctx._check(hooks_lib().sr_selftest_seqsum(ctx.h, C.c_void_p(xd.data_ptr()), len(x), s0, target,
                                         C.c_void_p(s.data_ptr()), C.c_void_p(idx.data_ptr())))
     ctx.synchronize()
     return np.float32(s.cpu().numpy()[0]), int(idx.cpu().numpy()[0])

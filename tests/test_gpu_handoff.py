@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 from opentail.stingray_amd import SamplerContext, SamplingParams, pack_allow_mask, synthetic
-from tests.helpers import oracle_tokens
+from tests.helpers import hooks_lib, oracle_tokens
 
 pytestmark = pytest.mark.gpu
 UNSUPPORTED = np.uint32(1 << 31)
@@ -19,7 +19,6 @@ UNSUPPORTED = np.uint32(1 << 31)
 @pytest.fixture()
 def ctx():
     c = SamplerContext(0)
-    c.L.sr_debug_set_spin_limit.argtypes = [C.c_void_p, C.c_uint32]
     yield c
     c.close()
 
@@ -83,13 +82,13 @@ def test_rows_selected_from_the_logits_alone_give_the_same_tokens_and_launches_d
     got, flags = _launch(ctx, batch, dev, rows)
     assert np.array_equal(got, want)
     # no tail waits for its row's other chunks: every row by the exact fallback, while the chunks still count themselves in
-    ctx._check(ctx.L.sr_debug_set_spin_limit(ctx.h, 0))
+    ctx._check(hooks_lib().sr_debug_set_spin_limit(ctx.h, 0))
     for _ in range(3):
         got, flags = _launch(ctx, batch, dev, rows)
         assert np.array_equal(got, want), np.nonzero(got != want)[0]
         assert not np.any(flags & UNSUPPORTED)
     # back to waiting: the counters of the launches before must not be seen
-    ctx._check(ctx.L.sr_debug_set_spin_limit(ctx.h, 1 << 22))
+    ctx._check(hooks_lib().sr_debug_set_spin_limit(ctx.h, 1 << 22))
     for _ in range(3):
         u = rng.random(rows)
         batch.set_uniforms(u)

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from opentail.stingray_amd import SamplerContext, SamplingParams, pack_allow_mask, synthetic
-from tests.helpers import oracle_tokens
+from tests.helpers import hooks_lib, oracle_tokens
 
 pytestmark = pytest.mark.gpu
 
@@ -164,8 +164,7 @@ def test_constrained_decode_loop_over_registered_states(ctx, vocab, rows, steps)
         u = rng.random(rows)
         batch.append_tokens(tokens, u, mask_ids=[ids[s] if s >= 0 else -1 for s in state])
     # the steps were taken in place: only a row that ran out of room for new history ids rebuilds the batch
-    ctx.L.sr_debug_append_rebuilds.argtypes = [C.c_void_p]
-    assert int(ctx.L.sr_debug_append_rebuilds(batch.h)) <= steps // 8
+    assert int(hooks_lib().sr_debug_append_rebuilds(batch.h)) <= steps // 8
     batch.close()
     for i in ids:
         ctx.release_mask(i)
