@@ -26,6 +26,8 @@ SR_API int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float 
 
 /* How many sr_batch_append_tokens calls on this batch rebuilt it instead of updating it in place. */
 SR_API int sr_debug_append_rebuilds(const sr_batch* batch);
+/* ... and how many rows such calls moved to the end of the batch's edit array because they had run out of room. */
+SR_API int sr_debug_append_moves(const sr_batch* batch);
 
 /* How often a row tail of the selection kernel polls its row's counter before it stops waiting for the row's other
  * chunks and selects the row from its logits alone, the way a row whose candidates overflow the kernel's lists is

@@ -776,7 +776,7 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
             if (d.scan_row >= 0 && (b->h_scan_need[(size_t)r] & SR_SCAN_ALLOW)) scan_again.push_back(d.scan_row);
         }
         if (tokens[r] < 0) {
-            if (mask_changed) rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel});
+            if (mask_changed) rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel, d.edit_off});
             continue;
         }
         const sr_row_params& p = b->keep_params[(size_t)r];
@@ -784,7 +784,7 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
         const int32_t n_new = (int32_t)hist.size(), n_old = n_new - 1;
         if (!has_history_penalty(p)) {  // the history is never looked at
             d.n_prev = n_new;
-            rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel});
+            rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel, d.edit_off});
             continue;
         }
         if (n_old == 0 || d.edit_cnt == 0 || d.path == SR_PATH_TOPK_WIDE) {
@@ -821,10 +821,31 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
             int32_t k = find(t);
             if (k < 0) {
                 const bool topk = d.path == SR_PATH_TOPK;
-                if (d.edit_cnt >= b->edit_cap[(size_t)r] || d.edit_cnt + 1 > SR_TK_SEL_MAX ||
-                    (topk && (int64_t)p.top_k + d.edit_cnt + 1 > SR_TK_SEL_MAX)) {
-                    rebuild = true;
+                if (d.edit_cnt + 1 > SR_TK_SEL_MAX || (topk && (int64_t)p.top_k + d.edit_cnt + 1 > SR_TK_SEL_MAX)) {
+                    rebuild = true;  // (the row leaves the selection kernel's limits: another path)
                     break;
+                }
+                if (d.edit_cnt >= b->edit_cap[(size_t)r]) {
+                    // No room behind the row's edits: the row moves to the end of the array, with room for as many again,
+                    // and all its edits are sent -- a patch like any other.  Only when the device array itself has no room
+                    // left (it was made for four times what the upload needed) is the batch rebuilt, which packs it again.
+                    const int32_t new_cap = std::max(2 * b->edit_cap[(size_t)r], d.edit_cnt + SR_EDIT_SLACK);
+                    const size_t new_off = b->h_edits.size();
+                    if ((new_off + (size_t)new_cap) * sizeof(SrEdit) > b->d_edits.cap || new_off + (size_t)new_cap > 0x7fffffffull) {
+                        rebuild = true;
+                        break;
+                    }
+                    b->h_edits.resize(new_off + (size_t)new_cap);
+                    b->edit_ids.resize(new_off + (size_t)new_cap, 0);
+                    std::copy(b->h_edits.begin() + d.edit_off, b->h_edits.begin() + d.edit_off + d.edit_cnt, b->h_edits.begin() + (ptrdiff_t)new_off);
+                    std::copy(b->edit_ids.begin() + d.edit_off, b->edit_ids.begin() + d.edit_off + d.edit_cnt, b->edit_ids.begin() + (ptrdiff_t)new_off);
+                    d.edit_off = (int32_t)new_off;
+                    b->edit_cap[(size_t)r] = new_cap;
+                    ed = b->h_edits.data() + d.edit_off;
+                    eids = b->edit_ids.data() + d.edit_off;
+                    touched.clear();
+                    for (int32_t j = 0; j < d.edit_cnt; j++) touched.push_back(j);
+                    b->append_moves++;
                 }
                 if (sorted) {
                     // the edits stay in order of their ids (a kernel searches them): the new one goes where it
@@ -858,7 +879,7 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
             d.sel = (int32_t)sel;
             b->max_sel = std::max(b->max_sel, d.sel);
         }
-        rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel});
+        rp.push_back(SrRowPatch{r, d.n_prev, d.edit_cnt, d.mask_row, d.sel, d.edit_off});
         std::sort(touched.begin(), touched.end());
         touched.erase(std::unique(touched.begin(), touched.end()), touched.end());
         for (int32_t k : touched) ep.push_back(SrEditPatch{d.edit_off + k, ed[k]});
@@ -1354,6 +1375,7 @@ int sr_pack_allow_mask(const float* masked_logits, int32_t vocab, uint32_t* out_
 // ---- test and measurement hooks (include/stingray_sampler_test.h) ------------------------------------------
 
 int sr_debug_append_rebuilds(const sr_batch* b) { return b ? b->append_rebuilds : -1; }
+int sr_debug_append_moves(const sr_batch* b) { return b ? b->append_moves : -1; }
 
 int sr_debug_set_spin_limit(sr_ctx* ctx, uint32_t polls)
 {

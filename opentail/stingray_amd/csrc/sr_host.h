@@ -255,6 +255,7 @@ struct sr_batch {
     // they came; the histories are split per row by the first append) and the room each row's edit range has.
     bool can_append = false, hist_split = false;
     int32_t append_rebuilds = 0;  // calls of sr_batch_append_tokens that rebuilt the batch (test hook)
+    int32_t append_moves = 0;     // ... rows that were moved to the end of the edit array instead
     std::vector<sr_row_params> keep_params;
     std::vector<int32_t> keep_hist_ids, keep_hist_off, keep_bias_ids, keep_bias_off;
     std::vector<float> keep_bias_vals;

@@ -2155,6 +2155,7 @@ __global__ __launch_bounds__(256) void k_apply_patches(SrRow* rows, const SrRowP
         rows[r.row].edit_cnt = r.edit_cnt;
         rows[r.row].mask_row = r.mask_row;
         rows[r.row].sel = r.sel;
+        rows[r.row].edit_off = r.edit_off;
     }
     if (i < n_edits) edits[e.index] = e.edit;
     if (i < n_clears) {

@@ -64,6 +64,7 @@ struct SrRowPatch {
     int32_t edit_cnt;
     int32_t mask_row;  // the row's allow-mask from now on (-1 none); rows of batches without registered masks keep theirs
     int32_t sel;
+    int32_t edit_off;  // where the row's edits lie from now on (a row that ran out of room moves to the array's end)
 };
 struct SrMaskClear {
     int32_t scan_row;

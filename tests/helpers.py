@@ -45,6 +45,7 @@ def hooks_lib():
         H.sr_selftest_expf.argtypes = [vp, vp, vp, C.c_int64]
         H.sr_selftest_seqsum.argtypes = [vp, vp, C.c_int32, C.c_float, C.c_float, vp, vp]
         H.sr_debug_append_rebuilds.argtypes = [vp]
+        H.sr_debug_append_moves.argtypes = [vp]
         H.sr_debug_set_spin_limit.argtypes = [vp, C.c_uint32]
         _hooks = H
     return _hooks

@@ -128,9 +128,10 @@ def test_decode_loop_with_appended_tokens_matches_oracle_and_fresh_upload(ctx, v
         for r in range(rows):
             if app[r] >= 0:
                 hists[r].append(int(app[r]))
-    n_rebuilt = _rebuilds(ctx, inc)
-    # only a row that ran out of room (or got its first history token) rebuilds: most calls must have been in place
-    assert n_rebuilt <= steps // 4, n_rebuilt
+    n_rebuilt, n_moved = _rebuilds(ctx, inc), int(hooks_lib().sr_debug_append_moves(inc.h))
+    # a row that runs out of room moves to the end of the edit array; only a row's first history token (or a change of
+    # path) rebuilds the batch
+    assert n_rebuilt <= (0 if in_place_only else 4), (n_rebuilt, n_moved)
     inc.close()
 
 
@@ -160,7 +161,8 @@ def test_append_before_the_first_launch_and_new_ids_every_step(ctx):
         ctx.sample_launch(b, torch.from_numpy(lg).cuda(), toks)
         ctx.synchronize()
         assert toks.cpu().numpy().tolist() == oracle_tokens(lg, now, u).tolist(), f"step {step}"
-    assert 1 <= _rebuilds(ctx, b) <= 4  # 40 unseen ids per row, room for 32 and more between rebuilds
+    # 40 unseen ids per row, room for 32: every row has moved to the end of the edit array once, none rebuilt the batch
+    assert _rebuilds(ctx, b) == 0 and int(hooks_lib().sr_debug_append_moves(b.h)) >= 6
     b.close()
 
 
@@ -206,5 +208,7 @@ def test_histories_that_outgrow_the_pinned_staging_memory_of_their_batch(ctx):
             ctx.synchronize()
             torch.cuda.synchronize()
             assert np.array_equal(toks.cpu().numpy(), oracle_tokens(logits, params, u)), step
-    assert _rebuilds(ctx, batch) >= 2
+    # rows move to the end of the edit array as they run out of room, until the device array (made for four times what
+    # the upload needed) is full and the batch is rebuilt, which packs it again
+    assert _rebuilds(ctx, batch) >= 1 and int(hooks_lib().sr_debug_append_moves(batch.h)) >= rows
     batch.close()
