@@ -25,6 +25,7 @@ namespace {
 constexpr int kT = SR_SEQ_THREADS;
 constexpr int kW = SR_SEQ_WAVES;
 constexpr int kSmall = SR_FULL_SMALL_CAP;  // survivors sorted inside the kernel
+constexpr int kCkpt = 128;                 // tiles of a row whose running sums are kept for the search that follows
 
 struct FullSmem {
     SrSeqSmem seq;
@@ -35,6 +36,7 @@ struct FullSmem {
     int redi[kW];
     uint32_t hist[256];
     uint32_t bc[16];
+    float ckpt[kCkpt];  // running sum behind every tile of a row's exact sum (SeqMarks)
     unsigned long long sortbuf[kSmall];
     float sprob[kSmall];
     uint32_t tags[kSmall];
@@ -178,18 +180,40 @@ __device__ __forceinline__ float seq_sum(Term term, int n, float s0, float targe
 //   issue_fast(base, raw)  starts the loads of the whole tile whose first term is `base`, no conditions
 //   issue_any(base, raw)   the same for any tile of any row (ragged end, unaligned row)
 //   finish(raw, x)         the tile's terms from what was loaded
+//
+// A sum that is followed by a search over the same terms (residual resampling: Sampler.cs:594-614) leaves marks: the
+// running sum behind every tile (SeqMarks::keep, rows of at most kCkpt tiles).  The running sum never decreases, so
+// the search's answer lies in the first tile whose mark has reached the target, and the state in front of that tile is
+// the mark before it: the search starts there (SeqMarks::from) instead of at the row's first term, and reads one
+// tile instead of, on average, half the row.
+struct SeqMarks {
+    float* keep = nullptr;  // a sum writes the running sum behind tile t to keep[t]
+    int from = 0;           // first tile that is looked at; s0 is the running sum in front of it
+};
+__device__ __forceinline__ bool seq_marks_fit(int n) { return (n + SR_SEQ_TILE - 1) / SR_SEQ_TILE <= kCkpt; }
+// the tile at which a search for `target` over the marked row starts, and the running sum in front of it (*s0); behind a
+// barrier that follows the sum
+__device__ __forceinline__ int seq_marks_find(const float* marks, int n, float target, float* s0)
+{
+    const int tiles = (n + SR_SEQ_TILE - 1) / SR_SEQ_TILE;
+    int t = 0;
+    while (t < tiles - 1 && !(marks[t] >= target)) t++;
+    *s0 = t > 0 ? marks[t - 1] : 0.0f;
+    return t;
+}
 template <bool kSearch, int kDepth, typename Raw, typename IssueFast, typename IssueAny, typename Finish>
 __device__ __forceinline__ float seq_sum_tiles(IssueFast issue_fast, IssueAny issue_any, Finish finish, bool fast_ok, int n,
-                                               float s0, float target, int* found, FullSmem& sm)
+                                               float s0, float target, int* found, FullSmem& sm, SeqMarks marks = SeqMarks())
 {
     float s = s0;
     *found = -1;
     const int n_full = fast_ok ? n / SR_SEQ_TILE : 0;  // whole tiles, taken by the pipelined loop
-    if (n_full > 0) {
+    const int tb = marks.from;
+    if (n_full > tb) {
         Raw r[kDepth];
 #pragma unroll
-        for (int k = 0; k < kDepth - 1; k++) issue_fast(min(k, n_full - 1) * SR_SEQ_TILE, r[k]);
-        for (int t0 = 0; t0 < n_full; t0 += kDepth) {
+        for (int k = 0; k < kDepth - 1; k++) issue_fast(min(tb + k, n_full - 1) * SR_SEQ_TILE, r[k]);
+        for (int t0 = tb; t0 < n_full; t0 += kDepth) {
 #pragma unroll
             for (int k = 0; k < kDepth; k++) {
                 const int t = t0 + k;
@@ -203,10 +227,11 @@ __device__ __forceinline__ float seq_sum_tiles(IssueFast issue_fast, IssueAny is
                     *found = t * SR_SEQ_TILE + f;
                     return s;
                 }
+                if (!kSearch && marks.keep && threadIdx.x == 0) marks.keep[t] = s;
             }
         }
     }
-    for (int base = n_full * SR_SEQ_TILE; base < n; base += SR_SEQ_TILE) {
+    for (int base = max(n_full, tb) * SR_SEQ_TILE; base < n; base += SR_SEQ_TILE) {
         Raw r;
         issue_any(base, r);
         float x[SR_SEQ_RUN];
@@ -217,6 +242,7 @@ __device__ __forceinline__ float seq_sum_tiles(IssueFast issue_fast, IssueAny is
             *found = base + f;
             return s;
         }
+        if (!kSearch && marks.keep && threadIdx.x == 0) marks.keep[base / SR_SEQ_TILE] = s;
     }
     return s;
 }
@@ -260,7 +286,8 @@ struct SeqNoMap {
 // map(x, i) stands between a scaled term and the sum: the term that is added (and watched) is what it returns
 template <bool kSearch, typename Watch = SeqNoWatch, typename Map = SeqNoMap>
 __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, float target, int* found, FullSmem& sm,
-                                             float m1 = 1.0f, float m2 = 1.0f, Watch watch = Watch(), Map map = Map())
+                                             float m1 = 1.0f, float m2 = 1.0f, Watch watch = Watch(), Map map = Map(),
+                                             SeqMarks marks = SeqMarks())
 {
     static_assert(SR_SEQ_ACTIVE == SR_SEQ_THREADS, "every thread of the block loads a run");
     const bool aligned = ((uintptr_t)p & 15u) == 0u;
@@ -277,13 +304,13 @@ __device__ __forceinline__ float seq_sum_row(const float* p, int n, float s0, fl
             watch(x[j], base + (int)threadIdx.x * SR_SEQ_RUN + j);
         }
     };
-    return seq_sum_tiles<kSearch, 3, SeqRaw1>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm);
+    return seq_sum_tiles<kSearch, 3, SeqRaw1>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm, marks);
 }
 
 // ... and over the positive part of the difference of two rows (residual resampling)
 template <bool kSearch>
 __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q, int n, float s0, float target, int* found,
-                                                  FullSmem& sm, float m1 = 1.0f, float m2 = 1.0f)
+                                                  FullSmem& sm, float m1 = 1.0f, float m2 = 1.0f, SeqMarks marks = SeqMarks())
 {
     const bool aligned = (((uintptr_t)p | (uintptr_t)q) & 15u) == 0u;
     auto issue_fast = [&](int base, SeqRaw2& r) __attribute__((always_inline)) {
@@ -303,7 +330,7 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
             x[j] = d > 0.0f ? d : 0.0f;
         }
     };
-    return seq_sum_tiles<kSearch, 2, SeqRaw2>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm);
+    return seq_sum_tiles<kSearch, 2, SeqRaw2>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm, marks);
 }
 
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
@@ -2363,7 +2390,9 @@ __device__ __forceinline__ int resample_residual_row(const float* p, const float
         const float r = __fsub_rn(__fmul_rn(__fmul_rn(p[i], m1), m2), q[i]);
         return r > 0.0f ? r : 0.0f;
     };
-    const float sum = seq_sum_residual<false>(p, q, n, 0.0f, 0.0f, &dummy, sm, m1, m2);
+    SeqMarks marks;
+    if (seq_marks_fit(n)) marks.keep = sm.ckpt;
+    const float sum = seq_sum_residual<false>(p, q, n, 0.0f, 0.0f, &dummy, sm, m1, m2, marks);
     if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm, m1, m2);  // sum <= 0 or NaN
     const float target = __fmul_rn(__double2float_rn(u), sum);
     // `target <= cum` is only tested on positive residuals: a zero target must not stop on a zero term
@@ -2381,7 +2410,13 @@ __device__ __forceinline__ int resample_residual_row(const float* p, const float
         __syncthreads();
         return f;  // sum > 0 guarantees a positive residual exists
     }
-    seq_sum_residual<true>(p, q, n, 0.0f, target, &found, sm, m1, m2);
+    float s0 = 0.0f;
+    SeqMarks from;
+    if (marks.keep) {
+        __syncthreads();  // (the marks were written by thread 0)
+        from.from = seq_marks_find(sm.ckpt, n, target, &s0);
+    }
+    seq_sum_residual<true>(p, q, n, s0, target, &found, sm, m1, m2, from);
     if (found >= 0) return found;
     // rounding fallback: the last index with a positive residual
     int last = -1;
@@ -2412,7 +2447,9 @@ __device__ __forceinline__ int resample_residual_stored(const float* res, const 
                                                         float m1, float m2)
 {
     int dummy;
-    const float sum = seq_sum_row<false>(res, n, 0.0f, 0.0f, &dummy, sm);
+    SeqMarks marks;
+    if (seq_marks_fit(n)) marks.keep = sm.ckpt;
+    const float sum = seq_sum_row<false>(res, n, 0.0f, 0.0f, &dummy, sm, 1.0f, 1.0f, SeqNoWatch(), SeqNoMap(), marks);
     if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm, m1, m2);  // sum <= 0 or NaN
     const float target = __fmul_rn(__double2float_rn(u), sum);
     auto edge = [&](bool first_one) -> int {  // the first / the last index with a positive residual
@@ -2433,7 +2470,13 @@ __device__ __forceinline__ int resample_residual_stored(const float* res, const 
     };
     if (target <= 0.0f) return edge(true);  // a zero target must not stop on a zero term
     int found;
-    seq_sum_row<true>(res, n, 0.0f, target, &found, sm);
+    float s0 = 0.0f;
+    SeqMarks from;
+    if (marks.keep) {
+        __syncthreads();  // (the marks were written by thread 0)
+        from.from = seq_marks_find(sm.ckpt, n, target, &s0);
+    }
+    seq_sum_row<true>(res, n, s0, target, &found, sm, 1.0f, 1.0f, SeqNoWatch(), SeqNoMap(), from);
     return found >= 0 ? found : edge(false);  // (rounding: the sum of the search fell short of the target)
 }
 
