@@ -171,6 +171,19 @@ __device__ __forceinline__ unsigned long long sr_wave_max_u64(unsigned long long
     }
     return r;
 }
+// inclusive prefix sum across the wave, single precision (the order of the additions is the scan's own)
+__device__ __forceinline__ float sr_wave_incl_sum_f32(float v)
+{
+    v += __uint_as_float(sr_dpp_u32<0x111>(__float_as_uint(v)));
+    v += __uint_as_float(sr_dpp_u32<0x112>(__float_as_uint(v)));
+    v += __uint_as_float(sr_dpp_u32<0x114>(__float_as_uint(v)));
+    v += __uint_as_float(sr_dpp_u32<0x118>(__float_as_uint(v)));
+    const float r0 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 15));
+    const float r1 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 31));
+    const float r2 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 47));
+    const int row = (int)(threadIdx.x & 63u) >> 4;
+    return v + ((row >= 1 ? r0 : 0.0f) + (row >= 2 ? r1 : 0.0f) + (row >= 3 ? r2 : 0.0f));
+}
 // inclusive prefix sum across the wave
 __device__ __forceinline__ int sr_wave_incl_scan_i32(int v)
 {

@@ -25,6 +25,7 @@ namespace {
 constexpr int kT = SR_SEQ_THREADS;
 constexpr int kW = SR_SEQ_WAVES;
 constexpr int kSmall = SR_FULL_SMALL_CAP;  // survivors sorted inside the kernel
+constexpr int kTagIndexBits = 19;          // a find's tag in the walk by slabs: rank << 19 | index
 constexpr int kCkpt = 128;                 // tiles of a row whose running sums are kept for the search that follows
 
 struct FullSmem {
@@ -37,6 +38,8 @@ struct FullSmem {
     uint32_t hist[256];
     uint32_t bc[16];
     float ckpt[kCkpt];  // running sum behind every tile of a row's exact sum (SeqMarks)
+    float segst[SR_SEG_MAX];  // running sum behind every segment of a prepared row (seg_walk)
+    uint32_t segbc[4];
     unsigned long long sortbuf[kSmall];
     float sprob[kSmall];
     uint32_t tags[kSmall];
@@ -331,6 +334,217 @@ __device__ __forceinline__ float seq_sum_residual(const float* p, const float* q
         }
     };
     return seq_sum_tiles<kSearch, 2, SeqRaw2>(issue_fast, issue_any, finish, aligned, n, s0, target, found, sm, marks);
+}
+
+// ---- exact sums prepared by the whole device ---------------------------------------------------------------
+// One workgroup adds a row at the rate at which one compute unit reads and scans it (1 MB in ~45 us).  Where the terms
+// lie in memory before that workgroup starts, the whole device prepares the sum: the row is cut into segments of
+// SR_SEG_TERMS terms, a first kernel leaves an approximate sum of every segment (double precision, any order), and
+// k_seq_funcs turns every segment into its increment function n -> n + a[n & 1] (sr_seqsum.h) for the binade that the
+// approximate prefix predicts for the segment's start.  The workgroup that needs the sum then only walks the
+// functions (seg_walk, one wave): a function is applied when the exact running sum in front of its segment lies in the
+// binade it was made for and stays there; any other segment -- one in which the sum changes binade (a sum that starts
+// at zero does that ~17 times, mostly within the first segments), a prediction that missed -- is added from its terms
+// by the wave's own exact scan (sr_seq_wave).  The result never depends on the prediction: only the time does.
+__device__ __forceinline__ int seg_count(int n) { return (n + SR_SEG_TERMS - 1) / SR_SEG_TERMS; }
+static_assert(SR_SEG_TERMS == SR_WAVE * SR_SEQ_RUN && sizeof(SeqSegFunc) == 96, "one run of 16 terms per lane; six 16-byte loads per record");
+
+struct SegRec {
+    uint4 f, g, x0, x1, x2, x3;
+};
+__device__ __forceinline__ void seg_load_rec(const SeqSegFunc* funcs, int seg, int nseg, SegRec& r)
+{
+    const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+    r.f = r.g = r.x0 = r.x1 = r.x2 = r.x3 = z;
+    if (seg < nseg) {
+        const uint4* q = (const uint4*)(funcs + seg);
+        r.f = q[0]; r.g = q[1]; r.x0 = q[2]; r.x1 = q[3]; r.x2 = q[4]; r.x3 = q[5];
+    }
+}
+
+// The exact running sum over terms[0, n) from s0, by the 64 lanes of ONE wave.  With kSearch it stops at the first term at
+// which the running sum reaches `target`: *found = its index and the returned value is the running sum at that term.
+// With `states` (not with kSearch) the running sum behind segment g is left at states[g].
+template <bool kSearch>
+__device__ __forceinline__ float seg_walk(const float* terms, int n, const SeqSegFunc* funcs, float s0, float target, int* found,
+                                          float* states)
+{
+    const int lane = sr_lane();
+    const int nseg = seg_count(n);
+    const bool aligned = ((uintptr_t)terms & 15u) == 0u;
+    float s = s0;
+    *found = -1;
+    SegRec next;
+    seg_load_rec(funcs, lane, nseg, next);
+    for (int base = 0; base < nseg; base += SR_WAVE) {
+        const int seg = base + lane;
+        const bool have = seg < nseg;
+        const SegRec r = next;
+        seg_load_rec(funcs, seg + SR_WAVE, nseg, next);  // (the records of the next 64 segments come in meanwhile)
+        const uint32_t kind = r.f.w & 0xffu;
+        int lstart = 0;  // the segments of the lanes below are settled
+        for (;;) {
+            uint32_t n_in;
+            int eb;
+            sr_split(s, &n_in, &eb);
+            SrInc m;
+            m.a0 = 0u; m.a1 = 0u;
+            if (have && lane >= lstart) {
+                if (kind == SR_SEG_PLAIN && (int)r.f.z == eb) { m.a0 = r.f.x; m.a1 = r.f.y; }
+                else { m.a0 = SR_SEQ_SAT; m.a1 = SR_SEQ_SAT; }  // made for another binade, or not one function
+            }
+            const SrInc sc = sr_scan_inc<false>(m);
+            SrInc ex;
+            ex.a0 = __shfl_up(sc.a0, 1);
+            ex.a1 = __shfl_up(sc.a1, 1);
+            if (lane == 0) { ex.a0 = 0u; ex.a1 = 0u; }
+            const bool odd = (n_in & 1u) != 0u;
+            const uint32_t before = sr_sat_add(n_in, odd ? ex.a1 : ex.a0);
+            const uint32_t after = sr_sat_add(n_in, odd ? sc.a1 : sc.a0);
+            bool ev = after >= (1u << 24);
+            if (kSearch) ev = ev || sr_join(after, eb) >= target;
+            const unsigned long long evl = __ballot(ev && have && lane >= lstart);
+            const int fl = evl ? (int)__ffsll((long long)evl) - 1 : SR_WAVE;
+            if (!kSearch && states && have && lane >= lstart && lane < fl) states[seg] = sr_join(after, eb);
+            if (!evl) {
+                const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)(odd ? sc.a1 : sc.a0), SR_WAVE - 1);
+                s = sr_join(n_in + tot, eb);
+                break;
+            }
+            // The first segment that the plain functions do not settle.  Its lane tries what its record offers, from
+            // the exact sum in front of the segment; every step is checked, and a record that does not fit that sum
+            // (or a search that would end inside the segment) leaves the segment to be added from its terms.
+            const float s_before = sr_u2f((uint32_t)__builtin_amdgcn_readlane((int)sr_f2u(sr_join(before, eb)), fl));
+            float s_try = 0.0f;
+            bool ok = false;
+            if (lane == fl) {
+                if (kind == SR_SEG_EXACT && sr_f2u(s_before) == 0u) {
+                    s_try = sr_u2f(r.g.w);
+                    ok = true;
+                } else if (kind == SR_SEG_SPLIT && (int)r.f.z == eb) {
+                    const uint32_t n1 = sr_sat_add(before, (before & 1u) ? r.f.y : r.f.x);
+                    if (n1 < (1u << 24)) {
+                        float acc = sr_join(n1, eb);
+                        const uint32_t xs[16] = {r.x0.x, r.x0.y, r.x0.z, r.x0.w, r.x1.x, r.x1.y, r.x1.z, r.x1.w,
+                                                 r.x2.x, r.x2.y, r.x2.z, r.x2.w, r.x3.x, r.x3.y, r.x3.z, r.x3.w};
+#pragma unroll
+                        for (int j = 0; j < 16; j++) acc = __fadd_rn(acc, sr_u2f(xs[j]));
+                        uint32_t n2;
+                        int eb2;
+                        sr_split(acc, &n2, &eb2);
+                        if (eb2 == (int)r.g.z) {
+                            const uint32_t n3 = sr_sat_add(n2, (n2 & 1u) ? r.g.y : r.g.x);
+                            if (n3 < (1u << 24)) {
+                                s_try = sr_join(n3, eb2);
+                                ok = true;
+                            }
+                        }
+                    }
+                }
+                if (kSearch && ok && s_try >= target) ok = false;  // the answer lies inside: from the terms
+            }
+            ok = __builtin_amdgcn_readlane((int)ok, fl) != 0;
+            if (ok) {
+                s = sr_u2f((uint32_t)__builtin_amdgcn_readlane((int)sr_f2u(s_try), fl));
+            } else {
+                float x[SR_SEQ_RUN];
+                seq_load_run(terms, aligned, (base + fl) * SR_SEG_TERMS + lane * SR_SEQ_RUN, n, x);
+                int at;
+                s = sr_seq_wave<SR_SEQ_RUN, kSearch>(x, s_before, target, &at);
+                if (kSearch && at >= 0) {
+                    *found = (base + fl) * SR_SEG_TERMS + at;
+                    return s;
+                }
+            }
+            if (!kSearch && states && lane == 0) states[base + fl] = s;
+            lstart = fl + 1;
+            if (lstart >= SR_WAVE) break;
+        }
+    }
+    return s;
+}
+
+// The record of one segment (SeqSegFunc) from its terms x (lane l holds the terms 16 l ... 16 l + 15 of the segment) and
+// the approximate sum `before` of everything in front of the segment.  One wave.
+__device__ __forceinline__ void seg_make_record(const float (&x)[SR_SEQ_RUN], int seg, double before, SeqSegFunc* out)
+{
+    const int lane = sr_lane();
+    // approximate running sum behind every lane's run (single precision does: a prediction that misses costs time only)
+    float own = 0.0f;
+#pragma unroll
+    for (int j = 0; j < SR_SEQ_RUN; j++) own += x[j];
+    const float incl = sr_wave_incl_sum_f32(own);
+    const float before_f = __double2float_rn(before);
+    const float p_end = before_f + incl;
+    uint32_t nn;
+    int eb_first, eb_last, eb_mine_end;
+    sr_split(before_f, &nn, &eb_first);
+    sr_split(__shfl(p_end, SR_WAVE - 1), &nn, &eb_last);
+    sr_split(p_end, &nn, &eb_mine_end);
+    SeqSegFunc f;
+    f.a0 = f.a1 = f.b0 = f.b1 = SR_SEQ_SAT;
+    f.eb = eb_first; f.eb2 = eb_last; f.kind = SR_SEG_PLAIN; f.end_bits = 0u;
+    int cross = -1;
+    if (seg == 0) {
+        // the row's first segment starts from +0 exactly: its end, once and for all
+        int dummy;
+        const float end = sr_seq_wave<SR_SEQ_RUN, false>(x, 0.0f, 0.0f, &dummy);
+        f.kind = SR_SEG_EXACT;
+        f.end_bits = sr_f2u(end);
+    } else if (eb_first == eb_last) {
+        const SrInc sc = sr_scan_inc<false>(sr_run_inc(x, eb_first));
+        f.a0 = (uint32_t)__builtin_amdgcn_readlane((int)sc.a0, SR_WAVE - 1);
+        f.a1 = (uint32_t)__builtin_amdgcn_readlane((int)sc.a1, SR_WAVE - 1);
+    } else {
+        // the first lane behind whose run the sum is expected in another binade; everything behind that lane must then
+        // lie in the segment's last binade, or the segment is no two functions
+        const unsigned long long left = __ballot(eb_mine_end != eb_first);
+        cross = left ? (int)__ffsll((long long)left) - 1 : SR_WAVE - 1;
+        const int eb_behind = __builtin_amdgcn_readlane(eb_mine_end, cross);
+        if (eb_behind == eb_last) {
+            SrInc m1, m2;
+            m1.a0 = m1.a1 = m2.a0 = m2.a1 = 0u;
+            if (lane < cross) m1 = sr_run_inc(x, eb_first);
+            if (lane > cross) m2 = sr_run_inc(x, eb_last);
+            const SrInc s1 = sr_scan_inc<false>(m1), s2 = sr_scan_inc<false>(m2);
+            f.a0 = (uint32_t)__builtin_amdgcn_readlane((int)s1.a0, SR_WAVE - 1);
+            f.a1 = (uint32_t)__builtin_amdgcn_readlane((int)s1.a1, SR_WAVE - 1);
+            f.b0 = (uint32_t)__builtin_amdgcn_readlane((int)s2.a0, SR_WAVE - 1);
+            f.b1 = (uint32_t)__builtin_amdgcn_readlane((int)s2.a1, SR_WAVE - 1);
+            f.kind = SR_SEG_SPLIT | ((uint32_t)cross << 8);
+        } else {
+            cross = -1;
+        }
+    }
+    if (lane == 0) {
+        uint4* q = (uint4*)out;
+        q[0] = make_uint4(f.a0, f.a1, (uint32_t)f.eb, f.kind);
+        q[1] = make_uint4(f.b0, f.b1, (uint32_t)f.eb2, f.end_bits);
+    }
+    if (lane == cross) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) out->x[j] = x[j];
+    }
+}
+
+// The search that follows a sum over the same terms: the first term at which the running sum reaches `target`, from
+// the states the sum left (one wave; -1 when the sum stays below the target).
+__device__ __forceinline__ int seg_search_states(const float* terms, int n, const float* states, float target, float* at_sum)
+{
+    const int lane = sr_lane();
+    const int nseg = seg_count(n);
+    const bool aligned = ((uintptr_t)terms & 15u) == 0u;
+    int first = nseg;
+    for (int g = lane; g < nseg; g += SR_WAVE)
+        if (states[g] >= target) { first = g; break; }
+    first = sr_wave_min_i32(first);
+    if (first >= nseg) return -1;
+    const float s_before = first > 0 ? states[first - 1] : 0.0f;
+    float x[SR_SEQ_RUN];
+    seq_load_run(terms, aligned, first * SR_SEG_TERMS + lane * SR_SEQ_RUN, n, x);
+    int at;
+    *at_sum = sr_seq_wave<SR_SEQ_RUN, true>(x, s_before, target, &at);
+    return at >= 0 ? first * SR_SEG_TERMS + at : -1;
 }
 
 // TensorPrimitives.Sum in its 256-bit shape: strided lane accumulators seeded with the first vector, the
@@ -814,6 +1028,7 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
     if (threadIdx.x == 0) {  // (the first kernel of the pipeline that runs for every row)
         a.state[slot].maxkey = 0u;
         a.state[slot].mul1 = a.state[slot].mul2 = 1.0f;
+        if (a.watch_cnt) a.watch_cnt[slot] = 0u;
     }
     if (rd.edit_cnt <= 0) return;
     const SrEdit* ed = a.edits + rd.edit_off;
@@ -831,6 +1046,7 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
         const bool scale = rd.temperature != 1.0f;
         const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
         const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u;
+        float* wseg = a.seg_func ? a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride : nullptr;
         uint32_t k = 0u;
         for (int e = threadIdx.x; e < rd.edit_cnt; e += 256) {
             const int id = ed[e].id;
@@ -840,6 +1056,7 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
             x = edited_logit(x, ed[e], rd, true, pen);
             if (scale) x = __fmul_rn(x, inv_temp);
             vals[e] = x;
+            if (wseg) wseg[id] = x;  // (the passes over segments take an edited id's value from the work row)
             const uint32_t kv = (x != x) ? 0xffffffffu : sr_okey(x);  // NaN propagates (TensorPrimitives.Max)
             k = kv > k ? kv : k;
         }
@@ -952,6 +1169,303 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
             for (int q = 0; q < 4; q++) e[q] = q < c ? sr_expf_tab(__fsub_rn(x[q], m), tab) : 0.0f;
             store_run(w, i, e, c);
         });
+    }
+}
+
+// ---- the same two passes, laid out for a denominator that the whole device prepares -------------------------
+// (launches whose rows are long and start on 16-byte boundaries: a.seg_func is set.)  A wave takes whole segments of
+// SR_SEG_TERMS elements, every lane 16 consecutive ones, so that the expf pass can leave, beside e = expf(x - max), the
+// record of the segment's exact sum (SeqSegFunc) for the row's workgroup to walk (seg_walk).  The binade that a
+// record is made for comes from approximate sums: the maximum pass leaves every segment's own maximum m and the
+// sum of exp(x - m) over it, and the expf pass, which knows the row's maximum M, adds up S exp(m - M) over the segments
+// in front.  The ids that the row's edits touch take their adjusted values from the work row, where k_full_edits left
+// them, in both passes: e is final when the expf pass has written it.
+__device__ __forceinline__ bool row_watch_min_p(const SrRow& rd, const SrFullArgs& a)
+{
+    return rd.min_p > 0.0f && !(rd.top_k > 0 && rd.top_k < a.vocab) && a.mode == 0 && a.vocab >= 8;
+}
+__device__ __forceinline__ bool row_fast_nucleus(const SrRow& rd, const SrFullArgs& a)
+{
+    const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
+    return use_top_p && !(rd.top_k > 0 && rd.top_k < a.vocab) && !(rd.min_p > 0.0f) && a.mode == 0 && a.vocab >= 8 &&
+           a.vocab <= (1 << kTagIndexBits) && a.sort_stride >= a.vocab;
+}
+template <int ES>
+struct SegSource {
+    const char* rowp;      // the row's logits, or null: the adjusted copy in w
+    const uint32_t* mrow;
+    const uint32_t* erow;
+    const float* w;
+    bool scale;
+    float inv_temp;
+};
+template <int ES>
+__device__ __forceinline__ SegSource<ES> seg_source(const SrRow& rd, const SrFullArgs& a, int slot, int row)
+{
+    SegSource<ES> src;
+    src.w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    src.rowp = nullptr;
+    src.mrow = nullptr;
+    src.erow = nullptr;
+    src.scale = false;
+    src.inv_temp = 1.0f;
+    if (row_is_direct(rd, a)) {
+        src.rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
+        src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
+        src.scale = rd.temperature != 1.0f;
+        src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
+        src.erow = rd.edit_cnt > 0 ? a.edit_tab + (size_t)slot * (size_t)a.edit_tab_stride : nullptr;
+    }
+    return src;
+}
+// The wave's segment as it is loaded: 16-byte vectors, lane l the vectors l, 64 + l, ... of the segment, so that every
+// load instruction of the wave covers consecutive memory.  x[k E + q] is element (k 64 + l) E + q of the segment
+// (E elements per vector: 4 for fp32 logits, 8 for bf16); -inf past the row's end.
+template <int ES>
+__device__ __forceinline__ int seg_elem(int seg, int lane, int slot_kq)
+{
+    constexpr int E = 16 / ES;
+    return seg * SR_SEG_TERMS + ((slot_kq / E) * SR_WAVE + lane) * E + (slot_kq % E);
+}
+template <int ES>
+__device__ __forceinline__ void seg_load_logits(const SegSource<ES>& src, int seg, int lane, int n, float (&x)[SR_SEQ_RUN])
+{
+    constexpr int E = 16 / ES, K = SR_SEG_TERMS / (SR_WAVE * E);
+    static_assert(K * E == SR_SEQ_RUN, "sixteen elements per lane");
+    if ((seg + 1) * SR_SEG_TERMS <= n) {
+        // a whole segment (all but a row's last): every load is issued before anything is done with one of them
+        if (src.rowp) {
+            uint4 raw[K];
+            uint32_t keep[K], hit[K];
+#pragma unroll
+            for (int k = 0; k < K; k++) {
+                const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
+                raw[k] = *(const uint4*)(src.rowp + (size_t)i0 * ES);
+                keep[k] = 0xffffffffu;
+                hit[k] = 0u;
+                if (src.mrow) keep[k] = src.mrow[i0 >> 5] >> (i0 & 31);
+                if (src.erow) hit[k] = (src.erow[i0 >> 5] >> (i0 & 31)) & ((1u << E) - 1u);
+            }
+#pragma unroll
+            for (int k = 0; k < K; k++) {
+                float* xv = &x[k * E];
+                if (ES == 4) {
+                    xv[0] = sr_u2f(raw[k].x); xv[1] = sr_u2f(raw[k].y); xv[2] = sr_u2f(raw[k].z); xv[3] = sr_u2f(raw[k].w);
+                } else {
+                    const uint32_t r[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        xv[(2 * q) % E] = sr_u2f(r[q] << 16);
+                        xv[(2 * q + 1) % E] = sr_u2f(r[q] & 0xffff0000u);
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < E; q++) {
+                    const float v = ((keep[k] >> q) & 1u) ? xv[q] : SR_NEG_INF;
+                    xv[q] = src.scale ? __fmul_rn(v, src.inv_temp) : v;
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < K; k++) {
+                if (hit[k] != 0u) {
+                    const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
+#pragma unroll
+                    for (int q = 0; q < E; q++)
+                        if ((hit[k] >> q) & 1u) x[k * E + q] = src.w[i0 + q];
+                }
+            }
+        } else {
+            float4 rw[K * E / 4];
+#pragma unroll
+            for (int k = 0; k < K; k++)
+#pragma unroll
+                for (int q4 = 0; q4 < E / 4; q4++)
+                    rw[k * (E / 4) + q4] = *(const float4*)(src.w + seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E + 4 * q4);
+#pragma unroll
+            for (int v = 0; v < K * E / 4; v++) {
+                x[4 * v] = rw[v].x; x[4 * v + 1] = rw[v].y; x[4 * v + 2] = rw[v].z; x[4 * v + 3] = rw[v].w;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
+        float* xv = &x[k * E];
+        if (i0 >= n) {
+#pragma unroll
+            for (int q = 0; q < E; q++) xv[q] = SR_NEG_INF;
+            continue;
+        }
+        const bool whole = i0 + E <= n;
+        if (!src.rowp) {  // the adjusted copy
+#pragma unroll
+            for (int q4 = 0; q4 < E; q4 += 4) {
+                if (whole) {
+                    const float4 v = *(const float4*)(src.w + i0 + q4);
+                    xv[q4] = v.x; xv[q4 + 1] = v.y; xv[q4 + 2] = v.z; xv[q4 + 3] = v.w;
+                } else {
+#pragma unroll
+                    for (int q = q4; q < q4 + 4; q++) xv[q] = (i0 + q < n) ? src.w[i0 + q] : SR_NEG_INF;
+                }
+            }
+            continue;
+        }
+        uint32_t keep = (1u << E) - 1u, hit = 0u;
+        if (src.mrow) keep = src.mrow[i0 >> 5] >> (i0 & 31);
+        if (src.erow) hit = (src.erow[i0 >> 5] >> (i0 & 31)) & ((1u << E) - 1u);
+        if (whole) {
+            const uint4 v = *(const uint4*)(src.rowp + (size_t)i0 * ES);
+            if (ES == 4) {
+                xv[0] = sr_u2f(v.x); xv[1] = sr_u2f(v.y); xv[2] = sr_u2f(v.z); xv[3] = sr_u2f(v.w);
+            } else {
+                const uint32_t r[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    xv[(2 * q) % E] = sr_u2f(r[q] << 16);
+                    xv[(2 * q + 1) % E] = sr_u2f(r[q] & 0xffff0000u);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < E; q++) xv[q] = (i0 + q < n) ? load_logit<ES>(src.rowp, i0 + q) : 0.0f;
+        }
+#pragma unroll
+        for (int q = 0; q < E; q++) {
+            float v = ((keep >> q) & 1u) ? xv[q] : SR_NEG_INF;
+            if (src.scale) v = __fmul_rn(v, src.inv_temp);
+            xv[q] = (i0 + q < n) ? v : SR_NEG_INF;
+        }
+        if (hit != 0u) {
+#pragma unroll
+            for (int q = 0; q < E; q++)
+                if ((hit >> q) & 1u) xv[q] = src.w[i0 + q];
+        }
+    }
+}
+template <int ES>
+__global__ __launch_bounds__(256) void k_full_max_seg(SrFullArgs a)
+{
+    const int slot = blockIdx.y, lane = sr_lane();
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    if (rd.temperature <= 0.0f) return;  // greedy rows keep their logits
+    const SegSource<ES> src = seg_source<ES>(rd, a, slot, row);
+    const int n = a.vocab, nseg = seg_count(n);
+    __shared__ uint32_t wmax[4];
+    uint32_t kmax = 0u;
+    for (int seg = (int)blockIdx.x * 4 + sr_wave_id(); seg < nseg; seg += (int)gridDim.x * 4) {
+        float x[SR_SEQ_RUN];
+        seg_load_logits<ES>(src, seg, lane, n, x);
+        uint32_t k = 0u;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t kv = (x[j] != x[j]) ? 0xffffffffu : sr_okey(x[j]);  // NaN propagates (TensorPrimitives.Max)
+            k = kv > k ? kv : k;
+        }
+        k = sr_wave_max_u32(k);
+        float m = SR_NEG_INF, sum = 0.0f;
+        if (k != 0xffffffffu && k > 0x007fffffu) {
+            m = sr_okey_inv(k);
+#pragma unroll
+            for (int j = 0; j < 16; j++) sum += __expf(x[j] - m);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+        if (lane == 0) a.seg_ms[(size_t)slot * a.seg_stride + seg] = make_float2(m, sum);
+        kmax = k > kmax ? k : kmax;
+    }
+    // (one atomic per workgroup: a row's hundreds of segments would queue on the one word)
+    if (lane == 0) wmax[sr_wave_id()] = kmax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        kmax = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+        if (kmax != 0u) atomicMax(&a.state[slot].maxkey, kmax);
+    }
+}
+template <int ES>
+__global__ __launch_bounds__(256) void k_full_exp_seg(SrFullArgs a)
+{
+    constexpr int E = 16 / ES, K = SR_SEG_TERMS / (SR_WAVE * E);
+    const int slot = blockIdx.y, lane = sr_lane(), wave = sr_wave_id();
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    if (rd.temperature <= 0.0f) return;
+    const uint32_t mk = a.state[slot].maxkey;
+    if (mk == 0xffffffffu || mk <= 0x007fffffu) return;  // NaN, or nothing above -inf: the row kernel makes it uniform
+    const float m = sr_okey_inv(mk);
+    __shared__ uint64_t tab[32];  // the expf table: a lookup per element from global memory is a long dependent load
+    __shared__ float4 turn[4][SR_SEG_TERMS / 4];  // a wave's segment on its way from the order of the loads to 16 terms a lane
+    if (threadIdx.x < 32) tab[threadIdx.x] = sr_exp2f_tab[threadIdx.x];
+    __syncthreads();
+    const SegSource<ES> src = seg_source<ES>(rd, a, slot, row);
+    float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    const int n = a.vocab, nseg = seg_count(n);
+    const bool watch = row_watch_min_p(rd, a);
+    const float e_low = __fmul_rn(rd.min_p, 0.999999f);
+    const bool record = !row_fast_nucleus(rd, a);  // (such a row counts a histogram while it adds: its workgroup adds)
+    const float2* ms = a.seg_ms + (size_t)slot * a.seg_stride;
+    for (int seg = (int)blockIdx.x * 4 + wave; seg < nseg; seg += (int)gridDim.x * 4) {
+        float x[SR_SEQ_RUN], e[SR_SEQ_RUN];
+        seg_load_logits<ES>(src, seg, lane, n, x);
+        // (the approximate sum in front of the segment, under the loads)
+        double before = 0.0;
+        if (record) {
+            for (int g = lane; g < seg; g += SR_WAVE) {
+                const float2 v = ms[g];
+                if (v.y > 0.0f) before += (double)(v.y * __expf(v.x - m));
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o);
+        }
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
+#pragma unroll
+            for (int q = 0; q < E; q++) e[k * E + q] = (i0 + q < n) ? sr_expf_tab(__fsub_rn(x[k * E + q], m), tab) : 0.0f;
+            if (i0 + E <= n) {
+#pragma unroll
+                for (int q = 0; q < E; q += 4)
+                    *(float4*)(w + i0 + q) = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < E; q++)
+                    if (i0 + q < n) w[i0 + q] = e[k * E + q];
+            }
+            if (watch) {
+#pragma unroll
+                for (int q = 0; q < E; q++)
+                    if (e[k * E + q] >= e_low && i0 + q < n) {
+                        const uint32_t pos = atomicAdd(&a.watch_cnt[slot], 1u);
+                        if (pos < (uint32_t)kSmall)
+                            a.watch[(size_t)slot * kSmall + pos] = ((unsigned long long)sr_f2u(e[k * E + q]) << 32) |
+                                                                   (unsigned long long)(0xffffffffu - (uint32_t)(i0 + q));
+                    }
+            }
+        }
+        if (record) {
+            // through shared memory into the order of the sum: lane l gets the terms 16 l ... 16 l + 15 of the segment
+            // (only this wave touches its part: the wave's own order of shared-memory operations is all it needs)
+            float4* mine = turn[wave];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+            for (int k = 0; k < K; k++)
+#pragma unroll
+                for (int q = 0; q < E; q += 4)
+                    mine[((k * SR_WAVE + lane) * E + q) / 4] = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            float t[SR_SEQ_RUN];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float4 v = mine[lane * 4 + k];
+                t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            seg_make_record(t, seg, before, a.seg_func + (size_t)slot * a.seg_stride + seg);
+        }
     }
 }
 
@@ -1169,7 +1683,6 @@ struct StretchToSegment {  // at the stretch's own positions of the row's sort s
     __device__ __forceinline__ int reserve(int before, int) const { return w0 + before; }
     __device__ __forceinline__ void put(int place, int, uint32_t ybits, int i) const { gk[place] = ybits; gi[place] = i; }
 };
-constexpr int kTagIndexBits = 19;  // a find's tag: rank << 19 | index
 struct StretchToPool {  // appended to a pool in LDS that all waves share: values to vals, tags to tags
     uint32_t* counter;
     uint32_t* vals;
@@ -1808,7 +2321,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             flags |= SR_KFLAG_DEGENERATE;
             __syncthreads();
         } else {
-            if (row_edits_on_the_fly(rd, a)) {
+            if (row_edits_on_the_fly(rd, a) && !a.seg_func) {
                 // the ids that the row's edits touch were left out of the expf pass: their e, from the adjusted values
                 // that k_full_edits kept
                 const float* vals = (const float*)(a.edit_tab + (size_t)slot * (size_t)a.edit_tab_stride + (n + 31) / 32);
@@ -1821,15 +2334,14 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             // A row that min-p cuts, with no top-k stage before the cut and no distribution to hand out, is not read a
             // second time for the cut: a survivor has fl(e * inv) >= fl(min_p * inv), so e >= min_p * (1 - 2^-22), and
             // the few entries that large are listed while the sum passes over them; the exact test follows below.
-            const bool watch_min_p = rd.min_p > 0.0f && !(rd.top_k > 0 && rd.top_k < n) && a.mode == 0 && n >= 8;
+            const bool watch_min_p = row_watch_min_p(rd, a);
             const float e_low = __fmul_rn(rd.min_p, 0.999999f);
             if (watch_min_p) {
                 if (tid == 0) sm.bc[4] = 0u;
                 __syncthreads();
             }
             // A row that only top-p cuts and that is only sampled from: see nucleus_from_histogram
-            const bool fast_nucleus = use_top_p && !(rd.top_k > 0 && rd.top_k < n) && !(rd.min_p > 0.0f) && a.mode == 0 &&
-                                      n >= 8 && n <= (1 << kTagIndexBits) && a.sort_stride >= n;
+            const bool fast_nucleus = row_fast_nucleus(rd, a);
             if (fast_nucleus) {
                 uint32_t* hcnt = (uint32_t*)sm.sortbuf;
                 for (int i = tid; i < kHistPos; i += kT) hcnt[i] = 0u;
@@ -1837,7 +2349,22 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                 __syncthreads();
             }
             float sum;
-            if (fast_nucleus) {
+            if (a.seg_func && !fast_nucleus) {
+                // the whole device has prepared the sum (k_full_exp_seg): one wave walks the segments' records, and the
+                // entries that can survive the min-p cut were listed by the same pass
+                __syncthreads();
+                if (sr_wave_id() == 0) {
+                    const float s = seg_walk<false>(p, n, a.seg_func + (size_t)slot * a.seg_stride, 0.0f, 0.0f, &dummy, nullptr);
+                    if (sr_lane() == 0) sm.segbc[0] = sr_f2u(s);
+                } else if (watch_min_p) {
+                    const uint32_t cw = a.watch_cnt[slot];
+                    const unsigned long long* wl = a.watch + (size_t)slot * kSmall;
+                    for (int i = tid - SR_WAVE; i < (int)min(cw, (uint32_t)kSmall); i += kT - SR_WAVE) sm.sortbuf[i] = wl[i];
+                    if (tid == SR_WAVE) sm.bc[4] = cw;
+                }
+                __syncthreads();
+                sum = sr_u2f(sm.segbc[0]);
+            } else if (fast_nucleus) {
                 uint32_t* hcnt = (uint32_t*)sm.sortbuf;
                 sum = seq_sum_row<false>(p, n, 0.0f, 0.0f, &dummy, sm, 1.0f, 1.0f, [&](float x, int) { hist_count(hcnt, &sm.bc[5], x); });
             } else if (watch_min_p) {
@@ -2480,6 +3007,67 @@ __device__ __forceinline__ int resample_residual_stored(const float* res, const 
     return found >= 0 ? found : edge(false);  // (rounding: the sum of the search fell short of the target)
 }
 
+// ... with the increment functions of the stored row's segments at hand (k_seq_funcs): one wave walks them
+__device__ __forceinline__ int residual_edge(const float* res, int n, bool first_one, FullSmem& sm)
+{
+    // the first / the last index with a positive residual
+    int at = first_one ? 0x7fffffff : -1;
+    for (int i = threadIdx.x; i < n; i += kT)
+        if (res[i] > 0.0f) {
+            at = i;
+            if (first_one) break;
+        }
+    at = first_one ? sr_wave_min_i32(at) : -sr_wave_min_i32(-at);
+    __syncthreads();
+    if (sr_lane() == 0) sm.redi[sr_wave_id()] = at;
+    __syncthreads();
+    int f = first_one ? 0x7fffffff : -1;
+    for (int w = 0; w < kW; w++) f = first_one ? min(f, sm.redi[w]) : max(f, sm.redi[w]);
+    __syncthreads();
+    return f;
+}
+__device__ __forceinline__ int resample_residual_prepared(const float* res, const SeqSegFunc* funcs, const float* p, int n, double u,
+                                                          FullSmem& sm, float m1, float m2)
+{
+    const bool walker = sr_wave_id() == 0;
+    int dummy;
+    __syncthreads();  // (sm.segst and sm.segbc are free)
+    if (walker) {
+        const float sum = seg_walk<false>(res, n, funcs, 0.0f, 0.0f, &dummy, sm.segst);
+        if (sr_lane() == 0) sm.segbc[0] = sr_f2u(sum);
+    }
+    __syncthreads();
+    const float sum = sr_u2f(sm.segbc[0]);
+    if (!(sum > 0.0f)) return draw_from_row(p, n, u, sm, m1, m2);  // sum <= 0 or NaN
+    const float target = __fmul_rn(__double2float_rn(u), sum);
+    if (target <= 0.0f) return residual_edge(res, n, true, sm);  // a zero target must not stop on a zero term
+    if (walker) {
+        float at;
+        const int found = seg_search_states(res, n, sm.segst, target, &at);
+        if (sr_lane() == 0) sm.segbc[1] = (uint32_t)found;
+    }
+    __syncthreads();
+    const int found = (int)sm.segbc[1];
+    return found >= 0 ? found : residual_edge(res, n, false, sm);  // (rounding: the sum of the search fell short of the target)
+}
+// SampleFromDistribution (Sampler.cs:564-576) over a stored row with its segments' functions: draw_from_row by one wave
+__device__ __forceinline__ int draw_from_prepared(const float* terms, const SeqSegFunc* funcs, int n, double u, FullSmem& sm)
+{
+    const float r = __double2float_rn(u);
+    __syncthreads();
+    if (sr_wave_id() == 0) {
+        int found;
+        const float at = seg_walk<true>(terms, n, funcs, 0.0f, r, &found, nullptr);
+        if (sr_lane() == 0) {
+            sm.segbc[1] = (uint32_t)found;
+            SR_AMB_IF(found >= 0 ? sr_stop_near(at, terms[found], r) : sr_near(at, r));
+        }
+    }
+    __syncthreads();
+    const int found = (int)sm.segbc[1];
+    return found >= 0 ? found : n - 1;
+}
+
 // Every position of a row is filtered with the row's own parameters (SpeculativeDecoder.cs:535): the batch's row
 // descriptors, one copy per position, without their allow-masks
 __global__ __launch_bounds__(256) void k_expand_rows(const SrRow* src, SrRow* dst, int rows, int positions)
@@ -2503,6 +3091,8 @@ __global__ __launch_bounds__(SR_WAVE) void k_spec_walk(SrSpecArgs a)
     const bool true_spec = !(rd.p_min > 0.0f && rd.p_min < 1.0f) && (rd.flags & SR_ROWBIT_DRAFT_FROM_LOOKUP) == 0u;
     int reject = -1;
     if (true_spec) {
+        // (every draft accepted, and a bonus token to draw: position L, whose scaled row k_spec_residual writes out)
+        if (a.seg_func && rd.temperature > 0.0f) reject = L;
         const float* pr = a.p_all + (size_t)row * (L + 1) * n;
         const double* u = a.uniforms + (size_t)row * a.uniforms_per_row;
         for (int i0 = 0; i0 < L; i0 += SR_WAVE) {
@@ -2531,34 +3121,73 @@ __global__ __launch_bounds__(SR_WAVE) void k_spec_walk(SrSpecArgs a)
     if (lane == 0) a.reject[row] = reject;
 }
 
+// The terms the row's workgroup will add, written by the whole device: max(0, fl(fl(p m1) m2) - q) of the first rejected
+// position, or the scaled target row fl(fl(p m1) m2) of the bonus position when every draft was accepted (reject == L).
+// A wave takes whole segments of SR_SEG_TERMS terms and leaves each segment's approximate sum for k_seq_funcs.
 __global__ __launch_bounds__(256) void k_spec_residual(SrSpecArgs a)
 {
     const int row = blockIdx.y;
     const int i = a.reject[row];
     if (i < 0) return;
-    const int n = a.vocab, L = a.n_draft;
+    const int n = a.vocab, L = a.n_draft, lane = sr_lane();
+    const bool bonus = i == L;
     const float* pd = a.p_all + ((size_t)row * (L + 1) + i) * n;
-    const float* qd = a.draft_probs + ((size_t)row * L + i) * n;
+    const float* qd = bonus ? pd : a.draft_probs + ((size_t)row * L + i) * n;
     const SrFullState* sl = a.state + (size_t)row * (L + 1) + i;
     const float m1 = sl->mul1, m2 = sl->mul2;
     float* out = a.resid + (size_t)row * (size_t)a.resid_stride;
     auto res = [&](float pv, float qv) -> float {
-        const float r = __fsub_rn(__fmul_rn(__fmul_rn(pv, m1), m2), qv);
+        const float sp = __fmul_rn(__fmul_rn(pv, m1), m2);
+        if (bonus) return sp;
+        const float r = __fsub_rn(sp, qv);
         return r > 0.0f ? r : 0.0f;
     };
-    const int t = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
-    if (((((uintptr_t)pd) | ((uintptr_t)qd)) & 15u) == 0u) {
-        const int nv = n / 4;
-        for (int v = t; v < nv; v += nt) {
-            const float4 pv = ((const float4*)pd)[v], qv = ((const float4*)qd)[v];
-            float4 o;
-            o.x = res(pv.x, qv.x); o.y = res(pv.y, qv.y); o.z = res(pv.z, qv.z); o.w = res(pv.w, qv.w);
-            ((float4*)out)[v] = o;
+    const bool aligned = ((((uintptr_t)pd) | ((uintptr_t)qd)) & 15u) == 0u;
+    const int nseg = seg_count(n);
+    for (int seg = (int)blockIdx.x * 4 + sr_wave_id(); seg < nseg; seg += (int)gridDim.x * 4) {
+        double acc = 0.0;
+#pragma unroll
+        for (int k = 0; k < SR_SEG_TERMS / (4 * SR_WAVE); k++) {
+            const int x0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * 4;
+            if (aligned && x0 + 4 <= n) {
+                const float4 pv = *(const float4*)(pd + x0), qv = *(const float4*)(qd + x0);
+                float4 o;
+                o.x = res(pv.x, qv.x); o.y = res(pv.y, qv.y); o.z = res(pv.z, qv.z); o.w = res(pv.w, qv.w);
+                *(float4*)(out + x0) = o;  // (the rows of a.resid start on 16-byte boundaries)
+                acc += ((double)o.x + (double)o.y) + ((double)o.z + (double)o.w);
+            } else {
+                for (int x = x0; x < min(x0 + 4, n); x++) {
+                    const float o = res(pd[x], qd[x]);
+                    out[x] = o;
+                    acc += (double)o;
+                }
+            }
         }
-        for (int x = nv * 4 + t; x < n; x += nt) out[x] = res(pd[x], qd[x]);
-    } else {
-        for (int x = t; x < n; x += nt) out[x] = res(pd[x], qd[x]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+        if (a.seg_part && lane == 0) a.seg_part[(size_t)row * a.seg_stride + seg] = acc;
     }
+}
+
+// The record of every segment of every row of terms (SeqSegFunc), for the binades that the approximate sums predict:
+// the sums of the segments in front (part, left by the kernel that wrote the terms) and, inside the segment, of the
+// lanes in front.  One wave per segment.
+__global__ __launch_bounds__(256) void k_seq_funcs(const float* terms, int64_t stride, int n, const double* part, SeqSegFunc* func,
+                                                   int seg_stride, const int32_t* active)
+{
+    const int row = blockIdx.y, lane = sr_lane();
+    if (active && active[row] < 0) return;
+    const int seg = (int)blockIdx.x * 4 + sr_wave_id();
+    if (seg >= seg_count(n)) return;
+    const double* pr = part + (size_t)row * seg_stride;
+    double before = 0.0;
+    for (int g = lane; g < seg; g += SR_WAVE) before += pr[g];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o);
+    const float* t = terms + (size_t)row * (size_t)stride;
+    float x[SR_SEQ_RUN];
+    seq_load_run(t, ((uintptr_t)t & 15u) == 0u, seg * SR_SEG_TERMS + lane * SR_SEQ_RUN, n, x);
+    seg_make_record(x, seg, before, func + (size_t)row * seg_stride + seg);
 }
 
 // ---- speculative verification: the accept loop of StepSampled (SpeculativeDecoder.cs:530-559) ---------
@@ -2624,7 +3253,10 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
         }
         const float m1 = sl->mul1, m2 = sl->mul2;
         const double uc = u[udraws++];
-        if (true_spec && a.reject && a.reject[row] == i)  // the residual row is there already
+        if (true_spec && a.reject && a.reject[row] == i && a.seg_func)  // the residual row and its segments' functions are there
+            correction = resample_residual_prepared(a.resid + (size_t)row * (size_t)a.resid_stride,
+                                                    a.seg_func + (size_t)row * a.seg_stride, pd, n, uc, sm, m1, m2);
+        else if (true_spec && a.reject && a.reject[row] == i)  // the residual row is there already
             correction = resample_residual_stored(a.resid + (size_t)row * (size_t)a.resid_stride, pd, n, uc, sm, m1, m2);
         else
             correction = true_spec ? resample_residual_row(pd, qd, n, uc, sm, m1, m2) : draw_from_row(pd, n, uc, sm, m1, m2);
@@ -2634,7 +3266,11 @@ __global__ __launch_bounds__(kT) void k_spec_verify(SrSpecArgs a)
         // every draft accepted: bonus token from the last position (greedy rows: its argmax, no draw)
         const float* pd = pr + (size_t)L * n;
         const SrFullState* sl = a.state + (size_t)row * (L + 1) + L;
-        correction = rd.temperature <= 0.0f ? row_argmax(pd, n, sm) : draw_from_row(pd, n, u[udraws++], sm, sl->mul1, sl->mul2);
+        if (rd.temperature <= 0.0f) correction = row_argmax(pd, n, sm);
+        else if (a.seg_func && a.reject[row] == L)  // the scaled row and its segments' functions are there
+            correction = draw_from_prepared(a.resid + (size_t)row * (size_t)a.resid_stride, a.seg_func + (size_t)row * a.seg_stride, n,
+                                            u[udraws++], sm);
+        else correction = draw_from_row(pd, n, u[udraws++], sm, sl->mul1, sl->mul2);
     }
     if (threadIdx.x == 0) {
         out[accepted] = correction;
@@ -2711,7 +3347,17 @@ hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
         if (a.any_copy) hipLaunchKernelGGL(k_full_prep<4>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(k_full_edits<4>, dim3(n_rows), dim3(256), 0, st, a);
     }
-    if (a.dtype == 1) {
+    if (a.seg_func) {
+        const int nseg = (a.vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
+        dim3 sgrid((unsigned)std::max(1, std::min(64, (nseg + 3) / 4)), n_rows);
+        if (a.dtype == 1) {
+            hipLaunchKernelGGL(k_full_max_seg<2>, sgrid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL(k_full_exp_seg<2>, sgrid, dim3(256), 0, st, a);
+        } else {
+            hipLaunchKernelGGL(k_full_max_seg<4>, sgrid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL(k_full_exp_seg<4>, sgrid, dim3(256), 0, st, a);
+        }
+    } else if (a.dtype == 1) {
         hipLaunchKernelGGL(k_full_max<2>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(k_full_exp<2>, grid, dim3(256), 0, st, a);
     } else {
@@ -2778,9 +3424,15 @@ hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st)
     if (!(b.resid && b.reject && b.n_draft > 0 && b.draft_probs && rows <= 65535)) {  // (rows are the grid's second dimension)
         b.resid = nullptr;
         b.reject = nullptr;
+        b.seg_func = nullptr;
     } else {
+        const int nseg = (b.vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
+        if (!(b.seg_func && b.seg_part && nseg <= SR_SEG_MAX && nseg <= b.seg_stride)) b.seg_func = nullptr;
         hipLaunchKernelGGL(k_spec_walk, dim3(rows), dim3(SR_WAVE), 0, st, b);
-        hipLaunchKernelGGL(k_spec_residual, dim3(64, rows), dim3(256), 0, st, b);
+        hipLaunchKernelGGL(k_spec_residual, dim3((unsigned)std::min(64, (nseg + 3) / 4), rows), dim3(256), 0, st, b);
+        if (b.seg_func)
+            hipLaunchKernelGGL(k_seq_funcs, dim3((unsigned)((nseg + 3) / 4), rows), dim3(256), 0, st, b.resid, b.resid_stride, b.vocab,
+                               b.seg_part, (SeqSegFunc*)b.seg_func, b.seg_stride, b.reject);
     }
     hipLaunchKernelGGL(k_spec_verify, dim3(rows), dim3(kT), 0, st, b);
     return hipGetLastError();

@@ -75,6 +75,25 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     // the kernels index sort segments with work_stride; keep both strides equal in mode 0 and pass the
     // segment stride separately otherwise
     a.sort_stride = seg_stride;
+    // Long rows that start on 16-byte boundaries, logits and work rows alike: the softmax denominators are prepared by
+    // the passes over the whole device (k_full_max_seg / k_full_exp_seg) and the rows' workgroups only walk the records
+    {
+        const int es = dtype == SR_DTYPE_BF16 ? 2 : 4;
+        const int nseg = (vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
+        const bool aligned = (((uintptr_t)logits_dev) & 15u) == 0u && ((row_stride * es) & 15) == 0 &&
+                             (((uintptr_t)a.work) & 15u) == 0u && ((a.work_stride * 4) & 15) == 0;
+        if (vocab >= SR_SEG_MIN_VOCAB && nseg <= SR_SEG_MAX && aligned) {
+            SR_HIP(ctx, ctx->full_seg_func.reserve((size_t)n_rows * (size_t)nseg * sizeof(SeqSegFunc), st));
+            SR_HIP(ctx, ctx->full_seg_ms.reserve((size_t)n_rows * (size_t)nseg * sizeof(float2), st));
+            SR_HIP(ctx, ctx->full_watch.reserve((size_t)n_rows * SR_FULL_SMALL_CAP * sizeof(unsigned long long), st));
+            SR_HIP(ctx, ctx->full_watch_cnt.reserve((size_t)n_rows * sizeof(uint32_t), st));
+            a.seg_func = (SeqSegFunc*)ctx->full_seg_func.p;
+            a.seg_ms = (float2*)ctx->full_seg_ms.p;
+            a.seg_stride = nseg;
+            a.watch = ctx->full_watch.as<unsigned long long>();
+            a.watch_cnt = ctx->full_watch_cnt.as<uint32_t>();
+        }
+    }
     a.uniforms = b->d_uniforms.as<double>();
     a.uniforms_per_row = b->upr;
     a.out_tokens = out_tokens_dev;
@@ -447,6 +466,13 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
     SR_HIP(ctx, ctx->spec_reject.reserve((size_t)rows * sizeof(int32_t), st));
     a.resid = ctx->spec_resid.as<float>();
     a.reject = ctx->spec_reject.as<int32_t>();
+    a.seg_stride = (V + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
+    if (a.seg_stride <= SR_SEG_MAX) {  // (longer rows are added by their workgroups alone)
+        SR_HIP(ctx, ctx->seg_part.reserve((size_t)rows * (size_t)a.seg_stride * sizeof(double), st));
+        SR_HIP(ctx, ctx->seg_func.reserve((size_t)rows * (size_t)a.seg_stride * sizeof(SeqSegFunc), st));
+        a.seg_part = ctx->seg_part.as<double>();
+        a.seg_func = (SeqSegFunc*)ctx->seg_func.p;
+    }
     SR_HIP(ctx, sr_launch_spec_verify(a, rows, st));
     return SR_OK;
 }

@@ -137,6 +137,7 @@ struct SrFullState {
     int32_t pad2;
 };
 
+struct SeqSegFunc;
 struct SrFullArgs {
     const void* logits;
     int64_t row_stride;
@@ -166,6 +167,13 @@ struct SrFullArgs {
     int32_t* out_tokens;       // [row], may be null in mode 1
     uint32_t* out_flags;       // [row], may be null
     unsigned long long* prof;  // optional phase timestamps of slot 0 [32] (test hook), normally null
+    // The softmax denominators prepared by the whole device (k_full_max_seg / k_full_exp_seg, seg_walk); seg_func is
+    // null when the launch is not laid out for it (short or unaligned rows) and the rows are added by their workgroups.
+    SeqSegFunc* seg_func;          // [slot][seg_stride]
+    float2* seg_ms;                // [slot][seg_stride]: a segment's maximum m and the sum of exp(x - m) over it, approximately
+    int32_t seg_stride;
+    unsigned long long* watch;     // [slot][SR_FULL_SMALL_CAP]: the entries that can survive a row's min-p cut (value << 32 | ~index)
+    uint32_t* watch_cnt;           // [slot]
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, hipStream_t st);
@@ -181,6 +189,23 @@ hipError_t sr_launch_draw_rows(const float* probs, int64_t stride, int n, int ro
 hipError_t sr_launch_residual_rows(const float* p, int64_t ps, const float* q, int64_t qs, int n, int rows,
                                    const double* u, int* out, hipStream_t st);
 
+// One segment of SR_SEG_TERMS terms of a row whose exact sum the whole device prepares (k_seq_funcs, seg_walk in
+// sr_full.hip): the increment function n -> n + a[n & 1] of its terms in the binade `eb` (sr_seqsum.h), and for a
+// segment in which the running sum is expected to change binade once, inside the 16 terms of lane `cross`: the function
+// of the terms in front of those 16 (a0, a1, eb), the 16 terms themselves, and the function of the terms behind them
+// (b0, b1) in the binade eb2.  The row's first segment, whose start is known exactly, carries its exact end instead.
+#define SR_SEG_PLAIN 0u
+#define SR_SEG_EXACT 1u
+#define SR_SEG_SPLIT 2u
+struct SeqSegFunc {  // 96 bytes
+    uint32_t a0, a1;
+    int32_t eb;
+    uint32_t kind;   // SR_SEG_* | cross << 8
+    uint32_t b0, b1;
+    int32_t eb2;
+    uint32_t end_bits;  // SR_SEG_EXACT: the running sum behind the segment when the sum in front of it is +0
+    float x[16];
+};
 struct SrSpecArgs {
     const SrRow* rows;
     int32_t vocab;
@@ -196,7 +221,11 @@ struct SrSpecArgs {
     int32_t* out_tokens;         // [rows][n_draft + 1]
     float* resid;                // [rows][resid_stride]: max(0, p - q) of the row's first rejected position
     int64_t resid_stride;
-    int32_t* reject;             // [rows]: that position, or -1 (none, or a row that does not take the ratio test)
+    int32_t* reject;             // [rows]: that position, or -1 (none, or a row that does not take the ratio test), or
+                                 // n_draft (every draft accepted and a bonus token to draw: resid holds the scaled row)
+    double* seg_part;            // [rows][seg_stride]: approximate sum of every SR_SEG_TERMS terms of the row of resid
+    SeqSegFunc* seg_func;        // [rows][seg_stride]: the increment functions of those segments; null: not prepared
+    int32_t seg_stride;
 };
 hipError_t sr_launch_spec_verify(const SrSpecArgs& a, int rows, hipStream_t st);
 hipError_t sr_launch_expand_rows(const SrRow* src, SrRow* dst, int rows, int positions, hipStream_t st);

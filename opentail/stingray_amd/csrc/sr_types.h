@@ -91,3 +91,6 @@ struct SrMaskClear {
 
 // Full-vocabulary path: nucleus candidates up to this count are sorted inside the row kernel.
 #define SR_FULL_SMALL_CAP 4096
+#define SR_SEG_TERMS 1024                  // terms per segment of a sum that the whole device prepares (64 lanes x 16)
+#define SR_SEG_MIN_VOCAB 4096              // shorter rows are not worth the preparation
+#define SR_SEG_MAX 1024                    // most segments of such a row: longer rows are added the plain way
