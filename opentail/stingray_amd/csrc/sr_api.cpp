@@ -315,7 +315,7 @@ void sr_destroy(sr_ctx* ctx)
                          &ctx->work, &ctx->edit_tab, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->full_state, &ctx->sort_k0, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs, &ctx->spec_resid, &ctx->spec_reject,
-                         &ctx->seg_part, &ctx->seg_func, &ctx->full_seg_func, &ctx->full_seg_ms, &ctx->full_watch, &ctx->full_watch_cnt};
+                         &ctx->seg_part, &ctx->seg_func, &ctx->full_seg_func, &ctx->full_seg_ms, &ctx->full_watch, &ctx->full_watch_cnt, &ctx->full_seg_keys};
     for (DeviceBuf* b : bufs) b->release();
     ctx->uni_ring.release();
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);

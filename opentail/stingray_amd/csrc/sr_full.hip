@@ -1001,6 +1001,30 @@ __device__ __forceinline__ void store_run(float* w, int i, const float (&x)[E], 
     }
 }
 
+// The histogram of a row's e = expf(x - max) by their upper 16 bits (kHistPos positions: position d holds the keys
+// 0x3f80 - d, position 0 is e = 1, the last position everything below): see nucleus_from_histogram
+constexpr int kHistPos = 8192;
+constexpr uint32_t kHistTopKey = 0x3f80u;
+__device__ __forceinline__ void hist_count(uint32_t* hcnt, uint32_t* bad, float e)
+{
+    if (e > 0.0f) {
+        const uint32_t key = sr_f2u(e) >> 16;
+        if (key <= kHistTopKey) atomicAdd(&hcnt[min(kHistTopKey - key, (uint32_t)(kHistPos - 1))], 1u);
+        else *bad = 1u;  // (no e exceeds 1; if one does, the general way takes the row)
+    }
+}
+
+// which rows take which way: asked by the passes over the whole device and by the row's workgroup alike
+__device__ __forceinline__ bool row_watch_min_p(const SrRow& rd, const SrFullArgs& a)
+{
+    return rd.min_p > 0.0f && !(rd.top_k > 0 && rd.top_k < a.vocab) && a.mode == 0 && a.vocab >= 8;
+}
+__device__ __forceinline__ bool row_fast_nucleus(const SrRow& rd, const SrFullArgs& a)
+{
+    const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
+    return use_top_p && !(rd.top_k > 0 && rd.top_k < a.vocab) && !(rd.min_p > 0.0f) && a.mode == 0 && a.vocab >= 8 &&
+           a.vocab <= (1 << kTagIndexBits) && a.sort_stride >= a.vocab;
+}
 // ---- stage 1: the masked (and temperature-scaled) copy of the row ------------------------------------
 template <int ES>
 __global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
@@ -1030,6 +1054,7 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
         a.state[slot].mul1 = a.state[slot].mul2 = 1.0f;
         if (a.watch_cnt) a.watch_cnt[slot] = 0u;
     }
+
     if (rd.edit_cnt <= 0) return;
     const SrEdit* ed = a.edits + rd.edit_off;
     if (row_edits_on_the_fly(rd, a)) {
@@ -1180,16 +1205,6 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
 // sum of exp(x - m) over it, and the expf pass, which knows the row's maximum M, adds up S exp(m - M) over the segments
 // in front.  The ids that the row's edits touch take their adjusted values from the work row, where k_full_edits left
 // them, in both passes: e is final when the expf pass has written it.
-__device__ __forceinline__ bool row_watch_min_p(const SrRow& rd, const SrFullArgs& a)
-{
-    return rd.min_p > 0.0f && !(rd.top_k > 0 && rd.top_k < a.vocab) && a.mode == 0 && a.vocab >= 8;
-}
-__device__ __forceinline__ bool row_fast_nucleus(const SrRow& rd, const SrFullArgs& a)
-{
-    const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
-    return use_top_p && !(rd.top_k > 0 && rd.top_k < a.vocab) && !(rd.min_p > 0.0f) && a.mode == 0 && a.vocab >= 8 &&
-           a.vocab <= (1 << kTagIndexBits) && a.sort_stride >= a.vocab;
-}
 template <int ES>
 struct SegSource {
     const char* rowp;      // the row's logits, or null: the adjusted copy in w
@@ -1396,14 +1411,19 @@ __global__ __launch_bounds__(256) void k_full_exp_seg(SrFullArgs a)
     const float m = sr_okey_inv(mk);
     __shared__ uint64_t tab[32];  // the expf table: a lookup per element from global memory is a long dependent load
     __shared__ float4 turn[4][SR_SEG_TERMS / 4];  // a wave's segment on its way from the order of the loads to 16 terms a lane
+    // A row that only top-p cuts needs the histogram of its e by their upper 16 bits.  Counting it here took longer
+    // than it saved (one atomic per element in device memory: +30 us; in shared memory, by few workgroups that take
+    // many segments each: +55 us), so the pass leaves those 16 bits of every e beside the row, and the row's workgroup
+    // counts them -- half the bytes of the row -- while one of its waves walks the sum.
+    uint16_t* keys = (row_fast_nucleus(rd, a) && a.seg_keys) ? a.seg_keys + (size_t)slot * (size_t)a.seg_key_stride : nullptr;
+    const int n = a.vocab, nseg = seg_count(n);
     if (threadIdx.x < 32) tab[threadIdx.x] = sr_exp2f_tab[threadIdx.x];
     __syncthreads();
     const SegSource<ES> src = seg_source<ES>(rd, a, slot, row);
     float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
-    const int n = a.vocab, nseg = seg_count(n);
     const bool watch = row_watch_min_p(rd, a);
     const float e_low = __fmul_rn(rd.min_p, 0.999999f);
-    const bool record = !row_fast_nucleus(rd, a);  // (such a row counts a histogram while it adds: its workgroup adds)
+    const bool record = true;
     const float2* ms = a.seg_ms + (size_t)slot * a.seg_stride;
     for (int seg = (int)blockIdx.x * 4 + wave; seg < nseg; seg += (int)gridDim.x * 4) {
         float x[SR_SEQ_RUN], e[SR_SEQ_RUN];
@@ -1431,6 +1451,20 @@ __global__ __launch_bounds__(256) void k_full_exp_seg(SrFullArgs a)
 #pragma unroll
                 for (int q = 0; q < E; q++)
                     if (i0 + q < n) w[i0 + q] = e[k * E + q];
+            }
+            if (keys) {
+                uint32_t kk[E];
+#pragma unroll
+                for (int q = 0; q < E; q++) kk[q] = e[k * E + q] > 0.0f ? max(sr_f2u(e[k * E + q]) >> 16, 1u) : 0u;
+                if (i0 + E <= n) {
+#pragma unroll
+                    for (int q = 0; q < E; q += 4)
+                        *(uint2*)(keys + i0 + q) = make_uint2(kk[q] | (kk[q + 1] << 16), kk[q + 2] | (kk[q + 3] << 16));
+                } else {
+#pragma unroll
+                    for (int q = 0; q < E; q++)
+                        if (i0 + q < n) keys[i0 + q] = (uint16_t)kk[q];
+                }
             }
             if (watch) {
 #pragma unroll
@@ -1786,16 +1820,6 @@ __device__ __forceinline__ int list_stretch(const float* p, int w0, int w1, bool
 // list, from which a nucleus of one slab is finished; one of several slabs has its members listed by one more read
 // of the row into the row's sort segment and is finished from there a block at a time.  Returns kNucleusDone, or
 // which general way the row has to go (nothing is written then but LDS and the row's sort segment).
-constexpr int kHistPos = 8192;
-constexpr uint32_t kHistTopKey = 0x3f80u;
-__device__ __forceinline__ void hist_count(uint32_t* hcnt, uint32_t* bad, float e)
-{
-    if (e > 0.0f) {
-        const uint32_t key = sr_f2u(e) >> 16;
-        if (key <= kHistTopKey) atomicAdd(&hcnt[min(kHistTopKey - key, (uint32_t)(kHistPos - 1))], 1u);
-        else *bad = 1u;  // (no e exceeds 1; if one does, the general way takes the row)
-    }
-}
 enum NucleusWay : int { kNucleusDone = 0, kNucleusGeneral = 1, kNucleusGeneralNoSlabs = 2 };
 constexpr int kNucleusMaxSlabs = 40;
 constexpr int kNucleusRowFinish = 4;  // a nucleus that took more slabs than this is finished by passes over the row
@@ -2342,6 +2366,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             }
             // A row that only top-p cuts and that is only sampled from: see nucleus_from_histogram
             const bool fast_nucleus = row_fast_nucleus(rd, a);
+            const bool walked = a.seg_func != nullptr && (!fast_nucleus || a.seg_keys != nullptr);
             if (fast_nucleus) {
                 uint32_t* hcnt = (uint32_t*)sm.sortbuf;
                 for (int i = tid; i < kHistPos; i += kT) hcnt[i] = 0u;
@@ -2349,13 +2374,33 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                 __syncthreads();
             }
             float sum;
-            if (a.seg_func && !fast_nucleus) {
+            if (walked) {
                 // the whole device has prepared the sum (k_full_exp_seg): one wave walks the segments' records, and the
                 // entries that can survive the min-p cut were listed by the same pass
                 __syncthreads();
                 if (sr_wave_id() == 0) {
                     const float s = seg_walk<false>(p, n, a.seg_func + (size_t)slot * a.seg_stride, 0.0f, 0.0f, &dummy, nullptr);
                     if (sr_lane() == 0) sm.segbc[0] = sr_f2u(s);
+                } else if (fast_nucleus) {
+                    // the histogram of e from the 16 bits per entry that the expf pass left
+                    uint32_t* hcnt = (uint32_t*)sm.sortbuf;
+                    const uint16_t* keys = a.seg_keys + (size_t)slot * (size_t)a.seg_key_stride;
+                    auto count = [&](uint32_t key) {
+                        if (key != 0u) {
+                            if (key <= kHistTopKey) atomicAdd(&hcnt[min(kHistTopKey - key, (uint32_t)(kHistPos - 1))], 1u);
+                            else sm.bc[5] = 1u;  // (no e exceeds 1; if one does, the general way takes the row)
+                        }
+                    };
+                    const int n8 = n / 8;  // (the rows of keys start on 16-byte boundaries)
+                    for (int v0 = tid - SR_WAVE; v0 < n8; v0 += 2 * (kT - SR_WAVE)) {
+                        const int v1 = v0 + (kT - SR_WAVE);
+                        const uint4 ka = ((const uint4*)keys)[v0];
+                        const uint4 kb = v1 < n8 ? ((const uint4*)keys)[v1] : make_uint4(0u, 0u, 0u, 0u);
+                        const uint32_t ww[8] = {ka.x, ka.y, ka.z, ka.w, kb.x, kb.y, kb.z, kb.w};
+#pragma unroll
+                        for (int q = 0; q < 8; q++) { count(ww[q] & 0xffffu); count(ww[q] >> 16); }
+                    }
+                    for (int i = n8 * 8 + tid - SR_WAVE; i < n; i += kT - SR_WAVE) count(keys[i]);
                 } else if (watch_min_p) {
                     const uint32_t cw = a.watch_cnt[slot];
                     const unsigned long long* wl = a.watch + (size_t)slot * kSmall;

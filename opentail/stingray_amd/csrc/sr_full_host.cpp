@@ -92,6 +92,11 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
             a.seg_stride = nseg;
             a.watch = ctx->full_watch.as<unsigned long long>();
             a.watch_cnt = ctx->full_watch_cnt.as<uint32_t>();
+            if (any_top_p && mode == 0) {
+                a.seg_key_stride = ((int64_t)vocab + 7) & ~(int64_t)7;
+                SR_HIP(ctx, ctx->full_seg_keys.reserve((size_t)n_rows * (size_t)a.seg_key_stride * sizeof(uint16_t), st));
+                a.seg_keys = ctx->full_seg_keys.as<uint16_t>();
+            }
         }
     }
     a.uniforms = b->d_uniforms.as<double>();

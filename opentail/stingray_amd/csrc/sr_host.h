@@ -199,7 +199,7 @@ struct sr_ctx {
     DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
     DeviceBuf spec_resid, spec_reject;  // ... the residual row of every row's first rejected position, that position
     DeviceBuf seg_part, seg_func;       // approximate sums and increment functions of the segments of prepared rows
-    DeviceBuf full_seg_func, full_seg_ms, full_watch, full_watch_cnt;  // ... of the full-vocabulary path's denominators
+    DeviceBuf full_seg_func, full_seg_ms, full_watch, full_watch_cnt, full_seg_keys;  // ... of the full-vocabulary path's denominators
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
     int last_epv = 4;                    // vector width of the last launch: what an upload builds scan masks for

@@ -174,6 +174,8 @@ struct SrFullArgs {
     int32_t seg_stride;
     unsigned long long* watch;     // [slot][SR_FULL_SMALL_CAP]: the entries that can survive a row's min-p cut (value << 32 | ~index)
     uint32_t* watch_cnt;           // [slot]
+    uint16_t* seg_keys;            // [slot][seg_key_stride]: the upper 16 bits of every e of a row that only top-p cuts (0: e = 0)
+    int64_t seg_key_stride;
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, hipStream_t st);
