@@ -24,6 +24,14 @@ SR_API int sr_selftest_expf(sr_ctx* ctx, const float* x_dev, float* y_dev, int64
 SR_API int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float s0, float target, float* out_sum_dev,
                               int32_t* out_idx_dev);
 
+/* The same sum and search the way the full-vocabulary path prepares long rows: the whole device turns every 1,024 terms
+ * into a record for the binade that an approximate prefix sum predicts, and one wave walks the records.  `skew`
+ * multiplies the approximate sums (1 = as in production; other values make the predictions miss: the results must
+ * not change).  out_sum_dev[2], out_idx_dev[2]: [0] the sum and the search from the states the sum left, [1] the
+ * running sum and index of the walk that searches by itself.  n <= 1,048,576. */
+SR_API int sr_selftest_segsum(sr_ctx* ctx, const float* x_dev, int32_t n, double skew, float target, float* out_sum_dev,
+                              int32_t* out_idx_dev);
+
 /* How many sr_batch_append_tokens calls on this batch rebuilt it instead of updating it in place. */
 SR_API int sr_debug_append_rebuilds(const sr_batch* batch);
 /* ... and how many rows such calls moved to the end of the batch's edit array because they had run out of room. */

@@ -3375,6 +3375,37 @@ __global__ __launch_bounds__(kT) void k_selftest_seqsum(const float* x, int n, f
         s = seq_sum_row<false>(x, n, s0, 0.0f, &found, sm);
     if (threadIdx.x == 0) { *out_sum = s; *out_idx = found; }
 }
+// The same sum the prepared way: approximate sums of the segments (times `skew`, to make the predictions miss), the
+// segments' records, and the walk of one wave -- the sum with the states it leaves and the search from those states
+// (out[0], idx[0]), and the walk that searches by itself (out[1], idx[1]).
+__global__ __launch_bounds__(256) void k_selftest_segpart(const float* x, int n, double skew, double* part)
+{
+    const int seg = (int)blockIdx.x * 4 + sr_wave_id(), lane = sr_lane();
+    if (seg >= seg_count(n)) return;
+    double acc = 0.0;
+    for (int j = 0; j < SR_SEQ_RUN; j++) {
+        const int i = seg * SR_SEG_TERMS + lane * SR_SEQ_RUN + j;
+        if (i < n) acc += (double)x[i];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+    if (lane == 0) part[seg] = acc * skew;
+}
+__global__ __launch_bounds__(kT) void k_selftest_segwalk(const float* x, int n, const SeqSegFunc* funcs, float target, float* out_sum,
+                                                          int* out_idx)
+{
+    __shared__ FullSmem sm;
+    if (sr_wave_id() != 0) return;
+    int found = -1, found2 = -1;
+    const float s = seg_walk<false>(x, n, funcs, 0.0f, 0.0f, &found, sm.segst);
+    float s2 = s;
+    if (target == target) {
+        float at = 0.0f;
+        found = seg_search_states(x, n, sm.segst, target, &at);
+        s2 = seg_walk<true>(x, n, funcs, 0.0f, target, &found2, nullptr);
+    }
+    if (sr_lane() == 0) { out_sum[0] = s; out_sum[1] = s2; out_idx[0] = found; out_idx[1] = found2; }
+}
 #endif
 
 }  // namespace
@@ -3495,6 +3526,16 @@ hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float targ
                                      hipStream_t st)
 {
     hipLaunchKernelGGL(k_selftest_seqsum, dim3(1), dim3(kT), 0, st, x, n, s0, target, out_sum, out_idx);
+    return hipGetLastError();
+}
+hipError_t sr_launch_selftest_segsum(const float* x, int n, double skew, float target, double* part, SeqSegFunc* funcs,
+                                     float* out_sum, int* out_idx, hipStream_t st)
+{
+    const int nseg = (n + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
+    hipLaunchKernelGGL(k_selftest_segpart, dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, st, x, n, skew, part);
+    hipLaunchKernelGGL(k_seq_funcs, dim3((unsigned)((nseg + 3) / 4), 1), dim3(256), 0, st, x, (int64_t)0, n, part, funcs, nseg,
+                       (const int32_t*)nullptr);
+    hipLaunchKernelGGL(k_selftest_segwalk, dim3(1), dim3(kT), 0, st, x, n, funcs, target, out_sum, out_idx);
     return hipGetLastError();
 }
 #endif

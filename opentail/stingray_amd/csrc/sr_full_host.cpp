@@ -509,6 +509,22 @@ int sr_selftest_seqsum(sr_ctx* ctx, const float* x_dev, int32_t n, float s0, flo
     SR_HIP(ctx, sr_launch_selftest_seqsum(x_dev, n, s0, target, out_sum_dev, out_idx_dev, ctx->stream));
     return SR_OK;
 }
+// Test hook: the same sum as the whole device prepares it (segments' records made for predictions that are `skew`
+// times the segments' true sums, the walk of one wave): out_sum_dev[0], out_idx_dev[0] from the sum and the search
+// over its states, [1] from the walk that searches by itself
+int sr_selftest_segsum(sr_ctx* ctx, const float* x_dev, int32_t n, double skew, float target, float* out_sum_dev,
+                       int32_t* out_idx_dev)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    if (n <= 0 || (n + SR_SEG_TERMS - 1) / SR_SEG_TERMS > SR_SEG_MAX) return sr_fail(ctx, SR_ERR_INVALID_ARGUMENT, "sr_selftest_segsum: length");
+    SR_HIP(ctx, hipSetDevice(ctx->device));
+    const size_t nseg = (size_t)(n + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
+    SR_HIP(ctx, ctx->seg_part.reserve(nseg * sizeof(double), ctx->stream));
+    SR_HIP(ctx, ctx->seg_func.reserve(nseg * sizeof(SeqSegFunc), ctx->stream));
+    SR_HIP(ctx, sr_launch_selftest_segsum(x_dev, n, skew, target, ctx->seg_part.as<double>(), (SeqSegFunc*)ctx->seg_func.p,
+                                          out_sum_dev, out_idx_dev, ctx->stream));
+    return SR_OK;
+}
 #endif  // SR_TEST_HOOKS
 
 }  // extern "C"

@@ -235,3 +235,5 @@ hipError_t sr_launch_mtp_verify(const float* logits, int64_t stride, int n, int 
                                 int* out_argmax, int* out_accept, float* out_prob, hipStream_t st);
 hipError_t sr_launch_selftest_seqsum(const float* x, int n, float s0, float target, float* out_sum, int* out_idx,
                                      hipStream_t st);
+hipError_t sr_launch_selftest_segsum(const float* x, int n, double skew, float target, double* part, SeqSegFunc* funcs,
+                                     float* out_sum, int* out_idx, hipStream_t st);

@@ -44,6 +44,7 @@ def hooks_lib():
         vp = C.c_void_p
         H.sr_selftest_expf.argtypes = [vp, vp, vp, C.c_int64]
         H.sr_selftest_seqsum.argtypes = [vp, vp, C.c_int32, C.c_float, C.c_float, vp, vp]
+        H.sr_selftest_segsum.argtypes = [vp, vp, C.c_int32, C.c_double, C.c_float, vp, vp]
         H.sr_debug_append_rebuilds.argtypes = [vp]
         H.sr_debug_append_moves.argtypes = [vp]
         H.sr_debug_set_spin_limit.argtypes = [vp, C.c_uint32]

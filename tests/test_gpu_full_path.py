@@ -73,6 +73,51 @@ def test_exact_running_sum_matches_the_left_to_right_loop(ctx):
     assert _gpu_seq_sum(ctx, x, 0.75)[0].tobytes() == orc.seq_sum(x, 0.75)[0].tobytes()
 
 
+def test_sums_prepared_by_the_whole_device_do_not_depend_on_the_predictions(ctx):
+    """The records of a row's segments are made for binades that approximate sums predict; the walk checks every
+    record against the exact running sum and adds from the terms where one does not fit.  With predictions that are
+    right, half, double and nothing of the truth, on rows that are ragged, misaligned, flat, peaked and sparse, the sum
+    and the searches must be those of the left-to-right loop."""
+    import torch
+
+    rng = np.random.default_rng(11)
+    rows = []
+    for n in (1, 15, 1024, 1025, 4096, 5000, 40000, 151936, 262144):
+        z = rng.normal(0, 2.5, n)
+        rows.append(np.exp(z - z.max()).astype(np.float32))
+    rows.append(rng.random(70001).astype(np.float32))                                    # flat: one binade for long
+    big = np.exp(rng.normal(0, 1.0, 60000)).astype(np.float32)
+    big[[100, 20000, 20001, 59999]] = [3.0e4, 7.0e5, 9.0e5, 2.0e7]                       # jumps over several binades
+    rows.append(big)
+    sparse = np.zeros(90000, dtype=np.float32)
+    sparse[rng.integers(0, 90000, 300)] = rng.random(300).astype(np.float32)             # a residual-like row
+    rows.append(sparse)
+    rows.append(np.zeros(3000, dtype=np.float32))
+    rows.append(np.concatenate([[1.0], np.full(50000, 2.0 ** -24)]).astype(np.float32))   # every add half way
+    s = torch.zeros(2, dtype=torch.float32, device="cuda")
+    idx = torch.zeros(2, dtype=torch.int32, device="cuda")
+    H = hooks_lib()
+    for x in rows:
+        for shift in (0, 1):                                                             # rows that start off a 16-byte boundary
+            buf = _cuda(np.concatenate([np.zeros(shift, np.float32), x]))
+            ptr = buf.data_ptr() + 4 * shift
+            want, _ = orc.seq_sum(x)
+            for skew in (1.0, 0.5, 2.0, 0.0, 1.0 + 1e-4):
+                for frac in (float("nan"), 0.0, 1e-9, 0.31, 0.77, 0.999999, 1.5):
+                    tgt = np.float32(frac * float(want)) if frac == frac else np.float32("nan")
+                    ctx._check(H.sr_selftest_segsum(ctx.h, C.c_void_p(ptr), len(x), skew, float(tgt),
+                                                    C.c_void_p(s.data_ptr()), C.c_void_p(idx.data_ptr())))
+                    ctx.synchronize()
+                    gs, gi = s.cpu().numpy(), idx.cpu().numpy()
+                    assert gs[0].tobytes() == want.tobytes(), (len(x), shift, skew, gs[0], want)
+                    if frac == frac:
+                        ws, wi = orc.seq_sum(x, 0.0, float(tgt))
+                        assert gi[0] == wi and gi[1] == wi, (len(x), shift, skew, frac, gi, wi)
+                        if wi >= 0:  # (the walk that searches hands back the running sum at the term it stops at)
+                            at = orc.seq_sum(x[: wi + 1])[0]
+                            assert gs[1].tobytes() == at.tobytes(), (len(x), skew, frac, gs[1], at)
+
+
 def _check_rows(ctx, logits, params, uniforms, allow_mask=None, mask_active=None):
     got, flags = ctx.sample_batch(_cuda(logits), params, uniforms, allow_mask, mask_active, return_flags=True)
     want = oracle_tokens(logits, params, uniforms, allow_mask, mask_active)
