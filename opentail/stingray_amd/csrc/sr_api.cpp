@@ -256,8 +256,10 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     b->scan_chunk_vecs = chunk_vecs;
     b->scan_base_addr = base_addr;
     b->scan_stride_bytes = stride_bytes;
-    if (rows_changed)
+    if (rows_changed) {
+        b->spec_positions = 0;
         SR_HIP(ctx, batch_copy(b, staged, b->d_rows.p, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow), st));
+    }
     SR_HIP(ctx, b->d_scan_desc.reserve(b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, batch_copy(b, staged, b->d_scan_desc.p, b->h_scan.data(), b->h_scan.size() * sizeof(SrScanDesc), st));
     SR_HIP(ctx, b->d_scan_mask.reserve(b->h_scan.size() * (size_t)b->scan_stride * sizeof(uint32_t), st));
@@ -314,7 +316,7 @@ void sr_destroy(sr_ctx* ctx)
     DeviceBuf* bufs[] = {&ctx->cand, &ctx->gmax, &ctx->gmax2, &ctx->gpos, &ctx->gbound, &ctx->row_done, &ctx->argmax_best, &ctx->argmax_done, &ctx->mask_pool, &ctx->mask_any,
                          &ctx->work, &ctx->edit_tab, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->full_state, &ctx->sort_k0, &ctx->sort_v0,
-                         &ctx->sort_v1, &ctx->ident, &ctx->redo_list, &ctx->spec_rows, &ctx->spec_probs, &ctx->spec_resid, &ctx->spec_reject,
+                         &ctx->sort_v1, &ctx->ident, &ctx->redo_list, &ctx->spec_probs, &ctx->spec_resid, &ctx->spec_reject,
                          &ctx->seg_part, &ctx->seg_func, &ctx->full_seg_func, &ctx->full_seg_ms, &ctx->full_watch, &ctx->full_watch_cnt, &ctx->full_seg_keys};
     for (DeviceBuf* b : bufs) b->release();
     ctx->uni_ring.release();
@@ -374,7 +376,7 @@ void sr_batch_destroy(sr_batch* b)
     if (!b) return;
     if (b->ctx) (void)hipStreamSynchronize(b->ctx->stream);
     DeviceBuf* bufs[] = {&b->d_rows, &b->d_edits, &b->d_sel_list, &b->d_full_list, &b->d_wide_list, &b->d_scan_desc,
-                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched};
+                         &b->d_mask, &b->d_scan_mask, &b->d_uniforms, &b->d_sched, &b->spec_rows};
     for (DeviceBuf* d : bufs) d->release();
     b->stage.release();
     b->patch_ring.release();
@@ -638,6 +640,7 @@ static int batch_upload_impl(sr_batch* b, int32_t rows, int32_t vocab, const sr_
         if (e != hipSuccess) return e;
         return batch_copy(b, true, dst.p, src, bytes, st);
     };
+    b->spec_positions = 0;
     SR_HIP(ctx, up(b->d_rows, b->h_rows.data(), b->h_rows.size() * sizeof(SrRow)));
     // (the edit lists of a batch that tokens are appended to grow with every rebuild: room for four times their size, so
     // that a rebuild finds its device memory in place)
@@ -906,6 +909,7 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     if (!rp_d || !ep_d || !mc_d || !un_d || !sa_d) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "sr_batch_append_tokens: no pinned memory");
     // scan masks that are not built yet are built from the patched edits when they are needed
     const bool masks = b->scan_epv != 0 && b->d_scan_mask.p != nullptr;
+    b->spec_positions = 0;
     SR_HIP(ctx, sr_launch_apply_patches(b->d_rows.as<SrRow>(), rp_d, (int)rp.size(), b->d_edits.as<SrEdit>(), ep_d,
                                         (int)ep.size(), mc_d, masks ? (int)mc.size() : 0, b->d_scan_mask.as<uint32_t>(),
                                         b->scan_stride, masks ? b->scan_epv : 4, masks ? b->scan_chunk_vecs : 64,

@@ -434,15 +434,19 @@ int sr_spec_verify_launch(sr_ctx* ctx, const sr_batch* b, const float* target_lo
         return sr_fail(ctx, SR_ERR_UNSUPPORTED, "sr_spec_verify_launch: rows x positions x vocab exceeds 2^31 entries");
     bool any_top_p = false;
     for (int r = 0; r < rows; r++) any_top_p = any_top_p || row_uses_top_p(b->h_rows[(size_t)r]);
-    SR_HIP(ctx, ctx->spec_rows.reserve((size_t)rows * P * sizeof(SrRow), st));
-    SR_HIP(ctx, sr_launch_expand_rows(b->d_rows.as<SrRow>(), ctx->spec_rows.as<SrRow>(), rows, P, st));  // (no wait for the host)
+    // (made by a kernel, so that the call does not wait for the host; kept with the batch until its descriptors change)
+    if (b->spec_positions != P) {
+        SR_HIP(ctx, b->spec_rows.reserve((size_t)rows * P * sizeof(SrRow), st));
+        SR_HIP(ctx, sr_launch_expand_rows(b->d_rows.as<SrRow>(), b->spec_rows.as<SrRow>(), rows, P, st));
+        b->spec_positions = P;
+    }
     SR_HIP(ctx, ctx->spec_probs.reserve((size_t)rows * P * V * sizeof(float), st));
     sr_batch tmp;  // a view: expanded rows, the original edits
     tmp.ctx = ctx;
     tmp.rows = rows * P;
     tmp.vocab = V;
     tmp.upr = 0;
-    tmp.d_rows.p = ctx->spec_rows.p;
+    tmp.d_rows.p = b->spec_rows.p;
     tmp.d_edits.p = b->d_edits.p;
     tmp.mask_stride = 0;
     const int32_t* list = nullptr;

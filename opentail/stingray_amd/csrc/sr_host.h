@@ -196,7 +196,7 @@ struct sr_ctx {
     DeviceBuf ident;         // identity row list
     DeviceBuf redo_list;     // rows given to sr_resample_rows_launch
     int ident_rows = 0;
-    DeviceBuf spec_rows, spec_probs;  // speculative verification: expanded rows, target distributions
+    DeviceBuf spec_probs;    // speculative verification: the target distributions of every position
     DeviceBuf spec_resid, spec_reject;  // ... the residual row of every row's first rejected position, that position
     DeviceBuf seg_part, seg_func;       // approximate sums and increment functions of the segments of prepared rows
     DeviceBuf full_seg_func, full_seg_ms, full_watch, full_watch_cnt, full_seg_keys;  // ... of the full-vocabulary path's denominators
@@ -235,6 +235,10 @@ struct sr_batch {
     std::vector<SrScanDesc> h_scan;    // scan-mask rows of the selection kernel
     std::vector<uint32_t> h_scan_need; // per batch row: SR_SCAN_* bits the row's scan mask must carry
     DeviceBuf d_rows, d_edits, d_sel_list, d_full_list, d_wide_list, d_scan_desc, d_mask, d_scan_mask, d_uniforms, d_sched;
+    // speculative verification: the rows' descriptors, one copy per position, for `spec_positions` positions (0: to be
+    // made again, because the descriptors have changed since)
+    mutable DeviceBuf spec_rows;
+    mutable int spec_positions = 0;
     int64_t mask_stride = 0, scan_stride = 0;
     // what the scan masks were built for: elements per 16-byte vector, the logits base address modulo 16 and
     // the row stride in bytes modulo 16 (rows share a mask row only when all start at the same offset)
