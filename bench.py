@@ -147,6 +147,11 @@ def bench_spec(args, w, ctx, stream) -> dict:
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
+    if args.copy_probe:
+        probe = torch.empty_like(sets[0][0])
+        for _ in range(3):
+            probe.copy_(sets[0][0])   # reads and writes rows * (L + 1) * V * 4 bytes
+        torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record(stream)
@@ -194,14 +199,24 @@ def bench_spec(args, w, ctx, stream) -> dict:
         "data": "synthetic (target = draft + N(0, .5^2), q = softmax(draft), 2 rotated resident sets)",
         "config": {"workload": "c5", "rows": rows, "n_draft": L, "vocab": V, "mean_tokens_emitted_per_row": emitted},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": committed_traffic("c5"),
+                     "traffic_source": "profiles/traffic_c5.json.txt: rocprofv3 --pmc runs of this command, whole step, committed; not measured by this run",
+                     "algorithmic_bytes_per_launch": alg_bytes,
                      "bytes_with_bonus_position_for_every_row": bytes_with_bonus, "bytes_reading_every_input": bytes_everything,
-                     "kernel": "k_full_row", "kernel_us": dev_us},
+                     "kernel": "k_full_exp_seg", "kernel_us": dev_us},
         "cpu_baseline": cpu, "parity": parity,
     }
     for _, _, _, b, _, _ in sets:
         b.close()
     return out_j
+
+
+def committed_traffic(workload):
+    """HBM bytes per step from the committed counter summary of this workload (profiles/traffic_<workload>.json.txt), or None."""
+    try:
+        return json.load(open(os.path.join(ROOT, "profiles", f"traffic_{workload}.json.txt"))).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
 
 
 def bench_argmax(args, ctx, stream) -> dict:
@@ -425,7 +440,7 @@ def run_workload(args, ctx, stream) -> dict:
                      "traffic_source": None if traffic is None else
                      f"profiles/{os.path.basename(tpath)}: rocprofv3 --pmc runs of this command, committed; not measured by this run",
                      "algorithmic_bytes_per_launch": alg_bytes,
-                     "kernel": "k_topk_rows" if args.workload.startswith(("c1", "c3")) else "k_full_row",
+                     "kernel": "k_topk_rows" if args.workload.startswith(("c1", "c3")) else ("k_full_exp_seg" if args.workload == "c2" else "k_full_row"),
                      "kernel_us": kern_us},
         "cpu_baseline": cpu,
         "parity": parity,

@@ -900,7 +900,9 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     const size_t n_uni = (uniforms && b->upr > 0) ? (size_t)rows * (size_t)b->upr : 0;
     const size_t need = rp.size() * sizeof(SrRowPatch) + ep.size() * sizeof(SrEditPatch) + mc.size() * sizeof(SrMaskClear) +
                         n_uni * sizeof(double) + scan_again.size() * sizeof(int32_t) + 5 * 256;
-    SR_HIP(ctx, b->patch_ring.begin(need, st));
+    // (a ring that is made now is made for the largest call to come as well: every row of the batch out of room at once,
+    // all edits sent again -- rows that were uploaded together run out of room together)
+    SR_HIP(ctx, b->patch_ring.begin(need, st, b->h_edits.size() * sizeof(SrEditPatch) + (size_t)rows * 64 + n_uni * sizeof(double) + 65536));
     const SrRowPatch* rp_d = (const SrRowPatch*)b->patch_ring.put(rp.data(), rp.size() * sizeof(SrRowPatch));
     const SrEditPatch* ep_d = (const SrEditPatch*)b->patch_ring.put(ep.data(), ep.size() * sizeof(SrEditPatch));
     const SrMaskClear* mc_d = (const SrMaskClear*)b->patch_ring.put(mc.data(), mc.size() * sizeof(SrMaskClear));

@@ -117,7 +117,8 @@ struct HostRing {
     bool dirty = false;             // pieces handed out since the last wait for a whole stream
     hipStream_t last = nullptr;     // the stream of those pieces' kernels
     // room for `need` bytes in the present half (its pieces are handed out by put)
-    hipError_t begin(size_t need, hipStream_t st)
+    // (want_half: what a half should hold when the ring has to be made or made again anyway)
+    hipError_t begin(size_t need, hipStream_t st, size_t want_half = 0)
     {
         hipError_t e = hipSuccess;
         if (dirty && st != last) {  // the caller changed streams: nothing orders the old stream's readers before new events
@@ -132,7 +133,9 @@ struct HostRing {
             p = nullptr;
             half = used = 0;
             pending[0] = pending[1] = dirty = false;
-            const size_t want = 16 * need + 65536;
+            // (room for many calls of the usual size; a call that needs much -- every row of a batch moving its edits at
+            // once -- gets room for two of its kind: pinned memory is slow to allocate)
+            const size_t want = std::max(want_half, (need <= 65536 ? 16 * need : 2 * need) + 65536);
             if ((e = hipHostMalloc((void**)&p, 2 * want, hipHostMallocDefault)) != hipSuccess) { p = nullptr; return e; }
             half = want;
             cur = 0;
