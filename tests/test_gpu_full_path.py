@@ -553,21 +553,25 @@ def test_bf16_and_unaligned_rows_on_the_full_path(ctx):
     import torch
 
     rng = np.random.default_rng(78)
-    for V, pad in [(10_007, 3), (4_096, 0), (33_001, 6)]:
-        rows = 6
+    # (rows of 4,096 entries and more that start on 16-byte boundaries have their sums prepared by the whole device, in
+    # segments of 1,024: 40,968 and 50,004 end in a ragged segment, 50,004 is aligned as fp32 only, 8,200 + 8 by its padding)
+    for V, pad in [(10_007, 3), (4_096, 0), (33_001, 6), (40_968, 0), (50_004, 0), (8_200, 8)]:
+        rows = 8
         f32 = rng.normal(0, 2.0, (rows, V)).astype(np.float32)
         bf = (f32.view(np.uint32) >> 16).astype(np.uint16)
         exact = (bf.astype(np.uint32) << 16).view(np.float32)             # what the bf16 tensor holds
         allowed = rng.random((rows, V)) < 0.7
         mask = pack_allow_mask(allowed)
-        active = np.array([0, 1, 0, 1, 0, 0], dtype=np.uint8)
+        active = np.array([0, 1, 0, 1, 0, 0, 1, 0], dtype=np.uint8)
         hist = rng.integers(0, V, 200).tolist()
         params = [SamplingParams(Temperature=0.9, TopP=0.9),                                   # nothing edits the row
                   SamplingParams(Temperature=1.0, TopP=0.95, MinP=0.001),
                   SamplingParams(Temperature=0.7, LogitBias={5: 3.0, V - 1: -2.0, 17: 1.5}, TopK=50, TopP=0.9),
                   SamplingParams(Temperature=1.2, RepetitionPenalty=1.3, FrequencyPenalty=0.2, PreviousTokens=hist),
                   SamplingParams(Temperature=0.0, LogitBias={3: 100.0}),                        # greedy ignores the bias
-                  SamplingParams(Temperature=1.0)]
+                  SamplingParams(Temperature=1.0),
+                  SamplingParams(Temperature=0.8, MinP=0.02, PresencePenalty=0.5, PreviousTokens=hist[:40]),   # min-p alone, edits
+                  SamplingParams(Temperature=0.6, TopP=0.97, FrequencyPenalty=0.3, PreviousTokens=hist[:90])]  # top-p alone, edits
         for logits, dev in [(exact, _strided(bf.view(np.int16), pad, torch.bfloat16)), (f32, _strided(f32, pad))]:
             for _ in range(2):
                 u = rng.random(rows)
