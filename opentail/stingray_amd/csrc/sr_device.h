@@ -171,6 +171,19 @@ __device__ __forceinline__ unsigned long long sr_wave_max_u64(unsigned long long
     }
     return r;
 }
+// the sum of v over the wave, single precision, the same in every lane (the order of the additions is the reduction's own)
+__device__ __forceinline__ float sr_wave_sum_f32(float v)
+{
+    v += __uint_as_float(sr_dpp_u32<kDppXor1>(__float_as_uint(v)));
+    v += __uint_as_float(sr_dpp_u32<kDppXor2>(__float_as_uint(v)));
+    v += __uint_as_float(sr_dpp_u32<kDppHalfMirror>(__float_as_uint(v)));
+    v += __uint_as_float(sr_dpp_u32<kDppMirror>(__float_as_uint(v)));
+    const float a = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 0));
+    const float b = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 16));
+    const float c = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 32));
+    const float d = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), 48));
+    return (a + b) + (c + d);
+}
 // inclusive prefix sum across the wave, single precision (the order of the additions is the scan's own)
 __device__ __forceinline__ float sr_wave_incl_sum_f32(float v)
 {

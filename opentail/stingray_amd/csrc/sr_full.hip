@@ -466,9 +466,28 @@ __device__ __forceinline__ float seg_walk(const float* terms, int n, const SeqSe
 
 // The record of one segment (SeqSegFunc) from its terms x (lane l holds the terms 16 l ... 16 l + 15 of the segment) and
 // the approximate sum `before` of everything in front of the segment.  One wave.
-__device__ __forceinline__ void seg_make_record(const float (&x)[SR_SEQ_RUN], int seg, double before, SeqSegFunc* out)
+// With `seg_sum` (>= 0: the approximate sum of the segment's own terms, known beforehand) a segment whose start and
+// end lie well inside one binade gets its one function without a look at where inside it the sum would change binade.
+__device__ __forceinline__ void seg_make_record(const float (&x)[SR_SEQ_RUN], int seg, double before, SeqSegFunc* out,
+                                                float seg_sum = -1.0f)
 {
     const int lane = sr_lane();
+    if (seg > 0 && seg_sum >= 0.0f) {
+        const float lo = __double2float_rn(before), hi = lo + seg_sum;
+        uint32_t nn;
+        int eb_lo, eb_hi;
+        sr_split(lo * 0.9999f, &nn, &eb_lo);
+        sr_split(hi * 1.0001f, &nn, &eb_hi);
+        if (eb_lo == eb_hi) {  // (wave-uniform: both are the same in every lane)
+            const SrInc sc = sr_scan_inc<false>(sr_run_inc(x, eb_lo));
+            if (lane == SR_WAVE - 1) {
+                uint4* q = (uint4*)out;
+                q[0] = make_uint4(sc.a0, sc.a1, (uint32_t)eb_lo, SR_SEG_PLAIN);
+                q[1] = make_uint4(SR_SEQ_SAT, SR_SEQ_SAT, (uint32_t)eb_lo, 0u);
+            }
+            return;
+        }
+    }
     // approximate running sum behind every lane's run (single precision does: a prediction that misses costs time only)
     float own = 0.0f;
 #pragma unroll
@@ -1410,7 +1429,9 @@ __global__ __launch_bounds__(256) void k_full_exp_seg(SrFullArgs a)
     if (mk == 0xffffffffu || mk <= 0x007fffffu) return;  // NaN, or nothing above -inf: the row kernel makes it uniform
     const float m = sr_okey_inv(mk);
     __shared__ uint64_t tab[32];  // the expf table: a lookup per element from global memory is a long dependent load
-    __shared__ float4 turn[4][SR_SEG_TERMS / 4];  // a wave's segment on its way from the order of the loads to 16 terms a lane
+    // a wave's segment on its way from the order of the loads to 16 terms a lane: a lane's 16 terms lie together, 16
+    // bytes apart from the next lane's, so that neither the stores nor the loads of 16 bytes a lane collide on a bank
+    __shared__ float4 turn[4][SR_WAVE * 5];
     // A row that only top-p cuts needs the histogram of its e by their upper 16 bits.  Counting it here took longer
     // than it saved (one atomic per element in device memory: +30 us; in shared memory, by few workgroups that take
     // many segments each: +55 us), so the pass leaves those 16 bits of every e beside the row, and the row's workgroup
@@ -1428,15 +1449,18 @@ __global__ __launch_bounds__(256) void k_full_exp_seg(SrFullArgs a)
     for (int seg = (int)blockIdx.x * 4 + wave; seg < nseg; seg += (int)gridDim.x * 4) {
         float x[SR_SEQ_RUN], e[SR_SEQ_RUN];
         seg_load_logits<ES>(src, seg, lane, n, x);
-        // (the approximate sum in front of the segment, under the loads)
-        double before = 0.0;
+        // (the approximate sums in front of the segment and of the segment itself, under the loads; single precision
+        // does: a prediction that misses costs time only)
+        float before = 0.0f, own_sum = 0.0f;
         if (record) {
-            for (int g = lane; g < seg; g += SR_WAVE) {
+            for (int g = lane; g <= seg; g += SR_WAVE) {
                 const float2 v = ms[g];
-                if (v.y > 0.0f) before += (double)(v.y * __expf(v.x - m));
+                const float t = v.y > 0.0f ? v.y * __expf(v.x - m) : 0.0f;
+                if (g < seg) before += t;
+                else own_sum = t;
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o);
+            before = sr_wave_sum_f32(before);
+            own_sum = sr_wave_sum_f32(own_sum);
         }
 #pragma unroll
         for (int k = 0; k < K; k++) {
@@ -1485,20 +1509,22 @@ __global__ __launch_bounds__(256) void k_full_exp_seg(SrFullArgs a)
 #pragma unroll
             for (int k = 0; k < K; k++)
 #pragma unroll
-                for (int q = 0; q < E; q += 4)
-                    mine[((k * SR_WAVE + lane) * E + q) / 4] = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+                for (int q = 0; q < E; q += 4) {
+                    const int i = (k * SR_WAVE + lane) * E + q;  // the element's place in the segment
+                    mine[(i >> 4) * 5 + ((i & 15) >> 2)] = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+                }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             float t[SR_SEQ_RUN];
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const float4 v = mine[lane * 4 + k];
+                const float4 v = mine[lane * 5 + k];
                 t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
             }
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             __builtin_amdgcn_wave_barrier();
-            seg_make_record(t, seg, before, a.seg_func + (size_t)slot * a.seg_stride + seg);
+            seg_make_record(t, seg, (double)before, a.seg_func + (size_t)slot * a.seg_stride + seg, own_sum);
         }
     }
 }
