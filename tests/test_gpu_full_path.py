@@ -637,3 +637,30 @@ def test_min_p_rows_with_few_and_with_thousands_of_survivors(ctx):
     for r, p in enumerate(params):
         t, d = orc.sample_with_distribution(logits[r], to_oracle(p), orc.Rng(replay=[0.999999]))
         assert toks[r] == t and np.array_equal(probs[r].cpu().numpy().view(np.uint32), np.asarray(d, np.float32).view(np.uint32)), r
+
+
+def test_rows_with_more_edited_ids_than_the_table_holds_keep_an_adjusted_copy(ctx):
+    """A full-vocabulary row whose history touches thousands of distinct ids is not read from the logits by the two
+    passes over the device but from its adjusted copy -- also where those passes run over segments (long rows on
+    16-byte boundaries): tokens and distributions against the oracle, fp32 and bf16."""
+    import torch
+
+    rng = np.random.default_rng(123)
+    V = 20_480
+    f32 = rng.normal(0, 2.0, (4, V)).astype(np.float32)
+    bf = (f32.view(np.uint32) >> 16).astype(np.uint16)
+    exact = (bf.astype(np.uint32) << 16).view(np.float32)
+    long_hist = rng.permutation(V)[:5000].tolist() + rng.integers(0, V, 3000).tolist()
+    params = [SamplingParams(Temperature=0.9, TopP=0.9, RepetitionPenalty=1.2, FrequencyPenalty=0.1, RepeatLastN=0, PreviousTokens=long_hist),
+              SamplingParams(Temperature=1.1, MinP=0.01, PresencePenalty=0.4, RepeatLastN=0, PreviousTokens=long_hist[:4000]),
+              SamplingParams(Temperature=0.7, TopP=0.95, PreviousTokens=long_hist[:10]),
+              SamplingParams(Temperature=0.0, RepetitionPenalty=1.3, RepeatLastN=0, PreviousTokens=long_hist)]
+    for logits, dev in [(f32, _cuda(f32)), (exact, torch.from_numpy(bf.view(np.int16)).view(torch.bfloat16).cuda())]:
+        for _ in range(3):
+            u = rng.random(4)
+            got = ctx.sample_batch(dev, params, u)
+            assert np.array_equal(got, oracle_tokens(logits, params, u)), str(dev.dtype)
+        got = ctx.build_distribution(dev, params).cpu().numpy()
+        for r, p in enumerate(params):
+            want = orc.build_filtered_distribution(logits[r], to_oracle(p))
+            assert np.array_equal(got[r].view(np.uint32), want.view(np.uint32)), (str(dev.dtype), r)
