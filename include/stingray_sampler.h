@@ -165,9 +165,12 @@ SR_API int sr_batch_upload(sr_batch* batch, int32_t rows, int32_t vocab,
  * the few entries that change instead of a pass over every history.
  *   tokens    [rows] host array; a negative entry leaves its row's history as it is.
  *   uniforms  [rows x uniforms_per_row] for the next step, or NULL to keep those on the device.
- * Rows the in-place update does not cover (the first history token of a row with penalties, a row that runs out of
- * the room it was given for new ids -- 32 and more per row --, a top-k beyond 2,048 entries) make the call rebuild the
- * whole batch from the inputs it kept: same result, the cost of an upload.  A batch uploaded with allow-masks of its own returns
+ * A row that runs out of the room it was given for new ids (32 and more per row) moves to the end of the batch's edit
+ * array, with twice the room.  Rows the in-place update does not cover (the first history token of a row with penalties,
+ * a top-k beyond 2,048 entries, an edit array that is full) make the call rebuild the whole batch from the inputs it
+ * kept: same result, the cost of an upload.  A call that fails after it has changed the host's copies leaves the batch
+ * marked, and the next call rebuilds it.  Like sr_sample_launch, the call keeps host-side state and must not be
+ * recorded into a HIP graph.  A batch uploaded with allow-masks of its own returns
  * SR_ERR_UNSUPPORTED (its masks change with every step: register them and use sr_batch_upload_mask_ids /
  * sr_batch_append_tokens_masks).  Copies run on the context's stream and are not waited for, as in sr_batch_upload. */
 SR_API int sr_batch_append_tokens(sr_batch* batch, const int32_t* tokens, const double* uniforms);

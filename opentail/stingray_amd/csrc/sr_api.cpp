@@ -335,7 +335,10 @@ static int switch_stream(sr_ctx* ctx, hipStream_t next)
 {
     // uploads of batches may still be running on the stream that is left: later launches are ordered behind them
     // only on the same stream
-    if (next != ctx->stream) SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (next != ctx->stream) {
+        SR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        ctx->stream_epoch++;  // (pinned rings of the context and its batches: nothing of the old stream reads them any more)
+    }
     ctx->stream = next;
     return SR_OK;
 }
@@ -766,7 +769,8 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     std::vector<SrEditPatch> ep;
     std::vector<SrMaskClear> mc;
     std::vector<int32_t> touched;
-    bool rebuild = false;
+    // (a call that failed after it had changed the host's copies left them ahead of the device: rebuild from the inputs)
+    bool rebuild = b->host_ahead;
     for (int32_t r = 0; r < rows && !rebuild; r++) {
         SrRow& d = b->h_rows[(size_t)r];
         bool mask_changed = false;
@@ -891,7 +895,10 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
     if (rebuild) {
         b->append_rebuilds++;
         if (new_mask_ids) b->keep_mask_ids.assign(new_mask_ids, new_mask_ids + rows);  // (the loop above stopped early)
-        return append_rebuild(b, uniforms);
+        b->host_ahead = true;
+        const int rc = append_rebuild(b, uniforms);
+        if (rc == SR_OK) b->host_ahead = false;
+        return rc;
     }
 
     // One kernel applies everything, reading the lists straight from the batch's pinned memory: no copy calls.
@@ -902,7 +909,9 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
                         n_uni * sizeof(double) + scan_again.size() * sizeof(int32_t) + 5 * 256;
     // (a ring that is made now is made for the largest call to come as well: every row of the batch out of room at once,
     // all edits sent again -- rows that were uploaded together run out of room together)
-    SR_HIP(ctx, b->patch_ring.begin(need, st, b->h_edits.size() * sizeof(SrEditPatch) + (size_t)rows * 64 + n_uni * sizeof(double) + 65536));
+    b->host_ahead = true;  // (until everything below has been enqueued)
+    SR_HIP(ctx, b->patch_ring.begin(need, st, b->h_edits.size() * sizeof(SrEditPatch) + (size_t)rows * 64 + n_uni * sizeof(double) + 65536,
+                                    ctx->stream_epoch));
     const SrRowPatch* rp_d = (const SrRowPatch*)b->patch_ring.put(rp.data(), rp.size() * sizeof(SrRowPatch));
     const SrEditPatch* ep_d = (const SrEditPatch*)b->patch_ring.put(ep.data(), ep.size() * sizeof(SrEditPatch));
     const SrMaskClear* mc_d = (const SrMaskClear*)b->patch_ring.put(mc.data(), mc.size() * sizeof(SrMaskClear));
@@ -923,6 +932,7 @@ static int append_impl(sr_batch* b, const int32_t* tokens, const double* uniform
                                               b->d_edits.as<SrEdit>(), sr_batch_mask_ptr(b), sr_batch_mask_stride(b),
                                               b->d_scan_mask.as<uint32_t>(), b->scan_stride, b->vocab, b->scan_epv,
                                               b->scan_chunks, b->scan_chunk_vecs, b->scan_base_addr, b->scan_stride_bytes, st));
+    b->host_ahead = false;
     return SR_OK;
 }
 
@@ -1305,7 +1315,15 @@ int sr_argmax_rows_launch(sr_ctx* ctx, const void* logits_dev, int dtype, int32_
     SrArgmaxArgs a = argmax_args(ctx, logits_dev, dtype, rows, vocab, row_stride_elems, out_idx_dev, out_val_dev);
     a.best = ctx->argmax_best.as<unsigned long long>();
     a.done = ctx->argmax_done.as<uint32_t>();
-    SR_HIP(ctx, sr_launch_argmax_rows(a, false, ctx->stream));
+    // (a launch that failed may have left slots and counters that are not zero: every later call would be wrong, silently)
+    if (ctx->argmax_scratch_dirty) {
+        SR_HIP(ctx, hipMemsetAsync(ctx->argmax_best.p, 0, ctx->argmax_best.cap, ctx->stream));
+        SR_HIP(ctx, hipMemsetAsync(ctx->argmax_done.p, 0, ctx->argmax_done.cap, ctx->stream));
+        ctx->argmax_scratch_dirty = false;
+    }
+    const hipError_t e = sr_launch_argmax_rows(a, false, ctx->stream);
+    if (e != hipSuccess) ctx->argmax_scratch_dirty = true;
+    SR_HIP(ctx, e);
     return SR_OK;
 }
 

@@ -140,7 +140,7 @@ int identity_list(sr_ctx* ctx, int rows, const int32_t** out)
 int upload_uniforms(sr_ctx* ctx, const double* uniforms, int rows, const double** dev)
 {
     const size_t bytes = (size_t)rows * sizeof(double);
-    SR_HIP(ctx, ctx->uni_ring.begin(bytes + 256, ctx->stream));
+    SR_HIP(ctx, ctx->uni_ring.begin(bytes + 256, ctx->stream, 0, ctx->stream_epoch));
     const void* at = ctx->uni_ring.put(uniforms, bytes);
     if (!at) return sr_fail(ctx, SR_ERR_OUT_OF_MEMORY, "no pinned memory for the uniforms");
     *dev = (const double*)at;

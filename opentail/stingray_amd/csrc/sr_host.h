@@ -116,16 +116,21 @@ struct HostRing {
     bool pending[2] = {false, false};
     bool dirty = false;             // pieces handed out since the last wait for a whole stream
     hipStream_t last = nullptr;     // the stream of those pieces' kernels
+    uint32_t epoch = 0;             // the owner's count of stream changes when the ring was last used
     // room for `need` bytes in the present half (its pieces are handed out by put)
     // (want_half: what a half should hold when the ring has to be made or made again anyway)
-    hipError_t begin(size_t need, hipStream_t st, size_t want_half = 0)
+    // (owner_epoch: the context counts its changes of stream, and waits for the stream it leaves at every one of them)
+    hipError_t begin(size_t need, hipStream_t st, size_t want_half = 0, uint32_t owner_epoch = 0)
     {
         hipError_t e = hipSuccess;
         if (dirty && st != last) {  // the caller changed streams: nothing orders the old stream's readers before new events
-            if ((e = hipStreamSynchronize(last)) != hipSuccess) return e;
+            // When the context itself made the change it has waited for the old stream already -- which the caller may
+            // have destroyed since: it is not touched again.
+            if (owner_epoch == epoch && (e = hipStreamSynchronize(last)) != hipSuccess) return e;
             pending[0] = pending[1] = dirty = false;
             used = 0;
         }
+        epoch = owner_epoch;
         last = st;
         if (need > half) {  // grow: nothing may still be reading the old memory
             if (dirty && (e = hipStreamSynchronize(st)) != hipSuccess) return e;
@@ -200,6 +205,8 @@ struct sr_ctx {
     DeviceBuf redo_list;     // rows given to sr_resample_rows_launch
     int ident_rows = 0;
     DeviceBuf spec_probs;    // speculative verification: the target distributions of every position
+    uint32_t stream_epoch = 0;  // changes of stream so far (each waits for the stream that is left)
+    bool argmax_scratch_dirty = false;  // a launch of sr_argmax_rows_launch failed: its slots and counters are cleared before the next
     DeviceBuf spec_resid, spec_reject;  // ... the residual row of every row's first rejected position, that position
     DeviceBuf seg_part, seg_func;       // approximate sums and increment functions of the segments of prepared rows
     DeviceBuf full_seg_func, full_seg_ms, full_watch, full_watch_cnt, full_seg_keys;  // ... of the full-vocabulary path's denominators
@@ -263,6 +270,7 @@ struct sr_batch {
     // What sr_batch_append_tokens needs of the last upload: the inputs of a batch without allow-masks (kept flat as
     // they came; the histories are split per row by the first append) and the room each row's edit range has.
     bool can_append = false, hist_split = false;
+    bool host_ahead = false;  // an append call failed after it had changed the host's copies: the next one rebuilds the batch
     int32_t append_rebuilds = 0;  // calls of sr_batch_append_tokens that rebuilt the batch (test hook)
     int32_t append_moves = 0;     // ... rows that were moved to the end of the edit array instead
     std::vector<sr_row_params> keep_params;

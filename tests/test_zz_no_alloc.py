@@ -84,6 +84,26 @@ def test_rows_that_do_not_start_on_16_bytes_bf16_and_single_chunk_rows(ctx):
     assert np.array_equal(i1, many.cpu().numpy().argmax(1))
 
 
+def test_calls_on_a_fresh_context_take_no_device_memory(ctx):
+    """Free device memory as the driver reports it (the whole device's, not torch's pool) is the same before and after
+    calls of several shapes on a context that has served nothing else."""
+    import torch
+
+    rng = np.random.default_rng(11)
+    devs = [torch.from_numpy(_logits(rng, r, v)).cuda() for r, v in ((64, 151_936), (7, 40_000), (2000, 700))]
+    outs = [(torch.empty(d.shape[0], dtype=torch.int32, device="cuda"), torch.empty(d.shape[0], dtype=torch.float32, device="cuda"))
+            for d in devs]
+    outs[0][0].cpu()  # (whatever torch sets up for its first download is there before the measurement)
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        for d, o in zip(devs, outs):
+            ctx.argmax_rows(d, out=o, noalloc=True)
+    ctx.synchronize()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+
+
 def test_more_rows_than_the_static_scratch_holds_is_an_error_not_a_fault(ctx):
     import torch
 
