@@ -1569,9 +1569,14 @@ struct NoFill {
 };
 template <typename Fill = NoFill>
 __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, float* p, int n, int m, int row, FullSmem& sm,
-                                                         Fill fill = Fill())
+                                                         Fill fill = Fill(), int cap = kSmall)
 {
+    // (cap: what a list that is in shared memory already may hold -- kSmall, or 2 kSmall where the launch gave the
+    // workgroup the room: the list then runs on from sm.sortbuf through the two arrays behind it)
     constexpr bool kResident = std::is_same<Fill, NoFill>::value;
+    constexpr int kPerT = 2 * kSmall / kT;
+    unsigned long long* const buf = &sm.sortbuf[0];
+    const int cpt = (kResident ? cap : kSmall) / kT;  // entries per thread of the list's new layout
     const int nv8 = (n / 8) * 8;
     const int lane = sr_lane(), wave = sr_wave_id();
     // One wave per chain: it passes over the whole list in index order, sixteen entries per lane at a time, with the
@@ -1580,20 +1585,21 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
     // thousand entries the list is laid out anew, entry 16 l + j at place 64 j + l.
     auto place_of = [](int i) -> int { return (i & ~1023) | ((i & 15) << 6) | ((i >> 4) & 63); };
     auto lay_out = [&]() __attribute__((always_inline)) {
-        static_assert(kSmall == 4 * kT, "four entries per thread");
-        unsigned long long t[4];
+        static_assert(kSmall == 4 * kT, "four entries per thread, or eight");
+        unsigned long long t[kPerT];
 #pragma unroll
-        for (int r = 0; r < 4; r++) t[r] = sm.sortbuf[4 * (int)threadIdx.x + r];
+        for (int r = 0; r < kPerT; r++) t[r] = r < cpt ? buf[cpt * (int)threadIdx.x + r] : 0ull;
         __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 4; r++) sm.sortbuf[place_of(4 * (int)threadIdx.x + r)] = t[r];
+        for (int r = 0; r < kPerT; r++)
+            if (r < cpt) buf[place_of(cpt * (int)threadIdx.x + r)] = t[r];
         __syncthreads();
     };
     auto load_terms = [&](int i0, int cnt, int chain, float mul, bool scale, float (&x)[16]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             const int i = i0 + j;
-            const unsigned long long v = i < cnt ? sm.sortbuf[place_of(i)] : 0ull;
+            const unsigned long long v = i < cnt ? buf[place_of(i)] : 0ull;
             const int e = (int)(0xffffffffu - (uint32_t)(v >> 32));
             const bool mine = chain < 0 || (e < nv8 ? (e & 7) : e - (n - 8)) == chain;
             const float t = sr_u2f((uint32_t)v);
@@ -1646,8 +1652,9 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
     }
     float sc = 0.0f;
     if (kResident) lay_out();
-    for (int first = 0; first < m; first += kSmall) {
-        const int cnt = min(kSmall, m - first);
+    const int step = kResident ? cap : kSmall;  // (a resident list is one block)
+    for (int first = 0; first < m; first += step) {
+        const int cnt = min(step, m - first);
         if (!kResident) {
             __syncthreads();
             fill(first, cnt);
@@ -1681,8 +1688,8 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
         done = true;
     }
     float acc = 0.0f;
-    for (int first = 0; first < m; first += kSmall) {
-        const int cnt = min(kSmall, m - first);
+    for (int first = 0; first < m; first += step) {
+        const int cnt = min(step, m - first);
         if (!kResident) {
             if (wave == 0 && lane == 0) sm.bc[10] = done ? 1u : 0u;
             __syncthreads();
@@ -1698,7 +1705,7 @@ __device__ __forceinline__ void finish_from_ordered_list(const SrFullArgs& a, fl
                 int f;
                 acc = sr_seq_wave<16, true>(x, acc, r, &f);
                 if (f >= 0) {
-                    const unsigned long long v = sm.sortbuf[place_of(b0 + f)];
+                    const unsigned long long v = buf[place_of(b0 + f)];
                     token = (int)(0xffffffffu - (uint32_t)(v >> 32));
                     done = true;
                     const float t = sr_u2f((uint32_t)v);
@@ -1747,6 +1754,7 @@ struct StretchToPool {  // appended to a pool in LDS that all waves share: value
     uint32_t* counter;
     uint32_t* vals;
     uint32_t* tags;
+    int cap;  // entries the pool holds
     __device__ __forceinline__ int reserve(int, int count) const
     {
         int b = 0;
@@ -1755,7 +1763,7 @@ struct StretchToPool {  // appended to a pool in LDS that all waves share: value
     }
     __device__ __forceinline__ void put(int place, int rank, uint32_t ybits, int i) const
     {
-        if (place < kSmall) { vals[place] = ybits; tags[place] = ((uint32_t)rank << kTagIndexBits) | (uint32_t)i; }
+        if (place < cap) { vals[place] = ybits; tags[place] = ((uint32_t)rank << kTagIndexBits) | (uint32_t)i; }
     }
 };
 struct StretchCount {  // nothing is kept: the wave's count is what list_stretch returns
@@ -1849,14 +1857,27 @@ __device__ __forceinline__ int list_stretch(const float* p, int w0, int w1, bool
 enum NucleusWay : int { kNucleusDone = 0, kNucleusGeneral = 1, kNucleusGeneralNoSlabs = 2 };
 constexpr int kNucleusMaxSlabs = 40;
 constexpr int kNucleusRowFinish = 4;  // a nucleus that took more slabs than this is finished by passes over the row
+// `extra`: 16 kSmall bytes of shared memory beyond sm, or null.  With them a slab holds 2 kSmall entries -- most nuclei of
+// a few thousand entries then close in one slab, which is listed by one read of the row and finished from the list,
+// where two slabs cost three reads --: the pool of values and tags lies there, and the lists that are sm.sortbuf
+// otherwise run on through the two arrays behind it.
 __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float top_p, const float* p, int n, int slot,
-                                                      int row, bool do_scale, float inv, FullSmem& sm)
+                                                      int row, bool do_scale, float inv, FullSmem& sm, uint32_t* extra)
 {
     constexpr int kPer = kHistPos / kT;
     static_assert(kHistPos * 4 <= kSmall * 8 && kHistPos % kT == 0, "the histogram fits the sort buffer");
+    static_assert(offsetof(FullSmem, sprob) == offsetof(FullSmem, sortbuf) + sizeof(FullSmem::sortbuf) &&
+                  offsetof(FullSmem, tags) == offsetof(FullSmem, sprob) + sizeof(FullSmem::sprob) &&
+                  sizeof(FullSmem::sortbuf) + sizeof(FullSmem::sprob) + sizeof(FullSmem::tags) >= 2 * kSmall * sizeof(unsigned long long),
+                  "a list of 2 kSmall entries fits the three arrays, which lie one behind the other");
+    constexpr int kPerT = 2 * kSmall / kT;  // most entries of a slab per thread
     const int tid = threadIdx.x, lane = sr_lane(), wave = sr_wave_id();
+    const int S = extra ? 2 * kSmall : kSmall;  // entries a slab may hold
+    const int cpt = S / kT;
     const uint32_t* hcnt = (const uint32_t*)sm.sortbuf;
-    uint32_t* sval = (uint32_t*)sm.sprob;
+    uint32_t* sval = extra ? extra : (uint32_t*)sm.sprob;
+    uint32_t* const tags = extra ? extra + 2 * kSmall : sm.tags;
+    unsigned long long* const list = &sm.sortbuf[0];  // [S]
     [[maybe_unused]] unsigned long long t_step = 0ull;
     FPROF_ADD(a, slot, 16, t_step);
     if (sm.bc[5] != 0u) return kNucleusGeneral;
@@ -1879,7 +1900,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     const uint32_t q0 = (uint32_t)blk_excl_scan((int)ownq, &totq, sm);
     int crowd = 0;  // entries at positions that hold more than a slab (runs of one value, if the row can be walked at all)
 #pragma unroll
-    for (int j = 0; j < kPer; j++) crowd += mine[j] > (uint32_t)kSmall ? (int)mine[j] : 0;
+    for (int j = 0; j < kPer; j++) crowd += mine[j] > (uint32_t)S ? (int)mine[j] : 0;
     const int crowded_total = blk_sum_i(crowd, sm);
     if (tid == 0) { sm.bc[7] = (uint32_t)kHistPos; sm.bc[11] = (uint32_t)tot; }
     __syncthreads();
@@ -1917,9 +1938,10 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     bool cut_in_run = false;   // the cut fell inside such a run: ycut / idx_last are set by the walk
     uint32_t ycut = 0u;
     int idx_last = -1;         // the last member among the entries equal to the cut value
-    uint32_t pv[4] = {0u, 0u, 0u, 0u};  // the last slab's entries that this thread read from the pool: values,
-    int pi[4] = {0, 0, 0, 0};            // indices
-    int lpos[4] = {0, 0, 0, 0};          // and places in index order
+    uint32_t pv[kPerT];  // the last slab's entries that this thread read from the pool: their values (index and place in
+                         // index order stay in the pool's tags)
+#pragma unroll
+    for (int r = 0; r < kPerT; r++) pv[r] = 0u;
     for (;; slab++) {
         if (slab >= kMaxSlabs) return kNucleusGeneralNoSlabs;  // (the general way would walk the same slabs)
         if (tid == 0) sm.bc[6] = (uint32_t)kHistPos;
@@ -1929,14 +1951,14 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
 #pragma unroll
             for (int j = 0; j < kPer; j++) {
                 c += (int)mine[j];
-                if (tid * kPer + j >= d_prev && c - taken > kSmall && d_first == kHistPos) d_first = tid * kPer + j;
+                if (tid * kPer + j >= d_prev && c - taken > S && d_first == kHistPos) d_first = tid * kPer + j;
             }
             if (d_first < kHistPos) atomicMin(&sm.bc[6], (uint32_t)d_first);
         }
         __syncthreads();
         // about how many entries the nucleus holds: a row that would need more slabs than are walked goes the general
         // way at once (its survivors are sorted where they lie)
-        if (slab == 0 && runs == 0 && (int)sm.bc[11] - min((int)sm.bc[11], crowded_total) > (kMaxSlabs - 2) * kSmall)
+        if (slab == 0 && runs == 0 && (int)sm.bc[11] - min((int)sm.bc[11], crowded_total) > (kMaxSlabs - 2) * S)
             return kNucleusGeneralNoSlabs;
         const int d_cnt = (int)sm.bc[6], d_mass = (int)sm.bc[7];
         const int d_end = d_mass + 1 > d_prev ? min(d_cnt, d_mass + 1) : d_cnt;
@@ -2051,27 +2073,29 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         // within the wave, from which its place in index order follows once all waves' counts are known
         if (tid == 0) sm.bc[4] = 0u;
         __syncthreads();
-        const int cw = list_stretch(p, w0, w1, do_scale, inv, StretchToPool{&sm.bc[4], sval, sm.tags},
+        const int cw = list_stretch(p, w0, w1, do_scale, inv, StretchToPool{&sm.bc[4], sval, tags, S},
                                     [&](float y, int) -> bool { return y > c_y && !(capped && y > hi_y); });
         if (lane == 0) sm.redi[wave] = cw;
         __syncthreads();
         taken = (int)sm.bc[8];
         nc = (int)sm.bc[4];
-        if (nc > kSmall) return kNucleusGeneral;
+        if (nc > S) return kNucleusGeneral;
         FPROF_ADD(a, slot, 12, t_step);
         if (nc > 0) {
-            // this thread's four entries of the pool, and their places in index order
+            // this thread's entries of the pool; their places in index order take the place of their numbers within
+            // the wave in the tags
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
+            for (int r = 0; r < kPerT; r++) {
                 const int e = r * kT + tid;
                 pv[r] = e < nc ? sval[e] : 0u;
-                const uint32_t tag = e < nc ? sm.tags[e] : 0u;
-                const int i = (int)(tag & ((1u << kTagIndexBits) - 1u)), w = i / chunk;
-                int off = (int)(tag >> kTagIndexBits);
+                if (e < nc) {
+                    const uint32_t tag = tags[e];
+                    const int i = (int)(tag & ((1u << kTagIndexBits) - 1u)), w = i / chunk;
+                    int off = (int)(tag >> kTagIndexBits);
 #pragma unroll
-                for (int k = 0; k < kW - 1; k++) off += k < w ? sm.redi[k] : 0;
-                pi[r] = i;
-                lpos[r] = off;
+                    for (int k = 0; k < kW - 1; k++) off += k < w ? sm.redi[k] : 0;
+                    tags[e] = ((uint32_t)off << kTagIndexBits) | (uint32_t)i;
+                }
             }
             // The values are sorted.  A long list is first cut into 4,096 groups of equal width in the values' bit
             // patterns between the slab's bounds -- counted, the counts summed, the values put group by group -- and
@@ -2085,13 +2109,13 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
             if (nc > 1024 && bhi >= blo) {
                 uint32_t* cur = (uint32_t*)sm.sortbuf;
                 uint32_t* grp = cur + kSmall;
-                __syncthreads();  // (sval and the tags have been read)
+                __syncthreads();  // (sval has been read)
 #pragma unroll
                 for (int r = 0; r < 4; r++) cur[r * kT + tid] = 0u;
                 if (tid == 0) sm.bc[12] = 0u;
                 __syncthreads();
 #pragma unroll
-                for (int r = 0; r < 4; r++)
+                for (int r = 0; r < kPerT; r++)
                     if (r * kT + tid < nc) atomicAdd(&cur[group_of(pv[r])], 1u);
                 __syncthreads();
                 uint32_t c4[4];
@@ -2112,11 +2136,11 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
                     for (int r = 0; r < 4; r++) { cur[4 * tid + r] = (uint32_t)at; at += (int)c4[r]; }
                     __syncthreads();
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
+                    for (int r = 0; r < kPerT; r++)
                         if (r * kT + tid < nc) grp[atomicAdd(&cur[group_of(pv[r])], 1u)] = pv[r];
                     __syncthreads();  // cur[g] is now where group g ends
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
+                    for (int r = 0; r < kPerT; r++) {
                         const int i = r * kT + tid;
                         if (i < nc) {
                             const uint32_t v = grp[i];
@@ -2134,6 +2158,7 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
                 }
             }
             if (!counted) {
+                if (nc > kSmall) return kNucleusGeneral;  // (the network sorts kSmall entries at most)
                 int P = 2;
                 while (P < nc) P <<= 1;
                 __syncthreads();
@@ -2142,9 +2167,9 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
                 sort_lds_desc(sval, P);
             }
             FPROF_ADD(a, slot, 13, t_step);
-            run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, top_p, &found, sm);
+            run = seq_sum<true>([&](int i) -> float { return sr_u2f(sval[i]); }, nc, run, top_p, &found, sm);
             if (found >= 0)
-                SR_AMB_IF(sr_stop_near(run, sm.sprob[found], top_p) || (found + 1 < nc && sm.sprob[found + 1] == sm.sprob[found]));
+                SR_AMB_IF(sr_stop_near(run, sr_u2f(sval[found]), top_p) || (found + 1 < nc && sval[found + 1] == sval[found]));
             FPROF_ADD(a, slot, 14, t_step);
         }
         if (a.prof && slot == 0 && tid == 0) a.prof[15] += 1ull;
@@ -2157,8 +2182,11 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
     // the last slab's entries in index order (the sort's scratch memory is free again)
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < 4; r++)
-        if (r * kT + tid < nc) sm.sortbuf[lpos[r]] = ((unsigned long long)(0xffffffffu - (uint32_t)pi[r]) << 32) | (unsigned long long)pv[r];
+    for (int r = 0; r < kPerT; r++)
+        if (r * kT + tid < nc) {
+            const uint32_t tag = tags[r * kT + tid];
+            list[tag >> kTagIndexBits] = ((unsigned long long)(0xffffffffu - (tag & ((1u << kTagIndexBits) - 1u))) << 32) | (unsigned long long)pv[r];
+        }
     __syncthreads();
     // Members: everything above the value at the cut, and of the entries equal to it the first ones by index.
     if (found >= 0 && !cut_in_run) {
@@ -2166,32 +2194,32 @@ __device__ __forceinline__ int nucleus_from_histogram(const SrFullArgs& a, float
         int gt = 0;
         for (int e = tid; e < nc; e += kT) gt += sval[e] > ycut ? 1 : 0;
         const int keep_eq = found + 1 - blk_sum_i(gt, sm);
-        unsigned long long ent[4];
+        unsigned long long ent[kPerT];
         int eqc = 0;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int e = 4 * tid + r;
-            ent[r] = e < nc ? sm.sortbuf[e] : 0ull;
-            eqc += (e < nc && (uint32_t)ent[r] == ycut) ? 1 : 0;
+        for (int r = 0; r < kPerT; r++) {
+            const int e = cpt * tid + r;
+            ent[r] = (r < cpt && e < nc) ? list[e] : 0ull;
+            eqc += (r < cpt && e < nc && (uint32_t)ent[r] == ycut) ? 1 : 0;
         }
         int tot_eq;
         int rank = blk_excl_scan(eqc, &tot_eq, sm);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int e = 4 * tid + r;
-            if (e < nc) {
+        for (int r = 0; r < kPerT; r++) {
+            const int e = cpt * tid + r;
+            if (r < cpt && e < nc) {
                 const uint32_t yb = (uint32_t)ent[r];
                 const bool keep = yb > ycut || (yb == ycut && rank < keep_eq);
                 if (yb == ycut && rank == keep_eq - 1) sm.bc[9] = 0xffffffffu - (uint32_t)(ent[r] >> 32);
                 if (yb == ycut) rank++;
-                if (!keep) sm.sortbuf[e] = ent[r] & 0xffffffff00000000ull;
+                if (!keep) list[e] = ent[r] & 0xffffffff00000000ull;
             }
         }
         __syncthreads();
         idx_last = (int)sm.bc[9];
     }
     if (slab == 0 && runs == 0) {
-        finish_from_ordered_list(a, const_cast<float*>(p), n, nc, row, sm);
+        finish_from_ordered_list(a, const_cast<float*>(p), n, nc, row, sm, NoFill(), S);
         return kNucleusDone;
     }
     // Several slabs: the members -- known by value and, at the cut value, by index -- are listed by one more read of
@@ -2470,7 +2498,10 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                 }
                 return;
             }
-            const int way = fast_nucleus ? nucleus_from_histogram(a, rd.top_p, p, n, slot, row, do_scale, inv, sm) : kNucleusGeneral;
+            extern __shared__ uint32_t more_lds[];  // 16 kSmall bytes when a.big_slabs, else nothing
+            const int way = fast_nucleus ? nucleus_from_histogram(a, rd.top_p, p, n, slot, row, do_scale, inv, sm,
+                                                                  a.big_slabs ? more_lds : nullptr)
+                                         : kNucleusGeneral;
             no_slabs = way == kNucleusGeneralNoSlabs;
             if (way == kNucleusDone) {
                 FPROF(a, slot, 9);
@@ -3496,7 +3527,21 @@ hipError_t sr_launch_wide_tail(const SrFullArgs& a, int n_rows, hipStream_t st)
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, hipStream_t st)
 {
     if (n_rows <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_full_row, dim3(n_rows), dim3(kT), 0, st, a);
+    // (rows that only top-p cuts walk their nucleus in slabs of twice the size when the launch gives the room: see
+    // nucleus_from_histogram)
+    const unsigned more = a.big_slabs ? 16u * (unsigned)kSmall : 0u;
+    if (more) {
+        static bool allowed[64] = {};  // (once per device)
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        if (dev < 0 || dev >= 64 || !allowed[dev]) {
+            e = hipFuncSetAttribute((const void*)k_full_row, hipFuncAttributeMaxDynamicSharedMemorySize, (int)more);
+            if (e != hipSuccess) return e;
+            if (dev >= 0 && dev < 64) allowed[dev] = true;
+        }
+    }
+    hipLaunchKernelGGL(k_full_row, dim3(n_rows), dim3(kT), more, st, a);
     return hipGetLastError();
 }
 hipError_t sr_launch_draw_rows(const float* probs, int64_t stride, int n, int rows, const double* u, int* out,

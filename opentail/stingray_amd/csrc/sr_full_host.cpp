@@ -103,6 +103,9 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     a.uniforms_per_row = b->upr;
     a.out_tokens = out_tokens_dev;
     a.out_flags = out_flags_dev;
+    // With a compute unit per row the row kernel's workgroups can have more shared memory each: rows that only top-p
+    // cuts then walk their nucleus in slabs of twice the size.  (With more rows, two workgroups share a compute unit.)
+    a.big_slabs = (mode == 0 && any_top_p && n_rows <= ctx->cu_count) ? 1 : 0;
 
     SR_HIP(ctx, sr_launch_full_prep(a, n_rows, st));
     SR_HIP(ctx, sr_launch_full_row(a, n_rows, st));  // (every row is finished by this one launch)

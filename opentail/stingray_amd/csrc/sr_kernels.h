@@ -176,6 +176,7 @@ struct SrFullArgs {
     uint32_t* watch_cnt;           // [slot]
     uint16_t* seg_keys;            // [slot][seg_key_stride]: the upper 16 bits of every e of a row that only top-p cuts (0: e = 0)
     int64_t seg_key_stride;
+    int32_t big_slabs;             // k_full_row gets 64 KB of shared memory more: slabs of 8,192 entries for rows that only top-p cuts
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
 hipError_t sr_launch_full_row(const SrFullArgs& a, int n_rows, hipStream_t st);

@@ -496,6 +496,28 @@ def test_rows_that_only_top_p_cuts_at_every_size_of_nucleus(ctx):
             _check_rows(ctx, sub, params, u)
 
 
+def test_top_p_rows_in_a_batch_of_more_rows_than_compute_units(ctx):
+    """With a compute unit per row the row kernel walks a nucleus in slabs of 8,192 entries, with more rows (two
+    workgroups share a compute unit's shared memory) in slabs of 4,096: the same rows both ways."""
+    rng = np.random.default_rng(4243)
+    V = 65_536
+    kinds = np.stack([rng.normal(0, 3.0, V), rng.normal(0, 1.6, V), rng.normal(0, 1.2, V), rng.normal(0, 1.0, V),
+                      np.round(rng.normal(0, 1.2, V) * 4) / 4, rng.normal(0, 0.4, V)]).astype(np.float32)
+    p6 = [SamplingParams(Temperature=1.0, TopP=0.95), SamplingParams(Temperature=1.0, TopP=0.9),
+          SamplingParams(Temperature=1.0, TopP=0.9), SamplingParams(Temperature=1.0, TopP=0.93),
+          SamplingParams(Temperature=0.9, TopP=0.8), SamplingParams(Temperature=1.0, TopP=0.95)]
+    u6 = rng.random(6)
+    few = _check_rows(ctx, kinds, p6, u6)
+    reps = 44                                             # 264 rows: more than the device has compute units
+    logits = np.tile(kinds, (reps, 1))
+    params = p6 * reps
+    u = np.tile(u6, reps)
+    got = ctx.sample_batch(_cuda(logits), params, u)
+    want = oracle_tokens(kinds, p6, u6)
+    assert np.array_equal(got, np.tile(want, reps))
+    assert few is not None
+
+
 def test_final_normalize_of_long_rows_at_ragged_lengths(ctx):
     # The eight-lane sum of a long row is taken by one wave per lane over blocks of 8,192 entries; lengths that leave
     # one to seven entries for the overlapped last vector, a last block that is nearly empty or nearly full, rows
