@@ -203,7 +203,7 @@ def bench_spec(args, w, ctx, stream) -> dict:
                      "traffic_source": "profiles/traffic_c5.json.txt: rocprofv3 --pmc runs of this command, whole step, committed; not measured by this run",
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "bytes_with_bonus_position_for_every_row": bytes_with_bonus, "bytes_reading_every_input": bytes_everything,
-                     "kernel": "k_full_exp_seg", "kernel_us": dev_us},
+                     "kernel": "k_full_softmax_seg", "kernel_us": dev_us},
         "cpu_baseline": cpu, "parity": parity,
     }
     for _, _, _, b, _, _ in sets:
@@ -440,7 +440,7 @@ def run_workload(args, ctx, stream) -> dict:
                      "traffic_source": None if traffic is None else
                      f"profiles/{os.path.basename(tpath)}: rocprofv3 --pmc runs of this command, committed; not measured by this run",
                      "algorithmic_bytes_per_launch": alg_bytes,
-                     "kernel": "k_topk_rows" if args.workload.startswith(("c1", "c3")) else ("k_full_exp_seg" if args.workload == "c2" else "k_full_row"),
+                     "kernel": "k_topk_rows" if args.workload.startswith(("c1", "c3")) else ("k_full_softmax_seg" if args.workload == "c2" else "k_full_row"),
                      "kernel_us": kern_us},
         "cpu_baseline": cpu,
         "parity": parity,

@@ -42,6 +42,12 @@ SR_API int sr_debug_append_moves(const sr_batch* batch);
  * selected (default 2^22, more than a second).  0 makes every row take that way: the results must not change. */
 SR_API int sr_debug_set_spin_limit(sr_ctx* ctx, uint32_t polls);
 
+/* How often a workgroup of the full-vocabulary path's pass over long rows polls its row's count (every workgroup of the
+ * row leaves its segments' maxima and counts itself in) before it stops waiting, marks its segments and leaves them to
+ * the last of the row's workgroups (default 2^15, tens of milliseconds).  0 makes every workgroup leave its segments;
+ * 1 or 2 make some of them do so: the results must not change. */
+SR_API int sr_debug_set_row_wait_limit(sr_ctx* ctx, uint32_t polls);
+
 /* Profiling builds (-DSR_PROFILE) only, SR_ERR_UNSUPPORTED otherwise: phase timestamps (wall_clock64, 100 MHz) of
  * the selection kernel go to prof_dev[unit][16], one unit per chunk item and per row; NULL switches them off. */
 SR_API int sr_debug_set_profile(sr_ctx* ctx, unsigned long long* prof_dev);

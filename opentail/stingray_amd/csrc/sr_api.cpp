@@ -317,7 +317,7 @@ void sr_destroy(sr_ctx* ctx)
                          &ctx->work, &ctx->edit_tab, &ctx->host_logits, &ctx->stage_probs, &ctx->out_tokens, &ctx->out_flags, &ctx->out_val,
                          &ctx->full_state, &ctx->sort_k0, &ctx->sort_v0,
                          &ctx->sort_v1, &ctx->ident, &ctx->redo_list, &ctx->spec_probs, &ctx->spec_resid, &ctx->spec_reject,
-                         &ctx->seg_part, &ctx->seg_func, &ctx->full_seg_func, &ctx->full_seg_ms, &ctx->full_watch, &ctx->full_watch_cnt, &ctx->full_seg_keys};
+                         &ctx->seg_part, &ctx->seg_func, &ctx->full_row_sync, &ctx->full_seg_func, &ctx->full_seg_ms, &ctx->full_watch, &ctx->full_watch_cnt, &ctx->full_seg_keys};
     for (DeviceBuf* b : bufs) b->release();
     ctx->uni_ring.release();
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
@@ -1406,6 +1406,13 @@ int sr_debug_set_spin_limit(sr_ctx* ctx, uint32_t polls)
 {
     if (!ctx) return SR_ERR_NULL_ARGUMENT;
     ctx->spin_limit = polls;
+    return SR_OK;
+}
+
+int sr_debug_set_row_wait_limit(sr_ctx* ctx, uint32_t polls)
+{
+    if (!ctx) return SR_ERR_NULL_ARGUMENT;
+    ctx->row_wait_limit = polls;
     return SR_OK;
 }
 

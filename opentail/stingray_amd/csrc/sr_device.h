@@ -58,14 +58,11 @@ __device__ __forceinline__ float sr_expf_tab(float x, const uint64_t* tab)
     const double c0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
     const double c1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
     const double c2 = 0x1.62e42ff0c52d6p-1 / 32.0;
-    uint32_t xb = sr_f2u(x);
-    uint32_t abstop = (xb >> 20) & 0x7ffu;
-    if (abstop >= (0x42b00000u >> 20)) {
-        if (xb == 0xff800000u) return 0.0f;
-        if (abstop >= (0x7f800000u >> 20)) return __fadd_rn(x, x);
-        if (x > 0x1.62e42ep6f) return sr_u2f(0x7f800000u);
-        if (x < -0x1.9fe368p6f) return 0.0f;
-    }
+    const uint32_t xb = sr_f2u(x);
+    const uint32_t abstop = (xb >> 20) & 0x7ffu;
+    // The main path runs for every input and the special ones are put in place of its result afterwards, by selects:
+    // without a branch per element the compiler interleaves the chains of several elements (each is a dozen dependent
+    // double-precision operations with a table lookup in the middle) instead of running them one behind the other.
     double xd = (double)x;
     double z = __dmul_rn(inv_ln2_n, xd);
     double kd = __dadd_rn(z, shift);
@@ -80,7 +77,13 @@ __device__ __forceinline__ float sr_expf_tab(float x, const uint64_t* tab)
     double y = __fma_rn(c2, r, 1.0);
     y = __fma_rn(zz, r2, y);
     y = __dmul_rn(y, s);
-    return __double2float_rn(y);
+    float e = __double2float_rn(y);
+    // underflow to 0, overflow to +inf, NaN and +inf propagate, -inf gives 0 (the later line wins)
+    e = (x < -0x1.9fe368p6f) ? 0.0f : e;
+    e = (x > 0x1.62e42ep6f) ? sr_u2f(0x7f800000u) : e;
+    e = (abstop >= (0x7f800000u >> 20)) ? __fadd_rn(x, x) : e;
+    e = (xb == 0xff800000u) ? 0.0f : e;
+    return e;
 }
 __device__ __forceinline__ float sr_expf(float x) { return sr_expf_tab(x, sr_exp2f_tab); }
 

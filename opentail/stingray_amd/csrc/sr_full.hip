@@ -1044,6 +1044,16 @@ __device__ __forceinline__ bool row_fast_nucleus(const SrRow& rd, const SrFullAr
     return use_top_p && !(rd.top_k > 0 && rd.top_k < a.vocab) && !(rd.min_p > 0.0f) && a.mode == 0 && a.vocab >= 8 &&
            a.vocab <= (1 << kTagIndexBits) && a.sort_stride >= a.vocab;
 }
+// the row's maximum in SrFullState: this launch's number in front of the key, and what the word holds of this launch
+__device__ __forceinline__ unsigned long long full_maxkey(const SrFullArgs& a, uint32_t key)
+{
+    return ((unsigned long long)a.seq << 32) | (unsigned long long)key;
+}
+__device__ __forceinline__ uint32_t full_maxkey_of(const SrFullArgs& a, unsigned long long word)
+{
+    return (uint32_t)(word >> 32) == a.seq ? (uint32_t)word : 0u;
+}
+
 // ---- stage 1: the masked (and temperature-scaled) copy of the row ------------------------------------
 template <int ES>
 __global__ __launch_bounds__(256) void k_full_prep(SrFullArgs a)
@@ -1068,12 +1078,6 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
     const int slot = blockIdx.x;
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
-    if (threadIdx.x == 0) {  // (the first kernel of the pipeline that runs for every row)
-        a.state[slot].maxkey = 0u;
-        a.state[slot].mul1 = a.state[slot].mul2 = 1.0f;
-        if (a.watch_cnt) a.watch_cnt[slot] = 0u;
-    }
-
     if (rd.edit_cnt <= 0) return;
     const SrEdit* ed = a.edits + rd.edit_off;
     if (row_edits_on_the_fly(rd, a)) {
@@ -1105,7 +1109,7 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
             k = kv > k ? kv : k;
         }
         k = sr_wave_max_u32(k);
-        if (sr_lane() == 0 && k != 0u) atomicMax(&a.state[slot].maxkey, k);
+        if (sr_lane() == 0 && k != 0u) atomicMax(&a.state[slot].maxkey, full_maxkey(a, k));
         return;
     }
     const char* rowp = (const char*)a.logits + (size_t)row * (size_t)a.row_stride * ES;
@@ -1171,7 +1175,7 @@ __global__ __launch_bounds__(256) void k_full_max(SrFullArgs a)
     __syncthreads();
     if (threadIdx.x == 0) {
         k = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
-        if (k != 0u) atomicMax(&a.state[slot].maxkey, k);
+        if (k != 0u) atomicMax(&a.state[slot].maxkey, full_maxkey(a, k));
     }
 }
 template <int ES>
@@ -1181,7 +1185,7 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
     const int row = a.row_list[slot];
     const SrRow rd = a.rows[row];
     if (rd.temperature <= 0.0f) return;
-    const uint32_t mk = a.state[slot].maxkey;
+    const uint32_t mk = full_maxkey_of(a, a.state[slot].maxkey);
     if (mk == 0xffffffffu || mk <= 0x007fffffu) return;  // NaN, or nothing above -inf: the row kernel makes it uniform
     const float m = sr_okey_inv(mk);
     __shared__ uint64_t tab[32];  // the expf table: a lookup per element from global memory is a long dependent load
@@ -1218,12 +1222,12 @@ __global__ __launch_bounds__(256) void k_full_exp(SrFullArgs a)
 
 // ---- the same two passes, laid out for a denominator that the whole device prepares -------------------------
 // (launches whose rows are long and start on 16-byte boundaries: a.seg_func is set.)  A wave takes whole segments of
-// SR_SEG_TERMS elements, every lane 16 consecutive ones, so that the expf pass can leave, beside e = expf(x - max), the
+// SR_SEG_TERMS elements, every lane 16 consecutive ones, so that the second pass can leave, beside e = expf(x - max), the
 // record of the segment's exact sum (SeqSegFunc) for the row's workgroup to walk (seg_walk).  The binade that a
-// record is made for comes from approximate sums: the maximum pass leaves every segment's own maximum m and the
-// sum of exp(x - m) over it, and the expf pass, which knows the row's maximum M, adds up S exp(m - M) over the segments
-// in front.  The ids that the row's edits touch take their adjusted values from the work row, where k_full_edits left
-// them, in both passes: e is final when the expf pass has written it.
+// record is made for comes from approximate sums: the first pass leaves every segment's own maximum m and the sum
+// of exp(x - m) over it, and the second, which knows the row's maximum M, adds up S exp(m - M) over the segments in
+// front.  The ids that the row's edits touch take their adjusted values from the work row, where k_full_edits left
+// them: e is final when the second pass has written it.
 template <int ES>
 struct SegSource {
     const char* rowp;      // the row's logits, or null: the adjusted copy in w
@@ -1377,155 +1381,295 @@ __device__ __forceinline__ void seg_load_logits(const SegSource<ES>& src, int se
         }
     }
 }
+
+// Both passes are one launch (k_full_softmax_seg): a wave keeps its segments in registers in between, so the logits
+// are read once.  The workgroups of a row meet between the passes: each leaves its segments' maxima and approximate
+// sums, counts itself in (SR_ROW_SYNC_STRIDE), and waits until the row's count is full.  Workgroups start in the order
+// of their numbers, a row's side by side, so those that a waiting workgroup waits for are running or next to start;
+// the wait is bounded all the same.  A workgroup whose wait runs out marks its segments (SR_SEG_LATE) and leaves;
+// whichever workgroup of the row is the last to get behind the meeting point -- the row's maxima are all in then --
+// finds the marks and finishes those segments, whose inputs nobody has touched.  What a segment gets is the same
+// whichever way it is finished.
+struct SegPass2 {
+    const uint64_t* tab;   // the expf table in shared memory
+    float4* turn;          // the wave's SR_WAVE * 5 vectors of shared memory
+    float* w;
+    uint16_t* keys;
+    bool watch;
+    float e_low, m;
+    int slot, n;
+};
+// e = expf(x - m) of one segment (x as seg_load_logits left it): written to the work row, its 16-bit keys and the
+// entries a min-p cut watches where the row asks for them, and the segment's record
 template <int ES>
-__global__ __launch_bounds__(256) void k_full_max_seg(SrFullArgs a)
-{
-    const int slot = blockIdx.y, lane = sr_lane();
-    const int row = a.row_list[slot];
-    const SrRow rd = a.rows[row];
-    if (rd.temperature <= 0.0f) return;  // greedy rows keep their logits
-    const SegSource<ES> src = seg_source<ES>(rd, a, slot, row);
-    const int n = a.vocab, nseg = seg_count(n);
-    __shared__ uint32_t wmax[4];
-    uint32_t kmax = 0u;
-    for (int seg = (int)blockIdx.x * 4 + sr_wave_id(); seg < nseg; seg += (int)gridDim.x * 4) {
-        float x[SR_SEQ_RUN];
-        seg_load_logits<ES>(src, seg, lane, n, x);
-        uint32_t k = 0u;
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t kv = (x[j] != x[j]) ? 0xffffffffu : sr_okey(x[j]);  // NaN propagates (TensorPrimitives.Max)
-            k = kv > k ? kv : k;
-        }
-        k = sr_wave_max_u32(k);
-        float m = SR_NEG_INF, sum = 0.0f;
-        if (k != 0xffffffffu && k > 0x007fffffu) {
-            m = sr_okey_inv(k);
-#pragma unroll
-            for (int j = 0; j < 16; j++) sum += __expf(x[j] - m);
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-        if (lane == 0) a.seg_ms[(size_t)slot * a.seg_stride + seg] = make_float2(m, sum);
-        kmax = k > kmax ? k : kmax;
-    }
-    // (one atomic per workgroup: a row's hundreds of segments would queue on the one word)
-    if (lane == 0) wmax[sr_wave_id()] = kmax;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        kmax = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
-        if (kmax != 0u) atomicMax(&a.state[slot].maxkey, kmax);
-    }
-}
-template <int ES>
-__global__ __launch_bounds__(256) void k_full_exp_seg(SrFullArgs a)
+__device__ __forceinline__ void seg_pass2(const SrFullArgs& a, const SegPass2& c, int seg, int lane, const float (&x)[SR_SEQ_RUN],
+                                          float before, float own_sum)
 {
     constexpr int E = 16 / ES, K = SR_SEG_TERMS / (SR_WAVE * E);
-    const int slot = blockIdx.y, lane = sr_lane(), wave = sr_wave_id();
-    const int row = a.row_list[slot];
-    const SrRow rd = a.rows[row];
-    if (rd.temperature <= 0.0f) return;
-    const uint32_t mk = a.state[slot].maxkey;
-    if (mk == 0xffffffffu || mk <= 0x007fffffu) return;  // NaN, or nothing above -inf: the row kernel makes it uniform
-    const float m = sr_okey_inv(mk);
-    __shared__ uint64_t tab[32];  // the expf table: a lookup per element from global memory is a long dependent load
-    // a wave's segment on its way from the order of the loads to 16 terms a lane: a lane's 16 terms lie together, 16
-    // bytes apart from the next lane's, so that neither the stores nor the loads of 16 bytes a lane collide on a bank
-    __shared__ float4 turn[4][SR_WAVE * 5];
-    // A row that only top-p cuts needs the histogram of its e by their upper 16 bits.  Counting it here took longer
-    // than it saved (one atomic per element in device memory: +30 us; in shared memory, by few workgroups that take
-    // many segments each: +55 us), so the pass leaves those 16 bits of every e beside the row, and the row's workgroup
-    // counts them -- half the bytes of the row -- while one of its waves walks the sum.
-    uint16_t* keys = (row_fast_nucleus(rd, a) && a.seg_keys) ? a.seg_keys + (size_t)slot * (size_t)a.seg_key_stride : nullptr;
-    const int n = a.vocab, nseg = seg_count(n);
-    if (threadIdx.x < 32) tab[threadIdx.x] = sr_exp2f_tab[threadIdx.x];
-    __syncthreads();
-    const SegSource<ES> src = seg_source<ES>(rd, a, slot, row);
-    float* w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
-    const bool watch = row_watch_min_p(rd, a);
-    const float e_low = __fmul_rn(rd.min_p, 0.999999f);
-    const bool record = true;
-    const float2* ms = a.seg_ms + (size_t)slot * a.seg_stride;
-    for (int seg = (int)blockIdx.x * 4 + wave; seg < nseg; seg += (int)gridDim.x * 4) {
-        float x[SR_SEQ_RUN], e[SR_SEQ_RUN];
-        seg_load_logits<ES>(src, seg, lane, n, x);
-        // (the approximate sums in front of the segment and of the segment itself, under the loads; single precision
-        // does: a prediction that misses costs time only)
-        float before = 0.0f, own_sum = 0.0f;
-        if (record) {
-            for (int g = lane; g <= seg; g += SR_WAVE) {
-                const float2 v = ms[g];
-                const float t = v.y > 0.0f ? v.y * __expf(v.x - m) : 0.0f;
-                if (g < seg) before += t;
-                else own_sum = t;
+    const int n = c.n;
+    float e[SR_SEQ_RUN];
+    // (a whole segment without a test per element: the 16 chains of a lane then run interleaved)
+    if ((seg + 1) * SR_SEG_TERMS <= n) {
+#pragma unroll
+        for (int j = 0; j < SR_SEQ_RUN; j++) e[j] = sr_expf_tab(__fsub_rn(x[j], c.m), c.tab);
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; k++)
+#pragma unroll
+            for (int q = 0; q < E; q++) {
+                const int i = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E + q;
+                e[k * E + q] = i < n ? sr_expf_tab(__fsub_rn(x[k * E + q], c.m), c.tab) : 0.0f;
             }
-            before = sr_wave_sum_f32(before);
-            own_sum = sr_wave_sum_f32(own_sum);
+    }
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
+        if (i0 + E <= n) {
+#pragma unroll
+            for (int q = 0; q < E; q += 4)
+                *(float4*)(c.w + i0 + q) = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+        } else {
+#pragma unroll
+            for (int q = 0; q < E; q++)
+                if (i0 + q < n) c.w[i0 + q] = e[k * E + q];
         }
+        if (c.keys) {
+            uint32_t kk[E];
 #pragma unroll
-        for (int k = 0; k < K; k++) {
-            const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
-#pragma unroll
-            for (int q = 0; q < E; q++) e[k * E + q] = (i0 + q < n) ? sr_expf_tab(__fsub_rn(x[k * E + q], m), tab) : 0.0f;
+            for (int q = 0; q < E; q++) kk[q] = e[k * E + q] > 0.0f ? max(sr_f2u(e[k * E + q]) >> 16, 1u) : 0u;
             if (i0 + E <= n) {
 #pragma unroll
                 for (int q = 0; q < E; q += 4)
-                    *(float4*)(w + i0 + q) = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+                    *(uint2*)(c.keys + i0 + q) = make_uint2(kk[q] | (kk[q + 1] << 16), kk[q + 2] | (kk[q + 3] << 16));
             } else {
 #pragma unroll
                 for (int q = 0; q < E; q++)
-                    if (i0 + q < n) w[i0 + q] = e[k * E + q];
-            }
-            if (keys) {
-                uint32_t kk[E];
-#pragma unroll
-                for (int q = 0; q < E; q++) kk[q] = e[k * E + q] > 0.0f ? max(sr_f2u(e[k * E + q]) >> 16, 1u) : 0u;
-                if (i0 + E <= n) {
-#pragma unroll
-                    for (int q = 0; q < E; q += 4)
-                        *(uint2*)(keys + i0 + q) = make_uint2(kk[q] | (kk[q + 1] << 16), kk[q + 2] | (kk[q + 3] << 16));
-                } else {
-#pragma unroll
-                    for (int q = 0; q < E; q++)
-                        if (i0 + q < n) keys[i0 + q] = (uint16_t)kk[q];
-                }
-            }
-            if (watch) {
-#pragma unroll
-                for (int q = 0; q < E; q++)
-                    if (e[k * E + q] >= e_low && i0 + q < n) {
-                        const uint32_t pos = atomicAdd(&a.watch_cnt[slot], 1u);
-                        if (pos < (uint32_t)kSmall)
-                            a.watch[(size_t)slot * kSmall + pos] = ((unsigned long long)sr_f2u(e[k * E + q]) << 32) |
-                                                                   (unsigned long long)(0xffffffffu - (uint32_t)(i0 + q));
-                    }
+                    if (i0 + q < n) c.keys[i0 + q] = (uint16_t)kk[q];
             }
         }
-        if (record) {
-            // through shared memory into the order of the sum: lane l gets the terms 16 l ... 16 l + 15 of the segment
-            // (only this wave touches its part: the wave's own order of shared-memory operations is all it needs)
-            float4* mine = turn[wave];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        if (c.watch) {
 #pragma unroll
-            for (int k = 0; k < K; k++)
-#pragma unroll
-                for (int q = 0; q < E; q += 4) {
-                    const int i = (k * SR_WAVE + lane) * E + q;  // the element's place in the segment
-                    mine[(i >> 4) * 5 + ((i & 15) >> 2)] = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+            for (int q = 0; q < E; q++)
+                if (e[k * E + q] >= c.e_low && i0 + q < n) {
+                    const uint32_t pos = atomicAdd(&a.watch_cnt[c.slot], 1u);
+                    if (pos < (uint32_t)kSmall)
+                        a.watch[(size_t)c.slot * kSmall + pos] = ((unsigned long long)sr_f2u(e[k * E + q]) << 32) |
+                                                                 (unsigned long long)(0xffffffffu - (uint32_t)(i0 + q));
                 }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            float t[SR_SEQ_RUN];
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float4 v = mine[lane * 5 + k];
-                t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
-            }
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            seg_make_record(t, seg, (double)before, a.seg_func + (size_t)slot * a.seg_stride + seg, own_sum);
         }
+    }
+    // through shared memory into the order of the sum: lane l gets the terms 16 l ... 16 l + 15 of the segment (only
+    // this wave touches its part: the wave's own order of shared-memory operations is all it needs)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+    for (int k = 0; k < K; k++)
+#pragma unroll
+        for (int q = 0; q < E; q += 4) {
+            const int i = (k * SR_WAVE + lane) * E + q;  // the element's place in the segment
+            c.turn[(i >> 4) * 5 + ((i & 15) >> 2)] = make_float4(e[k * E + q], e[k * E + q + 1], e[k * E + q + 2], e[k * E + q + 3]);
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float t[SR_SEQ_RUN];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const float4 v = c.turn[lane * 5 + k];
+        t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    seg_make_record(t, seg, (double)before, a.seg_func + (size_t)c.slot * a.seg_stride + seg, own_sum);
+}
+// a segment's own maximum (as an ordered key; 0xffffffff = it holds a NaN) and the sum of exp(x - that maximum)
+__device__ __forceinline__ unsigned long long seg_pass1(const float (&x)[SR_SEQ_RUN])
+{
+    uint32_t k = 0u;
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const uint32_t kv = (x[j] != x[j]) ? 0xffffffffu : sr_okey(x[j]);  // NaN propagates (TensorPrimitives.Max)
+        k = kv > k ? kv : k;
+    }
+    k = sr_wave_max_u32(k);
+    float sum = 0.0f;
+    if (k != 0xffffffffu && k > 0x007fffffu) {
+        const float m = sr_okey_inv(k);
+#pragma unroll
+        for (int j = 0; j < 16; j++) sum += __expf(x[j] - m);
+    }
+    sum = sr_wave_sum_f32(sum);
+    return ((unsigned long long)sr_f2u(sum) << 32) | (unsigned long long)k;
+}
+// what a segment's (maximum, sum) adds to the row's approximate sum when the row's maximum is m
+__device__ __forceinline__ float seg_share(unsigned long long ms, float m)
+{
+    const uint32_t k = (uint32_t)ms;
+    const float sum = sr_u2f((uint32_t)(ms >> 32));
+    return (sum > 0.0f && k != 0xffffffffu) ? sum * __expf(sr_okey_inv(k) - m) : 0.0f;
+}
+template <int ES, int kW, int kS>
+__global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 4) void k_full_softmax_seg(SrFullArgs a)
+{
+    constexpr int kThreads = kW * SR_WAVE;
+    const int slot = blockIdx.y, lane = sr_lane(), wave = sr_wave_id();
+    const int row = a.row_list[slot];
+    const SrRow rd = a.rows[row];
+    if (rd.temperature <= 0.0f) return;  // greedy rows keep their logits
+    __shared__ uint64_t tab[32];  // the expf table: a lookup per element from global memory is a long dependent load
+    // a wave's segment on its way from the order of the loads to 16 terms a lane: a lane's 16 terms lie together, 16
+    // bytes apart from the next lane's, so that neither the stores nor the loads of 16 bytes a lane collide on a bank
+    __shared__ float4 turn[kW][SR_WAVE * 5];
+    __shared__ float share[SR_SEG_MAX];  // every segment's part of the row's approximate sum
+    __shared__ uint32_t wkey[kW];
+    __shared__ uint32_t bc[2];           // 0: the row's count came in   1: what k_full_edits made the row's maximum
+    const int n = a.vocab, nseg = seg_count(n);
+    SrFullState* st = a.state + slot;
+    unsigned long long* sync = a.row_sync + (size_t)slot * SR_ROW_SYNC_STRIDE;
+    unsigned long long* ms = (unsigned long long*)(a.seg_ms + (size_t)slot * a.seg_stride);
+    const unsigned long long stamp = (unsigned long long)a.seq << 32;
+    SeqSegFunc* recs = a.seg_func + (size_t)slot * a.seg_stride;
+    if (threadIdx.x < 32) tab[threadIdx.x] = sr_exp2f_tab[threadIdx.x];
+    const SegSource<ES> src = seg_source<ES>(rd, a, slot, row);
+    SegPass2 c;
+    c.tab = tab;
+    c.turn = turn[wave];
+    c.w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
+    // (a row that only top-p cuts needs the histogram of its e by their upper 16 bits: counting it here, one atomic per
+    // element, took longer than it saved, so the pass leaves those 16 bits of every e beside the row, and the row's
+    // workgroup counts them -- half the bytes of the row -- while one of its waves walks the sum)
+    c.keys = (row_fast_nucleus(rd, a) && a.seg_keys) ? a.seg_keys + (size_t)slot * (size_t)a.seg_key_stride : nullptr;
+    c.watch = row_watch_min_p(rd, a);
+    c.e_low = __fmul_rn(rd.min_p, 0.999999f);
+    c.slot = slot;
+    c.n = n;
+    c.m = 0.0f;
+
+    // the first pass: the segment's maximum and approximate sum, written through for the row's other workgroups
+    // (a wave takes kS segments, the workgroup's waves side by side: every one of its loads is out before the first is used)
+    const int seg0 = (int)blockIdx.x * (kW * kS) + wave;
+    float xs[kS][SR_SEQ_RUN];
+#pragma unroll
+    for (int s = 0; s < kS; s++)
+        if (seg0 + s * kW < nseg) seg_load_logits<ES>(src, seg0 + s * kW, lane, n, xs[s]);
+#pragma unroll
+    for (int s = 0; s < kS; s++)
+        if (seg0 + s * kW < nseg) {
+            const unsigned long long v = seg_pass1(xs[s]);
+            if (lane == 0) sr_store_agent(&ms[seg0 + s * kW], v);
+        }
+    sr_drain_stores();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __hip_atomic_fetch_max(sync, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(sync, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long edited = sr_load_agent(&st->maxkey);  // (final: k_full_edits ran before)
+        uint32_t ok = 0u;
+        for (uint32_t it = 0; it < a.row_wait_limit; it++) {
+            const unsigned long long v = sr_load_agent(sync);
+            if ((uint32_t)(v >> 32) == a.seq && (uint32_t)(v & 0xffffu) == gridDim.x) { ok = 1u; break; }
+            __builtin_amdgcn_s_sleep(8);
+        }
+        bc[0] = ok;
+        bc[1] = full_maxkey_of(a, edited);
+    }
+    __syncthreads();
+    const bool met = bc[0] != 0u;
+    if (!met) {
+        // the wait ran out: the segments are left, marked, to the last of the row's workgroups
+#pragma unroll
+        for (int s = 0; s < kS; s++)
+            if (seg0 + s * kW < nseg && lane == 0) {
+                sr_store_agent(&recs[seg0 + s * kW].kind, SR_SEG_LATE);
+                sr_store_agent(&recs[seg0 + s * kW].a0, a.seq);
+            }
+        sr_drain_stores();
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            sr_store_agent(&st->late, a.seq);
+            sr_drain_stores();
+        }
+    }
+    // (the count as this workgroup found it is looked at behind the second pass: nothing waits for it here)
+    unsigned long long behind = 0ull;
+    if (threadIdx.x == 0) behind = __hip_atomic_fetch_add(sync, 1ull << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    uint32_t mk = 0u;
+    if (met) {
+        // the row's maximum and the segments' shares of the approximate sum (single precision does: a prediction that
+        // misses costs time only)
+        constexpr int kPer = (SR_SEG_MAX + kThreads - 1) / kThreads;
+        unsigned long long mv[kPer];
+        uint32_t kk = 0u;
+#pragma unroll
+        for (int j = 0; j < kPer; j++) {
+            const int g = (int)threadIdx.x + kThreads * j;
+            mv[j] = g < nseg ? sr_load_agent(&ms[g]) : 0ull;
+            kk = max(kk, (uint32_t)mv[j]);
+        }
+        kk = sr_wave_max_u32(kk);
+        if (lane == 0) wkey[wave] = kk;
+        __syncthreads();
+        mk = bc[1];
+#pragma unroll
+        for (int j = 0; j < kW; j++) mk = max(mk, wkey[j]);
+        if (blockIdx.x == 0 && threadIdx.x == 0 && mk != 0u) atomicMax(&st->maxkey, full_maxkey(a, mk));  // for the row's kernel
+        if (mk != 0xffffffffu && mk > 0x007fffffu) {  // (else a NaN, or nothing above -inf: the row kernel makes it uniform)
+            c.m = sr_okey_inv(mk);
+#pragma unroll
+            for (int j = 0; j < kPer; j++) {
+                const int g = (int)threadIdx.x + kThreads * j;
+                if (g < nseg) share[g] = seg_share(mv[j], c.m);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < kS; s++) {
+                const int seg = seg0 + s * kW;
+                if (seg < nseg) {
+                    float before = 0.0f;
+                    for (int g = lane; g < seg; g += SR_WAVE) before += share[g];
+                    before = sr_wave_sum_f32(before);
+                    seg_pass2<ES>(a, c, seg, lane, xs[s], before, share[seg]);
+                }
+            }
+        }
+    }
+    if (wave != 0) return;
+
+    // The last of the row's workgroups to get behind the meeting point finishes what others left: one wave, segment by
+    // segment.  (Every workgroup's first pass is complete by then, and the marks were written before their workgroup
+    // counted itself.)
+    const uint32_t was = __shfl((uint32_t)(behind >> 16) & 0xffffu, 0);
+    if (was != gridDim.x - 1u) return;
+    if (sr_load_agent(&st->late) != a.seq) return;
+    if (!met) {
+        uint32_t kk = bc[1];
+        for (int g = lane; g < nseg; g += SR_WAVE) kk = max(kk, (uint32_t)sr_load_agent(&ms[g]));
+        mk = sr_wave_max_u32(kk);
+    }
+    // (the row's first workgroup, which leaves the maximum for the row's kernel, may be one of those that left)
+    if (lane == 0 && mk != 0u) atomicMax(&st->maxkey, full_maxkey(a, mk));
+    if (mk == 0xffffffffu || mk <= 0x007fffffu) return;
+    if (!met) {
+        c.m = sr_okey_inv(mk);
+        for (int g = lane; g < nseg; g += SR_WAVE) share[g] = seg_share(sr_load_agent(&ms[g]), c.m);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    for (int g = 0; g < nseg; g++) {
+        uint32_t kind = 0u, whose = 0u;
+        if (lane == 0) {
+            kind = sr_load_agent(&recs[g].kind);
+            whose = sr_load_agent(&recs[g].a0);
+        }
+        kind = __shfl(kind, 0);
+        whose = __shfl(whose, 0);
+        if (kind != SR_SEG_LATE || whose != a.seq) continue;
+        seg_load_logits<ES>(src, g, lane, n, xs[0]);
+        float before = 0.0f;
+        for (int h = lane; h < g; h += SR_WAVE) before += share[h];
+        before = sr_wave_sum_f32(before);
+        seg_pass2<ES>(a, c, g, lane, xs[0], before, share[g]);
     }
 }
 
@@ -2364,7 +2508,17 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
     SrFullState* st = a.state + slot;
     const bool greedy = rd.temperature <= 0.0f;
     const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
-    if (tid == 0) sm.bc[SR_AMB_WORD] = 0u;  // (every path that can set it passes a barrier first)
+    if (tid == 0) {
+        sm.bc[SR_AMB_WORD] = 0u;  // (every path that can set it passes a barrier first)
+        // What the launch after this one expects of the row's scalars: the factors of a row that is not left to its
+        // reader are 1, and the list of entries to watch is empty (the expf pass only appends to it).  No kernel of the
+        // pipeline before this one runs for every row of every launch.
+        st->mul1 = st->mul2 = 1.0f;
+        if (a.watch_cnt) {
+            sm.segbc[3] = a.watch_cnt[slot];
+            a.watch_cnt[slot] = 0u;
+        }
+    }
 
     if (greedy) {
         // Greedy / GreedyWithHistoryPenalties on the adjusted row; distributions become one-hot
@@ -2383,7 +2537,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
     {
         FPROF(a, slot, 0);
         // Softmax (Sampler.cs:448-472): the maximum and e = expf(x - max) were computed by the kernels before
-        const uint32_t mk = st->maxkey;
+        const uint32_t mk = full_maxkey_of(a, st->maxkey);
         const bool any_nan = mk == 0xffffffffu;
         const float m = mk == 0u ? SR_NEG_INF : sr_okey_inv(mk);
         FPROF(a, slot, 1);
@@ -2429,7 +2583,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
             }
             float sum;
             if (walked) {
-                // the whole device has prepared the sum (k_full_exp_seg): one wave walks the segments' records, and the
+                // the whole device has prepared the sum (k_full_softmax_seg): one wave walks the segments' records, and the
                 // entries that can survive the min-p cut were listed by the same pass
                 __syncthreads();
                 if (sr_wave_id() == 0) {
@@ -2456,7 +2610,7 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                     }
                     for (int i = n8 * 8 + tid - SR_WAVE; i < n; i += kT - SR_WAVE) count(keys[i]);
                 } else if (watch_min_p) {
-                    const uint32_t cw = a.watch_cnt[slot];
+                    const uint32_t cw = sm.segbc[3];
                     const unsigned long long* wl = a.watch + (size_t)slot * kSmall;
                     for (int i = tid - SR_WAVE; i < (int)min(cw, (uint32_t)kSmall); i += kT - SR_WAVE) sm.sortbuf[i] = wl[i];
                     if (tid == SR_WAVE) sm.bc[4] = cw;
@@ -3475,20 +3629,24 @@ hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
     // (the adjusted copy only where some row keeps one: the host knows)
     if (a.dtype == 1) {
         if (a.any_copy) hipLaunchKernelGGL(k_full_prep<2>, grid, dim3(256), 0, st, a);
-        hipLaunchKernelGGL(k_full_edits<2>, dim3(n_rows), dim3(256), 0, st, a);
+        if (a.any_edits) hipLaunchKernelGGL(k_full_edits<2>, dim3(n_rows), dim3(256), 0, st, a);
     } else {
         if (a.any_copy) hipLaunchKernelGGL(k_full_prep<4>, grid, dim3(256), 0, st, a);
-        hipLaunchKernelGGL(k_full_edits<4>, dim3(n_rows), dim3(256), 0, st, a);
+        if (a.any_edits) hipLaunchKernelGGL(k_full_edits<4>, dim3(n_rows), dim3(256), 0, st, a);
     }
     if (a.seg_func) {
         const int nseg = (a.vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
-        dim3 sgrid((unsigned)std::max(1, std::min(64, (nseg + 3) / 4)), n_rows);
+        // a wave takes one segment, or two where the launch has more segments than the device holds waves of the
+        // one-segment kind at a time: the waves of a row's workgroups wait for each other between the passes
+        const bool two = (long long)n_rows * nseg > 2048;
+        const int per_group = 4 * (two ? 2 : 1);
+        dim3 fgrid((unsigned)((nseg + per_group - 1) / per_group), n_rows);
         if (a.dtype == 1) {
-            hipLaunchKernelGGL(k_full_max_seg<2>, sgrid, dim3(256), 0, st, a);
-            hipLaunchKernelGGL(k_full_exp_seg<2>, sgrid, dim3(256), 0, st, a);
+            if (two) hipLaunchKernelGGL((k_full_softmax_seg<2, 4, 2>), fgrid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((k_full_softmax_seg<2, 4, 1>), fgrid, dim3(256), 0, st, a);
         } else {
-            hipLaunchKernelGGL(k_full_max_seg<4>, sgrid, dim3(256), 0, st, a);
-            hipLaunchKernelGGL(k_full_exp_seg<4>, sgrid, dim3(256), 0, st, a);
+            if (two) hipLaunchKernelGGL((k_full_softmax_seg<4, 4, 2>), fgrid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((k_full_softmax_seg<4, 4, 1>), fgrid, dim3(256), 0, st, a);
         }
     } else if (a.dtype == 1) {
         hipLaunchKernelGGL(k_full_max<2>, grid, dim3(256), 0, st, a);

@@ -43,22 +43,34 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     a.lazy_scale = lazy_scale ? 1 : 0;
     // Which of the rows that come here keep an adjusted copy, and which have their edits applied where they are read
     // (the rows of the batch that take this path: every row in modes 1 / 2).
-    bool any_table = false, any_copy = false;
+    bool any_table = false, any_copy = false, any_edits = false;
     for (const SrRow& r : (host_rows ? *host_rows : b->h_rows)) {
         if (mode == 0 && r.path != SR_PATH_FULL) continue;
         const bool on_the_fly = sr_row_edits_on_the_fly(r, vocab);
         any_table = any_table || on_the_fly;
+        any_edits = any_edits || r.edit_cnt > 0;
         any_copy = any_copy || !(r.temperature > 0.0f && (r.edit_cnt <= 0 || on_the_fly));
     }
     a.any_copy = any_copy ? 1 : 0;
+    a.any_edits = any_edits ? 1 : 0;
     a.edit_tab = nullptr;
     a.edit_tab_stride = (((int64_t)vocab + 31) / 32 + SR_FULL_EDIT_VALUES + 3) & ~(int64_t)3;
     if (any_table) {
         SR_HIP(ctx, ctx->edit_tab.reserve((size_t)n_rows * (size_t)a.edit_tab_stride * sizeof(uint32_t), st));
         a.edit_tab = ctx->edit_tab.as<uint32_t>();
     }
-    SR_HIP(ctx, ctx->full_state.reserve((size_t)n_rows * sizeof(SrFullState), st));
+    // (cleared when new: the rows' maxima carry the number of the launch that wrote them, and the rows' scalars are
+    // otherwise left by each launch the way the next one expects them)
+    SR_HIP(ctx, ctx->full_state.reserve((size_t)n_rows * sizeof(SrFullState), st, true));
     a.state = ctx->full_state.as<SrFullState>();
+    if (++ctx->full_seq == 0u) {  // the numbers have gone round: nothing of an earlier launch may look like this one's
+        SR_HIP(ctx, hipMemsetAsync(ctx->full_state.p, 0, ctx->full_state.cap, st));
+        if (ctx->full_seg_func.p) SR_HIP(ctx, hipMemsetAsync(ctx->full_seg_func.p, 0, ctx->full_seg_func.cap, st));
+        if (ctx->full_row_sync.p) SR_HIP(ctx, hipMemsetAsync(ctx->full_row_sync.p, 0, ctx->full_row_sync.cap, st));
+        ctx->full_seq = 1u;
+    }
+    a.seq = ctx->full_seq;
+    a.row_wait_limit = ctx->row_wait_limit;
     // sort segments are laid out with the work stride of mode 0; in modes 1/2 use a private stride
     const int64_t seg_stride = (vocab + 3) & ~3;
     if ((int64_t)n_rows * seg_stride >= (int64_t)1 << 31)
@@ -76,17 +88,19 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     // segment stride separately otherwise
     a.sort_stride = seg_stride;
     // Long rows that start on 16-byte boundaries, logits and work rows alike: the softmax denominators are prepared by
-    // the passes over the whole device (k_full_max_seg / k_full_exp_seg) and the rows' workgroups only walk the records
+    // the pass over the whole device (k_full_softmax_seg) and the rows' workgroups only walk the records
     {
         const int es = dtype == SR_DTYPE_BF16 ? 2 : 4;
         const int nseg = (vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
         const bool aligned = (((uintptr_t)logits_dev) & 15u) == 0u && ((row_stride * es) & 15) == 0 &&
                              (((uintptr_t)a.work) & 15u) == 0u && ((a.work_stride * 4) & 15) == 0;
         if (vocab >= SR_SEG_MIN_VOCAB && nseg <= SR_SEG_MAX && aligned) {
-            SR_HIP(ctx, ctx->full_seg_func.reserve((size_t)n_rows * (size_t)nseg * sizeof(SeqSegFunc), st));
+            SR_HIP(ctx, ctx->full_seg_func.reserve((size_t)n_rows * (size_t)nseg * sizeof(SeqSegFunc), st, true));
             SR_HIP(ctx, ctx->full_seg_ms.reserve((size_t)n_rows * (size_t)nseg * sizeof(float2), st));
             SR_HIP(ctx, ctx->full_watch.reserve((size_t)n_rows * SR_FULL_SMALL_CAP * sizeof(unsigned long long), st));
-            SR_HIP(ctx, ctx->full_watch_cnt.reserve((size_t)n_rows * sizeof(uint32_t), st));
+            SR_HIP(ctx, ctx->full_watch_cnt.reserve((size_t)n_rows * sizeof(uint32_t), st, true));
+            SR_HIP(ctx, ctx->full_row_sync.reserve((size_t)n_rows * SR_ROW_SYNC_STRIDE * sizeof(unsigned long long), st, true));
+            a.row_sync = ctx->full_row_sync.as<unsigned long long>();
             a.seg_func = (SeqSegFunc*)ctx->full_seg_func.p;
             a.seg_ms = (float2*)ctx->full_seg_ms.p;
             a.seg_stride = nseg;

@@ -196,6 +196,7 @@ struct sr_ctx {
     DeviceBuf work;          // fp32 rows of the full-vocabulary path
     DeviceBuf edit_tab;      // per row: the table of its edits (bitmap of the vocabulary + slots)
     DeviceBuf full_state;    // per-row scalars of the full-vocabulary path
+    uint32_t full_seq = 0;   // number of the last launch of that path (SrFullState::maxkey)
     DeviceBuf host_logits;   // staging for host-resident logits
     DeviceBuf stage_probs;   // staging for host-resident distributions
     DeviceBuf out_tokens, out_flags, out_val;
@@ -209,6 +210,7 @@ struct sr_ctx {
     bool argmax_scratch_dirty = false;  // a launch of sr_argmax_rows_launch failed: its slots and counters are cleared before the next
     DeviceBuf spec_resid, spec_reject;  // ... the residual row of every row's first rejected position, that position
     DeviceBuf seg_part, seg_func;       // approximate sums and increment functions of the segments of prepared rows
+    DeviceBuf full_row_sync;
     DeviceBuf full_seg_func, full_seg_ms, full_watch, full_watch_cnt, full_seg_keys;  // ... of the full-vocabulary path's denominators
     sr_batch* tmp_batch = nullptr;
     unsigned long long* prof = nullptr;  // test hook: phase timestamps of the selection kernel
@@ -228,6 +230,7 @@ struct sr_ctx {
     size_t done_cap = 0;
     unsigned launch_no = 0;
     uint32_t spin_limit = 1u << 22;
+    uint32_t row_wait_limit = 1u << 15;  // SrFullArgs::row_wait_limit (a poll is a round trip to device memory: tens of ms)
 };
 
 struct sr_batch {

@@ -128,14 +128,21 @@ hipError_t sr_launch_selftest_expf(const float* x, float* y, int64_t n, hipStrea
 
 // ---- full-vocabulary path (sr_full.hip) ---------------------------------------------------------------
 struct SrFullState {
-    int32_t n_survivors;  // entries with probability > 0 when top-p starts
-    int32_t unused0;
+    // launch number << 32 | ordered key of the row's largest adjusted logit (0xffffffff = the row holds a NaN; 0 = none
+    // yet), raised with 64-bit atomic maxima: what an earlier launch left is below anything of the present one, so the
+    // word needs no clearing between launches
+    unsigned long long maxkey;
     uint32_t flags;
-    int32_t unused1;
-    uint32_t maxkey;      // ordered key of the row's largest adjusted logit (0xffffffff = the row holds a NaN)
+    int32_t n_survivors;  // entries with probability > 0 when top-p starts
     float mul1, mul2;     // the row's entries are to be multiplied by these two, in this order (1 unless lazy_scale)
-    int32_t pad2;
+    uint32_t late;        // the number of the last launch in which a workgroup of the row stopped waiting at the meeting point
+    int32_t pad;
 };
+static_assert(sizeof(SrFullState) == 32, "the 8-byte word, aligned, in front");
+// SrFullArgs::row_sync, a word per row (rows 256 bytes apart: every workgroup of a row adds to its word and polls it):
+// launch number << 32 | workgroups of k_full_softmax_seg behind the row's meeting point << 16 | workgroups counted in.
+// The number is put in by an atomic maximum before the first count of a launch, so nothing clears the words.
+#define SR_ROW_SYNC_STRIDE 32
 
 struct SeqSegFunc;
 struct SrFullArgs {
@@ -167,15 +174,20 @@ struct SrFullArgs {
     int32_t* out_tokens;       // [row], may be null in mode 1
     uint32_t* out_flags;       // [row], may be null
     unsigned long long* prof;  // optional phase timestamps of slot 0 [32] (test hook), normally null
-    // The softmax denominators prepared by the whole device (k_full_max_seg / k_full_exp_seg, seg_walk); seg_func is
+    // The softmax denominators prepared by the whole device (k_full_softmax_seg, seg_walk); seg_func is
     // null when the launch is not laid out for it (short or unaligned rows) and the rows are added by their workgroups.
     SeqSegFunc* seg_func;          // [slot][seg_stride]
-    float2* seg_ms;                // [slot][seg_stride]: a segment's maximum m and the sum of exp(x - m) over it, approximately
+    float2* seg_ms;                // [slot][seg_stride], 8 bytes each: a segment's maximum m (as an ordered key) and the
+                                   // sum of exp(x - m) over it, approximately
     int32_t seg_stride;
     unsigned long long* watch;     // [slot][SR_FULL_SMALL_CAP]: the entries that can survive a row's min-p cut (value << 32 | ~index)
     uint32_t* watch_cnt;           // [slot]
     uint16_t* seg_keys;            // [slot][seg_key_stride]: the upper 16 bits of every e of a row that only top-p cuts (0: e = 0)
     int64_t seg_key_stride;
+    uint32_t seq;                  // the launch's number (never 0): see SrFullState::maxkey
+    int32_t any_edits;             // some row of the launch has edits (else k_full_edits is not launched)
+    unsigned long long* row_sync;  // [slot * SR_ROW_SYNC_STRIDE]
+    uint32_t row_wait_limit;       // polls of a row's count before a workgroup of k_full_softmax_seg stops waiting for it
     int32_t big_slabs;             // k_full_row gets 64 KB of shared memory more: slabs of 8,192 entries for rows that only top-p cuts
 };
 hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st);
@@ -200,6 +212,7 @@ hipError_t sr_launch_residual_rows(const float* p, int64_t ps, const float* q, i
 #define SR_SEG_PLAIN 0u
 #define SR_SEG_EXACT 1u
 #define SR_SEG_SPLIT 2u
+#define SR_SEG_LATE 3u   // no record yet: left by a workgroup that stopped waiting, with the launch's number in a0
 struct SeqSegFunc {  // 96 bytes
     uint32_t a0, a1;
     int32_t eb;

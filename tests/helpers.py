@@ -48,6 +48,7 @@ def hooks_lib():
         H.sr_debug_append_rebuilds.argtypes = [vp]
         H.sr_debug_append_moves.argtypes = [vp]
         H.sr_debug_set_spin_limit.argtypes = [vp, C.c_uint32]
+        H.sr_debug_set_row_wait_limit.argtypes = [vp, C.c_uint32]
         _hooks = H
     return _hooks
 

@@ -686,3 +686,79 @@ def test_rows_with_more_edited_ids_than_the_table_holds_keep_an_adjusted_copy(ct
         for r, p in enumerate(params):
             want = orc.build_filtered_distribution(logits[r], to_oracle(p))
             assert np.array_equal(got[r].view(np.uint32), want.view(np.uint32)), (str(dev.dtype), r)
+
+
+def test_what_a_launch_leaves_for_the_next_one_on_the_same_context(ctx):
+    """The rows' scalars on the device (the maximum, the factors that a verifier applies, the list of entries that a
+    min-p cut watches) live with the context and are not cleared between launches; a launch whose rows have no edits
+    runs no kernel before the passes over the logits.  Launches of every kind in a row, each of them with larger and
+    with smaller logits than the one before and with other numbers of rows: every one against the oracle."""
+    rng = np.random.default_rng(3131)
+    V = 24_000
+    hist = rng.integers(0, V, 40).tolist()
+    with_edits = [SamplingParams(Temperature=0.9, TopP=0.9, RepetitionPenalty=1.3, PreviousTokens=hist),
+                  SamplingParams(Temperature=1.0, MinP=0.02, PresencePenalty=0.5, PreviousTokens=hist),
+                  SamplingParams(Temperature=0.0, FrequencyPenalty=0.4, PreviousTokens=hist),
+                  SamplingParams(Temperature=1.1, LogitBias={7: 3.0, 9: -2.0})]
+    plain = [SamplingParams(Temperature=1.0, MinP=0.01), SamplingParams(Temperature=0.8, TopP=0.9), SamplingParams(),
+             SamplingParams(Temperature=1.3, MinP=0.001, TopP=0.95), SamplingParams(Temperature=0.0),
+             SamplingParams(Temperature=1.0, MinP=0.05)]
+    spec_params = [SamplingParams() for _ in range(3)]  # (rows that no filter touches: their factors go to the verifier)
+    t, q, k, us = _spec_case(3, 2, V, spec_params, 77, False)
+    for it, shift in enumerate((0.0, 30.0, -30.0, 5.0, -80.0, 0.0)):
+        big = (rng.normal(0, 2.0, (6, V)) + shift).astype(np.float32)
+        _check_rows(ctx, big[:4], with_edits, rng.random(4))
+        _check_rows(ctx, (big - 2 * shift).astype(np.float32), plain, rng.random(6))
+        if it % 2 == 0:
+            _check_spec(ctx, t + np.float32(shift), q, k, spec_params, us)
+        _check_distribution(ctx, big[:2], plain[:2])
+        _check_rows(ctx, big[1:3], plain[3:5], rng.random(2))
+        _check_rows(ctx, big, plain, rng.random(6))
+
+
+def test_workgroups_that_stop_waiting_for_their_row_leave_their_segments_to_the_last_one(ctx):
+    """The pass over long rows keeps a wave's segments in registers between the row maximum and expf(x - max); the
+    workgroups of a row wait for each other in between.  The wait is bounded: with a limit of 0 polls every workgroup
+    stops waiting, marks its segments and leaves them to the row's last workgroup, with 1 to 3 polls some do.  Tokens,
+    distributions and verification results must not change: rows with edits applied on the fly and rows that keep an
+    adjusted copy, allow-masks, bf16, rows for the histogram of a top-p cut and for the list of a min-p cut, launches
+    with one and with two segments a wave."""
+    import torch
+
+    rng = np.random.default_rng(5150)
+    V = 40_968
+    hist = rng.integers(0, V, 60).tolist()
+    long_hist = rng.permutation(V)[:3000].tolist()
+    base = [SamplingParams(Temperature=0.9, TopP=0.9, RepetitionPenalty=1.2, PreviousTokens=hist),
+            SamplingParams(Temperature=1.0, MinP=0.02, PresencePenalty=0.4, PreviousTokens=hist),
+            SamplingParams(Temperature=0.8, TopP=0.95),
+            SamplingParams(Temperature=1.1, MinP=0.01, TopP=0.9, FrequencyPenalty=0.2, RepeatLastN=0, PreviousTokens=long_hist),
+            SamplingParams(Temperature=0.0, RepetitionPenalty=1.3, PreviousTokens=hist),
+            SamplingParams(), SamplingParams(Temperature=1.4, TopK=30_000)]
+    few = rng.normal(0, 2.0, (len(base), V)).astype(np.float32)
+    few[2] *= 2.0
+    many_rows = 56                                  # x 41 segments: two segments a wave
+    many = rng.normal(0, 2.0, (many_rows, V)).astype(np.float32)
+    many_params = [base[i % len(base)] for i in range(many_rows)]
+    allowed = rng.random((len(base), V)) < 0.6
+    mask, active = pack_allow_mask(allowed), np.ones(len(base), dtype=np.uint8)
+    bf_bits = synthetic.to_bf16_bits(few)
+    bf_exact = synthetic.bf16_bits_to_f32(bf_bits)
+    bf_dev = torch.from_numpy(bf_bits.view(np.int16)).view(torch.bfloat16).cuda()
+    spec_params = [SamplingParams(), SamplingParams(Temperature=0.8, TopP=0.9), SamplingParams()]
+    t, q, k, us = _spec_case(3, 2, 20_000, spec_params, 41, True)
+    H = hooks_lib()
+    try:
+        for polls in (0, 1, 2, 3, 1 << 15):
+            ctx._check(H.sr_debug_set_row_wait_limit(ctx.h, polls))
+            for _ in range(2):
+                _check_rows(ctx, few, base, rng.random(len(base)))
+                u = rng.random(many_rows)
+                assert np.array_equal(ctx.sample_batch(_cuda(many), many_params, u), oracle_tokens(many, many_params, u)), polls
+            _check_rows(ctx, few, base, rng.random(len(base)), mask, active)
+            _check_distribution(ctx, few, base)
+            u = rng.random(len(base))
+            assert np.array_equal(ctx.sample_batch(bf_dev, base, u), oracle_tokens(bf_exact, base, u)), polls
+            _check_spec(ctx, t, q, k, spec_params, us)
+    finally:
+        ctx._check(H.sr_debug_set_row_wait_limit(ctx.h, 1 << 15))
