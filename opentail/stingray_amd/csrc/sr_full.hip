@@ -921,7 +921,7 @@ __device__ __forceinline__ float load_logit(const char* rowp, int i)
 // batch holds such a row), and for a row with more edits than it takes, the row keeps its adjusted copy.
 __device__ __forceinline__ bool row_edits_on_the_fly(const SrRow& rd, const SrFullArgs& a)
 {
-    return a.edit_tab != nullptr && sr_row_edits_on_the_fly(rd, a.vocab);
+    return (a.edit_tab != nullptr || a.edits_in_pass) && sr_row_edits_on_the_fly(rd, a.vocab);
 }
 __device__ __forceinline__ bool row_is_direct(const SrRow& rd, const SrFullArgs& a)
 {
@@ -1080,6 +1080,7 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
     const SrRow rd = a.rows[row];
     if (rd.edit_cnt <= 0) return;
     const SrEdit* ed = a.edits + rd.edit_off;
+    if (a.edits_in_pass && row_edits_on_the_fly(rd, a)) return;  // (k_full_softmax_seg applies them where it loads the row)
     if (row_edits_on_the_fly(rd, a)) {
         // the row's bitmap (cleared first: the barrier's wait for the stores stands between them and the atomics on
         // the same words), the adjusted and scaled values of its edits, and their share of the row's maximum
@@ -1094,7 +1095,6 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
         const bool scale = rd.temperature != 1.0f;
         const float inv_temp = scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
         const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u;
-        float* wseg = a.seg_func ? a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride : nullptr;
         uint32_t k = 0u;
         for (int e = threadIdx.x; e < rd.edit_cnt; e += 256) {
             const int id = ed[e].id;
@@ -1104,7 +1104,6 @@ __global__ __launch_bounds__(256) void k_full_edits(SrFullArgs a)
             x = edited_logit(x, ed[e], rd, true, pen);
             if (scale) x = __fmul_rn(x, inv_temp);
             vals[e] = x;
-            if (wseg) wseg[id] = x;  // (the passes over segments take an edited id's value from the work row)
             const uint32_t kv = (x != x) ? 0xffffffffu : sr_okey(x);  // NaN propagates (TensorPrimitives.Max)
             k = kv > k ? kv : k;
         }
@@ -1232,7 +1231,6 @@ template <int ES>
 struct SegSource {
     const char* rowp;      // the row's logits, or null: the adjusted copy in w
     const uint32_t* mrow;
-    const uint32_t* erow;
     const float* w;
     bool scale;
     float inv_temp;
@@ -1244,7 +1242,6 @@ __device__ __forceinline__ SegSource<ES> seg_source(const SrRow& rd, const SrFul
     src.w = a.work + (size_t)(a.work_by_row ? row : slot) * a.work_stride;
     src.rowp = nullptr;
     src.mrow = nullptr;
-    src.erow = nullptr;
     src.scale = false;
     src.inv_temp = 1.0f;
     if (row_is_direct(rd, a)) {
@@ -1252,7 +1249,6 @@ __device__ __forceinline__ SegSource<ES> seg_source(const SrRow& rd, const SrFul
         src.mrow = (rd.mask_row >= 0) ? a.mask + (size_t)rd.mask_row * a.mask_stride : nullptr;
         src.scale = rd.temperature != 1.0f;
         src.inv_temp = src.scale ? __fdiv_rn(1.0f, rd.temperature) : 1.0f;
-        src.erow = rd.edit_cnt > 0 ? a.edit_tab + (size_t)slot * (size_t)a.edit_tab_stride : nullptr;
     }
     return src;
 }
@@ -1274,15 +1270,13 @@ __device__ __forceinline__ void seg_load_logits(const SegSource<ES>& src, int se
         // a whole segment (all but a row's last): every load is issued before anything is done with one of them
         if (src.rowp) {
             uint4 raw[K];
-            uint32_t keep[K], hit[K];
+            uint32_t keep[K];
 #pragma unroll
             for (int k = 0; k < K; k++) {
                 const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
                 raw[k] = *(const uint4*)(src.rowp + (size_t)i0 * ES);
                 keep[k] = 0xffffffffu;
-                hit[k] = 0u;
                 if (src.mrow) keep[k] = src.mrow[i0 >> 5] >> (i0 & 31);
-                if (src.erow) hit[k] = (src.erow[i0 >> 5] >> (i0 & 31)) & ((1u << E) - 1u);
             }
 #pragma unroll
             for (int k = 0; k < K; k++) {
@@ -1301,15 +1295,6 @@ __device__ __forceinline__ void seg_load_logits(const SegSource<ES>& src, int se
                 for (int q = 0; q < E; q++) {
                     const float v = ((keep[k] >> q) & 1u) ? xv[q] : SR_NEG_INF;
                     xv[q] = src.scale ? __fmul_rn(v, src.inv_temp) : v;
-                }
-            }
-#pragma unroll
-            for (int k = 0; k < K; k++) {
-                if (hit[k] != 0u) {
-                    const int i0 = seg * SR_SEG_TERMS + (k * SR_WAVE + lane) * E;
-#pragma unroll
-                    for (int q = 0; q < E; q++)
-                        if ((hit[k] >> q) & 1u) x[k * E + q] = src.w[i0 + q];
                 }
             }
         } else {
@@ -1349,9 +1334,8 @@ __device__ __forceinline__ void seg_load_logits(const SegSource<ES>& src, int se
             }
             continue;
         }
-        uint32_t keep = (1u << E) - 1u, hit = 0u;
+        uint32_t keep = (1u << E) - 1u;
         if (src.mrow) keep = src.mrow[i0 >> 5] >> (i0 & 31);
-        if (src.erow) hit = (src.erow[i0 >> 5] >> (i0 & 31)) & ((1u << E) - 1u);
         if (whole) {
             const uint4 v = *(const uint4*)(src.rowp + (size_t)i0 * ES);
             if (ES == 4) {
@@ -1374,10 +1358,46 @@ __device__ __forceinline__ void seg_load_logits(const SegSource<ES>& src, int se
             if (src.scale) v = __fmul_rn(v, src.inv_temp);
             xv[q] = (i0 + q < n) ? v : SR_NEG_INF;
         }
-        if (hit != 0u) {
+    }
+}
+// The ids of segment `seg` that the row's edits touch (a row that keeps no adjusted copy): their values in x, as
+// seg_load_logits left them, are replaced by the adjusted ones -- LogitBias and the history penalties on the masked
+// logit, then the temperature (Sampler.cs:51-58, :367-419).  entry(i, id, e) names the i-th candidate of `count`: an id and
+// its place in the row's edit list; 64 candidates at a time, a lane each, then the owners of the hits take them one
+// by one.
+template <int ES, typename Entry>
+__device__ __forceinline__ void seg_apply_edits(const SrFullArgs& a, const SrRow& rd, const SegSource<ES>& src, int seg, int lane,
+                                                int count, Entry entry, float (&x)[SR_SEQ_RUN])
+{
+    constexpr int E = 16 / ES;
+    const SrEdit* ed = a.edits + rd.edit_off;
+    const bool pen = (rd.flags & SR_ROWFLAG_HAS_PENALTY) != 0u;
+    const int lo = seg * SR_SEG_TERMS;
+    for (int base = 0; base < count; base += SR_WAVE) {
+        int id = -1;
+        float val = 0.0f;
+        if (base + lane < count) {
+            int e = 0;
+            entry(base + lane, id, e);
+            if (id >= lo && id < lo + SR_SEG_TERMS && id < a.vocab) {
+                float v = load_logit<ES>(src.rowp, id);
+                if (src.mrow && !((src.mrow[id >> 5] >> (id & 31)) & 1u)) v = SR_NEG_INF;
+                v = edited_logit(v, ed[e], rd, true, pen);
+                val = src.scale ? __fmul_rn(v, src.inv_temp) : v;
+            } else {
+                id = -1;
+            }
+        }
+        unsigned long long todo = __ballot(id >= 0);
+        while (todo != 0ull) {
+            const int h = __ffsll((long long)todo) - 1;
+            todo &= todo - 1ull;
+            const int local = __shfl(id, h) - lo;
+            const float vh = __shfl(val, h);
+            const int v = local / E, j = (v / SR_WAVE) * E + local % E;
+            const bool mine = lane == v % SR_WAVE;
 #pragma unroll
-            for (int q = 0; q < E; q++)
-                if ((hit >> q) & 1u) xv[q] = src.w[i0 + q];
+            for (int jj = 0; jj < SR_SEQ_RUN; jj++) x[jj] = (mine && jj == j) ? vh : x[jj];
         }
     }
 }
@@ -1508,7 +1528,7 @@ __device__ __forceinline__ float seg_share(unsigned long long ms, float m)
     return (sum > 0.0f && k != 0xffffffffu) ? sum * __expf(sr_okey_inv(k) - m) : 0.0f;
 }
 template <int ES, int kW, int kS>
-__global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 4) void k_full_softmax_seg(SrFullArgs a)
+__global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 3) void k_full_softmax_seg(SrFullArgs a)
 {
     constexpr int kThreads = kW * SR_WAVE;
     const int slot = blockIdx.y, lane = sr_lane(), wave = sr_wave_id();
@@ -1522,6 +1542,11 @@ __global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 4) void k_full_softmax_
     __shared__ float share[SR_SEG_MAX];  // every segment's part of the row's approximate sum
     __shared__ uint32_t wkey[kW];
     __shared__ uint32_t bc[2];           // 0: the row's count came in   1: what k_full_edits made the row's maximum
+    // the row's edits that fall into this workgroup's segments (id << 32 | place in the row's edit list), and how many
+    // there are (more than the list holds: the waves go through the row's whole edit list instead)
+    constexpr int kHitCap = 256;
+    __shared__ unsigned long long hits[kHitCap];
+    __shared__ uint32_t n_hits;
     const int n = a.vocab, nseg = seg_count(n);
     SrFullState* st = a.state + slot;
     unsigned long long* sync = a.row_sync + (size_t)slot * SR_ROW_SYNC_STRIDE;
@@ -1545,12 +1570,47 @@ __global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 4) void k_full_softmax_
     c.m = 0.0f;
 
     // the first pass: the segment's maximum and approximate sum, written through for the row's other workgroups
+    // A row that keeps no adjusted copy although bias or penalties touch some of its ids: the workgroup looks through
+    // the row's edit list for the ids of its own segments, and its waves put the adjusted values in place of what they load
+    const bool edits = src.rowp != nullptr && rd.edit_cnt > 0;
+    const SrEdit* ed = a.edits + rd.edit_off;
+    if (edits) {
+        if (threadIdx.x == 0) n_hits = 0u;
+        sr_barrier_lds();
+        const int lo = (int)blockIdx.x * (kW * kS) * SR_SEG_TERMS, hi = lo + kW * kS * SR_SEG_TERMS;
+        for (int e = (int)threadIdx.x; e < rd.edit_cnt; e += kThreads) {
+            const int id = ed[e].id;
+            if (id >= lo && id < hi) {
+                const uint32_t pos = atomicAdd(&n_hits, 1u);
+                if (pos < (uint32_t)kHitCap) hits[pos] = ((unsigned long long)(uint32_t)id << 32) | (unsigned long long)(uint32_t)e;
+            }
+        }
+        sr_barrier_lds();
+    }
+    auto apply_edits = [&](int seg, float (&x)[SR_SEQ_RUN], bool from_hits) {
+        if (from_hits && n_hits <= (uint32_t)kHitCap)
+            seg_apply_edits<ES>(a, rd, src, seg, lane, (int)n_hits, [&](int i, int& id, int& e) {
+                const unsigned long long h = hits[i];
+                id = (int)(h >> 32);
+                e = (int)(uint32_t)h;
+            }, x);
+        else
+            seg_apply_edits<ES>(a, rd, src, seg, lane, rd.edit_cnt, [&](int i, int& id, int& e) {
+                id = ed[i].id;
+                e = i;
+            }, x);
+    };
     // (a wave takes kS segments, the workgroup's waves side by side: every one of its loads is out before the first is used)
     const int seg0 = (int)blockIdx.x * (kW * kS) + wave;
     float xs[kS][SR_SEQ_RUN];
 #pragma unroll
     for (int s = 0; s < kS; s++)
         if (seg0 + s * kW < nseg) seg_load_logits<ES>(src, seg0 + s * kW, lane, n, xs[s]);
+    if (edits) {
+#pragma unroll
+        for (int s = 0; s < kS; s++)
+            if (seg0 + s * kW < nseg) apply_edits(seg0 + s * kW, xs[s], true);
+    }
 #pragma unroll
     for (int s = 0; s < kS; s++)
         if (seg0 + s * kW < nseg) {
@@ -1666,6 +1726,7 @@ __global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 4) void k_full_softmax_
         whose = __shfl(whose, 0);
         if (kind != SR_SEG_LATE || whose != a.seq) continue;
         seg_load_logits<ES>(src, g, lane, n, xs[0]);
+        if (edits) apply_edits(g, xs[0], false);  // (the list in shared memory is of this workgroup's own segments)
         float before = 0.0f;
         for (int h = lane; h < g; h += SR_WAVE) before += share[h];
         before = sr_wave_sum_f32(before);

@@ -43,12 +43,23 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     a.lazy_scale = lazy_scale ? 1 : 0;
     // Which of the rows that come here keep an adjusted copy, and which have their edits applied where they are read
     // (the rows of the batch that take this path: every row in modes 1 / 2).
+    // Long rows that start on 16-byte boundaries, logits and work rows alike: the softmax denominators are prepared by
+    // the pass over the whole device (k_full_softmax_seg) and the rows' workgroups only walk the records.  That pass also
+    // applies the edits of the rows without an adjusted copy itself: they need no table and no kernel in front.
+    const int nseg = (vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
+    const bool seg_mode = [&] {
+        const int es = dtype == SR_DTYPE_BF16 ? 2 : 4;
+        const bool aligned = (((uintptr_t)logits_dev) & 15u) == 0u && ((row_stride * es) & 15) == 0 &&
+                             (((uintptr_t)a.work) & 15u) == 0u && ((a.work_stride * 4) & 15) == 0;
+        return vocab >= SR_SEG_MIN_VOCAB && nseg <= SR_SEG_MAX && aligned;
+    }();
+    a.edits_in_pass = seg_mode ? 1 : 0;
     bool any_table = false, any_copy = false, any_edits = false;
     for (const SrRow& r : (host_rows ? *host_rows : b->h_rows)) {
         if (mode == 0 && r.path != SR_PATH_FULL) continue;
         const bool on_the_fly = sr_row_edits_on_the_fly(r, vocab);
-        any_table = any_table || on_the_fly;
-        any_edits = any_edits || r.edit_cnt > 0;
+        any_table = any_table || (on_the_fly && !seg_mode);
+        any_edits = any_edits || (r.edit_cnt > 0 && !(on_the_fly && seg_mode));
         any_copy = any_copy || !(r.temperature > 0.0f && (r.edit_cnt <= 0 || on_the_fly));
     }
     a.any_copy = any_copy ? 1 : 0;
@@ -87,14 +98,8 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     // the kernels index sort segments with work_stride; keep both strides equal in mode 0 and pass the
     // segment stride separately otherwise
     a.sort_stride = seg_stride;
-    // Long rows that start on 16-byte boundaries, logits and work rows alike: the softmax denominators are prepared by
-    // the pass over the whole device (k_full_softmax_seg) and the rows' workgroups only walk the records
     {
-        const int es = dtype == SR_DTYPE_BF16 ? 2 : 4;
-        const int nseg = (vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
-        const bool aligned = (((uintptr_t)logits_dev) & 15u) == 0u && ((row_stride * es) & 15) == 0 &&
-                             (((uintptr_t)a.work) & 15u) == 0u && ((a.work_stride * 4) & 15) == 0;
-        if (vocab >= SR_SEG_MIN_VOCAB && nseg <= SR_SEG_MAX && aligned) {
+        if (seg_mode) {
             SR_HIP(ctx, ctx->full_seg_func.reserve((size_t)n_rows * (size_t)nseg * sizeof(SeqSegFunc), st, true));
             SR_HIP(ctx, ctx->full_seg_ms.reserve((size_t)n_rows * (size_t)nseg * sizeof(float2), st));
             SR_HIP(ctx, ctx->full_watch.reserve((size_t)n_rows * SR_FULL_SMALL_CAP * sizeof(unsigned long long), st));

@@ -762,3 +762,34 @@ def test_workgroups_that_stop_waiting_for_their_row_leave_their_segments_to_the_
             _check_spec(ctx, t, q, k, spec_params, us)
     finally:
         ctx._check(H.sr_debug_set_row_wait_limit(ctx.h, 1 << 15))
+
+
+def test_edits_crowded_into_a_few_segments_of_a_long_row(ctx):
+    """The pass over long rows applies the edits of a sampled row where it loads the row: a workgroup lists the edits
+    that fall into its segments (room for 256) and goes through the row's whole edit list when there are more.  Rows
+    whose history and bias ids crowd into the first 3,000 ids, into one segment, and at the very end of the row."""
+    rng = np.random.default_rng(606)
+    V = 45_000  # (a ragged last segment)
+    logits = rng.normal(0, 2.0, (5, V)).astype(np.float32)
+    low = rng.permutation(3000)[:900].tolist()
+    one_seg = (2048 + rng.permutation(1024)[:700]).tolist()
+    tail = (V - 1 - rng.permutation(900)[:500]).tolist()
+    params = [SamplingParams(Temperature=0.9, TopP=0.9, RepetitionPenalty=1.3, RepeatLastN=0, PreviousTokens=low + low[:50]),
+              SamplingParams(Temperature=1.0, MinP=0.01, PresencePenalty=0.6, FrequencyPenalty=0.2, RepeatLastN=0, PreviousTokens=one_seg),
+              SamplingParams(Temperature=0.8, TopP=0.95, LogitBias={int(i): float(b) for i, b in zip(tail[:300], rng.normal(0, 2, 300))},
+                             PresencePenalty=0.3, RepeatLastN=0, PreviousTokens=tail),
+              SamplingParams(Temperature=1.1, RepetitionPenalty=0.8, RepeatLastN=0, PreviousTokens=low[:400] + tail[:400]),
+              SamplingParams(Temperature=0.7, LogitBias={int(i): 4.0 for i in one_seg[:280]})]
+    for p in params:
+        for i in (p.PreviousTokens or [])[:8]:
+            logits[params.index(p), i] += 6.0  # some of the edited ids carry mass: the edits decide
+    for _ in range(3):
+        _check_rows(ctx, logits, params, rng.random(5))
+    _check_distribution(ctx, logits, params)
+    bits = synthetic.to_bf16_bits(logits)
+    import torch
+
+    dev = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16).cuda()
+    exact = synthetic.bf16_bits_to_f32(bits)
+    u = rng.random(5)
+    assert np.array_equal(ctx.sample_batch(dev, params, u), oracle_tokens(exact, params, u))
