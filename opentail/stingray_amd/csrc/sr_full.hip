@@ -1572,20 +1572,20 @@ __global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 3) void k_full_softmax_
     // the first pass: the segment's maximum and approximate sum, written through for the row's other workgroups
     // A row that keeps no adjusted copy although bias or penalties touch some of its ids: the workgroup looks through
     // the row's edit list for the ids of its own segments, and its waves put the adjusted values in place of what they load
+    // (the ids are asked for in front of the logits and looked at behind them: the loads overlap)
     const bool edits = src.rowp != nullptr && rd.edit_cnt > 0;
     const SrEdit* ed = a.edits + rd.edit_off;
+    constexpr int kIds = SR_FULL_EDIT_VALUES / kThreads;
+    static_assert(kIds * kThreads == SR_FULL_EDIT_VALUES, "every edit of a row without an adjusted copy is looked at");
+    int ids[kIds];
     if (edits) {
         if (threadIdx.x == 0) n_hits = 0u;
         sr_barrier_lds();
-        const int lo = (int)blockIdx.x * (kW * kS) * SR_SEG_TERMS, hi = lo + kW * kS * SR_SEG_TERMS;
-        for (int e = (int)threadIdx.x; e < rd.edit_cnt; e += kThreads) {
-            const int id = ed[e].id;
-            if (id >= lo && id < hi) {
-                const uint32_t pos = atomicAdd(&n_hits, 1u);
-                if (pos < (uint32_t)kHitCap) hits[pos] = ((unsigned long long)(uint32_t)id << 32) | (unsigned long long)(uint32_t)e;
-            }
+#pragma unroll
+        for (int j = 0; j < kIds; j++) {
+            const int e = (int)threadIdx.x + j * kThreads;
+            ids[j] = e < rd.edit_cnt ? ed[e].id : -1;
         }
-        sr_barrier_lds();
     }
     auto apply_edits = [&](int seg, float (&x)[SR_SEQ_RUN], bool from_hits) {
         if (from_hits && n_hits <= (uint32_t)kHitCap)
@@ -1607,6 +1607,16 @@ __global__ __launch_bounds__(kW * SR_WAVE, kS == 2 ? 5 : 3) void k_full_softmax_
     for (int s = 0; s < kS; s++)
         if (seg0 + s * kW < nseg) seg_load_logits<ES>(src, seg0 + s * kW, lane, n, xs[s]);
     if (edits) {
+        const int lo = (int)blockIdx.x * (kW * kS) * SR_SEG_TERMS, hi = lo + kW * kS * SR_SEG_TERMS;
+#pragma unroll
+        for (int j = 0; j < kIds; j++) {
+            if (ids[j] >= lo && ids[j] < hi) {
+                const uint32_t pos = atomicAdd(&n_hits, 1u);
+                if (pos < (uint32_t)kHitCap)
+                    hits[pos] = ((unsigned long long)(uint32_t)ids[j] << 32) | (unsigned long long)(uint32_t)((int)threadIdx.x + j * kThreads);
+            }
+        }
+        sr_barrier_lds();
 #pragma unroll
         for (int s = 0; s < kS; s++)
             if (seg0 + s * kW < nseg) apply_edits(seg0 + s * kW, xs[s], true);
@@ -2962,7 +2972,25 @@ __global__ __launch_bounds__(kT) void k_full_row(SrFullArgs a)
                 for (int i = tid; i < nc; i += kT) sm.sprob[i] = sr_u2f((uint32_t)(sm.sortbuf[i] >> 32));
                 __syncthreads();
                 int found;
-                run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, rd.top_p, &found, sm);
+                if (nc <= SR_WAVE) {
+                    // a handful of survivors (a row that min-p has cut): one thread adds them the way the scalar loop does
+                    if (tid == 0) {
+                        float s = run;
+                        int f = -1;
+                        for (int i = 0; i < nc && f < 0; i++) {
+                            s = __fadd_rn(s, sm.sprob[i]);
+                            if (s >= rd.top_p) f = i;
+                        }
+                        sm.segbc[1] = (uint32_t)f;
+                        sm.segbc[2] = sr_f2u(s);
+                    }
+                    __syncthreads();
+                    found = (int)sm.segbc[1];
+                    run = sr_u2f(sm.segbc[2]);
+                    __syncthreads();  // (the words may be written again for the next slab)
+                } else {
+                    run = seq_sum<true>([&](int i) -> float { return sm.sprob[i]; }, nc, run, rd.top_p, &found, sm);
+                }
                 if (found >= 0)
                     SR_AMB_IF(sr_stop_near(run, sm.sprob[found], rd.top_p) || (found + 1 < nc && sm.sprob[found + 1] == sm.sprob[found]));
                 else if (taken + nc == ns)
@@ -3697,9 +3725,9 @@ hipError_t sr_launch_full_prep(const SrFullArgs& a, int n_rows, hipStream_t st)
     }
     if (a.seg_func) {
         const int nseg = (a.vocab + SR_SEG_TERMS - 1) / SR_SEG_TERMS;
-        // a wave takes one segment, or two where the launch has more segments than the device holds waves of the
-        // one-segment kind at a time: the waves of a row's workgroups wait for each other between the passes
-        const bool two = (long long)n_rows * nseg > 2048;
+        // a wave takes one segment, or two where the launch's sampled rows have more segments than the device holds waves
+        // of the one-segment kind at a time: the waves of a row's workgroups wait for each other between the passes
+        const bool two = (long long)a.n_sampled * nseg > 3072;
         const int per_group = 4 * (two ? 2 : 1);
         dim3 fgrid((unsigned)((nseg + per_group - 1) / per_group), n_rows);
         if (a.dtype == 1) {

@@ -55,15 +55,19 @@ int run_full(sr_ctx* ctx, const sr_batch* b, const int32_t* list_dev, int n_rows
     }();
     a.edits_in_pass = seg_mode ? 1 : 0;
     bool any_table = false, any_copy = false, any_edits = false;
+    int n_sampled = 0, n_seen = 0;
     for (const SrRow& r : (host_rows ? *host_rows : b->h_rows)) {
         if (mode == 0 && r.path != SR_PATH_FULL) continue;
         const bool on_the_fly = sr_row_edits_on_the_fly(r, vocab);
         any_table = any_table || (on_the_fly && !seg_mode);
+        n_sampled += r.temperature > 0.0f ? 1 : 0;
+        n_seen++;
         any_edits = any_edits || (r.edit_cnt > 0 && !(on_the_fly && seg_mode));
         any_copy = any_copy || !(r.temperature > 0.0f && (r.edit_cnt <= 0 || on_the_fly));
     }
     a.any_copy = any_copy ? 1 : 0;
     a.any_edits = any_edits ? 1 : 0;
+    a.n_sampled = (int)((long long)n_sampled * n_rows / std::max(1, n_seen));  // (a verifier's launch has every row several times)
     a.edit_tab = nullptr;
     a.edit_tab_stride = (((int64_t)vocab + 31) / 32 + SR_FULL_EDIT_VALUES + 3) & ~(int64_t)3;
     if (any_table) {

@@ -185,6 +185,7 @@ struct SrFullArgs {
     uint16_t* seg_keys;            // [slot][seg_key_stride]: the upper 16 bits of every e of a row that only top-p cuts (0: e = 0)
     int64_t seg_key_stride;
     uint32_t seq;                  // the launch's number (never 0): see SrFullState::maxkey
+    int32_t n_sampled;             // rows of the launch with a temperature above 0 (greedy rows leave the passes at once)
     int32_t any_edits;             // some row of the launch has edits for k_full_edits (else it is not launched)
     int32_t edits_in_pass;         // seg_func is set: sampled rows with up to SR_FULL_EDIT_VALUES edits keep no adjusted copy and
                                    // need no table either (k_full_softmax_seg applies their edits where it loads the row)
