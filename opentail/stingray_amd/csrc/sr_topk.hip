@@ -1589,10 +1589,10 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     // smallest of them has at least sel group maxima of the row at or above it.
     float tval = -3.402823466e38f;
     {
-        const int nb = S * kWaves;
+        const int nb = kKept ? kWaves : S * kWaves;  // (a worker that keeps its row's results: one share per wave and row)
         uint32_t k = 0xffffffffu, km = 0u;
         if constexpr (kKept) {
-            if (lane < nb) {  // nb <= kKeptChunks * kWaves
+            if (lane < nb) {
                 k = sm.hist[2 * lane];
                 km = sm.hist[2 * lane + 1];
             }
@@ -1903,6 +1903,55 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
         // vector, to no effect (one line, already in cache), so that the loop body is the same for every chunk: with
         // two bodies, or a condition around the loads, the compiler keeps the incoming vectors in registers of their
         // own and spills.
+        int last_sel = 0;
+        // (kKept) group maxima of the wave, over all chunks folded so far, at or above the value of key `cnd`
+        // (kKept) The wave's share of the row's bound, taken from the largest group maximum of every lane and chunk folded
+        // so far (one value per lane and chunk instead of four: a lane with two groups of a chunk at or above the value
+        // counts once, which can only lower the value and keeps it a bound -- a twelfth of the count at the largest
+        // shares -- and a count costs four ballots instead of sixteen): the largest key, to 16 bits, with at least
+        // `need` of those values at or above it; 0 when there is none.  *wmax = the wave's largest kept element.
+        // The value nearly always has the sign and exponent of the wave's largest maximum, or the exponent below: those
+        // nine bits are tried as a whole and the seven bits below them one by one, eight or nine counts instead of
+        // sixteen.
+        auto kept_share = [&](int need, uint32_t* wmax_out) SR_INL -> uint32_t {
+            float pool[kKeptChunks];
+#pragma unroll
+            for (int c = 0; c < kKeptChunks; c++)
+                pool[c] = fmaxf(fmaxf(kept.g1[c].x, kept.g1[c].y), fmaxf(kept.g1[c].z, kept.g1[c].w));
+            auto enough = [&](uint32_t cnd) SR_INL -> bool {
+                const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
+                int cge = 0;
+#pragma unroll
+                for (int c = 0; c < kKeptChunks; c++) cge += __popcll(__ballot(pool[c] >= fc));
+                return cge >= need;
+            };
+            const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(pool[0], pool[1]), fmaxf(pool[2], pool[3]))));
+            static_assert(kKeptChunks == 4, "four pool values");
+            *wmax_out = wmax;
+            uint32_t K = wmax & 0xff800000u;  // nothing lies at or above the next exponent's first key
+            bool head = false;
+#pragma unroll 1
+            for (int t = 0; t < 2 && !head; t++) {
+                if (enough(K)) head = true;
+                else if (K >= 0x00800000u) K -= 0x00800000u;
+                else break;
+            }
+            if (head) {
+#pragma unroll 1
+                for (int bit = 22; bit >= 16; bit--) {
+                    const uint32_t cnd = K | (1u << bit);
+                    if (enough(cnd)) K = cnd;
+                }
+            } else {
+                K = 0u;
+#pragma unroll 1
+                for (int bit = 31; bit >= 16; bit--) {
+                    const uint32_t cnd = K | (1u << bit);
+                    if (enough(cnd)) K = cnd;
+                }
+            }
+            return K;
+        };
         for (int k = 0; k < n_items; k++) {
             const bool has_next = k + 1 < n_items;
             Geom nxt = cur;
@@ -1981,7 +2030,10 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
             // The wave's share of the row's bound: a value, to 16 bits and rounded down, with at least
             // ceil(sel / (chunks x 8)) of the wave's 256 group maxima at or above it (found bit by bit with ballots).
             // The smallest of all the row's waves' values then has at least sel group maxima at or above it.
-            {
+            // (A worker that keeps its row's results takes its share once, behind the row's last chunk, from the
+            // group maxima of all its chunks.)
+            last_sel = cur.sel;
+            if constexpr (!kKept) {
                 const int need = (cur.sel + S * kWaves - 1) / (S * kWaves);
                 uint32_t K = 0u;
 #pragma unroll 1
@@ -1995,15 +2047,9 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
                 // ... and the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
                 const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(gm1[0], gm1[1]), fmaxf(gm1[2], gm1[3]))));
                 if (lane == 0) {
-                    if constexpr (kKept) {
-                        const int w = (min(cur.c, kKeptChunks - 1) * kWaves + (tid >> 6)) * 2;
-                        sm.hist[w] = K;
-                        sm.hist[w + 1] = wmax;
-                    } else {
-                        uint32_t* gb = a.gbound + (((size_t)cur.slot * S + cur.c) * kWaves + (tid >> 6)) * 2;
-                        __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        __hip_atomic_store(gb + 1, wmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
+                    uint32_t* gb = a.gbound + (((size_t)cur.slot * S + cur.c) * kWaves + (tid >> 6)) * 2;
+                    __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(gb + 1, wmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
 #ifdef SR_PROFILE
@@ -2022,6 +2068,18 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
             SR_PROF(ap, 5);
 #endif
             cur = nxt;
+        }
+        // One share per wave for the whole row, behind its last chunk: with at least ceil(sel / 8) of the wave's group
+        // maxima at or above every wave's value, the smallest of the eight has sel of the row's at or above it.  The
+        // larger pools over-select less than a share per chunk did (a share of 125 of 1,024 scatters by a tenth, a
+        // share of 32 of 256 by a fifth, and the bound is the smallest of the shares), and one loop replaces four.
+        if constexpr (kKept) {
+            uint32_t wmax;
+            const uint32_t K = kept_share((last_sel + kWaves - 1) / kWaves, &wmax);
+            if (lane == 0) {
+                sm.hist[(tid >> 6) * 2] = K;
+                sm.hist[(tid >> 6) * 2 + 1] = wmax;
+            }
         }
     }
     if (prog.z < 0) return;
@@ -2045,7 +2103,7 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
     if constexpr (kKept) {
         // the row's results are in this workgroup's registers and LDS; a worker whose program is not of that kind (the
         // host writes none for this kernel) selects its row from the logits alone
-        __syncthreads();  // the waves' shares of the bound
+        // (the waves' shares of the bound are read behind the barrier that follows the clearing of the tail's lists)
         handed_over = own_row && S <= kKeptChunks && a.spin_limit != 0u;
     } else {
         if (own_row) sr_drain_stores();  // every wave's own stores; the barrier below joins them
