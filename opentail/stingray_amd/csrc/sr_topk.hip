@@ -432,6 +432,38 @@ __device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
 
 #define SR_INL __attribute__((always_inline))
 
+// The largest key, to its upper 16 bits, for which `enough` holds (0: none); `enough` must hold for every key below one
+// for which it holds, must not hold above `kmax`, and must be the same in every lane.  The answer nearly always has the
+// sign and exponent of kmax, or the exponent below: those nine bits are tried as a whole and the seven bits below them
+// one by one, eight or nine tries instead of sixteen.
+template <typename Enough>
+__device__ __forceinline__ uint32_t largest_key16(uint32_t kmax, Enough enough)
+{
+    uint32_t K = kmax & 0xff800000u;  // nothing lies at or above the next exponent's first key
+    bool head = false;
+#pragma unroll 1
+    for (int t = 0; t < 4 && !head; t++) {
+        if (enough(K)) head = true;
+        else if (K >= 0x00800000u) K -= 0x00800000u;
+        else break;
+    }
+    if (head) {
+#pragma unroll 1
+        for (int bit = 22; bit >= 16; bit--) {
+            const uint32_t cnd = K | (1u << bit);
+            if (enough(cnd)) K = cnd;
+        }
+    } else {
+        K = 0u;
+#pragma unroll 1
+        for (int bit = 31; bit >= 16; bit--) {
+            const uint32_t cnd = K | (1u << bit);
+            if (enough(cnd)) K = cnd;
+        }
+    }
+    return K;
+}
+
 // ---- the row tail ----------------------------------------------------------------------------------
 // Called by every thread of the tail workgroup of a row once all chunks of the row have been counted in.
 // slot = position of the row in this launch.
@@ -1608,21 +1640,19 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
         // share - 1) that are at least its first.  The largest value with sel of all those at or above it is a bound
         // too, and a much closer one than the smallest first word when sel is small (a top-k of 40 asks every wave
         // for its second largest: the smallest of 32 of those has some 250 elements above it, the 40th largest of the
-        // 64 words about 50).  With one pair per lane it is found bit by bit with ballots, to 16 bits, rounded down.
-        // (Worth its 32 ballots, about 1 us, only where the shares are that small.)
+        // 64 words about 50).  With one pair per lane it is found with ballots, to 16 bits, rounded down (worth its
+        // eight or nine pairs of ballots only where the shares are that small).
         uint32_t k_close = 0u;
         const int share = (sel + nb - 1) / nb;  // (the waves' share was this or more)
+        const uint32_t km_lane = km;
+        km = sr_wave_max_u32(km);
         if (kShort && nb <= SR_WAVE && share <= 2) {
             const bool in = lane < nb;
-#pragma unroll 1
-            for (int bit = 31; bit >= 16; bit--) {
-                const uint32_t cnd = k_close | (1u << bit);
-                const int w = __popcll(__ballot(in && k >= cnd)) * (share - 1) + __popcll(__ballot(in && km >= cnd));
-                if (w >= sel) k_close = cnd;
-            }
+            k_close = largest_key16(km, [&](uint32_t cnd) SR_INL -> bool {
+                return __popcll(__ballot(in && k >= cnd)) * (share - 1) + __popcll(__ballot(in && km_lane >= cnd)) >= sel;
+            });
         }
         k = sr_wave_min_u32(k);
-        km = sr_wave_max_u32(km);
         k = max(k, k_close);
         if (k > kKeyNegInf) tval = sr_okey_inv(k);
         // An element 19 T below the row's largest kept element has expf((v - max) / T) < 2^-26 whatever else
@@ -1910,9 +1940,6 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
         // counts once, which can only lower the value and keeps it a bound -- a twelfth of the count at the largest
         // shares -- and a count costs four ballots instead of sixteen): the largest key, to 16 bits, with at least
         // `need` of those values at or above it; 0 when there is none.  *wmax = the wave's largest kept element.
-        // The value nearly always has the sign and exponent of the wave's largest maximum, or the exponent below: those
-        // nine bits are tried as a whole and the seven bits below them one by one, eight or nine counts instead of
-        // sixteen.
         auto kept_share = [&](int need, uint32_t* wmax_out) SR_INL -> uint32_t {
             float pool[kKeptChunks];
 #pragma unroll
@@ -1928,28 +1955,7 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
             const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(pool[0], pool[1]), fmaxf(pool[2], pool[3]))));
             static_assert(kKeptChunks == 4, "four pool values");
             *wmax_out = wmax;
-            uint32_t K = wmax & 0xff800000u;  // nothing lies at or above the next exponent's first key
-            bool head = false;
-#pragma unroll 1
-            for (int t = 0; t < 2 && !head; t++) {
-                if (enough(K)) head = true;
-                else if (K >= 0x00800000u) K -= 0x00800000u;
-                else break;
-            }
-            if (head) {
-#pragma unroll 1
-                for (int bit = 22; bit >= 16; bit--) {
-                    const uint32_t cnd = K | (1u << bit);
-                    if (enough(cnd)) K = cnd;
-                }
-            } else {
-                K = 0u;
-#pragma unroll 1
-                for (int bit = 31; bit >= 16; bit--) {
-                    const uint32_t cnd = K | (1u << bit);
-                    if (enough(cnd)) K = cnd;
-                }
-            }
+            const uint32_t K = largest_key16(wmax, enough);
             return K;
         };
         for (int k = 0; k < n_items; k++) {
@@ -2034,18 +2040,14 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
             // group maxima of all its chunks.)
             last_sel = cur.sel;
             if constexpr (!kKept) {
-                const int need = (cur.sel + S * kWaves - 1) / (S * kWaves);
-                uint32_t K = 0u;
-#pragma unroll 1
-                for (int bit = 31; bit >= 16; bit--) {
-                    const uint32_t cnd = K | (1u << bit);
-                    const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
-                    const int cge = __popcll(__ballot(gm1[0] >= fc)) + __popcll(__ballot(gm1[1] >= fc)) +
-                                    __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc));
-                    if (cge >= need) K = cnd;
-                }
-                // ... and the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
+                const int need = max((cur.sel + S * kWaves - 1) / (S * kWaves), 1);
+                // the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
                 const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(gm1[0], gm1[1]), fmaxf(gm1[2], gm1[3]))));
+                const uint32_t K = largest_key16(wmax, [&](uint32_t cnd) SR_INL -> bool {
+                    const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
+                    return __popcll(__ballot(gm1[0] >= fc)) + __popcll(__ballot(gm1[1] >= fc)) +
+                           __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc)) >= need;
+                });
                 if (lane == 0) {
                     uint32_t* gb = a.gbound + (((size_t)cur.slot * S + cur.c) * kWaves + (tid >> 6)) * 2;
                     __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -2075,7 +2077,7 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
         // share of 32 of 256 by a fifth, and the bound is the smallest of the shares), and one loop replaces four.
         if constexpr (kKept) {
             uint32_t wmax;
-            const uint32_t K = kept_share((last_sel + kWaves - 1) / kWaves, &wmax);
+            const uint32_t K = kept_share(max((last_sel + kWaves - 1) / kWaves, 1), &wmax);
             if (lane == 0) {
                 sm.hist[(tid >> 6) * 2] = K;
                 sm.hist[(tid >> 6) * 2 + 1] = wmax;
