@@ -863,16 +863,19 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             if (n_all == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
             if (short_list) {
                 const int kk = min(rd.top_k, n_all);
-                const int e = tid >> 2, part = tid & 3;
+                // four threads to an entry, eight when the list is at most half as long
                 static_assert(kShortList * 4 <= kThreads, "four threads to an entry");
+                const bool eight = n_all * 8 <= kThreads;
+                const int e = eight ? tid >> 3 : tid >> 2, part = eight ? tid & 7 : tid & 3, parts = eight ? 8 : 4;
                 uint32_t mh = 0u, mm = 0u, ml = 0u;
                 int ahead = 0;
                 if (e < n_all) {
                     mh = sm.xa[e]; mm = sm.xb[e]; ml = sm.xc[e];
-                    for (int j = part; j < n_all; j += 4) ahead += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
+                    for (int j = part; j < n_all; j += parts) ahead += key3_less(mh, mm, ml, sm.xa[j], sm.xb[j], sm.xc[j]) ? 1 : 0;
                 }
                 ahead += __shfl_xor(ahead, 1);
                 ahead += __shfl_xor(ahead, 2);
+                if (eight) ahead += __shfl_xor(ahead, 4);
                 if (e < n_all && part == 0 && ahead < kk) {
                     sm.vals[ahead] = sr_okey_inv(mh);
                     sm.idxs[ahead] = (int)(0xffffffffu - ml);
