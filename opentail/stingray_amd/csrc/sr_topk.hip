@@ -556,6 +556,8 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         else { hee[r] = SrEdit{}; hx[r] = SR_NEG_INF; }
     }
     const float inv_temp = rd.temperature == 1.0f ? 1.0f : __fdiv_rn(1.0f, rd.temperature);
+    // the row's uniform is asked for now: at the draw, the last step of the chain, it would be waited for
+    const float u_row = rd.path == SR_PATH_TOPK ? __double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]) : 0.0f;
     // rows without penalties that may raise a logit have their candidates binned while they are collected
     const bool want_bins = rd.path == SR_PATH_TOPK && (!use_edits || hist_regs);
     bool binned = false;
@@ -1277,7 +1279,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         const int hit = first_reach(top_p, count, &kept_sum);
         const int cnt = hit >= 0 ? hit + 1 : count;
         SR_PROF(a, 10);
-        const float r = __fmul_rn(__double2float_rn(a.uniforms[(size_t)row * a.uniforms_per_row]), kept_sum);
+        const float r = __fmul_rn(u_row, kept_sum);
         float at = 0.0f;
         const int first = first_reach(r, cnt, &at);
         int token = sm.idxs[first >= 0 ? first : 0];
@@ -1536,6 +1538,13 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
             gpr[c] = in ? a.gpos[((size_t)slot * S + c) * kThreads + tid] : 0u;
         }
     }
+    // (not kKept) the waves' shares of the bound, asked for with the group results: behind the barrier below they
+    // would be a round trip to memory of their own
+    const int nb = kKept ? kWaves : S * kWaves;  // (a worker that keeps its row's results: one share per wave and row)
+    uint2 gb0 = make_uint2(0xffffffffu, 0u);
+    if constexpr (!kKept) {
+        if (lane < nb) gb0 = ((const uint2*)a.gbound + (size_t)slot * nb)[lane];
+    }
     early();
     auto each_gm = [&](auto&& f) SR_INL {
 #pragma unroll
@@ -1624,7 +1633,6 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
     // smallest of them has at least sel group maxima of the row at or above it.
     float tval = -3.402823466e38f;
     {
-        const int nb = kKept ? kWaves : S * kWaves;  // (a worker that keeps its row's results: one share per wave and row)
         uint32_t k = 0xffffffffu, km = 0u;
         if constexpr (kKept) {
             if (lane < nb) {
@@ -1632,8 +1640,10 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
                 km = sm.hist[2 * lane + 1];
             }
         } else {
+            k = gb0.x;
+            km = gb0.y;
             const uint2* gb = (const uint2*)a.gbound + (size_t)slot * nb;
-            for (int i = lane; i < nb; i += SR_WAVE) {
+            for (int i = lane + SR_WAVE; i < nb; i += SR_WAVE) {
                 const uint2 b = gb[i];
                 k = min(k, b.x);
                 km = max(km, b.y);
