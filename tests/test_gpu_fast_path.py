@@ -309,6 +309,39 @@ def test_large_values_concentrated_in_few_lanes(ctx):
     _check_rows(ctx, logits, params, rng.random(rows), _cuda(logits))
 
 
+def test_large_values_concentrated_in_few_lanes_with_a_worker_per_row(ctx):
+    # The same with enough rows for the launch in which every worker keeps its row's results and takes one share of
+    # the bound per wave and row, from one value per lane and chunk: the large values of a row lie in sixteen lanes of
+    # one wave, in one lane, or in one lane's vectors of one group, so that a lane counts once for many of them and
+    # the wave's share falls far below the row's k-th largest (the exact selection has to take over), for top-k of
+    # every size, greedy rows and rows with a history.  fp32 and bf16.
+    import torch
+
+    rng = np.random.default_rng(36)
+    V, rows = 40_000, 150
+    logits = rng.normal(0, 1.0, (rows, V)).astype(np.float32)
+    e = np.arange(V)
+    vec = e // 4
+    kinds = [(vec % 512) < 16, (vec % 512) == 77, ((vec % 512) == 300) & ((vec // 512) % 4 == 1), (vec % 512) >= 448]
+    params = []
+    for r in range(rows):
+        hot = kinds[r % 4]
+        logits[r, hot] += 40.0 + rng.random(int(hot.sum())).astype(np.float32)
+        k = int(rng.choice([1, 2, 7, 40, 64, 65, 200, 500, 1000]))
+        if r % 11 == 0:
+            params.append(SamplingParams(Temperature=0.0))
+        elif r % 11 == 1:
+            params.append(SamplingParams(Temperature=0.9, TopK=k, TopP=0.97, RepetitionPenalty=1.2, FrequencyPenalty=0.1,
+                                         PreviousTokens=np.nonzero(hot)[0][:100].tolist()))
+        else:
+            params.append(SamplingParams(Temperature=float(rng.uniform(0.5, 1.4)), TopK=k, TopP=float(rng.choice([1.0, 0.97])),
+                                         MinP=float(rng.choice([0.0, 0.01]))))
+    u = rng.random(rows)
+    _check_rows(ctx, logits, params, u, _cuda(logits))
+    bits = synthetic.to_bf16_bits(logits)
+    _check_rows(ctx, synthetic.bf16_bits_to_f32(bits), params, u, _cuda(bits.view(np.int16), torch.bfloat16))
+
+
 def test_flat_rows_with_a_history(ctx):
     # every logit equal: the candidates all tie, the lowest indices win, and the penalised history ids drop out
     V = 50_000
