@@ -892,9 +892,11 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         }
         if (!short_list) {
         int bstar = kBins - 1, n_live = 0, n_keep = 0, max_bin = 0;
-        // every wave reads the histogram: live entries, and the first bin at which the k best are complete;
-        // wave 0 leaves every bin's first list position in sm.boff
+        // one wave reads the histogram: live entries, the first bin at which the k best are complete, and every bin's
+        // first list position (sm.boff); its results go out through sm.bcast[8..11], see scan_results
         auto scan_bins = [&]() SR_INL {
+            // (two waves share a SIMD: what every wave does for itself takes twice as long as what one wave does for all)
+            if (sr_wave_id() != 0) return;
             // lane l owns bins [l * kBinsPerLane, (l + 1) * kBinsPerLane)
             const int lane = sr_lane();
             const uint32_t* hb = sm.bhist + lane * (kBinsPerLane + 1);
@@ -909,11 +911,10 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             int c = incl - tot, bq = lane * kBinsPerLane + kBinsPerLane - 1, cq = incl;
             bool found = false;
             uint32_t hm = 0u;
-            const bool w0 = sr_wave_id() == 0;
 #pragma unroll
             for (int q = 0; q < kBinsPerLane; q++) {
                 const uint32_t h = hb[q];
-                if (w0) sm.boff[lane * (kBinsPerLane + 1) + q] = (uint32_t)c;
+                sm.boff[lane * (kBinsPerLane + 1) + q] = (uint32_t)c;
                 c += (int)h;
                 if (!found) hm = max(hm, h);  // bins up to and including the one that completes the k best
                 if (!found && c >= need) { bq = lane * kBinsPerLane + q; cq = c; found = true; }
@@ -923,6 +924,11 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             // the fullest kept bin bounds the ranking loop below
             if (lane > L) hm = 0u;
             max_bin = (int)sr_wave_max_u32(hm);
+            if (lane == 0) { sm.bcast[8] = (uint32_t)bstar; sm.bcast[9] = (uint32_t)n_live; sm.bcast[10] = (uint32_t)n_keep; sm.bcast[11] = (uint32_t)max_bin; }
+        };
+        // (one wave scans; the others take its results behind the barrier that follows)
+        auto scan_results = [&]() SR_INL {
+            bstar = (int)sm.bcast[8]; n_live = (int)sm.bcast[9]; n_keep = (int)sm.bcast[10]; max_bin = (int)sm.bcast[11];
         };
         bool by_bins = true;  // kept entries are laid out bin by bin and ranked inside their bin
         if (binned) {
@@ -948,9 +954,10 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
             }
             __syncthreads();
             scan_bins();
+            __syncthreads();  // sm.boff written, the scan's results out
+            scan_results();
             // no finite logit in the row: Greedy over the raw row = index 0 (Sampler.cs:254-255, :442-446)
             if (n_live == 0) { give_up(SR_KFLAG_DEGENERATE, 0); return; }
-            __syncthreads();  // sm.boff written, every wave done with the histogram
             SR_PROF(a, 6);
             if (n_keep <= kSelMax && max_bin <= ((EPV == 8 && bmap.exact) ? 256 : 96)) {
                 const uint32_t* meta = (const uint32_t*)sm.probs;
@@ -1005,6 +1012,8 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
         }
         __syncthreads();
         scan_bins();
+        __syncthreads();
+        scan_results();
         if (n_keep > kSelMax) {
             // a flat row: only the k best candidates outside the history can matter
             by_bins = false;
