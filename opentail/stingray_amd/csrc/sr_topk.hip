@@ -2064,12 +2064,25 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
             if constexpr (!kKept) {
                 const int need = max((cur.sel + S * kWaves - 1) / (S * kWaves), 1);
                 // the wave's largest kept element: the row tail drops what lies hopelessly far below the row's
-                const uint32_t wmax = sr_wave_max_u32(sr_okey(fmaxf(fmaxf(gm1[0], gm1[1]), fmaxf(gm1[2], gm1[3]))));
-                const uint32_t K = largest_key16(wmax, [&](uint32_t cnd) SR_INL -> bool {
-                    const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
-                    return __popcll(__ballot(gm1[0] >= fc)) + __popcll(__ballot(gm1[1] >= fc)) +
-                           __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc)) >= need;
-                });
+                const float pa = fmaxf(gm1[0], gm1[1]), pb = fminf(gm1[0], gm1[1]), pc = fmaxf(gm1[2], gm1[3]), pd = fminf(gm1[2], gm1[3]);
+                const uint32_t k1 = sr_okey(fmaxf(pa, pc));  // the lane's largest group maximum
+                const uint32_t wmax = sr_wave_max_u32(k1);
+                uint32_t K;
+                if (kShort && need <= 2) {
+                    // (a share of one or two, as every launch of short lists asks for: the wave's largest or second
+                    // largest group maximum itself, from two reductions instead of a search with ballots)
+                    const uint32_t k2 = sr_okey(fmaxf(fminf(pa, pc), fmaxf(pb, pd)));  // the lane's second largest
+                    const unsigned long long top = __ballot(k1 == wmax);
+                    const bool owner = lane == (int)__ffsll((long long)top) - 1;
+                    const uint32_t w2 = sr_wave_max_u32(owner ? k2 : k1);
+                    K = (need == 1 ? wmax : w2) & 0xffff0000u;
+                } else {
+                    K = largest_key16(wmax, [&](uint32_t cnd) SR_INL -> bool {
+                        const float fc = sr_okey_inv(cnd);  // a key in the NaN range compares false: the right answer for it
+                        return __popcll(__ballot(gm1[0] >= fc)) + __popcll(__ballot(gm1[1] >= fc)) +
+                               __popcll(__ballot(gm1[2] >= fc)) + __popcll(__ballot(gm1[3] >= fc)) >= need;
+                    });
+                }
                 if (lane == 0) {
                     uint32_t* gb = a.gbound + (((size_t)cur.slot * S + cur.c) * kWaves + (tid >> 6)) * 2;
                     __hip_atomic_store(gb, K, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
