@@ -108,6 +108,58 @@ def test_random_batches_tokens_and_distributions(ctx, seed):
                 assert toks[r] == wt and _same_bits(d[r], wd), (seed, trial, r, n, p)
 
 
+def test_random_batches_with_a_worker_per_row(ctx):
+    # 136 .. 256 rows: the launch in which every worker streams its own row, keeps the chunk results in registers and
+    # takes one share of the bound per wave and row.  Row widths of one to four chunks, rows of ties, of negative
+    # logits only, with whole chunks masked out, top-k from 1 to 2,000 (beyond the kernel's lists: the wide path),
+    # histories that lower and that raise, allow-masks; fp32 and bf16.
+    import torch
+
+    from opentail.stingray_amd import synthetic
+
+    rng = np.random.default_rng(77)
+    for trial in range(60):
+        rows = int(rng.integers(136, 257))
+        n = int(rng.choice([rng.integers(600, 3000), rng.integers(3000, 40000), rng.integers(40000, 160000)]))
+        kind = rng.integers(0, 5)
+        if kind == 0:
+            lg = (rng.integers(-14, 14, (rows, n)) / 2.0).astype(np.float32)
+        elif kind == 1:
+            lg = rng.normal(0, rng.choice([0.3, 2.0, 6.0]), (rows, n)).astype(np.float32)
+        elif kind == 2:
+            lg = np.round(rng.normal(0, 2, (rows, n)) * 4).astype(np.float32) / 4
+        elif kind == 3:
+            lg = synthetic.zipf_head_logits(rng, rows, n)
+        else:
+            lg = -np.abs(rng.normal(0, 3, (rows, n))).astype(np.float32) - 5.0
+        if rng.random() < 0.3:
+            lg[rng.random((rows, n)) < 0.2] = NEG
+        if rng.random() < 0.3:
+            lg[:, : n // 2] = NEG
+        params = []
+        for _ in range(rows):
+            hist = rng.integers(0, n, int(rng.choice([0, 3, 40, 400]))).tolist()
+            params.append(SamplingParams(
+                Temperature=float(rng.choice([0.0, 0.3, 0.8, 1.0, 1.6])),
+                TopK=int(rng.choice([1, 2, 7, 40, 64, 65, 300, 900, 1000, 2000])),
+                TopP=float(rng.choice([1.0, 0.95, 0.7, 0.2])), MinP=float(rng.choice([0.0, 1e-4, 0.05, 0.4])),
+                RepetitionPenalty=float(rng.choice([1.0, 1.2, 1.2, 0.8])),
+                PresencePenalty=float(rng.choice([0.0, 0.5, 0.5, -0.5])),
+                FrequencyPenalty=float(rng.choice([0.0, 0.2, 0.2, -0.1])), RepeatLastN=int(rng.choice([0, 5, 64])),
+                PreviousTokens=hist))
+        mask, act = _mask(rng, rows, n)
+        u = rng.random(rows)
+        if trial % 3 == 1:
+            bits = synthetic.to_bf16_bits(lg)
+            lg = synthetic.bf16_bits_to_f32(bits)
+            dev = torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
+        else:
+            dev = torch.from_numpy(lg).cuda()
+        got = ctx.sample_batch(dev, params, u, mask, act)
+        want = oracle_tokens(lg, params, u, mask, act)
+        assert np.array_equal(got, want), (trial, rows, n, int(kind), str(dev.dtype), np.nonzero(got != want)[0][:4])
+
+
 def test_random_speculative_verification_rows(ctx):
     import torch
 
