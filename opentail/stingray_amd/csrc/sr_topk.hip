@@ -1171,10 +1171,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     // rounds (0.4 us each) instead of a chain of a thousand dependent additions (4 us); a short list is quicker
     // summed by one lane.
     constexpr int kRun = 16;
-#ifndef SR_AB_KSUM
-#define SR_AB_KSUM 384
-#endif
-    constexpr int kSumByOneLane = SR_AB_KSUM;
+    constexpr int kSumByOneLane = 384;
     auto load_run = [&](int base, int limit, float (&x)[kRun]) SR_INL {
         const float4* p4 = (const float4*)(sm.probs + base) + sr_lane() * (kRun / 4);
 #pragma unroll
