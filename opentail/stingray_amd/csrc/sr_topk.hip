@@ -434,8 +434,10 @@ __device__ __forceinline__ int block_min_i32(int v, TopkSmem& sm)
 
 // The largest key, to its upper 16 bits, for which `enough` holds (0: none); `enough` must hold for every key below one
 // for which it holds, must not hold above `kmax`, and must be the same in every lane.  The answer nearly always has the
-// sign and exponent of kmax, or the exponent below: those nine bits are tried as a whole and the seven bits below them
-// one by one, eight or nine tries instead of sixteen.
+// sign and exponent of kmax or one of the exponents just below (a peaked row's k-th largest lies two below its
+// largest): those nine bits are tried as a whole, from kmax's downwards, four times at most, and then the seven bits
+// below them one by one -- eight to eleven tries instead of sixteen; all sixteen bits one by one when none of the four
+// holds.
 template <typename Enough>
 __device__ __forceinline__ uint32_t largest_key16(uint32_t kmax, Enough enough)
 {
@@ -1953,7 +1955,6 @@ __global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArg
         // two bodies, or a condition around the loads, the compiler keeps the incoming vectors in registers of their
         // own and spills.
         int last_sel = 0;
-        // (kKept) group maxima of the wave, over all chunks folded so far, at or above the value of key `cnd`
         // (kKept) The wave's share of the row's bound, taken from the largest group maximum of every lane and chunk folded
         // so far (one value per lane and chunk instead of four: a lane with two groups of a chunk at or above the value
         // counts once, which can only lower the value and keeps it a bound -- a twelfth of the count at the largest
