@@ -1236,7 +1236,7 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     // one chain of additions (every lane the same one): whole blocks of 32 entries without a look (eight loads in
     // flight, the sums never decrease) until a block's last sum has reached the target, then that block entry by
     // entry.  A search that goes on from there takes the wave's exact scan.
-    constexpr int kChainFirst = 256;
+    constexpr int kChainFirst = 32;
     if (sr_wave_id() == 0) {
         const bool use_top_p = rd.top_p < 1.0f && rd.top_p > 0.0f;
         const float top_p = use_top_p ? rd.top_p : __uint_as_float(0x7f800000u);  // +inf: never reached
