@@ -1193,7 +1193,22 @@ __device__ __forceinline__ void topk_row_tail(const SrTopkArgs& a, int slot, int
     if (n_sum > kSumByOneLane) {
         if (sr_wave_id() == 0) {
             float sum = 0.0f;
-            for (int base = 0; base < n_sum; base += SR_WAVE * kRun) {
+            constexpr int kHead = 32;
+            static_assert(kHead % 4 == 0 && kHead <= kSumByOneLane, "whole vectors of a list that is longer");
+            {
+                // (the sum doubles quickly at first: its first entries are added as a chain, every lane the same one, so
+                // that the scan behind them starts in the binade in which most of the list is added)
+                const float4* p4 = (const float4*)sm.probs;
+                float4 v[kHead / 4];
+#pragma unroll
+                for (int i = 0; i < kHead / 4; i++) v[i] = p4[i];
+#pragma unroll
+                for (int i = 0; i < kHead / 4; i++) {
+                    sum = __fadd_rn(sum, v[i].x); sum = __fadd_rn(sum, v[i].y);
+                    sum = __fadd_rn(sum, v[i].z); sum = __fadd_rn(sum, v[i].w);
+                }
+            }
+            for (int base = kHead; base < n_sum; base += SR_WAVE * kRun) {
                 float x[kRun];
                 load_run(base, n_sum, x);
                 int unused;
