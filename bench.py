@@ -306,7 +306,9 @@ def run_workload(args, ctx, stream) -> dict:
         b = i % n_buf
         ctx.sample_launch(batches[b], bufs[b], toks[b], flags[b])
 
-    for i in range(args.warmup):
+    # every rotated buffer is launched once before the timed steps whatever --warmup says: a batch builds its scan masks
+    # at its first launch (they depend on where the logits lie), and that is set-up, not a step
+    for i in range(max(args.warmup, n_buf)):
         step(i)
     torch.cuda.synchronize()
     if args.copy_probe:
