@@ -133,8 +133,10 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
     topk_geometry(b->vocab, epv == 8 ? SR_DTYPE_BF16 : SR_DTYPE_F32, n_sel, ctx->cu_count, &chunks, &chunk_vecs);
     {
         // The selection kernel's grid: workers with a program each -- chunk items to stream, then at most one row to
-        // finish.  A CU holds two workgroups of this kernel, so 2 x CUs workers are resident from the start and a
-        // later one starts when one of them ends.
+        // finish.  One worker per CU is resident from the start and a later one starts when one of them ends.  (A CU
+        // holds two workgroups of the kernel that launches of more workers than CUs take; with one per CU the launch
+        // takes the kernel that is compiled for half as many waves and keeps its row tails' registers: 80 rows
+        // 29.8 -> 27.3 us, 112 rows 32.5 -> 31.1 us against two workers per CU, measured.)
         //
         // The programs are written by a simulation of the launch: the chunk items, rows in order of decreasing tail
         // length, are dealt out one by one to the worker that will be free first; the worker that gets a row's last
@@ -148,7 +150,7 @@ int prepare_scan(sr_batch* b, int epv, unsigned long long base_addr, long long s
         // so that what a row's chunks write is in the L2 that its tail reads from.  Nothing depends on that placement
         // for correctness.  A batch of few rows deals its items out to all dies instead.
         const int n_xcd = std::min(SR_TK_MAX_XCD, std::max(1, ctx->cu_count / 32));
-        const int resident = 2 * std::max(ctx->cu_count, n_xcd);
+        const int resident = std::max(ctx->cu_count, n_xcd);
         const int total_items = n_sel * chunks;
         const bool spread = n_sel < 2 * n_xcd;
         const int n_pool = spread ? 1 : n_xcd;        // pools of workers that share a list of items
@@ -1136,6 +1138,7 @@ int sr_sample_launch(sr_ctx* ctx, const sr_batch* b, const void* logits_dev, int
         a.progs = b->d_sched.as<int4>();
         a.items = b->d_sched.as<int4>() + b->n_workers;
         a.n_workers = b->n_workers;
+        a.cu_count = ctx->cu_count;
         a.own_rows = b->own_rows ? 1 : 0;
         a.kept = (b->own_rows && b->n_workers <= ctx->cu_count) ? 1 : 0;
         a.short_lists = b->max_sel <= SR_TK_SHORT_SEL ? 1 : 0;

@@ -45,6 +45,7 @@ struct SrTopkArgs {
     const int4* items;
     const int4* progs;
     int32_t n_workers, n_items;
+    int32_t cu_count;        // compute units of the device
     int32_t own_rows;        // every worker's program is one whole row (all its chunks, then its tail)
     int32_t kept;            // ... and there is at most one worker per compute unit
     int32_t short_lists;     // no row of the launch asks for more than SR_TK_SHORT_SEL entries

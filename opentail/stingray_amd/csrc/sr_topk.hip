@@ -1857,8 +1857,12 @@ __device__ __forceinline__ int build_candidates(const SrTopkArgs& a, int slot, i
 // worker per compute unit.  Nothing is handed over then, so nothing is written out: the group results of all chunks
 // stay in the thread's registers (the workgroup has the register file of its compute unit to itself) and the waves'
 // shares of the bound go through LDS.
-template <int EPV, int kVec, int kWindow, bool kKept, bool kShort>
-__global__ __launch_bounds__(kThreads, kKept ? 2 : 4) void k_topk_rows(SrTopkArgs a)
+// kRoomy: a launch of at most one worker per compute unit whose rows' chunks several workers stream (a batch of few
+// rows): compiled for two waves a SIMD like the register-keeping shape, so that the row tail keeps its registers
+// (with four waves a SIMD it spills a hundred bytes a lane, which the tails of a launch that has the compute units to
+// itself need not pay for).
+template <int EPV, int kVec, int kWindow, bool kKept, bool kShort, bool kRoomy = false>
+__global__ __launch_bounds__(kThreads, (kKept || kRoomy) ? 2 : 4) void k_topk_rows(SrTopkArgs a)
 {
     __shared__ TopkSmem sm;
     using VO = VecOps<EPV>;
@@ -2398,6 +2402,7 @@ hipError_t sr_launch_topk(const SrTopkArgs& a, int n_rows, hipStream_t stream)
         constexpr bool kS = decltype(shrt)::value;
         if (kept) hipLaunchKernelGGL((k_topk_rows<kE, kV, SR_TK_WINDOW_KEPT, true, kS>), grid, block, 0, stream, a);
         else if (a.own_rows) hipLaunchKernelGGL((k_topk_rows<kE, kV, SR_TK_WINDOW_OWN, false, kS>), grid, block, 0, stream, a);
+        else if (a.n_workers <= a.cu_count) hipLaunchKernelGGL((k_topk_rows<kE, kV, SR_TK_WINDOW, false, kS, true>), grid, block, 0, stream, a);
         else hipLaunchKernelGGL((k_topk_rows<kE, kV, SR_TK_WINDOW, false, kS>), grid, block, 0, stream, a);
     };
     using std::integral_constant;
