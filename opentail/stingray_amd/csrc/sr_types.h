@@ -81,7 +81,9 @@ struct SrMaskClear {
 #define SR_ARGMAX_STATIC_ROWS 16384        // rows the argmax entry point that allocates nothing takes per call
 #define SR_TK_WINDOW 5                     // ... of which a thread has in flight or in registers at a time
 #define SR_TK_WINDOW_OWN 10                // ... when every worker streams one row of its own
-#define SR_TK_WINDOW_KEPT 19               // ... and has a compute unit to itself
+#define SR_TK_WINDOW_KEPT 5                // ... and has a compute unit to itself (the whole chunk in flight, 19, was the setting while
+                                           // every chunk ended with a bound loop for the loads to hide; without those loops it costs
+                                           // 1.3 us a launch at 256 rows: what is in flight beyond the window only queues)
 #define SR_TK_MASK_WORDS 3                 // 32-bit keep-words per chunk thread: 19 x 4 and 10 x 8 bits both fit 96
 #define SR_TK_GROUPS 4                     // group maxima per thread
 #define SR_TK_SHORT_SEL 64                 // a launch whose rows all ask for at most this many entries: see k_topk_rows
